@@ -1,0 +1,226 @@
+/*
+ * ughip.h -- C ABI of the MI355X (gfx950) backend for ug.
+ *
+ * This is the boundary a Rust `ug-hip` crate binds with `extern "C"` to implement
+ * ug-core's `trait Device` / `trait Slice` (ug-core/src/lib.rs:29-73) and ug-llama's
+ * `trait Device` (ug-llama/src/main.rs:22-28).  Plain pointers and sizes only.
+ *
+ * Conventions
+ *   - every function returns 0 on success and a non-zero UGHIP_ERR_* code on failure;
+ *     ughip_last_error() then returns a thread-local, NUL-terminated message
+ *     (the shim maps it to ug::Error::Msg, ug-core/src/error.rs:3-100);
+ *   - lengths are in ELEMENTS unless the name says bytes;
+ *   - one HIP stream per device; work is stream-ordered and asynchronous unless stated;
+ *   - the caller is single-threaded per device, like ug's Arc<RefCell<..>> graph
+ *     (ug-core/src/lazy_buffer.rs:101-106).
+ */
+#ifndef UGHIP_H_
+#define UGHIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- error codes -------------------------------------------------------------------- */
+enum {
+  UGHIP_OK = 0,
+  UGHIP_ERR_INVALID = 1,      /* bad argument, dtype/len mismatch (cpu_runtime.rs:380-391) */
+  UGHIP_ERR_HIP = 2,          /* a HIP runtime call failed */
+  UGHIP_ERR_COMPILE = 3,      /* hiprtc rejected generated code, or malformed SSA */
+  UGHIP_ERR_STRIDING = 4,     /* Error::MatMulUnexpectedStriding (error.rs:110-116) */
+  UGHIP_ERR_UNSUPPORTED = 5,  /* dtype / op combination not implemented */
+  UGHIP_ERR_BOUNDS = 6        /* a kernel would index past the end of one of its slices */
+};
+
+/* ---- ug::DType (ug-core/src/dtype.rs:5-12), same order ------------------------------ */
+enum {
+  UGHIP_BF16 = 0,
+  UGHIP_F16 = 1,
+  UGHIP_F32 = 2,
+  UGHIP_I32 = 3,
+  UGHIP_I64 = 4
+};
+
+/* ---- ssa IR on the wire (ug-core/src/lang.rs:611-753) ------------------------------- *
+ * `ssa::Kernel` is a flat instruction list; the line number of an instruction is the
+ * VarId of its result.  The structs below are a field-for-field POD image of
+ * `ssa::A`, `ssa::Instr`, `(Arg, usize)` and `LaunchConfig` built from the public
+ * accessors `instrs()`, `args()`, `launch_config()` (lang.rs:719-729).               */
+
+/* ssa::A (lang.rs:642-646): a variable reference or an inline constant. */
+typedef struct ughip_a {
+  uint8_t is_const; /* 0: Var(var), 1: Const */
+  uint8_t dtype;    /* Const only: UGHIP_* dtype of the constant */
+  uint16_t pad_;
+  uint32_t var;     /* Var only: VarId */
+  int64_t i;        /* Const I32 / I64 value */
+  float f;          /* Const F32 / F16 / BF16 value (exact: both widen losslessly to f32) */
+  uint32_t pad2_;
+} ughip_a;
+
+/* ssa::Instr discriminant (lang.rs:690-709), same order. */
+enum {
+  UGHIP_I_DEFINE_ACC = 0,    /* a = initial Const */
+  UGHIP_I_DEFINE_GLOBAL = 1, /* n = index, dtype */
+  UGHIP_I_DEFINE_LOCAL = 2,  /* n = size (elements), dtype */
+  UGHIP_I_SPECIAL = 3,       /* sub = UGHIP_SPECIAL_* */
+  UGHIP_I_CONST = 4,         /* a = Const */
+  UGHIP_I_UNARY = 5,         /* sub = UGHIP_U_*, a = arg, dtype = result dtype */
+  UGHIP_I_BINARY = 6,        /* sub = UGHIP_B_*, a = lhs, b = rhs, dtype */
+  UGHIP_I_RANGE = 7,         /* a = lo, b = up, n = step, v = end_idx */
+  UGHIP_I_LOAD = 8,          /* v = src pointer var, a = offset, dtype */
+  UGHIP_I_ASSIGN = 9,        /* v = dst var, a = src */
+  UGHIP_I_END_RANGE = 10,    /* v = start_idx */
+  UGHIP_I_IF = 11,           /* a = cond, v = end_idx */
+  UGHIP_I_END_IF = 12,
+  UGHIP_I_STORE = 13,        /* v = dst pointer var, a = offset, b = value, dtype */
+  UGHIP_I_BARRIER = 14,
+  UGHIP_I_REDUCE_LOCAL = 15  /* sub = UGHIP_R_*, a = arg, dtype */
+};
+
+enum { UGHIP_SPECIAL_THREAD_IDX = 0, UGHIP_SPECIAL_BLOCK_IDX = 1 };           /* lang.rs:637-640 */
+enum { UGHIP_R_SUM = 0, UGHIP_R_MAX = 1, UGHIP_R_MIN = 2 };                   /* lang.rs:6-10   */
+enum { UGHIP_U_ID = 0, UGHIP_U_EXP, UGHIP_U_SIN, UGHIP_U_COS, UGHIP_U_NEG,
+       UGHIP_U_SQRT, UGHIP_U_CAST };                                          /* lang.rs:13-21  */
+enum { UGHIP_B_ADD = 0, UGHIP_B_SUB, UGHIP_B_MUL, UGHIP_B_DIV, UGHIP_B_MOD,
+       UGHIP_B_MIN, UGHIP_B_MAX };                                            /* lang.rs:24-32  */
+
+typedef struct ughip_instr {
+  int32_t op;    /* UGHIP_I_* */
+  int32_t dtype; /* UGHIP_* dtype where the instruction carries one */
+  int32_t sub;   /* op-specific selector, see the enum comments */
+  uint32_t v;    /* VarId operand (pointer var, assign target, range partner) */
+  uint64_t n;    /* index / size / step */
+  ughip_a a;
+  ughip_a b;
+} ughip_instr;
+
+/* One entry of ssa::Kernel::args(): (Arg, line_no) (lang.rs:714,727). */
+typedef struct ughip_kernel_arg {
+  uint64_t arg_id; /* ArgId, informational */
+  uint8_t is_ptr;  /* Type::Ptr vs Type::Value; only pointers are supported (lower_op.rs:413-416) */
+  uint8_t dtype;
+  uint16_t pad_;
+  uint32_t var;    /* line number of the DefineGlobal that introduces it */
+} ughip_kernel_arg;
+
+typedef struct ughip_ssa {
+  const ughip_instr* instrs;
+  size_t n_instrs;
+  const ughip_kernel_arg* args;
+  size_t n_args;
+  uint32_t grid_dim;   /* LaunchConfig (lang.rs:34-39); honoured only for kernels that use */
+  uint32_t block_dim;  /* Special / Barrier / ReduceLocal / DefineLocal -- serial loop nests */
+  uint32_t shared_mem; /* are re-parallelised by the backend and ignore it.               */
+  uint32_t pad_;
+} ughip_ssa;
+
+/* ---- opaque handles ------------------------------------------------------------------ */
+typedef struct ughip_device ughip_device; /* ug_cuda::runtime::Device  (ug-cuda/src/runtime.rs:80-85) */
+typedef struct ughip_slice ughip_slice;   /* ug_cuda::runtime::Slice   (runtime.rs:88-101)            */
+typedef struct ughip_func ughip_func;     /* ug_cuda::runtime::Func    (runtime.rs:49-54)             */
+typedef struct ughip_event ughip_event;
+
+const char* ughip_last_error(void);
+
+/* ---- device: Device::new / Clone / synchronize (runtime.rs:158-177,243-246) ---------- */
+int ughip_device_create(int ordinal, ughip_device** out);
+int ughip_device_retain(ughip_device* dev);
+int ughip_device_release(ughip_device* dev);
+int ughip_synchronize(ughip_device* dev);
+/* "gfx950" etc.; buf receives a NUL-terminated arch name. */
+int ughip_device_arch(ughip_device* dev, char* buf, size_t buf_len);
+/* `Device::use_grid()` (lib.rs:72): this backend returns 0 -- it wants the serial loop
+ * nest and chooses grid/block itself. */
+int ughip_use_grid(void);
+
+/* ---- memory: Device::allocate_uninit, trait Slice (lib.rs:29-54) --------------------- */
+/* Zero-filled like CpuDevice::allocate_uninit (cpu_runtime.rs:255-264).  len 0 is legal
+ * (ug-llama/src/model.rs:192) and yields a slice with a null device pointer. */
+int ughip_alloc(ughip_device* dev, int dtype, size_t len, ughip_slice** out);
+int ughip_free(ughip_slice* s);
+size_t ughip_slice_len(const ughip_slice* s);
+int ughip_slice_dtype(const ughip_slice* s);
+void* ughip_slice_ptr(const ughip_slice* s); /* raw device pointer (for interop / tests) */
+/* Slice::copy_host_to_device / copy_device_to_host (lib.rs:35-36): error unless
+ * dtype == slice dtype and len == slice len (cpu_runtime.rs:376-412).  The result is
+ * visible when the call returns. */
+int ughip_h2d(ughip_slice* dst, const void* src, int dtype, size_t len);
+int ughip_d2h(const ughip_slice* src, void* dst, int dtype, size_t len);
+
+/* ---- kernels: Device::compile / Device::run (lib.rs:56-60) --------------------------- */
+/* name may be NULL; it is sanitised and uniquified (runtime.rs:249-253).  Constants are
+ * baked into the SSA (lib.rs:57-59). */
+int ughip_compile(ughip_device* dev, const ughip_ssa* ssa, const char* name, ughip_func** out);
+int ughip_func_release(ughip_func* f);
+/* args in ssa.args() order (schedule.rs:190-195); asynchronous; zero-sized launch is a
+ * no-op (runtime.rs:269-277).  Fails with UGHIP_ERR_BOUNDS if a slice is shorter than the
+ * largest offset the kernel can form. */
+int ughip_run(ughip_device* dev, ughip_func* f, ughip_slice* const* args, size_t n_args);
+/* HIP source the SSA was lowered to (counterpart of `Kernel.cuda_code()`,
+ * ug-pyo3/src/lib.rs:396-401).  Returns the length excluding NUL; copies at most buf_len. */
+size_t ughip_func_source(const ughip_func* f, char* buf, size_t buf_len);
+/* Lowering strategy and launch shape picked by the backend (for tests and profiling). */
+typedef struct ughip_func_info {
+  int32_t strategy; /* UGHIP_STRAT_* */
+  uint32_t grid_dim;
+  uint32_t block_dim;
+  uint32_t lds_bytes;
+  uint64_t scratch_bytes;
+} ughip_func_info;
+enum {
+  UGHIP_STRAT_LITERAL = 0,     /* 1:1 translation, SSA launch config */
+  UGHIP_STRAT_ELEMENTWISE = 1, /* flat thread-per-element(s) */
+  UGHIP_STRAT_ROW_BLOCK = 2,   /* workgroup (or wave) per row, cooperative reduce */
+  UGHIP_STRAT_ROW_THREAD = 3,  /* thread per row, serial reduce (strided reduce dims) */
+  UGHIP_STRAT_GRID_REDUCE = 4  /* many workgroups per row + deterministic second stage */
+};
+int ughip_func_get_info(const ughip_func* f, ughip_func_info* out);
+/* Lowering only, no device needed: SSA -> HIP source (for CPU-side inspection/tests). */
+int ughip_codegen(const ughip_ssa* ssa, const char* name, char* buf, size_t buf_len,
+                  size_t* out_len, ughip_func_info* info);
+
+/* hiprtc only, no device needed: does `source` build for `arch` ("gfx950")?  Lets the CPU-side
+ * test-suite check that every generated kernel compiles. */
+int ughip_rtc_check(const char* source, const char* arch, size_t* code_size);
+
+/* ---- matmul: Device::matmul (lib.rs:62-70) ------------------------------------------- */
+/* dst[b,m,n] = lhs[b,m,k] x rhs[b,k,n], beta = 0, f32 accumulate.  `rank` (2..4) strides
+ * per operand, in elements, as in ug::Layout (layout.rs:577-583); batch strides follow
+ * the rules of cpu_runtime.rs:527-549 and ug-cuda/src/gemm.rs:59-74.  dtype triple must
+ * match: F32 or BF16 (F16 is UGHIP_ERR_UNSUPPORTED). */
+int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs,
+                 const ughip_slice* rhs, size_t b, size_t m, size_t n, size_t k, size_t rank,
+                 const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset,
+                 const size_t* rhs_dims, const size_t* rhs_strides, size_t rhs_offset);
+
+/* ---- ug-llama custom ops (ug-llama/src/main.rs:22-28; oracle cpu_ops.rs:6-167) ------- */
+/* rope / rope_i (cuda_ops.rs:17-104): src, dst are [bh, t*d] f32, cos/sin [max_pos, d/2]
+ * f32, pos i32 (only pos[0] is read, cpu_ops.rs:67,100). */
+int ughip_rope(ughip_device* dev, const ughip_slice* src, const ughip_slice* cos,
+               const ughip_slice* sin, const ughip_slice* pos, ughip_slice* dst, size_t bh,
+               size_t t, size_t d, int interleaved);
+/* cat (cuda_ops.rs:106-141): [d1, d2_l] ++ [d1, d2_r] -> [d1, d2_l + d2_r], f32. */
+int ughip_cat(ughip_device* dev, const ughip_slice* lhs, const ughip_slice* rhs,
+              ughip_slice* dst, size_t d1, size_t d2_l, size_t d2_r);
+/* custom_softmax (cuda_ops.rs:143-174): row softmax over the last dim, f32. */
+int ughip_softmax_rows(ughip_device* dev, const ughip_slice* src, ughip_slice* dst,
+                       size_t n_rows, size_t n_cols);
+/* causal_mask (cpu_ops.rs:33-56; the CUDA and Metal backends bail): per [s1, s2] chunk,
+ * keep i2 <= i1, else -inf. */
+int ughip_causal_mask(ughip_device* dev, const ughip_slice* src, ughip_slice* dst, size_t bh,
+                      size_t s1, size_t s2);
+
+/* ---- timing on the device stream ----------------------------------------------------- */
+int ughip_event_create(ughip_device* dev, ughip_event** out);
+int ughip_event_record(ughip_event* ev);
+int ughip_event_elapsed_ms(ughip_event* start, ughip_event* stop, float* ms); /* waits for stop */
+int ughip_event_destroy(ughip_event* ev);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* UGHIP_H_ */

@@ -1,0 +1,449 @@
+// Flat C API over the host-side front-end, for ctypes (tests, bench) and other FFI callers.
+// Every function returns 0 on success; ugh_last_error() holds the message otherwise.
+#include "capi.h"
+
+#include <cstring>
+
+#include "hip_device.h"
+#include "llama.h"
+#include "ug/lazy_buffer.h"
+#include "ug/samples.h"
+
+using namespace ug;
+
+namespace {
+thread_local std::string g_err;
+
+template <typename F>
+int guard(F&& f) {
+  try {
+    f();
+    return 0;
+  } catch (const std::exception& e) {
+    g_err = e.what();
+    return 1;
+  } catch (...) {
+    g_err = "unknown error";
+    return 1;
+  }
+}
+
+DevicePtr& dev_of(void* d) {
+  if (!d) bail("null device");
+  return *static_cast<DevicePtr*>(d);
+}
+LazyBuffer& lb_of(void* p) {
+  if (!p) bail("null lazy buffer");
+  return *static_cast<LazyBuffer*>(p);
+}
+void* box(LazyBuffer lb) { return new LazyBuffer(std::move(lb)); }
+Shape shape_of(const size_t* dims, size_t rank) { return Shape(std::vector<size_t>(dims, dims + rank)); }
+
+Const const_of(int dtype, double v) {
+  switch ((DType)dtype) {
+    case DType::F32: return Const::f32((float)v);
+    case DType::BF16: return Const::bf16((float)v);
+    case DType::I32: return Const::i32((int32_t)v);
+    case DType::I64: return Const::i64((int64_t)v);
+    default: bail("unable to create const for this dtype");
+  }
+}
+
+std::function<void(const std::vector<Slice*>&)> wrap_cb(ugh_custom_fn fn, void* user) {
+  return [fn, user](const std::vector<Slice*>& vs) {
+    std::vector<void*> raw(vs.begin(), vs.end());
+    if (fn(user, raw.data(), raw.size())) bail("custom op callback failed");
+  };
+}
+
+struct CompiledBox {
+  CompiledSchedule cs;
+};
+}  // namespace
+
+extern "C" {
+
+const char* ugh_last_error(void) { return g_err.c_str(); }
+
+// ---- devices -------------------------------------------------------------------------------
+int ugh_hip_device_new(int ordinal, void** out) {
+  return guard([&] { *out = new DevicePtr(std::make_shared<HipDevice>(ordinal)); });
+}
+void ugh_device_free(void* d) { delete static_cast<DevicePtr*>(d); }
+int ugh_device_synchronize(void* d) {
+  return guard([&] { dev_of(d)->synchronize(); });
+}
+const char* ugh_device_name(void* d) { return d ? (*static_cast<DevicePtr*>(d))->name() : ""; }
+int ugh_device_use_grid(void* d) { return d && (*static_cast<DevicePtr*>(d))->use_grid(); }
+void* ugh_device_raw_hip(void* d) {
+  HipDevice* h = d ? dynamic_cast<HipDevice*>(static_cast<DevicePtr*>(d)->get()) : nullptr;
+  return h ? h->raw() : nullptr;
+}
+
+// ---- slices / funcs at the Device boundary -----------------------------------------------------
+int ugh_device_alloc(void* d, int dtype, size_t len, void** out) {
+  return guard([&] { *out = dev_of(d)->allocate_uninit((DType)dtype, len).release(); });
+}
+void ugh_slice_free(void* s) { delete static_cast<Slice*>(s); }
+size_t ugh_slice_len(void* s) { return static_cast<Slice*>(s)->len(); }
+int ugh_slice_dtype(void* s) { return (int)static_cast<Slice*>(s)->dtype(); }
+int ugh_slice_h2d(void* s, const void* src, int dtype, size_t len) {
+  return guard([&] { static_cast<Slice*>(s)->copy_host_to_device(src, (DType)dtype, len); });
+}
+int ugh_slice_d2h(void* s, void* dst, int dtype, size_t len) {
+  return guard([&] { static_cast<Slice*>(s)->copy_device_to_host(dst, (DType)dtype, len); });
+}
+int ugh_device_compile(void* d, void* kernel, const char* name, void** out) {
+  return guard([&] {
+    std::string n = name ? name : "";
+    *out = new std::shared_ptr<Func>(dev_of(d)->compile(*static_cast<ssa::Kernel*>(kernel), name ? &n : nullptr));
+  });
+}
+void ugh_func_free(void* f) { delete static_cast<std::shared_ptr<Func>*>(f); }
+int ugh_device_run(void* d, void* f, void** slices, size_t n) {
+  return guard([&] {
+    std::vector<Slice*> vs;
+    for (size_t i = 0; i < n; ++i) vs.push_back(static_cast<Slice*>(slices[i]));
+    dev_of(d)->run(**static_cast<std::shared_ptr<Func>*>(f), vs);
+  });
+}
+void* ugh_func_raw_hip(void* f) {
+  HipFunc* h = f ? dynamic_cast<HipFunc*>(static_cast<std::shared_ptr<Func>*>(f)->get()) : nullptr;
+  return h ? h->raw() : nullptr;
+}
+int ugh_device_matmul(void* d, void* dst, void* lhs, void* rhs, size_t b, size_t m, size_t n, size_t k, size_t rank, const size_t* ldims,
+                      const size_t* lstrides, size_t loff, const size_t* rdims, const size_t* rstrides, size_t roff) {
+  return guard([&] {
+    Layout ll, rl;
+    ll.shape_ = shape_of(ldims, rank);
+    ll.strides_.assign(lstrides, lstrides + rank);
+    ll.offset_ = loff;
+    rl.shape_ = shape_of(rdims, rank);
+    rl.strides_.assign(rstrides, rstrides + rank);
+    rl.offset_ = roff;
+    dev_of(d)->matmul(*static_cast<Slice*>(dst), *static_cast<Slice*>(lhs), *static_cast<Slice*>(rhs), b, m, n, k, ll, rl);
+  });
+}
+
+// ---- ssa kernels --------------------------------------------------------------------------------
+int ugh_sample_ssa(const char* name, size_t p0, size_t p1, size_t p2, void** out) {
+  return guard([&] {
+    std::string n = name;
+    ssa::Kernel k;
+    namespace S = samples::ssa_k;
+    if (n == "simple_add") k = S::simple_add(p0);
+    else if (n == "simple_dotprod") k = S::simple_dotprod(p0);
+    else if (n == "exp") k = S::exp(p0);
+    else if (n == "exp_block") k = S::exp_block(p0, p1);
+    else if (n == "softmax_barrier" || n == "softmax") k = S::softmax_barrier(p0, p1);
+    else if (n == "softmax_reduce") k = S::softmax_reduce(p0, p1);
+    else if (n == "softmax_block") k = S::softmax_block(p0, p1, p2);
+    else bail("unknown sample kernel " + n);
+    *out = new ssa::Kernel(std::move(k));
+  });
+}
+int ugh_sample_op_ssa(const char* name, size_t p0, size_t p1, long block_axis, long thread_dim, size_t thread_block_dim, void** out) {
+  return guard([&] {
+    std::string n = name;
+    op::Kernel k;
+    if (n == "softmax") k = samples::op_softmax(p0, p1);
+    else if (n == "affine") k = samples::op_affine(p0);
+    else bail("unknown sample op kernel " + n);
+    op::Opts opts;
+    if (block_axis >= 0) opts = opts.with_block_axis((size_t)block_axis);
+    if (thread_dim >= 0) opts = opts.with_thread_block((size_t)thread_dim, thread_block_dim);
+    *out = new ssa::Kernel(k.lower(opts));
+  });
+}
+int ugh_ssa_from_raw(const ughip_instr* instrs, size_t n, uint32_t grid, uint32_t block, uint32_t shared, void** out) {
+  return guard([&] {
+    ssa::Kernel k = ssa::Kernel::from_instrs(std::vector<ssa::Instr>(instrs, instrs + n));
+    k.launch_config = LaunchConfig{grid, block, shared};
+    *out = new ssa::Kernel(std::move(k));
+  });
+}
+int ugh_ssa_wire(void* kernel, ughip_ssa* out) {
+  return guard([&] { *out = static_cast<ssa::Kernel*>(kernel)->wire(); });
+}
+void ugh_ssa_set_launch(void* kernel, uint32_t grid, uint32_t block, uint32_t shared) {
+  static_cast<ssa::Kernel*>(kernel)->launch_config = LaunchConfig{grid, block, shared};
+}
+void ugh_ssa_free(void* kernel) { delete static_cast<ssa::Kernel*>(kernel); }
+
+// ---- lazy buffers ---------------------------------------------------------------------------------
+int ugh_lb_cst(void* d, int dtype, double v, const size_t* dims, size_t rank, void** out) {
+  return guard([&] { *out = box(LazyBuffer::cst(const_of(dtype, v), shape_of(dims, rank), dev_of(d))); });
+}
+int ugh_lb_copy(void* d, int dtype, const void* data, size_t len, const size_t* dims, size_t rank, void** out) {
+  return guard([&] { *out = box(LazyBuffer::copy(data, (DType)dtype, len, shape_of(dims, rank), dev_of(d))); });
+}
+int ugh_lb_alloc_uninit(void* d, int dtype, const size_t* dims, size_t rank, void** out) {
+  return guard([&] { *out = box(LazyBuffer::alloc_uninit((DType)dtype, shape_of(dims, rank), dev_of(d))); });
+}
+void ugh_lb_free(void* lb) { delete static_cast<LazyBuffer*>(lb); }
+int ugh_lb_unary(void* lb, int op, void** out) {
+  return guard([&] { *out = box(lb_of(lb).unary((UnaryOp)op)); });
+}
+int ugh_lb_cast(void* lb, int dtype, void** out) {
+  return guard([&] { *out = box(lb_of(lb).cast((DType)dtype)); });
+}
+int ugh_lb_binary(void* lb, int op, void* rhs, void** out) {
+  return guard([&] { *out = box(lb_of(lb).binary((BinaryOp)op, lb_of(rhs))); });
+}
+int ugh_lb_reduce(void* lb, int op, long dim, void** out) {
+  return guard([&] { *out = box(lb_of(lb).reduce((ReduceOp)op, dim)); });
+}
+int ugh_lb_matmul(void* lb, void* rhs, int transpose, void** out) {
+  return guard([&] { *out = box(lb_of(lb).matmul_(lb_of(rhs), transpose != 0)); });
+}
+int ugh_lb_split_dim(void* lb, long dim, size_t s1, size_t s2, void** out) {
+  return guard([&] { *out = box(lb_of(lb).split_dim(dim, s1, s2)); });
+}
+int ugh_lb_merge_dims(void* lb, long dim, void** out) {
+  return guard([&] { *out = box(lb_of(lb).merge_dims(dim)); });
+}
+int ugh_lb_squeeze(void* lb, long dim, void** out) {
+  return guard([&] { *out = box(lb_of(lb).squeeze(dim)); });
+}
+int ugh_lb_unsqueeze(void* lb, long dim, void** out) {
+  return guard([&] { *out = box(lb_of(lb).unsqueeze(dim)); });
+}
+int ugh_lb_get_on_dim(void* lb, long dim, size_t index, void** out) {
+  return guard([&] { *out = box(lb_of(lb).get_on_dim(dim, index)); });
+}
+int ugh_lb_reshape(void* lb, const size_t* dims, size_t rank, void** out) {
+  return guard([&] { *out = box(lb_of(lb).reshape(shape_of(dims, rank))); });
+}
+int ugh_lb_narrow(void* lb, long dim, size_t offset, size_t length, void** out) {
+  return guard([&] { *out = box(lb_of(lb).narrow(dim, offset, length)); });
+}
+int ugh_lb_broadcast(void* lb, const size_t* dims, size_t rank, void** out) {
+  return guard([&] { *out = box(lb_of(lb).broadcast(shape_of(dims, rank))); });
+}
+int ugh_lb_transpose(void* lb, long d1, long d2, void** out) {
+  return guard([&] { *out = box(lb_of(lb).transpose(d1, d2)); });
+}
+int ugh_lb_cat(void** lbs, size_t n, long dim, void** out) {
+  return guard([&] {
+    std::vector<LazyBuffer> v;
+    for (size_t i = 0; i < n; ++i) v.push_back(lb_of(lbs[i]));
+    *out = box(LazyBuffer::cat(v, dim));
+  });
+}
+int ugh_lb_set(void* lb, void* values, void** out) {
+  return guard([&] { *out = box(lb_of(lb).set(lb_of(values))); });
+}
+int ugh_lb_set_l(void* lb, void* values, const size_t* dims, const size_t* strides, size_t rank, size_t offset, void** out) {
+  return guard([&] {
+    Layout l;
+    l.shape_ = shape_of(dims, rank);
+    l.strides_.assign(strides, strides + rank);
+    l.offset_ = offset;
+    *out = box(lb_of(lb).set_l(lb_of(values), l));
+  });
+}
+int ugh_lb_custom(void* d, ugh_custom_fn fn, void* user, void** args, size_t n, const size_t* dims, size_t rank, int dtype, void** out) {
+  return guard([&] {
+    std::vector<LazyBuffer> v;
+    for (size_t i = 0; i < n; ++i) v.push_back(lb_of(args[i]));
+    *out = box(LazyBuffer::custom(wrap_cb(fn, user), v, shape_of(dims, rank), (DType)dtype, dev_of(d)));
+  });
+}
+int ugh_lb_custom_ip(void* lb, ugh_custom_fn fn, void* user, void** args, size_t n, void** out) {
+  return guard([&] {
+    std::vector<LazyBuffer> v;
+    for (size_t i = 0; i < n; ++i) v.push_back(lb_of(args[i]));
+    *out = box(lb_of(lb).custom_ip(wrap_cb(fn, user), v));
+  });
+}
+int ugh_lb_ssa(void* d, void* kernel, void** args, size_t n, const size_t* dims, size_t rank, int dtype, void** out) {
+  return guard([&] {
+    std::vector<LazyBuffer> v;
+    for (size_t i = 0; i < n; ++i) v.push_back(lb_of(args[i]));
+    *out = box(LazyBuffer::ssa(*static_cast<ssa::Kernel*>(kernel), v, shape_of(dims, rank), (DType)dtype, dev_of(d)));
+  });
+}
+size_t ugh_lb_rank(void* lb) { return static_cast<LazyBuffer*>(lb)->rank(); }
+void ugh_lb_dims(void* lb, size_t* out) {
+  const auto& d = static_cast<LazyBuffer*>(lb)->dims();
+  std::memcpy(out, d.data(), d.size() * sizeof(size_t));
+}
+int ugh_lb_dtype(void* lb) { return (int)static_cast<LazyBuffer*>(lb)->dtype(); }
+size_t ugh_lb_elem_count(void* lb) { return static_cast<LazyBuffer*>(lb)->elem_count(); }
+int ugh_lb_realized(void* lb) { return static_cast<LazyBuffer*>(lb)->realized(); }
+int ugh_lb_realize(void* lb) {
+  return guard([&] { lb_of(lb).realize(); });
+}
+int ugh_lb_data_vec(void* lb, int dtype, void* out, size_t len) {
+  return guard([&] {
+    if (len != lb_of(lb).elem_count()) bail("data_vec: output length mismatch");
+    lb_of(lb).data_vec(out, (DType)dtype);
+  });
+}
+// Overwrite the realised storage behind `lb` (the tests that poke at `lb.data()` in lb_tests.rs:82-94).
+int ugh_lb_write(void* lb, const void* data, int dtype, size_t len) {
+  return guard([&] {
+    LazyBuffer& b = lb_of(lb);
+    if (!b.data()->slice) bail("no data");
+    b.data()->slice->copy_host_to_device(data, (DType)dtype, len);
+  });
+}
+
+// ---- schedules ----------------------------------------------------------------------------------------
+int ugh_schedule_create(void** lbs, size_t n, void** out) {
+  return guard([&] {
+    std::vector<LazyBuffer> v;
+    for (size_t i = 0; i < n; ++i) v.push_back(lb_of(lbs[i]));
+    *out = new Schedule(Schedule::create(v));
+  });
+}
+void ugh_schedule_free(void* s) { delete static_cast<Schedule*>(s); }
+size_t ugh_schedule_n_items(void* s) { return static_cast<Schedule*>(s)->items().size(); }
+int ugh_schedule_item_kind(void* s, size_t i) { return (int)static_cast<Schedule*>(s)->items().at(i).kind; }
+size_t ugh_schedule_item_n_args(void* s, size_t i) {
+  const ScheduleItem& it = static_cast<Schedule*>(s)->items().at(i);
+  return it.kind == ScheduleItem::Kernel ? it.kernel.args.size() : it.args.size();
+}
+// Kernel items only: name (lower_op.rs:561-633) and the SSA from `optimize().lower(Opts::default())`.
+int ugh_schedule_item_name(void* s, size_t i, char* buf, size_t buf_len) {
+  return guard([&] {
+    const ScheduleItem& it = static_cast<Schedule*>(s)->items().at(i);
+    if (it.kind != ScheduleItem::Kernel) bail("not a kernel item");
+    std::string n = it.kernel.kernel().ops[0].name();
+    snprintf(buf, buf_len, "%s", n.c_str());
+  });
+}
+int ugh_schedule_item_ssa(void* s, size_t i, int optimize, void** out) {
+  return guard([&] {
+    const ScheduleItem& it = static_cast<Schedule*>(s)->items().at(i);
+    if (it.kind == ScheduleItem::Ssa) {
+      *out = new ssa::Kernel(it.ssa);
+      return;
+    }
+    if (it.kind != ScheduleItem::Kernel) bail("not a kernel item");
+    op::Kernel k = it.kernel.kernel();
+    if (optimize) k = k.optimize();
+    *out = new ssa::Kernel(k.lower(op::Opts()));
+  });
+}
+void* ugh_cache_new(void) { return new CompilationCache(); }
+void ugh_cache_free(void* c) { delete static_cast<CompilationCache*>(c); }
+size_t ugh_cache_size(void* c) {
+  CompilationCache* cc = static_cast<CompilationCache*>(c);
+  return cc->op_cache.size() + cc->ssa_cache.size();
+}
+int ugh_schedule_compile(void* s, void* cache, void** out) {
+  return guard([&] {
+    Schedule* sc = static_cast<Schedule*>(s);
+    CompiledBox* b = new CompiledBox();
+    try {
+      if (cache) b->cs = sc->compile_with_cache(*static_cast<CompilationCache*>(cache));
+      else b->cs = sc->compile();
+    } catch (...) {
+      delete b;
+      throw;
+    }
+    *out = b;
+  });
+}
+void ugh_compiled_free(void* c) { delete static_cast<CompiledBox*>(c); }
+int ugh_compiled_run(void* c) {
+  return guard([&] { static_cast<CompiledBox*>(c)->cs.run(); });
+}
+size_t ugh_compiled_n_funcs(void* c) { return static_cast<CompiledBox*>(c)->cs.funcs.size(); }
+int ugh_compiled_func_kind(void* c, size_t i) { return (int)static_cast<CompiledBox*>(c)->cs.funcs.at(i).kind; }
+void* ugh_compiled_func_raw_hip(void* c, size_t i) {
+  const CompiledFunc& f = static_cast<CompiledBox*>(c)->cs.funcs.at(i);
+  HipFunc* h = f.func ? dynamic_cast<HipFunc*>(f.func.get()) : nullptr;
+  return h ? h->raw() : nullptr;
+}
+
+// ---- ug-llama ---------------------------------------------------------------------------------------------
+using OpsPtr = std::shared_ptr<ug_llama::Ops>;
+int ugh_llama_ops_hip(void** out) {
+  return guard([&] { *out = new OpsPtr(ug_llama::hip_ops()); });
+}
+void ugh_llama_ops_free(void* o) { delete static_cast<OpsPtr*>(o); }
+static ug_llama::Ops& ops_of(void* o) {
+  if (!o) bail("null ops");
+  return **static_cast<OpsPtr*>(o);
+}
+int ugh_llama_rope(void* ops, void* src, void* cos, void* sin, void* pos, int interleaved, void** out) {
+  return guard([&] {
+    *out = box(interleaved ? ops_of(ops).rope_i(lb_of(src), lb_of(cos), lb_of(sin), lb_of(pos))
+                           : ops_of(ops).rope(lb_of(src), lb_of(cos), lb_of(sin), lb_of(pos)));
+  });
+}
+int ugh_llama_cat(void* ops, void* lhs, void* rhs, size_t axis, void** out) {
+  return guard([&] { *out = box(ops_of(ops).cat(lb_of(lhs), lb_of(rhs), axis)); });
+}
+int ugh_llama_custom_softmax(void* ops, void* src, void** out) {
+  return guard([&] { *out = box(ops_of(ops).custom_softmax(lb_of(src))); });
+}
+int ugh_llama_causal_mask(void* ops, void* src, void** out) {
+  return guard([&] { *out = box(ops_of(ops).causal_mask(lb_of(src))); });
+}
+int ugh_llama_rms_norm(void* src, void* alpha, float eps, void** out) {
+  return guard([&] { *out = box(ug_llama::rms_norm(lb_of(src), lb_of(alpha), eps)); });
+}
+int ugh_llama_softmax(void* src, void** out) {
+  return guard([&] { *out = box(ug_llama::softmax(lb_of(src))); });
+}
+int ugh_llama_silu(void* src, void** out) {
+  return guard([&] { *out = box(ug_llama::silu(lb_of(src))); });
+}
+int ugh_llama_repeat(void* src, size_t axis, size_t n_rep, void** out) {
+  return guard([&] { *out = box(ug_llama::repeat(lb_of(src), axis, n_rep)); });
+}
+int ugh_llama_index_select(void* src, void* ids, void** out) {
+  return guard([&] { *out = box(ug_llama::index_select(lb_of(src), lb_of(ids))); });
+}
+static ug_llama::Config cfg_of(const ugh_llama_config* c) {
+  ug_llama::Config cfg;
+  cfg.hidden_size = c->hidden_size;
+  cfg.intermediate_size = c->intermediate_size;
+  cfg.max_position_embeddings = c->max_position_embeddings;
+  cfg.num_attention_heads = c->num_attention_heads;
+  cfg.num_key_value_heads = c->num_key_value_heads;
+  cfg.num_hidden_layers = c->num_hidden_layers;
+  cfg.rms_norm_eps = c->rms_norm_eps;
+  cfg.rope_interleaved = c->rope_interleaved != 0;
+  cfg.rope_theta = c->rope_theta;
+  cfg.vocab_size = c->vocab_size;
+  return cfg;
+}
+int ugh_llama_rope_tables(void* d, const ugh_llama_config* c, void** cos, void** sin) {
+  return guard([&] {
+    ug_llama::Rope r = ug_llama::Rope::create(cfg_of(c), dev_of(d));
+    *cos = box(r.cos);
+    *sin = box(r.sin);
+  });
+}
+int ugh_llama_model_new(void* d, void* ops, const ugh_llama_config* c, int custom_softmax, uint64_t seed, float std, int round_bf16, void** out) {
+  return guard([&] {
+    auto w = ug_llama::synthetic_weights(seed, std, round_bf16 != 0);
+    *out = new ug_llama::Model(cfg_of(c), custom_softmax != 0, *w, dev_of(d), *static_cast<OpsPtr*>(ops));
+  });
+}
+void ugh_llama_model_free(void* m) { delete static_cast<ug_llama::Model*>(m); }
+int ugh_llama_generate(void* m, const int32_t* prompt, size_t n_prompt, size_t n_steps, int32_t* out_tokens, double* prefill_ms,
+                       double* decode_ms, float* margins) {
+  return guard([&] {
+    ug_llama::GenerateStats st;
+    std::vector<int32_t> p(prompt, prompt + n_prompt);
+    std::vector<int32_t> toks = ug_llama::generate_greedy(*static_cast<ug_llama::Model*>(m), p, n_steps, &st);
+    std::memcpy(out_tokens, toks.data(), toks.size() * sizeof(int32_t));
+    if (prefill_ms) *prefill_ms = st.prefill_ms;
+    if (decode_ms) *decode_ms = st.decode_ms;
+    if (margins) std::memcpy(margins, st.top1_margin.data(), st.top1_margin.size() * sizeof(float));
+  });
+}
+int ugh_synthetic_weights(uint64_t seed, float std, int round_bf16, const char* name, size_t n, float* out) {
+  return guard([&] {
+    auto w = ug_llama::synthetic_weights(seed, std, round_bf16 != 0);
+    std::vector<float> v = w->get(name, {n});
+    std::memcpy(out, v.data(), n * sizeof(float));
+  });
+}
+
+}  // extern "C"

@@ -1,0 +1,384 @@
+// Llama graph over ug::LazyBuffer.  Mirrors ug-llama/src/model.rs op for op, so the kernels
+// a device sees (names, shapes, argument order) are those of the reference.
+#include "llama.h"
+
+#include <chrono>
+#include <cmath>
+#include <thread>
+
+#include "hip_device.h"
+#include "rng.h"
+#include "ug/block.h"
+
+namespace ug_llama {
+
+using namespace ug;
+
+// ---- HIP custom ops (counterpart of ug-llama/src/cuda_ops.rs:17-179) -------------------------
+namespace {
+
+void hip_check(int rc, const char* what) {
+  if (rc) bail(std::string(what) + ": " + ughip_last_error());
+}
+
+ughip_device* hip_dev(const LB& lb) {
+  HipDevice* d = dynamic_cast<HipDevice*>(lb.device().get());
+  if (!d) bail("hip custom op used with a non-hip device");
+  return d->raw();
+}
+
+struct HipOps : Ops {
+  LB rope_any(const LB& src, const LB& cos, const LB& sin, const LB& pos, int interleaved) const {
+    if (src.rank() != 4) bail("rope: expected a rank-4 tensor, got " + src.shape().str());
+    size_t b = src.dims()[0], h = src.dims()[1], t = src.dims()[2], d = src.dims()[3];
+    ughip_device* dev = hip_dev(src);
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != 5) bail("rope: expected 5 slices");
+      hip_check(ughip_rope(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), hip_raw_slice(*vs[3]), hip_raw_slice(*vs[4]),
+                           b * h, t, d, interleaved),
+                "rope");
+    };
+    return LB::custom(f, {src, cos, sin, pos}, src.shape(), src.dtype(), src.device());
+  }
+  LB rope_i(const LB& src, const LB& cos, const LB& sin, const LB& pos) const override { return rope_any(src, cos, sin, pos, 1); }
+  LB rope(const LB& src, const LB& cos, const LB& sin, const LB& pos) const override { return rope_any(src, cos, sin, pos, 0); }
+
+  LB cat(const LB& lhs, const LB& rhs, size_t axis) const override {
+    const auto& ld = lhs.dims();
+    const auto& rd = rhs.dims();
+    if (axis >= ld.size()) bail("unexpected axis " + std::to_string(axis) + " for cat " + lhs.shape().str());
+    if (ld.size() != rd.size()) bail("unexpected shapes for cat " + lhs.shape().str() + " " + rhs.shape().str());
+    for (size_t i = 0; i < ld.size(); ++i)
+      if (i != axis && ld[i] != rd[i]) bail("unexpected shapes for cat " + lhs.shape().str() + " " + rhs.shape().str());
+    std::vector<size_t> dd = ld;
+    dd[axis] = ld[axis] + rd[axis];
+    size_t d1 = 1, d2_l = 1, d2_r = 1;
+    for (size_t i = 0; i < axis; ++i) d1 *= ld[i];
+    for (size_t i = axis; i < ld.size(); ++i) {
+      d2_l *= ld[i];
+      d2_r *= rd[i];
+    }
+    ughip_device* dev = hip_dev(lhs);
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != 3) bail("cat: expected 3 slices");
+      hip_check(ughip_cat(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), d1, d2_l, d2_r), "cat");
+    };
+    return LB::custom(f, {lhs, rhs}, Shape(dd), lhs.dtype(), lhs.device());
+  }
+
+  LB custom_softmax(const LB& src) const override {
+    size_t dim_m1 = src.dims()[src.rank() - 1];
+    size_t rows = dim_m1 ? src.elem_count() / dim_m1 : 0;
+    ughip_device* dev = hip_dev(src);
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != 2) bail("softmax: expected 2 slices");
+      hip_check(ughip_softmax_rows(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), rows, dim_m1), "custom_softmax");
+    };
+    return LB::custom(f, {src}, src.shape(), src.dtype(), src.device());
+  }
+
+  LB causal_mask(const LB& src) const override {
+    if (src.rank() != 4) bail("causal_mask: expected a rank-4 tensor, got " + src.shape().str());
+    size_t bh = src.dims()[0] * src.dims()[1], s1 = src.dims()[2], s2 = src.dims()[3];
+    ughip_device* dev = hip_dev(src);
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != 2) bail("causal_mask: expected 2 slices");
+      hip_check(ughip_causal_mask(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), bh, s1, s2), "causal_mask");
+    };
+    return LB::custom(f, {src}, src.shape(), src.dtype(), src.device());
+  }
+};
+
+}  // namespace
+
+std::shared_ptr<Ops> hip_ops() { return std::make_shared<HipOps>(); }
+
+// ---- synthetic weights -----------------------------------------------------------------------------
+namespace {
+struct SyntheticWeights : WeightSource {
+  uint64_t seed;
+  float std;
+  bool round_bf16;
+  SyntheticWeights(uint64_t s, float sd, bool r) : seed(s), std(sd), round_bf16(r) {}
+  std::vector<float> get(const std::string& name, const std::vector<size_t>& shape) override {
+    size_t n = 1;
+    for (size_t d : shape) n *= d;
+    std::vector<float> out(n);
+    uint64_t ts = ugrng::tensor_seed(seed, name);
+    unsigned nt = std::max(1u, std::min(16u, std::thread::hardware_concurrency()));
+    if (n < (1u << 16)) nt = 1;
+    size_t pairs = (n + 1) / 2, per = (pairs + nt - 1) / nt;
+    std::vector<std::thread> ths;
+    for (unsigned t = 0; t < nt; ++t) {
+      size_t p0 = t * per, p1 = std::min(pairs, p0 + per);
+      if (p0 >= p1) break;
+      ths.emplace_back([&, p0, p1] {
+        for (size_t p = p0; p < p1; ++p) {
+          double z0, z1;
+          ugrng::normal_pair(ts, p, &z0, &z1);
+          float a = (float)(z0 * std), b = (float)(z1 * std);
+          if (round_bf16) {
+            a = bf16_bits_to_f32(f32_to_bf16_bits(a));
+            b = bf16_bits_to_f32(f32_to_bf16_bits(b));
+          }
+          out[2 * p] = a;
+          if (2 * p + 1 < n) out[2 * p + 1] = b;
+        }
+      });
+    }
+    for (auto& th : ths) th.join();
+    return out;
+  }
+};
+}  // namespace
+
+std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16) {
+  return std::make_shared<SyntheticWeights>(seed, std, round_bf16);
+}
+
+// ---- graph builders (model.rs:32-109) --------------------------------------------------------------------
+// model.rs:32-63: hand-written SSA; the ids load is typed F32 although the buffer holds I32,
+// so the row offset is (int)((float)id * h).
+LB index_select(const LB& src, const LB& ids) {
+  DType dtype = DType::F32;
+  if (ids.rank() != 2 || src.rank() != 2) bail("index_select: expected rank-2 ids and table");
+  size_t b_sz = ids.dims()[0], seq_len = ids.dims()[1], h = src.dims()[1];
+  block::Block b;
+  uint32_t src_v = b.push(ssa::define_global(0, dtype)).to_varid();
+  uint32_t ids_v = b.push(ssa::define_global(1, DType::I32)).to_varid();
+  uint32_t dst_v = b.push(ssa::define_global(2, dtype)).to_varid();
+  block::Range r1 = b.range(ssa::i32(0), ssa::i32((int32_t)(b_sz * seq_len)), 1);
+  block::Id src_off = b.push(ssa::load(ids_v, r1.id().to_a(), dtype));
+  src_off = b.mul(src_off, (int32_t)h);
+  block::Id dst_off = b.mul(r1.id(), (int32_t)h);
+  block::Range r2 = b.range(ssa::i32(0), ssa::i32((int32_t)h), 1);
+  block::Id so = b.binary(BinaryOp::Add, src_off.to_a(), r2.id().to_a(), DType::I32);
+  block::Id d_o = b.binary(BinaryOp::Add, dst_off.to_a(), r2.id().to_a(), DType::I32);
+  block::Id ld = b.push(ssa::load(src_v, so.to_a(), dtype));
+  b.push(ssa::store(dst_v, d_o.to_a(), ld.to_a(), dtype));
+  b.end_range(r2);
+  b.end_range(r1);
+  ssa::Kernel k = ssa::Kernel::from_instrs(b.relocate());
+  return LB::ssa(k, {src, ids}, Shape({b_sz, seq_len, h}), src.dtype(), src.device());
+}
+
+// model.rs:65-78
+LB rms_norm(const LB& src, const LB& alpha, float eps) {
+  const DevicePtr& dev = src.device();
+  size_t rank = src.rank();
+  size_t dim_m1 = src.dims()[rank - 1];
+  LB sum2 = src.binary(BinaryOp::Mul, src).reduce(ReduceOp::Sum, (long)rank - 1);
+  const Shape& s2s = sum2.shape();
+  LB m = sum2.binary(BinaryOp::Mul, LB::cst(Const::f32(1.f / (float)dim_m1), s2s, dev))
+             .binary(BinaryOp::Add, LB::cst(Const::f32(eps), s2s, dev))
+             .unary(UnaryOp::Sqrt);
+  return src.binary(BinaryOp::Div, m.broadcast(src.shape())).binary(BinaryOp::Mul, alpha.broadcast(src.shape()));
+}
+
+// model.rs:80-92
+LB repeat(const LB& lb, size_t axis, size_t n_rep) {
+  if (n_rep == 1) return lb;
+  if (axis >= lb.rank()) bail("unexpected axis " + std::to_string(axis) + " for repeat " + lb.shape().str());
+  LB s = lb.split_dim((long)axis, lb.dims()[axis], 1);
+  std::vector<size_t> dims = s.dims();
+  dims[axis + 1] = n_rep;
+  return s.broadcast(Shape(dims)).merge_dims((long)axis);
+}
+
+// model.rs:94-101
+LB softmax(const LB& src) {
+  const Shape& s = src.shape();
+  LB mx = src.reduce(ReduceOp::Max, -1);
+  LB diff = src.binary(BinaryOp::Sub, mx.broadcast(s));
+  LB e = diff.unary(UnaryOp::Exp);
+  LB se = e.reduce(ReduceOp::Sum, -1);
+  return e.binary(BinaryOp::Div, se.broadcast(s));
+}
+
+// model.rs:103-109
+LB silu(const LB& src) {
+  LB exp_m = src.unary(UnaryOp::Neg).unary(UnaryOp::Exp);
+  LB one = LB::cst(Const::f32(1.f), Shape(), src.device()).broadcast(exp_m.shape());
+  LB den = exp_m.binary(BinaryOp::Add, one);
+  return src.binary(BinaryOp::Div, den);
+}
+
+// model.rs:277-296: theta on the host in f32 powf, then a [max_pos,1]x[1,d/2] matmul, cos/sin.
+Rope Rope::create(const Config& cfg, const DevicePtr& dev) {
+  size_t head_dim = cfg.head_dim(), max_seq_len = cfg.max_position_embeddings;
+  std::vector<float> theta;
+  for (size_t i = 0; i < head_dim; i += 2) theta.push_back(1.f / std::pow(cfg.rope_theta, (float)i / (float)head_dim));
+  LB theta_lb = LB::copy(theta.data(), DType::F32, theta.size(), Shape({1, head_dim / 2}), dev);
+  std::vector<float> idx(max_seq_len);
+  for (size_t i = 0; i < max_seq_len; ++i) idx[i] = (float)i;
+  LB idx_theta = LB::copy(idx.data(), DType::F32, idx.size(), Shape({max_seq_len, 1}), dev);
+  LB mm = idx_theta.matmul(theta_lb);
+  return Rope{mm.unary(UnaryOp::Cos), mm.unary(UnaryOp::Sin)};
+}
+
+// model.rs:188-197: zero-length caches.
+std::vector<Cache> Cache::create(const Config& cfg, const DevicePtr& dev) {
+  std::vector<Cache> c;
+  for (size_t i = 0; i < cfg.num_hidden_layers; ++i) {
+    Shape s({1, cfg.num_key_value_heads, 0, cfg.head_dim()});
+    c.push_back(Cache{LB::cst(Const::f32(0.f), s, dev), LB::cst(Const::f32(0.f), s, dev)});
+  }
+  return c;
+}
+
+// ---- model (model.rs:299-373) --------------------------------------------------------------------------------
+namespace {
+LB load_w(WeightSource& w, const std::string& name, const std::vector<size_t>& shape, const DevicePtr& dev) {
+  std::vector<float> v = w.get(name, shape);
+  size_t n = 1;
+  for (size_t d : shape) n *= d;
+  if (v.size() != n) bail("unexpected shape for " + name);
+  return LB::copy(v.data(), DType::F32, v.size(), Shape(shape), dev);
+}
+}  // namespace
+
+Model::Model(const Config& cfg, bool custom_softmax, WeightSource& w, const DevicePtr& dev, std::shared_ptr<Ops> ops)
+    : cfg_(cfg), custom_softmax_(custom_softmax), dev_(dev), ops_(std::move(ops)) {
+  if (!cfg.tie_word_embeddings) bail("tie_word_embeddings == false is not supported yet");
+  size_t h = cfg.hidden_size, isz = cfg.intermediate_size, kv = cfg.head_dim() * cfg.num_key_value_heads;
+  embedding_ = load_w(w, "model.embed_tokens.weight", {cfg.vocab_size, h}, dev);
+  ln_f_ = load_w(w, "model.norm.weight", {h}, dev);
+  for (size_t i = 0; i < cfg.num_hidden_layers; ++i) {
+    std::string p = "model.layers." + std::to_string(i);
+    Layer l;
+    l.rms1 = load_w(w, p + ".input_layernorm.weight", {h}, dev);
+    l.rms2 = load_w(w, p + ".post_attention_layernorm.weight", {h}, dev);
+    l.gate_proj = load_w(w, p + ".mlp.gate_proj.weight", {isz, h}, dev);
+    l.up_proj = load_w(w, p + ".mlp.up_proj.weight", {isz, h}, dev);
+    l.down_proj = load_w(w, p + ".mlp.down_proj.weight", {h, isz}, dev);
+    l.q_proj = load_w(w, p + ".self_attn.q_proj.weight", {h, h}, dev);
+    l.k_proj = load_w(w, p + ".self_attn.k_proj.weight", {kv, h}, dev);
+    l.v_proj = load_w(w, p + ".self_attn.v_proj.weight", {kv, h}, dev);
+    l.o_proj = load_w(w, p + ".self_attn.o_proj.weight", {h, h}, dev);
+    layers_.push_back(std::move(l));
+  }
+  rope_ = Rope::create(cfg, dev);
+}
+
+// model.rs:203-248
+LB Model::attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache) const {
+  if (xs.rank() != 3) bail("attention: expected [b, t, hidden]");
+  size_t seq_len = xs.dims()[1];
+  size_t nh = cfg_.num_attention_heads, nkv = cfg_.num_key_value_heads, hd = cfg_.head_dim();
+  LB q = xs.matmul_t(l.q_proj);
+  LB k = xs.matmul_t(l.k_proj);
+  LB v = xs.matmul_t(l.v_proj);
+  q = q.split_dim(2, nh, hd).transpose(2, 1);
+  k = k.split_dim(2, nkv, hd).transpose(2, 1);
+  v = v.split_dim(2, nkv, hd).transpose(2, 1);
+  if (cfg_.rope_interleaved) {
+    q = ops_->rope_i(q, rope_.cos, rope_.sin, pos);
+    k = ops_->rope_i(k, rope_.cos, rope_.sin, pos);
+  } else {
+    q = ops_->rope(q, rope_.cos, rope_.sin, pos);
+    k = ops_->rope(k, rope_.cos, rope_.sin, pos);
+  }
+  k = ops_->cat(cache.prev_k, k, 2);
+  v = ops_->cat(cache.prev_v, v, 2);
+  cache.prev_k = k;
+  cache.prev_v = v;
+  LB kr = repeat(k, 1, nh / nkv);
+  LB vr = repeat(v, 1, nh / nkv);
+
+  LB att = q.matmul_t(kr);
+  LB scale = LB::cst(Const::f32(std::pow((float)hd, -0.5f)), Shape(), q.device()).broadcast(att.shape());
+  att = att.binary(BinaryOp::Mul, scale);
+  if (seq_len != 1) att = ops_->causal_mask(att);
+  att = custom_softmax_ ? ops_->custom_softmax(att) : softmax(att);
+  LB out = att.matmul(vr);
+  out = out.transpose(2, 1).merge_dims(-2);
+  return out.matmul_t(l.o_proj);
+}
+
+// model.rs:160-168
+LB Model::mlp(const Layer& l, const LB& xs) const {
+  LB xs1 = xs.matmul_t(l.gate_proj);
+  LB xs2 = xs.matmul_t(l.up_proj);
+  xs1 = silu(xs1);
+  return xs1.binary(BinaryOp::Mul, xs2).matmul_t(l.down_proj);
+}
+
+// model.rs:259-269, 365-373
+LB Model::fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const {
+  if (cache.size() != layers_.size()) bail("cache/layer count mismatch");
+  LB xs = index_select(embedding_, tokens);
+  float eps = (float)cfg_.rms_norm_eps;
+  for (size_t i = 0; i < layers_.size(); ++i) {
+    const Layer& l = layers_[i];
+    LB residual = xs;
+    LB h = rms_norm(xs, l.rms1, eps);
+    h = attention(l, h, pos, cache[i]);
+    h = h.binary(BinaryOp::Add, residual);
+    residual = h;
+    LB m = rms_norm(h, l.rms2, eps);
+    m = mlp(l, m);
+    xs = m.binary(BinaryOp::Add, residual);
+  }
+  xs = rms_norm(xs, ln_f_, eps);
+  return xs.matmul_t(embedding_);
+}
+
+// One prefill call over the prompt, then `n_steps` greedy single-token steps (graph rebuilt per
+// step with a shared CompilationCache, as ug-llama/src/main.rs:124-146 does).  Returns the
+// n_steps + 1 argmax ids: one from the prefill logits, one per decode step.
+std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32_t>& prompt, size_t n_steps, GenerateStats* stats) {
+  using clock = std::chrono::steady_clock;
+  const Config& cfg = model.config();
+  const DevicePtr& dev = model.device();
+  if (prompt.empty()) bail("empty prompt");
+  if (prompt.size() + n_steps > cfg.max_position_embeddings) bail("prompt + steps exceed max_position_embeddings");
+  std::vector<Cache> cache = Cache::create(cfg, dev);
+  CompilationCache ccache;
+  std::vector<int32_t> out;
+  std::vector<float> logits;
+  std::vector<int32_t> feed = prompt;
+  size_t pos_v = 0;
+  for (size_t step = 0; step <= n_steps; ++step) {
+    auto t0 = clock::now();
+    size_t t = feed.size();
+    LB tokens = LB::copy(feed.data(), DType::I32, t, Shape({1, t}), dev);
+    int32_t p32 = (int32_t)pos_v;
+    LB pos = LB::copy(&p32, DType::I32, 1, Shape({1, 1}), dev);
+    LB lg = model.fwd(tokens, pos, cache);
+    Schedule::create_one(lg).compile_with_cache(ccache).run();
+    logits.resize(lg.elem_count());
+    lg.data_vec(logits.data(), DType::F32);
+    const float* last = logits.data() + (t - 1) * cfg.vocab_size;
+    size_t best = 0;
+    float second = -INFINITY;
+    for (size_t i = 1; i < cfg.vocab_size; ++i) {
+      if (last[i] > last[best]) {
+        second = last[best];
+        best = i;
+      } else if (last[i] > second) {
+        second = last[i];
+      }
+    }
+    double ms = std::chrono::duration<double, std::milli>(clock::now() - t0).count();
+    if (stats) {
+      if (step == 0) stats->prefill_ms = ms;
+      else {
+        stats->decode_ms += ms;
+        stats->step_ms.push_back(ms);
+      }
+      stats->top1_margin.push_back(last[best] - second);
+    }
+    pos_v += t;
+    out.push_back((int32_t)best);
+    feed.assign(1, (int32_t)best);
+    // The caches are realised now; dropping the graph that produced them keeps the DAG from
+    // growing with every step.
+    for (Cache& c : cache) {
+      c.prev_k.detach();
+      c.prev_v.detach();
+    }
+  }
+  return out;
+}
+
+}  // namespace ug_llama

@@ -1,0 +1,106 @@
+// ug-llama: the model graph (ug-llama/src/model.rs) over any ug::Device, plus the five custom
+// ops a device has to bring (`trait Device` of ug-llama/src/main.rs:22-28).
+#pragma once
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "ug/lazy_buffer.h"
+
+namespace ug_llama {
+
+using LB = ug::LazyBuffer;
+
+// ug-llama/src/main.rs:22-28
+struct Ops {
+  virtual ~Ops() = default;
+  virtual LB rope_i(const LB& src, const LB& cos, const LB& sin, const LB& pos) const = 0;
+  virtual LB rope(const LB& src, const LB& cos, const LB& sin, const LB& pos) const = 0;
+  virtual LB cat(const LB& lhs, const LB& rhs, size_t axis) const = 0;
+  virtual LB custom_softmax(const LB& src) const = 0;
+  virtual LB causal_mask(const LB& src) const = 0;
+};
+
+// The HIP implementation (counterpart of ug-llama/src/cuda_ops.rs).
+std::shared_ptr<Ops> hip_ops();
+
+// ug-llama/src/model.rs:10-30
+struct Config {
+  size_t hidden_size = 2048;
+  size_t intermediate_size = 5632;
+  size_t max_position_embeddings = 2048;
+  size_t num_attention_heads = 32;
+  size_t num_key_value_heads = 4;
+  size_t num_hidden_layers = 22;
+  double rms_norm_eps = 1e-5;
+  bool rope_interleaved = false;
+  float rope_theta = 10000.f;
+  bool tie_word_embeddings = true;
+  size_t vocab_size = 32000;
+  size_t head_dim() const { return hidden_size / num_attention_heads; }
+};
+
+// Where the weights come from: tensors by HF name (model.rs:313-346), already f32 on the host
+// (the reference always loads with `load_with_cast(.., F32, ..)`, model.rs:118,140,313).
+struct WeightSource {
+  virtual ~WeightSource() = default;
+  virtual std::vector<float> get(const std::string& name, const std::vector<size_t>& shape) = 0;
+};
+
+// Random-init weights: N(0, std) from a counter-based generator keyed by (seed, tensor name),
+// optionally rounded to bf16 (round-to-nearest-even) and widened back.
+std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16);
+
+// Graph builders of model.rs:32-109, usable on their own.
+LB index_select(const LB& src, const LB& ids);
+LB rms_norm(const LB& src, const LB& alpha, float eps);
+LB repeat(const LB& lb, size_t axis, size_t n_rep);
+LB softmax(const LB& src);
+LB silu(const LB& src);
+struct Rope {
+  LB cos, sin;
+  static Rope create(const Config& cfg, const ug::DevicePtr& dev);
+};
+
+// model.rs:183-198
+struct Cache {
+  LB prev_k, prev_v;
+  static std::vector<Cache> create(const Config& cfg, const ug::DevicePtr& dev);
+};
+
+// model.rs:299-373
+class Model {
+ public:
+  Model(const Config& cfg, bool custom_softmax, WeightSource& weights, const ug::DevicePtr& dev, std::shared_ptr<Ops> ops);
+  LB fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const;
+  const Config& config() const { return cfg_; }
+  const ug::DevicePtr& device() const { return dev_; }
+
+ private:
+  struct Layer {
+    LB rms1, rms2;
+    LB q_proj, k_proj, v_proj, o_proj;
+    LB gate_proj, up_proj, down_proj;
+  };
+  LB attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache) const;
+  LB mlp(const Layer& l, const LB& xs) const;
+  Config cfg_;
+  bool custom_softmax_;
+  ug::DevicePtr dev_;
+  std::shared_ptr<Ops> ops_;
+  LB embedding_, ln_f_;
+  Rope rope_;
+  std::vector<Layer> layers_;
+};
+
+// The harness of BASELINE config 5: one prefill call over `prompt`, then `n_steps` greedy
+// (argmax) single-token steps with the KV cache.  Returns the generated ids; timings in ms.
+struct GenerateStats {
+  double prefill_ms = 0, decode_ms = 0;
+  std::vector<double> step_ms;
+  std::vector<float> top1_margin;  // logit gap between the best and second-best token per step
+};
+std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32_t>& prompt, size_t n_steps, GenerateStats* stats);
+
+}  // namespace ug_llama

@@ -1,0 +1,50 @@
+// Shared between the translation units of libughip.so; not part of the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <map>
+#include <mutex>
+#include <string>
+
+#include "ughip.h"
+
+struct CachedModule {
+  hipModule_t module = nullptr;
+  hipFunction_t function = nullptr;
+};
+
+struct ughip_device {
+  std::atomic<int> refs{1};
+  int ordinal = 0;
+  hipStream_t stream = nullptr;
+  std::string arch;
+  int num_cus = 0;
+  std::mutex mu;
+  // Size-class free lists: freed blocks are reused by later allocations on the same stream.
+  std::multimap<size_t, void*> pool;
+  size_t pool_bytes = 0, live_bytes = 0;
+  std::map<std::string, CachedModule> modules;  // generated source -> loaded code object
+};
+
+struct ughip_slice {
+  ughip_device* dev = nullptr;
+  void* ptr = nullptr;
+  int dtype = UGHIP_F32;
+  size_t len = 0, cap_bytes = 0;
+};
+
+namespace ughip {
+
+// Records the thread-local message returned by ughip_last_error() and returns `code`.
+int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int device_activate(ughip_device* d);
+const char* dtype_name(int dt);
+
+}  // namespace ughip
+
+#define UGHIP_HIPCHK(expr)                                                                                 \
+  do {                                                                                                     \
+    hipError_t e_ = (expr);                                                                                \
+    if (e_ != hipSuccess) return ughip::set_error(UGHIP_ERR_HIP, "%s: %s", #expr, hipGetErrorString(e_)); \
+  } while (0)

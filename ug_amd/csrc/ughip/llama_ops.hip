@@ -1,0 +1,369 @@
+// ug-llama's five custom ops as hand-written gfx950 kernels (wave64, 128-bit accesses).
+// Semantics follow the CPU implementations in ug-llama/src/cpu_ops.rs:6-167; all f32.
+#include <hip/hip_runtime.h>
+
+#include "internal.h"
+#include "ughip.h"
+
+using namespace ughip;
+
+namespace {
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// Reduction across the NW waves of a workgroup through LDS; every thread gets the result.
+template <int NW, bool IS_MAX>
+__device__ __forceinline__ float block_reduce(float v, float* lds) {
+  v = IS_MAX ? wave_max(v) : wave_sum(v);
+  if (NW == 1) return v;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = lds[0];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) r = IS_MAX ? fmaxf(r, lds[i]) : r + lds[i];
+  return r;
+}
+
+// ---- custom_softmax (cpu_ops.rs:6-31) --------------------------------------------------------
+// One workgroup of NW waves per row; the row lives in registers (V float4 per thread), so HBM
+// sees one read and one write per element.  Requires n_cols % 4 == 0 and
+// n_cols <= NW * 64 * 4 * V.
+template <int NW, int V>
+__global__ void __launch_bounds__(NW * 64) softmax_rows_reg(const float* __restrict__ src, float* __restrict__ dst, int n_cols) {
+  __shared__ float lds[NW > 1 ? NW : 1];
+  const size_t row = blockIdx.x;
+  const float4* s4 = reinterpret_cast<const float4*>(src + row * n_cols);
+  float4* d4 = reinterpret_cast<float4*>(dst + row * n_cols);
+  const int n4 = n_cols >> 2;
+  float4 x[V];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    int c = threadIdx.x + i * NW * 64;
+    if (c < n4) {
+      x[i] = s4[c];
+      m = fmaxf(fmaxf(m, fmaxf(x[i].x, x[i].y)), fmaxf(x[i].z, x[i].w));
+    }
+  }
+  m = block_reduce<NW, true>(m, lds);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    int c = threadIdx.x + i * NW * 64;
+    if (c < n4) {
+      x[i].x = expf(x[i].x - m);
+      x[i].y = expf(x[i].y - m);
+      x[i].z = expf(x[i].z - m);
+      x[i].w = expf(x[i].w - m);
+      s += (x[i].x + x[i].y) + (x[i].z + x[i].w);
+    }
+  }
+  s = block_reduce<NW, false>(s, lds);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    int c = threadIdx.x + i * NW * 64;
+    if (c < n4) {
+      x[i].x /= s;
+      x[i].y /= s;
+      x[i].z /= s;
+      x[i].w /= s;
+      d4[c] = x[i];
+    }
+  }
+}
+
+// Wave per row for short rows (4 rows per workgroup), any n_cols <= 64 * V.
+template <int V>
+__global__ void __launch_bounds__(256) softmax_rows_wave(const float* __restrict__ src, float* __restrict__ dst, int n_rows, int n_cols) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= n_rows) return;
+  const int lane = threadIdx.x & 63;
+  const float* s = src + (size_t)row * n_cols;
+  float* d = dst + (size_t)row * n_cols;
+  float x[V];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    int c = lane + i * 64;
+    x[i] = c < n_cols ? s[c] : -INFINITY;
+    m = fmaxf(m, x[i]);
+  }
+  m = wave_max(m);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    int c = lane + i * 64;
+    x[i] = c < n_cols ? expf(x[i] - m) : 0.f;
+    sum += x[i];
+  }
+  sum = wave_sum(sum);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    int c = lane + i * 64;
+    if (c < n_cols) d[c] = x[i] / sum;
+  }
+}
+
+// Any row length: three passes over the row (the re-reads hit L2 for rows of this size).
+__global__ void __launch_bounds__(1024) softmax_rows_generic(const float* __restrict__ src, float* __restrict__ dst, int n_cols) {
+  __shared__ float lds[16];
+  const size_t row = blockIdx.x;
+  const float* s = src + row * n_cols;
+  float* d = dst + row * n_cols;
+  float m = -INFINITY;
+  for (int c = threadIdx.x; c < n_cols; c += 1024) m = fmaxf(m, s[c]);
+  m = block_reduce<16, true>(m, lds);
+  float sum = 0.f;
+  for (int c = threadIdx.x; c < n_cols; c += 1024) {
+    float e = expf(s[c] - m);
+    d[c] = e;
+    sum += e;
+  }
+  sum = block_reduce<16, false>(sum, lds);
+  for (int c = threadIdx.x; c < n_cols; c += 1024) d[c] /= sum;
+}
+
+// ---- causal_mask (cpu_ops.rs:33-56) --------------------------------------------------------------
+// dst[b, i1, i2] = i2 <= i1 ? src : -inf.  Fully masked float4s never touch src.
+__global__ void __launch_bounds__(256) causal_mask_v4(const float* __restrict__ src, float* __restrict__ dst, size_t n4, int s1, int s2) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n4) return;
+  const int s2q = s2 >> 2;
+  const int i2 = (int)(g % s2q) << 2;
+  const int i1 = (int)((g / s2q) % s1);
+  float4 v;
+  if (i2 > i1) {
+    v = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+  } else {
+    v = reinterpret_cast<const float4*>(src)[g];
+    if (i2 + 1 > i1) v.y = -INFINITY;
+    if (i2 + 2 > i1) v.z = -INFINITY;
+    if (i2 + 3 > i1) v.w = -INFINITY;
+  }
+  reinterpret_cast<float4*>(dst)[g] = v;
+}
+
+__global__ void __launch_bounds__(256) causal_mask_scalar(const float* __restrict__ src, float* __restrict__ dst, size_t n, int s1, int s2) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n) return;
+  const int i2 = (int)(g % s2);
+  const int i1 = (int)((g / s2) % s1);
+  dst[g] = i2 <= i1 ? src[g] : -INFINITY;
+}
+
+// ---- rope (cpu_ops.rs:91-126) and rope_i (cpu_ops.rs:58-89) -------------------------------------------
+// src/dst are [bh, t, d]; the tables are read at row pos[0] + i_t.  A position that would run
+// past the table poisons the output with NaN instead of faulting.
+template <int W>  // pairs per thread: 4 (float4 path) or 1
+__global__ void __launch_bounds__(256) rope_kernel(const float* __restrict__ src, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                   const int* __restrict__ pos, float* __restrict__ dst, size_t n_groups, int t, int d,
+                                                   size_t table_len) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n_groups) return;
+  const int h = d >> 1;
+  const int hq = h / W;
+  const int i_d = (int)(g % hq) * W;
+  const size_t bt = g / hq;  // flat (bh, t)
+  const int i_t = (int)(bt % t);
+  const long long p = pos[0];
+  const size_t i1 = bt * d + i_d;
+  const size_t i2 = i1 + h;
+  const size_t ics = ((size_t)p + i_t) * h + i_d;
+  const bool ok = p >= 0 && ics + W <= table_len;
+  if (W == 4) {
+    float4 x1 = *reinterpret_cast<const float4*>(src + i1);
+    float4 x2 = *reinterpret_cast<const float4*>(src + i2);
+    float4 c, s;
+    if (ok) {
+      c = *reinterpret_cast<const float4*>(cos_t + ics);
+      s = *reinterpret_cast<const float4*>(sin_t + ics);
+    } else {
+      c = s = make_float4(NAN, NAN, NAN, NAN);
+    }
+    float4 o1 = make_float4(x1.x * c.x - x2.x * s.x, x1.y * c.y - x2.y * s.y, x1.z * c.z - x2.z * s.z, x1.w * c.w - x2.w * s.w);
+    float4 o2 = make_float4(x1.x * s.x + x2.x * c.x, x1.y * s.y + x2.y * c.y, x1.z * s.z + x2.z * c.z, x1.w * s.w + x2.w * c.w);
+    *reinterpret_cast<float4*>(dst + i1) = o1;
+    *reinterpret_cast<float4*>(dst + i2) = o2;
+  } else {
+    float x1 = src[i1], x2 = src[i2];
+    float c = ok ? cos_t[ics] : NAN, s = ok ? sin_t[ics] : NAN;
+    dst[i1] = x1 * c - x2 * s;
+    dst[i2] = x1 * s + x2 * c;
+  }
+}
+
+template <int W>  // pairs per thread: 2 (float4 path) or 1
+__global__ void __launch_bounds__(256) rope_i_kernel(const float* __restrict__ src, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                     const int* __restrict__ pos, float* __restrict__ dst, size_t n_groups, int t, int d,
+                                                     size_t table_len) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n_groups) return;
+  const int h = d >> 1;
+  const size_t pair = g * W;             // flat pair index over [bh, t, d/2]
+  const size_t chunk = (size_t)t * h;    // pairs per bh
+  const size_t in_chunk = pair % chunk;  // == i_t * (d/2) + i_d  (cpu_ops.rs:74-80)
+  const long long p = pos[0];
+  const size_t ics = (size_t)p * h + in_chunk;
+  const bool ok = p >= 0 && ics + W <= table_len;
+  if (W == 2) {
+    float4 x = reinterpret_cast<const float4*>(src)[g];
+    float2 c, s;
+    if (ok) {
+      c = *reinterpret_cast<const float2*>(cos_t + ics);
+      s = *reinterpret_cast<const float2*>(sin_t + ics);
+    } else {
+      c = s = make_float2(NAN, NAN);
+    }
+    float4 o = make_float4(x.x * c.x - x.y * s.x, x.x * s.x + x.y * c.x, x.z * c.y - x.w * s.y, x.z * s.y + x.w * c.y);
+    reinterpret_cast<float4*>(dst)[g] = o;
+  } else {
+    float a = src[2 * pair], b = src[2 * pair + 1];
+    float c = ok ? cos_t[ics] : NAN, s = ok ? sin_t[ics] : NAN;
+    dst[2 * pair] = a * c - b * s;
+    dst[2 * pair + 1] = a * s + b * c;
+  }
+}
+
+// ---- cat (cpu_ops.rs:128-167) ----------------------------------------------------------------------------
+template <typename VT, int W>
+__global__ void __launch_bounds__(256) cat_kernel(const float* __restrict__ lhs, const float* __restrict__ rhs, float* __restrict__ dst, size_t n_groups,
+                                                  size_t d2_l, size_t d2_r) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n_groups) return;
+  const size_t d2 = (d2_l + d2_r) / W;
+  const size_t i1 = g / d2;
+  const size_t j = (g % d2) * W;
+  const float* s = j < d2_l ? lhs + i1 * d2_l + j : rhs + i1 * d2_r + (j - d2_l);
+  reinterpret_cast<VT*>(dst)[g] = *reinterpret_cast<const VT*>(s);
+}
+
+int check_f32(const ughip_slice* s, size_t need, const char* what) {
+  if (!s) return set_error(UGHIP_ERR_INVALID, "%s: null slice", what);
+  if (s->dtype != UGHIP_F32) return set_error(UGHIP_ERR_INVALID, "%s: unexpected dtype %s, expected F32", what, dtype_name(s->dtype));
+  if (s->len < need) return set_error(UGHIP_ERR_BOUNDS, "%s: slice has %zu elements, op needs %zu", what, s->len, need);
+  return UGHIP_OK;
+}
+
+unsigned blocks_for(size_t n, unsigned per_block) { return (unsigned)((n + per_block - 1) / per_block); }
+
+}  // namespace
+
+extern "C" {
+
+int ughip_softmax_rows(ughip_device* dev, const ughip_slice* src, ughip_slice* dst, size_t n_rows, size_t n_cols) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  if (int rc = check_f32(src, n_rows * n_cols, "softmax src")) return rc;
+  if (int rc = check_f32(dst, n_rows * n_cols, "softmax dst")) return rc;
+  if (src == dst) return set_error(UGHIP_ERR_INVALID, "softmax: src and dst alias");
+  if (n_rows == 0 || n_cols == 0) return UGHIP_OK;
+  if (n_rows > 0x7fffffffull || n_cols > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "softmax: shape too large");
+  if (int rc = device_activate(dev)) return rc;
+  const float* s = static_cast<const float*>(src->ptr);
+  float* d = static_cast<float*>(dst->ptr);
+  hipStream_t st = dev->stream;
+  const int nc = (int)n_cols, nr = (int)n_rows;
+  if (n_cols <= 256) {
+    softmax_rows_wave<4><<<blocks_for(n_rows, 4), 256, 0, st>>>(s, d, nr, nc);
+  } else if (n_cols % 4 != 0 || n_cols > 16384) {
+    softmax_rows_generic<<<nr, 1024, 0, st>>>(s, d, nc);
+  } else if (n_cols <= 1024) {
+    softmax_rows_reg<4, 1><<<nr, 256, 0, st>>>(s, d, nc);
+  } else if (n_cols <= 2048) {
+    softmax_rows_reg<4, 2><<<nr, 256, 0, st>>>(s, d, nc);
+  } else if (n_cols <= 4096) {
+    softmax_rows_reg<8, 2><<<nr, 512, 0, st>>>(s, d, nc);
+  } else if (n_cols <= 8192) {
+    softmax_rows_reg<16, 2><<<nr, 1024, 0, st>>>(s, d, nc);
+  } else {
+    softmax_rows_reg<16, 4><<<nr, 1024, 0, st>>>(s, d, nc);
+  }
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+int ughip_causal_mask(ughip_device* dev, const ughip_slice* src, ughip_slice* dst, size_t bh, size_t s1, size_t s2) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  const size_t n = bh * s1 * s2;
+  if (int rc = check_f32(src, n, "causal_mask src")) return rc;
+  if (int rc = check_f32(dst, n, "causal_mask dst")) return rc;
+  if (src == dst) return set_error(UGHIP_ERR_INVALID, "causal_mask: src and dst alias");
+  if (n == 0) return UGHIP_OK;
+  if (s1 > 0x7fffffffull || s2 > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "causal_mask: shape too large");
+  if (int rc = device_activate(dev)) return rc;
+  const float* s = static_cast<const float*>(src->ptr);
+  float* d = static_cast<float*>(dst->ptr);
+  if (s2 % 4 == 0)
+    causal_mask_v4<<<blocks_for(n / 4, 256), 256, 0, dev->stream>>>(s, d, n / 4, (int)s1, (int)s2);
+  else
+    causal_mask_scalar<<<blocks_for(n, 256), 256, 0, dev->stream>>>(s, d, n, (int)s1, (int)s2);
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+int ughip_rope(ughip_device* dev, const ughip_slice* src, const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos,
+               ughip_slice* dst, size_t bh, size_t t, size_t d, int interleaved) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  const size_t n = bh * t * d;
+  if (d % 2 != 0) return set_error(UGHIP_ERR_INVALID, "rope: head dim %zu is odd", d);
+  if (int rc = check_f32(src, n, "rope src")) return rc;
+  if (int rc = check_f32(dst, n, "rope dst")) return rc;
+  if (int rc = check_f32(cos, t * d / 2, "rope cos")) return rc;
+  if (int rc = check_f32(sin, t * d / 2, "rope sin")) return rc;
+  if (!pos || pos->dtype != UGHIP_I32 || pos->len < 1) return set_error(UGHIP_ERR_INVALID, "rope: pos must be a non-empty I32 slice");
+  if (src == dst) return set_error(UGHIP_ERR_INVALID, "rope: src and dst alias");
+  if (n == 0) return UGHIP_OK;
+  if (t > 0x7fffffffull || d > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "rope: shape too large");
+  if (int rc = device_activate(dev)) return rc;
+  const float* s = static_cast<const float*>(src->ptr);
+  const float* c = static_cast<const float*>(cos->ptr);
+  const float* sn = static_cast<const float*>(sin->ptr);
+  const int* p = static_cast<const int*>(pos->ptr);
+  float* o = static_cast<float*>(dst->ptr);
+  const size_t table_len = cos->len < sin->len ? cos->len : sin->len;
+  const size_t pairs = n / 2;
+  if (!interleaved) {
+    if ((d / 2) % 4 == 0)
+      rope_kernel<4><<<blocks_for(pairs / 4, 256), 256, 0, dev->stream>>>(s, c, sn, p, o, pairs / 4, (int)t, (int)d, table_len);
+    else
+      rope_kernel<1><<<blocks_for(pairs, 256), 256, 0, dev->stream>>>(s, c, sn, p, o, pairs, (int)t, (int)d, table_len);
+  } else {
+    if ((d / 2) % 2 == 0)
+      rope_i_kernel<2><<<blocks_for(pairs / 2, 256), 256, 0, dev->stream>>>(s, c, sn, p, o, pairs / 2, (int)t, (int)d, table_len);
+    else
+      rope_i_kernel<1><<<blocks_for(pairs, 256), 256, 0, dev->stream>>>(s, c, sn, p, o, pairs, (int)t, (int)d, table_len);
+  }
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+int ughip_cat(ughip_device* dev, const ughip_slice* lhs, const ughip_slice* rhs, ughip_slice* dst, size_t d1, size_t d2_l, size_t d2_r) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  if (int rc = check_f32(lhs, d1 * d2_l, "cat lhs")) return rc;
+  if (int rc = check_f32(rhs, d1 * d2_r, "cat rhs")) return rc;
+  const size_t n = d1 * (d2_l + d2_r);
+  if (int rc = check_f32(dst, n, "cat dst")) return rc;
+  if (dst == lhs || dst == rhs) return set_error(UGHIP_ERR_INVALID, "cat: dst aliases an input");
+  if (n == 0) return UGHIP_OK;
+  if (int rc = device_activate(dev)) return rc;
+  const float* l = static_cast<const float*>(lhs->ptr);
+  const float* r = static_cast<const float*>(rhs->ptr);
+  float* o = static_cast<float*>(dst->ptr);
+  if (d2_l % 4 == 0 && d2_r % 4 == 0)
+    cat_kernel<float4, 4><<<blocks_for(n / 4, 256), 256, 0, dev->stream>>>(l, r, o, n / 4, d2_l, d2_r);
+  else
+    cat_kernel<float, 1><<<blocks_for(n, 256), 256, 0, dev->stream>>>(l, r, o, n, d2_l, d2_r);
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,32 @@
+// SSA -> HIP lowering for gfx950.  Pure host code: no HIP runtime calls, so it can be
+// exercised without a GPU.
+#pragma once
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "ughip.h"
+
+namespace ughip {
+
+struct Lowered {
+  std::string source;  // complete translation unit handed to hiprtc
+  std::string entry;   // extern "C" kernel symbol
+  int strategy = UGHIP_STRAT_LITERAL;
+  unsigned grid = 1, block = 1, lds_bytes = 0;
+  // Device scratch the kernel takes as two trailing pointer arguments (partials, counters).
+  // Zero-initialised once when the func is created; the kernel restores the zeros itself.
+  size_t scratch_part_bytes = 0, scratch_cnt_bytes = 0;
+  std::vector<int> arg_dtype;      // per kernel argument, UGHIP_* dtype
+  std::vector<long long> min_len;  // per argument: 1 + largest offset the kernel forms, -1 if unknown
+  std::vector<char> arg_written;   // per argument: has a Store
+  bool empty_launch = false;       // a loop of the nest has zero trips: nothing to run
+};
+
+// Throws std::runtime_error on malformed SSA.
+Lowered lower_ssa(const ughip_ssa& ssa, const std::string& entry);
+
+const char* dtype_c_name(int dtype);
+size_t dtype_size(int dtype);
+
+}  // namespace ughip

@@ -1,0 +1,289 @@
+// Device::matmul for gfx950: MFMA kernels with f32 accumulation (f32 via v_mfma_f32_32x32x2_f32,
+// bf16 via v_mfma_f32_32x32x16_bf16), plus a bandwidth-bound GEMV for the m <= 8 rows of decode.
+// dst[b,m,n] = lhs[b,m,k] x rhs[b,k,n], beta = 0 (ug-core/src/lib.rs:62-70; stride rules follow
+// ug-core/src/cpu_runtime.rs:527-619).
+#include <hip/hip_runtime.h>
+
+#include "internal.h"
+#include "ughip.h"
+
+using namespace ughip;
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+struct MMArgs {
+  const void* a;
+  const void* b;
+  void* c;
+  int M, N, K;
+  long long a_rs, a_cs;  // lhs strides of (m, k)
+  long long b_rs, b_cs;  // rhs strides of (k, n)
+  long long a_bs, b_bs, c_bs;
+};
+
+// MFMA 32x32 accumulator layout: lane l, register i -> row (i/4)*8 + (l/32)*4 + i%4, col l%32.
+template <typename T>
+__device__ __forceinline__ void store_acc(T* __restrict__ C, const floatx16& acc, int row0, int col, int M, int N, int lane) {
+  if (col >= N) return;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    int row = row0 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+    if (row < M) C[(size_t)row * N + col] = (T)acc[i];
+  }
+}
+
+// ---- any shape, any strides: 64x64 tile per workgroup, one 32x32 MFMA tile per wave ----------------
+__global__ void __launch_bounds__(256) gemm_f32_any(MMArgs p) {
+  __shared__ float As[64][17];  // [m][k], odd stride: conflict-free column reads
+  __shared__ float Bs[16][65];  // [k][n]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const float* __restrict__ A = static_cast<const float*>(p.a) + (size_t)blockIdx.z * p.a_bs;
+  const float* __restrict__ B = static_cast<const float*>(p.b) + (size_t)blockIdx.z * p.b_bs;
+  float* __restrict__ C = static_cast<float*>(p.c) + (size_t)blockIdx.z * p.c_bs;
+  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+  floatx16 acc = {0};
+  for (int k0 = 0; k0 < p.K; k0 += 16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int e = tid + i * 256, r, k;
+      if (p.a_cs == 1) {
+        r = e >> 4;
+        k = e & 15;
+      } else {
+        r = e & 63;
+        k = e >> 6;
+      }
+      As[r][k] = (m0 + r < p.M && k0 + k < p.K) ? A[(long long)(m0 + r) * p.a_rs + (long long)(k0 + k) * p.a_cs] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int e = tid + i * 256, k, n;
+      if (p.b_cs == 1) {
+        k = e >> 6;
+        n = e & 63;
+      } else {
+        k = e & 15;
+        n = e >> 4;
+      }
+      Bs[k][n] = (k0 + k < p.K && n0 + n < p.N) ? B[(long long)(k0 + k) * p.b_rs + (long long)(n0 + n) * p.b_cs] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; kk += 2) {
+      float a = As[wm + (lane & 31)][kk + (lane >> 5)];
+      float b = Bs[kk + (lane >> 5)][wn + (lane & 31)];
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  store_acc(C, acc, m0 + wm, n0 + wn + (lane & 31), p.M, p.N, lane);
+}
+
+__global__ void __launch_bounds__(256) gemm_bf16_any(MMArgs p) {
+  __shared__ __attribute__((aligned(16))) __bf16 As[64][40];  // [m][k], 80-byte rows: conflict-free b128 reads
+  __shared__ __attribute__((aligned(16))) __bf16 Bs[64][40];  // [n][k]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  const __bf16* __restrict__ A = static_cast<const __bf16*>(p.a) + (size_t)blockIdx.z * p.a_bs;
+  const __bf16* __restrict__ B = static_cast<const __bf16*>(p.b) + (size_t)blockIdx.z * p.b_bs;
+  __bf16* __restrict__ C = static_cast<__bf16*>(p.c) + (size_t)blockIdx.z * p.c_bs;
+  const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+  floatx16 acc = {0};
+  for (int k0 = 0; k0 < p.K; k0 += 32) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int e = tid + i * 256, r, k;
+      if (p.a_cs == 1) {
+        r = e >> 5;
+        k = e & 31;
+      } else {
+        r = e & 63;
+        k = e >> 6;
+      }
+      As[r][k] = (m0 + r < p.M && k0 + k < p.K) ? A[(long long)(m0 + r) * p.a_rs + (long long)(k0 + k) * p.a_cs] : (__bf16)0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int e = tid + i * 256, k, n;
+      if (p.b_cs == 1) {
+        k = e >> 6;
+        n = e & 63;
+      } else {
+        k = e & 31;
+        n = e >> 5;
+      }
+      Bs[n][k] = (k0 + k < p.K && n0 + n < p.N) ? B[(long long)(k0 + k) * p.b_rs + (long long)(n0 + n) * p.b_cs] : (__bf16)0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 32; kk += 16) {
+      bf16x8 a = *reinterpret_cast<const bf16x8*>(&As[wm + (lane & 31)][kk + (lane >> 5) * 8]);
+      bf16x8 b = *reinterpret_cast<const bf16x8*>(&Bs[wn + (lane & 31)][kk + (lane >> 5) * 8]);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  store_acc(C, acc, m0 + wm, n0 + wn + (lane & 31), p.M, p.N, lane);
+}
+
+// ---- GEMV for decode: y[r, n] = sum_k x[r, k] * W[n, k], rows r < R <= 8 --------------------------------
+// One wave per output column; K is walked with 128-bit loads by the 64 lanes, so W is streamed
+// from HBM exactly once and x comes from L2.  Needs x and W contiguous along k and K % VEC == 0.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+template <int R>
+__global__ void __launch_bounds__(256) gemv_nt_f32(MMArgs p) {
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= p.N) return;
+  const float* __restrict__ X = static_cast<const float*>(p.a) + (size_t)blockIdx.z * p.a_bs;
+  const float* __restrict__ W = static_cast<const float*>(p.b) + (size_t)blockIdx.z * p.b_bs + (size_t)n * p.b_cs;
+  float* __restrict__ Y = static_cast<float*>(p.c) + (size_t)blockIdx.z * p.c_bs;
+  float acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = 0.f;
+  for (int k = lane * 4; k < p.K; k += 256) {
+    const float4 w = *reinterpret_cast<const float4*>(W + k);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (r < p.M) {
+        const float4 x = *reinterpret_cast<const float4*>(X + (size_t)r * p.a_rs + k);
+        acc[r] += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float s = wave_sum(acc[r]);
+    if (lane == 0 && r < p.M) Y[(size_t)r * p.N + n] = s;
+  }
+}
+
+template <int R>
+__global__ void __launch_bounds__(256) gemv_nt_bf16(MMArgs p) {
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= p.N) return;
+  const __bf16* __restrict__ X = static_cast<const __bf16*>(p.a) + (size_t)blockIdx.z * p.a_bs;
+  const __bf16* __restrict__ W = static_cast<const __bf16*>(p.b) + (size_t)blockIdx.z * p.b_bs + (size_t)n * p.b_cs;
+  __bf16* __restrict__ Y = static_cast<__bf16*>(p.c) + (size_t)blockIdx.z * p.c_bs;
+  float acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = 0.f;
+  for (int k = lane * 8; k < p.K; k += 512) {
+    const bf16x8 w = *reinterpret_cast<const bf16x8*>(W + k);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (r < p.M) {
+        const bf16x8 x = *reinterpret_cast<const bf16x8*>(X + (size_t)r * p.a_rs + k);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[r] += (float)w[j] * (float)x[j];
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float s = wave_sum(acc[r]);
+    if (lane == 0 && r < p.M) Y[(size_t)r * p.N + n] = (__bf16)s;
+  }
+}
+
+// Batch stride of one operand: cpu_runtime.rs:527-549 / ug-cuda/src/gemm.rs:59-74.
+bool batch_stride(size_t rank, const size_t* dims, const size_t* strides, size_t dflt, long long* out) {
+  if (rank == 2) {
+    *out = (long long)dflt;
+    return true;
+  }
+  if (rank == 3) {
+    *out = (long long)strides[0];
+    return true;
+  }
+  size_t s1 = strides[0], s2 = strides[1];
+  if (s1 == s2 * dims[1]) {
+    *out = (long long)s2;
+    return true;
+  }
+  if (dims[0] == 1) {
+    *out = (long long)s2;
+    return true;
+  }
+  if (dims[1] == 1) {
+    *out = (long long)s1;
+    return true;
+  }
+  return false;
+}
+
+}  // namespace
+
+extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs, const ughip_slice* rhs, size_t b, size_t m, size_t n,
+                            size_t k, size_t rank, const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset, const size_t* rhs_dims,
+                            const size_t* rhs_strides, size_t rhs_offset) {
+  if (!dev || !dst || !lhs || !rhs) return set_error(UGHIP_ERR_INVALID, "matmul: null argument");
+  if (rank < 2 || rank > 4 || !lhs_dims || !lhs_strides || !rhs_dims || !rhs_strides)
+    return set_error(UGHIP_ERR_INVALID, "matmul: rank %zu layouts are not supported", rank);
+  if (dst->dtype != lhs->dtype || dst->dtype != rhs->dtype || (dst->dtype != UGHIP_F32 && dst->dtype != UGHIP_BF16)) {
+    int code = (dst->dtype == lhs->dtype && dst->dtype == rhs->dtype) ? UGHIP_ERR_UNSUPPORTED : UGHIP_ERR_INVALID;
+    return set_error(code, "incorrect dtypes for matmul, dst: %s, lhs: %s, rhs: %s", dtype_name(dst->dtype), dtype_name(lhs->dtype),
+                     dtype_name(rhs->dtype));
+  }
+  if (dst == lhs || dst == rhs) return set_error(UGHIP_ERR_INVALID, "matmul: dst aliases an operand (already borrowed)");
+  if (b > 65535 || m > 0x7fffffffull || n > 0x7fffffffull || k > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "matmul: shape too large");
+  MMArgs p;
+  p.M = (int)m;
+  p.N = (int)n;
+  p.K = (int)k;
+  p.a_rs = (long long)lhs_strides[rank - 2];
+  p.a_cs = (long long)lhs_strides[rank - 1];
+  p.b_rs = (long long)rhs_strides[rank - 2];
+  p.b_cs = (long long)rhs_strides[rank - 1];
+  if (!batch_stride(rank, lhs_dims, lhs_strides, m * k, &p.a_bs)) return set_error(UGHIP_ERR_STRIDING, "matmul: non-contiguous lhs batch strides");
+  if (!batch_stride(rank, rhs_dims, rhs_strides, n * k, &p.b_bs)) return set_error(UGHIP_ERR_STRIDING, "matmul: non-contiguous rhs batch strides");
+  p.c_bs = (long long)(m * n);
+  if (dst->len < b * m * n) return set_error(UGHIP_ERR_BOUNDS, "matmul: dst has %zu elements, needs %zu", dst->len, b * m * n);
+  if (b == 0 || m == 0 || n == 0) return UGHIP_OK;
+  // Furthest element each operand can touch.
+  size_t a_max = lhs_offset + (b - 1) * (size_t)p.a_bs + (m - 1) * (size_t)p.a_rs + (k ? (k - 1) * (size_t)p.a_cs : 0);
+  size_t b_max = rhs_offset + (b - 1) * (size_t)p.b_bs + (n - 1) * (size_t)p.b_cs + (k ? (k - 1) * (size_t)p.b_rs : 0);
+  if (k && (a_max >= lhs->len || b_max >= rhs->len))
+    return set_error(UGHIP_ERR_BOUNDS, "matmul: operand too short for its layout (lhs %zu/%zu, rhs %zu/%zu)", a_max, lhs->len, b_max, rhs->len);
+  if (int rc = device_activate(dev)) return rc;
+  const size_t esz = dst->dtype == UGHIP_F32 ? 4 : 2;
+  p.a = static_cast<const char*>(lhs->ptr) + lhs_offset * esz;
+  p.b = static_cast<const char*>(rhs->ptr) + rhs_offset * esz;
+  p.c = dst->ptr;
+  const bool f32 = dst->dtype == UGHIP_F32;
+  hipStream_t st = dev->stream;
+  const size_t vec = f32 ? 4 : 8;
+  const bool gemv_ok = m <= 8 && k >= 256 && k % vec == 0 && p.a_cs == 1 && p.b_rs == 1 && p.a_rs % (long long)vec == 0 && p.b_cs % (long long)vec == 0 &&
+                       p.a_bs % (long long)vec == 0 && p.b_bs % (long long)vec == 0 && lhs_offset % vec == 0 && rhs_offset % vec == 0;
+  if (gemv_ok) {
+    dim3 grid((unsigned)((n + 3) / 4), 1, (unsigned)b);
+    if (f32) {
+      if (m == 1) gemv_nt_f32<1><<<grid, 256, 0, st>>>(p);
+      else if (m <= 4) gemv_nt_f32<4><<<grid, 256, 0, st>>>(p);
+      else gemv_nt_f32<8><<<grid, 256, 0, st>>>(p);
+    } else {
+      if (m == 1) gemv_nt_bf16<1><<<grid, 256, 0, st>>>(p);
+      else if (m <= 4) gemv_nt_bf16<4><<<grid, 256, 0, st>>>(p);
+      else gemv_nt_bf16<8><<<grid, 256, 0, st>>>(p);
+    }
+  } else {
+    dim3 grid((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64), (unsigned)b);
+    if (grid.y > 65535) return set_error(UGHIP_ERR_INVALID, "matmul: m too large for this kernel");
+    if (f32) gemm_f32_any<<<grid, 256, 0, st>>>(p);
+    else gemm_bf16_any<<<grid, 256, 0, st>>>(p);
+  }
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
