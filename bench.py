@@ -1,0 +1,213 @@
+#!/usr/bin/env python3
+"""Benchmark of the ug HIP backend on one MI355X.
+
+Headline (the JSON line): BASELINE config 2 -- sum(a*b + 0.5*a) over two f32 vectors of length
+2^24, built as one lazy graph, scheduled and lowered like ug does, run on the HIP device.  A "step"
+is one run of the compiled schedule (one kernel launch) with a and b resident in HBM.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--extras] [--llama]
+
+--extras adds the other single-GPU configs (softmax sweep, batched matmul, llama pieces) under
+"extras"; --llama adds the config-5 decode run.  Only one GPU is ever used.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, vendor figure
+MFMA_BF16_PEAK_TF = 2500.0      # dense bf16
+MFMA_F32_PEAK_TF = 157.3        # f32 matrix
+N = 1 << 24
+ALGO_BYTES = 2 * N * 4 + 4      # read a, read b, write one f32
+
+# HBM bytes per launch of the dominant kernel from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`,
+# scaled by a plain copy kernel of known size (see profiles/); None until measured.
+TRAFFIC_BYTES = None
+
+
+def hip_events(dev):
+    import ug_amd
+    lib = ug_amd.ughip_lib()
+    raw = C.c_void_p(dev.raw_hip())
+    evs = []
+    for _ in range(2):
+        e = C.c_void_p()
+        assert lib.ughip_event_create(raw, C.byref(e)) == 0, lib.ughip_last_error()
+        evs.append(e)
+    return lib, evs
+
+
+def timed(dev, fn, steps, warmup):
+    """(wall seconds, HIP-event milliseconds) for `steps` calls of fn after `warmup` calls."""
+    lib, (e0, e1) = hip_events(dev)
+    for _ in range(warmup):
+        fn()
+    dev.synchronize()
+    t0 = time.perf_counter()
+    lib.ughip_event_record(e0)
+    for _ in range(steps):
+        fn()
+    lib.ughip_event_record(e1)
+    dev.synchronize()
+    wall = time.perf_counter() - t0
+    ms = C.c_float()
+    assert lib.ughip_event_elapsed_ms(e0, e1, C.byref(ms)) == 0, lib.ughip_last_error()
+    lib.ughip_event_destroy(e0)
+    lib.ughip_event_destroy(e1)
+    return wall, float(ms.value)
+
+
+def fused_reduce(dev, a, b):
+    import ref_suite
+    from ug_amd import LazyBuffer as LB, Schedule
+    la, lb = LB.copy(a, (a.size,), dev), LB.copy(b, (b.size,), dev)
+    r = ref_suite.fused_reduce_graph(la, lb, dev)
+    cs = Schedule.create_one(r).compile()
+    return r, cs, (la, lb)
+
+
+def cpu_baseline(a, b, truth, budget_s=12.0):
+    """The CPU oracle (restatement of ug's CPU backend: same emitted C, same gcc flags, one thread)
+    on the same workload, timed on this box's host cores."""
+    from conftest import _oracle_lib
+    import ug_amd
+    lib = _oracle_lib()
+    out = C.c_void_p()
+    assert lib.ugo_cpu_device_new(C.byref(out)) == 0
+    cpu = ug_amd.Device(out.value)
+    r, cs, keep = fused_reduce(cpu, a, b)
+    cs.run()
+    val = float(r.data_vec()[0])
+    assert abs(val - truth) <= 1e-3 * abs(truth) + 1.0, (val, truth)
+    passes, t0 = 0, time.perf_counter()
+    while True:
+        cs.run()
+        passes += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or passes >= 2000:
+            break
+    return {"value": round(ALGO_BYTES * passes / el / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{passes} passes of the full 2^24-element workload in {el:.1f} s (oracle/: C emitted as ug-core/src/cpu_code_gen.rs does, "
+                      "gcc -O3 -march=native -ffast-math, single thread like the reference)",
+            "host_cpus": os.cpu_count()}
+
+
+def extras(dev, steps, warmup):
+    """Other single-GPU configs of BASELINE.json: GB/s or TFLOP/s with the roofline fraction."""
+    import ug_amd
+    from ug_amd import LazyBuffer as LB, Schedule, rng
+    out = {}
+    # config 1 and the reference's own sweep (ug-cuda/examples/benchmark.rs:110): 8 B per element
+    for rows, cols in [(32, 1024)] + [(4096, c) for c in (128, 256, 512, 768, 1024, 1536, 2048, 3072, 4096)]:
+        x = rng.normal(1, rows * cols, 3.0)
+        src = LB.copy(x, (rows, cols), dev)
+        sm = ug_amd.llama.softmax(src)
+        cs = Schedule.create_one(sm).compile()
+        _, ms = timed(dev, cs.run, steps, warmup)
+        gbs = 8.0 * rows * cols * steps / (ms * 1e-3) / 1e9
+        out[f"softmax_lazy_{rows}x{cols}"] = {"GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "us_per_softmax": round(ms * 1e3 / steps, 2),
+                                             "launches": 2}
+        ops = ug_amd.LlamaOps.hip()
+        cm = ops.custom_softmax(src)
+        cs2 = Schedule.create_one(cm).compile()
+        _, ms = timed(dev, cs2.run, steps, warmup)
+        gbs = 8.0 * rows * cols * steps / (ms * 1e-3) / 1e9
+        out[f"softmax_custom_{rows}x{cols}"] = {"GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "us_per_softmax": round(ms * 1e3 / steps, 2),
+                                               "launches": 1}
+    # config 3: batched matmul 8 x 1024^3
+    b, m = 8, 1024
+    flop = 2.0 * b * m * m * m
+    a = rng.uniform_pm1(4, b * m * m)
+    w = rng.uniform_pm1(5, b * m * m)
+    la, lw = LB.copy(a, (b, m, m), dev), LB.copy(w, (b, m, m), dev)
+    mm = la.matmul(lw)
+    cs = Schedule.create_one(mm).compile()
+    _, ms = timed(dev, cs.run, steps, warmup)
+    tf = flop * steps / (ms * 1e-3) / 1e12
+    out["bmm_f32_8x1024^3"] = {"TFLOP/s": round(tf, 2), "frac_mfma_f32": round(tf / MFMA_F32_PEAK_TF, 4), "us": round(ms * 1e3 / steps, 1)}
+    sa, sw = dev.slice_from(rng.to_bf16_bits(a)), dev.slice_from(rng.to_bf16_bits(w))
+    dst = dev.allocate_uninit(ug_amd.BF16, b * m * m)
+    lay = ((b, m, m), (m * m, m, 1), 0)
+    _, ms = timed(dev, lambda: dev.matmul(dst, sa, sw, (b, m, m, m), lay, lay), steps, warmup)
+    tf = flop * steps / (ms * 1e-3) / 1e12
+    out["bmm_bf16_8x1024^3"] = {"TFLOP/s": round(tf, 2), "frac_mfma_bf16": round(tf / MFMA_BF16_PEAK_TF, 4), "us": round(ms * 1e3 / steps, 1)}
+    return out
+
+
+def llama_decode(dev, n_prompt=128, n_steps=128):
+    import ug_amd
+    from ug_amd import rng
+    cfg = ug_amd.LlamaConfig()
+    ops = ug_amd.LlamaOps.hip()
+    t0 = time.perf_counter()
+    model = ug_amd.LlamaModel(dev, ops, cfg, custom_softmax=True, seed=9, std=0.02)
+    load_s = time.perf_counter() - t0
+    prompt = rng.token_ids(10, n_prompt, cfg.vocab_size)
+    toks, st = model.generate(prompt, n_steps)
+    weights_bytes = 4 * 1034512384
+    tok_s = n_steps / (st["decode_ms"] * 1e-3)
+    return {"tok/s": round(tok_s, 2), "decode_ms_per_token": round(st["decode_ms"] / n_steps, 3), "prefill_ms": round(st["prefill_ms"], 1),
+            "frac_hbm_weights_only": round(tok_s * weights_bytes / 1e9 / HBM_PEAK_GBS, 4), "load_s": round(load_s, 1), "dtype": "f32",
+            "first_ids": toks[:8].tolist(), "min_top1_margin": float(st["margins"].min())}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--extras", action="store_true")
+    ap.add_argument("--llama", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on one GPU only (nothing in the path is sharded); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import ug_amd
+    from ug_amd import rng
+    dev = ug_amd.hip_device(0)
+    a, b = rng.uniform_pm1(2, N), rng.uniform_pm1(3, N)
+    truth = float(np.sum(a.astype(np.float64) * b + 0.5 * a.astype(np.float64)))
+    r, cs, keep = fused_reduce(dev, a, b)
+    cs.run()
+    got = float(r.data_vec()[0])
+    if not abs(got - truth) <= 1e-5 * abs(truth) + 1e-2:
+        raise SystemExit(f"bench.py: wrong result {got} vs {truth}")
+    info = cs.funcs()[0]["info"]
+
+    wall, ev_ms = timed(dev, cs.run, args.steps, args.warmup)
+    ms_per_step = wall * 1e3 / args.steps
+    value = ALGO_BYTES * args.steps / wall / 1e9
+    achieved = ALGO_BYTES / (ev_ms * 1e-3 / args.steps) / 1e9
+
+    line = {
+        "metric": "GB/s (reductions) vs HBM roofline", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "fused elementwise+reduce sum(a*b + 0.5*a), f32, len 2^24, U(-1,1) seeds 2/3, one lazy graph ending in narrow(0,0,1)",
+                   "algorithmic_bytes_per_step": ALGO_BYTES, "kernel": info},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": TRAFFIC_BYTES, "kernel_us": round(ev_ms * 1e3 / args.steps, 3)},
+        "result": got, "truth_f64": truth,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(a, b, truth)
+    if args.extras:
+        line["extras"] = extras(dev, max(20, args.steps // 4), args.warmup)
+    if args.llama:
+        line.setdefault("extras", {})["llama_decode_f32"] = llama_decode(dev)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,200 @@
+"""Lazy-graph cases shared by the CPU-side lowering tests and the GPU parity tests.  Each case builds
+its graph on the device it is given, from seeded inputs, and says how the result is compared with
+the CPU oracle: "exact" for copies / integer work, or the relative tolerance for f32 arithmetic."""
+import numpy as np
+
+import ug_amd
+from ug_amd import F32, I32, LazyBuffer as LB, rng
+
+L = ug_amd.llama
+
+
+def _n(seed, shape, std=1.0):
+    return rng.normal(seed, int(np.prod(shape)), std)
+
+
+def _u(seed, shape):
+    return rng.uniform_pm1(seed, int(np.prod(shape)))
+
+
+def softmax(shape, seed=1, std=3.0):
+    def build(dev):
+        return L.softmax(LB.copy(_n(seed, shape, std), shape, dev))
+    return build
+
+
+def reduce_dim(shape, op, dim, seed=11):
+    def build(dev):
+        return LB.copy(_n(seed, shape), shape, dev).reduce(op, dim)
+    return build
+
+
+def reduce_narrow(shape, op, dim, seed=12):
+    def build(dev):
+        return LB.copy(_n(seed, shape), shape, dev).reduce(op, dim).narrow(dim, 0, 1)
+    return build
+
+
+def fused_reduce(n, seed_a=2, seed_b=3):
+    def build(dev):
+        a = LB.copy(_u(seed_a, (n,)), (n,), dev)
+        b = LB.copy(_u(seed_b, (n,)), (n,), dev)
+        half = LB.cst(0.5, (n,), dev)
+        return a.binary("mul", b).binary("add", a.binary("mul", half)).reduce("sum", 0).narrow(0, 0, 1)
+    return build
+
+
+def rms_norm(shape, seed=6):
+    def build(dev):
+        x = LB.copy(_n(seed, shape), shape, dev)
+        alpha = LB.copy(_n(seed + 100, (shape[-1],), 0.02), (shape[-1],), dev)
+        return L.rms_norm(x, alpha, 1e-5)
+    return build
+
+
+def swiglu(shape, seed=21):
+    def build(dev):
+        g = LB.copy(_n(seed, shape), shape, dev)
+        u = LB.copy(_n(seed + 1, shape), shape, dev)
+        return L.silu(g).binary("mul", u)
+    return build
+
+
+def scale(shape, seed=22):
+    def build(dev):
+        x = LB.copy(_n(seed, shape), shape, dev)
+        s = LB.cst(64.0 ** -0.5, (), dev).broadcast(shape)
+        return x.binary("mul", s)
+    return build
+
+
+def transpose_merge(b, h, t, d, seed=23):
+    """[b,h,t,d] -> transpose(2,1) -> merge_dims(-2): the attention output copy (model.rs:244-245)."""
+    def build(dev):
+        x = LB.copy(_n(seed, (b, h, t, d)), (b, h, t, d), dev)
+        return x.transpose(2, 1).merge_dims(-2)
+    return build
+
+
+def split_transpose(b, t, h, d, seed=24):
+    """[b,t,h*d] -> split_dim(2,h,d) -> transpose(2,1) (model.rs:209-210)."""
+    def build(dev):
+        x = LB.copy(_n(seed, (b, t, h * d)), (b, t, h * d), dev)
+        return x.split_dim(2, h, d).transpose(2, 1)
+    return build
+
+
+def repeat_kv(b, h, s, d, n_rep, seed=25):
+    def build(dev):
+        x = LB.copy(_n(seed, (b, h, s, d)), (b, h, s, d), dev)
+        return L.repeat(x, 1, n_rep)
+    return build
+
+
+def index_select(vocab, h, ids_shape, seed=26):
+    def build(dev):
+        table = LB.copy(_n(seed, (vocab, h)), (vocab, h), dev)
+        ids = LB.copy(rng.token_ids(seed + 1, int(np.prod(ids_shape)), vocab), ids_shape, dev)
+        return L.index_select(table, ids)
+    return build
+
+
+def residual_add(shape, seed=27):
+    def build(dev):
+        return LB.copy(_n(seed, shape), shape, dev).binary("add", LB.copy(_n(seed + 1, shape), shape, dev))
+    return build
+
+
+def cos_sin(shape, seed=28):
+    def build(dev):
+        x = LB.copy(_u(seed, shape) * np.float32(50.0), shape, dev)
+        return x.unary("cos").binary("add", x.unary("sin"))
+    return build
+
+
+def narrow_mid(shape, dim, off, length, seed=29):
+    def build(dev):
+        return LB.copy(_n(seed, shape), shape, dev).narrow(dim, off, length).binary("mul", LB.cst(2.0, (), dev).broadcast(
+            tuple(length if i == dim else s for i, s in enumerate(shape))))
+    return build
+
+
+def cast_roundtrip(n, seed=30):
+    def build(dev):
+        x = LB.copy(_u(seed, (n,)) * np.float32(100.0), (n,), dev)
+        return x.cast(I32).cast(F32)
+    return build
+
+
+def max_min(shape, seed=31):
+    def build(dev):
+        a = LB.copy(_n(seed, shape), shape, dev)
+        b = LB.copy(_n(seed + 1, shape), shape, dev)
+        return a.binary("max", b).binary("sub", a.binary("min", b))
+    return build
+
+
+def sum_of_exp_minus_max(shape, seed=32):
+    """A reduce nested in a reduce over the same dim (lower_op.rs:254-298 extracts the inner one)."""
+    def build(dev):
+        x = LB.copy(_n(seed, shape), shape, dev)
+        mx = x.reduce("max", -1).broadcast(shape)
+        return x.binary("sub", mx).unary("exp").reduce("sum", -1).narrow(len(shape) - 1, 0, 1)
+    return build
+
+
+def matmul_case(lshape, rshape, transpose=False, seed=40):
+    def build(dev):
+        a = LB.copy(_u(seed, lshape), lshape, dev)
+        b = LB.copy(_u(seed + 1, rshape), rshape, dev)
+        return a.matmul_t(b) if transpose else a.matmul(b)
+    return build
+
+
+# (name, builder, tolerance)
+ELEMENTWISE_AND_REDUCE = [
+    ("softmax_2x4", softmax((2, 4)), 1e-5),
+    ("softmax_32x1024", softmax((32, 1024)), 1e-5),
+    ("softmax_7x333", softmax((7, 333)), 1e-5),
+    ("softmax_3x5000", softmax((3, 5000)), 1e-5),
+    ("softmax_64x64", softmax((64, 64)), 1e-5),
+    ("softmax_1x8193", softmax((1, 8193)), 1e-5),
+    ("softmax_2x3x5x130", softmax((2, 3, 5, 130)), 1e-5),
+    ("softmax_decode_1x32x1x129", softmax((1, 32, 1, 129)), 1e-5),
+    ("sum_dim0_300x70", reduce_dim((300, 70), "sum", 0), 2e-5),
+    ("sum_dim1_70x300", reduce_dim((70, 300), "sum", 1), 2e-5),
+    ("max_dim0_narrow_513x9", reduce_narrow((513, 9), "max", 0), "exact"),
+    ("min_dim1_narrow_9x513", reduce_narrow((9, 513), "min", 1), "exact"),
+    ("sum_mid_4x100x6", reduce_narrow((4, 100, 6), "sum", 1), 2e-5),
+    ("fused_reduce_1000", fused_reduce(1000), 1e-5),
+    ("fused_reduce_65536", fused_reduce(1 << 16), 1e-4),
+    ("fused_reduce_1M", fused_reduce(1 << 20), 1e-4),
+    ("rms_norm_2x7x64", rms_norm((2, 7, 64)), 1e-5),
+    ("rms_norm_1x1x2048", rms_norm((1, 1, 2048)), 1e-5),
+    ("rms_norm_1x5x2048", rms_norm((1, 5, 2048)), 1e-5),
+    ("swiglu_1x3x5632", swiglu((1, 3, 5632)), 1e-5),
+    ("scale_1x4x3x9", scale((1, 4, 3, 9)), 1e-6),
+    ("transpose_merge_1x4x5x8", transpose_merge(1, 4, 5, 8), "exact"),
+    ("transpose_merge_1x32x16x64", transpose_merge(1, 32, 16, 64), "exact"),
+    ("split_transpose_1x5x4x8", split_transpose(1, 5, 4, 8), "exact"),
+    ("repeat_kv_1x4x7x64_x8", repeat_kv(1, 4, 7, 64, 8), "exact"),
+    ("index_select_50x64", index_select(50, 64, (1, 9)), "exact"),
+    ("residual_add_1x3x2048", residual_add((1, 3, 2048)), 1e-6),
+    ("cos_sin_1000", cos_sin((1000,)), 1e-4),
+    ("narrow_mid_6x50", narrow_mid((6, 50), 1, 7, 20), 1e-6),
+    ("cast_roundtrip_100", cast_roundtrip(100), "exact"),
+    ("max_min_17x33", max_min((17, 33)), 1e-6),
+    ("sum_exp_minus_max_5x77", sum_of_exp_minus_max((5, 77)), 1e-5),
+]
+
+MATMUL = [
+    ("mm_4x2_2x3", matmul_case((4, 2), (2, 3)), 1e-5),
+    ("mm_65x33_33x70", matmul_case((65, 33), (33, 70)), 1e-4),
+    ("mm_b3_40x20_20x50", matmul_case((3, 40, 20), (3, 20, 50)), 1e-4),
+    ("mm_t_1x7x64_96x64", matmul_case((1, 7, 64), (96, 64), True), 1e-4),
+    ("mm_t_decode_1x1x2048_256x2048", matmul_case((1, 1, 2048), (256, 2048), True), 1e-4),
+    ("mm_t_attn_1x4x9x64_1x4x9x64", matmul_case((1, 4, 9, 64), (1, 4, 9, 64), True), 1e-4),
+    ("mm_attn_v_1x4x9x9_1x4x9x64", matmul_case((1, 4, 9, 9), (1, 4, 9, 64)), 1e-4),
+    ("mm_rope_table_64x1_1x32", matmul_case((64, 1), (1, 32)), 1e-6),
+    ("mm_128x128x128", matmul_case((128, 128), (128, 128)), 1e-4),
+]

@@ -1,0 +1,151 @@
+"""CPU-side checks of the HIP backend: the C ABI exports what include/ughip.h declares, and every
+kernel the lazy-graph cases produce lowers to HIP source that hiprtc accepts for gfx950 (no GPU is
+needed to compile).  No compute call is made here."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import cases
+import ref_suite
+import ug_amd
+from ug_amd import LazyBuffer as LB, Schedule, SsaKernel
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_c_abi_exports_every_declared_symbol():
+    text = open(os.path.join(ROOT, "include", "ughip.h")).read()
+    names = sorted(set(re.findall(r"\b(ughip_[a-z0-9_]+)\s*\(", text)))
+    assert len(names) >= 25
+    lib = ug_amd.ughip_lib()
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+    assert lib.ughip_use_grid() == 0
+
+
+def test_no_gpu_is_a_loud_error_not_a_fallback():
+    lib = ug_amd.ughip_lib()
+    dev = C.c_void_p()
+    rc = lib.ughip_device_create(0, C.byref(dev))
+    if rc == 0:  # running on a GPU box: nothing to check here
+        lib.ughip_device_release(dev)
+        return
+    assert b"HIP" in lib.ughip_last_error() or b"device" in lib.ughip_last_error()
+    with pytest.raises(ug_amd.UgError):
+        ug_amd.hip_device(0)
+
+
+def rtc_ok(source):
+    lib = ug_amd.ughip_lib()
+    n = C.c_size_t()
+    rc = lib.ughip_rtc_check(source.encode(), b"gfx950", C.byref(n))
+    assert rc == 0, lib.ughip_last_error().decode()
+    assert n.value > 0
+
+
+def kernels_of(build, cpu):
+    s = Schedule.create_one(build(cpu))
+    out = []
+    for i, item in enumerate(s.items()):
+        if item["kind"] in ("kernel", "ssa"):
+            out.append((item.get("name", "ssa"), s.item_ssa(i)))
+    return out
+
+
+@pytest.mark.parametrize("name,build,tol", cases.ELEMENTWISE_AND_REDUCE, ids=[c[0] for c in cases.ELEMENTWISE_AND_REDUCE])
+def test_case_kernels_lower_and_compile(cpu, name, build, tol):
+    ks = kernels_of(build, cpu)
+    assert ks
+    for kname, k in ks:
+        src, info = k.hip_code(kname)
+        assert 'extern "C" __global__' in src
+        assert info["grid_dim"] >= 1 and 1 <= info["block_dim"] <= 1024
+        rtc_ok(src)
+
+
+def strategies(build, cpu):
+    return [k.hip_code(n)[1]["strategy"] for n, k in kernels_of(build, cpu)]
+
+
+def test_strategy_selection(cpu):
+    assert strategies(cases.softmax((32, 1024)), cpu) == ["row_block", "row_block"]
+    assert strategies(cases.softmax((4096, 128)), cpu) == ["row_block", "row_block"]
+    assert strategies(cases.residual_add((1, 3, 2048)), cpu) == ["elementwise"]
+    assert strategies(cases.rms_norm((1, 5, 2048)), cpu) == ["row_block"]
+    # a reduce over the strided dim walks memory along the rows: one thread per column
+    assert strategies(cases.reduce_dim((300, 70), "sum", 0), cpu) == ["row_thread"]
+    assert strategies(cases.reduce_dim((70, 300), "sum", 1), cpu) == ["row_block"]
+    # config 2: one output, 2^24-long reduction -> whole-device reduction
+    (k,) = kernels_of(cases.fused_reduce(1 << 24), cpu)
+    src, info = k[1].hip_code(k[0])
+    assert info["strategy"] == "grid_reduce" and info["grid_dim"] >= 256 and info["scratch_bytes"] > 0
+    rtc_ok(src)
+
+
+def test_gpu_style_ssa_is_translated_literally():
+    for name, args, launch in [("exp", (64,), (4, 64)), ("exp_block", (256, 64), (4, 64)), ("softmax_barrier", (2, 64), (2, 64)),
+                               ("softmax_reduce", (2, 64), (2, 64)), ("softmax_block", (2, 256, 64), (2, 64))]:
+        k = SsaKernel.sample(name, *args)
+        k.set_launch(*launch)
+        src, info = k.hip_code(name)
+        assert info["strategy"] == "literal" and (info["grid_dim"], info["block_dim"]) == launch
+        rtc_ok(src)
+
+
+def test_scheduler_grid_ssa_with_reduce_local_compiles():
+    # what a `use_grid() == true` device would receive (schedule.rs:162-188)
+    k = SsaKernel.sample_op("softmax", 32, 1024, block_axis=0, thread_dim=1, thread_block_dim=32)
+    src, info = k.hip_code("softmax_grid")
+    assert info["strategy"] == "literal" and "ug_block_reduce_dyn" in src
+    rtc_ok(src)
+
+
+def test_malformed_ssa_is_rejected():
+    from ug_amd.api import Instr
+    bad = Instr()
+    bad.op = 8  # Load from an undefined pointer var
+    bad.v = 5
+    k = SsaKernel.from_instrs([bad])
+    with pytest.raises(ug_amd.UgError, match="ssa lowering"):
+        k.hip_code()
+
+
+def test_zero_sized_nest_is_an_empty_launch(cpu):
+    # the initial KV cache: cst(0) of shape [1,4,0,64] (ug-llama/src/model.rs:192)
+    lb = LB.cst(0.0, (1, 4, 0, 64), cpu)
+    s = Schedule.create_one(lb)
+    k = s.item_ssa(0)
+    src, info = k.hip_code("empty")
+    assert "extern" in src
+    assert lb.data_vec().size == 0
+
+
+def test_rng_matches_native_generator():
+    lib = ug_amd.host_lib()
+    out = np.zeros(1001, np.float32)
+    assert lib.ugh_synthetic_weights(C.c_uint64(9), C.c_float(0.02), 0, b"model.norm.weight", C.c_size_t(1001), out.ctypes.data_as(C.c_void_p)) == 0
+    # python restatement of tensor_seed (FNV-1a folded into the seed)
+    h = 0xcbf29ce484222325
+    for c in b"model.norm.weight":
+        h = ((h ^ c) * 0x100000001b3) & 0xFFFFFFFFFFFFFFFF
+    from ug_amd.rng import _mix, normal
+    with np.errstate(over="ignore"):
+        ts = int(_mix(np.uint64(9 ^ h)))
+    ref = normal(ts, 1001, 0.02)
+    np.testing.assert_allclose(out, ref, rtol=1e-6, atol=1e-9)
+    assert abs(float(out.std()) - 0.02) < 0.002
+    # bf16 rounding helper agrees with the native one
+    out16 = np.zeros(1001, np.float32)
+    lib.ugh_synthetic_weights(C.c_uint64(9), C.c_float(0.02), 1, b"model.norm.weight", C.c_size_t(1001), out16.ctypes.data_as(C.c_void_p))
+    np.testing.assert_array_equal(out16, ug_amd.rng.bf16_round(out))
+
+
+def test_ref_suite_graph_shapes(cpu):
+    a = LB.copy(np.ones(8, np.float32), (8,), cpu)
+    b = LB.copy(np.ones(8, np.float32), (8,), cpu)
+    r = ref_suite.fused_reduce_graph(a, b, cpu)
+    assert r.dims() == [1]
+    assert r.data_vec().tolist() == [12.0]

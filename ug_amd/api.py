@@ -582,7 +582,7 @@ class Schedule(_Handle):
 
     def compile(self, cache=None):
         out = C.c_void_p()
-        _chk(host_lib().ugh_schedule_compile(_p(self.h), _p(cache.h) if cache else None, C.byref(out)))
+        _chk(host_lib().ugh_schedule_compile(_p(self.h), _p(cache.h) if cache is not None else None, C.byref(out)))
         cs = CompiledSchedule(out.value)
         cs._keep = [self, cache]
         return cs

@@ -11,7 +11,7 @@
 
 struct CachedModule {
   hipModule_t module = nullptr;
-  hipFunction_t function = nullptr;
+  hipFunction_t function = nullptr, function2 = nullptr;
 };
 
 struct ughip_device {

@@ -730,7 +730,7 @@ class Lowering {
     }
     if (scratch) {
       if (s_.n_args) o << ", ";
-      o << "void* __restrict__ ug_part_raw, unsigned* __restrict__ ug_cnt";
+      o << "void* __restrict__ ug_part_raw";
     }
     return o.str();
   }
@@ -1157,8 +1157,11 @@ class Lowering {
       const Region& r = regions_[0];
       int vec = pick_vec(r.trip, tpr);
       i64 per_block_iter = (i64)tpr * vec;
-      i64 want = (r.trip + per_block_iter * 8 - 1) / (per_block_iter * 8);  // ~8 iterations per thread
-      unsigned cap = std::max<i64>(1, 4096 / nr);
+      // Measured on MI355X (2 x 64 MiB streamed): 256-512 workgroups of 256 threads, each thread
+      // walking >= 4 slabs with four 128-bit loads in flight, is where the curve is flat (~6.2 TB/s);
+      // more workgroups only add scheduling cost.
+      i64 want = (r.trip + per_block_iter * 4 - 1) / (per_block_iter * 4);
+      unsigned cap = std::max<i64>(1, 512 / nr);
       nb = (unsigned)std::max<i64>(1, std::min<i64>(want, cap));
       nb = env_u("UGHIP_GRID_REDUCE_BLOCKS", nb);
       o << "  const int ug_row = (int)blockIdx.x / " << nb << ";\n";
@@ -1172,13 +1175,14 @@ class Lowering {
     if (!grid_reduce) {
       emit_items(o, false, col_mask, 2, true, tpr, false);
     } else {
-      // Row phase up to and including the reduction; the last workgroup to finish a row folds
-      // the partials in index order and carries on with the rest of the row.
+      // Stage 1 (this kernel): every workgroup folds its slabs of the reduction and stores one
+      // partial.  Stage 2 (`<entry>_fin`, one workgroup per row, launched right behind on the same
+      // stream) folds the partials in index order and carries on with the rest of the row.  The
+      // kernel boundary is the only synchronisation: no fences, no atomics, same bits every run.
       const Region& r = regions_[0];
       std::string ty = dtype_c_name(vt_[r.acc].dtype);
       std::string fn = reduce_functor(r.op);
       std::string part = "ug_p" + std::to_string(r.acc);
-      size_t k = 0;
       std::vector<const Item*> before, after;
       bool seen = false;
       for (const Item& it : items_) {
@@ -1189,25 +1193,24 @@ class Lowering {
         }
         (seen ? after : before).push_back(&it);
       }
-      (void)k;
+      // Only what the reduction body needs has to run in stage 1, but the row-invariant prefix is
+      // a handful of scalar instructions: emit it in both stages.
       for (const Item* it : before) emit_range(o, it->idx, it->end, 2);
       o << "    " << ty << "* __restrict__ ug_part = (" << ty << "*)ug_part_raw;\n";
       emit_region_partial(o, r, 2, tpr, nb);
-      o << "    __shared__ int ug_last;\n";
-      o << "    if (ug_t == 0) {\n";
-      o << "      __hip_atomic_store(&ug_part[ug_row * " << nb << " + ug_blk], " << part << ", __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
-      o << "      __threadfence();\n";
-      o << "      const unsigned ug_ticket = atomicAdd(&ug_cnt[ug_row], 1u);\n";
-      o << "      ug_last = ug_ticket == " << nb - 1 << "u;\n";
-      o << "    }\n";
-      o << "    __syncthreads();\n";
-      o << "    if (!ug_last) return;\n";
-      o << "    __threadfence();\n";
-      o << "    " << part << " = " << identity_lit(r.op, vt_[r.acc].dtype) << ";\n";
+      o << "    if (ug_t == 0) ug_part[ug_row * " << nb << " + ug_blk] = " << part << ";\n";
+      o << "  }\n}\n";
+      // ---- stage 2
+      o << "\nextern \"C\" __global__ void __launch_bounds__(" << tpr << ") " << entry_ << "_fin(" << signature(true) << ") {\n";
+      o << "  const int ug_t = (int)threadIdx.x;\n";
+      o << "  const int ug_row = (int)blockIdx.x;\n";
+      o << "  {\n";
+      emit_decode(o, rows, "ug_row", 1, 2);
+      for (const Item* it : before) emit_range(o, it->idx, it->end, 2);
+      o << "    const " << ty << "* __restrict__ ug_part = (const " << ty << "*)ug_part_raw;\n";
+      o << "    " << ty << " " << part << " = " << identity_lit(r.op, vt_[r.acc].dtype) << ";\n";
       o << "    for (int ug_i = ug_t; ug_i < " << nb << "; ug_i += " << tpr << ")\n";
-      o << "      " << part << " = " << fn << "::f(" << part << ", __hip_atomic_load(&ug_part[ug_row * " << nb
-        << " + ug_i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));\n";
-      o << "    if (ug_t == 0) ug_cnt[ug_row] = 0u;\n";
+      o << "      " << part << " = " << fn << "::f(" << part << ", ug_part[ug_row * " << nb << " + ug_i]);\n";
       emit_region_finish(o, r, 2, tpr);
       for (const Item* it : after) {
         if (it->kind == 0 && I_[it->idx].op == UGHIP_I_STORE)
@@ -1216,7 +1219,9 @@ class Lowering {
           emit_range(o, it->idx, it->end, 2);
       }
       out_.scratch_part_bytes = (size_t)nr * nb * dtype_size(vt_[r.acc].dtype);
-      out_.scratch_cnt_bytes = (size_t)nr * sizeof(unsigned);
+      out_.entry2 = entry_ + "_fin";
+      out_.grid2 = (unsigned)nr;
+      out_.block2 = (unsigned)tpr;
     }
     bool any_col = false;
     for (const Item& it : items_) any_col |= (it.deps & col_mask) != 0;
@@ -1246,8 +1251,19 @@ class Lowering {
     int vec = pick_vec(L.trip, tpr);
     std::string part = "ug_p" + std::to_string(r.acc);
     o << pad << ty << " " << part << " = " << identity_lit(r.op, vt_[r.acc].dtype) << ";\n";
-    o << pad << "for (long long ug_i = ((long long)ug_blk * " << tpr << " + ug_t) * " << vec << "; ug_i < " << L.trip << "LL; ug_i += "
-      << (i64)nb * tpr * vec << "LL) {\n";
+    // 32-bit indices (ssa offsets are i32 anyway) keep the `vec` unrolled accesses visibly
+    // consecutive, so they merge into one 128-bit load; a constant trip count lets the compiler
+    // batch the loads of several slabs before the first use.
+    const i64 stride = (i64)nb * tpr * vec;
+    const i64 iters = (L.trip + stride - 1) / stride;
+    const bool tail = L.trip % stride != 0;
+    const bool wide = L.trip + stride >= (1ll << 31);
+    const char* it_ty = wide ? "long long" : "int";
+    o << pad << "const " << it_ty << " ug_base = ((" << it_ty << ")ug_blk * " << tpr << " + ug_t) * " << vec << ";\n";
+    o << pad << "#pragma unroll " << (iters >= 4 ? 4 : (int)iters) << "\n";
+    o << pad << "for (int ug_it = 0; ug_it < " << iters << "; ++ug_it) {\n";
+    o << pad << "  const " << it_ty << " ug_i = ug_base + (" << it_ty << ")ug_it * " << stride << (wide ? "LL" : "") << ";\n";
+    if (tail) o << pad << "  if (ug_i >= " << L.trip << ") break;\n";
     o << pad << "#pragma unroll\n";
     o << pad << "  for (int ug_u = 0; ug_u < " << vec << "; ++ug_u) {\n";
     o << pad << "    const int " << var(L.begin) << " = ";

@@ -14,9 +14,11 @@ struct Lowered {
   std::string entry;   // extern "C" kernel symbol
   int strategy = UGHIP_STRAT_LITERAL;
   unsigned grid = 1, block = 1, lds_bytes = 0;
-  // Device scratch the kernel takes as two trailing pointer arguments (partials, counters).
-  // Zero-initialised once when the func is created; the kernel restores the zeros itself.
-  size_t scratch_part_bytes = 0, scratch_cnt_bytes = 0;
+  // A grid-wide reduction runs as two kernels, `entry` then `entry2`, that share one device
+  // scratch buffer of partial results, passed as a trailing pointer argument to both.
+  std::string entry2;
+  unsigned grid2 = 0, block2 = 0;
+  size_t scratch_part_bytes = 0;
   std::vector<int> arg_dtype;      // per kernel argument, UGHIP_* dtype
   std::vector<long long> min_len;  // per argument: 1 + largest offset the kernel forms, -1 if unknown
   std::vector<char> arg_written;   // per argument: has a Store

@@ -38,9 +38,8 @@ using namespace ughip;
 struct ughip_func {
   ughip_device* dev = nullptr;
   Lowered low;
-  hipFunction_t function = nullptr;
+  hipFunction_t function = nullptr, function2 = nullptr;
   void* scratch_part = nullptr;
-  void* scratch_cnt = nullptr;
 };
 
 struct ughip_event {
@@ -251,7 +250,7 @@ int ughip_codegen(const ughip_ssa* ssa, const char* name, char* buf, size_t buf_
     info->grid_dim = low.grid;
     info->block_dim = low.block;
     info->lds_bytes = low.lds_bytes;
-    info->scratch_bytes = low.scratch_part_bytes + low.scratch_cnt_bytes;
+    info->scratch_bytes = low.scratch_part_bytes;
   }
   return UGHIP_OK;
 }
@@ -304,15 +303,13 @@ int ughip_compile(ughip_device* dev, const ughip_ssa* ssa, const char* name, ugh
       CachedModule cm;
       HIPCHK(hipModuleLoadData(&cm.module, code.data()));
       HIPCHK(hipModuleGetFunction(&cm.function, cm.module, f->low.entry.c_str()));
+      if (!f->low.entry2.empty()) HIPCHK(hipModuleGetFunction(&cm.function2, cm.module, f->low.entry2.c_str()));
       it = dev->modules.emplace(f->low.source, cm).first;
     }
     f->function = it->second.function;
+    f->function2 = it->second.function2;
   }
-  if (f->low.scratch_part_bytes) {
-    HIPCHK(hipMalloc(&f->scratch_part, f->low.scratch_part_bytes));
-    HIPCHK(hipMalloc(&f->scratch_cnt, f->low.scratch_cnt_bytes));
-    HIPCHK(hipMemsetAsync(f->scratch_cnt, 0, f->low.scratch_cnt_bytes, dev->stream));
-  }
+  if (f->low.scratch_part_bytes) HIPCHK(hipMalloc(&f->scratch_part, f->low.scratch_part_bytes));
   ughip_device_retain(dev);
   *out = f.release();
   return UGHIP_OK;
@@ -321,11 +318,10 @@ int ughip_compile(ughip_device* dev, const ughip_ssa* ssa, const char* name, ugh
 int ughip_func_release(ughip_func* f) {
   if (!f) return UGHIP_OK;
   ughip_device* dev = f->dev;
-  if (f->scratch_part || f->scratch_cnt) {
+  if (f->scratch_part) {
     hipSetDevice(dev->ordinal);
     hipStreamSynchronize(dev->stream);
-    if (f->scratch_part) hipFree(f->scratch_part);
-    if (f->scratch_cnt) hipFree(f->scratch_cnt);
+    hipFree(f->scratch_part);
   }
   delete f;
   ughip_device_release(dev);
@@ -348,7 +344,7 @@ int ughip_func_get_info(const ughip_func* f, ughip_func_info* out) {
   out->grid_dim = f->low.grid;
   out->block_dim = f->low.block;
   out->lds_bytes = f->low.lds_bytes;
-  out->scratch_bytes = f->low.scratch_part_bytes + f->low.scratch_cnt_bytes;
+  out->scratch_bytes = f->low.scratch_part_bytes;
   return UGHIP_OK;
 }
 
@@ -376,12 +372,10 @@ int ughip_run(ughip_device* dev, ughip_func* f, ughip_slice* const* args, size_t
     params[a] = &ptrs[a];
   }
   size_t np = n_args;
-  if (low.scratch_part_bytes) {
-    params[np++] = &f->scratch_part;
-    params[np++] = &f->scratch_cnt;
-  }
+  if (low.scratch_part_bytes) params[np++] = &f->scratch_part;
   if (int rc = device_activate(dev)) return rc;
   HIPCHK(hipModuleLaunchKernel(f->function, low.grid, 1, 1, low.block, 1, 1, low.lds_bytes, dev->stream, params, nullptr));
+  if (f->function2) HIPCHK(hipModuleLaunchKernel(f->function2, low.grid2, 1, 1, low.block2, 1, 1, 0, dev->stream, params, nullptr));
   return UGHIP_OK;
 }
 
