@@ -29,9 +29,9 @@ MFMA_F32_PEAK_TF = 157.3        # f32 matrix
 N = 1 << 24
 ALGO_BYTES = 2 * N * 4 + 4      # read a, read b, write one f32
 
-# HBM bytes per launch of the dominant kernel from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`,
-# scaled by a plain copy kernel of known size (see profiles/); None until measured.
-TRAFFIC_BYTES = None
+# HBM bytes per step from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`, scaled by the counters'
+# reading for the --copy-probe kernel (profiles/fused_reduce_2pow24_hbm_traffic.txt).
+TRAFFIC_BYTES = 134222039
 
 
 def hip_events(dev):
@@ -168,6 +168,7 @@ def main():
     ap.add_argument("--extras", action="store_true")
     ap.add_argument("--llama", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true", help="also run a plain 2^24-element copy kernel (counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU only (nothing in the path is sharded); use --gpus 1", file=sys.stderr)
@@ -200,6 +201,15 @@ def main():
                      "traffic": TRAFFIC_BYTES, "kernel_us": round(ev_ms * 1e3 / args.steps, 3)},
         "result": got, "truth_f64": truth,
     }
+    if args.copy_probe:
+        # A plain f32 copy of known size (2^24 elements: 64 MiB read, 64 MiB written) in the same
+        # process: the scale for rocprofv3's FETCH_SIZE / WRITE_SIZE counters.
+        from ug_amd import LazyBuffer as LB, Schedule
+        cp = LB.copy(a, (N,), dev).unary("id")
+        ccs = Schedule.create_one(cp).compile()
+        _, cms = timed(dev, ccs.run, args.steps, args.warmup)
+        line["copy_probe"] = {"kernel": ccs.funcs()[0]["info"], "bytes_read": 4 * N, "bytes_written": 4 * N,
+                              "GB/s": round(8.0 * N * args.steps / (cms * 1e-3) / 1e9, 1)}
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(a, b, truth)
     if args.extras:
