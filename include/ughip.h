@@ -133,6 +133,9 @@ int ughip_device_release(ughip_device* dev);
 int ughip_synchronize(ughip_device* dev);
 /* "gfx950" etc.; buf receives a NUL-terminated arch name. */
 int ughip_device_arch(ughip_device* dev, char* buf, size_t buf_len);
+/* Introspection: code objects built by hiprtc so far, bytes cached in the allocation pool, bytes
+ * handed out to live slices.  Any out pointer may be NULL. */
+int ughip_device_stats(ughip_device* dev, size_t* n_code_objects, size_t* pool_bytes, size_t* live_bytes);
 /* `Device::use_grid()` (lib.rs:72): this backend returns 0 -- it wants the serial loop
  * nest and chooses grid/block itself. */
 int ughip_use_grid(void);
@@ -141,6 +144,10 @@ int ughip_use_grid(void);
 /* Zero-filled like CpuDevice::allocate_uninit (cpu_runtime.rs:255-264).  len 0 is legal
  * (ug-llama/src/model.rs:192) and yields a slice with a null device pointer. */
 int ughip_alloc(ughip_device* dev, int dtype, size_t len, ughip_slice** out);
+/* Turn the zero-fill of ughip_alloc off (on = 0) or back on: ug-cuda's allocate_uninit leaves memory
+ * uninitialised (ug-cuda/src/runtime.rs:217-241), and a caller whose kernels overwrite every
+ * destination -- the llama graph does -- saves one fill launch per allocation. */
+int ughip_device_set_zero_fill(ughip_device* dev, int on);
 int ughip_free(ughip_slice* s);
 size_t ughip_slice_len(const ughip_slice* s);
 int ughip_slice_dtype(const ughip_slice* s);

@@ -282,6 +282,67 @@ def test_matmul_bf16(hip):
     np.testing.assert_array_equal(dst2.to_vec(), dst.to_vec())
 
 
+def _raw_matmul(hip, dtype, a, w, rhs_nk):
+    """a: [b, m, k], w: [b, k, n] as numpy f32; rhs_nk stores the rhs as [b, n, k] (transposed view)."""
+    b, m, k = a.shape
+    n = w.shape[2]
+    enc = rng.to_bf16_bits if dtype == ug_amd.BF16 else (lambda v: v)
+    dst = hip.allocate_uninit(dtype, b * m * n)
+    sa = hip.slice_from(enc(np.ascontiguousarray(a)))
+    if rhs_nk:
+        sw = hip.slice_from(enc(np.ascontiguousarray(np.swapaxes(w, 1, 2))))
+        rhs = ((b, k, n), (k * n, 1, k), 0)
+    else:
+        sw = hip.slice_from(enc(np.ascontiguousarray(w)))
+        rhs = ((b, k, n), (k * n, n, 1), 0)
+    hip.matmul(dst, sa, sw, (b, m, n, k), ((b, m, k), (m * k, k, 1), 0), rhs)
+    out = dst.to_vec()
+    return (rng.from_bf16_bits(out) if dtype == ug_amd.BF16 else out).reshape(b, m, n)
+
+
+# Shapes that are whole multiples of the 256 x 128 x (32 | 64) tile take the tuned MFMA kernel; the
+# neighbours that are one element off take the generic one.  Both are held to the same bound.
+@pytest.mark.parametrize("rhs_nk", [False, True])
+@pytest.mark.parametrize("bmnk", [(2, 256, 128, 96), (1, 512, 384, 160), (3, 256, 256, 32), (1, 255, 128, 96), (1, 256, 129, 96)])
+def test_matmul_f32_tile_multiples(hip, bmnk, rhs_nk):
+    b, m, n, k = bmnk
+    print("matmul f32", bmnk, "rhs_nk", rhs_nk, flush=True)
+    a = rng.uniform_pm1(21, b * m * k).reshape(b, m, k)
+    w = rng.uniform_pm1(22, b * k * n).reshape(b, k, n)
+    got = _raw_matmul(hip, F32, a, w, rhs_nk)
+    truth = a.astype(np.float64) @ w.astype(np.float64)
+    bound = k * np.finfo(np.float32).eps * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64))
+    assert np.all(np.abs(got - truth) <= bound + 1e-12)
+
+
+@pytest.mark.parametrize("rhs_nk", [False, True])
+@pytest.mark.parametrize("bmnk", [(2, 256, 128, 192), (1, 512, 384, 64), (3, 256, 256, 320), (1, 256, 128, 96), (1, 248, 128, 128)])
+def test_matmul_bf16_tile_multiples(hip, bmnk, rhs_nk):
+    b, m, n, k = bmnk
+    print("matmul bf16", bmnk, "rhs_nk", rhs_nk, flush=True)
+    a = rng.bf16_round(rng.uniform_pm1(23, b * m * k)).reshape(b, m, k)
+    w = rng.bf16_round(rng.uniform_pm1(24, b * k * n)).reshape(b, k, n)
+    got = _raw_matmul(hip, ug_amd.BF16, a, w, rhs_nk)
+    exact = a.astype(np.float64) @ w.astype(np.float64)
+    # f32 accumulation of exact bf16 products, then one rounding to bf16 (2^-8 relative)
+    bound = (2.0 ** -8) * np.abs(exact) + k * np.finfo(np.float32).eps * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64))
+    assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-12)
+
+
+def test_matmul_tiled_matches_generic_on_integers(hip):
+    """Small-integer operands make every partial sum exact in f32, so the tuned kernel, the generic
+    kernel (reached through a shape one column short) and numpy must agree bit for bit."""
+    b, m, n, k = 2, 256, 256, 128
+    a = np.floor(rng.uniform_pm1(31, b * m * k) * 8).astype(np.float32).reshape(b, m, k)
+    w = np.floor(rng.uniform_pm1(32, b * k * n) * 8).astype(np.float32).reshape(b, k, n)
+    want = (a.astype(np.float64) @ w.astype(np.float64)).astype(np.float32)
+    for rhs_nk in (False, True):
+        np.testing.assert_array_equal(_raw_matmul(hip, F32, a, w, rhs_nk), want)
+        # sums up to 128 * 64 = 8192 are not all bf16-representable: one final rounding is expected
+        np.testing.assert_array_equal(_raw_matmul(hip, ug_amd.BF16, a, w, rhs_nk), rng.bf16_round(want.reshape(-1)).reshape(want.shape))
+    np.testing.assert_array_equal(_raw_matmul(hip, F32, a, w[:, :, :255], False), want[:, :, :255])
+
+
 def test_matmul_errors(hip):
     dst = hip.allocate_uninit(F32, 4)
     a, b = hip.slice_from(np.ones(4, np.float32)), hip.slice_from(np.ones(4, np.float32))
@@ -334,6 +395,31 @@ def test_compilation_cache_reuses_funcs(hip):
     assert len(cache) == 1
 
 
+def n_code_objects(hip):
+    n = C.c_size_t()
+    assert ug_amd.ughip_lib().ughip_device_stats(C.c_void_p(hip.raw_hip()), C.byref(n), None, None) == 0
+    return n.value
+
+
+def test_growing_shapes_share_one_code_object(hip, cpu):
+    """Decode-step kernels whose shape follows the KV length (repeat of k/v, score scaling) are
+    lowered parametrically: a new length is a new func but not a new hiprtc compile."""
+    def step(dev, s):
+        kv = LB.copy(rng.normal(50 + s, 4 * s * 64), (1, 4, s, 64), dev)
+        att = LB.copy(rng.normal(90 + s, 32 * s), (1, 32, 1, s), dev)
+        scale = LB.cst(0.125, (), dev).broadcast((1, 32, 1, s))
+        return ug_amd.llama.repeat(kv, 1, 8).data_vec(), att.binary("mul", scale).data_vec()
+
+    step(hip, 3)     # scalar variant (small problems favour more threads)
+    step(hip, 200)   # 4-wide variant
+    before = n_code_objects(hip)
+    for s in (4, 5, 9, 130):
+        got, want = step(hip, s), step(cpu, s)
+        np.testing.assert_array_equal(got[0], want[0])
+        np.testing.assert_allclose(got[1], want[1], rtol=1e-6)
+    assert n_code_objects(hip) == before
+
+
 # ---- the model: identical greedy ids on a small llama ------------------------------------------------------------------------
 @pytest.mark.parametrize("custom_softmax", [False, True])
 def test_small_llama_greedy_ids_match_cpu(hip, cpu, hip_ops, cpu_ops, custom_softmax):
@@ -345,3 +431,21 @@ def test_small_llama_greedy_ids_match_cpu(hip, cpu, hip_ops, cpu_ops, custom_sof
     toks_c, st_c = ug_amd.LlamaModel(cpu, cpu_ops, cfg, custom_softmax, seed=9, std=0.3).generate(prompt, 10)
     print("hip", toks_h.tolist(), "cpu", toks_c.tolist(), "min margin", float(st_c["margins"].min()), flush=True)
     assert toks_h.tolist() == toks_c.tolist()
+
+
+@pytest.mark.parametrize("round_bf16", [False, True])
+def test_llama_config5_width_greedy_ids_match_cpu(hip, cpu, hip_ops, cpu_ops, round_bf16):
+    """BASELINE config 5 at full width (hidden 2048, 32/4 heads, FFN 5632, vocab 32000, N(0,0.02)
+    weights, seed 9) but 2 layers and a short run, so the CPU oracle finishes in seconds; weights
+    f32 or bf16-rounded (what the reference's load_with_cast(F32) makes of a bf16 checkpoint)."""
+    cfg = ug_amd.LlamaConfig(num_hidden_layers=2, max_position_embeddings=256)
+    prompt = rng.token_ids(10, 16, cfg.vocab_size)
+    hip.set_zero_fill(False)  # like ug-cuda's allocate_uninit; every kernel of the graph overwrites its output
+    try:
+        toks_h, st_h = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=0.02, round_bf16=round_bf16).generate(prompt, 6)
+    finally:
+        hip.set_zero_fill(True)
+    toks_c, st_c = ug_amd.LlamaModel(cpu, cpu_ops, cfg, True, seed=9, std=0.02, round_bf16=round_bf16).generate(prompt, 6)
+    print("hip", toks_h.tolist(), "cpu", toks_c.tolist(), "margins", st_c["margins"].tolist(), flush=True)
+    assert toks_h.tolist() == toks_c.tolist()
+    np.testing.assert_allclose(st_h["margins"], st_c["margins"], rtol=1e-2, atol=1e-7)

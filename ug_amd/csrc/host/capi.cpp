@@ -75,6 +75,13 @@ int ugh_device_synchronize(void* d) {
 }
 const char* ugh_device_name(void* d) { return d ? (*static_cast<DevicePtr*>(d))->name() : ""; }
 int ugh_device_use_grid(void* d) { return d && (*static_cast<DevicePtr*>(d))->use_grid(); }
+int ugh_hip_device_set_zero_fill(void* d, int on) {
+  return guard([&] {
+    HipDevice* h = dynamic_cast<HipDevice*>(dev_of(d).get());
+    if (!h) bail("not a hip device");
+    if (ughip_device_set_zero_fill(h->raw(), on)) bail(ughip_last_error());
+  });
+}
 void* ugh_device_raw_hip(void* d) {
   HipDevice* h = d ? dynamic_cast<HipDevice*>(static_cast<DevicePtr*>(d)->get()) : nullptr;
   return h ? h->raw() : nullptr;

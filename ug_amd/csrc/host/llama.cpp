@@ -338,6 +338,7 @@ std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32
   std::vector<float> logits;
   std::vector<int32_t> feed = prompt;
   size_t pos_v = 0;
+  const bool verbose = getenv("UG_LLAMA_VERBOSE") != nullptr;
   for (size_t step = 0; step <= n_steps; ++step) {
     auto t0 = clock::now();
     size_t t = feed.size();
@@ -345,9 +346,21 @@ std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32
     int32_t p32 = (int32_t)pos_v;
     LB pos = LB::copy(&p32, DType::I32, 1, Shape({1, 1}), dev);
     LB lg = model.fwd(tokens, pos, cache);
-    Schedule::create_one(lg).compile_with_cache(ccache).run();
+    auto t1 = clock::now();
+    Schedule schedule = Schedule::create_one(lg);
+    auto t2 = clock::now();
+    CompiledSchedule compiled = schedule.compile_with_cache(ccache);
+    auto t3 = clock::now();
+    compiled.run();
+    auto t4 = clock::now();
     logits.resize(lg.elem_count());
     lg.data_vec(logits.data(), DType::F32);
+    if (verbose) {
+      // the per-token breakdown ug-llama prints with --verbose (main.rs:154-161)
+      auto ms_of = [](clock::time_point a, clock::time_point b) { return std::chrono::duration<double, std::milli>(b - a).count(); };
+      fprintf(stderr, "step %zu: build %.2fms, gen %.2fms, comp: %.2fms, run: %.2fms, sync+d2h: %.2fms, items %zu\n", step, ms_of(t0, t1),
+              ms_of(t1, t2), ms_of(t2, t3), ms_of(t3, t4), ms_of(t4, clock::now()), schedule.items().size());
+    }
     const float* last = logits.data() + (t - 1) * cfg.vocab_size;
     size_t best = 0;
     float second = -INFINITY;

@@ -1,0 +1,24 @@
+// Shared between matmul.hip (dispatch, generic kernels, GEMV) and gemm_tiled.hip (tuned MFMA kernel).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+
+namespace ughip {
+
+struct MMArgs {
+  const void* a;
+  const void* b;
+  void* c;
+  int M, N, K;
+  long long a_rs, a_cs;  // lhs strides of (m, k), in elements
+  long long b_rs, b_cs;  // rhs strides of (k, n), in elements
+  long long a_bs, b_bs, c_bs;
+};
+
+// Tuned kernel: 256x128 tiles, contiguous operands, M % 256 == 0, N % 128 == 0, K % 64 == 0
+// (bf16) / K % 32 == 0 (f32), rhs either [k, n] row-major or [n, k] row-major.
+bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch);
+hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch);
+
+}  // namespace ughip

@@ -24,6 +24,7 @@ struct ughip_device {
   // Size-class free lists: freed blocks are reused by later allocations on the same stream.
   std::multimap<size_t, void*> pool;
   size_t pool_bytes = 0, live_bytes = 0;
+  bool zero_fill = true;
   std::map<std::string, CachedModule> modules;  // generated source -> loaded code object
 };
 

@@ -624,7 +624,22 @@ class Lowering {
     fail("bad const dtype");
   }
 
-  std::string opnd(const ughip_a& a) const { return a.is_const ? const_lit(a) : var((int)a.var); }
+  // Parametric mode: 32-bit integer constants are not printed but read from a by-value kernel
+  // argument (`ug_k.v[i]`).  Two kernels that differ only in such constants -- the same op on
+  // another shape, e.g. the KV length growing by one per decode step -- then share their source
+  // text and therefore the compiled code object.
+  bool parametric_ = false;
+  mutable std::vector<int> kparams_;
+  std::string kparam(i64 v) const {
+    kparams_.push_back((int)v);
+    return "ug_k.v[" + std::to_string(kparams_.size() - 1) + "]";
+  }
+  std::string lit(const ughip_a& a) const {
+    if (parametric_ && a.dtype == UGHIP_I32) return kparam(a.i);
+    return const_lit(a);
+  }
+
+  std::string opnd(const ughip_a& a) const { return a.is_const ? lit(a) : var((int)a.var); }
 
   static const char* reduce_functor(int op) { return op == UGHIP_R_SUM ? "ug_sum" : (op == UGHIP_R_MAX ? "ug_max" : "ug_min"); }
 
@@ -654,7 +669,7 @@ class Lowering {
       case UGHIP_I_DEFINE_GLOBAL: return "";
       case UGHIP_I_DEFINE_LOCAL: o << "__shared__ " << dtype_c_name(in.dtype) << " " << var(i) << "[" << in.n << "];"; break;
       case UGHIP_I_DEFINE_ACC:
-      case UGHIP_I_CONST: o << ty << " " << var(i) << " = " << const_lit(in.a) << ";"; break;
+      case UGHIP_I_CONST: o << ty << " " << var(i) << " = " << lit(in.a) << ";"; break;
       case UGHIP_I_SPECIAL:
         o << "const int " << var(i) << " = " << (in.sub == UGHIP_SPECIAL_THREAD_IDX ? "(int)threadIdx.x" : "(int)blockIdx.x") << ";";
         break;
@@ -993,14 +1008,20 @@ class Lowering {
       const LoopInfo& L = loops_[ls[k]];
       bool inner = k == (int)ls.size() - 1;
       i64 radix = inner ? L.trip / vec : L.trip;
-      std::string digit = k == 0 ? "ug_r" : "(ug_r % " + std::to_string(radix) + ")";
+      // one spelling of the radix per loop, so the % and / below share it (one parameter slot)
+      std::string rs = !k ? "" : (parametric_ ? kparam(radix) : std::to_string(radix));
+      std::string digit = k == 0 ? "ug_r" : "(ug_r % " + rs + ")";
       if (inner && vec > 1) digit = "(" + digit + " * " + std::to_string(vec) + " + ug_u)";
       o << pad << "const int " << var(L.begin) << " = ";
-      if (L.lo) o << L.lo << " + ";
-      o << digit;
-      if (L.step != 1) o << " * " << L.step;
+      if (parametric_) {
+        o << kparam(L.lo) << " + " << digit << " * " << kparam(L.step);
+      } else {
+        if (L.lo) o << L.lo << " + ";
+        o << digit;
+        if (L.step != 1) o << " * " << L.step;
+      }
       o << ";\n";
-      if (k) o << pad << "ug_r /= " << radix << ";\n";
+      if (k) o << pad << "ug_r /= " << rs << ";\n";
     }
   }
 
@@ -1086,18 +1107,32 @@ class Lowering {
     int vec = inner % 4 == 0 ? 4 : (inner % 2 == 0 ? 2 : 1);
     if (total < (i64)block * vec * 64) vec = 1;  // small problem: favour more threads
     i64 groups = total / vec;
-    std::ostringstream o;
-    o << kPrelude << "\nextern \"C\" __global__ void __launch_bounds__(" << block << ") " << entry_ << "(" << signature(false) << ") {\n";
-    o << "  const int ug_g = (int)blockIdx.x * " << block << " + (int)threadIdx.x;\n";
-    o << "  if (ug_g >= " << groups << ") return;\n";
+    // Small kernels (the per-token elementwise work of a decode step, whose shapes follow the KV
+    // length) are emitted parametric so that a new shape does not mean a new hiprtc compile; large
+    // ones keep their constants, which lets the compiler strength-reduce the index arithmetic.
+    parametric_ = total <= (1 << 20) && !getenv("UGHIP_NO_PARAMETRIC");
+    kparams_.clear();
+    std::ostringstream b;
+    b << "  const int ug_g = (int)blockIdx.x * " << block << " + (int)threadIdx.x;\n";
+    b << "  if (ug_g >= " << (parametric_ ? kparam(groups) : std::to_string(groups)) << ") return;\n";
     // Items that depend on no loop are computed once per thread, ahead of the unrolled part.
     uint64_t all = 0;
     for (int l : chain_) all |= 1ull << l;
-    emit_items(o, false, all, 1, false, 1, true);
-    o << "#pragma unroll\n  for (int ug_u = 0; ug_u < " << vec << "; ++ug_u) {\n";
-    emit_decode(o, chain_, "ug_g", vec, 2);
-    emit_items(o, true, all, 2, false, 1, true);
-    o << "  }\n}\n";
+    emit_items(b, false, all, 1, false, 1, true);
+    b << "#pragma unroll\n  for (int ug_u = 0; ug_u < " << vec << "; ++ug_u) {\n";
+    emit_decode(b, chain_, "ug_g", vec, 2);
+    emit_items(b, true, all, 2, false, 1, true);
+    b << "  }\n}\n";
+    std::ostringstream o;
+    o << kPrelude << "\n";
+    std::string sig = signature(false);
+    if (parametric_) {
+      o << "struct ug_params { int v[" << kparams_.size() << "]; };\n";
+      sig += std::string(sig.empty() ? "" : ", ") + "const ug_params ug_k";
+      out_.kparams = kparams_;
+    }
+    o << "extern \"C\" __global__ void __launch_bounds__(" << block << ") " << entry_ << "(" << sig << ") {\n" << b.str();
+    parametric_ = false;
     out_.source = o.str();
     out_.strategy = UGHIP_STRAT_ELEMENTWISE;
     out_.block = block;

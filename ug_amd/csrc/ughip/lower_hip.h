@@ -19,6 +19,9 @@ struct Lowered {
   std::string entry2;
   unsigned grid2 = 0, block2 = 0;
   size_t scratch_part_bytes = 0;
+  // Parametric kernels: integer constants of the SSA, passed by value as the last kernel
+  // argument (`struct { int v[n]; }`) instead of being printed into the source.
+  std::vector<int> kparams;
   std::vector<int> arg_dtype;      // per kernel argument, UGHIP_* dtype
   std::vector<long long> min_len;  // per argument: 1 + largest offset the kernel forms, -1 if unknown
   std::vector<char> arg_written;   // per argument: has a Store

@@ -4,6 +4,7 @@
 // ug-core/src/cpu_runtime.rs:527-619).
 #include <hip/hip_runtime.h>
 
+#include "gemm.h"
 #include "internal.h"
 #include "ughip.h"
 
@@ -15,16 +16,6 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-
-struct MMArgs {
-  const void* a;
-  const void* b;
-  void* c;
-  int M, N, K;
-  long long a_rs, a_cs;  // lhs strides of (m, k)
-  long long b_rs, b_cs;  // rhs strides of (k, n)
-  long long a_bs, b_bs, c_bs;
-};
 
 // MFMA 32x32 accumulator layout: lane l, register i -> row (i/4)*8 + (l/32)*4 + i%4, col l%32.
 template <typename T>
@@ -267,6 +258,10 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
   const size_t vec = f32 ? 4 : 8;
   const bool gemv_ok = m <= 8 && k >= 256 && k % vec == 0 && p.a_cs == 1 && p.b_rs == 1 && p.a_rs % (long long)vec == 0 && p.b_cs % (long long)vec == 0 &&
                        p.a_bs % (long long)vec == 0 && p.b_bs % (long long)vec == 0 && lhs_offset % vec == 0 && rhs_offset % vec == 0;
+  if (!gemv_ok && gemm_tiled_supported(dst->dtype, p, b)) {
+    UGHIP_HIPCHK(gemm_tiled_launch(st, dst->dtype, p, b));
+    return UGHIP_OK;
+  }
   if (gemv_ok) {
     dim3 grid((unsigned)((n + 3) / 4), 1, (unsigned)b);
     if (f32) {

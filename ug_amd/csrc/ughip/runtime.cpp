@@ -125,6 +125,21 @@ int ughip_synchronize(ughip_device* dev) {
   return UGHIP_OK;
 }
 
+int ughip_device_set_zero_fill(ughip_device* dev, int on) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  dev->zero_fill = on != 0;
+  return UGHIP_OK;
+}
+
+int ughip_device_stats(ughip_device* dev, size_t* n_code_objects, size_t* pool_bytes, size_t* live_bytes) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  std::lock_guard<std::mutex> g(dev->mu);
+  if (n_code_objects) *n_code_objects = dev->modules.size();
+  if (pool_bytes) *pool_bytes = dev->pool_bytes;
+  if (live_bytes) *live_bytes = dev->live_bytes;
+  return UGHIP_OK;
+}
+
 int ughip_device_arch(ughip_device* dev, char* buf, size_t buf_len) {
   if (!dev || !buf || !buf_len) return set_error(UGHIP_ERR_INVALID, "bad arguments");
   snprintf(buf, buf_len, "%s", dev->arch.c_str());
@@ -167,7 +182,7 @@ int ughip_alloc(ughip_device* dev, int dtype, size_t len, ughip_slice** out) {
     }
     s->cap_bytes = cls;
     dev->live_bytes += cls;
-    HIPCHK(hipMemsetAsync(s->ptr, 0, bytes, dev->stream));
+    if (dev->zero_fill) HIPCHK(hipMemsetAsync(s->ptr, 0, bytes, dev->stream));
   }
   ughip_device_retain(dev);
   *out = s.release();
@@ -373,6 +388,7 @@ int ughip_run(ughip_device* dev, ughip_func* f, ughip_slice* const* args, size_t
   }
   size_t np = n_args;
   if (low.scratch_part_bytes) params[np++] = &f->scratch_part;
+  if (!low.kparams.empty()) params[np++] = const_cast<int*>(low.kparams.data());
   if (int rc = device_activate(dev)) return rc;
   HIPCHK(hipModuleLaunchKernel(f->function, low.grid, 1, 1, low.block, 1, 1, low.lds_bytes, dev->stream, params, nullptr));
   if (f->function2) HIPCHK(hipModuleLaunchKernel(f->function2, low.grid2, 1, 1, low.block2, 1, 1, 0, dev->stream, params, nullptr));
