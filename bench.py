@@ -140,23 +140,80 @@ def extras(dev, steps, warmup):
     _, ms = timed(dev, lambda: dev.matmul(dst, sa, sw, (b, m, m, m), lay, lay), steps, warmup)
     tf = flop * steps / (ms * 1e-3) / 1e12
     out["bmm_bf16_8x1024^3"] = {"TFLOP/s": round(tf, 2), "frac_mfma_bf16": round(tf / MFMA_BF16_PEAK_TF, 4), "us": round(ms * 1e3 / steps, 1)}
+    out.update(llama_pieces(dev, steps, warmup))
+    return out
+
+
+def llama_pieces(dev, steps, warmup):
+    """Config 4: the llama layer pieces at T=512, hidden 2048, 32 heads x 64 (f32), each as the lazy
+    graph ug-llama builds for it (ug-llama/src/model.rs:32-109,203-248), with its algorithmic bytes."""
+    import ug_amd
+    from ug_amd import LazyBuffer as LB, Schedule, rng
+    ll, ops = ug_amd.llama, ug_amd.LlamaOps.hip()
+    out = {}
+    t, hidden, heads, hd = 512, 2048, 32, 64
+
+    def hbm(name, lb, nbytes, keep=()):
+        cs = Schedule.create_one(lb).compile()
+        _, ms = timed(dev, cs.run, steps, warmup)
+        gbs = nbytes * steps / (ms * 1e-3) / 1e9
+        out[name] = {"GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "us": round(ms * 1e3 / steps, 2), "algorithmic_bytes": nbytes}
+
+    x = LB.copy(rng.normal(6, t * hidden), (1, t, hidden), dev)
+    alpha = LB.copy(rng.normal(6 + 100, hidden, 0.02), (hidden,), dev)
+    hbm("c4_rms_norm_512x2048", ll.rms_norm(x, alpha, 1e-5), 2 * 4 * t * hidden + 4 * hidden)
+    cfg = ug_amd.LlamaConfig()
+    cos, sin = ll.rope_tables(dev, cfg)
+    cos.realize()   # the tables are built once per model (ug-llama/src/model.rs:147-168), not per layer call
+    sin.realize()
+    q = LB.copy(rng.normal(7, heads * t * hd), (1, heads, t, hd), dev)
+    pos = LB.copy(np.zeros(1, np.int32), (1,), dev)
+    hbm("c4_rope_q_1x32x512x64", ops.rope(q, cos, sin, pos), 2 * 4 * heads * t * hd + 2 * 4 * t * (hd // 2))
+    s = LB.copy(rng.normal(8, heads * t * t), (1, heads, t, t), dev)
+    hbm("c4_causal_mask_1x32x512x512", ops.causal_mask(s), 2 * 4 * heads * t * t)
+    hbm("c4_softmax_lazy_1x32x512x512", ll.softmax(s), 2 * 4 * heads * t * t)
+    hbm("c4_softmax_custom_1x32x512x512", ops.custom_softmax(s), 2 * 4 * heads * t * t)
+    hbm("c4_mask_then_softmax_custom", ops.custom_softmax(ops.causal_mask(s)), 4 * 4 * heads * t * t)
+    gate = LB.copy(rng.normal(8 + 100, t * 5632), (1, t, 5632), dev)
+    up = LB.copy(rng.normal(8 + 101, t * 5632), (1, t, 5632), dev)
+    hbm("c4_silu_mul_512x5632", ll.silu(gate).binary("mul", up), 3 * 4 * t * 5632)
+
+    def gemm(name, lhs, rhs, transposed, b, m, n, k):
+        mm = lhs.matmul_t(rhs) if transposed else lhs.matmul(rhs)
+        cs = Schedule.create_one(mm).compile()
+        _, ms = timed(dev, cs.run, steps, warmup)
+        flop, nbytes = 2.0 * b * m * n * k, 4.0 * b * (m * k + k * n + m * n)
+        sec = ms * 1e-3 / steps
+        out[name] = {"TFLOP/s": round(flop / sec / 1e12, 2), "frac_mfma_f32": round(flop / sec / 1e12 / MFMA_F32_PEAK_TF, 4), "GB/s": round(nbytes / sec / 1e9, 1),
+                     "frac_hbm": round(nbytes / sec / 1e9 / HBM_PEAK_GBS, 4), "us": round(sec * 1e6, 2)}
+
+    kk = LB.copy(rng.normal(8 + 200, heads * t * hd), (1, heads, t, hd), dev)
+    v = LB.copy(rng.normal(8 + 300, heads * t * hd), (1, heads, t, hd), dev)
+    gemm("c4_qk_t_b32_512x512x64", q, kk, True, heads, t, t, hd)
+    gemm("c4_att_v_b32_512x64x512", s, v, False, heads, t, hd, t)
     return out
 
 
 def llama_decode(dev, n_prompt=128, n_steps=128):
+    """Config 5: TinyLlama-1.1B shape, random-init f32 weights, prefill 128 then 128 greedy steps.
+    Fresh buffers are not zero-filled here (every kernel of the model writes its whole output; the
+    ids are the same either way, which the GPU tests check)."""
     import ug_amd
     from ug_amd import rng
     cfg = ug_amd.LlamaConfig()
     ops = ug_amd.LlamaOps.hip()
+    dev.set_zero_fill(False)
     t0 = time.perf_counter()
     model = ug_amd.LlamaModel(dev, ops, cfg, custom_softmax=True, seed=9, std=0.02)
     load_s = time.perf_counter() - t0
     prompt = rng.token_ids(10, n_prompt, cfg.vocab_size)
+    model.generate(prompt, 4)          # compiles every kernel shape family once
     toks, st = model.generate(prompt, n_steps)
+    dev.set_zero_fill(True)
     weights_bytes = 4 * 1034512384
     tok_s = n_steps / (st["decode_ms"] * 1e-3)
     return {"tok/s": round(tok_s, 2), "decode_ms_per_token": round(st["decode_ms"] / n_steps, 3), "prefill_ms": round(st["prefill_ms"], 1),
-            "frac_hbm_weights_only": round(tok_s * weights_bytes / 1e9 / HBM_PEAK_GBS, 4), "load_s": round(load_s, 1), "dtype": "f32",
+            "frac_hbm_weights_only": round(tok_s * weights_bytes / 1e9 / HBM_PEAK_GBS, 4), "load_s": round(load_s, 1), "dtype": "f32", "zero_fill": False,
             "first_ids": toks[:8].tolist(), "min_top1_margin": float(st["margins"].min())}
 
 

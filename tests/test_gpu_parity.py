@@ -215,7 +215,8 @@ def test_cat(hip, cpu, hip_ops, cpu_ops, shape_l, shape_r, axis):
         np.testing.assert_array_equal(outs[0], np.concatenate([l.reshape(shape_l), r.reshape(shape_r)], axis=axis).ravel())
 
 
-@pytest.mark.parametrize("shape", [(1, 32, 1, 129), (1, 4, 16, 16), (2, 2, 33, 300), (1, 1, 3, 1024), (1, 1, 2, 2048), (1, 1, 2, 4096), (1, 1, 2, 10000),
+@pytest.mark.parametrize("shape", [(1, 32, 1, 129), (1, 4, 16, 16), (2, 2, 33, 300), (1, 1, 3, 1024), (1, 3, 5, 260), (1, 2, 9, 512), (1, 1, 7, 508),
+                                   (1, 8, 256, 1024), (1, 4, 520, 772), (1, 1, 2, 2048), (1, 1, 2, 4096), (1, 1, 2, 10000),
                                    (1, 1, 1, 16384), (1, 1, 1, 20000)])
 def test_custom_softmax(hip, cpu, hip_ops, cpu_ops, shape):
     x = rng.normal(10, int(np.prod(shape)), 3.0)
@@ -300,10 +301,12 @@ def _raw_matmul(hip, dtype, a, w, rhs_nk):
     return (rng.from_bf16_bits(out) if dtype == ug_amd.BF16 else out).reshape(b, m, n)
 
 
-# Shapes that are whole multiples of the 256 x 128 x (32 | 64) tile take the tuned MFMA kernel; the
-# neighbours that are one element off take the generic one.  Both are held to the same bound.
+# Shapes that are whole multiples of a 256x128, 128x128 or 128x64 tile (K a multiple of 32 f32 / 64
+# bf16) take the tuned MFMA kernel; neighbours one element off take the generic one.  Both are held
+# to the same bound.
 @pytest.mark.parametrize("rhs_nk", [False, True])
-@pytest.mark.parametrize("bmnk", [(2, 256, 128, 96), (1, 512, 384, 160), (3, 256, 256, 32), (1, 255, 128, 96), (1, 256, 129, 96)])
+@pytest.mark.parametrize("bmnk", [(2, 256, 128, 96), (1, 512, 384, 160), (3, 256, 256, 32), (1, 255, 128, 96), (1, 256, 129, 96),
+                                  (1, 128, 128, 64), (2, 128, 64, 96), (1, 384, 192, 64), (40, 256, 128, 32), (32, 512, 64, 512)])
 def test_matmul_f32_tile_multiples(hip, bmnk, rhs_nk):
     b, m, n, k = bmnk
     print("matmul f32", bmnk, "rhs_nk", rhs_nk, flush=True)
@@ -316,7 +319,8 @@ def test_matmul_f32_tile_multiples(hip, bmnk, rhs_nk):
 
 
 @pytest.mark.parametrize("rhs_nk", [False, True])
-@pytest.mark.parametrize("bmnk", [(2, 256, 128, 192), (1, 512, 384, 64), (3, 256, 256, 320), (1, 256, 128, 96), (1, 248, 128, 128)])
+@pytest.mark.parametrize("bmnk", [(2, 256, 128, 192), (1, 512, 384, 64), (3, 256, 256, 320), (1, 256, 128, 96), (1, 248, 128, 128),
+                                  (1, 128, 128, 64), (2, 128, 64, 128), (1, 384, 192, 192), (40, 256, 128, 64)])
 def test_matmul_bf16_tile_multiples(hip, bmnk, rhs_nk):
     b, m, n, k = bmnk
     print("matmul bf16", bmnk, "rhs_nk", rhs_nk, flush=True)
@@ -327,6 +331,51 @@ def test_matmul_bf16_tile_multiples(hip, bmnk, rhs_nk):
     # f32 accumulation of exact bf16 products, then one rounding to bf16 (2^-8 relative)
     bound = (2.0 ** -8) * np.abs(exact) + k * np.finfo(np.float32).eps * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64))
     assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-12)
+
+
+# The m <= 8 shapes of decode: wave-per-column GEMV with 1, 2 or 4 waves per column, the short-k
+# variant (attention scores) and the [k, n]-major variant (attention output).
+GEMV_SHAPES = [(1, 1, 2048, 2048), (1, 1, 5000, 512), (1, 1, 7000, 256), (1, 3, 640, 320), (2, 8, 300, 1024), (32, 1, 129, 64), (32, 1, 77, 128),
+               (4, 5, 33, 16), (1, 1, 256, 2048), (1, 2, 2048, 5632)]
+
+
+@pytest.mark.parametrize("bmnk", GEMV_SHAPES)
+def test_gemv_rhs_nk_f32(hip, bmnk):
+    b, m, n, k = bmnk
+    print("gemv nt f32", bmnk, flush=True)
+    a = rng.uniform_pm1(41, b * m * k).reshape(b, m, k)
+    w = rng.uniform_pm1(42, b * k * n).reshape(b, k, n)
+    got = _raw_matmul(hip, F32, a, w, True)
+    truth = a.astype(np.float64) @ w.astype(np.float64)
+    bound = k * np.finfo(np.float32).eps * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64))
+    assert np.all(np.abs(got - truth) <= bound + 1e-12)
+
+
+@pytest.mark.parametrize("bmnk", GEMV_SHAPES)
+def test_gemv_rhs_nk_bf16(hip, bmnk):
+    b, m, n, k = bmnk
+    print("gemv nt bf16", bmnk, flush=True)
+    a = rng.bf16_round(rng.uniform_pm1(43, b * m * k)).reshape(b, m, k)
+    w = rng.bf16_round(rng.uniform_pm1(44, b * k * n)).reshape(b, k, n)
+    got = _raw_matmul(hip, ug_amd.BF16, a, w, True)
+    exact = a.astype(np.float64) @ w.astype(np.float64)
+    bound = (2.0 ** -8) * np.abs(exact) + k * np.finfo(np.float32).eps * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64))
+    assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-12)
+
+
+@pytest.mark.parametrize("bmnk", [(32, 1, 64, 129), (32, 1, 64, 1), (2, 3, 100, 300), (1, 8, 64, 5), (3, 1, 256, 1000), (1, 4, 4, 64)])
+def test_gemv_rhs_kn_f32(hip, bmnk):
+    b, m, n, k = bmnk
+    print("gemv nn f32", bmnk, flush=True)
+    a = rng.uniform_pm1(45, b * m * k).reshape(b, m, k)
+    w = rng.uniform_pm1(46, b * k * n).reshape(b, k, n)
+    got = _raw_matmul(hip, F32, a, w, False)
+    truth = a.astype(np.float64) @ w.astype(np.float64)
+    bound = k * np.finfo(np.float32).eps * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64))
+    assert np.all(np.abs(got - truth) <= bound + 1e-12)
+    # the same integers through the generic kernel (n not a multiple of 4) agree exactly
+    ai, wi = np.floor(a * 8), np.floor(w * 8)
+    np.testing.assert_array_equal(_raw_matmul(hip, F32, ai, wi, False), (ai.astype(np.float64) @ wi.astype(np.float64)).astype(np.float32))
 
 
 def test_matmul_tiled_matches_generic_on_integers(hip):

@@ -326,6 +326,29 @@ LB Model::fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const 
 // One prefill call over the prompt, then `n_steps` greedy single-token steps (graph rebuilt per
 // step with a shared CompilationCache, as ug-llama/src/main.rs:124-146 does).  Returns the
 // n_steps + 1 argmax ids: one from the prefill logits, one per decode step.
+namespace {
+
+// One token step, built and compiled but not yet run.
+struct PreparedStep {
+  LB tokens, logits;
+  size_t t = 0, n_items = 0;
+  std::unique_ptr<CompiledSchedule> compiled;
+  double build_ms = 0, gen_ms = 0, comp_ms = 0;
+};
+
+double ms_between(std::chrono::steady_clock::time_point a, std::chrono::steady_clock::time_point b) {
+  return std::chrono::duration<double, std::milli>(b - a).count();
+}
+
+}  // namespace
+
+// The loop of ug-llama/src/main.rs:118-170 (rebuild the graph, schedule, compile against the cache,
+// run, read the logits back, argmax) with one change of order: the graph of step i+1 depends on the
+// position but not on the token value, so it is built, scheduled and compiled while the device is
+// still executing step i (on a second host thread when the device only queues work, so that it
+// also overlaps the launches of step i), and the token id is uploaded into its input buffer once
+// known.  Every value computed is the same as in the reference's order.
+// UG_LLAMA_NO_OVERLAP=1 keeps everything on the calling thread.
 std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32_t>& prompt, size_t n_steps, GenerateStats* stats) {
   using clock = std::chrono::steady_clock;
   const Config& cfg = model.config();
@@ -336,32 +359,89 @@ std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32
   CompilationCache ccache;
   std::vector<int32_t> out;
   std::vector<float> logits;
-  std::vector<int32_t> feed = prompt;
-  size_t pos_v = 0;
   const bool verbose = getenv("UG_LLAMA_VERBOSE") != nullptr;
-  for (size_t step = 0; step <= n_steps; ++step) {
-    auto t0 = clock::now();
-    size_t t = feed.size();
-    LB tokens = LB::copy(feed.data(), DType::I32, t, Shape({1, t}), dev);
+  const bool overlap = dev->runs_async() && getenv("UG_LLAMA_NO_OVERLAP") == nullptr;
+  // The rotary tables are shared by every step: realise them once, before two steps can be in
+  // preparation and in flight at the same time.
+  model.rope().cos.realize();
+  model.rope().sin.realize();
+
+  auto upload_inputs = [&](const std::vector<int32_t>& ids, size_t pos_v, PreparedStep& st, LB& pos) {
+    st.t = ids.size();
+    st.tokens = LB::copy(ids.data(), DType::I32, st.t, Shape({1, st.t}), dev);
     int32_t p32 = (int32_t)pos_v;
-    LB pos = LB::copy(&p32, DType::I32, 1, Shape({1, 1}), dev);
-    LB lg = model.fwd(tokens, pos, cache);
+    pos = LB::copy(&p32, DType::I32, 1, Shape({1, 1}), dev);
+  };
+  auto build = [&](PreparedStep& st, const LB& pos) {
+    auto t0 = clock::now();
+    st.logits = model.fwd(st.tokens, pos, cache);
     auto t1 = clock::now();
-    Schedule schedule = Schedule::create_one(lg);
+    Schedule schedule = Schedule::create_one(st.logits);
     auto t2 = clock::now();
-    CompiledSchedule compiled = schedule.compile_with_cache(ccache);
-    auto t3 = clock::now();
-    compiled.run();
-    auto t4 = clock::now();
-    logits.resize(lg.elem_count());
-    lg.data_vec(logits.data(), DType::F32);
-    if (verbose) {
-      // the per-token breakdown ug-llama prints with --verbose (main.rs:154-161)
-      auto ms_of = [](clock::time_point a, clock::time_point b) { return std::chrono::duration<double, std::milli>(b - a).count(); };
-      fprintf(stderr, "step %zu: build %.2fms, gen %.2fms, comp: %.2fms, run: %.2fms, sync+d2h: %.2fms, items %zu\n", step, ms_of(t0, t1),
-              ms_of(t1, t2), ms_of(t2, t3), ms_of(t3, t4), ms_of(t4, clock::now()), schedule.items().size());
+    st.compiled = std::make_unique<CompiledSchedule>(schedule.compile_with_cache(ccache));
+    st.n_items = schedule.items().size();
+    st.build_ms = ms_between(t0, t1);
+    st.gen_ms = ms_between(t1, t2);
+    st.comp_ms = ms_between(t2, clock::now());
+  };
+
+  size_t pos_v = 0;
+  PreparedStep cur, done;  // `done`: the previous step, kept until its graph can be freed off the critical path
+  auto t_step = clock::now();
+  {
+    LB pos;
+    upload_inputs(prompt, pos_v, cur, pos);
+    build(cur, pos);
+  }
+  for (size_t step = 0; step <= n_steps; ++step) {
+    const bool more = step < n_steps;
+    PreparedStep next;
+    LB next_pos;
+    // Host-to-device copies synchronise the stream: the inputs of the next step are uploaded
+    // before this step is queued (the token id is a placeholder until the argmax below).
+    if (more) upload_inputs({0}, pos_v + cur.t, next, next_pos);
+    // The cache buffers this step writes become leaves for the next graph: allocate them now and
+    // drop the graph behind them (the compiled schedule keeps what it needs alive), which also
+    // keeps the DAG from growing with every step.
+    for (Cache& c : cache) {
+      c.prev_k.maybe_allocate_uninit();
+      c.prev_v.maybe_allocate_uninit();
+      c.prev_k.detach();
+      c.prev_v.detach();
     }
-    const float* last = logits.data() + (t - 1) * cfg.vocab_size;
+    // The launches go to a second thread; this thread (whose allocator arena holds the graphs)
+    // prepares the next step meanwhile.
+    auto t0 = clock::now();
+    auto t1 = t0;
+    if (more && overlap) {
+      std::exception_ptr run_err;
+      std::thread launcher([&] {
+        try {
+          cur.compiled->run();
+        } catch (...) {
+          run_err = std::current_exception();
+        }
+        t1 = clock::now();
+      });
+      try {
+        build(next, next_pos);
+        done = PreparedStep();
+      } catch (...) {
+        launcher.join();
+        throw;
+      }
+      launcher.join();
+      if (run_err) std::rethrow_exception(run_err);
+    } else {
+      cur.compiled->run();
+      t1 = clock::now();
+      if (more) build(next, next_pos);
+    }
+    auto t2 = clock::now();
+    logits.resize(cur.logits.elem_count());
+    cur.logits.data_vec(logits.data(), DType::F32);
+    auto t3 = clock::now();
+    const float* last = logits.data() + (cur.t - 1) * cfg.vocab_size;
     size_t best = 0;
     float second = -INFINITY;
     for (size_t i = 1; i < cfg.vocab_size; ++i) {
@@ -372,7 +452,19 @@ std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32
         second = last[i];
       }
     }
-    double ms = std::chrono::duration<double, std::milli>(clock::now() - t0).count();
+    if (more) {
+      int32_t id = (int32_t)best;
+      next.tokens.data()->slice->copy_host_to_device(&id, DType::I32, 1);
+    }
+    auto t4 = clock::now();
+    if (verbose) {
+      // the per-token breakdown ug-llama prints with --verbose (main.rs:154-161)
+      fprintf(stderr, "step %zu: run %.2fms, next build %.2fms gen %.2fms comp %.2fms (%s), run+prepare %.2fms, sync+d2h %.2fms, argmax+h2d %.2fms, items %zu\n",
+              step, ms_between(t0, t1), next.build_ms, next.gen_ms, next.comp_ms, overlap ? "second thread" : "after the launches", ms_between(t0, t2),
+              ms_between(t2, t3), ms_between(t3, t4), cur.n_items);
+    }
+    double ms = ms_between(t_step, t4);
+    t_step = t4;
     if (stats) {
       if (step == 0) stats->prefill_ms = ms;
       else {
@@ -381,15 +473,10 @@ std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32
       }
       stats->top1_margin.push_back(last[best] - second);
     }
-    pos_v += t;
+    pos_v += cur.t;
     out.push_back((int32_t)best);
-    feed.assign(1, (int32_t)best);
-    // The caches are realised now; dropping the graph that produced them keeps the DAG from
-    // growing with every step.
-    for (Cache& c : cache) {
-      c.prev_k.detach();
-      c.prev_v.detach();
-    }
+    done = std::move(cur);
+    cur = std::move(next);
   }
   return out;
 }

@@ -76,6 +76,7 @@ class Model {
   LB fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const;
   const Config& config() const { return cfg_; }
   const ug::DevicePtr& device() const { return dev_; }
+  const Rope& rope() const { return rope_; }
 
  private:
   struct Layer {

@@ -38,6 +38,8 @@ struct Device {
                       const Layout& rhs_l) = 0;
   virtual bool use_grid() const = 0;
   virtual const char* name() const = 0;
+  // True when run/matmul only queue work (results are ready after synchronize or a copy back).
+  virtual bool runs_async() const { return false; }
 };
 
 }  // namespace ug

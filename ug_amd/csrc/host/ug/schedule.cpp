@@ -317,17 +317,19 @@ CompiledSchedule Schedule::compile_with_cache(CompilationCache& cache) const {
 
 // schedule.rs:234-305
 void CompiledSchedule::run() const {
+  std::vector<Slice*> bs;
   for (const CompiledFunc& f : funcs) {
     switch (f.kind) {
       case CompiledFunc::Kernel:
       case CompiledFunc::Custom: {
-        std::vector<Slice*> bs;
-        std::set<const DataCell*> borrowed;
+        bs.clear();
         for (const auto& a : f.args) {
           a.second.maybe_allocate_uninit();
           // RefCell::try_borrow_mut: a cell may appear once.
-          if (!borrowed.insert(a.second.data().get()).second) bail("already borrowed: BorrowMutError");
-          bs.push_back(a.second.data()->slice.get());
+          Slice* s = a.second.data()->slice.get();
+          for (Slice* seen : bs)
+            if (seen == s) bail("already borrowed: BorrowMutError");
+          bs.push_back(s);
         }
         if (f.kind == CompiledFunc::Kernel) device->run(*f.func, bs);
         else (*f.f)(bs);

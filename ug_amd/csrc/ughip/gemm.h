@@ -16,8 +16,8 @@ struct MMArgs {
   long long a_bs, b_bs, c_bs;
 };
 
-// Tuned kernel: 256x128 tiles, contiguous operands, M % 256 == 0, N % 128 == 0, K % 64 == 0
-// (bf16) / K % 32 == 0 (f32), rhs either [k, n] row-major or [n, k] row-major.
+// Tuned kernel: 256x128, 128x128 or 128x64 tiles that divide M x N, K % 64 == 0 (bf16) /
+// K % 32 == 0 (f32), lhs rows contiguous, rhs either [k, n] row-major or [n, k] row-major.
 bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch);
 hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch);
 

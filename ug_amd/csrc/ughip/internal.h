@@ -5,6 +5,8 @@
 #include <atomic>
 #include <map>
 #include <mutex>
+#include <vector>
+#include <unordered_map>
 #include <string>
 
 #include "ughip.h"
@@ -22,7 +24,7 @@ struct ughip_device {
   int num_cus = 0;
   std::mutex mu;
   // Size-class free lists: freed blocks are reused by later allocations on the same stream.
-  std::multimap<size_t, void*> pool;
+  std::unordered_map<size_t, std::vector<void*>> pool;  // free blocks by size class
   size_t pool_bytes = 0, live_bytes = 0;
   bool zero_fill = true;
   std::map<std::string, CachedModule> modules;  // generated source -> loaded code object

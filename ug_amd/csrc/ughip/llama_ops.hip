@@ -114,6 +114,42 @@ __global__ void __launch_bounds__(256) softmax_rows_wave(const float* __restrict
   }
 }
 
+// Wave per row with 128-bit accesses (4 rows per workgroup): n_cols % 4 == 0, n_cols <= 256 * V.
+// No LDS and no barrier: both reductions stay inside the wave.
+template <int V>
+__global__ void __launch_bounds__(256) softmax_rows_wave_v4(const float* __restrict__ src, float* __restrict__ dst, int n_rows, int n_cols) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= n_rows) return;
+  const int lane = threadIdx.x & 63, n4 = n_cols >> 2;
+  const float4* s4 = reinterpret_cast<const float4*>(src + (size_t)row * n_cols);
+  float4* d4 = reinterpret_cast<float4*>(dst + (size_t)row * n_cols);
+  float4 x[V];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const int c = lane + i * 64;
+    x[i] = c < n4 ? s4[c] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    m = fmaxf(fmaxf(m, fmaxf(x[i].x, x[i].y)), fmaxf(x[i].z, x[i].w));
+  }
+  m = wave_max(m);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    // columns past the row end hold -inf and contribute exp(-inf) = 0
+    x[i].x = expf(x[i].x - m);
+    x[i].y = expf(x[i].y - m);
+    x[i].z = expf(x[i].z - m);
+    x[i].w = expf(x[i].w - m);
+    sum += (x[i].x + x[i].y) + (x[i].z + x[i].w);
+  }
+  sum = wave_sum(sum);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const int c = lane + i * 64;
+    if (c < n4) d4[c] = make_float4(x[i].x / sum, x[i].y / sum, x[i].z / sum, x[i].w / sum);
+  }
+}
+
 // Any row length: three passes over the row (the re-reads hit L2 for rows of this size).
 __global__ void __launch_bounds__(1024) softmax_rows_generic(const float* __restrict__ src, float* __restrict__ dst, int n_cols) {
   __shared__ float lds[16];
@@ -272,7 +308,13 @@ int ughip_softmax_rows(ughip_device* dev, const ughip_slice* src, ughip_slice* d
   float* d = static_cast<float*>(dst->ptr);
   hipStream_t st = dev->stream;
   const int nc = (int)n_cols, nr = (int)n_rows;
-  if (n_cols <= 256) {
+  if (n_cols % 4 == 0 && n_cols <= 256) {
+    softmax_rows_wave_v4<1><<<blocks_for(n_rows, 4), 256, 0, st>>>(s, d, nr, nc);
+  } else if (n_cols % 4 == 0 && n_cols <= 512) {
+    softmax_rows_wave_v4<2><<<blocks_for(n_rows, 4), 256, 0, st>>>(s, d, nr, nc);
+  } else if (n_cols % 4 == 0 && n_cols <= 1024 && n_rows >= 2048) {
+    softmax_rows_wave_v4<4><<<blocks_for(n_rows, 4), 256, 0, st>>>(s, d, nr, nc);
+  } else if (n_cols <= 256) {
     softmax_rows_wave<4><<<blocks_for(n_rows, 4), 256, 0, st>>>(s, d, nr, nc);
   } else if (n_cols % 4 != 0 || n_cols > 16384) {
     softmax_rows_generic<<<nr, 1024, 0, st>>>(s, d, nc);

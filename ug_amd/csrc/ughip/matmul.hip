@@ -123,70 +123,228 @@ __global__ void __launch_bounds__(256) gemm_bf16_any(MMArgs p) {
   store_acc(C, acc, m0 + wm, n0 + wn + (lane & 31), p.M, p.N, lane);
 }
 
-// ---- GEMV for decode: y[r, n] = sum_k x[r, k] * W[n, k], rows r < R <= 8 --------------------------------
-// One wave per output column; K is walked with 128-bit loads by the 64 lanes, so W is streamed
-// from HBM exactly once and x comes from L2.  Needs x and W contiguous along k and K % VEC == 0.
+// ---- GEMV kernels for the m <= 8 rows of decode ---------------------------------------------------
+// All of them stream the big operand from HBM exactly once with 128-bit loads (x comes from L2),
+// accumulate in f32 and reduce in a fixed order, so results do not change from run to run.
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
   return v;
 }
 
-template <int R>
-__global__ void __launch_bounds__(256) gemv_nt_f32(MMArgs p) {
-  const int lane = threadIdx.x & 63;
-  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (n >= p.N) return;
-  const float* __restrict__ X = static_cast<const float*>(p.a) + (size_t)blockIdx.z * p.a_bs;
-  const float* __restrict__ W = static_cast<const float*>(p.b) + (size_t)blockIdx.z * p.b_bs + (size_t)n * p.b_cs;
-  float* __restrict__ Y = static_cast<float*>(p.c) + (size_t)blockIdx.z * p.c_bs;
+template <typename T>
+struct Vec;
+template <>
+struct Vec<float> {
+  typedef floatx4 type;
+  static constexpr int N = 4;
+};
+template <>
+struct Vec<__bf16> {
+  typedef bf16x8 type;
+  static constexpr int N = 8;
+};
+
+template <typename T>
+__device__ __forceinline__ float dot_vec(const typename Vec<T>::type& w, const typename Vec<T>::type& x, float acc) {
+#pragma unroll
+  for (int j = 0; j < Vec<T>::N; ++j) acc += (float)w[j] * (float)x[j];
+  return acc;
+}
+
+// y[r, n] = sum_k x[r, k] * W[n, k] (rhs stored [n, k]).  KS waves share one column, each walking
+// every KS-th 64-lane slab of k with four loads in flight per lane; a workgroup covers 4 / KS
+// columns.  Short matrices take KS = 4 so that enough waves are in flight to cover HBM latency.
+template <typename T, int R, int KS>
+__global__ void __launch_bounds__(256) gemv_nt(MMArgs p) {
+  typedef typename Vec<T>::type V;
+  constexpr int VE = Vec<T>::N;
+  __shared__ float part[4][R];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = blockIdx.x * (4 / KS) + wave / KS, ks = wave % KS;
+  const bool live = n < p.N;
   float acc[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) acc[r] = 0.f;
-  for (int k = lane * 4; k < p.K; k += 256) {
-    const float4 w = *reinterpret_cast<const float4*>(W + k);
+  if (live) {
+    const T* __restrict__ X = static_cast<const T*>(p.a) + (size_t)blockIdx.z * p.a_bs;
+    const T* __restrict__ W = static_cast<const T*>(p.b) + (size_t)blockIdx.z * p.b_bs + (size_t)n * p.b_cs;
+    constexpr int stride = 64 * VE * KS;
+    int k = (ks * 64 + lane) * VE;
+    for (; k + 3 * stride < p.K; k += 4 * stride) {
+      const V w0 = *reinterpret_cast<const V*>(W + k), w1 = *reinterpret_cast<const V*>(W + k + stride);
+      const V w2 = *reinterpret_cast<const V*>(W + k + 2 * stride), w3 = *reinterpret_cast<const V*>(W + k + 3 * stride);
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      if (r < p.M) {
-        const float4 x = *reinterpret_cast<const float4*>(X + (size_t)r * p.a_rs + k);
-        acc[r] += (w.x * x.x + w.y * x.y) + (w.z * x.z + w.w * x.w);
+      for (int r = 0; r < R; ++r) {
+        if (r < p.M) {
+          const T* Xr = X + (size_t)r * p.a_rs + k;
+          acc[r] = dot_vec<T>(w0, *reinterpret_cast<const V*>(Xr), acc[r]);
+          acc[r] = dot_vec<T>(w1, *reinterpret_cast<const V*>(Xr + stride), acc[r]);
+          acc[r] = dot_vec<T>(w2, *reinterpret_cast<const V*>(Xr + 2 * stride), acc[r]);
+          acc[r] = dot_vec<T>(w3, *reinterpret_cast<const V*>(Xr + 3 * stride), acc[r]);
+        }
       }
+    }
+    for (; k < p.K; k += stride) {
+      const V w = *reinterpret_cast<const V*>(W + k);
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (r < p.M) acc[r] = dot_vec<T>(w, *reinterpret_cast<const V*>(X + (size_t)r * p.a_rs + k), acc[r]);
     }
   }
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    float s = wave_sum(acc[r]);
-    if (lane == 0 && r < p.M) Y[(size_t)r * p.N + n] = s;
+  for (int r = 0; r < R; ++r) acc[r] = wave_sum(acc[r]);
+  T* __restrict__ Y = static_cast<T*>(p.c) + (size_t)blockIdx.z * p.c_bs;
+  if (KS == 1) {
+    if (live && lane == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (r < p.M) Y[(size_t)r * p.N + n] = (T)acc[r];
+    }
+  } else {
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) part[wave][r] = acc[r];
+    }
+    __syncthreads();
+    if (live && ks == 0 && lane == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        if (r < p.M) {
+          float s = part[wave][r];
+#pragma unroll
+          for (int j = 1; j < KS; ++j) s += part[wave + j][r];
+          Y[(size_t)r * p.N + n] = (T)s;
+        }
+      }
+    }
   }
 }
 
-template <int R>
-__global__ void __launch_bounds__(256) gemv_nt_bf16(MMArgs p) {
-  const int lane = threadIdx.x & 63;
-  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (n >= p.N) return;
-  const __bf16* __restrict__ X = static_cast<const __bf16*>(p.a) + (size_t)blockIdx.z * p.a_bs;
-  const __bf16* __restrict__ W = static_cast<const __bf16*>(p.b) + (size_t)blockIdx.z * p.b_bs + (size_t)n * p.b_cs;
-  __bf16* __restrict__ Y = static_cast<__bf16*>(p.c) + (size_t)blockIdx.z * p.c_bs;
+// Same product for short k (attention scores of one query: k = head size): 16 lanes per column,
+// 16 columns per workgroup, no LDS.
+template <typename T, int R>
+__global__ void __launch_bounds__(256) gemv_nt_short_k(MMArgs p) {
+  typedef typename Vec<T>::type V;
+  constexpr int VE = Vec<T>::N;
+  const int lane = threadIdx.x & 63, sub = lane & 15;
+  const int n = blockIdx.x * 16 + (threadIdx.x >> 4);
+  const bool live = n < p.N;
   float acc[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) acc[r] = 0.f;
-  for (int k = lane * 8; k < p.K; k += 512) {
-    const bf16x8 w = *reinterpret_cast<const bf16x8*>(W + k);
+  if (live) {
+    const T* __restrict__ X = static_cast<const T*>(p.a) + (size_t)blockIdx.z * p.a_bs;
+    const T* __restrict__ W = static_cast<const T*>(p.b) + (size_t)blockIdx.z * p.b_bs + (size_t)n * p.b_cs;
+    for (int k = sub * VE; k < p.K; k += 16 * VE) {
+      const V w = *reinterpret_cast<const V*>(W + k);
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (r < p.M) acc[r] = dot_vec<T>(w, *reinterpret_cast<const V*>(X + (size_t)r * p.a_rs + k), acc[r]);
+    }
+  }
+  T* __restrict__ Y = static_cast<T*>(p.c) + (size_t)blockIdx.z * p.c_bs;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float v = acc[r];
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    if (live && sub == 0 && r < p.M) Y[(size_t)r * p.N + n] = (T)v;
+  }
+}
+
+// y[r, n] = sum_k x[r, k] * B[k, n] with B stored [k, n] (attention output of one query: k = the
+// sequence).  A workgroup of 1024 threads owns 64 columns: 16 lanes read one 256-byte row segment,
+// 64 row slices run in parallel, partial sums meet through LDS.  f32 only, N % 4 == 0.
+template <int R>
+__global__ void __launch_bounds__(1024) gemv_nn_f32(MMArgs p) {
+  __shared__ floatx4 part[16][16][R];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c4 = tid & 15, ksl = tid >> 4;
+  const int n = blockIdx.x * 64 + c4 * 4;
+  const bool live = n < p.N;
+  floatx4 acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = floatx4{0.f, 0.f, 0.f, 0.f};
+  if (live) {
+    const float* __restrict__ X = static_cast<const float*>(p.a) + (size_t)blockIdx.z * p.a_bs;
+    const float* __restrict__ B = static_cast<const float*>(p.b) + (size_t)blockIdx.z * p.b_bs + n;
+    int k = ksl;
+    for (; k + 192 < p.K; k += 256) {
+      const floatx4 b0 = *reinterpret_cast<const floatx4*>(B + (size_t)k * p.b_rs);
+      const floatx4 b1 = *reinterpret_cast<const floatx4*>(B + (size_t)(k + 64) * p.b_rs);
+      const floatx4 b2 = *reinterpret_cast<const floatx4*>(B + (size_t)(k + 128) * p.b_rs);
+      const floatx4 b3 = *reinterpret_cast<const floatx4*>(B + (size_t)(k + 192) * p.b_rs);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        if (r < p.M) {
+          const float* Xr = X + (size_t)r * p.a_rs + k;
+          acc[r] += Xr[0] * b0;
+          acc[r] += Xr[64] * b1;
+          acc[r] += Xr[128] * b2;
+          acc[r] += Xr[192] * b3;
+        }
+      }
+    }
+    for (; k < p.K; k += 64) {
+      const floatx4 b0 = *reinterpret_cast<const floatx4*>(B + (size_t)k * p.b_rs);
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (r < p.M) acc[r] += X[(size_t)r * p.a_rs + k] * b0;
+    }
+  }
+  // the 4 row slices of one wave (lanes 16 apart), then the 16 waves in order
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      float v = acc[r][c];
+      v += __shfl_xor(v, 16, 64);
+      v += __shfl_xor(v, 32, 64);
+      acc[r][c] = v;
+    }
+    if (lane < 16) part[wave][lane][r] = acc[r];
+  }
+  __syncthreads();
+  if (tid < 16 && live) {
+    float* __restrict__ Y = static_cast<float*>(p.c) + (size_t)blockIdx.z * p.c_bs;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       if (r < p.M) {
-        const bf16x8 x = *reinterpret_cast<const bf16x8*>(X + (size_t)r * p.a_rs + k);
+        floatx4 s = part[0][tid][r];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[r] += (float)w[j] * (float)x[j];
+        for (int w = 1; w < 16; ++w) s += part[w][tid][r];
+        *reinterpret_cast<floatx4*>(Y + (size_t)r * p.N + n) = s;
       }
     }
   }
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-    float s = wave_sum(acc[r]);
-    if (lane == 0 && r < p.M) Y[(size_t)r * p.N + n] = (__bf16)s;
+}
+
+template <typename T, int KS>
+void launch_gemv_nt(hipStream_t st, const MMArgs& p, size_t b) {
+  dim3 grid((unsigned)((p.N + 4 / KS - 1) / (4 / KS)), 1, (unsigned)b);
+  if (p.M == 1) gemv_nt<T, 1, KS><<<grid, 256, 0, st>>>(p);
+  else if (p.M <= 4) gemv_nt<T, 4, KS><<<grid, 256, 0, st>>>(p);
+  else gemv_nt<T, 8, KS><<<grid, 256, 0, st>>>(p);
+}
+
+template <typename T>
+void launch_gemv_nt_any(hipStream_t st, const MMArgs& p, size_t b) {
+  constexpr int VE = Vec<T>::N;
+  if (p.K < 64 * VE) {
+    dim3 grid((unsigned)((p.N + 15) / 16), 1, (unsigned)b);
+    if (p.M == 1) gemv_nt_short_k<T, 1><<<grid, 256, 0, st>>>(p);
+    else if (p.M <= 4) gemv_nt_short_k<T, 4><<<grid, 256, 0, st>>>(p);
+    else gemv_nt_short_k<T, 8><<<grid, 256, 0, st>>>(p);
+    return;
   }
+  // enough waves to hide HBM latency: about 8192 over the chip
+  const size_t cols = (size_t)p.N * b;
+  int ks = cols <= 2048 ? 4 : cols <= 6144 ? 2 : 1;
+  while (ks > 1 && p.K < 64 * VE * ks) ks >>= 1;
+  if (ks == 4) launch_gemv_nt<T, 4>(st, p, b);
+  else if (ks == 2) launch_gemv_nt<T, 2>(st, p, b);
+  else launch_gemv_nt<T, 1>(st, p, b);
 }
 
 // Batch stride of one operand: cpu_runtime.rs:527-549 / ug-cuda/src/gemm.rs:59-74.
@@ -256,26 +414,27 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
   const bool f32 = dst->dtype == UGHIP_F32;
   hipStream_t st = dev->stream;
   const size_t vec = f32 ? 4 : 8;
-  const bool gemv_ok = m <= 8 && k >= 256 && k % vec == 0 && p.a_cs == 1 && p.b_rs == 1 && p.a_rs % (long long)vec == 0 && p.b_cs % (long long)vec == 0 &&
-                       p.a_bs % (long long)vec == 0 && p.b_bs % (long long)vec == 0 && lhs_offset % vec == 0 && rhs_offset % vec == 0;
-  if (!gemv_ok && gemm_tiled_supported(dst->dtype, p, b)) {
+  // m <= 8: GEMV kernels.  Vector loads need 16-byte aligned rows; strides of size-1 dims are never used.
+  const long long lv = (long long)vec;
+  const bool small_m = m <= 8 && p.a_cs == 1 && b <= 65535;
+  const bool lhs_vec_ok = (m == 1 || p.a_rs % lv == 0) && (b == 1 || p.a_bs % lv == 0) && lhs_offset % vec == 0;
+  const bool rhs_vec_ok = (b == 1 || p.b_bs % lv == 0) && rhs_offset % vec == 0;
+  const bool gemv_nt_ok = small_m && lhs_vec_ok && rhs_vec_ok && k % vec == 0 && p.b_rs == 1 && (n == 1 || p.b_cs % lv == 0);
+  const bool gemv_nn_ok = small_m && f32 && rhs_vec_ok && n % 4 == 0 && p.b_cs == 1 && (k == 1 || p.b_rs % 4 == 0);
+  if (gemv_nt_ok) {
+    if (f32) launch_gemv_nt_any<float>(st, p, b);
+    else launch_gemv_nt_any<__bf16>(st, p, b);
+  } else if (gemv_nn_ok) {
+    dim3 grid((unsigned)((n + 63) / 64), 1, (unsigned)b);
+    if (m == 1) gemv_nn_f32<1><<<grid, 1024, 0, st>>>(p);
+    else if (m <= 4) gemv_nn_f32<4><<<grid, 1024, 0, st>>>(p);
+    else gemv_nn_f32<8><<<grid, 1024, 0, st>>>(p);
+  } else if (gemm_tiled_supported(dst->dtype, p, b)) {
     UGHIP_HIPCHK(gemm_tiled_launch(st, dst->dtype, p, b));
     return UGHIP_OK;
-  }
-  if (gemv_ok) {
-    dim3 grid((unsigned)((n + 3) / 4), 1, (unsigned)b);
-    if (f32) {
-      if (m == 1) gemv_nt_f32<1><<<grid, 256, 0, st>>>(p);
-      else if (m <= 4) gemv_nt_f32<4><<<grid, 256, 0, st>>>(p);
-      else gemv_nt_f32<8><<<grid, 256, 0, st>>>(p);
-    } else {
-      if (m == 1) gemv_nt_bf16<1><<<grid, 256, 0, st>>>(p);
-      else if (m <= 4) gemv_nt_bf16<4><<<grid, 256, 0, st>>>(p);
-      else gemv_nt_bf16<8><<<grid, 256, 0, st>>>(p);
-    }
   } else {
     dim3 grid((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64), (unsigned)b);
-    if (grid.y > 65535) return set_error(UGHIP_ERR_INVALID, "matmul: m too large for this kernel");
+    if (grid.y > 65535 || b > 65535) return set_error(UGHIP_ERR_INVALID, "matmul: m or batch too large for this kernel");
     if (f32) gemm_f32_any<<<grid, 256, 0, st>>>(p);
     else gemm_bf16_any<<<grid, 256, 0, st>>>(p);
   }

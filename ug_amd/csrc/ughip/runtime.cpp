@@ -111,7 +111,8 @@ int ughip_device_release(ughip_device* dev) {
   if (dev->refs.fetch_sub(1) != 1) return UGHIP_OK;
   hipSetDevice(dev->ordinal);
   hipStreamSynchronize(dev->stream);
-  for (auto& kv : dev->pool) hipFree(kv.second);
+  for (auto& kv : dev->pool)
+    for (void* p : kv.second) hipFree(p);
   for (auto& kv : dev->modules) hipModuleUnload(kv.second.module);
   hipStreamDestroy(dev->stream);
   delete dev;
@@ -161,9 +162,9 @@ int ughip_alloc(ughip_device* dev, int dtype, size_t len, ughip_slice** out) {
     {
       std::lock_guard<std::mutex> g(dev->mu);
       auto it = dev->pool.find(cls);
-      if (it != dev->pool.end()) {
-        s->ptr = it->second;
-        dev->pool.erase(it);
+      if (it != dev->pool.end() && !it->second.empty()) {
+        s->ptr = it->second.back();
+        it->second.pop_back();
         dev->pool_bytes -= cls;
       }
     }
@@ -173,7 +174,8 @@ int ughip_alloc(ughip_device* dev, int dtype, size_t len, ughip_slice** out) {
         // Give cached blocks back to the driver and retry once.
         std::lock_guard<std::mutex> g(dev->mu);
         hipStreamSynchronize(dev->stream);
-        for (auto& kv : dev->pool) hipFree(kv.second);
+        for (auto& kv : dev->pool)
+          for (void* p : kv.second) hipFree(p);
         dev->pool.clear();
         dev->pool_bytes = 0;
         e = hipMalloc(&s->ptr, cls);
@@ -181,7 +183,10 @@ int ughip_alloc(ughip_device* dev, int dtype, size_t len, ughip_slice** out) {
       }
     }
     s->cap_bytes = cls;
-    dev->live_bytes += cls;
+    {
+      std::lock_guard<std::mutex> g(dev->mu);
+      dev->live_bytes += cls;
+    }
     if (dev->zero_fill) HIPCHK(hipMemsetAsync(s->ptr, 0, bytes, dev->stream));
   }
   ughip_device_retain(dev);
@@ -194,7 +199,7 @@ int ughip_free(ughip_slice* s) {
   ughip_device* dev = s->dev;
   if (s->ptr) {
     std::lock_guard<std::mutex> g(dev->mu);
-    dev->pool.emplace(s->cap_bytes, s->ptr);
+    dev->pool[s->cap_bytes].push_back(s->ptr);
     dev->pool_bytes += s->cap_bytes;
     dev->live_bytes -= s->cap_bytes;
   }
