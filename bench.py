@@ -5,10 +5,11 @@ Headline (the JSON line): BASELINE config 2 -- sum(a*b + 0.5*a) over two f32 vec
 2^24, built as one lazy graph, scheduled and lowered like ug does, run on the HIP device.  A "step"
 is one run of the compiled schedule (one kernel launch) with a and b resident in HBM.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--extras] [--llama]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--headline-only]
 
---extras adds the other single-GPU configs (softmax sweep, batched matmul, llama pieces) under
-"extras"; --llama adds the config-5 decode run.  Only one GPU is ever used.
+The other single-GPU configs (softmax sweep, batched matmul, llama pieces, llama decode) are
+reported under "extras" of the same line; --headline-only (or --no-extras / --no-llama) leaves
+them out, which is what the profiler runs use.  Only one GPU is ever used.
 """
 import argparse
 import ctypes as C
@@ -93,7 +94,7 @@ def cpu_baseline(a, b, truth, budget_s=12.0):
         cs.run()
         passes += 1
         el = time.perf_counter() - t0
-        if el > budget_s or passes >= 2000:
+        if el > budget_s or passes >= 100000:
             break
     return {"value": round(ALGO_BYTES * passes / el / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": f"{passes} passes of the full 2^24-element workload in {el:.1f} s (oracle/: C emitted as ug-core/src/cpu_code_gen.rs does, "
@@ -101,8 +102,19 @@ def cpu_baseline(a, b, truth, budget_s=12.0):
             "host_cpus": os.cpu_count()}
 
 
-def extras(dev, steps, warmup):
+def extras(dev, steps, warmup, only=None):
     """Other single-GPU configs of BASELINE.json: GB/s or TFLOP/s with the roofline fraction."""
+    out = {}
+    if only in (None, "softmax"):
+        out.update(softmax_sweep(dev, steps, warmup))
+    if only in (None, "bmm"):
+        out.update(bmm(dev, steps, warmup))
+    if only in (None, "llama_pieces"):
+        out.update(llama_pieces(dev, steps, warmup))
+    return out
+
+
+def softmax_sweep(dev, steps, warmup):
     import ug_amd
     from ug_amd import LazyBuffer as LB, Schedule, rng
     out = {}
@@ -123,7 +135,14 @@ def extras(dev, steps, warmup):
         gbs = 8.0 * rows * cols * steps / (ms * 1e-3) / 1e9
         out[f"softmax_custom_{rows}x{cols}"] = {"GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "us_per_softmax": round(ms * 1e3 / steps, 2),
                                                "launches": 1}
-    # config 3: batched matmul 8 x 1024^3
+    return out
+
+
+def bmm(dev, steps, warmup):
+    """Config 3: batched matmul 8 x 1024^3, f32 through the lazy graph and bf16 through Device::matmul."""
+    import ug_amd
+    from ug_amd import LazyBuffer as LB, Schedule, rng
+    out = {}
     b, m = 8, 1024
     flop = 2.0 * b * m * m * m
     a = rng.uniform_pm1(4, b * m * m)
@@ -140,7 +159,6 @@ def extras(dev, steps, warmup):
     _, ms = timed(dev, lambda: dev.matmul(dst, sa, sw, (b, m, m, m), lay, lay), steps, warmup)
     tf = flop * steps / (ms * 1e-3) / 1e12
     out["bmm_bf16_8x1024^3"] = {"TFLOP/s": round(tf, 2), "frac_mfma_bf16": round(tf / MFMA_BF16_PEAK_TF, 4), "us": round(ms * 1e3 / steps, 1)}
-    out.update(llama_pieces(dev, steps, warmup))
     return out
 
 
@@ -222,8 +240,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--extras", action="store_true")
-    ap.add_argument("--llama", action="store_true")
+    ap.add_argument("--extras", action="store_true", help="(default) kept for older command lines")
+    ap.add_argument("--llama", action="store_true", help="(default) kept for older command lines")
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--no-llama", action="store_true")
+    ap.add_argument("--headline-only", action="store_true", help="only the config-2 kernel: no extras, no llama, no CPU baseline")
+    ap.add_argument("--only", choices=["softmax", "bmm", "llama_pieces", "llama"], help="besides the headline, run just this group (profiler runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true", help="also run a plain 2^24-element copy kernel (counter calibration)")
     args = ap.parse_args()
@@ -267,12 +289,24 @@ def main():
         _, cms = timed(dev, ccs.run, args.steps, args.warmup)
         line["copy_probe"] = {"kernel": ccs.funcs()[0]["info"], "bytes_read": 4 * N, "bytes_written": 4 * N,
                               "GB/s": round(8.0 * N * args.steps / (cms * 1e-3) / 1e9, 1)}
-    if not args.no_cpu_baseline:
+    if args.only:
+        args.no_cpu_baseline = True
+        args.no_extras = args.only == "llama"
+        args.no_llama = args.only != "llama"
+    if not (args.no_cpu_baseline or args.headline_only):
         line["cpu_baseline"] = cpu_baseline(a, b, truth)
-    if args.extras:
-        line["extras"] = extras(dev, max(20, args.steps // 4), args.warmup)
-    if args.llama:
-        line.setdefault("extras", {})["llama_decode_f32"] = llama_decode(dev)
+    del keep, cs, r
+    # The other configs ride along; a failure there is reported, it does not take the headline down.
+    if not (args.no_extras or args.headline_only):
+        try:
+            line["extras"] = extras(dev, max(20, args.steps // 4), args.warmup, None if args.only in (None, "llama") else args.only)
+        except Exception as e:  # noqa: BLE001
+            line["extras"] = {"error": f"{type(e).__name__}: {e}"}
+    if not (args.no_llama or args.headline_only):
+        try:
+            line.setdefault("extras", {})["llama_decode_f32"] = llama_decode(dev)
+        except Exception as e:  # noqa: BLE001
+            line.setdefault("extras", {})["llama_decode_f32"] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(line), flush=True)
 
 

@@ -1,11 +1,12 @@
 // Tuned MFMA GEMM for gfx950: C[b] = A[b] x B[b], f32 accumulate.
 //
-//   block tile BM x BN (256x128, 128x128 or 128x64), 4 waves (2 x 2), each wave owns a
-//   (BM/2) x (BN/2) block of MFMA 32x32 accumulators
-//   K tile = 128 bytes per matrix row (64 bf16 / 32 f32), double-buffered in LDS, the next tile
-//   prefetched into registers while the current one feeds the matrix cores
-//   LDS rows are 8 chunks of 16 bytes, chunk' = chunk ^ (row & 7): every 128-bit fragment read and
-//   every staging write is bank-conflict free
+//   block tile BM x BN: 256x128 with 8 waves (4 x 2, two per SIMD), 128x128 or 128x64 with 4 waves
+//   (2 x 2); each wave owns a block of MFMA 32x32 accumulators
+//   K tile = 128 bytes per matrix row (64 bf16 / 32 f32), double-buffered in LDS; global loads run
+//   two tiles ahead through two register sets, LDS staging stores and fragment reads are spread
+//   between the MFMAs of the tile being multiplied
+//   LDS rows are 8 chunks of 16 bytes, chunk' = chunk ^ ((row / 2) & 7): every 128-bit fragment read
+//   and every staging write is bank-conflict free on the 64-bank LDS
 //   a row-major B ([k, n]) is transposed in registers on its way to LDS so that both MFMA
 //   operands read 128 bits of consecutive k (v_perm_b32 for bf16; free for f32)
 //   tiles are handed to workgroups XCD by XCD so that the tiles of one batch element share an L2
@@ -14,6 +15,8 @@
 // f32:  v_mfma_f32_32x32x2_f32   (lane l feeds row/col l%32, k = l/32); the 4 floats of a 128-bit
 //       fragment feed 4 consecutive MFMAs, lanes 0-31 holding k..k+3 and lanes 32-63 k+4..k+7.
 #include <hip/hip_runtime.h>
+
+#include <cstdlib>
 
 #include "gemm.h"
 #include "ughip.h"
@@ -42,29 +45,33 @@ struct Elt<__bf16> {
   static constexpr int BK = 64, VE = 8;
 };
 
-__device__ __forceinline__ int lds_idx(int row, int chunk) { return row * CHUNKS + (chunk ^ (row & 7)); }
+// 64 banks x 4 bytes: two 128-byte rows span the banks once, so the chunk is rotated by row / 2 --
+// 16 lanes reading one chunk column of 16 consecutive rows then touch 16 different bank groups.
+__device__ __forceinline__ int lds_swz(int row) { return (row >> 1) & 7; }
+__device__ __forceinline__ int lds_idx(int row, int chunk) { return row * CHUNKS + (chunk ^ lds_swz(row)); }
 
 // The tile being prefetched from global memory while the previous one is multiplied.
-template <int BM>
+template <int BM, int NT>
 struct Staged {
-  u32x4 a[BM / 32];
+  u32x4 a[BM * 8 / NT];  // NT threads move NT / 8 rows of 8 chunks per pass
   u32x4 b[4];
 };
 
-template <typename T, bool B_NK, int BM, int BN>
-__device__ __forceinline__ void load_tiles(const T* __restrict__ A, const T* __restrict__ B, const MMArgs& p, int kt, int tid, Staged<BM>& r) {
+template <typename T, bool B_NK, int BM, int BN, int NT>
+__device__ __forceinline__ void load_tiles(const T* __restrict__ A, const T* __restrict__ B, const MMArgs& p, int kt, int tid, Staged<BM, NT>& r) {
+  constexpr int RP = NT / 8;  // rows per pass
   constexpr int BK = Elt<T>::BK, VE = Elt<T>::VE;
   constexpr bool IS_BF16 = sizeof(T) == 2;
   const size_t k0 = (size_t)kt * BK;
-  const T* Ap = A + (size_t)(tid >> 3) * p.a_rs + k0 + (tid & 7) * VE;  // row tid/8 (+32 per step), chunk tid%8
-  const size_t a_step = (size_t)32 * p.a_rs;
+  const T* Ap = A + (size_t)(tid >> 3) * p.a_rs + k0 + (tid & 7) * VE;  // row tid/8 (+RP per pass), chunk tid%8
+  const size_t a_step = (size_t)RP * p.a_rs;
 #pragma unroll
-  for (int i = 0; i < BM / 32; ++i) r.a[i] = *reinterpret_cast<const u32x4*>(Ap + i * a_step);
+  for (int i = 0; i < BM / RP; ++i) r.a[i] = *reinterpret_cast<const u32x4*>(Ap + i * a_step);
   if (B_NK) {
     const T* Bp = B + (size_t)(tid >> 3) * p.b_cs + k0 + (tid & 7) * VE;
-    const size_t b_step = (size_t)32 * p.b_cs;
+    const size_t b_step = (size_t)RP * p.b_cs;
 #pragma unroll
-    for (int i = 0; i < BN / 32; ++i) r.b[i] = *reinterpret_cast<const u32x4*>(Bp + i * b_step);
+    for (int i = 0; i < BN / RP; ++i) r.b[i] = *reinterpret_cast<const u32x4*>(Bp + i * b_step);
   } else if (tid < 2 * BN) {
     // 4 (k) x 8 (n) bf16 block or 4 (k) x 4 (n) f32 block per thread; 2 * BN threads cover the tile
     const int kg = IS_BF16 ? (tid & 15) : (tid & 7), ng = IS_BF16 ? (tid >> 4) : (tid >> 3);
@@ -74,72 +81,124 @@ __device__ __forceinline__ void load_tiles(const T* __restrict__ A, const T* __r
   }
 }
 
-template <typename T, bool B_NK, int BM, int BN>
-__device__ __forceinline__ void store_tiles(u32x4* __restrict__ S, int tid, const Staged<BM>& r) {
+// Staging stores of one prefetched tile, split into four parts (PART = 0..3) so that they can be
+// spread between the MFMAs of a K tile.  PART < 0 issues all of them.
+template <typename T, bool B_NK, int BM, int BN, int NT, int PART>
+__device__ __forceinline__ void store_tiles(u32x4* __restrict__ S, int tid, const Staged<BM, NT>& r) {
   constexpr bool IS_BF16 = sizeof(T) == 2;
-  const int row = tid >> 3, chunk = tid & 7;  // (row + 32 i) & 7 == row & 7: one swizzle for all steps
-  u32x4* Sa = S + row * CHUNKS + (chunk ^ (row & 7));
+  constexpr int RP = NT / 8, NA = BM / RP;
+  const int row = tid >> 3, chunk = tid & 7;  // rows RP (32 or 64) apart share one swizzle
+  u32x4* Sa = S + row * CHUNKS + (chunk ^ lds_swz(row));
 #pragma unroll
-  for (int i = 0; i < BM / 32; ++i) Sa[i * 32 * CHUNKS] = r.a[i];
+  for (int i = 0; i < NA; ++i)
+    if (PART < 0 || (i & 3) == PART) Sa[i * RP * CHUNKS] = r.a[i];
   if (B_NK) {
     u32x4* Sb = Sa + BM * CHUNKS;
 #pragma unroll
-    for (int i = 0; i < BN / 32; ++i) Sb[i * 32 * CHUNKS] = r.b[i];
+    for (int i = 0; i < BN / RP; ++i)
+      if (PART < 0 || ((NA + i) & 3) == PART) Sb[i * RP * CHUNKS] = r.b[i];
   } else if (tid < 2 * BN) {
     if (IS_BF16) {
       const int kg = tid & 15, ng = tid >> 4;
       u32x2* S2 = reinterpret_cast<u32x2*>(S);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        // column j of the 4 x 8 block: rows (k, k+1) and (k+2, k+3) packed as two dwords
-        const unsigned sel = (j & 1) ? 0x07060302u : 0x05040100u;
-        u32x2 v;
-        v.x = __builtin_amdgcn_perm(r.b[1][j >> 1], r.b[0][j >> 1], sel);
-        v.y = __builtin_amdgcn_perm(r.b[3][j >> 1], r.b[2][j >> 1], sel);
-        S2[lds_idx(BM + ng * 8 + j, kg >> 1) * 2 + (kg & 1)] = v;
+        if (PART < 0 || (j & 3) == PART) {
+          // column j of the 4 x 8 block: rows (k, k+1) and (k+2, k+3) packed as two dwords
+          const unsigned sel = (j & 1) ? 0x07060302u : 0x05040100u;
+          u32x2 v;
+          v.x = __builtin_amdgcn_perm(r.b[1][j >> 1], r.b[0][j >> 1], sel);
+          v.y = __builtin_amdgcn_perm(r.b[3][j >> 1], r.b[2][j >> 1], sel);
+          S2[lds_idx(BM + ng * 8 + j, kg >> 1) * 2 + (kg & 1)] = v;
+        }
       }
     } else {
       const int kg = tid & 7, ng = tid >> 3;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) S[lds_idx(BM + ng * 4 + j, kg)] = u32x4{r.b[0][j], r.b[1][j], r.b[2][j], r.b[3][j]};
+      for (int j = 0; j < 4; ++j)
+        if (PART < 0 || j == PART) S[lds_idx(BM + ng * 4 + j, kg)] = u32x4{r.b[0][j], r.b[1][j], r.b[2][j], r.b[3][j]};
     }
   }
 }
 
-template <typename T, int BM, int MI, int NJ>
-__device__ __forceinline__ void compute_tile(const u32x4* __restrict__ S, int lane, int wm, int wn, floatx16 (&acc)[MI][NJ]) {
-  constexpr bool IS_BF16 = sizeof(T) == 2;
+// MFMA operands of one 16-wide (bf16) / 8-wide (f32) k step of the wave's tile.
+template <int MI, int NJ>
+struct Frags {
+  u32x4 a[MI], b[NJ];
+};
+
+template <int BM, int MI, int NJ>
+__device__ __forceinline__ void load_frags(const u32x4* __restrict__ S, int lane, int wm, int wn, int s, Frags<MI, NJ>& f) {
+  const int chunk = 2 * s + (lane >> 5);
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    const int chunk = 2 * s + (lane >> 5);
-    u32x4 a[MI], b[NJ];
+  for (int i = 0; i < MI; ++i) f.a[i] = S[lds_idx(wm + i * 32 + (lane & 31), chunk)];
 #pragma unroll
-    for (int i = 0; i < MI; ++i) a[i] = S[lds_idx(wm + i * 32 + (lane & 31), chunk)];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) b[j] = S[lds_idx(BM + wn + j * 32 + (lane & 31), chunk)];
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        if (IS_BF16) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[i]), __builtin_bit_cast(bf16x8, b[j]), acc[i][j], 0, 0, 0);
-        } else {
-          // whole-vector casts: __builtin_bit_cast applied to one element of an ext vector reads element 0
-          const f32x4 af = __builtin_bit_cast(f32x4, a[i]), bf = __builtin_bit_cast(f32x4, b[j]);
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af.x, bf.x, acc[i][j], 0, 0, 0);
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af.y, bf.y, acc[i][j], 0, 0, 0);
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af.z, bf.z, acc[i][j], 0, 0, 0);
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af.w, bf.w, acc[i][j], 0, 0, 0);
-        }
-      }
-  }
+  for (int j = 0; j < NJ; ++j) f.b[j] = S[lds_idx(BM + wn + j * 32 + (lane & 31), chunk)];
 }
 
-template <typename T, bool B_NK, int BM, int BN>
-__global__ void __launch_bounds__(256) gemm_tiled(MMArgs p, int tiles_m, int tiles_n, int remap) {
+template <typename T, int MI, int NJ>
+__device__ __forceinline__ void mma_frags(const Frags<MI, NJ>& f, floatx16 (&acc)[MI][NJ]) {
+  constexpr bool IS_BF16 = sizeof(T) == 2;
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      if (IS_BF16) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, f.a[i]), __builtin_bit_cast(bf16x8, f.b[j]), acc[i][j], 0, 0, 0);
+      } else {
+        // whole-vector casts: __builtin_bit_cast applied to one element of an ext vector reads element 0
+        const f32x4 af = __builtin_bit_cast(f32x4, f.a[i]), bf = __builtin_bit_cast(f32x4, f.b[j]);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af.x, bf.x, acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af.y, bf.y, acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af.z, bf.z, acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af.w, bf.w, acc[i][j], 0, 0, 0);
+      }
+    }
+}
+
+// One K tile: multiply the tile in LDS stage `cur`; meanwhile move the tile held in `wr` (loaded
+// from global memory one phase ago) into stage `nxt`, a quarter between each group of MFMAs, and
+// start the global loads of tile `load_kt` into `ld`.  Fragments are double-buffered in registers:
+// the LDS reads of k step s+1 are in flight while the MFMAs of step s run.
+// The loads are unconditional (LOAD is a compile-time switch): a load under a run-time branch makes
+// the compiler wait for every outstanding load before the staging stores, which would undo the
+// two-tile lead.
+template <typename T, bool B_NK, int BM, int BN, int NT, int MI, int NJ, bool LOAD>
+__device__ __forceinline__ void k_phase(const T* __restrict__ A, const T* __restrict__ B, const MMArgs& p, const u32x4* __restrict__ cur, u32x4* __restrict__ nxt,
+                                        bool do_write, const Staged<BM, NT>& wr, int load_kt, Staged<BM, NT>& ld, int tid, int lane, int wm, int wn,
+                                        floatx16 (&acc)[MI][NJ]) {
+  if (LOAD) load_tiles<T, B_NK, BM, BN, NT>(A, B, p, load_kt, tid, ld);
+  // Issue order within a k step: LDS reads of the next step, the MFMAs of this step (their issue
+  // time covers the LDS latency), then a quarter of the staging stores.  The scheduling barriers
+  // keep the compiler from sinking the reads next to their uses, which would serialise every
+  // LDS round trip with the matrix pipe.
+  Frags<MI, NJ> f0, f1;
+  load_frags<BM, MI, NJ>(cur, lane, wm, wn, 0, f0);
+  load_frags<BM, MI, NJ>(cur, lane, wm, wn, 1, f1);
+  __builtin_amdgcn_sched_barrier(0);
+  mma_frags<T, MI, NJ>(f0, acc);
+  if (do_write) store_tiles<T, B_NK, BM, BN, NT, 0>(nxt, tid, wr);
+  __builtin_amdgcn_sched_barrier(0);
+  load_frags<BM, MI, NJ>(cur, lane, wm, wn, 2, f0);
+  mma_frags<T, MI, NJ>(f1, acc);
+  if (do_write) store_tiles<T, B_NK, BM, BN, NT, 1>(nxt, tid, wr);
+  __builtin_amdgcn_sched_barrier(0);
+  load_frags<BM, MI, NJ>(cur, lane, wm, wn, 3, f1);
+  mma_frags<T, MI, NJ>(f0, acc);
+  if (do_write) store_tiles<T, B_NK, BM, BN, NT, 2>(nxt, tid, wr);
+  __builtin_amdgcn_sched_barrier(0);
+  mma_frags<T, MI, NJ>(f1, acc);
+  if (do_write) store_tiles<T, B_NK, BM, BN, NT, 3>(nxt, tid, wr);
+}
+
+// NT threads = NT / 64 waves laid out (NT / 128) x 2 over the tile: 4 waves give each wave a
+// (BM/2) x (BN/2) block; 8 waves halve the rows per wave and put two waves on every SIMD, so that
+// one can feed the matrix pipe while the other is blocked on the LDS or load queues.
+template <typename T, bool B_NK, int BM, int BN, int NT>
+__global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p, int tiles_m, int tiles_n, int remap) {
   extern __shared__ u32x4 lds[];
   constexpr int BK = Elt<T>::BK;
-  constexpr int WM = BM / 2, WN = BN / 2, MI = WM / 32, NJ = WN / 32;
+  constexpr int WM = BM / (NT / 128), WN = BN / 2, MI = WM / 32, NJ = WN / 32;
   constexpr int STAGE = (BM + BN) * CHUNKS;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int bid = blockIdx.x;
@@ -154,7 +213,6 @@ __global__ void __launch_bounds__(256) gemm_tiled(MMArgs p, int tiles_m, int til
   const int KT = p.K / BK;
   const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
 
-  Staged<BM> st;
   floatx16 acc[MI][NJ];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
@@ -163,17 +221,25 @@ __global__ void __launch_bounds__(256) gemm_tiled(MMArgs p, int tiles_m, int til
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  load_tiles<T, B_NK, BM, BN>(A, B, p, 0, tid, st);
-  store_tiles<T, B_NK, BM, BN>(lds, tid, st);
+  // Global loads run two tiles ahead of the MFMAs: tile kt+2 is on its way into one register set
+  // while tile kt+1 moves from the other set into the idle LDS stage and tile kt is multiplied.
+  Staged<BM, NT> r0, r1;
+  u32x4* lds0 = lds;
+  u32x4* lds1 = lds + STAGE;
+  load_tiles<T, B_NK, BM, BN, NT>(A, B, p, 0, tid, r0);
+  if (KT > 1) load_tiles<T, B_NK, BM, BN, NT>(A, B, p, 1, tid, r1);
+  store_tiles<T, B_NK, BM, BN, NT, -1>(lds0, tid, r0);
   __syncthreads();
-  for (int kt = 0; kt < KT; ++kt) {
-    const bool more = kt + 1 < KT;
-    if (more) load_tiles<T, B_NK, BM, BN>(A, B, p, kt + 1, tid, st);
-    compute_tile<T, BM, MI, NJ>(lds + (kt & 1) * STAGE, lane, wm, wn, acc);
-    // stage (kt+1)&1 was last read during iteration kt-1; every wave has passed the barrier since
-    if (more) store_tiles<T, B_NK, BM, BN>(lds + ((kt + 1) & 1) * STAGE, tid, st);
+  int kt = 0;
+  for (; kt + 1 < KT; kt += 2) {
+    // Past the end the last tile is loaded again (and never stored): same instruction stream for
+    // every iteration.  Stage 1 was last read in the previous odd phase, a barrier ago.
+    k_phase<T, B_NK, BM, BN, NT, MI, NJ, true>(A, B, p, lds0, lds1, true, r1, min(kt + 2, KT - 1), r0, tid, lane, wm, wn, acc);
+    __syncthreads();
+    k_phase<T, B_NK, BM, BN, NT, MI, NJ, true>(A, B, p, lds1, lds0, kt + 2 < KT, r0, min(kt + 3, KT - 1), r1, tid, lane, wm, wn, acc);
     __syncthreads();
   }
+  if (kt < KT) k_phase<T, B_NK, BM, BN, NT, MI, NJ, false>(A, B, p, lds0, lds1, false, r1, 0, r0, tid, lane, wm, wn, acc);  // odd tile count: the last tile
 
   // accumulator register r of lane l: row (r/4)*8 + (l/32)*4 + r%4, column l%32
 #pragma unroll
@@ -186,11 +252,11 @@ __global__ void __launch_bounds__(256) gemm_tiled(MMArgs p, int tiles_m, int til
     }
 }
 
-template <typename T, bool B_NK, int BM, int BN>
+template <typename T, bool B_NK, int BM, int BN, int NT>
 hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch) {
   constexpr int LDS_BYTES = 2 * (BM + BN) * CHUNKS * 16;
   static bool configured = false;
-  auto kernel = gemm_tiled<T, B_NK, BM, BN>;
+  auto kernel = gemm_tiled<T, B_NK, BM, BN, NT>;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if (e != hipSuccess) return e;
@@ -199,16 +265,16 @@ hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch) {
   const int tiles_m = p.M / BM, tiles_n = p.N / BN;
   const size_t total = batch * (size_t)tiles_m * tiles_n;
   const int remap = total % 8 == 0 ? 1 : 0;
-  kernel<<<dim3((unsigned)total), dim3(256), LDS_BYTES, stream>>>(p, tiles_m, tiles_n, remap);
+  kernel<<<dim3((unsigned)total), dim3(NT), LDS_BYTES, stream>>>(p, tiles_m, tiles_n, remap);
   return hipGetLastError();
 }
 
 template <typename T, bool B_NK>
 hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int shape) {
   switch (shape) {
-    case 0: return launch<T, B_NK, 256, 128>(stream, p, batch);
-    case 1: return launch<T, B_NK, 128, 128>(stream, p, batch);
-    default: return launch<T, B_NK, 128, 64>(stream, p, batch);
+    case 0: return getenv("UGHIP_GEMM_4WAVES") ? launch<T, B_NK, 256, 128, 256>(stream, p, batch) : launch<T, B_NK, 256, 128, 512>(stream, p, batch);
+    case 1: return launch<T, B_NK, 128, 128, 256>(stream, p, batch);
+    default: return launch<T, B_NK, 128, 64, 256>(stream, p, batch);
   }
 }
 
@@ -219,6 +285,11 @@ constexpr int kShapes[3][2] = {{256, 128}, {128, 128}, {128, 64}};
 // The largest tile that divides the problem and still gives every CU a workgroup; failing that,
 // the dividing tile with the most workgroups.  -1: no tile divides M x N.
 int pick_shape(const MMArgs& p, size_t batch) {
+  // UGHIP_GEMM_SHAPE=0|1|2 forces a tile shape (tuning aid); ignored when it does not divide M x N.
+  if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
+    const int s = atoi(e);
+    if (s >= 0 && s < 3 && p.M % kShapes[s][0] == 0 && p.N % kShapes[s][1] == 0) return s;
+  }
   int best = -1;
   size_t best_tiles = 0;
   for (int s = 0; s < 3; ++s) {
