@@ -192,6 +192,8 @@ def llama_pieces(dev, steps, warmup):
     hbm("c4_softmax_lazy_1x32x512x512", ll.softmax(s), 2 * 4 * heads * t * t)
     hbm("c4_softmax_custom_1x32x512x512", ops.custom_softmax(s), 2 * 4 * heads * t * t)
     hbm("c4_mask_then_softmax_custom", ops.custom_softmax(ops.causal_mask(s)), 4 * 4 * heads * t * t)
+    # the same two ops as one kernel: reads the kept triangle, writes every element
+    hbm("c4_causal_softmax_fused", ops.causal_softmax(s), 2 * 4 * heads * t * t)
     gate = LB.copy(rng.normal(8 + 100, t * 5632), (1, t, 5632), dev)
     up = LB.copy(rng.normal(8 + 101, t * 5632), (1, t, 5632), dev)
     hbm("c4_silu_mul_512x5632", ll.silu(gate).binary("mul", up), 3 * 4 * t * 5632)
@@ -212,17 +214,18 @@ def llama_pieces(dev, steps, warmup):
     return out
 
 
-def llama_decode(dev, n_prompt=128, n_steps=128):
+def llama_decode(dev, n_prompt=128, n_steps=128, fused_attention=False):
     """Config 5: TinyLlama-1.1B shape, random-init f32 weights, prefill 128 then 128 greedy steps.
     Fresh buffers are not zero-filled here (every kernel of the model writes its whole output; the
-    ids are the same either way, which the GPU tests check)."""
+    ids are the same either way, which the GPU tests check).  fused_attention routes attention
+    through ughip_causal_softmax_rows / ughip_attention_decode instead of the op-by-op graph."""
     import ug_amd
     from ug_amd import rng
     cfg = ug_amd.LlamaConfig()
     ops = ug_amd.LlamaOps.hip()
     dev.set_zero_fill(False)
     t0 = time.perf_counter()
-    model = ug_amd.LlamaModel(dev, ops, cfg, custom_softmax=True, seed=9, std=0.02)
+    model = ug_amd.LlamaModel(dev, ops, cfg, custom_softmax=True, seed=9, std=0.02, fused_attention=fused_attention)
     load_s = time.perf_counter() - t0
     prompt = rng.token_ids(10, n_prompt, cfg.vocab_size)
     model.generate(prompt, 4)          # compiles every kernel shape family once
@@ -231,7 +234,7 @@ def llama_decode(dev, n_prompt=128, n_steps=128):
     weights_bytes = 4 * 1034512384
     tok_s = n_steps / (st["decode_ms"] * 1e-3)
     return {"tok/s": round(tok_s, 2), "decode_ms_per_token": round(st["decode_ms"] / n_steps, 3), "prefill_ms": round(st["prefill_ms"], 1),
-            "frac_hbm_weights_only": round(tok_s * weights_bytes / 1e9 / HBM_PEAK_GBS, 4), "load_s": round(load_s, 1), "dtype": "f32", "zero_fill": False,
+            "frac_hbm_weights_only": round(tok_s * weights_bytes / 1e9 / HBM_PEAK_GBS, 4), "load_s": round(load_s, 1), "dtype": "f32", "zero_fill": False, "fused_attention": fused_attention,
             "first_ids": toks[:8].tolist(), "min_top1_margin": float(st["margins"].min())}
 
 
@@ -303,10 +306,11 @@ def main():
         except Exception as e:  # noqa: BLE001
             line["extras"] = {"error": f"{type(e).__name__}: {e}"}
     if not (args.no_llama or args.headline_only):
-        try:
-            line.setdefault("extras", {})["llama_decode_f32"] = llama_decode(dev)
-        except Exception as e:  # noqa: BLE001
-            line.setdefault("extras", {})["llama_decode_f32"] = {"error": f"{type(e).__name__}: {e}"}
+        for key, fused in (("llama_decode_f32", False), ("llama_decode_f32_fused_attention", True)):
+            try:
+                line.setdefault("extras", {})[key] = llama_decode(dev, fused_attention=fused)
+            except Exception as e:  # noqa: BLE001
+                line.setdefault("extras", {})[key] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(line), flush=True)
 
 

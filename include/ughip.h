@@ -221,6 +221,21 @@ int ughip_softmax_rows(ughip_device* dev, const ughip_slice* src, ughip_slice* d
 int ughip_causal_mask(ughip_device* dev, const ughip_slice* src, ughip_slice* dst, size_t bh,
                       size_t s1, size_t s2);
 
+/* ---- attention fusions (no counterpart in the reference's device trait) ----------------------
+ * The step either side of the softmax kernel: what ug-llama builds from several ops
+ * (ug-llama/src/model.rs:231-244) as one launch each.  A caller opts in; the unfused ops above
+ * stay the reference behaviour. */
+/* causal_mask followed by custom_softmax over [bh, s1, s2], f32: row i1 keeps columns
+ * i2 <= i1 (cpu_ops.rs:33-56), masked columns come out as 0. */
+int ughip_causal_softmax_rows(ughip_device* dev, const ughip_slice* src, ughip_slice* dst,
+                              size_t bh, size_t s1, size_t s2);
+/* Attention of one query position, f32: q [b, n_heads, d], k and v [b, n_kv_heads, s, d]
+ * (query head h reads kv head h / (n_heads / n_kv_heads), i.e. model.rs:80-92's repeat),
+ * dst [b, n_heads, d] = softmax(q k^T * scale) v.  d a power of two in 16..256, s <= 15000. */
+int ughip_attention_decode(ughip_device* dev, const ughip_slice* q, const ughip_slice* k,
+                           const ughip_slice* v, ughip_slice* dst, size_t b, size_t n_heads,
+                           size_t n_kv_heads, size_t s, size_t d, float scale);
+
 /* ---- timing on the device stream ----------------------------------------------------- */
 int ughip_event_create(ughip_device* dev, ughip_event** out);
 int ughip_event_record(ughip_event* ev);

@@ -498,3 +498,83 @@ def test_llama_config5_width_greedy_ids_match_cpu(hip, cpu, hip_ops, cpu_ops, ro
     print("hip", toks_h.tolist(), "cpu", toks_c.tolist(), "margins", st_c["margins"].tolist(), flush=True)
     assert toks_h.tolist() == toks_c.tolist()
     np.testing.assert_allclose(st_h["margins"], st_c["margins"], rtol=1e-2, atol=1e-7)
+
+
+# ---- attention fusions: one kernel on the HIP device against the op-by-op graph on the oracle ----------------------------
+@pytest.mark.parametrize("shape", [(1, 32, 16, 16), (2, 3, 5, 5), (1, 2, 128, 128), (1, 1, 7, 7), (1, 2, 512, 512), (1, 1, 300, 300), (1, 1, 33, 33),
+                                   (1, 2, 40, 1500), (1, 1, 9, 2100), (1, 1, 1024, 1024), (1, 1, 3, 2048)])
+def test_causal_softmax_fused(hip, cpu, hip_ops, cpu_ops, shape):
+    print("causal softmax", shape, flush=True)
+    x = rng.normal(61, int(np.prod(shape)), 2.0)
+    got = hip_ops.causal_softmax(LB.copy(x, shape, hip)).data_vec().reshape(shape)
+    want = cpu_ops.causal_softmax(LB.copy(x, shape, cpu)).data_vec().reshape(shape)   # custom_softmax(causal_mask(x)) op by op
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-30)
+    s1, s2 = shape[2], shape[3]
+    keep = np.arange(s2)[None, :] <= np.arange(s1)[:, None]
+    xm = np.where(keep, x.reshape(shape).astype(np.float64), -np.inf)
+    e = np.exp(xm - xm.max(-1, keepdims=True))
+    np.testing.assert_allclose(got, e / e.sum(-1, keepdims=True), rtol=1e-5, atol=1e-30)
+    assert np.all(got[..., ~keep] == 0.0)
+    # and the same through the unfused ops on the HIP device
+    unfused = hip_ops.custom_softmax(hip_ops.causal_mask(LB.copy(x, shape, hip))).data_vec().reshape(shape)
+    np.testing.assert_allclose(got, unfused, rtol=2e-6, atol=1e-30)
+
+
+@pytest.mark.parametrize("b,nh,nkv,s,d", [(1, 32, 4, 1, 64), (1, 32, 4, 5, 64), (1, 32, 4, 129, 64), (2, 8, 2, 700, 64), (1, 8, 8, 33, 128), (3, 4, 1, 17, 16),
+                                          (1, 2, 1, 2100, 256), (1, 32, 4, 2047, 64)])
+def test_attention_decode_fused(hip, cpu, hip_ops, cpu_ops, b, nh, nkv, s, d):
+    print("attention decode", (b, nh, nkv, s, d), flush=True)
+    q = rng.normal(62, b * nh * d)
+    k = rng.normal(63, b * nkv * s * d)
+    v = rng.normal(64, b * nkv * s * d)
+    scale = float(np.float32(d) ** np.float32(-0.5))
+
+    def run(dev, ops):
+        return ops.attention_decode(LB.copy(q, (b, nh, 1, d), dev), LB.copy(k, (b, nkv, s, d), dev), LB.copy(v, (b, nkv, s, d), dev), scale).data_vec()
+
+    got = run(hip, hip_ops).reshape(b, nh, d)
+    want = run(cpu, cpu_ops).reshape(b, nh, d)    # repeat, matmul_t, scale, custom_softmax, matmul (model.rs:231-244)
+    q6, k6, v6 = q.reshape(b, nh, d).astype(np.float64), k.reshape(b, nkv, s, d).astype(np.float64), v.reshape(b, nkv, s, d).astype(np.float64)
+    rep = nh // nkv
+    sc = np.einsum("bhd,bhsd->bhs", q6, np.repeat(k6, rep, 1)) * scale
+    p = np.exp(sc - sc.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    truth = np.einsum("bhs,bhsd->bhd", p, np.repeat(v6, rep, 1))
+    tol = 1e-5 * np.abs(truth).max() + 1e-5 * np.abs(truth)
+    assert np.all(np.abs(got - truth) <= tol)
+    assert np.all(np.abs(got - want) <= 2 * tol)
+
+
+def test_attention_fusion_errors(hip, hip_ops):
+    q = LB.copy(np.zeros(2 * 24, np.float32), (1, 2, 1, 24), hip)
+    def kv(shape):
+        return LB.copy(np.zeros(int(np.prod(shape)), np.float32), shape, hip)
+
+    with pytest.raises(ug_amd.UgError, match="power of two"):
+        hip_ops.attention_decode(q, kv((1, 2, 3, 24)), kv((1, 2, 3, 24)), 1.0).data_vec()
+    q2 = LB.copy(np.zeros(3 * 16, np.float32), (1, 3, 1, 16), hip)
+    with pytest.raises(ug_amd.UgError, match="not a multiple"):
+        hip_ops.attention_decode(q2, kv((1, 2, 3, 16)), kv((1, 2, 3, 16)), 1.0).data_vec()
+    # one buffer passed as both k and v is refused like any double borrow (schedule.rs:254-262)
+    same = kv((1, 2, 3, 16))
+    q3 = LB.copy(np.zeros(2 * 16, np.float32), (1, 2, 1, 16), hip)
+    with pytest.raises(ug_amd.UgError, match="already borrowed"):
+        hip_ops.attention_decode(q3, same, same, 1.0).data_vec()
+
+
+@pytest.mark.parametrize("width", ["small", "config5"])
+def test_llama_fused_attention_ids_match_unfused_cpu(hip, cpu, hip_ops, cpu_ops, width):
+    """The model with both fusions switched on (HIP) against the reference's op-by-op graph (oracle)."""
+    if width == "small":
+        cfg = ug_amd.LlamaConfig(hidden_size=128, intermediate_size=320, max_position_embeddings=64, num_attention_heads=4, num_key_value_heads=2,
+                                 num_hidden_layers=2, vocab_size=512)
+        n_prompt, n_steps, std = 12, 10, 0.3
+    else:
+        cfg = ug_amd.LlamaConfig(num_hidden_layers=2, max_position_embeddings=256)
+        n_prompt, n_steps, std = 16, 6, 0.02
+    prompt = rng.token_ids(10, n_prompt, cfg.vocab_size)
+    toks_h, st_h = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=std, fused_attention=True).generate(prompt, n_steps)
+    toks_c, st_c = ug_amd.LlamaModel(cpu, cpu_ops, cfg, True, seed=9, std=std).generate(prompt, n_steps)
+    print("hip fused", toks_h.tolist(), "cpu", toks_c.tolist(), flush=True)
+    assert toks_h.tolist() == toks_c.tolist()
+    np.testing.assert_allclose(st_h["margins"], st_c["margins"], rtol=1e-2, atol=1e-7)

@@ -630,6 +630,16 @@ class LlamaOps(_Handle):
     def causal_mask(self, src):
         return self._op("ugh_llama_causal_mask", src)
 
+    def causal_softmax(self, src):
+        """softmax(causal_mask(src)); one kernel on the HIP device, op by op elsewhere."""
+        return self._op("ugh_llama_causal_softmax", src)
+
+    def attention_decode(self, q, k, v, scale):
+        """One query position: q [b, nh, 1, d], k and v [b, nkv, s, d] -> [b, nh, 1, d]."""
+        lb = self._op("ugh_llama_attention_decode", q, _p(k.h), _p(v.h), C.c_float(scale))
+        lb._keep += [k, v]
+        return lb
+
 
 class _Llama:
     """Graph builders of ug-llama/src/model.rs:32-109."""
@@ -670,11 +680,13 @@ class LlamaModel(_Handle):
     """ug_llama::Model with random-init weights N(0, std) from the seeded generator."""
     _free = "ugh_llama_model_free"
 
-    def __init__(self, device, ops, cfg, custom_softmax=False, seed=9, std=0.02, round_bf16=False):
+    def __init__(self, device, ops, cfg, custom_softmax=False, seed=9, std=0.02, round_bf16=False, fused_attention=False):
         out = C.c_void_p()
         _chk(host_lib().ugh_llama_model_new(_p(device.h), _p(ops.h), C.byref(cfg), int(custom_softmax), C.c_uint64(seed), C.c_float(std),
                                             int(round_bf16), C.byref(out)))
         super().__init__(out.value)
+        if fused_attention:
+            _chk(host_lib().ugh_llama_model_set_fused_attention(_p(self.h), 1))
         self._keep = [device, ops]
         self.cfg = cfg
 

@@ -390,6 +390,12 @@ int ugh_llama_custom_softmax(void* ops, void* src, void** out) {
 int ugh_llama_causal_mask(void* ops, void* src, void** out) {
   return guard([&] { *out = box(ops_of(ops).causal_mask(lb_of(src))); });
 }
+int ugh_llama_causal_softmax(void* ops, void* src, void** out) {
+  return guard([&] { *out = box(ops_of(ops).causal_softmax(lb_of(src))); });
+}
+int ugh_llama_attention_decode(void* ops, void* q, void* k, void* v, float scale, void** out) {
+  return guard([&] { *out = box(ops_of(ops).attention_decode(lb_of(q), lb_of(k), lb_of(v), scale)); });
+}
 int ugh_llama_rms_norm(void* src, void* alpha, float eps, void** out) {
   return guard([&] { *out = box(ug_llama::rms_norm(lb_of(src), lb_of(alpha), eps)); });
 }
@@ -433,6 +439,9 @@ int ugh_llama_model_new(void* d, void* ops, const ugh_llama_config* c, int custo
   });
 }
 void ugh_llama_model_free(void* m) { delete static_cast<ug_llama::Model*>(m); }
+int ugh_llama_model_set_fused_attention(void* m, int on) {
+  return guard([&] { static_cast<ug_llama::Model*>(m)->set_fused_attention(on != 0); });
+}
 int ugh_llama_generate(void* m, const int32_t* prompt, size_t n_prompt, size_t n_steps, int32_t* out_tokens, double* prefill_ms,
                        double* decode_ms, float* margins) {
   return guard([&] {

@@ -77,6 +77,30 @@ struct HipOps : Ops {
     return LB::custom(f, {src}, src.shape(), src.dtype(), src.device());
   }
 
+  LB causal_softmax(const LB& att) const override {
+    if (att.rank() != 4) bail("causal_softmax: expected a rank-4 tensor, got " + att.shape().str());
+    size_t bh = att.dims()[0] * att.dims()[1], s1 = att.dims()[2], s2 = att.dims()[3];
+    ughip_device* dev = hip_dev(att);
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != 2) bail("causal_softmax: expected 2 slices");
+      hip_check(ughip_causal_softmax_rows(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), bh, s1, s2), "causal_softmax");
+    };
+    return LB::custom(f, {att}, att.shape(), att.dtype(), att.device());
+  }
+
+  LB attention_decode(const LB& q, const LB& k, const LB& v, float scale) const override {
+    if (q.rank() != 4 || k.rank() != 4 || v.rank() != 4 || q.dims()[2] != 1) bail("attention_decode: expected q [b, nh, 1, d] and k, v [b, nkv, s, d]");
+    size_t b = q.dims()[0], nh = q.dims()[1], d = q.dims()[3], nkv = k.dims()[1], s = k.dims()[2];
+    if (k.dims() != v.dims() || k.dims()[0] != b || k.dims()[3] != d) bail("attention_decode: mismatched shapes " + q.shape().str() + " " + k.shape().str());
+    ughip_device* dev = hip_dev(q);
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != 4) bail("attention_decode: expected 4 slices");
+      hip_check(ughip_attention_decode(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), hip_raw_slice(*vs[3]), b, nh, nkv, s, d, scale),
+                "attention_decode");
+    };
+    return LB::custom(f, {q, k, v}, q.shape(), q.dtype(), q.device());
+  }
+
   LB causal_mask(const LB& src) const override {
     if (src.rank() != 4) bail("causal_mask: expected a rank-4 tensor, got " + src.shape().str());
     size_t bh = src.dims()[0] * src.dims()[1], s1 = src.dims()[2], s2 = src.dims()[3];
@@ -131,6 +155,16 @@ struct SyntheticWeights : WeightSource {
   }
 };
 }  // namespace
+
+// model.rs:231-244 for one query position, op by op.
+LB Ops::attention_decode(const LB& q, const LB& k, const LB& v, float scale) const {
+  size_t n_rep = q.dims()[1] / k.dims()[1];
+  LB kr = repeat(k, 1, n_rep);
+  LB vr = repeat(v, 1, n_rep);
+  LB att = q.matmul_t(kr);
+  att = att.binary(BinaryOp::Mul, LB::cst(Const::f32(scale), Shape(), q.device()).broadcast(att.shape()));
+  return custom_softmax(att).matmul(vr);
+}
 
 std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16) {
   return std::make_shared<SyntheticWeights>(seed, std, round_bf16);
@@ -282,15 +316,24 @@ LB Model::attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache) c
   v = ops_->cat(cache.prev_v, v, 2);
   cache.prev_k = k;
   cache.prev_v = v;
-  LB kr = repeat(k, 1, nh / nkv);
-  LB vr = repeat(v, 1, nh / nkv);
-
-  LB att = q.matmul_t(kr);
-  LB scale = LB::cst(Const::f32(std::pow((float)hd, -0.5f)), Shape(), q.device()).broadcast(att.shape());
-  att = att.binary(BinaryOp::Mul, scale);
-  if (seq_len != 1) att = ops_->causal_mask(att);
-  att = custom_softmax_ ? ops_->custom_softmax(att) : softmax(att);
-  LB out = att.matmul(vr);
+  const float scale_v = std::pow((float)hd, -0.5f);
+  LB out;
+  if (fused_attention_ && seq_len == 1) {
+    out = ops_->attention_decode(q, k, v, scale_v);
+  } else {
+    LB kr = repeat(k, 1, nh / nkv);
+    LB vr = repeat(v, 1, nh / nkv);
+    LB att = q.matmul_t(kr);
+    LB scale = LB::cst(Const::f32(scale_v), Shape(), q.device()).broadcast(att.shape());
+    att = att.binary(BinaryOp::Mul, scale);
+    if (fused_attention_ && seq_len != 1) {
+      att = ops_->causal_softmax(att);
+    } else {
+      if (seq_len != 1) att = ops_->causal_mask(att);
+      att = custom_softmax_ ? ops_->custom_softmax(att) : softmax(att);
+    }
+    out = att.matmul(vr);
+  }
   out = out.transpose(2, 1).merge_dims(-2);
   return out.matmul_t(l.o_proj);
 }
@@ -379,6 +422,9 @@ std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32
     Schedule schedule = Schedule::create_one(st.logits);
     auto t2 = clock::now();
     st.compiled = std::make_unique<CompiledSchedule>(schedule.compile_with_cache(ccache));
+    // Buffers are taken from the pool here, on the preparing thread, so that the launches of this
+    // step (possibly issued from another thread) do not allocate.
+    st.compiled->allocate_all();
     st.n_items = schedule.items().size();
     st.build_ms = ms_between(t0, t1);
     st.gen_ms = ms_between(t1, t2);

@@ -20,6 +20,13 @@ struct Ops {
   virtual LB cat(const LB& lhs, const LB& rhs, size_t axis) const = 0;
   virtual LB custom_softmax(const LB& src) const = 0;
   virtual LB causal_mask(const LB& src) const = 0;
+
+  // Optional fusions (not part of the reference's trait).  The defaults compose the ops above
+  // exactly as ug-llama/src/model.rs:231-244 does; a device may answer with one kernel.
+  // softmax(causal_mask(att)) over the last dim of [b, h, t, s].
+  virtual LB causal_softmax(const LB& att) const { return custom_softmax(causal_mask(att)); }
+  // One query position: q [b, nh, 1, d], k and v [b, nkv, s, d] -> [b, nh, 1, d].
+  virtual LB attention_decode(const LB& q, const LB& k, const LB& v, float scale) const;
 };
 
 // The HIP implementation (counterpart of ug-llama/src/cuda_ops.rs).
@@ -73,6 +80,10 @@ struct Cache {
 class Model {
  public:
   Model(const Config& cfg, bool custom_softmax, WeightSource& weights, const ug::DevicePtr& dev, std::shared_ptr<Ops> ops);
+  // Route attention through Ops::causal_softmax (prefill) and Ops::attention_decode (one query
+  // position) instead of the op-by-op graph.  Off by default: the graph is then the reference's.
+  void set_fused_attention(bool on) { fused_attention_ = on; }
+  bool fused_attention() const { return fused_attention_; }
   LB fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const;
   const Config& config() const { return cfg_; }
   const ug::DevicePtr& device() const { return dev_; }
@@ -88,6 +99,7 @@ class Model {
   LB mlp(const Layer& l, const LB& xs) const;
   Config cfg_;
   bool custom_softmax_;
+  bool fused_attention_ = false;
   ug::DevicePtr dev_;
   std::shared_ptr<Ops> ops_;
   LB embedding_, ln_f_;

@@ -158,6 +158,9 @@ struct CompiledSchedule {
   std::vector<CompiledFunc> funcs;
   DevicePtr device;
   void run() const;
+  // Allocates every buffer run() would allocate lazily (schedule.rs:247-250, 268-270), so that a
+  // later run() only dispatches.
+  void allocate_all() const;
 };
 
 // schedule.rs:61-208

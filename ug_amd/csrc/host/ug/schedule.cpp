@@ -315,6 +315,18 @@ CompiledSchedule Schedule::compile_with_cache(CompilationCache& cache) const {
   return out;
 }
 
+void CompiledSchedule::allocate_all() const {
+  for (const CompiledFunc& f : funcs) {
+    if (f.kind == CompiledFunc::MatMul) {
+      f.dst.maybe_allocate_uninit();
+      f.lhs.maybe_allocate_uninit();
+      f.rhs.maybe_allocate_uninit();
+    } else {
+      for (const auto& a : f.args) a.second.maybe_allocate_uninit();
+    }
+  }
+}
+
 // schedule.rs:234-305
 void CompiledSchedule::run() const {
   std::vector<Slice*> bs;

@@ -1,0 +1,223 @@
+// Attention fusions for gfx950 that go one step past the reference's op set (f32):
+//
+//   ughip_causal_softmax_rows  = causal_mask followed by custom_softmax (cpu_ops.rs:33-56, 6-31)
+//                                in one pass: masked columns are never read and come out as 0.
+//   ughip_attention_decode     = for one query position, the chain of ug-llama/src/model.rs:231-244
+//                                repeat(k), repeat(v), q x k^T, * scale, softmax, x v
+//                                in one launch, reading each K/V head once (no repeated copies).
+//
+// Both reduce in a fixed order (no atomics): results do not change from run to run.
+#include <hip/hip_runtime.h>
+
+#include "internal.h"
+#include "ughip.h"
+
+using namespace ughip;
+
+namespace {
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// All threads of a 256-thread workgroup get the max / the sum of v.
+template <bool IS_MAX>
+__device__ __forceinline__ float block_reduce_256(float v, float* lds4) {
+  v = IS_MAX ? wave_max(v) : wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = v;
+  __syncthreads();
+  const float a = lds4[0], b = lds4[1], c = lds4[2], d = lds4[3];
+  return IS_MAX ? fmaxf(fmaxf(a, b), fmaxf(c, d)) : (a + b) + (c + d);
+}
+
+// ---- causal softmax -------------------------------------------------------------------------
+// Rows of [bh, s1, s2]; row r keeps columns 0 .. r % s1.  Wave per row, 128-bit accesses:
+// n_cols % 4 == 0 and n_cols <= 256 * V.
+template <int V>
+__global__ void __launch_bounds__(256) causal_softmax_wave_v4(const float* __restrict__ src, float* __restrict__ dst, int n_rows, int s1, int n_cols) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= n_rows) return;
+  const int lane = threadIdx.x & 63, n4 = n_cols >> 2;
+  const int lim = min(n_cols, row % s1 + 1);  // columns kept
+  const float4* s4 = reinterpret_cast<const float4*>(src + (size_t)row * n_cols);
+  float4* d4 = reinterpret_cast<float4*>(dst + (size_t)row * n_cols);
+  float4 x[V];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const int c = (lane + i * 64) * 4;
+    x[i] = c < lim ? s4[lane + i * 64] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    if (c + 1 >= lim) x[i].y = -INFINITY;
+    if (c + 2 >= lim) x[i].z = -INFINITY;
+    if (c + 3 >= lim) x[i].w = -INFINITY;
+    m = fmaxf(fmaxf(m, fmaxf(x[i].x, x[i].y)), fmaxf(x[i].z, x[i].w));
+  }
+  m = wave_max(m);  // column 0 is always kept: m is finite unless the data is not
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    x[i].x = expf(x[i].x - m);
+    x[i].y = expf(x[i].y - m);
+    x[i].z = expf(x[i].z - m);
+    x[i].w = expf(x[i].w - m);
+    sum += (x[i].x + x[i].y) + (x[i].z + x[i].w);
+  }
+  sum = wave_sum(sum);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const int c = lane + i * 64;
+    if (c < n4) d4[c] = make_float4(x[i].x / sum, x[i].y / sum, x[i].z / sum, x[i].w / sum);
+  }
+}
+
+// Any row length: one workgroup per row, the kept part of the row is read twice.
+__global__ void __launch_bounds__(256) causal_softmax_generic(const float* __restrict__ src, float* __restrict__ dst, int s1, int n_cols) {
+  __shared__ float lds4[4];
+  const size_t row = blockIdx.x;
+  const int lim = min(n_cols, (int)(row % s1) + 1);
+  const float* s = src + row * n_cols;
+  float* d = dst + row * n_cols;
+  float m = -INFINITY;
+  for (int c = threadIdx.x; c < lim; c += 256) m = fmaxf(m, s[c]);
+  m = block_reduce_256<true>(m, lds4);
+  float sum = 0.f;
+  for (int c = threadIdx.x; c < lim; c += 256) sum += expf(s[c] - m);
+  sum = block_reduce_256<false>(sum, lds4);
+  for (int c = threadIdx.x; c < n_cols; c += 256) d[c] = c < lim ? expf(s[c] - m) / sum : 0.f;
+}
+
+// ---- single-query attention -----------------------------------------------------------------------
+// One workgroup (256 threads) per query head.  q: [b, nh, d]; k, v: [b, nkv, s, d]; dst: [b, nh, d].
+// LPK = d / 4 lanes share one key row (one 128-bit load each, a row is one contiguous 4*d bytes);
+// 256 / LPK keys are in flight per step.  Scores and probabilities live in LDS (s floats).
+__global__ void __launch_bounds__(256) attention_decode_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
+                                                               float* __restrict__ dst, int nh, int nkv, int s, int d, float scale) {
+  extern __shared__ __attribute__((aligned(16))) float sc[];  // s scores, then 256 float4 of reduction space
+  __shared__ float lds4[4];
+  const int tid = threadIdx.x;
+  const int lpk = d >> 2, kpb = 256 / lpk;  // lanes per key, keys per step
+  const int c4 = tid % lpk, slot = tid / lpk;
+  const int bh = blockIdx.x, b = bh / nh, h = bh % nh, kvh = h / (nh / nkv);
+  const float4* q4 = reinterpret_cast<const float4*>(q + (size_t)bh * d);
+  const float4* k4 = reinterpret_cast<const float4*>(k + ((size_t)b * nkv + kvh) * (size_t)s * d);
+  const float4* v4 = reinterpret_cast<const float4*>(v + ((size_t)b * nkv + kvh) * (size_t)s * d);
+
+  // scores = (q . k_j) * scale
+  const float4 qv = q4[c4];
+  float m = -INFINITY;
+  for (int j0 = 0; j0 < s; j0 += kpb) {
+    const int j = j0 + slot;
+    float p = 0.f;
+    if (j < s) {
+      const float4 kv = k4[(size_t)j * lpk + c4];
+      p = (qv.x * kv.x + qv.y * kv.y) + (qv.z * kv.z + qv.w * kv.w);
+    }
+    for (int o = lpk >> 1; o > 0; o >>= 1) p += __shfl_xor(p, o, 64);  // lpk is a power of two <= 64: stays inside the key's lanes
+    p *= scale;
+    if (j < s) {
+      if (c4 == 0) sc[j] = p;
+      m = fmaxf(m, p);
+    }
+  }
+  m = block_reduce_256<true>(m, lds4);  // the barriers inside also publish sc[]
+  float sum = 0.f;
+  for (int j = tid; j < s; j += 256) {
+    const float e = expf(sc[j] - m);
+    sc[j] = e;
+    sum += e;
+  }
+  sum = block_reduce_256<false>(sum, lds4);
+
+  // out = sum_j p_j v_j / sum: slot walks the keys, c4 owns 4 output columns
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int j = slot; j < s; j += kpb) {
+    const float p = sc[j];
+    const float4 vv = v4[(size_t)j * lpk + c4];
+    acc.x += p * vv.x;
+    acc.y += p * vv.y;
+    acc.z += p * vv.z;
+    acc.w += p * vv.w;
+  }
+  float4* red = reinterpret_cast<float4*>(sc + s + ((4 - (s & 3)) & 3));  // 16-byte aligned space after the scores
+  red[tid] = acc;
+  __syncthreads();
+  if (tid < lpk) {
+    float4 o = red[tid];
+    for (int i = 1; i < kpb; ++i) {
+      const float4 t = red[i * lpk + tid];
+      o.x += t.x;
+      o.y += t.y;
+      o.z += t.z;
+      o.w += t.w;
+    }
+    reinterpret_cast<float4*>(dst + (size_t)bh * d)[tid] = make_float4(o.x / sum, o.y / sum, o.z / sum, o.w / sum);
+  }
+}
+
+int check_f32(const ughip_slice* s, size_t need, const char* what) {
+  if (!s) return set_error(UGHIP_ERR_INVALID, "%s: null slice", what);
+  if (s->dtype != UGHIP_F32) return set_error(UGHIP_ERR_INVALID, "%s: unexpected dtype %s, expected F32", what, dtype_name(s->dtype));
+  if (s->len < need) return set_error(UGHIP_ERR_BOUNDS, "%s: slice has %zu elements, op needs %zu", what, s->len, need);
+  return UGHIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ughip_causal_softmax_rows(ughip_device* dev, const ughip_slice* src, ughip_slice* dst, size_t bh, size_t s1, size_t s2) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  const size_t n_rows = bh * s1, n = n_rows * s2;
+  if (int rc = check_f32(src, n, "causal_softmax src")) return rc;
+  if (int rc = check_f32(dst, n, "causal_softmax dst")) return rc;
+  if (src == dst) return set_error(UGHIP_ERR_INVALID, "causal_softmax: src and dst alias");
+  if (n == 0) return UGHIP_OK;
+  if (n_rows > 0x7fffffffull || s2 > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "causal_softmax: shape too large");
+  if (int rc = device_activate(dev)) return rc;
+  const float* s = static_cast<const float*>(src->ptr);
+  float* d = static_cast<float*>(dst->ptr);
+  hipStream_t st = dev->stream;
+  const int nr = (int)n_rows, nc = (int)s2, is1 = (int)s1;
+  const unsigned wave_blocks = (unsigned)((n_rows + 3) / 4);
+  if (s2 % 4 == 0 && s2 <= 256) causal_softmax_wave_v4<1><<<wave_blocks, 256, 0, st>>>(s, d, nr, is1, nc);
+  else if (s2 % 4 == 0 && s2 <= 512) causal_softmax_wave_v4<2><<<wave_blocks, 256, 0, st>>>(s, d, nr, is1, nc);
+  else if (s2 % 4 == 0 && s2 <= 1024) causal_softmax_wave_v4<4><<<wave_blocks, 256, 0, st>>>(s, d, nr, is1, nc);
+  else if (s2 % 4 == 0 && s2 <= 2048) causal_softmax_wave_v4<8><<<wave_blocks, 256, 0, st>>>(s, d, nr, is1, nc);
+  else causal_softmax_generic<<<nr, 256, 0, st>>>(s, d, is1, nc);
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+int ughip_attention_decode(ughip_device* dev, const ughip_slice* q, const ughip_slice* k, const ughip_slice* v, ughip_slice* dst, size_t b,
+                           size_t n_heads, size_t n_kv_heads, size_t s, size_t d, float scale) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  if (n_kv_heads == 0 || n_heads % n_kv_heads != 0)
+    return set_error(UGHIP_ERR_INVALID, "attention_decode: %zu heads are not a multiple of %zu kv heads", n_heads, n_kv_heads);
+  if (d < 16 || d > 256 || (d & (d - 1)) != 0) return set_error(UGHIP_ERR_INVALID, "attention_decode: head size %zu is not a power of two in 16..256", d);
+  if (s == 0) return set_error(UGHIP_ERR_INVALID, "attention_decode: empty key sequence");
+  if (s > 15000) return set_error(UGHIP_ERR_INVALID, "attention_decode: %zu keys exceed the 15000 this kernel holds in LDS", s);
+  if (int rc = check_f32(q, b * n_heads * d, "attention_decode q")) return rc;
+  if (int rc = check_f32(k, b * n_kv_heads * s * d, "attention_decode k")) return rc;
+  if (int rc = check_f32(v, b * n_kv_heads * s * d, "attention_decode v")) return rc;
+  if (int rc = check_f32(dst, b * n_heads * d, "attention_decode dst")) return rc;
+  if (dst == q || dst == k || dst == v) return set_error(UGHIP_ERR_INVALID, "attention_decode: dst aliases an input");
+  if (b * n_heads == 0) return UGHIP_OK;
+  if (b * n_heads > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "attention_decode: too many heads");
+  if (int rc = device_activate(dev)) return rc;
+  const size_t lds = (s + 3 + 256 * 4) * sizeof(float);  // scores, alignment slack, 256 float4
+  attention_decode_kernel<<<(unsigned)(b * n_heads), 256, lds, dev->stream>>>(static_cast<const float*>(q->ptr), static_cast<const float*>(k->ptr),
+                                                                              static_cast<const float*>(v->ptr), static_cast<float*>(dst->ptr), (int)n_heads,
+                                                                              (int)n_kv_heads, (int)s, (int)d, scale);
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+}  // extern "C"
