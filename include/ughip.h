@@ -235,6 +235,23 @@ int ughip_causal_softmax_rows(ughip_device* dev, const ughip_slice* src, ughip_s
 int ughip_attention_decode(ughip_device* dev, const ughip_slice* q, const ughip_slice* k,
                            const ughip_slice* v, ughip_slice* dst, size_t b, size_t n_heads,
                            size_t n_kv_heads, size_t s, size_t d, float scale);
+/* The same with rope (interleaved = 0, cpu_ops.rs:91-126) or rope_i (1, cpu_ops.rs:58-89) applied
+ * to q first, at table row pos[0]; q and dst are the flat [b, n_heads * d] rows the projections
+ * read and write, so the transposes of model.rs:210 and :245 disappear for one position.
+ * cos = sin = pos = NULL: no rotation. */
+int ughip_attention_decode_rope(ughip_device* dev, const ughip_slice* q, const ughip_slice* k,
+                                const ughip_slice* v, ughip_slice* dst, size_t b, size_t n_heads,
+                                size_t n_kv_heads, size_t s, size_t d, float scale,
+                                const ughip_slice* cos, const ughip_slice* sin,
+                                const ughip_slice* pos, int interleaved);
+/* Cache growth for one new position (model.rs:211-230 at t = 1): dst [bh, s_old + 1, d] =
+ * cat(cache [bh, s_old, d], x [bh, 1, d]) with x rotated first when cos/sin/pos are given
+ * (keys) and copied as is when they are NULL (values).  s_old may be 0 (cache may then be an
+ * empty slice or NULL).  d % 8 == 0. */
+int ughip_rope_append(ughip_device* dev, const ughip_slice* cache, const ughip_slice* x,
+                      ughip_slice* dst, size_t bh, size_t s_old, size_t d,
+                      const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos,
+                      int interleaved);
 
 /* ---- timing on the device stream ----------------------------------------------------- */
 int ughip_event_create(ughip_device* dev, ughip_event** out);

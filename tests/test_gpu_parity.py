@@ -578,3 +578,62 @@ def test_llama_fused_attention_ids_match_unfused_cpu(hip, cpu, hip_ops, cpu_ops,
     print("hip fused", toks_h.tolist(), "cpu", toks_c.tolist(), flush=True)
     assert toks_h.tolist() == toks_c.tolist()
     np.testing.assert_allclose(st_h["margins"], st_c["margins"], rtol=1e-2, atol=1e-7)
+
+
+def _rope_tables(dev, hd, max_pos=64):
+    cfg = ug_amd.LlamaConfig(hidden_size=hd * 4, num_attention_heads=4, num_key_value_heads=2, max_position_embeddings=max_pos)
+    cos, sin = ug_amd.llama.rope_tables(dev, cfg)
+    cos.realize()
+    sin.realize()
+    return cos, sin
+
+
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("b,n,s_old,d,with_rope", [(1, 4, 0, 64, True), (1, 4, 1, 64, True), (2, 2, 7, 64, True), (1, 4, 200, 64, True), (1, 4, 5, 64, False),
+                                                   (1, 3, 9, 16, True), (1, 2, 3, 128, True), (1, 2, 3, 12, True)])
+def test_rope_append_fused(hip, cpu, hip_ops, cpu_ops, interleaved, b, n, s_old, d, with_rope):
+    print("rope append", (b, n, s_old, d, with_rope, interleaved), flush=True)
+    cache = rng.normal(71, b * n * s_old * d) if s_old else np.zeros(0, np.float32)
+    x = rng.normal(72, b * n * d)
+
+    def run(dev, ops):
+        c = LB.copy(cache, (b, n, s_old, d), dev) if s_old else LB.cst(0.0, (b, n, 0, d), dev)
+        xs = LB.copy(x, (b, 1, n * d), dev)
+        if not with_rope:
+            return ops.rope_append(c, xs).data_vec()
+        cos, sin = _rope_tables(dev, d)
+        pos = LB.copy(np.array([min(s_old + 3, 60)], np.int32), (1, 1), dev)   # the table has 64 rows
+        return ops.rope_append(c, xs, cos, sin, pos, interleaved).data_vec()
+
+    got, want = run(hip, hip_ops), run(cpu, cpu_ops)      # split/transpose + rope + cat, op by op
+    # x1*c - x2*s cancels: fused multiply-adds on one side leave differences of an ulp of the operands
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6)
+    got = got.reshape(b, n, s_old + 1, d)
+    if s_old:
+        np.testing.assert_array_equal(got[:, :, :s_old], cache.reshape(b, n, s_old, d))   # the old rows are copied bit for bit
+    if not with_rope:
+        np.testing.assert_array_equal(got[:, :, s_old], x.reshape(b, n, d))
+    else:
+        np.testing.assert_allclose(np.linalg.norm(got[:, :, s_old], axis=-1), np.linalg.norm(x.reshape(b, n, d), axis=-1), rtol=1e-5)
+
+
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("b,nh,nkv,s,d,with_rope", [(1, 32, 4, 1, 64, True), (1, 32, 4, 130, 64, True), (2, 8, 2, 40, 64, True), (1, 8, 8, 33, 128, True),
+                                                    (1, 32, 4, 77, 64, False), (1, 4, 1, 9, 16, True)])
+def test_attention_decode_flat_fused(hip, cpu, hip_ops, cpu_ops, interleaved, b, nh, nkv, s, d, with_rope):
+    print("attention decode flat", (b, nh, nkv, s, d, with_rope, interleaved), flush=True)
+    q, k, v = rng.normal(73, b * nh * d), rng.normal(74, b * nkv * s * d), rng.normal(75, b * nkv * s * d)
+    scale = float(np.float32(d) ** np.float32(-0.5))
+
+    def run(dev, ops):
+        args = [LB.copy(q, (b, 1, nh * d), dev), LB.copy(k, (b, nkv, s, d), dev), LB.copy(v, (b, nkv, s, d), dev), scale]
+        if with_rope:
+            cos, sin = _rope_tables(dev, d)
+            args += [cos, sin, LB.copy(np.array([min(s, 60)], np.int32), (1, 1), dev), interleaved]
+        out = ops.attention_decode_flat(*args)
+        assert tuple(out.dims()) == (b, 1, nh * d)
+        return out.data_vec()
+
+    got, want = run(hip, hip_ops), run(cpu, cpu_ops)
+    scale_abs = float(np.abs(want).max())
+    np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-5 * scale_abs)

@@ -102,13 +102,15 @@ class NumpyLlama:
 
 
 @pytest.mark.parametrize("interleaved", [False, True])
-@pytest.mark.parametrize("custom_softmax", [False, True])
-def test_llama_restatement_matches_numpy_f64(cpu, cpu_ops, interleaved, custom_softmax):
+@pytest.mark.parametrize("custom_softmax,fused", [(False, False), (True, False), (True, True)])
+def test_llama_restatement_matches_numpy_f64(cpu, cpu_ops, interleaved, custom_softmax, fused):
+    """fused=True routes attention through the optional Ops hooks, whose defaults (used by the CPU
+    ops) are the same ops composed one by one: the graph changes shape, the values must not."""
     cfg = ug_amd.LlamaConfig(hidden_size=128, intermediate_size=320, max_position_embeddings=64, num_attention_heads=4, num_key_value_heads=2,
                              num_hidden_layers=2, vocab_size=512, rope_interleaved=interleaved)
     prompt = rng.token_ids(10, 12, cfg.vocab_size)
     want_ids, want_margins = NumpyLlama(cfg).generate(prompt.tolist(), 6)
-    model = ug_amd.LlamaModel(cpu, cpu_ops, cfg, custom_softmax, seed=SEED, std=STD)
+    model = ug_amd.LlamaModel(cpu, cpu_ops, cfg, custom_softmax, seed=SEED, std=STD, fused_attention=fused)
     ids, st = model.generate(prompt, 6)
     assert ids.tolist() == want_ids.tolist()
     np.testing.assert_allclose(st["margins"], want_margins, rtol=1e-3, atol=1e-4)

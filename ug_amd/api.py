@@ -641,6 +641,23 @@ class LlamaOps(_Handle):
         return lb
 
 
+    def rope_append(self, cache, x, cos=None, sin=None, pos=None, interleaved=False):
+        """cache [b, n, s, d] grown by the row(s) of x [b, 1, n * d], rotated when a table is given."""
+        rope = cos is not None
+        lb = self._op("ugh_llama_rope_append", cache, _p(x.h), _p(cos.h) if rope else None, _p(sin.h) if rope else None,
+                      _p(pos.h) if rope else None, int(interleaved))
+        lb._keep += [x] + ([cos, sin, pos] if rope else [])
+        return lb
+
+    def attention_decode_flat(self, q, k, v, scale, cos=None, sin=None, pos=None, interleaved=False):
+        """q [b, 1, nh * d] (rotated first when a table is given), k and v [b, nkv, s, d] -> [b, 1, nh * d]."""
+        rope = cos is not None
+        lb = self._op("ugh_llama_attention_decode_flat", q, _p(k.h), _p(v.h), C.c_float(scale), _p(cos.h) if rope else None,
+                      _p(sin.h) if rope else None, _p(pos.h) if rope else None, int(interleaved))
+        lb._keep += [k, v] + ([cos, sin, pos] if rope else [])
+        return lb
+
+
 class _Llama:
     """Graph builders of ug-llama/src/model.rs:32-109."""
 

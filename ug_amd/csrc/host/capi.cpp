@@ -396,6 +396,18 @@ int ugh_llama_causal_softmax(void* ops, void* src, void** out) {
 int ugh_llama_attention_decode(void* ops, void* q, void* k, void* v, float scale, void** out) {
   return guard([&] { *out = box(ops_of(ops).attention_decode(lb_of(q), lb_of(k), lb_of(v), scale)); });
 }
+int ugh_llama_rope_append(void* ops, void* cache, void* x, void* cos, void* sin, void* pos, int interleaved, void** out) {
+  return guard([&] {
+    if (cos) *out = box(ops_of(ops).rope_append(lb_of(cache), lb_of(x), &lb_of(cos), &lb_of(sin), &lb_of(pos), interleaved != 0));
+    else *out = box(ops_of(ops).rope_append(lb_of(cache), lb_of(x), nullptr, nullptr, nullptr, false));
+  });
+}
+int ugh_llama_attention_decode_flat(void* ops, void* q, void* k, void* v, float scale, void* cos, void* sin, void* pos, int interleaved, void** out) {
+  return guard([&] {
+    if (cos) *out = box(ops_of(ops).attention_decode_flat(lb_of(q), lb_of(k), lb_of(v), scale, &lb_of(cos), &lb_of(sin), &lb_of(pos), interleaved != 0));
+    else *out = box(ops_of(ops).attention_decode_flat(lb_of(q), lb_of(k), lb_of(v), scale, nullptr, nullptr, nullptr, false));
+  });
+}
 int ugh_llama_rms_norm(void* src, void* alpha, float eps, void** out) {
   return guard([&] { *out = box(ug_llama::rms_norm(lb_of(src), lb_of(alpha), eps)); });
 }

@@ -101,6 +101,56 @@ struct HipOps : Ops {
     return LB::custom(f, {q, k, v}, q.shape(), q.dtype(), q.device());
   }
 
+  LB rope_append(const LB& cache, const LB& x, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const override {
+    if (cache.rank() != 4 || x.rank() != 3 || x.dims()[1] != 1) bail("rope_append: expected cache [b, n, s, d] and x [b, 1, n * d]");
+    size_t b = cache.dims()[0], n = cache.dims()[1], s_old = cache.dims()[2], d = cache.dims()[3];
+    if (x.dims()[0] != b || x.dims()[2] != n * d) bail("rope_append: mismatched shapes " + cache.shape().str() + " " + x.shape().str());
+    if (d % 8 != 0) return Ops::rope_append(cache, x, cos, sin, pos, interleaved);
+    ughip_device* dev = hip_dev(x);
+    const bool with_rope = cos != nullptr;
+    int il = interleaved ? 1 : 0;
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != (with_rope ? 6u : 3u)) bail("rope_append: unexpected number of slices");
+      ughip_slice* dst = hip_raw_slice(*vs.back());
+      hip_check(ughip_rope_append(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), dst, b * n, s_old, d, with_rope ? hip_raw_slice(*vs[2]) : nullptr,
+                                  with_rope ? hip_raw_slice(*vs[3]) : nullptr, with_rope ? hip_raw_slice(*vs[4]) : nullptr, il),
+                "rope_append");
+    };
+    std::vector<LB> args = {cache, x};
+    if (with_rope) {
+      args.push_back(*cos);
+      args.push_back(*sin);
+      args.push_back(*pos);
+    }
+    return LB::custom(f, args, Shape({b, n, s_old + 1, d}), x.dtype(), x.device());
+  }
+
+  LB attention_decode_flat(const LB& q, const LB& k, const LB& v, float scale, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const override {
+    if (q.rank() != 3 || q.dims()[1] != 1 || k.rank() != 4 || v.rank() != 4) bail("attention_decode_flat: expected q [b, 1, nh * d] and k, v [b, nkv, s, d]");
+    size_t b = q.dims()[0], nkv = k.dims()[1], s = k.dims()[2], d = k.dims()[3];
+    if (k.dims() != v.dims() || k.dims()[0] != b || d == 0 || q.dims()[2] % d != 0)
+      bail("attention_decode_flat: mismatched shapes " + q.shape().str() + " " + k.shape().str());
+    size_t nh = q.dims()[2] / d;
+    ughip_device* dev = hip_dev(q);
+    const bool with_rope = cos != nullptr;
+    int il = interleaved ? 1 : 0;
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != (with_rope ? 7u : 4u)) bail("attention_decode_flat: unexpected number of slices");
+      ughip_slice* dst = hip_raw_slice(*vs.back());
+      hip_check(ughip_attention_decode_rope(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), dst, b, nh, nkv, s, d, scale,
+                                            with_rope ? hip_raw_slice(*vs[3]) : nullptr, with_rope ? hip_raw_slice(*vs[4]) : nullptr,
+                                            with_rope ? hip_raw_slice(*vs[5]) : nullptr, il),
+                "attention_decode_flat");
+    };
+    std::vector<LB> args = {q, k, v};
+    if (with_rope) {
+      args.push_back(*cos);
+      args.push_back(*sin);
+      args.push_back(*pos);
+    }
+    return LB::custom(f, args, q.shape(), q.dtype(), q.device());
+  }
+
   LB causal_mask(const LB& src) const override {
     if (src.rank() != 4) bail("causal_mask: expected a rank-4 tensor, got " + src.shape().str());
     size_t bh = src.dims()[0] * src.dims()[1], s1 = src.dims()[2], s2 = src.dims()[3];
@@ -164,6 +214,22 @@ LB Ops::attention_decode(const LB& q, const LB& k, const LB& v, float scale) con
   LB att = q.matmul_t(kr);
   att = att.binary(BinaryOp::Mul, LB::cst(Const::f32(scale), Shape(), q.device()).broadcast(att.shape()));
   return custom_softmax(att).matmul(vr);
+}
+
+// model.rs:207-230 for one new position, op by op.
+LB Ops::rope_append(const LB& cache, const LB& x, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const {
+  size_t n = cache.dims()[1], d = cache.dims()[3];
+  LB row = x.split_dim(2, n, d).transpose(2, 1);
+  if (cos) row = interleaved ? rope_i(row, *cos, *sin, *pos) : rope(row, *cos, *sin, *pos);
+  return cat(cache, row, 2);
+}
+
+// model.rs:207-210, 231-245 for one query position, op by op.
+LB Ops::attention_decode_flat(const LB& q, const LB& k, const LB& v, float scale, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const {
+  size_t d = k.dims()[3], nh = q.dims()[2] / d;
+  LB qh = q.split_dim(2, nh, d).transpose(2, 1);
+  if (cos) qh = interleaved ? rope_i(qh, *cos, *sin, *pos) : rope(qh, *cos, *sin, *pos);
+  return attention_decode(qh, k, v, scale).transpose(2, 1).merge_dims(-2);
 }
 
 std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16) {
@@ -302,6 +368,14 @@ LB Model::attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache) c
   LB q = xs.matmul_t(l.q_proj);
   LB k = xs.matmul_t(l.k_proj);
   LB v = xs.matmul_t(l.v_proj);
+  if (fused_attention_ && seq_len == 1) {
+    // one new position: rows go from the projections into the caches and the attention kernel
+    // without the split/transpose copies, and the result comes back in the layout o_proj reads
+    cache.prev_k = ops_->rope_append(cache.prev_k, k, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved);
+    cache.prev_v = ops_->rope_append(cache.prev_v, v, nullptr, nullptr, nullptr, false);
+    LB out = ops_->attention_decode_flat(q, cache.prev_k, cache.prev_v, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved);
+    return out.matmul_t(l.o_proj);
+  }
   q = q.split_dim(2, nh, hd).transpose(2, 1);
   k = k.split_dim(2, nkv, hd).transpose(2, 1);
   v = v.split_dim(2, nkv, hd).transpose(2, 1);
@@ -318,9 +392,7 @@ LB Model::attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache) c
   cache.prev_v = v;
   const float scale_v = std::pow((float)hd, -0.5f);
   LB out;
-  if (fused_attention_ && seq_len == 1) {
-    out = ops_->attention_decode(q, k, v, scale_v);
-  } else {
+  {
     LB kr = repeat(k, 1, nh / nkv);
     LB vr = repeat(v, 1, nh / nkv);
     LB att = q.matmul_t(kr);

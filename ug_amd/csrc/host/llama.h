@@ -27,6 +27,13 @@ struct Ops {
   virtual LB causal_softmax(const LB& att) const { return custom_softmax(causal_mask(att)); }
   // One query position: q [b, nh, 1, d], k and v [b, nkv, s, d] -> [b, nh, 1, d].
   virtual LB attention_decode(const LB& q, const LB& k, const LB& v, float scale) const;
+  // One new position straight from the projections (model.rs:207-230 at t = 1): x [b, 1, n * d]
+  // becomes one row per head, rotated when a table is given (cos/sin/pos non-null), appended to
+  // cache [b, n, s, d] -> [b, n, s + 1, d].
+  virtual LB rope_append(const LB& cache, const LB& x, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const;
+  // q [b, 1, nh * d] (rotated first when a table is given), k and v [b, nkv, s, d] -> [b, 1, nh * d].
+  virtual LB attention_decode_flat(const LB& q, const LB& k, const LB& v, float scale, const LB* cos, const LB* sin, const LB* pos,
+                                   bool interleaved) const;
 };
 
 // The HIP implementation (counterpart of ug-llama/src/cuda_ops.rs).

@@ -5,8 +5,12 @@
 //   ughip_attention_decode     = for one query position, the chain of ug-llama/src/model.rs:231-244
 //                                repeat(k), repeat(v), q x k^T, * scale, softmax, x v
 //                                in one launch, reading each K/V head once (no repeated copies).
+//   ughip_rope_append          = for one new position, split/transpose + rope (or nothing) + cat
+//                                (model.rs:213-230): the cache grows by one rotated row per head.
+//   ughip_attention_decode with a rope table = the same with rope applied to q first, q and the
+//                                result in the flat [b, nh * d] layout the projections use.
 //
-// Both reduce in a fixed order (no atomics): results do not change from run to run.
+// All reduce in a fixed order (no atomics): results do not change from run to run.
 #include <hip/hip_runtime.h>
 
 #include "internal.h"
@@ -98,10 +102,15 @@ __global__ void __launch_bounds__(256) causal_softmax_generic(const float* __res
 // One workgroup (256 threads) per query head.  q: [b, nh, d]; k, v: [b, nkv, s, d]; dst: [b, nh, d].
 // LPK = d / 4 lanes share one key row (one 128-bit load each, a row is one contiguous 4*d bytes);
 // 256 / LPK keys are in flight per step.  Scores and probabilities live in LDS (s floats).
+// With a rope table (cos_t != nullptr) q is rotated first, at table row pos[0] (rope: pairs
+// (i, i + d/2); rope_i: pairs (2i, 2i + 1); cpu_ops.rs:58-126 for t = 1).
 __global__ void __launch_bounds__(256) attention_decode_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
-                                                               float* __restrict__ dst, int nh, int nkv, int s, int d, float scale) {
+                                                               float* __restrict__ dst, int nh, int nkv, int s, int d, float scale,
+                                                               const float* __restrict__ cos_t, const float* __restrict__ sin_t, const int* __restrict__ pos,
+                                                               size_t table_len, int interleaved) {
   extern __shared__ __attribute__((aligned(16))) float sc[];  // s scores, then 256 float4 of reduction space
   __shared__ float lds4[4];
+  __shared__ __attribute__((aligned(16))) float qs[256];
   const int tid = threadIdx.x;
   const int lpk = d >> 2, kpb = 256 / lpk;  // lanes per key, keys per step
   const int c4 = tid % lpk, slot = tid / lpk;
@@ -110,8 +119,25 @@ __global__ void __launch_bounds__(256) attention_decode_kernel(const float* __re
   const float4* k4 = reinterpret_cast<const float4*>(k + ((size_t)b * nkv + kvh) * (size_t)s * d);
   const float4* v4 = reinterpret_cast<const float4*>(v + ((size_t)b * nkv + kvh) * (size_t)s * d);
 
+  float4 qv;
+  if (cos_t) {
+    const int half = d >> 1;
+    if (tid < half) {
+      const long long p = pos[0];
+      const size_t ics = (size_t)p * half + tid;
+      const bool ok = p >= 0 && ics < table_len;
+      const float c = ok ? cos_t[ics] : NAN, sn = ok ? sin_t[ics] : NAN;
+      const int i1 = interleaved ? 2 * tid : tid, i2 = interleaved ? 2 * tid + 1 : tid + half;
+      const float x1 = q[(size_t)bh * d + i1], x2 = q[(size_t)bh * d + i2];
+      qs[i1] = x1 * c - x2 * sn;
+      qs[i2] = x1 * sn + x2 * c;
+    }
+    __syncthreads();
+    qv = reinterpret_cast<const float4*>(qs)[c4];
+  } else {
+    qv = q4[c4];
+  }
   // scores = (q . k_j) * scale
-  const float4 qv = q4[c4];
   float m = -INFINITY;
   for (int j0 = 0; j0 < s; j0 += kpb) {
     const int j = j0 + slot;
@@ -162,6 +188,47 @@ __global__ void __launch_bounds__(256) attention_decode_kernel(const float* __re
   }
 }
 
+// ---- cache append for one new position ------------------------------------------------------------
+// dst [bh, s_old + 1, d] = cat(cache [bh, s_old, d], row(x [bh, d])) along the middle dim, the new
+// row rotated when a table is given.  One thread per float4 of dst (d % 8 == 0).
+__global__ void __launch_bounds__(256) rope_append_kernel(const float* __restrict__ cache, const float* __restrict__ x, float* __restrict__ dst, size_t n4,
+                                                          int s_old, int d, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                          const int* __restrict__ pos, size_t table_len, int interleaved) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n4) return;
+  const int d4 = d >> 2;
+  const int c4 = (int)(g % d4);
+  const size_t row = g / d4;  // flat (bh, j), j in 0..s_old
+  const int j = (int)(row % (s_old + 1));
+  const size_t bh = row / (s_old + 1);
+  float4 out;
+  if (j < s_old) {
+    out = reinterpret_cast<const float4*>(cache)[(bh * s_old + j) * d4 + c4];
+  } else if (!cos_t) {
+    out = reinterpret_cast<const float4*>(x)[bh * d4 + c4];
+  } else {
+    const float* xr = x + bh * d;
+    const int half = d >> 1;
+    const long long p = pos[0];
+    float o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int i = c4 * 4 + e;  // output element
+      // pair index and whether i is the first or the second element of its pair
+      const int pr = interleaved ? i >> 1 : (i < half ? i : i - half);
+      const bool first = interleaved ? (i & 1) == 0 : i < half;
+      const int i1 = interleaved ? 2 * pr : pr, i2 = interleaved ? 2 * pr + 1 : pr + half;
+      const size_t ics = (size_t)p * half + pr;
+      const bool ok = p >= 0 && ics < table_len;
+      const float c = ok ? cos_t[ics] : NAN, sn = ok ? sin_t[ics] : NAN;
+      const float x1 = xr[i1], x2 = xr[i2];
+      o[e] = first ? x1 * c - x2 * sn : x1 * sn + x2 * c;
+    }
+    out = make_float4(o[0], o[1], o[2], o[3]);
+  }
+  reinterpret_cast<float4*>(dst)[g] = out;
+}
+
 int check_f32(const ughip_slice* s, size_t need, const char* what) {
   if (!s) return set_error(UGHIP_ERR_INVALID, "%s: null slice", what);
   if (s->dtype != UGHIP_F32) return set_error(UGHIP_ERR_INVALID, "%s: unexpected dtype %s, expected F32", what, dtype_name(s->dtype));
@@ -196,9 +263,27 @@ int ughip_causal_softmax_rows(ughip_device* dev, const ughip_slice* src, ughip_s
   return UGHIP_OK;
 }
 
+namespace {
+int check_rope_table(const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos, size_t d, const char* what) {
+  if (!cos || !sin || cos->dtype != UGHIP_F32 || sin->dtype != UGHIP_F32) return set_error(UGHIP_ERR_INVALID, "%s: cos/sin must be F32 slices", what);
+  if (cos->len < d / 2 || sin->len < d / 2) return set_error(UGHIP_ERR_BOUNDS, "%s: rope table shorter than one row of %zu", what, d / 2);
+  if (!pos || pos->dtype != UGHIP_I32 || pos->len < 1) return set_error(UGHIP_ERR_INVALID, "%s: pos must be a non-empty I32 slice", what);
+  return UGHIP_OK;
+}
+}  // namespace
+
 int ughip_attention_decode(ughip_device* dev, const ughip_slice* q, const ughip_slice* k, const ughip_slice* v, ughip_slice* dst, size_t b,
                            size_t n_heads, size_t n_kv_heads, size_t s, size_t d, float scale) {
+  return ughip_attention_decode_rope(dev, q, k, v, dst, b, n_heads, n_kv_heads, s, d, scale, nullptr, nullptr, nullptr, 0);
+}
+
+int ughip_attention_decode_rope(ughip_device* dev, const ughip_slice* q, const ughip_slice* k, const ughip_slice* v, ughip_slice* dst, size_t b,
+                                size_t n_heads, size_t n_kv_heads, size_t s, size_t d, float scale, const ughip_slice* cos, const ughip_slice* sin,
+                                const ughip_slice* pos, int interleaved) {
   if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  const bool rope = cos || sin || pos;
+  if (rope)
+    if (int rc = check_rope_table(cos, sin, pos, d, "attention_decode")) return rc;
   if (n_kv_heads == 0 || n_heads % n_kv_heads != 0)
     return set_error(UGHIP_ERR_INVALID, "attention_decode: %zu heads are not a multiple of %zu kv heads", n_heads, n_kv_heads);
   if (d < 16 || d > 256 || (d & (d - 1)) != 0) return set_error(UGHIP_ERR_INVALID, "attention_decode: head size %zu is not a power of two in 16..256", d);
@@ -215,7 +300,38 @@ int ughip_attention_decode(ughip_device* dev, const ughip_slice* q, const ughip_
   const size_t lds = (s + 3 + 256 * 4) * sizeof(float);  // scores, alignment slack, 256 float4
   attention_decode_kernel<<<(unsigned)(b * n_heads), 256, lds, dev->stream>>>(static_cast<const float*>(q->ptr), static_cast<const float*>(k->ptr),
                                                                               static_cast<const float*>(v->ptr), static_cast<float*>(dst->ptr), (int)n_heads,
-                                                                              (int)n_kv_heads, (int)s, (int)d, scale);
+                                                                              (int)n_kv_heads, (int)s, (int)d, scale,
+                                                                              rope ? static_cast<const float*>(cos->ptr) : nullptr,
+                                                                              rope ? static_cast<const float*>(sin->ptr) : nullptr,
+                                                                              rope ? static_cast<const int*>(pos->ptr) : nullptr,
+                                                                              rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved);
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+int ughip_rope_append(ughip_device* dev, const ughip_slice* cache, const ughip_slice* x, ughip_slice* dst, size_t bh, size_t s_old, size_t d,
+                      const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos, int interleaved) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  if (d == 0 || d % 8 != 0) return set_error(UGHIP_ERR_INVALID, "rope_append: head size %zu is not a multiple of 8", d);
+  const bool rope = cos || sin || pos;
+  if (rope)
+    if (int rc = check_rope_table(cos, sin, pos, d, "rope_append")) return rc;
+  if (s_old) {
+    if (int rc = check_f32(cache, bh * s_old * d, "rope_append cache")) return rc;
+  } else if (cache && cache->dtype != UGHIP_F32) {
+    return set_error(UGHIP_ERR_INVALID, "rope_append cache: unexpected dtype %s, expected F32", dtype_name(cache->dtype));
+  }
+  if (int rc = check_f32(x, bh * d, "rope_append x")) return rc;
+  if (int rc = check_f32(dst, bh * (s_old + 1) * d, "rope_append dst")) return rc;
+  if (dst == cache || dst == x) return set_error(UGHIP_ERR_INVALID, "rope_append: dst aliases an input");
+  if (bh == 0) return UGHIP_OK;
+  if (s_old + 1 > 0x7fffffffull || d > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "rope_append: shape too large");
+  if (int rc = device_activate(dev)) return rc;
+  const size_t n4 = bh * (s_old + 1) * d / 4;
+  rope_append_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, dev->stream>>>(
+      s_old ? static_cast<const float*>(cache->ptr) : nullptr, static_cast<const float*>(x->ptr), static_cast<float*>(dst->ptr), n4, (int)s_old, (int)d,
+      rope ? static_cast<const float*>(cos->ptr) : nullptr, rope ? static_cast<const float*>(sin->ptr) : nullptr,
+      rope ? static_cast<const int*>(pos->ptr) : nullptr, rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
 }

@@ -4,6 +4,8 @@
 // ug-core/src/cpu_runtime.rs:527-619).
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "gemm.h"
 #include "internal.h"
 #include "ughip.h"
@@ -341,6 +343,8 @@ void launch_gemv_nt_any(hipStream_t st, const MMArgs& p, size_t b) {
   // enough waves to hide HBM latency: about 8192 over the chip
   const size_t cols = (size_t)p.N * b;
   int ks = cols <= 2048 ? 4 : cols <= 6144 ? 2 : 1;
+  if (const char* e = getenv("UGHIP_GEMV_KS")) ks = atoi(e);  // tuning aid: 1, 2 or 4
+  if (ks != 1 && ks != 2 && ks != 4) ks = 1;
   while (ks > 1 && p.K < 64 * VE * ks) ks >>= 1;
   if (ks == 4) launch_gemv_nt<T, 4>(st, p, b);
   else if (ks == 2) launch_gemv_nt<T, 2>(st, p, b);
