@@ -99,20 +99,36 @@ __global__ void __launch_bounds__(256) causal_softmax_generic(const float* __res
 }
 
 // ---- single-query attention -----------------------------------------------------------------------
-// One workgroup (256 threads) per query head.  q: [b, nh, d]; k, v: [b, nkv, s, d]; dst: [b, nh, d].
+// One workgroup of 1024 threads per query head.  q: [b, nh, d]; k, v: [b, nkv, s, d]; dst: [b, nh, d].
 // LPK = d / 4 lanes share one key row (one 128-bit load each, a row is one contiguous 4*d bytes);
-// 256 / LPK keys are in flight per step.  Scores and probabilities live in LDS (s floats).
+// 1024 / LPK keys are in flight per step and four steps per loop trip, because at batch 1 this
+// kernel is a chain of L2 round trips, not a bandwidth problem.  Scores and probabilities live in
+// LDS (s floats).
 // With a rope table (cos_t != nullptr) q is rotated first, at table row pos[0] (rope: pairs
 // (i, i + d/2); rope_i: pairs (2i, 2i + 1); cpu_ops.rs:58-126 for t = 1).
-__global__ void __launch_bounds__(256) attention_decode_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
-                                                               float* __restrict__ dst, int nh, int nkv, int s, int d, float scale,
-                                                               const float* __restrict__ cos_t, const float* __restrict__ sin_t, const int* __restrict__ pos,
-                                                               size_t table_len, int interleaved) {
-  extern __shared__ __attribute__((aligned(16))) float sc[];  // s scores, then 256 float4 of reduction space
-  __shared__ float lds4[4];
+constexpr int ATT_THREADS = 1024, ATT_WAVES = ATT_THREADS / 64;
+
+template <bool IS_MAX>
+__device__ __forceinline__ float att_block_reduce(float v, float* lds16) {
+  v = IS_MAX ? wave_max(v) : wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds16[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = lds16[0];
+#pragma unroll
+  for (int i = 1; i < ATT_WAVES; ++i) r = IS_MAX ? fmaxf(r, lds16[i]) : r + lds16[i];
+  return r;
+}
+
+__global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
+                                                                       float* __restrict__ dst, int nh, int nkv, int s, int d, float scale,
+                                                                       const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                                       const int* __restrict__ pos, size_t table_len, int interleaved) {
+  extern __shared__ __attribute__((aligned(16))) float sc[];  // s scores, then ATT_WAVES * 64 float4 of reduction space
+  __shared__ float lds16[ATT_WAVES];
   __shared__ __attribute__((aligned(16))) float qs[256];
   const int tid = threadIdx.x;
-  const int lpk = d >> 2, kpb = 256 / lpk;  // lanes per key, keys per step
+  const int lpk = d >> 2, kpb = ATT_THREADS / lpk;  // lanes per key, keys per step
   const int c4 = tid % lpk, slot = tid / lpk;
   const int bh = blockIdx.x, b = bh / nh, h = bh % nh, kvh = h / (nh / nkv);
   const float4* q4 = reinterpret_cast<const float4*>(q + (size_t)bh * d);
@@ -137,48 +153,74 @@ __global__ void __launch_bounds__(256) attention_decode_kernel(const float* __re
   } else {
     qv = q4[c4];
   }
-  // scores = (q . k_j) * scale
+  // scores = (q . k_j) * scale, four key rows per lane group in flight
   float m = -INFINITY;
-  for (int j0 = 0; j0 < s; j0 += kpb) {
-    const int j = j0 + slot;
-    float p = 0.f;
-    if (j < s) {
-      const float4 kv = k4[(size_t)j * lpk + c4];
-      p = (qv.x * kv.x + qv.y * kv.y) + (qv.z * kv.z + qv.w * kv.w);
+  for (int j0 = 0; j0 < s; j0 += 4 * kpb) {
+    float p[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u * kpb + slot;
+      p[u] = 0.f;
+      if (j < s) {
+        const float4 kv = k4[(size_t)j * lpk + c4];
+        p[u] = (qv.x * kv.x + qv.y * kv.y) + (qv.z * kv.z + qv.w * kv.w);
+      }
     }
-    for (int o = lpk >> 1; o > 0; o >>= 1) p += __shfl_xor(p, o, 64);  // lpk is a power of two <= 64: stays inside the key's lanes
-    p *= scale;
-    if (j < s) {
-      if (c4 == 0) sc[j] = p;
-      m = fmaxf(m, p);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      float pu = p[u];
+      for (int o = lpk >> 1; o > 0; o >>= 1) pu += __shfl_xor(pu, o, 64);  // lpk is a power of two <= 64: stays inside the key's lanes
+      pu *= scale;
+      const int j = j0 + u * kpb + slot;
+      if (j < s) {
+        if (c4 == 0) sc[j] = pu;
+        m = fmaxf(m, pu);
+      }
     }
   }
-  m = block_reduce_256<true>(m, lds4);  // the barriers inside also publish sc[]
+  m = att_block_reduce<true>(m, lds16);  // the barriers inside also publish sc[]
   float sum = 0.f;
-  for (int j = tid; j < s; j += 256) {
+  for (int j = tid; j < s; j += ATT_THREADS) {
     const float e = expf(sc[j] - m);
     sc[j] = e;
     sum += e;
   }
-  sum = block_reduce_256<false>(sum, lds4);
+  sum = att_block_reduce<false>(sum, lds16);
 
   // out = sum_j p_j v_j / sum: slot walks the keys, c4 owns 4 output columns
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int j = slot; j < s; j += kpb) {
-    const float p = sc[j];
-    const float4 vv = v4[(size_t)j * lpk + c4];
-    acc.x += p * vv.x;
-    acc.y += p * vv.y;
-    acc.z += p * vv.z;
-    acc.w += p * vv.w;
+  for (int j0 = slot; j0 < s; j0 += 4 * kpb) {
+    float4 vv[4];
+    float pj[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u * kpb;
+      pj[u] = j < s ? sc[j] : 0.f;
+      vv[u] = j < s ? v4[(size_t)j * lpk + c4] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      acc.x += pj[u] * vv[u].x;
+      acc.y += pj[u] * vv[u].y;
+      acc.z += pj[u] * vv[u].z;
+      acc.w += pj[u] * vv[u].w;
+    }
+  }
+  // the slots of one wave (lanes lpk apart), then the waves in order
+  for (int o = lpk; o < 64; o <<= 1) {
+    acc.x += __shfl_xor(acc.x, o, 64);
+    acc.y += __shfl_xor(acc.y, o, 64);
+    acc.z += __shfl_xor(acc.z, o, 64);
+    acc.w += __shfl_xor(acc.w, o, 64);
   }
   float4* red = reinterpret_cast<float4*>(sc + s + ((4 - (s & 3)) & 3));  // 16-byte aligned space after the scores
-  red[tid] = acc;
+  const int lane = tid & 63, wave = tid >> 6;
+  if (lane < lpk) red[wave * 64 + lane] = acc;
   __syncthreads();
   if (tid < lpk) {
     float4 o = red[tid];
-    for (int i = 1; i < kpb; ++i) {
-      const float4 t = red[i * lpk + tid];
+    for (int w = 1; w < ATT_WAVES; ++w) {
+      const float4 t = red[w * 64 + tid];
       o.x += t.x;
       o.y += t.y;
       o.z += t.z;
@@ -288,7 +330,7 @@ int ughip_attention_decode_rope(ughip_device* dev, const ughip_slice* q, const u
     return set_error(UGHIP_ERR_INVALID, "attention_decode: %zu heads are not a multiple of %zu kv heads", n_heads, n_kv_heads);
   if (d < 16 || d > 256 || (d & (d - 1)) != 0) return set_error(UGHIP_ERR_INVALID, "attention_decode: head size %zu is not a power of two in 16..256", d);
   if (s == 0) return set_error(UGHIP_ERR_INVALID, "attention_decode: empty key sequence");
-  if (s > 15000) return set_error(UGHIP_ERR_INVALID, "attention_decode: %zu keys exceed the 15000 this kernel holds in LDS", s);
+  if (s > 12000) return set_error(UGHIP_ERR_INVALID, "attention_decode: %zu keys exceed the 12000 this kernel holds in LDS", s);
   if (int rc = check_f32(q, b * n_heads * d, "attention_decode q")) return rc;
   if (int rc = check_f32(k, b * n_kv_heads * s * d, "attention_decode k")) return rc;
   if (int rc = check_f32(v, b * n_kv_heads * s * d, "attention_decode v")) return rc;
@@ -297,8 +339,8 @@ int ughip_attention_decode_rope(ughip_device* dev, const ughip_slice* q, const u
   if (b * n_heads == 0) return UGHIP_OK;
   if (b * n_heads > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "attention_decode: too many heads");
   if (int rc = device_activate(dev)) return rc;
-  const size_t lds = (s + 3 + 256 * 4) * sizeof(float);  // scores, alignment slack, 256 float4
-  attention_decode_kernel<<<(unsigned)(b * n_heads), 256, lds, dev->stream>>>(static_cast<const float*>(q->ptr), static_cast<const float*>(k->ptr),
+  const size_t lds = (s + 3 + ATT_WAVES * 64 * 4) * sizeof(float);  // scores, alignment slack, one float4 per lane slot of every wave
+  attention_decode_kernel<<<(unsigned)(b * n_heads), ATT_THREADS, lds, dev->stream>>>(static_cast<const float*>(q->ptr), static_cast<const float*>(k->ptr),
                                                                               static_cast<const float*>(v->ptr), static_cast<float*>(dst->ptr), (int)n_heads,
                                                                               (int)n_kv_heads, (int)s, (int)d, scale,
                                                                               rope ? static_cast<const float*>(cos->ptr) : nullptr,
