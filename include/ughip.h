@@ -253,6 +253,14 @@ int ughip_rope_append(ughip_device* dev, const ughip_slice* cache, const ughip_s
                       const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos,
                       int interleaved);
 
+/* ---- element type conversion ------------------------------------------------------------------
+ * dst[i] = (dtype of dst) src[i], same length, any pair of the five dtypes.  Replaces the host
+ * loops of ug-core/src/safetensors.rs:141-271 (load_with_cast converts on the CPU, then uploads):
+ * a checkpoint is uploaded in its stored dtype and widened on the device.  Same numerics as that
+ * code: half::{bf16,f16}::from_f32 rounding, Rust `as` for float -> integer (truncate, saturate,
+ * NaN -> 0) and for i64 -> i32 (wrap); integers reach bf16/f16 through f32. */
+int ughip_convert(ughip_device* dev, const ughip_slice* src, ughip_slice* dst);
+
 /* ---- timing on the device stream ----------------------------------------------------- */
 int ughip_event_create(ughip_device* dev, ughip_event** out);
 int ughip_event_record(ughip_event* ev);

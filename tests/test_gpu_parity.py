@@ -637,3 +637,62 @@ def test_attention_decode_flat_fused(hip, cpu, hip_ops, cpu_ops, interleaved, b,
     got, want = run(hip, hip_ops), run(cpu, cpu_ops)
     scale_abs = float(np.abs(want).max())
     np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-5 * scale_abs)
+
+
+# ---- safetensors: upload in the stored dtype, convert on the device ----------------------------------------------------
+@pytest.mark.parametrize("dst", ["BF16", "F16", "F32", "I32", "I64"])
+@pytest.mark.parametrize("src", ["BF16", "F16", "F32", "I32", "I64"])
+def test_load_with_cast_converts_on_the_device(hip, tmp_path, src, dst):
+    import st_files
+    import test_safetensors_cpu as ref
+    n = 100003                                   # not a multiple of 4: exercises the scalar tail
+    x = np.tile(ref.sample_values(1000), 101)[:n]
+    raw = ref.raw_of(x, src)
+    path = str(tmp_path / "t.safetensors")
+    st_files.write_safetensors(path, [("pad", "U8", (3,), np.zeros(3, np.uint8)), ("t", src, (n,), raw)], pad_header_to=1)   # unaligned data
+    st = ug_amd.Safetensors(path)
+    if dst == "I64" and src in ("BF16", "F16"):
+        with pytest.raises(ug_amd.UgError, match="dtype mismatch"):
+            st.load("t", hip, ref.DT[dst])
+        return
+    lb = st.load("t", hip, ref.DT[dst])
+    assert lb.dtype == ref.DT[dst]
+    assert st.last_cast_on_device == (src != dst)
+    got, want = lb.data_vec(), ref.expected(raw, src, dst)
+    if dst in ("F32", "F16"):
+        g = got.view(np.uint32 if dst == "F32" else np.uint16)
+        w = want.astype(np.float32).view(np.uint32) if dst == "F32" else ref.bits(want)
+        nan = np.isnan(got.astype(np.float32))
+        np.testing.assert_array_equal(nan, np.isnan(want.astype(np.float32)))
+        np.testing.assert_array_equal(g[~nan], w[~nan])
+    else:
+        np.testing.assert_array_equal(got, want)
+
+
+def test_llama_from_a_bf16_checkpoint_on_the_device(hip, cpu, hip_ops, cpu_ops, tmp_path):
+    """Config-5 width, 2 layers: a bf16 safetensors checkpoint is uploaded as bf16, widened by
+    ughip_convert, and generates the ids of the CPU oracle running on host-converted weights."""
+    import ctypes as C
+    import st_files
+    cfg = ug_amd.LlamaConfig(num_hidden_layers=2, max_position_embeddings=256)
+    h, isz, kv = cfg.hidden_size, cfg.intermediate_size, cfg.head_dim * cfg.num_key_value_heads
+    shapes = {"model.embed_tokens.weight": (cfg.vocab_size, h), "model.norm.weight": (h,)}
+    for i in range(cfg.num_hidden_layers):
+        p = f"model.layers.{i}"
+        shapes.update({p + ".input_layernorm.weight": (h,), p + ".post_attention_layernorm.weight": (h,), p + ".mlp.gate_proj.weight": (isz, h),
+                       p + ".mlp.up_proj.weight": (isz, h), p + ".mlp.down_proj.weight": (h, isz), p + ".self_attn.q_proj.weight": (h, h),
+                       p + ".self_attn.k_proj.weight": (kv, h), p + ".self_attn.v_proj.weight": (kv, h), p + ".self_attn.o_proj.weight": (h, h)})
+    tensors = []
+    for name, shape in shapes.items():
+        n = int(np.prod(shape))
+        w = np.zeros(n, np.float32)
+        assert ug_amd.host_lib().ugh_synthetic_weights(C.c_uint64(9), C.c_float(0.02), 0, name.encode(), C.c_size_t(n), w.ctypes.data_as(C.c_void_p)) == 0
+        tensors.append((name, "BF16", shape, rng.to_bf16_bits(w)))
+    path = str(tmp_path / "llama_2l_bf16.safetensors")
+    st_files.write_safetensors(path, tensors)
+    prompt = rng.token_ids(10, 16, cfg.vocab_size)
+    ids_h, st_h = ug_amd.LlamaModel.from_safetensors(hip, hip_ops, cfg, path, custom_softmax=True).generate(prompt, 6)
+    ids_c, st_c = ug_amd.LlamaModel.from_safetensors(cpu, cpu_ops, cfg, path, custom_softmax=True).generate(prompt, 6)
+    ids_s, _ = ug_amd.LlamaModel(cpu, cpu_ops, cfg, True, seed=9, std=0.02, round_bf16=True).generate(prompt, 6)
+    assert ids_h.tolist() == ids_c.tolist() == ids_s.tolist()
+    np.testing.assert_allclose(st_h["margins"], st_c["margins"], rtol=1e-2, atol=1e-7)

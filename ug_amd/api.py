@@ -693,6 +693,41 @@ class _Llama:
 llama = _Llama()
 
 
+class Safetensors(_Handle):
+    """Memory-mapped safetensors file(s): ug-core/src/safetensors.rs (MmapedSafetensors)."""
+    _free = "ugh_safetensors_free"
+
+    def __init__(self, paths):
+        if isinstance(paths, (str, bytes, os.PathLike)):
+            paths = [paths]
+        arr = (C.c_char_p * len(paths))(*[os.fsencode(p) for p in paths])
+        out = C.c_void_p()
+        _chk(host_lib().ugh_safetensors_open(arr, C.c_size_t(len(paths)), C.byref(out)))
+        super().__init__(out.value)
+        self.last_cast_on_device = False
+
+    def tensors(self):
+        """[(name, dtype string, shape, nbytes)] in file order."""
+        lib = host_lib()
+        lib.ugh_safetensors_count.restype = C.c_size_t
+        out = []
+        for i in range(lib.ugh_safetensors_count(_p(self.h))):
+            name, dt = C.create_string_buffer(1024), C.create_string_buffer(32)
+            rank, nbytes, dims = C.c_size_t(), C.c_size_t(), (C.c_size_t * 8)()
+            _chk(lib.ugh_safetensors_entry(_p(self.h), C.c_size_t(i), name, C.c_size_t(1024), dt, C.c_size_t(32), C.byref(rank), dims, C.byref(nbytes)))
+            out.append((name.value.decode(), dt.value.decode(), tuple(dims[: rank.value]), nbytes.value))
+        return out
+
+    def load(self, name, device, dtype=None):
+        """`load` (stored dtype) or, with dtype, `load_with_cast`."""
+        out, on_dev = C.c_void_p(), C.c_int()
+        _chk(host_lib().ugh_safetensors_load(_p(self.h), name.encode(), _p(device.h), -1 if dtype is None else int(dtype), C.byref(out), C.byref(on_dev)))
+        self.last_cast_on_device = bool(on_dev.value)
+        lb = LazyBuffer(out.value, device)
+        lb._keep = [self]
+        return lb
+
+
 class LlamaModel(_Handle):
     """ug_llama::Model with random-init weights N(0, std) from the seeded generator."""
     _free = "ugh_llama_model_free"
@@ -706,6 +741,22 @@ class LlamaModel(_Handle):
             _chk(host_lib().ugh_llama_model_set_fused_attention(_p(self.h), 1))
         self._keep = [device, ops]
         self.cfg = cfg
+
+    @classmethod
+    def from_safetensors(cls, device, ops, cfg, paths, custom_softmax=False, fused_attention=False):
+        """Weights by their HF names from safetensors file(s), cast to f32 (model.rs:299-346)."""
+        if isinstance(paths, (str, bytes, os.PathLike)):
+            paths = [paths]
+        arr = (C.c_char_p * len(paths))(*[os.fsencode(p) for p in paths])
+        out = C.c_void_p()
+        _chk(host_lib().ugh_llama_model_from_safetensors(_p(device.h), _p(ops.h), C.byref(cfg), int(custom_softmax), arr, C.c_size_t(len(paths)), C.byref(out)))
+        self = cls.__new__(cls)
+        _Handle.__init__(self, out.value)
+        self._keep = [device, ops]
+        self.cfg = cfg
+        if fused_attention:
+            _chk(host_lib().ugh_llama_model_set_fused_attention(_p(self.h), 1))
+        return self
 
     def generate(self, prompt, n_steps):
         """Prefill over `prompt`, then n_steps greedy single-token steps.  Returns

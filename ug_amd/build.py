@@ -35,14 +35,14 @@ def _run(cmd):
 def build_ughip():
     os.makedirs(LIB, exist_ok=True)
     src = os.path.join(CSRC, "ughip")
-    files = [os.path.join(src, f) for f in ("runtime.cpp", "lower_hip.cpp", "llama_ops.hip", "matmul.hip", "gemm_tiled.hip", "attention.hip")]
+    files = [os.path.join(src, f) for f in ("runtime.cpp", "lower_hip.cpp", "llama_ops.hip", "matmul.hip", "gemm_tiled.hip", "attention.hip", "convert.hip")]
     _run([os.path.join(ROCM, "bin", "hipcc")] + HIP_FLAGS + ["-shared", "-I" + INC, "-I" + src] + files +
          ["-L" + os.path.join(ROCM, "lib"), "-lhiprtc", "-Wl,-rpath," + os.path.join(ROCM, "lib"), "-o", os.path.join(LIB, "libughip.so")])
 
 
 def build_host():
     src = os.path.join(CSRC, "host")
-    files = [os.path.join(src, f) for f in ("ug/lower_op.cpp", "ug/lazy_buffer.cpp", "ug/schedule.cpp", "hip_device.cpp", "llama.cpp", "capi.cpp")]
+    files = [os.path.join(src, f) for f in ("ug/lower_op.cpp", "ug/lazy_buffer.cpp", "ug/schedule.cpp", "ug/safetensors.cpp", "hip_device.cpp", "llama.cpp", "capi.cpp")]
     _run(["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-I" + INC, "-I" + src] + files +
          ["-L" + LIB, "-lughip", "-Wl,-rpath,$ORIGIN", "-lpthread", "-o", os.path.join(LIB, "libug_host.so")])
 

@@ -2,6 +2,10 @@
 // Every function returns 0 on success; ugh_last_error() holds the message otherwise.
 #include "capi.h"
 
+#include <cstdio>
+
+#include "ug/safetensors.h"
+
 #include <cstring>
 
 #include "hip_device.h"
@@ -365,6 +369,47 @@ void* ugh_compiled_func_raw_hip(void* c, size_t i) {
   return h ? h->raw() : nullptr;
 }
 
+// ---- safetensors (ug-core/src/safetensors.rs) ---------------------------------------------------------
+int ugh_safetensors_open(const char* const* paths, size_t n_paths, void** out) {
+  return guard([&] {
+    if (n_paths == 0) bail("no safetensors file given");
+    if (n_paths == 1) {
+      *out = new ug::MmapedSafetensors(ug::MmapedSafetensors::open(paths[0]));
+    } else {
+      std::vector<std::string> ps(paths, paths + n_paths);
+      *out = new ug::MmapedSafetensors(ug::MmapedSafetensors::multi(ps));
+    }
+  });
+}
+void ugh_safetensors_free(void* h) { delete static_cast<ug::MmapedSafetensors*>(h); }
+size_t ugh_safetensors_count(void* h) { return static_cast<ug::MmapedSafetensors*>(h)->tensors().size(); }
+// Entry i in file/header order: name and dtype as NUL-terminated strings, up to 8 dims.
+int ugh_safetensors_entry(void* h, size_t i, char* name, size_t name_cap, char* dtype, size_t dtype_cap, size_t* rank, size_t* dims, size_t* nbytes) {
+  return guard([&] {
+    auto ts = static_cast<ug::MmapedSafetensors*>(h)->tensors();
+    if (i >= ts.size()) bail("entry index out of range");
+    snprintf(name, name_cap, "%s", ts[i].first.c_str());
+    snprintf(dtype, dtype_cap, "%s", ts[i].second.dtype.c_str());
+    if (ts[i].second.shape.size() > 8) bail("more than 8 dims");
+    *rank = ts[i].second.shape.size();
+    for (size_t k = 0; k < ts[i].second.shape.size(); ++k) dims[k] = ts[i].second.shape[k];
+    *nbytes = ts[i].second.nbytes;
+  });
+}
+// cast_dtype < 0: load in the stored dtype (safetensors.rs:71-74), else load_with_cast (:76-84).
+int ugh_safetensors_load(void* h, const char* name, void* device, int cast_dtype, void** out_lb, int* cast_on_device) {
+  return guard([&] {
+    auto& st = *static_cast<ug::MmapedSafetensors*>(h);
+    if (cast_dtype < 0) {
+      *out_lb = box(st.load(name, dev_of(device)));
+      if (cast_on_device) *cast_on_device = 0;
+    } else {
+      *out_lb = box(st.load_with_cast(name, (DType)cast_dtype, dev_of(device)));
+      if (cast_on_device) *cast_on_device = st.last_cast_on_device() ? 1 : 0;
+    }
+  });
+}
+
 // ---- ug-llama ---------------------------------------------------------------------------------------------
 using OpsPtr = std::shared_ptr<ug_llama::Ops>;
 int ugh_llama_ops_hip(void** out) {
@@ -447,6 +492,13 @@ int ugh_llama_rope_tables(void* d, const ugh_llama_config* c, void** cos, void**
 int ugh_llama_model_new(void* d, void* ops, const ugh_llama_config* c, int custom_softmax, uint64_t seed, float std, int round_bf16, void** out) {
   return guard([&] {
     auto w = ug_llama::synthetic_weights(seed, std, round_bf16 != 0);
+    *out = new ug_llama::Model(cfg_of(c), custom_softmax != 0, *w, dev_of(d), *static_cast<OpsPtr*>(ops));
+  });
+}
+int ugh_llama_model_from_safetensors(void* d, void* ops, const ugh_llama_config* c, int custom_softmax, const char* const* paths, size_t n_paths, void** out) {
+  return guard([&] {
+    std::vector<std::string> ps(paths, paths + n_paths);
+    auto w = ug_llama::safetensors_weights(ps);
     *out = new ug_llama::Model(cfg_of(c), custom_softmax != 0, *w, dev_of(d), *static_cast<OpsPtr*>(ops));
   });
 }

@@ -65,6 +65,11 @@ void HipDevice::matmul(Slice& dst, const Slice& lhs, const Slice& rhs, size_t b,
     fail("matmul");
 }
 
+bool HipDevice::convert(Slice& dst, const Slice& src) {
+  if (ughip_convert(d_, raw_slice(src), raw_slice(dst))) fail("convert");
+  return true;
+}
+
 ughip_slice* hip_raw_slice(const Slice& s) { return raw_slice(s); }
 
 }  // namespace ug

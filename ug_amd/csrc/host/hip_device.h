@@ -41,6 +41,7 @@ class HipDevice : public Device {
   // The backend re-parallelises serial loop nests itself (ug-core/src/schedule.rs:162).
   bool use_grid() const override { return false; }
   bool runs_async() const override { return true; }
+  bool convert(Slice& dst, const Slice& src) override;
   const char* name() const override { return "hip"; }
   ughip_device* raw() const { return d_; }
 

@@ -9,6 +9,7 @@
 #include "hip_device.h"
 #include "rng.h"
 #include "ug/block.h"
+#include "ug/safetensors.h"
 
 namespace ug_llama {
 
@@ -236,6 +237,49 @@ std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool r
   return std::make_shared<SyntheticWeights>(seed, std, round_bf16);
 }
 
+LB WeightSource::load(const std::string& name, const std::vector<size_t>& shape, const DevicePtr& dev) {
+  std::vector<float> v = get(name, shape);
+  size_t n = 1;
+  for (size_t d : shape) n *= d;
+  if (v.size() != n) bail("unexpected shape for " + name);
+  return LB::copy(v.data(), DType::F32, v.size(), Shape(shape), dev);
+}
+
+namespace {
+struct SafetensorsWeights : WeightSource {
+  ug::MmapedSafetensors st;
+  explicit SafetensorsWeights(const std::vector<std::string>& paths)
+      : st(paths.size() == 1 ? ug::MmapedSafetensors::open(paths[0]) : ug::MmapedSafetensors::multi(paths)) {}
+  void check_shape(const std::string& name, const std::vector<size_t>& got, const std::vector<size_t>& want) {
+    if (got != want) bail("unexpected shape for " + name + ": " + Shape(got).str() + ", expected " + Shape(want).str());
+  }
+  std::vector<float> get(const std::string& name, const std::vector<size_t>& shape) override {
+    ug::TensorView v = st.get(name);
+    check_shape(name, v.shape, shape);
+    size_t n = Shape(v.shape).num_elements();
+    std::vector<float> out(n);
+    DType src = DType::F32;
+    if (v.dtype == "BF16") src = DType::BF16;
+    else if (v.dtype == "F16") src = DType::F16;
+    else if (v.dtype == "I32") src = DType::I32;
+    else if (v.dtype == "I64") src = DType::I64;
+    else if (v.dtype != "F32") bail("unsupported dtype for " + name + ": " + v.dtype);
+    ug::convert_on_host(v.data, src, out.data(), DType::F32, n, name);
+    return out;
+  }
+  LB load(const std::string& name, const std::vector<size_t>& shape, const DevicePtr& dev) override {
+    LB lb = st.load_with_cast(name, DType::F32, dev);
+    check_shape(name, lb.dims(), shape);
+    return lb;
+  }
+};
+}  // namespace
+
+std::shared_ptr<WeightSource> safetensors_weights(const std::vector<std::string>& paths) {
+  if (paths.empty()) bail("no safetensors file given");
+  return std::make_shared<SafetensorsWeights>(paths);
+}
+
 // ---- graph builders (model.rs:32-109) --------------------------------------------------------------------
 // model.rs:32-63: hand-written SSA; the ids load is typed F32 although the buffer holds I32,
 // so the row offset is (int)((float)id * h).
@@ -328,13 +372,7 @@ std::vector<Cache> Cache::create(const Config& cfg, const DevicePtr& dev) {
 
 // ---- model (model.rs:299-373) --------------------------------------------------------------------------------
 namespace {
-LB load_w(WeightSource& w, const std::string& name, const std::vector<size_t>& shape, const DevicePtr& dev) {
-  std::vector<float> v = w.get(name, shape);
-  size_t n = 1;
-  for (size_t d : shape) n *= d;
-  if (v.size() != n) bail("unexpected shape for " + name);
-  return LB::copy(v.data(), DType::F32, v.size(), Shape(shape), dev);
-}
+LB load_w(WeightSource& w, const std::string& name, const std::vector<size_t>& shape, const DevicePtr& dev) { return w.load(name, shape, dev); }
 }  // namespace
 
 Model::Model(const Config& cfg, bool custom_softmax, WeightSource& w, const DevicePtr& dev, std::shared_ptr<Ops> ops)

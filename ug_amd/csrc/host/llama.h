@@ -60,11 +60,17 @@ struct Config {
 struct WeightSource {
   virtual ~WeightSource() = default;
   virtual std::vector<float> get(const std::string& name, const std::vector<size_t>& shape) = 0;
+  // The tensor as an f32 buffer on `dev`; the default uploads what get() returns.
+  virtual LB load(const std::string& name, const std::vector<size_t>& shape, const ug::DevicePtr& dev);
 };
 
 // Random-init weights: N(0, std) from a counter-based generator keyed by (seed, tensor name),
 // optionally rounded to bf16 (round-to-nearest-even) and widened back.
 std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16);
+
+// Weights from safetensors files, any stored dtype, delivered as f32 (model.rs:118,140,313:
+// `load_with_cast(name, DType::F32, device)`); conversion happens on the device when it can.
+std::shared_ptr<WeightSource> safetensors_weights(const std::vector<std::string>& paths);
 
 // Graph builders of model.rs:32-109, usable on their own.
 LB index_select(const LB& src, const LB& ids);

@@ -40,6 +40,13 @@ struct Device {
   virtual const char* name() const = 0;
   // True when run/matmul only queue work (results are ready after synchronize or a copy back).
   virtual bool runs_async() const { return false; }
+  // Element type conversion between two slices of equal length, if the device can do it in its
+  // own memory; false = not offered (the caller converts on the host).
+  virtual bool convert(Slice& dst, const Slice& src) {
+    (void)dst;
+    (void)src;
+    return false;
+  }
 };
 
 }  // namespace ug
