@@ -111,6 +111,44 @@ def extras(dev, steps, warmup, only=None):
         out.update(bmm(dev, steps, warmup))
     if only in (None, "llama_pieces"):
         out.update(llama_pieces(dev, steps, warmup))
+    if only in (None, "safetensors"):
+        out.update(safetensors_load(dev))
+    return out
+
+
+def safetensors_load(dev, n=1 << 27):
+    """A 256 MiB bf16 tensor in a safetensors file (page cache warm) loaded as f32: upload + widen
+    on the device against widen on the host + upload (the order of ug-core/src/safetensors.rs:141-271),
+    and the widening kernel alone (6 bytes per element)."""
+    import tempfile
+    import st_files
+    import ug_amd
+    from ug_amd import rng
+    out = {}
+    bits = np.tile(rng.to_bf16_bits(rng.normal(11, 1 << 20)), n >> 20)
+    with tempfile.TemporaryDirectory() as tmp:
+        path = os.path.join(tmp, "w.safetensors")
+        st_files.write_safetensors(path, [("w", "BF16", (n,), bits)])
+        st = ug_amd.Safetensors(path)
+        for key, env in (("device_cast", None), ("host_cast", "1")):
+            if env:
+                os.environ["UG_SAFETENSORS_HOST_CAST"] = env
+            try:
+                st.load("w", dev, ug_amd.F32).data_vec()[:1]      # first touch: page in, warm the pool
+                dev.synchronize()
+                t0 = time.perf_counter()
+                lb = st.load("w", dev, ug_amd.F32)
+                dev.synchronize()
+                dt = time.perf_counter() - t0
+            finally:
+                os.environ.pop("UG_SAFETENSORS_HOST_CAST", None)
+            out[f"safetensors_bf16_to_f32_{key}"] = {"file_GB/s": round(2.0 * n / dt / 1e9, 2), "ms": round(dt * 1e3, 1), "on_device": st.last_cast_on_device}
+            del lb
+    src = dev.slice_from(bits)
+    dst = dev.allocate_uninit(ug_amd.F32, n)
+    _, ms = timed(dev, lambda: dev.convert(dst, src), 20, 3)
+    gbs = 6.0 * n * 20 / (ms * 1e-3) / 1e9
+    out["convert_bf16_to_f32_2pow27"] = {"GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "us": round(ms * 1e3 / 20, 1), "algorithmic_bytes": 6 * n}
     return out
 
 
@@ -248,7 +286,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-llama", action="store_true")
     ap.add_argument("--headline-only", action="store_true", help="only the config-2 kernel: no extras, no llama, no CPU baseline")
-    ap.add_argument("--only", choices=["softmax", "bmm", "llama_pieces", "llama"], help="besides the headline, run just this group (profiler runs)")
+    ap.add_argument("--only", choices=["softmax", "bmm", "llama_pieces", "safetensors", "llama"], help="besides the headline, run just this group (profiler runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true", help="also run a plain 2^24-element copy kernel (counter calibration)")
     args = ap.parse_args()

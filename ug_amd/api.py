@@ -303,6 +303,12 @@ class Device(_Handle):
                                           C.c_size_t(k), C.c_size_t(rank), sz(*lhs_l[0]), sz(*lhs_l[1]), C.c_size_t(lhs_l[2]),
                                           sz(*rhs_l[0]), sz(*rhs_l[1]), C.c_size_t(rhs_l[2])))
 
+    def convert(self, dst, src):
+        """Element type conversion between two slices in device memory; False if the device has none."""
+        done = C.c_int()
+        _chk(host_lib().ugh_device_convert(_p(self.h), _p(dst.h), _p(src.h), C.byref(done)))
+        return bool(done.value)
+
     def set_zero_fill(self, on):
         """HIP device only: zero-fill fresh allocations (default, like ug's CpuDevice) or not (like ug-cuda)."""
         _chk(host_lib().ugh_hip_device_set_zero_fill(_p(self.h), int(on)))

@@ -95,6 +95,10 @@ void* ugh_device_raw_hip(void* d) {
 int ugh_device_alloc(void* d, int dtype, size_t len, void** out) {
   return guard([&] { *out = dev_of(d)->allocate_uninit((DType)dtype, len).release(); });
 }
+// Device::convert: *done = 0 when the device does not offer it.
+int ugh_device_convert(void* d, void* dst, void* src, int* done) {
+  return guard([&] { *done = dev_of(d)->convert(*static_cast<Slice*>(dst), *static_cast<Slice*>(src)) ? 1 : 0; });
+}
 void ugh_slice_free(void* s) { delete static_cast<Slice*>(s); }
 size_t ugh_slice_len(void* s) { return static_cast<Slice*>(s)->len(); }
 int ugh_slice_dtype(void* s) { return (int)static_cast<Slice*>(s)->dtype(); }

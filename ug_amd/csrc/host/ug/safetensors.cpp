@@ -8,6 +8,7 @@
 #include <cmath>
 #include <algorithm>
 #include <cerrno>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 
@@ -347,7 +348,8 @@ std::pair<Shape, std::unique_ptr<Slice>> MmapedSafetensors::load_slice_with_cast
   std::unique_ptr<Slice> dst = dev->allocate_uninit(dst_dtype, n);
   last_cast_on_device_ = false;
   if (n == 0) return {shape, std::move(dst)};
-  {
+  // UG_SAFETENSORS_HOST_CAST=1 forces the reference's order (convert on the host, then upload).
+  if (!getenv("UG_SAFETENSORS_HOST_CAST")) {
     std::unique_ptr<Slice> staged = dev->allocate_uninit(src_dtype, n);
     staged->copy_host_to_device(v.data, src_dtype, n);
     if (dev->convert(*dst, *staged)) {
