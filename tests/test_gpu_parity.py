@@ -378,6 +378,36 @@ def test_gemv_rhs_kn_f32(hip, bmnk):
     np.testing.assert_array_equal(_raw_matmul(hip, F32, ai, wi, False), (ai.astype(np.float64) @ wi.astype(np.float64)).astype(np.float32))
 
 
+# Skinny products with a long K (the projections of a 128-token prefill) split K over several
+# workgroups per output tile and add the partial tiles in slab order.
+@pytest.mark.parametrize("dtype_name", ["f32", "bf16"])
+@pytest.mark.parametrize("rhs_nk", [False, True])
+@pytest.mark.parametrize("bmnk", [(1, 128, 2048, 2048), (1, 128, 256, 2048), (1, 128, 128, 2112), (2, 128, 128, 1024), (1, 256, 128, 4096), (1, 128, 2048, 5632)])
+def test_matmul_split_k(hip, bmnk, rhs_nk, dtype_name):
+    b, m, n, k = bmnk
+    print("matmul split-k", dtype_name, bmnk, "rhs_nk", rhs_nk, flush=True)
+    a = rng.uniform_pm1(25, b * m * k).reshape(b, m, k)
+    w = rng.uniform_pm1(26, b * k * n).reshape(b, k, n)
+    absprod_bound = None
+    if dtype_name == "f32":
+        got = _raw_matmul(hip, F32, a, w, rhs_nk)
+        exact = a.astype(np.float64) @ w.astype(np.float64)
+        bound = k * np.finfo(np.float32).eps * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64))
+    else:
+        a, w = rng.bf16_round(a.ravel()).reshape(a.shape), rng.bf16_round(w.ravel()).reshape(w.shape)
+        got = _raw_matmul(hip, ug_amd.BF16, a, w, rhs_nk)
+        exact = a.astype(np.float64) @ w.astype(np.float64)
+        bound = (2.0 ** -8) * np.abs(exact) + k * np.finfo(np.float32).eps * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64))
+    assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-12)
+    # exact on small integers, whatever the split
+    ai, wi = np.floor(a * 4), np.floor(w * 4)
+    want = (ai.astype(np.float64) @ wi.astype(np.float64)).astype(np.float32)
+    if dtype_name == "f32":
+        np.testing.assert_array_equal(_raw_matmul(hip, F32, ai, wi, rhs_nk), want)
+    else:
+        np.testing.assert_array_equal(_raw_matmul(hip, ug_amd.BF16, ai, wi, rhs_nk), rng.bf16_round(want.ravel()).reshape(want.shape))
+
+
 def test_matmul_tiled_matches_generic_on_integers(hip):
     """Small-integer operands make every partial sum exact in f32, so the tuned kernel, the generic
     kernel (reached through a shape one column short) and numpy must agree bit for bit."""

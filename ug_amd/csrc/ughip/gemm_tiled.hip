@@ -16,6 +16,7 @@
 //       fragment feed 4 consecutive MFMAs, lanes 0-31 holding k..k+3 and lanes 32-63 k+4..k+7.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdlib>
 
 #include "gemm.h"
@@ -194,8 +195,13 @@ __device__ __forceinline__ void k_phase(const T* __restrict__ A, const T* __rest
 // NT threads = NT / 64 waves laid out (NT / 128) x 2 over the tile: 4 waves give each wave a
 // (BM/2) x (BN/2) block; 8 waves halve the rows per wave and put two waves on every SIMD, so that
 // one can feed the matrix pipe while the other is blocked on the LDS or load queues.
-template <typename T, bool B_NK, int BM, int BN, int NT>
-__global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p, int tiles_m, int tiles_n, int remap) {
+//
+// SPLIT: the K tiles are dealt to `nsplit` workgroups per output tile (slab s takes tiles
+// [s * kt_per, (s + 1) * kt_per)), each writes its f32 partial tile to ws[s][batch][m][n], and
+// gemm_split_reduce adds the slabs in index order.  For skinny products (few output tiles, long K:
+// the projections of a 128-token prefill) this is what puts every CU to work.
+template <typename T, bool B_NK, int BM, int BN, int NT, bool SPLIT>
+__global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p, int tiles_m, int tiles_n, int remap, int nsplit, int kt_per, float* __restrict__ ws) {
   extern __shared__ u32x4 lds[];
   constexpr int BK = Elt<T>::BK;
   constexpr int WM = BM / (NT / 128), WN = BN / 2, MI = WM / 32, NJ = WN / 32;
@@ -203,14 +209,21 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p, int tiles_m, int tile
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int bid = blockIdx.x;
   if (remap) bid = (bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3);
+  int slab = 0;
+  if (SPLIT) {
+    slab = bid % nsplit;  // the slabs of one tile sit next to each other: they share the A and B rows
+    bid /= nsplit;
+  }
   const int tpb = tiles_m * tiles_n;
   const int batch = bid / tpb;
   const int t_in = bid - batch * tpb;
   const int m0 = (t_in / tiles_n) * BM, n0 = (t_in % tiles_n) * BN;
-  const T* __restrict__ A = static_cast<const T*>(p.a) + (size_t)batch * p.a_bs + (size_t)m0 * p.a_rs;
-  const T* __restrict__ B = static_cast<const T*>(p.b) + (size_t)batch * p.b_bs + (B_NK ? (size_t)n0 * p.b_cs : (size_t)n0);
-  T* __restrict__ C = static_cast<T*>(p.c) + (size_t)batch * p.c_bs + (size_t)m0 * p.N + n0;
-  const int KT = p.K / BK;
+  const int kt0 = SPLIT ? slab * kt_per : 0;
+  const size_t k_off = (size_t)kt0 * BK;
+  const T* __restrict__ A = static_cast<const T*>(p.a) + (size_t)batch * p.a_bs + (size_t)m0 * p.a_rs + k_off;
+  const T* __restrict__ B =
+      static_cast<const T*>(p.b) + (size_t)batch * p.b_bs + (B_NK ? (size_t)n0 * p.b_cs + k_off : (size_t)n0 + k_off * (size_t)p.b_rs);
+  const int KT = SPLIT ? min(kt_per, p.K / BK - kt0) : p.K / BK;
   const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
 
   floatx16 acc[MI][NJ];
@@ -242,39 +255,77 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p, int tiles_m, int tile
   if (kt < KT) k_phase<T, B_NK, BM, BN, NT, MI, NJ, false>(A, B, p, lds0, lds1, false, r1, 0, r0, tid, lane, wm, wn, acc);  // odd tile count: the last tile
 
   // accumulator register r of lane l: row (r/4)*8 + (l/32)*4 + r%4, column l%32
+  if (SPLIT) {
+    float* __restrict__ W = ws + ((size_t)slab * (gridDim.x / (nsplit * tpb)) + batch) * (size_t)p.M * p.N + (size_t)m0 * p.N + n0;
 #pragma unroll
-  for (int i = 0; i < MI; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      T* Ct = C + (size_t)(wm + i * 32 + (lane >> 5) * 4) * p.N + wn + j * 32 + (lane & 31);
+      for (int j = 0; j < NJ; ++j) {
+        float* Wt = W + (size_t)(wm + i * 32 + (lane >> 5) * 4) * p.N + wn + j * 32 + (lane & 31);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) Ct[(size_t)((r >> 2) * 8 + (r & 3)) * p.N] = (T)acc[i][j][r];
-    }
+        for (int r = 0; r < 16; ++r) Wt[(size_t)((r >> 2) * 8 + (r & 3)) * p.N] = acc[i][j][r];
+      }
+  } else {
+    T* __restrict__ C = static_cast<T*>(p.c) + (size_t)batch * p.c_bs + (size_t)m0 * p.N + n0;
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        T* Ct = C + (size_t)(wm + i * 32 + (lane >> 5) * 4) * p.N + wn + j * 32 + (lane & 31);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) Ct[(size_t)((r >> 2) * 8 + (r & 3)) * p.N] = (T)acc[i][j][r];
+      }
+  }
 }
 
-template <typename T, bool B_NK, int BM, int BN, int NT>
-hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch) {
+// c[i] = (T)(ws[0][i] + ws[1][i] + ... in slab order); n4 groups of 4 elements.
+template <typename T>
+__global__ void __launch_bounds__(256) gemm_split_reduce(const float* __restrict__ ws, T* __restrict__ c, size_t n4, size_t slab_elems, int nsplit) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n4) return;
+  f32x4 s = reinterpret_cast<const f32x4*>(ws)[g];
+  for (int k = 1; k < nsplit; ++k) s += reinterpret_cast<const f32x4*>(ws + (size_t)k * slab_elems)[g];
+  T* o = c + g * 4;
+  o[0] = (T)s.x;
+  o[1] = (T)s.y;
+  o[2] = (T)s.z;
+  o[3] = (T)s.w;
+}
+
+template <typename T, bool B_NK, int BM, int BN, int NT, bool SPLIT>
+hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch, int nsplit, float* ws) {
   constexpr int LDS_BYTES = 2 * (BM + BN) * CHUNKS * 16;
+  constexpr int BK = Elt<T>::BK;
   static bool configured = false;
-  auto kernel = gemm_tiled<T, B_NK, BM, BN, NT>;
+  auto kernel = gemm_tiled<T, B_NK, BM, BN, NT, SPLIT>;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if (e != hipSuccess) return e;
     configured = true;
   }
   const int tiles_m = p.M / BM, tiles_n = p.N / BN;
-  const size_t total = batch * (size_t)tiles_m * tiles_n;
-  const int remap = total % 8 == 0 ? 1 : 0;
-  kernel<<<dim3((unsigned)total), dim3(NT), LDS_BYTES, stream>>>(p, tiles_m, tiles_n, remap);
-  return hipGetLastError();
+  const int kt = p.K / BK, kt_per = SPLIT ? (kt + nsplit - 1) / nsplit : kt;
+  if (SPLIT) nsplit = (kt + kt_per - 1) / kt_per;  // no empty slab
+  const size_t total = batch * (size_t)tiles_m * tiles_n * (SPLIT ? nsplit : 1);
+  const int remap = !SPLIT && total % 8 == 0 ? 1 : 0;
+  kernel<<<dim3((unsigned)total), dim3(NT), LDS_BYTES, stream>>>(p, tiles_m, tiles_n, remap, nsplit, kt_per, ws);
+  if (hipError_t e = hipGetLastError()) return e;
+  if (SPLIT) {
+    const size_t elems = batch * (size_t)p.M * p.N;  // contiguous [batch, M, N] result: c_bs == M * N
+    gemm_split_reduce<T><<<dim3((unsigned)((elems / 4 + 255) / 256)), dim3(256), 0, stream>>>(ws, static_cast<T*>(p.c), elems / 4, elems, nsplit);
+    return hipGetLastError();
+  }
+  return hipSuccess;
 }
 
-template <typename T, bool B_NK>
-hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int shape) {
+template <typename T, bool B_NK, bool SPLIT>
+hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int shape, int nsplit, float* ws) {
   switch (shape) {
-    case 0: return getenv("UGHIP_GEMM_4WAVES") ? launch<T, B_NK, 256, 128, 256>(stream, p, batch) : launch<T, B_NK, 256, 128, 512>(stream, p, batch);
-    case 1: return launch<T, B_NK, 128, 128, 256>(stream, p, batch);
-    default: return launch<T, B_NK, 128, 64, 256>(stream, p, batch);
+    case 0:
+      return getenv("UGHIP_GEMM_4WAVES") ? launch<T, B_NK, 256, 128, 256, SPLIT>(stream, p, batch, nsplit, ws)
+                                         : launch<T, B_NK, 256, 128, 512, SPLIT>(stream, p, batch, nsplit, ws);
+    case 1: return launch<T, B_NK, 128, 128, 256, SPLIT>(stream, p, batch, nsplit, ws);
+    default: return launch<T, B_NK, 128, 64, 256, SPLIT>(stream, p, batch, nsplit, ws);
   }
 }
 
@@ -301,6 +352,19 @@ int pick_shape(const MMArgs& p, size_t batch) {
   return best;
 }
 
+// How many K slabs per output tile: only when the tiles alone leave most CUs idle and K is long
+// enough that every slab still has a few tiles to pipeline.
+int pick_split(int dtype, const MMArgs& p, size_t batch, int shape) {
+  if (const char* e = getenv("UGHIP_GEMM_SPLIT")) return std::max(1, atoi(e));  // tuning aid
+  const int bk = dtype == UGHIP_F32 ? 32 : 64;
+  const size_t tiles = batch * (size_t)(p.M / kShapes[shape][0]) * (size_t)(p.N / kShapes[shape][1]);
+  const int kt = p.K / bk;
+  if (tiles >= 128 || kt < 8) return 1;
+  int want = (int)((256 + tiles - 1) / tiles);
+  want = std::min(want, kt / 4);  // at least 4 K tiles per slab
+  return std::max(1, std::min(want, 32));
+}
+
 }  // namespace
 
 bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch) {
@@ -315,15 +379,30 @@ bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch) {
   if (!aligned16(p.a) || !aligned16(p.b) || !aligned16(p.c)) return false;
   const int s = pick_shape(p, batch);
   if (s < 0) return false;
-  return batch * (size_t)(p.M / kShapes[s][0]) * (size_t)(p.N / kShapes[s][1]) < (1u << 30);
+  return batch * (size_t)(p.M / kShapes[s][0]) * (size_t)(p.N / kShapes[s][1]) < (1u << 24);
 }
 
-hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch) {
+size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch) {
+  const int s = pick_shape(p, batch);
+  if (s < 0) return 0;
+  const int nsplit = pick_split(dtype, p, batch, s);
+  return nsplit > 1 ? (size_t)nsplit * batch * (size_t)p.M * p.N * sizeof(float) : 0;
+}
+
+hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, float* workspace) {
   const bool nt = p.b_rs == 1 && p.b_cs != 1;
   const int s = pick_shape(p, batch);
   if (s < 0) return hipErrorInvalidValue;
-  if (dtype == UGHIP_F32) return nt ? launch_shape<float, true>(stream, p, batch, s) : launch_shape<float, false>(stream, p, batch, s);
-  return nt ? launch_shape<__bf16, true>(stream, p, batch, s) : launch_shape<__bf16, false>(stream, p, batch, s);
+  const int nsplit = pick_split(dtype, p, batch, s);
+  if (nsplit > 1) {
+    if (!workspace) return hipErrorInvalidValue;
+    if (dtype == UGHIP_F32)
+      return nt ? launch_shape<float, true, true>(stream, p, batch, s, nsplit, workspace) : launch_shape<float, false, true>(stream, p, batch, s, nsplit, workspace);
+    return nt ? launch_shape<__bf16, true, true>(stream, p, batch, s, nsplit, workspace) : launch_shape<__bf16, false, true>(stream, p, batch, s, nsplit, workspace);
+  }
+  if (dtype == UGHIP_F32)
+    return nt ? launch_shape<float, true, false>(stream, p, batch, s, 1, nullptr) : launch_shape<float, false, false>(stream, p, batch, s, 1, nullptr);
+  return nt ? launch_shape<__bf16, true, false>(stream, p, batch, s, 1, nullptr) : launch_shape<__bf16, false, false>(stream, p, batch, s, 1, nullptr);
 }
 
 }  // namespace ughip

@@ -28,6 +28,10 @@ struct ughip_device {
   size_t pool_bytes = 0, live_bytes = 0;
   bool zero_fill = true;
   std::map<std::string, CachedModule> modules;  // generated source -> loaded code object
+  // Scratch of the split-K matmul (partial tiles); grown on demand, reused by every launch of the
+  // device's one stream, freed with the device.
+  void* gemm_ws = nullptr;
+  size_t gemm_ws_bytes = 0;
 };
 
 struct ughip_slice {

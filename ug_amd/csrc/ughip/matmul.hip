@@ -4,7 +4,9 @@
 // ug-core/src/cpu_runtime.rs:527-619).
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdlib>
+#include <mutex>
 
 #include "gemm.h"
 #include "internal.h"
@@ -434,7 +436,18 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
     else if (m <= 4) gemv_nn_f32<4><<<grid, 1024, 0, st>>>(p);
     else gemv_nn_f32<8><<<grid, 1024, 0, st>>>(p);
   } else if (gemm_tiled_supported(dst->dtype, p, b)) {
-    UGHIP_HIPCHK(gemm_tiled_launch(st, dst->dtype, p, b));
+    const size_t ws_bytes = gemm_tiled_workspace_bytes(dst->dtype, p, b);
+    if (ws_bytes > dev->gemm_ws_bytes) {
+      std::lock_guard<std::mutex> g(dev->mu);
+      UGHIP_HIPCHK(hipStreamSynchronize(st));  // earlier launches may still read the old block
+      if (dev->gemm_ws) hipFree(dev->gemm_ws);
+      dev->gemm_ws = nullptr;
+      dev->gemm_ws_bytes = 0;
+      const size_t want = std::max<size_t>(ws_bytes, (size_t)32 << 20);
+      UGHIP_HIPCHK(hipMalloc(&dev->gemm_ws, want));
+      dev->gemm_ws_bytes = want;
+    }
+    UGHIP_HIPCHK(gemm_tiled_launch(st, dst->dtype, p, b, ws_bytes ? static_cast<float*>(dev->gemm_ws) : nullptr));
     return UGHIP_OK;
   } else {
     dim3 grid((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64), (unsigned)b);

@@ -111,6 +111,7 @@ int ughip_device_release(ughip_device* dev) {
   if (dev->refs.fetch_sub(1) != 1) return UGHIP_OK;
   hipSetDevice(dev->ordinal);
   hipStreamSynchronize(dev->stream);
+  if (dev->gemm_ws) hipFree(dev->gemm_ws);
   for (auto& kv : dev->pool)
     for (void* p : kv.second) hipFree(p);
   for (auto& kv : dev->modules) hipModuleUnload(kv.second.module);
