@@ -10,7 +10,8 @@
 //                   exact-copy slices with dtype/len checks (:376-412);
 //   * matmul:       stride rules of cpu_runtime.rs:527-619.  The arithmetic of the reference
 //                   lives in the un-vendored `gemm` 0.18.0 crate; here it is a plain f32
-//                   multiply-accumulate in k order per output element.  PARITY UNPINNED beyond
+//                   multiply-accumulate in k order per output element (F32, and F16 widened to
+//                   f32 with one final rounding).  PARITY UNPINNED beyond
 //                   the reference's own `mm` test (common_tests.rs:15-22): the tests therefore
 //                   also compare against an f64 product with a k*eps bound.
 // Pinned by: the golden vectors of ug-core/tests/{basic_tests,lb_tests,cpu_tests}.rs and
@@ -297,15 +298,29 @@ void CpuDevice::matmul(Slice& dst_s, const Slice& lhs_s, const Slice& rhs_s, siz
   CpuSlice& dst = cpu_slice(dst_s);
   const CpuSlice& lhs = cpu_slice(lhs_s);
   const CpuSlice& rhs = cpu_slice(rhs_s);
-  // cpu_runtime.rs:345-356: F16 and F32 only (F16 is not representable with this gcc -> F32 only here).
-  if (!(dst.dtype() == DType::F32 && lhs.dtype() == DType::F32 && rhs.dtype() == DType::F32))
+  // cpu_runtime.rs:345-356: F16 and F32 only.
+  const bool all_f32 = dst.dtype() == DType::F32 && lhs.dtype() == DType::F32 && rhs.dtype() == DType::F32;
+  const bool all_f16 = dst.dtype() == DType::F16 && lhs.dtype() == DType::F16 && rhs.dtype() == DType::F16;
+  if (!all_f32 && !all_f16)
     bail(std::string("incorrect dtypes for matmul, dst: ") + dtype_str(dst.dtype()) + ", lhs: " + dtype_str(lhs.dtype()) + ", rhs: " +
          dtype_str(rhs.dtype()));
   size_t rank = lhs_l.rank();
   if (rank < 2 || rhs_l.rank() != rank) bail("matmul: unexpected layout ranks");
-  const float* A = reinterpret_cast<const float*>(lhs.data()) + lhs_l.offset();
-  const float* B = reinterpret_cast<const float*>(rhs.data()) + rhs_l.offset();
-  float* C = reinterpret_cast<float*>(dst.data());
+  // F16: operands widened to f32, f32 accumulation in k order, one rounding to f16 at the end
+  // (the arithmetic of the gemm crate's f16 path is unpinned here, like its f32 path).
+  std::vector<float> a32, b32, c32;
+  if (all_f16) {
+    const uint16_t* ha = reinterpret_cast<const uint16_t*>(lhs.data());
+    const uint16_t* hb = reinterpret_cast<const uint16_t*>(rhs.data());
+    a32.resize(lhs.len());
+    b32.resize(rhs.len());
+    for (size_t i = 0; i < lhs.len(); ++i) a32[i] = f16_bits_to_f32(ha[i]);
+    for (size_t i = 0; i < rhs.len(); ++i) b32[i] = f16_bits_to_f32(hb[i]);
+    c32.resize(b * m * n);
+  }
+  const float* A = (all_f16 ? a32.data() : reinterpret_cast<const float*>(lhs.data())) + lhs_l.offset();
+  const float* B = (all_f16 ? b32.data() : reinterpret_cast<const float*>(rhs.data())) + rhs_l.offset();
+  float* C = all_f16 ? c32.data() : reinterpret_cast<float*>(dst.data());
   size_t a_cs = lhs_l.strides()[rank - 1], a_rs = lhs_l.strides()[rank - 2];
   size_t b_cs = rhs_l.strides()[rank - 1], b_rs = rhs_l.strides()[rank - 2];
   size_t a_skip = skip(lhs_l, m * k, "lhs"), b_skip = skip(rhs_l, n * k, "rhs"), c_skip = m * n;
@@ -355,6 +370,10 @@ void CpuDevice::matmul(Slice& dst_s, const Slice& lhs_s, const Slice& rhs_s, siz
       if (t0 < t1) ths.emplace_back(work, t0, t1);
     }
     for (auto& th : ths) th.join();
+  }
+  if (all_f16) {
+    uint16_t* hc = reinterpret_cast<uint16_t*>(dst.data());
+    for (size_t i = 0; i < c32.size(); ++i) hc[i] = f32_to_f16_bits(c32[i]);
   }
 }
 

@@ -287,7 +287,7 @@ def _raw_matmul(hip, dtype, a, w, rhs_nk):
     """a: [b, m, k], w: [b, k, n] as numpy f32; rhs_nk stores the rhs as [b, n, k] (transposed view)."""
     b, m, k = a.shape
     n = w.shape[2]
-    enc = rng.to_bf16_bits if dtype == ug_amd.BF16 else (lambda v: v)
+    enc = rng.to_bf16_bits if dtype == ug_amd.BF16 else (lambda v: v.astype(np.float16)) if dtype == ug_amd.F16 else (lambda v: v)
     dst = hip.allocate_uninit(dtype, b * m * n)
     sa = hip.slice_from(enc(np.ascontiguousarray(a)))
     if rhs_nk:
@@ -298,7 +298,7 @@ def _raw_matmul(hip, dtype, a, w, rhs_nk):
         rhs = ((b, k, n), (k * n, n, 1), 0)
     hip.matmul(dst, sa, sw, (b, m, n, k), ((b, m, k), (m * k, k, 1), 0), rhs)
     out = dst.to_vec()
-    return (rng.from_bf16_bits(out) if dtype == ug_amd.BF16 else out).reshape(b, m, n)
+    return (rng.from_bf16_bits(out) if dtype == ug_amd.BF16 else out.astype(np.float32)).reshape(b, m, n)
 
 
 # Shapes that are whole multiples of a 256x128, 128x128 or 128x64 tile (K a multiple of 32 f32 / 64
@@ -406,6 +406,31 @@ def test_matmul_split_k(hip, bmnk, rhs_nk, dtype_name):
         np.testing.assert_array_equal(_raw_matmul(hip, F32, ai, wi, rhs_nk), want)
     else:
         np.testing.assert_array_equal(_raw_matmul(hip, ug_amd.BF16, ai, wi, rhs_nk), rng.bf16_round(want.ravel()).reshape(want.shape))
+
+
+# F16 (the reference's CPU backend and its CUDA backend both take it): every kernel family.
+@pytest.mark.parametrize("rhs_nk", [False, True])
+@pytest.mark.parametrize("bmnk", [(2, 96, 80, 160), (1, 256, 128, 192), (2, 128, 64, 128), (1, 128, 2048, 2048), (1, 1, 2048, 2048), (2, 3, 300, 1024),
+                                  (32, 1, 129, 64), (1, 255, 130, 70)])
+def test_matmul_f16(hip, cpu, bmnk, rhs_nk):
+    b, m, n, k = bmnk
+    print("matmul f16", bmnk, "rhs_nk", rhs_nk, flush=True)
+    a = rng.uniform_pm1(27, b * m * k).astype(np.float16).astype(np.float32).reshape(b, m, k)
+    w = rng.uniform_pm1(28, b * k * n).astype(np.float16).astype(np.float32).reshape(b, k, n)
+    got = _raw_matmul(hip, ug_amd.F16, a, w, rhs_nk)
+    exact = a.astype(np.float64) @ w.astype(np.float64)
+    # f32 accumulation of exact f16 products, then one rounding to f16 (2^-11 relative)
+    bound = (2.0 ** -11) * np.abs(exact) + k * np.finfo(np.float32).eps * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64))
+    assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-7)
+    if b * m * n * k <= 1 << 24:
+        # the oracle's F16 matmul (cpu_runtime.rs:345-356 allows F16): same operands through the lazy graph
+        la, lw = LB.copy(a.astype(np.float16), a.shape, cpu), LB.copy(w.astype(np.float16), w.shape, cpu)
+        want = la.matmul(lw).data_vec().astype(np.float32).reshape(b, m, n)
+        # two f32 accumulation orders (each within k*eps*sum|a||w| of the exact product), each rounded once to f16
+        ulp = np.maximum(np.abs(want), 2.0 ** -14) * 2.0 ** -10
+        assert np.all(np.abs(got - want) <= ulp + 2 * k * np.finfo(np.float32).eps * (np.abs(a).astype(np.float64) @ np.abs(w).astype(np.float64)))
+    ai, wi = np.floor(a * 4), np.floor(w * 4)
+    np.testing.assert_array_equal(_raw_matmul(hip, ug_amd.F16, ai, wi, rhs_nk), (ai.astype(np.float64) @ wi.astype(np.float64)).astype(np.float16).astype(np.float32))
 
 
 def test_matmul_tiled_matches_generic_on_integers(hip):

@@ -7,7 +7,8 @@ import pytest
 
 import ref_suite
 from ref_suite import GOLD, f32
-from ug_amd import F32, I32, LazyBuffer as LB, Schedule, SsaKernel
+import ug_amd
+from ug_amd import F32, I32, LazyBuffer as LB, Schedule, SsaKernel, rng
 
 
 def eval_ssa(oracle, kernel, buffers, n_lanes, grid_idx=0):
@@ -166,3 +167,19 @@ def test_copy_checks(cpu):
         s.copy_host_to_device(np.zeros(3, np.float32))
     with pytest.raises(Exception, match="dtype mismatch"):
         s.copy_host_to_device(np.zeros(4, np.int32))
+
+
+def test_cpu_matmul_f16(cpu):
+    """cpu_runtime.rs:345-356 accepts F16 as well as F32; f32 accumulation, one rounding at the end."""
+    a = np.floor(rng.uniform_pm1(40, 2 * 5 * 7) * 8).astype(np.float16).reshape(2, 5, 7)
+    w = np.floor(rng.uniform_pm1(41, 2 * 7 * 3) * 8).astype(np.float16).reshape(2, 7, 3)
+    got = LB.copy(a, a.shape, cpu).matmul(LB.copy(w, w.shape, cpu))
+    assert got.dtype == ug_amd.F16
+    np.testing.assert_array_equal(got.data_vec().reshape(2, 5, 3), (a.astype(np.float32) @ w.astype(np.float32)).astype(np.float16))
+    x = rng.uniform_pm1(42, 4 * 64).astype(np.float16).reshape(4, 64)
+    y = rng.uniform_pm1(43, 64 * 6).astype(np.float16).reshape(64, 6)
+    got = LB.copy(x, x.shape, cpu).matmul(LB.copy(y, y.shape, cpu)).data_vec().astype(np.float64).reshape(4, 6)
+    exact = x.astype(np.float64) @ y.astype(np.float64)
+    assert np.all(np.abs(got - exact) <= 2.0 ** -11 * np.abs(exact) + 64 * np.finfo(np.float32).eps * (np.abs(x).astype(np.float64) @ np.abs(y).astype(np.float64)))
+    with pytest.raises(ug_amd.UgError, match="incorrect dtypes"):
+        LB.copy(rng.to_bf16_bits(x.astype(np.float32)), x.shape, cpu).matmul(LB.copy(rng.to_bf16_bits(y.astype(np.float32)), y.shape, cpu)).data_vec()

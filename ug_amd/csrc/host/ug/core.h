@@ -62,6 +62,55 @@ inline float bf16_bits_to_f32(uint16_t b) {
   return f;
 }
 
+// IEEE binary16 <-> f32 (half::f16::{to_f32, from_f32}: round to nearest even).
+inline float f16_bits_to_f32(uint16_t h) {
+  const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  const uint32_t exp = (h >> 10) & 0x1f, man = h & 0x3ffu;
+  uint32_t u;
+  if (exp == 0) {
+    if (man == 0) {
+      u = sign;
+    } else {  // subnormal: normalise
+      int e = -1;
+      uint32_t m = man;
+      do {
+        ++e;
+        m <<= 1;
+      } while ((m & 0x400u) == 0);
+      u = sign | ((uint32_t)(127 - 15 - e) << 23) | ((m & 0x3ffu) << 13);
+    }
+  } else if (exp == 31) {
+    u = sign | 0x7f800000u | (man << 13);
+  } else {
+    u = sign | ((exp + 127 - 15) << 23) | (man << 13);
+  }
+  float f;
+  std::memcpy(&f, &u, 4);
+  return f;
+}
+inline uint16_t f32_to_f16_bits(float f) {
+  uint32_t x;
+  std::memcpy(&x, &f, 4);
+  const uint32_t sign = (x >> 16) & 0x8000u;
+  const uint32_t man = x & 0x007fffffu;
+  const int32_t exp = (int32_t)((x >> 23) & 0xff);
+  if (exp == 255) return (uint16_t)(sign | 0x7c00u | (man ? (0x0200u | (man >> 13)) : 0));
+  const int32_t half_exp = exp - 127 + 15;
+  if (half_exp >= 31) return (uint16_t)(sign | 0x7c00u);
+  if (half_exp <= 0) {
+    if (14 - half_exp > 24) return (uint16_t)sign;
+    const uint32_t m = man | 0x00800000u;
+    const int shift = 14 - half_exp;
+    uint32_t half_man = m >> shift;
+    const uint32_t round_bit = 1u << (shift - 1);
+    if ((m & round_bit) != 0 && (m & (3 * round_bit - 1)) != 0) half_man += 1;
+    return (uint16_t)(sign | half_man);
+  }
+  uint32_t out = sign | ((uint32_t)half_exp << 10) | (man >> 13);
+  const uint32_t round_bit = 0x00001000u;
+  if ((man & round_bit) != 0 && (man & (3 * round_bit - 1)) != 0) out += 1;  // may carry into the exponent: correct
+  return (uint16_t)out;
+}
 // ug::Const (const.rs:83-174): a typed scalar; floats may not be NaN.
 struct Const {
   DType dtype = DType::F32;

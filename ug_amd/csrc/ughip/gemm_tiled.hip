@@ -11,7 +11,7 @@
 //   operands read 128 bits of consecutive k (v_perm_b32 for bf16; free for f32)
 //   tiles are handed to workgroups XCD by XCD so that the tiles of one batch element share an L2
 //
-// bf16: v_mfma_f32_32x32x16_bf16 (lane l feeds row/col l%32, k = 8*(l/32)..+7).
+// bf16, f16: v_mfma_f32_32x32x16_{bf16,f16} (lane l feeds row/col l%32, k = 8*(l/32)..+7).
 // f32:  v_mfma_f32_32x32x2_f32   (lane l feeds row/col l%32, k = l/32); the 4 floats of a 128-bit
 //       fragment feed 4 consecutive MFMAs, lanes 0-31 holding k..k+3 and lanes 32-63 k+4..k+7.
 #include <hip/hip_runtime.h>
@@ -27,6 +27,7 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 // native vectors, not HIP's uint4/uint2 structs: copies of those become memcpy calls that keep the
 // prefetch registers in scratch memory
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
@@ -45,6 +46,19 @@ template <>
 struct Elt<__bf16> {
   static constexpr int BK = 64, VE = 8;
 };
+template <>
+struct Elt<_Float16> {
+  static constexpr int BK = 64, VE = 8;
+};
+
+// One 32x32x16 MFMA on 8 consecutive k of a 16-bit type.
+__device__ __forceinline__ floatx16 mma16(__bf16, const u32x4& a, const u32x4& b, const floatx16& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ floatx16 mma16(_Float16, const u32x4& a, const u32x4& b, const floatx16& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ floatx16 mma16(float, const u32x4&, const u32x4&, const floatx16& c) { return c; }  // never taken
 
 // 64 banks x 4 bytes: two 128-byte rows span the banks once, so the chunk is rotated by row / 2 --
 // 16 lanes reading one chunk column of 16 consecutive rows then touch 16 different bank groups.
@@ -62,7 +76,7 @@ template <typename T, bool B_NK, int BM, int BN, int NT>
 __device__ __forceinline__ void load_tiles(const T* __restrict__ A, const T* __restrict__ B, const MMArgs& p, int kt, int tid, Staged<BM, NT>& r) {
   constexpr int RP = NT / 8;  // rows per pass
   constexpr int BK = Elt<T>::BK, VE = Elt<T>::VE;
-  constexpr bool IS_BF16 = sizeof(T) == 2;
+  constexpr bool IS_16BIT = sizeof(T) == 2;
   const size_t k0 = (size_t)kt * BK;
   const T* Ap = A + (size_t)(tid >> 3) * p.a_rs + k0 + (tid & 7) * VE;  // row tid/8 (+RP per pass), chunk tid%8
   const size_t a_step = (size_t)RP * p.a_rs;
@@ -75,7 +89,7 @@ __device__ __forceinline__ void load_tiles(const T* __restrict__ A, const T* __r
     for (int i = 0; i < BN / RP; ++i) r.b[i] = *reinterpret_cast<const u32x4*>(Bp + i * b_step);
   } else if (tid < 2 * BN) {
     // 4 (k) x 8 (n) bf16 block or 4 (k) x 4 (n) f32 block per thread; 2 * BN threads cover the tile
-    const int kg = IS_BF16 ? (tid & 15) : (tid & 7), ng = IS_BF16 ? (tid >> 4) : (tid >> 3);
+    const int kg = IS_16BIT ? (tid & 15) : (tid & 7), ng = IS_16BIT ? (tid >> 4) : (tid >> 3);
     const T* Bp = B + (k0 + kg * 4) * (size_t)p.b_rs + ng * VE;
 #pragma unroll
     for (int i = 0; i < 4; ++i) r.b[i] = *reinterpret_cast<const u32x4*>(Bp + i * (size_t)p.b_rs);
@@ -86,7 +100,7 @@ __device__ __forceinline__ void load_tiles(const T* __restrict__ A, const T* __r
 // spread between the MFMAs of a K tile.  PART < 0 issues all of them.
 template <typename T, bool B_NK, int BM, int BN, int NT, int PART>
 __device__ __forceinline__ void store_tiles(u32x4* __restrict__ S, int tid, const Staged<BM, NT>& r) {
-  constexpr bool IS_BF16 = sizeof(T) == 2;
+  constexpr bool IS_16BIT = sizeof(T) == 2;
   constexpr int RP = NT / 8, NA = BM / RP;
   const int row = tid >> 3, chunk = tid & 7;  // rows RP (32 or 64) apart share one swizzle
   u32x4* Sa = S + row * CHUNKS + (chunk ^ lds_swz(row));
@@ -99,7 +113,7 @@ __device__ __forceinline__ void store_tiles(u32x4* __restrict__ S, int tid, cons
     for (int i = 0; i < BN / RP; ++i)
       if (PART < 0 || ((NA + i) & 3) == PART) Sb[i * RP * CHUNKS] = r.b[i];
   } else if (tid < 2 * BN) {
-    if (IS_BF16) {
+    if (IS_16BIT) {
       const int kg = tid & 15, ng = tid >> 4;
       u32x2* S2 = reinterpret_cast<u32x2*>(S);
 #pragma unroll
@@ -139,13 +153,13 @@ __device__ __forceinline__ void load_frags(const u32x4* __restrict__ S, int lane
 
 template <typename T, int MI, int NJ>
 __device__ __forceinline__ void mma_frags(const Frags<MI, NJ>& f, floatx16 (&acc)[MI][NJ]) {
-  constexpr bool IS_BF16 = sizeof(T) == 2;
+  constexpr bool IS_16BIT = sizeof(T) == 2;
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-      if (IS_BF16) {
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, f.a[i]), __builtin_bit_cast(bf16x8, f.b[j]), acc[i][j], 0, 0, 0);
+      if (IS_16BIT) {
+        acc[i][j] = mma16(T(), f.a[i], f.b[j], acc[i][j]);
       } else {
         // whole-vector casts: __builtin_bit_cast applied to one element of an ext vector reads element 0
         const f32x4 af = __builtin_bit_cast(f32x4, f.a[i]), bf = __builtin_bit_cast(f32x4, f.b[j]);
@@ -368,7 +382,7 @@ int pick_split(int dtype, const MMArgs& p, size_t batch, int shape) {
 }  // namespace
 
 bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch) {
-  if (dtype != UGHIP_F32 && dtype != UGHIP_BF16) return false;
+  if (dtype != UGHIP_F32 && dtype != UGHIP_BF16 && dtype != UGHIP_F16) return false;
   const int ve = dtype == UGHIP_F32 ? 4 : 8, bk = dtype == UGHIP_F32 ? 32 : 64;
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.K % bk || batch == 0) return false;
   if (p.a_cs != 1 || p.a_rs % ve || p.a_bs % ve || p.b_bs % ve || p.c_bs % ve) return false;
@@ -398,10 +412,14 @@ hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, siz
     if (!workspace) return hipErrorInvalidValue;
     if (dtype == UGHIP_F32)
       return nt ? launch_shape<float, true, true>(stream, p, batch, s, nsplit, workspace) : launch_shape<float, false, true>(stream, p, batch, s, nsplit, workspace);
+    if (dtype == UGHIP_F16)
+      return nt ? launch_shape<_Float16, true, true>(stream, p, batch, s, nsplit, workspace) : launch_shape<_Float16, false, true>(stream, p, batch, s, nsplit, workspace);
     return nt ? launch_shape<__bf16, true, true>(stream, p, batch, s, nsplit, workspace) : launch_shape<__bf16, false, true>(stream, p, batch, s, nsplit, workspace);
   }
   if (dtype == UGHIP_F32)
     return nt ? launch_shape<float, true, false>(stream, p, batch, s, 1, nullptr) : launch_shape<float, false, false>(stream, p, batch, s, 1, nullptr);
+  if (dtype == UGHIP_F16)
+    return nt ? launch_shape<_Float16, true, false>(stream, p, batch, s, 1, nullptr) : launch_shape<_Float16, false, false>(stream, p, batch, s, 1, nullptr);
   return nt ? launch_shape<__bf16, true, false>(stream, p, batch, s, 1, nullptr) : launch_shape<__bf16, false, false>(stream, p, batch, s, 1, nullptr);
 }
 

@@ -20,6 +20,10 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ floatx16 mma16(const bf16x8& a, const bf16x8& b, const floatx16& c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+__device__ __forceinline__ floatx16 mma16(const f16x8& a, const f16x8& b, const floatx16& c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
 
 // MFMA 32x32 accumulator layout: lane l, register i -> row (i/4)*8 + (l/32)*4 + i%4, col l%32.
 template <typename T>
@@ -80,14 +84,16 @@ __global__ void __launch_bounds__(256) gemm_f32_any(MMArgs p) {
   store_acc(C, acc, m0 + wm, n0 + wn + (lane & 31), p.M, p.N, lane);
 }
 
-__global__ void __launch_bounds__(256) gemm_bf16_any(MMArgs p) {
-  __shared__ __attribute__((aligned(16))) __bf16 As[64][40];  // [m][k], 80-byte rows: conflict-free b128 reads
-  __shared__ __attribute__((aligned(16))) __bf16 Bs[64][40];  // [n][k]
+template <typename T>
+__global__ void __launch_bounds__(256) gemm_half_any(MMArgs p) {
+  typedef T TV __attribute__((ext_vector_type(8)));
+  __shared__ __attribute__((aligned(16))) T As[64][40];  // [m][k], 80-byte rows: conflict-free b128 reads
+  __shared__ __attribute__((aligned(16))) T Bs[64][40];  // [n][k]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
-  const __bf16* __restrict__ A = static_cast<const __bf16*>(p.a) + (size_t)blockIdx.z * p.a_bs;
-  const __bf16* __restrict__ B = static_cast<const __bf16*>(p.b) + (size_t)blockIdx.z * p.b_bs;
-  __bf16* __restrict__ C = static_cast<__bf16*>(p.c) + (size_t)blockIdx.z * p.c_bs;
+  const T* __restrict__ A = static_cast<const T*>(p.a) + (size_t)blockIdx.z * p.a_bs;
+  const T* __restrict__ B = static_cast<const T*>(p.b) + (size_t)blockIdx.z * p.b_bs;
+  T* __restrict__ C = static_cast<T*>(p.c) + (size_t)blockIdx.z * p.c_bs;
   const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
   floatx16 acc = {0};
   for (int k0 = 0; k0 < p.K; k0 += 32) {
@@ -101,7 +107,7 @@ __global__ void __launch_bounds__(256) gemm_bf16_any(MMArgs p) {
         r = e & 63;
         k = e >> 6;
       }
-      As[r][k] = (m0 + r < p.M && k0 + k < p.K) ? A[(long long)(m0 + r) * p.a_rs + (long long)(k0 + k) * p.a_cs] : (__bf16)0.f;
+      As[r][k] = (m0 + r < p.M && k0 + k < p.K) ? A[(long long)(m0 + r) * p.a_rs + (long long)(k0 + k) * p.a_cs] : (T)0.f;
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -113,14 +119,14 @@ __global__ void __launch_bounds__(256) gemm_bf16_any(MMArgs p) {
         k = e & 31;
         n = e >> 5;
       }
-      Bs[n][k] = (k0 + k < p.K && n0 + n < p.N) ? B[(long long)(k0 + k) * p.b_rs + (long long)(n0 + n) * p.b_cs] : (__bf16)0.f;
+      Bs[n][k] = (k0 + k < p.K && n0 + n < p.N) ? B[(long long)(k0 + k) * p.b_rs + (long long)(n0 + n) * p.b_cs] : (T)0.f;
     }
     __syncthreads();
 #pragma unroll
     for (int kk = 0; kk < 32; kk += 16) {
-      bf16x8 a = *reinterpret_cast<const bf16x8*>(&As[wm + (lane & 31)][kk + (lane >> 5) * 8]);
-      bf16x8 b = *reinterpret_cast<const bf16x8*>(&Bs[wn + (lane & 31)][kk + (lane >> 5) * 8]);
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+      TV a = *reinterpret_cast<const TV*>(&As[wm + (lane & 31)][kk + (lane >> 5) * 8]);
+      TV b = *reinterpret_cast<const TV*>(&Bs[wn + (lane & 31)][kk + (lane >> 5) * 8]);
+      acc = mma16(a, b, acc);
     }
     __syncthreads();
   }
@@ -146,6 +152,11 @@ struct Vec<float> {
 template <>
 struct Vec<__bf16> {
   typedef bf16x8 type;
+  static constexpr int N = 8;
+};
+template <>
+struct Vec<_Float16> {
+  typedef f16x8 type;
   static constexpr int N = 8;
 };
 
@@ -387,7 +398,7 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
   if (!dev || !dst || !lhs || !rhs) return set_error(UGHIP_ERR_INVALID, "matmul: null argument");
   if (rank < 2 || rank > 4 || !lhs_dims || !lhs_strides || !rhs_dims || !rhs_strides)
     return set_error(UGHIP_ERR_INVALID, "matmul: rank %zu layouts are not supported", rank);
-  if (dst->dtype != lhs->dtype || dst->dtype != rhs->dtype || (dst->dtype != UGHIP_F32 && dst->dtype != UGHIP_BF16)) {
+  if (dst->dtype != lhs->dtype || dst->dtype != rhs->dtype || (dst->dtype != UGHIP_F32 && dst->dtype != UGHIP_BF16 && dst->dtype != UGHIP_F16)) {
     int code = (dst->dtype == lhs->dtype && dst->dtype == rhs->dtype) ? UGHIP_ERR_UNSUPPORTED : UGHIP_ERR_INVALID;
     return set_error(code, "incorrect dtypes for matmul, dst: %s, lhs: %s, rhs: %s", dtype_name(dst->dtype), dtype_name(lhs->dtype),
                      dtype_name(rhs->dtype));
@@ -429,6 +440,7 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
   const bool gemv_nn_ok = small_m && f32 && rhs_vec_ok && n % 4 == 0 && p.b_cs == 1 && (k == 1 || p.b_rs % 4 == 0);
   if (gemv_nt_ok) {
     if (f32) launch_gemv_nt_any<float>(st, p, b);
+    else if (dst->dtype == UGHIP_F16) launch_gemv_nt_any<_Float16>(st, p, b);
     else launch_gemv_nt_any<__bf16>(st, p, b);
   } else if (gemv_nn_ok) {
     dim3 grid((unsigned)((n + 63) / 64), 1, (unsigned)b);
@@ -453,7 +465,8 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
     dim3 grid((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64), (unsigned)b);
     if (grid.y > 65535 || b > 65535) return set_error(UGHIP_ERR_INVALID, "matmul: m or batch too large for this kernel");
     if (f32) gemm_f32_any<<<grid, 256, 0, st>>>(p);
-    else gemm_bf16_any<<<grid, 256, 0, st>>>(p);
+    else if (dst->dtype == UGHIP_F16) gemm_half_any<_Float16><<<grid, 256, 0, st>>>(p);
+    else gemm_half_any<__bf16><<<grid, 256, 0, st>>>(p);
   }
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
