@@ -198,7 +198,7 @@ int ughip_rtc_check(const char* source, const char* arch, size_t* code_size);
 /* dst[b,m,n] = lhs[b,m,k] x rhs[b,k,n], beta = 0, f32 accumulate.  `rank` (2..4) strides
  * per operand, in elements, as in ug::Layout (layout.rs:577-583); batch strides follow
  * the rules of cpu_runtime.rs:527-549 and ug-cuda/src/gemm.rs:59-74.  dtype triple must
- * match: F32 or BF16 (F16 is UGHIP_ERR_UNSUPPORTED). */
+ * match: F32, F16 or BF16 (ug-cuda/src/gemm.rs:303-330); integers are UGHIP_ERR_UNSUPPORTED. */
 int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs,
                  const ughip_slice* rhs, size_t b, size_t m, size_t n, size_t k, size_t rank,
                  const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset,
