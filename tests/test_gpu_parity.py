@@ -751,3 +751,41 @@ def test_llama_from_a_bf16_checkpoint_on_the_device(hip, cpu, hip_ops, cpu_ops, 
     ids_s, _ = ug_amd.LlamaModel(cpu, cpu_ops, cfg, True, seed=9, std=0.02, round_bf16=True).generate(prompt, 6)
     assert ids_h.tolist() == ids_c.tolist() == ids_s.tolist()
     np.testing.assert_allclose(st_h["margins"], st_c["margins"], rtol=1e-2, atol=1e-7)
+
+
+# ---- 16-bit float kernels: no CPU reference exists (this gcc rejects the types, cpu_runtime.rs:478-486 compiles
+# with plain gcc), so the expectation is numpy with every op computed in f32 and rounded once to the 16-bit type.
+def _half_io(dtype):
+    if dtype == ug_amd.F16:
+        return (lambda v: v.astype(np.float16)), (lambda o: o.astype(np.float32))
+    return rng.to_bf16_bits, rng.from_bf16_bits
+
+
+@pytest.mark.parametrize("dtype", [ug_amd.F16, ug_amd.BF16], ids=["f16", "bf16"])
+def test_half_precision_elementwise_and_reduce(hip, dtype):
+    enc, dec = _half_io(dtype)
+    rnd = lambda v: dec(enc(np.asarray(v, np.float32)))      # round to the 16-bit type, back as f32
+    rows, cols = 37, 264
+    x = rnd(rng.normal(81, rows * cols)).reshape(rows, cols)
+    y = rnd(rng.uniform_pm1(82, rows * cols)).reshape(rows, cols)
+    lx, ly = LB.copy(enc(x), (rows, cols), hip), LB.copy(enc(y), (rows, cols), hip)
+    assert lx.dtype == dtype
+    # one rounding per op
+    np.testing.assert_array_equal(dec(lx.binary("add", ly).data_vec()).reshape(rows, cols), rnd(x + y))
+    np.testing.assert_array_equal(dec(lx.binary("mul", ly).data_vec()).reshape(rows, cols), rnd(x * y))
+    # two fused ops: the compiler may contract a*b+c into one fused multiply-add (one rounding instead of two)
+    got = dec(lx.binary("mul", ly).binary("add", lx).data_vec()).reshape(rows, cols)
+    two, one = rnd(rnd(x * y) + x), rnd(x.astype(np.float64) * y + x)
+    assert np.all((got == two) | (got == one))
+    got = dec(ly.unary("exp").data_vec()).reshape(rows, cols)
+    want = rnd(np.exp(y.astype(np.float64)))
+    assert np.all(np.abs(got - want) <= np.abs(want) * (2.0 ** -7 if dtype == ug_amd.BF16 else 2.0 ** -10))
+    # casts: widening is exact, narrowing rounds to nearest even
+    np.testing.assert_array_equal(lx.cast(F32).data_vec().reshape(rows, cols), x)
+    z = rng.normal(83, rows * cols)
+    np.testing.assert_array_equal(dec(LB.copy(z, (rows, cols), hip).cast(dtype).data_vec()), rnd(z))
+    # reductions: max is exact; a sum in a 16-bit accumulator is only bounded (order differs from any serial loop)
+    np.testing.assert_array_equal(dec(lx.reduce("max", 1).data_vec()).reshape(rows, -1)[:, 0], x.max(1))
+    s = dec(ly.reduce("sum", 1).data_vec()).reshape(rows, -1)[:, 0]
+    eps16 = 2.0 ** -8 if dtype == ug_amd.BF16 else 2.0 ** -11
+    assert np.all(np.abs(s - y.astype(np.float64).sum(1)) <= cols * eps16 * np.abs(y).sum(1))
