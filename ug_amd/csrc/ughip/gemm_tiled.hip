@@ -171,39 +171,84 @@ __device__ __forceinline__ void mma_frags(const Frags<MI, NJ>& f, floatx16 (&acc
     }
 }
 
+// Issue order of one k step, as scheduling groups: every MFMA is followed by its share of the step's
+// memory instructions (LDS reads of the next step first, then staging stores, global loads spread
+// in between), so that each of them issues in the shadow of a running MFMA instead of in a burst
+// that fills the LDS queue and blocks the wave.
+template <int N_MFMA, int N_READ, int N_WRITE, int N_VMEM>
+__device__ __forceinline__ void interleave_step() {
+  constexpr int N_DS = N_READ + N_WRITE;
+#pragma unroll
+  for (int i = 0; i < N_MFMA; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+#pragma unroll
+    for (int d = i * N_DS / N_MFMA; d < (i + 1) * N_DS / N_MFMA; ++d) {
+      if (d < N_READ) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+      else __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);             // one LDS write
+    }
+#pragma unroll
+    for (int v = i * N_VMEM / N_MFMA; v < (i + 1) * N_VMEM / N_MFMA; ++v) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+  }
+}
+
+// Staging stores of part PART (see store_tiles): A stores i with i % 4 == PART, then B's.
+template <typename T, bool B_NK, int BM, int BN, int NT>
+constexpr int stores_in_part(int part) {
+  const int rp = NT / 8, na = BM / rp;
+  int n = 0;
+  for (int i = 0; i < na; ++i) n += (i & 3) == part;
+  if (B_NK) {
+    for (int i = 0; i < BN / rp; ++i) n += ((na + i) & 3) == part;
+  } else if (sizeof(T) == 2) {
+    n += 2;  // 8 columns, two per part
+  } else {
+    n += 1;  // 4 columns, one per part
+  }
+  return n;
+}
+
 // One K tile: multiply the tile in LDS stage `cur`; meanwhile move the tile held in `wr` (loaded
-// from global memory one phase ago) into stage `nxt`, a quarter between each group of MFMAs, and
-// start the global loads of tile `load_kt` into `ld`.  Fragments are double-buffered in registers:
-// the LDS reads of k step s+1 are in flight while the MFMAs of step s run.
+// from global memory one phase ago) into stage `nxt`, a quarter per k step, and start the global
+// loads of tile `load_kt` into `ld`.  Fragments are double-buffered in registers: the LDS reads of
+// k step s+1 are in flight while the MFMAs of step s run.
+// WRITE: 1 = always store, 0 = never, 2 = decided at run time by `do_write` (tail phases; a
+// run-time branch splits the scheduling region, so the steady state uses the compile-time forms).
 // The loads are unconditional (LOAD is a compile-time switch): a load under a run-time branch makes
 // the compiler wait for every outstanding load before the staging stores, which would undo the
 // two-tile lead.
-template <typename T, bool B_NK, int BM, int BN, int NT, int MI, int NJ, bool LOAD>
+template <typename T, bool B_NK, int BM, int BN, int NT, int MI, int NJ, bool LOAD, int WRITE>
 __device__ __forceinline__ void k_phase(const T* __restrict__ A, const T* __restrict__ B, const MMArgs& p, const u32x4* __restrict__ cur, u32x4* __restrict__ nxt,
                                         bool do_write, const Staged<BM, NT>& wr, int load_kt, Staged<BM, NT>& ld, int tid, int lane, int wm, int wn,
                                         floatx16 (&acc)[MI][NJ]) {
-  if (LOAD) load_tiles<T, B_NK, BM, BN, NT>(A, B, p, load_kt, tid, ld);
-  // Issue order within a k step: LDS reads of the next step, the MFMAs of this step (their issue
-  // time covers the LDS latency), then a quarter of the staging stores.  The scheduling barriers
-  // keep the compiler from sinking the reads next to their uses, which would serialise every
-  // LDS round trip with the matrix pipe.
+  constexpr int N_MFMA = MI * NJ * (sizeof(T) == 4 ? 4 : 1), N_READ = MI + NJ;
+  constexpr int N_VMEM = LOAD ? BM * 8 / NT + (B_NK ? BN * 8 / NT : 4) : 0;
+  constexpr bool FINE = WRITE != 2;
   Frags<MI, NJ> f0, f1;
   load_frags<BM, MI, NJ>(cur, lane, wm, wn, 0, f0);
+  __builtin_amdgcn_sched_barrier(0);
+  // step 0
+  if (LOAD) load_tiles<T, B_NK, BM, BN, NT>(A, B, p, load_kt, tid, ld);
   load_frags<BM, MI, NJ>(cur, lane, wm, wn, 1, f1);
-  __builtin_amdgcn_sched_barrier(0);
   mma_frags<T, MI, NJ>(f0, acc);
-  if (do_write) store_tiles<T, B_NK, BM, BN, NT, 0>(nxt, tid, wr);
+  if (WRITE == 1 || (WRITE == 2 && do_write)) store_tiles<T, B_NK, BM, BN, NT, 0>(nxt, tid, wr);
+  if (FINE) interleave_step<N_MFMA, N_READ, WRITE ? stores_in_part<T, B_NK, BM, BN, NT>(0) : 0, N_VMEM>();
   __builtin_amdgcn_sched_barrier(0);
+  // step 1
   load_frags<BM, MI, NJ>(cur, lane, wm, wn, 2, f0);
   mma_frags<T, MI, NJ>(f1, acc);
-  if (do_write) store_tiles<T, B_NK, BM, BN, NT, 1>(nxt, tid, wr);
+  if (WRITE == 1 || (WRITE == 2 && do_write)) store_tiles<T, B_NK, BM, BN, NT, 1>(nxt, tid, wr);
+  if (FINE) interleave_step<N_MFMA, N_READ, WRITE ? stores_in_part<T, B_NK, BM, BN, NT>(1) : 0, 0>();
   __builtin_amdgcn_sched_barrier(0);
+  // step 2
   load_frags<BM, MI, NJ>(cur, lane, wm, wn, 3, f1);
   mma_frags<T, MI, NJ>(f0, acc);
-  if (do_write) store_tiles<T, B_NK, BM, BN, NT, 2>(nxt, tid, wr);
+  if (WRITE == 1 || (WRITE == 2 && do_write)) store_tiles<T, B_NK, BM, BN, NT, 2>(nxt, tid, wr);
+  if (FINE) interleave_step<N_MFMA, N_READ, WRITE ? stores_in_part<T, B_NK, BM, BN, NT>(2) : 0, 0>();
   __builtin_amdgcn_sched_barrier(0);
+  // step 3
   mma_frags<T, MI, NJ>(f1, acc);
-  if (do_write) store_tiles<T, B_NK, BM, BN, NT, 3>(nxt, tid, wr);
+  if (WRITE == 1 || (WRITE == 2 && do_write)) store_tiles<T, B_NK, BM, BN, NT, 3>(nxt, tid, wr);
+  if (FINE) interleave_step<N_MFMA, 0, WRITE ? stores_in_part<T, B_NK, BM, BN, NT>(3) : 0, 0>();
 }
 
 // NT threads = NT / 64 waves laid out (NT / 128) x 2 over the tile: 4 waves give each wave a
@@ -258,15 +303,23 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p, int tiles_m, int tile
   store_tiles<T, B_NK, BM, BN, NT, -1>(lds0, tid, r0);
   __syncthreads();
   int kt = 0;
-  for (; kt + 1 < KT; kt += 2) {
-    // Past the end the last tile is loaded again (and never stored): same instruction stream for
-    // every iteration.  Stage 1 was last read in the previous odd phase, a barrier ago.
-    k_phase<T, B_NK, BM, BN, NT, MI, NJ, true>(A, B, p, lds0, lds1, true, r1, min(kt + 2, KT - 1), r0, tid, lane, wm, wn, acc);
+  // steady state: both phases store and load unconditionally (tiles kt+2 and kt+3 exist)
+  for (; kt + 3 < KT; kt += 2) {
+    // stage 1 was last read in the previous odd phase, a barrier ago
+    k_phase<T, B_NK, BM, BN, NT, MI, NJ, true, 1>(A, B, p, lds0, lds1, true, r1, kt + 2, r0, tid, lane, wm, wn, acc);
     __syncthreads();
-    k_phase<T, B_NK, BM, BN, NT, MI, NJ, true>(A, B, p, lds1, lds0, kt + 2 < KT, r0, min(kt + 3, KT - 1), r1, tid, lane, wm, wn, acc);
+    k_phase<T, B_NK, BM, BN, NT, MI, NJ, true, 1>(A, B, p, lds1, lds0, true, r0, kt + 3, r1, tid, lane, wm, wn, acc);
     __syncthreads();
   }
-  if (kt < KT) k_phase<T, B_NK, BM, BN, NT, MI, NJ, false>(A, B, p, lds0, lds1, false, r1, 0, r0, tid, lane, wm, wn, acc);  // odd tile count: the last tile
+  // the last two or three tiles: tile kt+2, if there is one, still has to be fetched (past the end
+  // the last tile is loaded again and never stored)
+  for (; kt + 1 < KT; kt += 2) {
+    k_phase<T, B_NK, BM, BN, NT, MI, NJ, true, 1>(A, B, p, lds0, lds1, true, r1, min(kt + 2, KT - 1), r0, tid, lane, wm, wn, acc);
+    __syncthreads();
+    k_phase<T, B_NK, BM, BN, NT, MI, NJ, false, 2>(A, B, p, lds1, lds0, kt + 2 < KT, r0, 0, r1, tid, lane, wm, wn, acc);
+    __syncthreads();
+  }
+  if (kt < KT) k_phase<T, B_NK, BM, BN, NT, MI, NJ, false, 0>(A, B, p, lds0, lds1, false, r1, 0, r0, tid, lane, wm, wn, acc);  // odd tile count: the last tile
 
   // accumulator register r of lane l: row (r/4)*8 + (l/32)*4 + r%4, column l%32
   if (SPLIT) {
