@@ -249,14 +249,30 @@ def llama_pieces(dev, steps, warmup):
     v = LB.copy(rng.normal(8 + 300, heads * t * hd), (1, heads, t, hd), dev)
     gemm("c4_qk_t_b32_512x512x64", q, kk, True, heads, t, t, hd)
     gemm("c4_att_v_b32_512x64x512", s, v, False, heads, t, hd, t)
+
+    # the whole chain either side of the softmax (rope(q), repeat, q k^T, scale, mask, softmax, x v, transposes) as one
+    # kernel over preallocated caches of 4 kv heads: scores stay in registers.  flop = the two causal products.
+    nkv, cap = 4, 2048
+    qf = LB.copy(rng.normal(7, t * heads * hd), (1, t, heads * hd), dev)
+    kc = LB.copy(rng.normal(8 + 200, nkv * cap * hd), (1, nkv, cap, hd), dev)
+    vc = LB.copy(rng.normal(8 + 300, nkv * cap * hd), (1, nkv, cap, hd), dev)
+    att = ops.attention_cached(qf, kc, vc, t, float(np.float32(hd) ** np.float32(-0.5)), cos, sin, pos, False)
+    cs = Schedule.create_one(att).compile()
+    _, ms = timed(dev, cs.run, steps, warmup)
+    sec = ms * 1e-3 / steps
+    flop = 2 * 2.0 * heads * hd * t * (t + 1) / 2
+    nbytes = 4.0 * (2 * t * heads * hd + 2 * nkv * t * hd)
+    out["c4_attention_cached_t512"] = {"us": round(sec * 1e6, 2), "TFLOP/s": round(flop / sec / 1e12, 2), "frac_mfma_f32": round(flop / sec / 1e12 / MFMA_F32_PEAK_TF, 4),
+                                       "algorithmic_bytes": int(nbytes), "replaces": "c4_rope_q + c4_qk_t + c4_causal_softmax_fused + c4_att_v + 2 repeats + 2 transposes"}
     return out
 
 
-def llama_decode(dev, n_prompt=128, n_steps=128, fused_attention=False):
+def llama_decode(dev, n_prompt=128, n_steps=128, fused_attention=0):
     """Config 5: TinyLlama-1.1B shape, random-init f32 weights, prefill 128 then 128 greedy steps.
     Fresh buffers are not zero-filled here (every kernel of the model writes its whole output; the
-    ids are the same either way, which the GPU tests check).  fused_attention routes attention
-    through ughip_causal_softmax_rows / ughip_attention_decode instead of the op-by-op graph."""
+    ids are the same either way, which the GPU tests check).  fused_attention: 0 = the reference's
+    op-by-op graph; 1 = ughip_causal_softmax_rows / ughip_rope_append / ughip_attention_decode;
+    2 = caches written in place (ughip_kv_append) and ughip_attention_cached for prefill and decode."""
     import ug_amd
     from ug_amd import rng
     cfg = ug_amd.LlamaConfig()
@@ -344,7 +360,7 @@ def main():
         except Exception as e:  # noqa: BLE001
             line["extras"] = {"error": f"{type(e).__name__}: {e}"}
     if not (args.no_llama or args.headline_only):
-        for key, fused in (("llama_decode_f32", False), ("llama_decode_f32_fused_attention", True)):
+        for key, fused in (("llama_decode_f32", 0), ("llama_decode_f32_fused_attention", 1), ("llama_decode_f32_inplace_cache", 2)):
             try:
                 line.setdefault("extras", {})[key] = llama_decode(dev, fused_attention=fused)
             except Exception as e:  # noqa: BLE001

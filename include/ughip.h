@@ -252,6 +252,28 @@ int ughip_rope_append(ughip_device* dev, const ughip_slice* cache, const ughip_s
                       ughip_slice* dst, size_t bh, size_t s_old, size_t d,
                       const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos,
                       int interleaved);
+/* The same growth in place, for t new positions at once (replaces the cat of model.rs:226-230,
+ * which copies the whole cache every step): cache [b, n, cap, d] is preallocated for cap
+ * positions; rows s_old .. s_old + t - 1 of every head receive x [b, t, n * d] (the layout the
+ * k / v projections write), rotated at table rows pos[0] + i when cos/sin/pos are given.
+ * s_old + t <= cap, d % 4 == 0.  Rows past s_old + t are left untouched. */
+int ughip_kv_append(ughip_device* dev, ughip_slice* cache, const ughip_slice* x, size_t b,
+                    size_t n, size_t cap, size_t s_old, size_t t, size_t d,
+                    const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos,
+                    int interleaved);
+/* Causal attention of t query positions over such caches, f32, without materialising the
+ * [heads, t, s] scores (the chain model.rs:231-245: repeat, q k^T, scale, causal_mask, softmax,
+ * x v, transpose, in one launch): q and dst [b, t, n_heads * d] (projection layout), k and v
+ * [b, n_kv_heads, cap, d] with rows 0 .. s - 1 valid; query i sits at position s - t + i and
+ * attends to keys 0 .. s - t + i; rope / rope_i is applied to q at table rows pos[0] + i when
+ * cos/sin/pos are given.  t == 1 is ughip_attention_decode_rope on a cache of capacity cap;
+ * t > 1 needs d = 32, 64 or 128 (UGHIP_ERR_UNSUPPORTED otherwise).  s - t == 0 and cap == s give
+ * the reference's prefill. */
+int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, const ughip_slice* k,
+                           const ughip_slice* v, ughip_slice* dst, size_t b, size_t n_heads,
+                           size_t n_kv_heads, size_t t, size_t s, size_t cap, size_t d,
+                           float scale, const ughip_slice* cos, const ughip_slice* sin,
+                           const ughip_slice* pos, int interleaved);
 
 /* ---- element type conversion ------------------------------------------------------------------
  * dst[i] = (dtype of dst) src[i], same length, any pair of the five dtypes.  Replaces the host

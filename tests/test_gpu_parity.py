@@ -617,9 +617,11 @@ def test_attention_fusion_errors(hip, hip_ops):
         hip_ops.attention_decode(q3, same, same, 1.0).data_vec()
 
 
+@pytest.mark.parametrize("level", [1, 2])
 @pytest.mark.parametrize("width", ["small", "config5"])
-def test_llama_fused_attention_ids_match_unfused_cpu(hip, cpu, hip_ops, cpu_ops, width):
-    """The model with both fusions switched on (HIP) against the reference's op-by-op graph (oracle)."""
+def test_llama_fused_attention_ids_match_unfused_cpu(hip, cpu, hip_ops, cpu_ops, width, level):
+    """The model with the attention fusions switched on (HIP; level 2 = caches written in place and
+    attention without materialised scores) against the reference's op-by-op graph (oracle)."""
     if width == "small":
         cfg = ug_amd.LlamaConfig(hidden_size=128, intermediate_size=320, max_position_embeddings=64, num_attention_heads=4, num_key_value_heads=2,
                                  num_hidden_layers=2, vocab_size=512)
@@ -628,7 +630,7 @@ def test_llama_fused_attention_ids_match_unfused_cpu(hip, cpu, hip_ops, cpu_ops,
         cfg = ug_amd.LlamaConfig(num_hidden_layers=2, max_position_embeddings=256)
         n_prompt, n_steps, std = 16, 6, 0.02
     prompt = rng.token_ids(10, n_prompt, cfg.vocab_size)
-    toks_h, st_h = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=std, fused_attention=True).generate(prompt, n_steps)
+    toks_h, st_h = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=std, fused_attention=level).generate(prompt, n_steps)
     toks_c, st_c = ug_amd.LlamaModel(cpu, cpu_ops, cfg, True, seed=9, std=std).generate(prompt, n_steps)
     print("hip fused", toks_h.tolist(), "cpu", toks_c.tolist(), flush=True)
     assert toks_h.tolist() == toks_c.tolist()
@@ -692,6 +694,141 @@ def test_attention_decode_flat_fused(hip, cpu, hip_ops, cpu_ops, interleaved, b,
     got, want = run(hip, hip_ops), run(cpu, cpu_ops)
     scale_abs = float(np.abs(want).max())
     np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-5 * scale_abs)
+
+
+# ---- caches written in place, attention over them without materialised scores ---------------------------------------------
+def _rope_rows_f64(x, cos, sin, pos0, interleaved):
+    """x [b, t, n, d] float64 rotated at table rows pos0 + i (cpu_ops.rs:58-126 written with numpy)."""
+    t, d = x.shape[1], x.shape[3]
+    c = cos.reshape(-1, d // 2)[pos0:pos0 + t].astype(np.float64)[None, :, None, :]
+    sn = sin.reshape(-1, d // 2)[pos0:pos0 + t].astype(np.float64)[None, :, None, :]
+    out = np.empty_like(x)
+    if interleaved:
+        a, b2 = x[..., 0::2], x[..., 1::2]
+        out[..., 0::2], out[..., 1::2] = a * c - b2 * sn, a * sn + b2 * c
+    else:
+        a, b2 = x[..., :d // 2], x[..., d // 2:]
+        out[..., :d // 2], out[..., d // 2:] = a * c - b2 * sn, a * sn + b2 * c
+    return out
+
+
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("b,n,cap,length,t,d,with_rope", [(1, 4, 64, 0, 1, 64, True), (1, 4, 64, 5, 1, 64, True), (1, 4, 300, 0, 200, 64, True), (2, 2, 40, 7, 9, 64, True),
+                                                          (1, 4, 64, 63, 1, 64, False), (1, 3, 50, 9, 4, 16, True), (1, 2, 20, 3, 17, 128, True), (1, 2, 30, 3, 2, 12, True)])
+def test_kv_append_in_place(hip, cpu, hip_ops, cpu_ops, interleaved, b, n, cap, length, t, d, with_rope):
+    print("kv append", (b, n, cap, length, t, d, with_rope, interleaved), flush=True)
+    assert hip_ops.kv_cache_capacity(2048, 64) == 2048 and hip_ops.kv_cache_capacity(2048, 48) == 0 and cpu_ops.kv_cache_capacity(2048, 64) == 0
+    store = rng.normal(81, b * n * cap * d)
+    x = rng.normal(82, b * t * n * d)
+    pos0 = length + 2
+    cache = LB.copy(store, (b, n, cap, d), hip)
+    cache.realize()
+    args = [LB.copy(x, (b, t, n * d), hip)]
+    if with_rope:
+        cos, sin = _rope_tables(hip, d, max_pos=cap + 8)
+        args += [cos, sin, LB.copy(np.array([pos0], np.int32), (1, 1), hip), interleaved]
+    out = hip_ops.kv_append(cache, length, *args)
+    assert tuple(out.dims()) == (b, n, cap, d)
+    got = out.data_vec().reshape(b, n, cap, d)
+    np.testing.assert_array_equal(cache.data_vec().reshape(b, n, cap, d), got)   # the same storage: the write happened in place
+    before = store.reshape(b, n, cap, d)
+    np.testing.assert_array_equal(got[:, :, :length], before[:, :, :length])       # rows outside the appended range are untouched
+    np.testing.assert_array_equal(got[:, :, length + t:], before[:, :, length + t:])
+    rows = x.reshape(b, t, n, d)
+    if with_rope:
+        want = _rope_rows_f64(rows.astype(np.float64), cos.data_vec(), sin.data_vec(), pos0, interleaved)
+        np.testing.assert_allclose(got[:, :, length:length + t], want.transpose(0, 2, 1, 3), rtol=1e-5, atol=1e-6)
+    else:
+        np.testing.assert_array_equal(got[:, :, length:length + t], rows.transpose(0, 2, 1, 3))
+    # and against the oracle's op-by-op growth (split/transpose + rope + cat on a cache of exactly `length` rows)
+    ccache = LB.copy(np.ascontiguousarray(before[:, :, :length]).ravel(), (b, n, length, d), cpu) if length else LB.cst(0.0, (b, n, 0, d), cpu)
+    cargs = [LB.copy(x, (b, t, n * d), cpu)]
+    if with_rope:
+        ccos, csin = _rope_tables(cpu, d, max_pos=cap + 8)
+        cargs += [ccos, csin, LB.copy(np.array([pos0], np.int32), (1, 1), cpu), interleaved]
+    want_c = cpu_ops.kv_append(ccache, length, *cargs).data_vec().reshape(b, n, length + t, d)
+    np.testing.assert_allclose(got[:, :, :length + t], want_c, rtol=1e-5, atol=1e-6)
+
+
+def test_kv_append_errors(hip, hip_ops):
+    cache = LB.copy(np.zeros(2 * 8 * 16, np.float32), (1, 2, 8, 16), hip)
+    with pytest.raises(ug_amd.UgError, match="exceed the cache capacity"):
+        hip_ops.kv_append(cache, 7, LB.copy(np.zeros(2 * 2 * 16, np.float32), (1, 2, 32), hip)).data_vec()
+    with pytest.raises(ug_amd.UgError, match="mismatched shapes"):
+        hip_ops.kv_append(cache, 0, LB.copy(np.zeros(48, np.float32), (1, 1, 48), hip)).data_vec()
+
+
+def _attention_truth(q, k, v, s, t, scale, rep):
+    """float64: q [b, nh, t, d], k and v [b, nkv, s, d]; query i sees keys 0 .. s - t + i."""
+    sc = np.einsum("bhtd,bhsd->bhts", q, np.repeat(k, rep, 1)) * scale
+    keep = np.arange(s)[None, :] <= (s - t + np.arange(t))[:, None]
+    sc = np.where(keep, sc, -np.inf)
+    p = np.exp(sc - sc.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    return np.einsum("bhts,bhsd->bhtd", p, np.repeat(v, rep, 1))
+
+
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("b,nh,nkv,t,s,cap,d,with_rope", [
+    (1, 32, 4, 128, 128, 256, 64, True),     # the prefill of config 5
+    (1, 8, 2, 33, 33, 33, 64, True),         # ragged last block, cache exactly full
+    (2, 4, 2, 70, 70, 100, 128, True),
+    (1, 4, 4, 200, 200, 512, 64, False),
+    (1, 8, 2, 2, 2, 16, 64, True),           # two positions
+    (1, 4, 2, 50, 50, 64, 32, True),
+    (1, 8, 2, 40, 100, 128, 64, True),       # 40 new positions after 60 cached ones
+    (1, 4, 1, 5, 300, 300, 128, True),
+    (1, 32, 4, 1, 77, 128, 64, True),        # one position: the single-query kernel on a cache with spare rows
+    (1, 4, 1, 1, 9, 64, 16, True),
+])
+def test_attention_cached(hip, cpu, hip_ops, cpu_ops, interleaved, b, nh, nkv, t, s, cap, d, with_rope):
+    print("attention cached", (b, nh, nkv, t, s, cap, d, with_rope, interleaved), flush=True)
+    q = rng.normal(83, b * t * nh * d)
+    k = rng.normal(84, b * nkv * cap * d)
+    v = rng.normal(85, b * nkv * cap * d)
+    # rows past s must not matter: poison them
+    k4, v4 = k.reshape(b, nkv, cap, d).copy(), v.reshape(b, nkv, cap, d).copy()
+    k4[:, :, s:], v4[:, :, s:] = np.nan, np.inf
+    scale = float(np.float32(d) ** np.float32(-0.5))
+    pos0 = s - t
+    args = [LB.copy(q, (b, t, nh * d), hip), LB.copy(k4.ravel(), (b, nkv, cap, d), hip), LB.copy(v4.ravel(), (b, nkv, cap, d), hip), s, scale]
+    if with_rope:
+        cos, sin = _rope_tables(hip, d, max_pos=s + 8)
+        args += [cos, sin, LB.copy(np.array([pos0], np.int32), (1, 1), hip), interleaved]
+    out = hip_ops.attention_cached(*args)
+    assert tuple(out.dims()) == (b, t, nh * d)
+    got = out.data_vec().reshape(b, t, nh, d)
+    q6 = q.reshape(b, t, nh, d).astype(np.float64)
+    if with_rope:
+        q6 = _rope_rows_f64(q6, cos.data_vec(), sin.data_vec(), pos0, interleaved)
+    truth = _attention_truth(q6.transpose(0, 2, 1, 3), k4[:, :, :s].astype(np.float64), v4[:, :, :s].astype(np.float64), s, t, scale, nh // nkv).transpose(0, 2, 1, 3)
+    tol = 2e-5 * np.abs(truth).max() + 2e-5 * np.abs(truth)
+    assert np.all(np.abs(got - truth) <= tol), float(np.abs(got - truth).max())
+    if t == 1 or t == s:
+        # the reference's chain on the oracle (its causal mask only covers queries that start at position 0)
+        cargs = [LB.copy(q, (b, t, nh * d), cpu), LB.copy(np.ascontiguousarray(k4[:, :, :s]).ravel(), (b, nkv, s, d), cpu),
+                 LB.copy(np.ascontiguousarray(v4[:, :, :s]).ravel(), (b, nkv, s, d), cpu), s, scale]
+        if with_rope:
+            ccos, csin = _rope_tables(cpu, d, max_pos=s + 8)
+            cargs += [ccos, csin, LB.copy(np.array([pos0], np.int32), (1, 1), cpu), interleaved]
+        want = cpu_ops.attention_cached(*cargs).data_vec().reshape(b, t, nh, d)
+        assert np.all(np.abs(got - want) <= 2 * tol), float(np.abs(got - want).max())
+
+
+def test_attention_cached_errors(hip, cpu, hip_ops, cpu_ops):
+    def lb(shape, dev=hip):
+        return LB.copy(np.zeros(int(np.prod(shape)), np.float32), shape, dev)
+    with pytest.raises(ug_amd.UgError, match="mismatched shapes"):
+        hip_ops.attention_cached(lb((1, 4, 128)), lb((1, 2, 8, 64)), lb((1, 2, 8, 64)), 9, 1.0).data_vec()       # more keys than the cache holds
+    with pytest.raises(ug_amd.UgError, match="mismatched shapes"):
+        hip_ops.attention_cached(lb((1, 4, 128)), lb((1, 2, 8, 64)), lb((1, 2, 8, 64)), 3, 1.0).data_vec()       # more queries than keys
+    # a head size without a multi-query kernel falls back to the op-by-op chain, which needs exact-length caches
+    with pytest.raises(ug_amd.UgError, match="exactly"):
+        hip_ops.attention_cached(lb((1, 4, 32)), lb((1, 2, 8, 16)), lb((1, 2, 8, 16)), 4, 1.0).data_vec()
+    out = hip_ops.attention_cached(lb((1, 4, 32)), lb((1, 2, 4, 16)), lb((1, 2, 4, 16)), 4, 1.0).data_vec()
+    assert out.shape == (4 * 32,) and np.all(out == 0)
+    with pytest.raises(ug_amd.UgError, match="need a device kernel"):
+        cpu_ops.attention_cached(lb((1, 2, 128), cpu), lb((1, 2, 5, 64), cpu), lb((1, 2, 5, 64), cpu), 5, 1.0).data_vec()
 
 
 # ---- safetensors: upload in the stored dtype, convert on the device ----------------------------------------------------

@@ -663,6 +663,29 @@ class LlamaOps(_Handle):
         lb._keep += [k, v] + ([cos, sin, pos] if rope else [])
         return lb
 
+    def kv_cache_capacity(self, max_positions, head_dim=64):
+        """Rows this device preallocates per cache head (0: caches grow by concatenation)."""
+        out = C.c_size_t()
+        _chk(host_lib().ugh_llama_kv_cache_capacity(_p(self.h), C.c_size_t(max_positions), C.c_size_t(head_dim), C.byref(out)))
+        return out.value
+
+    def kv_append(self, cache, length, x, cos=None, sin=None, pos=None, interleaved=False):
+        """cache [b, n, cap, d] holding `length` rows receives x [b, t, n * d] as rows length .. length + t - 1
+        (rotated when a table is given): in place when cap > length, by concatenation when cap == length."""
+        rope = cos is not None
+        lb = self._op("ugh_llama_kv_append", cache, C.c_size_t(length), _p(x.h), _p(cos.h) if rope else None, _p(sin.h) if rope else None,
+                      _p(pos.h) if rope else None, int(interleaved))
+        lb._keep += [x] + ([cos, sin, pos] if rope else [])
+        return lb
+
+    def attention_cached(self, q, k, v, s, scale, cos=None, sin=None, pos=None, interleaved=False):
+        """Causal attention of q [b, t, nh * d] over the first s rows of k, v [b, nkv, cap, d] -> [b, t, nh * d]."""
+        rope = cos is not None
+        lb = self._op("ugh_llama_attention_cached", q, _p(k.h), _p(v.h), C.c_size_t(s), C.c_float(scale), _p(cos.h) if rope else None,
+                      _p(sin.h) if rope else None, _p(pos.h) if rope else None, int(interleaved))
+        lb._keep += [k, v] + ([cos, sin, pos] if rope else [])
+        return lb
+
 
 class _Llama:
     """Graph builders of ug-llama/src/model.rs:32-109."""
@@ -744,7 +767,7 @@ class LlamaModel(_Handle):
                                             int(round_bf16), C.byref(out)))
         super().__init__(out.value)
         if fused_attention:
-            _chk(host_lib().ugh_llama_model_set_fused_attention(_p(self.h), 1))
+            _chk(host_lib().ugh_llama_model_set_fused_attention(_p(self.h), int(fused_attention)))
         self._keep = [device, ops]
         self.cfg = cfg
 
@@ -761,7 +784,7 @@ class LlamaModel(_Handle):
         self._keep = [device, ops]
         self.cfg = cfg
         if fused_attention:
-            _chk(host_lib().ugh_llama_model_set_fused_attention(_p(self.h), 1))
+            _chk(host_lib().ugh_llama_model_set_fused_attention(_p(self.h), int(fused_attention)))
         return self
 
     def generate(self, prompt, n_steps):

@@ -457,6 +457,21 @@ int ugh_llama_attention_decode_flat(void* ops, void* q, void* k, void* v, float 
     else *out = box(ops_of(ops).attention_decode_flat(lb_of(q), lb_of(k), lb_of(v), scale, nullptr, nullptr, nullptr, false));
   });
 }
+int ugh_llama_kv_cache_capacity(void* ops, size_t max_positions, size_t head_dim, size_t* out) {
+  return guard([&] { *out = ops_of(ops).kv_cache_capacity(max_positions, head_dim); });
+}
+int ugh_llama_kv_append(void* ops, void* cache, size_t len, void* x, void* cos, void* sin, void* pos, int interleaved, void** out) {
+  return guard([&] {
+    if (cos) *out = box(ops_of(ops).kv_append(lb_of(cache), len, lb_of(x), &lb_of(cos), &lb_of(sin), &lb_of(pos), interleaved != 0));
+    else *out = box(ops_of(ops).kv_append(lb_of(cache), len, lb_of(x), nullptr, nullptr, nullptr, false));
+  });
+}
+int ugh_llama_attention_cached(void* ops, void* q, void* k, void* v, size_t s, float scale, void* cos, void* sin, void* pos, int interleaved, void** out) {
+  return guard([&] {
+    if (cos) *out = box(ops_of(ops).attention_cached(lb_of(q), lb_of(k), lb_of(v), s, scale, &lb_of(cos), &lb_of(sin), &lb_of(pos), interleaved != 0));
+    else *out = box(ops_of(ops).attention_cached(lb_of(q), lb_of(k), lb_of(v), s, scale, nullptr, nullptr, nullptr, false));
+  });
+}
 int ugh_llama_rms_norm(void* src, void* alpha, float eps, void** out) {
   return guard([&] { *out = box(ug_llama::rms_norm(lb_of(src), lb_of(alpha), eps)); });
 }
@@ -508,7 +523,7 @@ int ugh_llama_model_from_safetensors(void* d, void* ops, const ugh_llama_config*
 }
 void ugh_llama_model_free(void* m) { delete static_cast<ug_llama::Model*>(m); }
 int ugh_llama_model_set_fused_attention(void* m, int on) {
-  return guard([&] { static_cast<ug_llama::Model*>(m)->set_fused_attention(on != 0); });
+  return guard([&] { static_cast<ug_llama::Model*>(m)->set_fused_attention(on); });
 }
 int ugh_llama_generate(void* m, const int32_t* prompt, size_t n_prompt, size_t n_steps, int32_t* out_tokens, double* prefill_ms,
                        double* decode_ms, float* margins) {

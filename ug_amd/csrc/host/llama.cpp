@@ -162,6 +162,65 @@ struct HipOps : Ops {
     };
     return LB::custom(f, {src}, src.shape(), src.dtype(), src.device());
   }
+
+  // head sizes attention_cached has kernels for at any number of query positions
+  size_t kv_cache_capacity(size_t max_positions, size_t head_dim) const override {
+    return head_dim == 32 || head_dim == 64 || head_dim == 128 ? max_positions : 0;
+  }
+
+  LB kv_append(const LB& cache, size_t len, const LB& x, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const override {
+    if (cache.rank() != 4 || x.rank() != 3) bail("kv_append: expected cache [b, n, cap, d] and x [b, t, n * d]");
+    size_t b = cache.dims()[0], n = cache.dims()[1], cap = cache.dims()[2], d = cache.dims()[3], t = x.dims()[1];
+    if (x.dims()[0] != b || x.dims()[2] != n * d) bail("kv_append: mismatched shapes " + cache.shape().str() + " " + x.shape().str());
+    if (cap == len || d % 4 != 0) return Ops::kv_append(cache, len, x, cos, sin, pos, interleaved);
+    if (len + t > cap) bail("kv_append: " + std::to_string(len + t) + " rows exceed the cache capacity " + std::to_string(cap));
+    ughip_device* dev = hip_dev(x);
+    const bool with_rope = cos != nullptr;
+    int il = interleaved ? 1 : 0;
+    // in-place op: arguments first, the cache last (schedule.rs:404-413)
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != (with_rope ? 5u : 2u)) bail("kv_append: unexpected number of slices");
+      hip_check(ughip_kv_append(dev, hip_raw_slice(*vs.back()), hip_raw_slice(*vs[0]), b, n, cap, len, t, d, with_rope ? hip_raw_slice(*vs[1]) : nullptr,
+                                with_rope ? hip_raw_slice(*vs[2]) : nullptr, with_rope ? hip_raw_slice(*vs[3]) : nullptr, il),
+                "kv_append");
+    };
+    std::vector<LB> args = {x};
+    if (with_rope) {
+      args.push_back(*cos);
+      args.push_back(*sin);
+      args.push_back(*pos);
+    }
+    return cache.custom_ip(f, args);
+  }
+
+  LB attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float scale, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const override {
+    if (q.rank() != 3 || k.rank() != 4 || v.rank() != 4) bail("attention_cached: expected q [b, t, nh * d] and k, v [b, nkv, cap, d]");
+    size_t b = q.dims()[0], t = q.dims()[1], nkv = k.dims()[1], cap = k.dims()[2], d = k.dims()[3];
+    if (k.dims() != v.dims() || k.dims()[0] != b || d == 0 || q.dims()[2] % d != 0 || s > cap || t > s)
+      bail("attention_cached: mismatched shapes " + q.shape().str() + " " + k.shape().str() + " with " + std::to_string(s) + " keys");
+    size_t nh = q.dims()[2] / d;
+    const bool one = t == 1 && d >= 16 && d <= 256 && (d & (d - 1)) == 0 && s <= 12000;
+    const bool many = t > 1 && (d == 32 || d == 64 || d == 128);
+    if (!one && !many) return Ops::attention_cached(q, k, v, s, scale, cos, sin, pos, interleaved);
+    ughip_device* dev = hip_dev(q);
+    const bool with_rope = cos != nullptr;
+    int il = interleaved ? 1 : 0;
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != (with_rope ? 7u : 4u)) bail("attention_cached: unexpected number of slices");
+      ughip_slice* dst = hip_raw_slice(*vs.back());
+      hip_check(ughip_attention_cached(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), dst, b, nh, nkv, t, s, cap, d, scale,
+                                       with_rope ? hip_raw_slice(*vs[3]) : nullptr, with_rope ? hip_raw_slice(*vs[4]) : nullptr,
+                                       with_rope ? hip_raw_slice(*vs[5]) : nullptr, il),
+                "attention_cached");
+    };
+    std::vector<LB> args = {q, k, v};
+    if (with_rope) {
+      args.push_back(*cos);
+      args.push_back(*sin);
+      args.push_back(*pos);
+    }
+    return LB::custom(f, args, q.shape(), q.dtype(), q.device());
+  }
 };
 
 }  // namespace
@@ -231,6 +290,33 @@ LB Ops::attention_decode_flat(const LB& q, const LB& k, const LB& v, float scale
   LB qh = q.split_dim(2, nh, d).transpose(2, 1);
   if (cos) qh = interleaved ? rope_i(qh, *cos, *sin, *pos) : rope(qh, *cos, *sin, *pos);
   return attention_decode(qh, k, v, scale).transpose(2, 1).merge_dims(-2);
+}
+
+// model.rs:207-230 for t new positions, op by op (a cache that holds exactly `len` rows).
+LB Ops::kv_append(const LB& cache, size_t len, const LB& x, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const {
+  if (cache.rank() != 4 || x.rank() != 3) bail("kv_append: expected cache [b, n, cap, d] and x [b, t, n * d]");
+  if (cache.dims()[2] != len) bail("kv_append: this device appends by concatenation and needs a cache of exactly " + std::to_string(len) + " rows, got " + cache.shape().str());
+  size_t n = cache.dims()[1], d = cache.dims()[3];
+  LB rows = x.split_dim(2, n, d).transpose(2, 1);
+  if (cos) rows = interleaved ? rope_i(rows, *cos, *sin, *pos) : rope(rows, *cos, *sin, *pos);
+  return cat(cache, rows, 2);
+}
+
+// model.rs:207-210, 231-245, op by op.
+LB Ops::attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float scale, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const {
+  if (q.rank() != 3 || k.rank() != 4 || v.rank() != 4) bail("attention_cached: expected q [b, t, nh * d] and k, v [b, nkv, s, d]");
+  size_t t = q.dims()[1], d = k.dims()[3], nh = q.dims()[2] / d, nkv = k.dims()[1];
+  if (k.dims()[2] != s) bail("attention_cached: this device needs caches of exactly " + std::to_string(s) + " rows, got " + k.shape().str());
+  // the reference's causal_mask (cpu_ops.rs:33-56) is only right when the queries are the first t positions
+  if (t != 1 && t != s) bail("attention_cached: " + std::to_string(t) + " query positions after " + std::to_string(s - t) + " cached ones need a device kernel");
+  LB qh = q.split_dim(2, nh, d).transpose(2, 1);
+  if (cos) qh = interleaved ? rope_i(qh, *cos, *sin, *pos) : rope(qh, *cos, *sin, *pos);
+  LB kr = repeat(k, 1, nh / nkv);
+  LB vr = repeat(v, 1, nh / nkv);
+  LB att = qh.matmul_t(kr);
+  att = att.binary(BinaryOp::Mul, LB::cst(Const::f32(scale), Shape(), q.device()).broadcast(att.shape()));
+  att = t == 1 ? custom_softmax(att) : causal_softmax(att);
+  return att.matmul(vr).transpose(2, 1).merge_dims(-2);
 }
 
 std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16) {
@@ -360,12 +446,24 @@ Rope Rope::create(const Config& cfg, const DevicePtr& dev) {
   return Rope{mm.unary(UnaryOp::Cos), mm.unary(UnaryOp::Sin)};
 }
 
-// model.rs:188-197: zero-length caches.
-std::vector<Cache> Cache::create(const Config& cfg, const DevicePtr& dev) {
+// model.rs:188-197: zero-length caches; with a capacity, buffers of that many rows per head
+// (contents undefined until written) that attention appends to in place.
+std::vector<Cache> Cache::create(const Config& cfg, const DevicePtr& dev, size_t capacity) {
   std::vector<Cache> c;
   for (size_t i = 0; i < cfg.num_hidden_layers; ++i) {
-    Shape s({1, cfg.num_key_value_heads, 0, cfg.head_dim()});
-    c.push_back(Cache{LB::cst(Const::f32(0.f), s, dev), LB::cst(Const::f32(0.f), s, dev)});
+    Shape s({1, cfg.num_key_value_heads, capacity, cfg.head_dim()});
+    Cache one;
+    if (capacity) {
+      one.prev_k = LB::alloc_uninit(DType::F32, s, dev);
+      one.prev_v = LB::alloc_uninit(DType::F32, s, dev);
+      one.prev_k.maybe_allocate_uninit();
+      one.prev_v.maybe_allocate_uninit();
+    } else {
+      one.prev_k = LB::cst(Const::f32(0.f), s, dev);
+      one.prev_v = LB::cst(Const::f32(0.f), s, dev);
+    }
+    one.capacity = capacity;
+    c.push_back(std::move(one));
   }
   return c;
 }
@@ -406,6 +504,20 @@ LB Model::attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache) c
   LB q = xs.matmul_t(l.q_proj);
   LB k = xs.matmul_t(l.k_proj);
   LB v = xs.matmul_t(l.v_proj);
+  if (fused_attention_ >= 2) {
+    // rows go from the projections into the caches (in place when they were preallocated) and
+    // the attention kernel reads them there; the result comes back in the layout o_proj reads
+    const size_t len = cache.capacity ? cache.len : cache.prev_k.dims()[2];
+    LB kc = ops_->kv_append(cache.prev_k, len, k, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved);
+    LB vc = ops_->kv_append(cache.prev_v, len, v, nullptr, nullptr, nullptr, false);
+    if (cache.capacity == 0) {
+      cache.prev_k = kc;
+      cache.prev_v = vc;
+    }  // else: kc and vc are this step's in-place writes of the storage prev_k / prev_v keep naming
+    cache.len = len + seq_len;
+    LB out = ops_->attention_cached(q, kc, vc, cache.len, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved);
+    return out.matmul_t(l.o_proj);
+  }
   if (fused_attention_ && seq_len == 1) {
     // one new position: rows go from the projections into the caches and the attention kernel
     // without the split/transpose copies, and the result comes back in the layout o_proj reads
@@ -454,6 +566,10 @@ LB Model::mlp(const Layer& l, const LB& xs) const {
   LB xs2 = xs.matmul_t(l.up_proj);
   xs1 = silu(xs1);
   return xs1.binary(BinaryOp::Mul, xs2).matmul_t(l.down_proj);
+}
+
+std::vector<Cache> Model::new_cache() const {
+  return Cache::create(cfg_, dev_, fused_attention_ >= 2 ? ops_->kv_cache_capacity(cfg_.max_position_embeddings, cfg_.head_dim()) : 0);
 }
 
 // model.rs:259-269, 365-373
@@ -508,7 +624,7 @@ std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32
   const DevicePtr& dev = model.device();
   if (prompt.empty()) bail("empty prompt");
   if (prompt.size() + n_steps > cfg.max_position_embeddings) bail("prompt + steps exceed max_position_embeddings");
-  std::vector<Cache> cache = Cache::create(cfg, dev);
+  std::vector<Cache> cache = model.new_cache();
   CompilationCache ccache;
   std::vector<int32_t> out;
   std::vector<float> logits;

@@ -34,6 +34,25 @@ struct Ops {
   // q [b, 1, nh * d] (rotated first when a table is given), k and v [b, nkv, s, d] -> [b, 1, nh * d].
   virtual LB attention_decode_flat(const LB& q, const LB& k, const LB& v, float scale, const LB* cos, const LB* sin, const LB* pos,
                                    bool interleaved) const;
+
+  // Caches that are written in place.  kv_cache_capacity: rows to preallocate per head for a model
+  // of max_positions and this head size (0 = this device grows its caches by concatenation, as
+  // model.rs:226-230 does).
+  virtual size_t kv_cache_capacity(size_t max_positions, size_t head_dim) const {
+    (void)max_positions;
+    (void)head_dim;
+    return 0;
+  }
+  // cache [b, n, cap, d] holds `len` rows per head; x [b, t, n * d] comes from the k or v projection
+  // and is rotated at table rows pos[0] + i when a table is given.  Returns the cache with rows
+  // len .. len + t - 1 written: the same storage when cap > len (in place), otherwise (cap == len,
+  // the default) a new buffer [b, n, len + t, d] built with rope and cat.
+  virtual LB kv_append(const LB& cache, size_t len, const LB& x, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const;
+  // Causal attention of q [b, t, nh * d] (rotated first when a table is given) over the first s rows
+  // of k and v [b, nkv, cap, d]; query i sees keys 0 .. s - t + i.  Returns [b, t, nh * d].  The
+  // default composes model.rs:207-210, 231-245 and needs cap == s and, for t > 1, s == t.
+  virtual LB attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float scale, const LB* cos, const LB* sin, const LB* pos,
+                              bool interleaved) const;
 };
 
 // The HIP implementation (counterpart of ug-llama/src/cuda_ops.rs).
@@ -86,17 +105,26 @@ struct Rope {
 // model.rs:183-198
 struct Cache {
   LB prev_k, prev_v;
-  static std::vector<Cache> create(const Config& cfg, const ug::DevicePtr& dev);
+  // Used by the in-place mode only: rows written so far, rows allocated (0 = prev_k / prev_v have
+  // exactly the rows written, the reference's representation).
+  size_t len = 0, capacity = 0;
+  static std::vector<Cache> create(const Config& cfg, const ug::DevicePtr& dev, size_t capacity = 0);
 };
 
 // model.rs:299-373
 class Model {
  public:
   Model(const Config& cfg, bool custom_softmax, WeightSource& weights, const ug::DevicePtr& dev, std::shared_ptr<Ops> ops);
-  // Route attention through Ops::causal_softmax (prefill) and Ops::attention_decode (one query
-  // position) instead of the op-by-op graph.  Off by default: the graph is then the reference's.
-  void set_fused_attention(bool on) { fused_attention_ = on; }
-  bool fused_attention() const { return fused_attention_; }
+  // 0 (default): the reference's op-by-op graph.
+  // 1: attention through Ops::causal_softmax (prefill) and Ops::rope_append +
+  //    Ops::attention_decode_flat (one query position); caches still grow by copying.
+  // 2: Ops::kv_append + Ops::attention_cached for any number of positions; with a device that
+  //    preallocates (Ops::kv_cache_capacity) the caches are written in place and scores never
+  //    reach memory.
+  void set_fused_attention(int level) { fused_attention_ = level; }
+  int fused_attention() const { return fused_attention_; }
+  // Caches of the kind fwd() expects at the current fusion level.
+  std::vector<Cache> new_cache() const;
   LB fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const;
   const Config& config() const { return cfg_; }
   const ug::DevicePtr& device() const { return dev_; }
@@ -112,7 +140,7 @@ class Model {
   LB mlp(const Layer& l, const LB& xs) const;
   Config cfg_;
   bool custom_softmax_;
-  bool fused_attention_ = false;
+  int fused_attention_ = 0;
   ug::DevicePtr dev_;
   std::shared_ptr<Ops> ops_;
   LB embedding_, ln_f_;

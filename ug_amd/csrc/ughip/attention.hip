@@ -99,7 +99,8 @@ __global__ void __launch_bounds__(256) causal_softmax_generic(const float* __res
 }
 
 // ---- single-query attention -----------------------------------------------------------------------
-// One workgroup of 1024 threads per query head.  q: [b, nh, d]; k, v: [b, nkv, s, d]; dst: [b, nh, d].
+// One workgroup of 1024 threads per query head.  q: [b, nh, d]; k, v: [b, nkv, s, d] (heads
+// kv_head_stride elements apart: s * d, or capacity * d for a preallocated cache); dst: [b, nh, d].
 // LPK = d / 4 lanes share one key row (one 128-bit load each, a row is one contiguous 4*d bytes);
 // 1024 / LPK keys are in flight per step and four steps per loop trip, because at batch 1 this
 // kernel is a chain of L2 round trips, not a bandwidth problem.  Scores and probabilities live in
@@ -121,8 +122,8 @@ __device__ __forceinline__ float att_block_reduce(float v, float* lds16) {
 }
 
 __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
-                                                                       float* __restrict__ dst, int nh, int nkv, int s, int d, float scale,
-                                                                       const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                                       float* __restrict__ dst, int nh, int nkv, int s, size_t kv_head_stride, int d,
+                                                                       float scale, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                                                        const int* __restrict__ pos, size_t table_len, int interleaved) {
   extern __shared__ __attribute__((aligned(16))) float sc[];  // s scores, then ATT_WAVES * 64 float4 of reduction space
   __shared__ float lds16[ATT_WAVES];
@@ -132,8 +133,8 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
   const int c4 = tid % lpk, slot = tid / lpk;
   const int bh = blockIdx.x, b = bh / nh, h = bh % nh, kvh = h / (nh / nkv);
   const float4* q4 = reinterpret_cast<const float4*>(q + (size_t)bh * d);
-  const float4* k4 = reinterpret_cast<const float4*>(k + ((size_t)b * nkv + kvh) * (size_t)s * d);
-  const float4* v4 = reinterpret_cast<const float4*>(v + ((size_t)b * nkv + kvh) * (size_t)s * d);
+  const float4* k4 = reinterpret_cast<const float4*>(k + ((size_t)b * nkv + kvh) * kv_head_stride);
+  const float4* v4 = reinterpret_cast<const float4*>(v + ((size_t)b * nkv + kvh) * kv_head_stride);
 
   float4 qv;
   if (cos_t) {
@@ -271,6 +272,263 @@ __global__ void __launch_bounds__(256) rope_append_kernel(const float* __restric
   reinterpret_cast<float4*>(dst)[g] = out;
 }
 
+// ---- cache append in place ------------------------------------------------------------------------
+// cache [b, n, cap, d], x [b, t, n * d]: cache[b, h, s_old + i, :] = x[b, i, h * d .. (h + 1) * d),
+// rotated at table row pos[0] + i when a table is given.  One thread per float4 of x (d % 4 == 0).
+__global__ void __launch_bounds__(256) kv_append_kernel(float* __restrict__ cache, const float* __restrict__ x, size_t n4, int t, int n, int d, size_t cap,
+                                                        int s_old, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                        const int* __restrict__ pos, size_t table_len, int interleaved) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n4) return;
+  const int d4 = d >> 2;
+  const int c4 = (int)(g % d4);
+  size_t rest = g / d4;
+  const int h = (int)(rest % n);
+  rest /= n;
+  const int i = (int)(rest % t);
+  const size_t b = rest / t;
+  const float* xr = x + ((b * t + i) * n + h) * (size_t)d;
+  float4 out;
+  if (!cos_t) {
+    out = reinterpret_cast<const float4*>(xr)[c4];
+  } else {
+    const int half = d >> 1;
+    const long long p = (long long)pos[0] + i;
+    float o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int c = c4 * 4 + e;  // output element; its pair and whether it is the pair's first element
+      const int pr = interleaved ? c >> 1 : (c < half ? c : c - half);
+      const bool first = interleaved ? (c & 1) == 0 : c < half;
+      const int i1 = interleaved ? 2 * pr : pr, i2 = interleaved ? 2 * pr + 1 : pr + half;
+      const size_t ics = (size_t)p * half + pr;
+      const bool ok = p >= 0 && ics < table_len;
+      const float cs = ok ? cos_t[ics] : NAN, sn = ok ? sin_t[ics] : NAN;
+      const float x1 = xr[i1], x2 = xr[i2];
+      o[e] = first ? x1 * cs - x2 * sn : x1 * sn + x2 * cs;
+    }
+    out = make_float4(o[0], o[1], o[2], o[3]);
+  }
+  reinterpret_cast<float4*>(cache + ((b * n + h) * cap + (size_t)s_old + i) * d)[c4] = out;
+}
+
+// ---- causal attention over a cache, many query positions ------------------------------------------
+// q, dst: [b, t, nh * D]; k, v: [b, nkv, cap, D] with rows 0 .. s-1 valid.  Query i sits at position
+// s - t + i and sees keys 0 .. s - t + i (model.rs:231-244 with the mask of cpu_ops.rs:33-56 moved to
+// that offset).  Scores never reach memory: a group of 4 waves owns 32 queries of one head, its waves
+// take every fourth block of 32 keys and keep a running (max, sum, output) per query, merged at the
+// end in wave order.
+//
+// Everything is v_mfma_f32_32x32x2_f32 on transposed products, so that a lane owns ONE query
+// (column lane % 32) and the softmax statistics never cross lanes except between the two halves:
+//   S^T = K Q^T   (M = keys, N = queries, K = D): A = K[key = lane % 32][c], B = Q[query = lane % 32][c]
+//                 with c = j for lanes 0-31 and D/2 + j for lanes 32-63 in MFMA j -- both operands are
+//                 D/2 consecutive floats per lane, loaded once per block (K) or once per kernel (Q).
+//   O^T = V^T P^T (M = D, N = queries, K = keys): accumulator register r of S^T holds key
+//                 8 (r / 4) + 4 (lane / 32) + r % 4, which is exactly the pair of keys MFMA r consumes
+//                 (lower half one key, upper half the other): P feeds back as the B operand without
+//                 any data movement; A = V[that key][lane % 32 + 32 * block].
+typedef float att_f32x16 __attribute__((ext_vector_type(16)));
+
+template <int D, int GROUPS>
+__global__ void __launch_bounds__(256 * GROUPS) attention_prefill_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
+                                                                float* __restrict__ dst, int nh, int nkv, int t, int s, size_t cap, float scale,
+                                                                const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                                const int* __restrict__ pos, size_t table_len, int interleaved) {
+  constexpr int H = D / 2, DB = D / 32;  // floats of q / k per lane; 32-wide blocks of the head dimension
+  __shared__ float merge_ml_all[GROUPS][3][2][64];
+  __shared__ float merge_o_all[GROUPS][3][DB * 16][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = (tid >> 6) & 3, group = tid >> 8;
+  const int col = lane & 31, hh = lane >> 5;
+  const int bh = blockIdx.y, b = bh / nh, head = bh % nh, kvh = head / (nh / nkv);
+  // GROUPS == 2: a workgroup takes the query blocks x and n - 1 - x, one per group of 4 waves, so
+  // that under the causal mask every workgroup has the same number of key blocks to go through
+  const int n_qb = (t + 31) / 32;
+  const int qb = GROUPS == 1 ? n_qb - 1 - (int)blockIdx.x : (group == 0 ? n_qb - 1 - (int)blockIdx.x : (int)blockIdx.x);
+  const bool idle = GROUPS == 2 && group == 1 && qb == n_qb - 1 - qb;  // odd count: the middle block belongs to group 0
+  float (*merge_ml)[2][64] = merge_ml_all[group];
+  float (*merge_o)[64] = merge_o_all[group][0];
+  const int q0 = qb * 32;
+  const int qi = min(q0 + col, t - 1);        // rows past t repeat the last query and are not stored
+  const int q_pos = s - t + qi;               // last key this query sees
+  const int last_pos = s - t + min(q0 + 31, t - 1);
+  const float* kb_ptr = k + ((size_t)b * nkv + kvh) * cap * D;
+  const float* vb_ptr = v + ((size_t)b * nkv + kvh) * cap * D;
+
+  // K operand of a block: D/2 consecutive floats of key row key0 + col.  Rows past s repeat row s-1
+  // (they are masked, and a block index past the end is harmless).
+  auto load_k = [&](int kb, float (&kr)[H]) {
+    const float* krow = kb_ptr + (size_t)min(kb * 32 + col, s - 1) * D + hh * H;
+#pragma unroll
+    for (int j = 0; j < H; j += 4) {
+      const float4 x = *reinterpret_cast<const float4*>(krow + j);
+      kr[j] = x.x, kr[j + 1] = x.y, kr[j + 2] = x.z, kr[j + 3] = x.w;
+    }
+  };
+
+  // the first K block is requested before the query row, whose table row hangs off a load of pos
+  float kn[H];
+  load_k(wave, kn);
+
+  // this lane's half of its (rotated) query row
+  float qr[H];
+  {
+    const float* qrow = q + ((size_t)b * t + qi) * ((size_t)nh * D) + (size_t)head * D;
+    if (!cos_t) {
+#pragma unroll
+      for (int j = 0; j < H; j += 4) {
+        const float4 x = *reinterpret_cast<const float4*>(qrow + hh * H + j);
+        qr[j] = x.x, qr[j + 1] = x.y, qr[j + 2] = x.z, qr[j + 3] = x.w;
+      }
+    } else {
+      // table row pos[0] + qi, read with 128-bit loads from a clamped address; a row outside the
+      // table turns the query into NaN (what the bounds error of the op-by-op path would flag)
+      const long long p = (long long)pos[0] + qi;
+      const bool ok = p >= 0 && (size_t)(p + 1) * H <= table_len;
+      const size_t row = ok ? (size_t)p * H : 0;
+      if (interleaved) {
+        // pairs (2i, 2i + 1): both elements and their table entry lie in this lane's half
+        float xh[H], ch[H / 2], sh[H / 2];
+#pragma unroll
+        for (int j = 0; j < H; j += 4) {
+          const float4 x = *reinterpret_cast<const float4*>(qrow + hh * H + j);
+          xh[j] = x.x, xh[j + 1] = x.y, xh[j + 2] = x.z, xh[j + 3] = x.w;
+        }
+#pragma unroll
+        for (int j = 0; j < H / 2; j += 4) {
+          const float4 c = *reinterpret_cast<const float4*>(cos_t + row + hh * (H / 2) + j);
+          const float4 sn = *reinterpret_cast<const float4*>(sin_t + row + hh * (H / 2) + j);
+          ch[j] = c.x, ch[j + 1] = c.y, ch[j + 2] = c.z, ch[j + 3] = c.w;
+          sh[j] = sn.x, sh[j + 1] = sn.y, sh[j + 2] = sn.z, sh[j + 3] = sn.w;
+        }
+#pragma unroll
+        for (int j = 0; j < H; ++j) {
+          const float x1 = xh[j & ~1], x2 = xh[j | 1], cs = ch[j >> 1], sn = sh[j >> 1];
+          qr[j] = (j & 1) ? x1 * sn + x2 * cs : x1 * cs - x2 * sn;
+        }
+      } else {
+        // pairs (i, i + D/2): the lower half of the lanes produces x1 c - x2 s, the upper x1 s + x2 c
+        float xa[H], xb[H], ch[H], sh[H];
+#pragma unroll
+        for (int j = 0; j < H; j += 4) {
+          const float4 a = *reinterpret_cast<const float4*>(qrow + j);
+          const float4 bq = *reinterpret_cast<const float4*>(qrow + H + j);
+          const float4 c = *reinterpret_cast<const float4*>(cos_t + row + j);
+          const float4 sn = *reinterpret_cast<const float4*>(sin_t + row + j);
+          xa[j] = a.x, xa[j + 1] = a.y, xa[j + 2] = a.z, xa[j + 3] = a.w;
+          xb[j] = bq.x, xb[j + 1] = bq.y, xb[j + 2] = bq.z, xb[j + 3] = bq.w;
+          ch[j] = c.x, ch[j + 1] = c.y, ch[j + 2] = c.z, ch[j + 3] = c.w;
+          sh[j] = sn.x, sh[j + 1] = sn.y, sh[j + 2] = sn.z, sh[j + 3] = sn.w;
+        }
+#pragma unroll
+        for (int j = 0; j < H; ++j) qr[j] = hh ? xa[j] * sh[j] + xb[j] * ch[j] : xa[j] * ch[j] - xb[j] * sh[j];
+      }
+      if (!ok) {
+#pragma unroll
+        for (int j = 0; j < H; ++j) qr[j] = NAN;
+      }
+    }
+  }
+
+  float m_run = -INFINITY, l_half = 0.f;  // l_half: sum over the keys this half of the query's lanes holds
+  att_f32x16 o[DB];
+#pragma unroll
+  for (int e = 0; e < DB; ++e)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[e][r] = 0.f;
+
+  const int n_blocks = idle ? 0 : last_pos / 32 + 1;
+  // K of the next block is in flight while this one is multiplied; V of this block is requested at
+  // the top and first needed after the scores and their exponentials
+  for (int kb = wave; kb < n_blocks; kb += 4) {
+    const int key0 = kb * 32;
+    float kr[H], vr[DB][16];
+#pragma unroll
+    for (int j = 0; j < H; ++j) kr[j] = kn[j];
+    // V operand of MFMA r: row key0 + 8 (r / 4) + 4 hh + r % 4, column col + 32 e
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float* vrow = vb_ptr + (size_t)min(key0 + (r >> 2) * 8 + hh * 4 + (r & 3), s - 1) * D + col;
+#pragma unroll
+      for (int e = 0; e < DB; ++e) vr[e][r] = vrow[e * 32];
+    }
+    load_k(kb + 4, kn);
+    __builtin_amdgcn_sched_barrier(0);  // keeps the loads up here instead of next to their uses
+    att_f32x16 sc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+#pragma unroll
+    for (int j = 0; j < H; ++j) sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j], qr[j], sc, 0, 0, 0);
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int key = key0 + (r >> 2) * 8 + hh * 4 + (r & 3);
+      sc[r] = key <= q_pos ? sc[r] * scale : -INFINITY;
+      mx = fmaxf(mx, sc[r]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // no key seen yet: every exp below is exp(-inf) = 0
+    const float alpha = expf(m_run - m_use);
+    m_run = m_new;
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      sc[r] = expf(sc[r] - m_use);
+      psum += sc[r];
+    }
+    l_half = l_half * alpha + psum;
+#pragma unroll
+    for (int e = 0; e < DB; ++e) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[e][r] *= alpha;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[e][r], sc[r], o[e], 0, 0, 0);
+    }
+  }
+
+  // merge the four waves' partial results in wave order
+  if (wave != 0) {
+    merge_ml[wave - 1][0][lane] = m_run;
+    merge_ml[wave - 1][1][lane] = l_half;
+#pragma unroll
+    for (int e = 0; e < DB; ++e)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) merge_o[(wave - 1) * DB * 16 + e * 16 + r][lane] = o[e][r];
+  }
+  __syncthreads();
+  if (wave != 0 || idle) return;
+  float m_tot = m_run;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) m_tot = fmaxf(m_tot, merge_ml[w][0][lane]);
+  // key 0 is visible to every query and belongs to wave 0's first block: m_tot is finite
+  float f = expf(m_run - m_tot);
+  float l_tot = l_half * f;
+#pragma unroll
+  for (int e = 0; e < DB; ++e)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[e][r] *= f;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+    f = expf(merge_ml[w][0][lane] - m_tot);
+    l_tot += merge_ml[w][1][lane] * f;
+#pragma unroll
+    for (int e = 0; e < DB; ++e)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[e][r] += merge_o[w * DB * 16 + e * 16 + r][lane] * f;
+  }
+  l_tot += __shfl_xor(l_tot, 32, 64);
+  if (q0 + col < t) {
+    float* orow = dst + ((size_t)b * t + qi) * ((size_t)nh * D) + (size_t)head * D;
+#pragma unroll
+    for (int e = 0; e < DB; ++e)
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+        *reinterpret_cast<float4*>(orow + e * 32 + a * 8 + hh * 4) =
+            make_float4(o[e][a * 4] / l_tot, o[e][a * 4 + 1] / l_tot, o[e][a * 4 + 2] / l_tot, o[e][a * 4 + 3] / l_tot);
+  }
+}
+
 int check_f32(const ughip_slice* s, size_t need, const char* what) {
   if (!s) return set_error(UGHIP_ERR_INVALID, "%s: null slice", what);
   if (s->dtype != UGHIP_F32) return set_error(UGHIP_ERR_INVALID, "%s: unexpected dtype %s, expected F32", what, dtype_name(s->dtype));
@@ -319,9 +577,11 @@ int ughip_attention_decode(ughip_device* dev, const ughip_slice* q, const ughip_
   return ughip_attention_decode_rope(dev, q, k, v, dst, b, n_heads, n_kv_heads, s, d, scale, nullptr, nullptr, nullptr, 0);
 }
 
-int ughip_attention_decode_rope(ughip_device* dev, const ughip_slice* q, const ughip_slice* k, const ughip_slice* v, ughip_slice* dst, size_t b,
-                                size_t n_heads, size_t n_kv_heads, size_t s, size_t d, float scale, const ughip_slice* cos, const ughip_slice* sin,
-                                const ughip_slice* pos, int interleaved) {
+namespace {
+// One query position per head against s keys of caches whose heads are cap rows apart.
+int attention_decode_launch(ughip_device* dev, const ughip_slice* q, const ughip_slice* k, const ughip_slice* v, ughip_slice* dst, size_t b, size_t n_heads,
+                            size_t n_kv_heads, size_t s, size_t cap, size_t d, float scale, const ughip_slice* cos, const ughip_slice* sin,
+                            const ughip_slice* pos, int interleaved) {
   if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
   const bool rope = cos || sin || pos;
   if (rope)
@@ -330,25 +590,31 @@ int ughip_attention_decode_rope(ughip_device* dev, const ughip_slice* q, const u
     return set_error(UGHIP_ERR_INVALID, "attention_decode: %zu heads are not a multiple of %zu kv heads", n_heads, n_kv_heads);
   if (d < 16 || d > 256 || (d & (d - 1)) != 0) return set_error(UGHIP_ERR_INVALID, "attention_decode: head size %zu is not a power of two in 16..256", d);
   if (s == 0) return set_error(UGHIP_ERR_INVALID, "attention_decode: empty key sequence");
+  if (s > cap) return set_error(UGHIP_ERR_INVALID, "attention_decode: %zu keys exceed the cache capacity %zu", s, cap);
   if (s > 12000) return set_error(UGHIP_ERR_INVALID, "attention_decode: %zu keys exceed the 12000 this kernel holds in LDS", s);
   if (int rc = check_f32(q, b * n_heads * d, "attention_decode q")) return rc;
-  if (int rc = check_f32(k, b * n_kv_heads * s * d, "attention_decode k")) return rc;
-  if (int rc = check_f32(v, b * n_kv_heads * s * d, "attention_decode v")) return rc;
+  if (int rc = check_f32(k, b * n_kv_heads * cap * d, "attention_decode k")) return rc;
+  if (int rc = check_f32(v, b * n_kv_heads * cap * d, "attention_decode v")) return rc;
   if (int rc = check_f32(dst, b * n_heads * d, "attention_decode dst")) return rc;
   if (dst == q || dst == k || dst == v) return set_error(UGHIP_ERR_INVALID, "attention_decode: dst aliases an input");
   if (b * n_heads == 0) return UGHIP_OK;
   if (b * n_heads > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "attention_decode: too many heads");
   if (int rc = device_activate(dev)) return rc;
   const size_t lds = (s + 3 + ATT_WAVES * 64 * 4) * sizeof(float);  // scores, alignment slack, one float4 per lane slot of every wave
-  attention_decode_kernel<<<(unsigned)(b * n_heads), ATT_THREADS, lds, dev->stream>>>(static_cast<const float*>(q->ptr), static_cast<const float*>(k->ptr),
-                                                                              static_cast<const float*>(v->ptr), static_cast<float*>(dst->ptr), (int)n_heads,
-                                                                              (int)n_kv_heads, (int)s, (int)d, scale,
-                                                                              rope ? static_cast<const float*>(cos->ptr) : nullptr,
-                                                                              rope ? static_cast<const float*>(sin->ptr) : nullptr,
-                                                                              rope ? static_cast<const int*>(pos->ptr) : nullptr,
-                                                                              rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved);
+  attention_decode_kernel<<<(unsigned)(b * n_heads), ATT_THREADS, lds, dev->stream>>>(
+      static_cast<const float*>(q->ptr), static_cast<const float*>(k->ptr), static_cast<const float*>(v->ptr), static_cast<float*>(dst->ptr), (int)n_heads,
+      (int)n_kv_heads, (int)s, cap * d, (int)d, scale, rope ? static_cast<const float*>(cos->ptr) : nullptr,
+      rope ? static_cast<const float*>(sin->ptr) : nullptr, rope ? static_cast<const int*>(pos->ptr) : nullptr,
+      rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
+}
+}  // namespace
+
+int ughip_attention_decode_rope(ughip_device* dev, const ughip_slice* q, const ughip_slice* k, const ughip_slice* v, ughip_slice* dst, size_t b,
+                                size_t n_heads, size_t n_kv_heads, size_t s, size_t d, float scale, const ughip_slice* cos, const ughip_slice* sin,
+                                const ughip_slice* pos, int interleaved) {
+  return attention_decode_launch(dev, q, k, v, dst, b, n_heads, n_kv_heads, s, s, d, scale, cos, sin, pos, interleaved);
 }
 
 int ughip_rope_append(ughip_device* dev, const ughip_slice* cache, const ughip_slice* x, ughip_slice* dst, size_t bh, size_t s_old, size_t d,
@@ -374,6 +640,77 @@ int ughip_rope_append(ughip_device* dev, const ughip_slice* cache, const ughip_s
       s_old ? static_cast<const float*>(cache->ptr) : nullptr, static_cast<const float*>(x->ptr), static_cast<float*>(dst->ptr), n4, (int)s_old, (int)d,
       rope ? static_cast<const float*>(cos->ptr) : nullptr, rope ? static_cast<const float*>(sin->ptr) : nullptr,
       rope ? static_cast<const int*>(pos->ptr) : nullptr, rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved);
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+int ughip_kv_append(ughip_device* dev, ughip_slice* cache, const ughip_slice* x, size_t b, size_t n, size_t cap, size_t s_old, size_t t, size_t d,
+                    const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos, int interleaved) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  if (d == 0 || d % 4 != 0) return set_error(UGHIP_ERR_INVALID, "kv_append: head size %zu is not a multiple of 4", d);
+  const bool rope = cos || sin || pos;
+  if (rope) {
+    if (d % 2 != 0) return set_error(UGHIP_ERR_INVALID, "kv_append: odd head size %zu", d);
+    if (int rc = check_rope_table(cos, sin, pos, d, "kv_append")) return rc;
+  }
+  if (s_old + t > cap) return set_error(UGHIP_ERR_BOUNDS, "kv_append: rows %zu..%zu do not fit a cache of %zu rows", s_old, s_old + t, cap);
+  if (int rc = check_f32(cache, b * n * cap * d, "kv_append cache")) return rc;
+  if (int rc = check_f32(x, b * t * n * d, "kv_append x")) return rc;
+  if (cache == x) return set_error(UGHIP_ERR_INVALID, "kv_append: x aliases the cache");
+  const size_t n4 = b * t * n * d / 4;
+  if (n4 == 0) return UGHIP_OK;
+  if (cap > 0x7fffffffull || t > 0x7fffffffull || n > 0x7fffffffull || d > 0x7fffffffull || n4 > (size_t)0x7fffffff * 256)
+    return set_error(UGHIP_ERR_INVALID, "kv_append: shape too large");
+  if (int rc = device_activate(dev)) return rc;
+  kv_append_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, dev->stream>>>(
+      static_cast<float*>(cache->ptr), static_cast<const float*>(x->ptr), n4, (int)t, (int)n, (int)d, cap, (int)s_old,
+      rope ? static_cast<const float*>(cos->ptr) : nullptr, rope ? static_cast<const float*>(sin->ptr) : nullptr,
+      rope ? static_cast<const int*>(pos->ptr) : nullptr, rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved);
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, const ughip_slice* k, const ughip_slice* v, ughip_slice* dst, size_t b, size_t n_heads,
+                           size_t n_kv_heads, size_t t, size_t s, size_t cap, size_t d, float scale, const ughip_slice* cos, const ughip_slice* sin,
+                           const ughip_slice* pos, int interleaved) {
+  if (t == 1) return attention_decode_launch(dev, q, k, v, dst, b, n_heads, n_kv_heads, s, cap, d, scale, cos, sin, pos, interleaved);
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  const bool rope = cos || sin || pos;
+  if (rope)
+    if (int rc = check_rope_table(cos, sin, pos, d, "attention_cached")) return rc;
+  if (n_kv_heads == 0 || n_heads % n_kv_heads != 0)
+    return set_error(UGHIP_ERR_INVALID, "attention_cached: %zu heads are not a multiple of %zu kv heads", n_heads, n_kv_heads);
+  if (d != 32 && d != 64 && d != 128)
+    return set_error(UGHIP_ERR_UNSUPPORTED, "attention_cached: head size %zu (32, 64 and 128 are built for more than one query position)", d);
+  if (t == 0 || s < t) return set_error(UGHIP_ERR_INVALID, "attention_cached: %zu query positions need at least as many keys, got %zu", t, s);
+  if (s > cap) return set_error(UGHIP_ERR_INVALID, "attention_cached: %zu keys exceed the cache capacity %zu", s, cap);
+  if (int rc = check_f32(q, b * t * n_heads * d, "attention_cached q")) return rc;
+  if (int rc = check_f32(k, b * n_kv_heads * cap * d, "attention_cached k")) return rc;
+  if (int rc = check_f32(v, b * n_kv_heads * cap * d, "attention_cached v")) return rc;
+  if (int rc = check_f32(dst, b * t * n_heads * d, "attention_cached dst")) return rc;
+  if (dst == q || dst == k || dst == v) return set_error(UGHIP_ERR_INVALID, "attention_cached: dst aliases an input");
+  if (b * n_heads == 0) return UGHIP_OK;
+  if (b * n_heads > 65535 || s > 0x7fffffffull || cap > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "attention_cached: shape too large");
+  if (int rc = device_activate(dev)) return rc;
+  const unsigned n_qb = (unsigned)((t + 31) / 32);
+  const float* cp = rope ? static_cast<const float*>(cos->ptr) : nullptr;
+  const float* sp = rope ? static_cast<const float*>(sin->ptr) : nullptr;
+  const int* pp = rope ? static_cast<const int*>(pos->ptr) : nullptr;
+  const size_t tl = rope ? (cos->len < sin->len ? cos->len : sin->len) : 0;
+  const float* qp = static_cast<const float*>(q->ptr);
+  const float* kp = static_cast<const float*>(k->ptr);
+  const float* vp = static_cast<const float*>(v->ptr);
+  float* op = static_cast<float*>(dst->ptr);
+  const int inh = (int)n_heads, inkv = (int)n_kv_heads, it = (int)t, is = (int)s;
+  // Two query blocks per workgroup of 8 waves (equal work under the causal mask) once one block per
+  // workgroup would give every CU two workgroups anyway; d = 128 needs the whole register file for 4 waves.
+  const dim3 paired((n_qb + 1) / 2, (unsigned)(b * n_heads)), single(n_qb, (unsigned)(b * n_heads));
+  const bool pair = d <= 64 && (size_t)n_qb * b * n_heads >= 512;
+  if (d == 32 && pair) attention_prefill_kernel<32, 2><<<paired, 512, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, scale, cp, sp, pp, tl, interleaved);
+  else if (d == 32) attention_prefill_kernel<32, 1><<<single, 256, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, scale, cp, sp, pp, tl, interleaved);
+  else if (d == 64 && pair) attention_prefill_kernel<64, 2><<<paired, 512, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, scale, cp, sp, pp, tl, interleaved);
+  else if (d == 64) attention_prefill_kernel<64, 1><<<single, 256, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, scale, cp, sp, pp, tl, interleaved);
+  else attention_prefill_kernel<128, 1><<<single, 256, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, scale, cp, sp, pp, tl, interleaved);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
 }
