@@ -272,7 +272,8 @@ def llama_decode(dev, n_prompt=128, n_steps=128, fused_attention=0):
     Fresh buffers are not zero-filled here (every kernel of the model writes its whole output; the
     ids are the same either way, which the GPU tests check).  fused_attention: 0 = the reference's
     op-by-op graph; 1 = ughip_causal_softmax_rows / ughip_rope_append / ughip_attention_decode;
-    2 = caches written in place (ughip_kv_append) and ughip_attention_cached for prefill and decode."""
+    2 = caches written in place (ughip_kv_append) and ughip_attention_cached for prefill and decode;
+    3 = 2 plus packed q|k|v, gate/up + SwiGLU and residual projections (ughip_gemv_multi / _gate_up / _add)."""
     import ug_amd
     from ug_amd import rng
     cfg = ug_amd.LlamaConfig()
@@ -360,7 +361,8 @@ def main():
         except Exception as e:  # noqa: BLE001
             line["extras"] = {"error": f"{type(e).__name__}: {e}"}
     if not (args.no_llama or args.headline_only):
-        for key, fused in (("llama_decode_f32", 0), ("llama_decode_f32_fused_attention", 1), ("llama_decode_f32_inplace_cache", 2)):
+        for key, fused in (("llama_decode_f32", 0), ("llama_decode_f32_fused_attention", 1), ("llama_decode_f32_inplace_cache", 2),
+                           ("llama_decode_f32_fused_projections", 3)):
             try:
                 line.setdefault("extras", {})[key] = llama_decode(dev, fused_attention=fused)
             except Exception as e:  # noqa: BLE001

@@ -256,9 +256,13 @@ int ughip_rope_append(ughip_device* dev, const ughip_slice* cache, const ughip_s
  * which copies the whole cache every step): cache [b, n, cap, d] is preallocated for cap
  * positions; rows s_old .. s_old + t - 1 of every head receive x [b, t, n * d] (the layout the
  * k / v projections write), rotated at table rows pos[0] + i when cos/sin/pos are given.
- * s_old + t <= cap, d % 4 == 0.  Rows past s_old + t are left untouched. */
-int ughip_kv_append(ughip_device* dev, ughip_slice* cache, const ughip_slice* x, size_t b,
-                    size_t n, size_t cap, size_t s_old, size_t t, size_t d,
+ * s_old + t <= cap, d % 4 == 0.  Rows past s_old + t are left untouched.
+ * x may be a column range of wider rows (the k or v part of a packed q|k|v projection): row i
+ * then starts at element x_offset + i * x_row_stride of the slice (multiples of 4);
+ * x_row_stride = 0 means dense rows of n * d. */
+int ughip_kv_append(ughip_device* dev, ughip_slice* cache, const ughip_slice* x, size_t x_offset,
+                    size_t x_row_stride, size_t b, size_t n, size_t cap, size_t s_old, size_t t,
+                    size_t d,
                     const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos,
                     int interleaved);
 /* Causal attention of t query positions over such caches, f32, without materialising the
@@ -268,12 +272,28 @@ int ughip_kv_append(ughip_device* dev, ughip_slice* cache, const ughip_slice* x,
  * attends to keys 0 .. s - t + i; rope / rope_i is applied to q at table rows pos[0] + i when
  * cos/sin/pos are given.  t == 1 is ughip_attention_decode_rope on a cache of capacity cap;
  * t > 1 needs d = 32, 64 or 128 (UGHIP_ERR_UNSUPPORTED otherwise).  s - t == 0 and cap == s give
- * the reference's prefill. */
-int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, const ughip_slice* k,
-                           const ughip_slice* v, ughip_slice* dst, size_t b, size_t n_heads,
-                           size_t n_kv_heads, size_t t, size_t s, size_t cap, size_t d,
-                           float scale, const ughip_slice* cos, const ughip_slice* sin,
+ * the reference's prefill.  q_offset / q_row_stride: as x_offset / x_row_stride of
+ * ughip_kv_append (dst is always dense). */
+int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_offset,
+                           size_t q_row_stride, const ughip_slice* k, const ughip_slice* v,
+                           ughip_slice* dst, size_t b, size_t n_heads, size_t n_kv_heads,
+                           size_t t, size_t s, size_t cap, size_t d, float scale, const ughip_slice* cos, const ughip_slice* sin,
                            const ughip_slice* pos, int interleaved);
+
+/* ---- projections of one position with their neighbours folded in (f32, one input row) ----------
+ * No counterpart in the reference's device trait: there each is a matmul (lib.rs:62-70) followed
+ * by the small kernels of the lazy graph.  Every product is x (k elements) against the rows of a
+ * row-major [n, k] matrix, k % 4 == 0, summed in a fixed order.
+ * ughip_gemv_multi: dst[0 .. n0+n1+n2) = [x W_0^T | x W_1^T | x W_2^T] for n_mats <= 3 matrices
+ * (the q, k, v projections of ug-llama/src/model.rs:206-208 in one launch). */
+int ughip_gemv_multi(ughip_device* dev, const ughip_slice* x, size_t n_mats,
+                     const ughip_slice* const* w, const size_t* n, size_t k, ughip_slice* dst);
+/* dst[c] = silu(x . gate[c]) * (x . up[c]), silu(g) = g / (1 + exp(-g)) (model.rs:99-109,160-168). */
+int ughip_gemv_gate_up(ughip_device* dev, const ughip_slice* x, const ughip_slice* w_gate,
+                       const ughip_slice* w_up, ughip_slice* dst, size_t n, size_t k);
+/* dst[c] = x . w[c] + residual[c] (a projection followed by the residual add, model.rs:366-372). */
+int ughip_gemv_add(ughip_device* dev, const ughip_slice* x, const ughip_slice* w,
+                   const ughip_slice* residual, ughip_slice* dst, size_t n, size_t k);
 
 /* ---- element type conversion ------------------------------------------------------------------
  * dst[i] = (dtype of dst) src[i], same length, any pair of the five dtypes.  Replaces the host

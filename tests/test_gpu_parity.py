@@ -617,11 +617,12 @@ def test_attention_fusion_errors(hip, hip_ops):
         hip_ops.attention_decode(q3, same, same, 1.0).data_vec()
 
 
-@pytest.mark.parametrize("level", [1, 2])
+@pytest.mark.parametrize("level", [1, 2, 3])
 @pytest.mark.parametrize("width", ["small", "config5"])
 def test_llama_fused_attention_ids_match_unfused_cpu(hip, cpu, hip_ops, cpu_ops, width, level):
-    """The model with the attention fusions switched on (HIP; level 2 = caches written in place and
-    attention without materialised scores) against the reference's op-by-op graph (oracle)."""
+    """The model with the fusions switched on (HIP; level 2 = caches written in place and attention
+    without materialised scores, level 3 = also packed q|k|v, gate/up and residual projections)
+    against the reference's op-by-op graph (oracle)."""
     if width == "small":
         cfg = ug_amd.LlamaConfig(hidden_size=128, intermediate_size=320, max_position_embeddings=64, num_attention_heads=4, num_key_value_heads=2,
                                  num_hidden_layers=2, vocab_size=512)
@@ -829,6 +830,127 @@ def test_attention_cached_errors(hip, cpu, hip_ops, cpu_ops):
     assert out.shape == (4 * 32,) and np.all(out == 0)
     with pytest.raises(ug_amd.UgError, match="need a device kernel"):
         cpu_ops.attention_cached(lb((1, 2, 128), cpu), lb((1, 2, 5, 64), cpu), lb((1, 2, 5, 64), cpu), 5, 1.0).data_vec()
+
+
+# ---- projections of one position with their neighbours folded in ------------------------------------------------------------
+def _f64_rows(x, w):
+    return w.astype(np.float64) @ x.astype(np.float64)
+
+
+def _gemv_tol(x, w, rel=2e-6):
+    """k * eps forward bound of an f32 dot product, per output."""
+    return rel * (np.abs(w.astype(np.float64)) @ np.abs(x.astype(np.float64))) * np.sqrt(x.size) / 8 + 1e-30
+
+
+@pytest.mark.parametrize("ns,k", [((2048, 256, 256), 2048), ((64, 8, 8), 128), ((5, 3), 260), ((7,), 1024), ((4096, 512, 512), 4096), ((33, 1, 2), 2052)])
+def test_linear_packed(hip, cpu, hip_ops, cpu_ops, ns, k):
+    print("linear packed", ns, k, flush=True)
+    x = rng.normal(91, k)
+    ws = [rng.normal(92 + i, n * k, 0.05).reshape(n, k) for i, n in enumerate(ns)]
+    assert hip_ops.packed_projections() and not cpu_ops.packed_projections()
+    got = hip_ops.linear_packed(LB.copy(x, (1, 1, k), hip), [LB.copy(w.ravel(), w.shape, hip) for w in ws])
+    assert tuple(got.dims()) == (1, 1, sum(ns))
+    got = got.data_vec()
+    want = cpu_ops.linear_packed(LB.copy(x, (1, 1, k), cpu), [LB.copy(w.ravel(), w.shape, cpu) for w in ws]).data_vec()   # matmul_t x3 + cat
+    wall = np.concatenate(ws, 0)
+    truth, tol = _f64_rows(x, wall), _gemv_tol(x, wall)
+    assert np.all(np.abs(got - truth) <= tol)
+    assert np.all(np.abs(got - want) <= 2 * tol)
+    # each part is what a separate matmul of the same device gives, to the last rounding of the sum order
+    off = 0
+    for w in ws:
+        sep = LB.copy(x, (1, 1, k), hip).matmul_t(LB.copy(w.ravel(), w.shape, hip)).data_vec()
+        assert np.all(np.abs(got[off:off + w.shape[0]] - sep) <= 2 * tol[off:off + w.shape[0]])
+        off += w.shape[0]
+
+
+@pytest.mark.parametrize("n,k", [(5632, 2048), (64, 128), (9, 260), (11008, 4096)])
+def test_gate_up_fused(hip, cpu, hip_ops, cpu_ops, n, k):
+    print("gate up", n, k, flush=True)
+    x = rng.normal(94, k)
+    wg, wu = rng.normal(95, n * k, 0.05).reshape(n, k), rng.normal(96, n * k, 0.05).reshape(n, k)
+
+    def run(dev, ops):
+        return ops.gate_up(LB.copy(x, (1, 1, k), dev), LB.copy(wg.ravel(), (n, k), dev), LB.copy(wu.ravel(), (n, k), dev)).data_vec()
+
+    got, want = run(hip, hip_ops), run(cpu, cpu_ops)      # silu(x.matmul_t(gate)) * x.matmul_t(up) through the lazy graph
+    g, u = _f64_rows(x, wg), _f64_rows(x, wu)
+    sig = 1.0 / (1.0 + np.exp(-g))
+    truth = g * sig * u
+    tg, tu = _gemv_tol(x, wg), _gemv_tol(x, wu)
+    # d/dg [g sigmoid(g)] is bounded by 1.1; two more f32 roundings on top
+    tol = 1.1 * tg * np.abs(u) + np.abs(g * sig) * tu + 4e-7 * np.abs(truth) + 1e-30
+    assert np.all(np.abs(got - truth) <= tol), float((np.abs(got - truth) / tol).max())
+    assert np.all(np.abs(got - want) <= 2 * tol)
+
+
+@pytest.mark.parametrize("n,k", [(2048, 2048), (2048, 5632), (64, 128), (9, 260)])
+def test_linear_add_fused(hip, cpu, hip_ops, cpu_ops, n, k):
+    print("linear add", n, k, flush=True)
+    x, r = rng.normal(97, k), rng.normal(98, n)
+    w = rng.normal(99, n * k, 0.05).reshape(n, k)
+
+    def run(dev, ops):
+        return ops.linear_add(LB.copy(x, (1, 1, k), dev), LB.copy(w.ravel(), (n, k), dev), LB.copy(r, (1, 1, n), dev)).data_vec()
+
+    got, want = run(hip, hip_ops), run(cpu, cpu_ops)
+    truth = _f64_rows(x, w) + r
+    tol = _gemv_tol(x, w) + 1.2e-7 * np.abs(truth)
+    assert np.all(np.abs(got - truth) <= tol)
+    assert np.all(np.abs(got - want) <= 2 * tol)
+    # the separate matmul of this device followed by the add kernel of the lazy graph: bit for bit when both
+    # walk k in the same order (short rows go to another kernel in ughip_matmul)
+    sep = LB.copy(x, (1, 1, k), hip).matmul_t(LB.copy(w.ravel(), (n, k), hip)).binary("add", LB.copy(r, (1, 1, n), hip)).data_vec()
+    if k >= 256:
+        np.testing.assert_array_equal(got, sep)
+    else:
+        assert np.all(np.abs(got - sep) <= 2 * tol)
+
+
+def test_fused_projections_fall_back_for_several_rows(hip, cpu, hip_ops, cpu_ops):
+    """More than one input row (prefill): the hooks answer with the op-by-op composition on any device."""
+    t, k, n = 5, 64, 24
+    x, r = rng.normal(101, t * k), rng.normal(102, t * n)
+    w1, w2 = rng.normal(103, n * k, 0.1), rng.normal(104, n * k, 0.1)
+    for name, args in (("linear_packed", lambda d: (LB.copy(x, (1, t, k), d), [LB.copy(w1, (n, k), d), LB.copy(w2, (n, k), d)])),
+                       ("gate_up", lambda d: (LB.copy(x, (1, t, k), d), LB.copy(w1, (n, k), d), LB.copy(w2, (n, k), d))),
+                       ("linear_add", lambda d: (LB.copy(x, (1, t, k), d), LB.copy(w1, (n, k), d), LB.copy(r, (1, t, n), d)))):
+        got = getattr(hip_ops, name)(*args(hip)).data_vec()
+        want = getattr(cpu_ops, name)(*args(cpu)).data_vec()
+        np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-6)
+
+
+def test_packed_rows_feed_cache_and_attention(hip, hip_ops):
+    """q | k | v side by side in one buffer, read in place by kv_append and attention_cached: same
+    results as the three parts handed over separately."""
+    nh, nkv, d, cap, length = 8, 2, 64, 32, 5
+    nq, nk = nh * d, nkv * d
+    row = nq + 2 * nk
+    qkv = rng.normal(105, row)
+    store_k, store_v = rng.normal(106, nkv * cap * d), rng.normal(107, nkv * cap * d)
+    cos, sin = _rope_tables(hip, d, max_pos=cap)
+    pos = LB.copy(np.array([length], np.int32), (1, 1), hip)
+    scale = float(np.float32(d) ** np.float32(-0.5))
+
+    def run(packed):
+        ck, cv = LB.copy(store_k, (1, nkv, cap, d), hip), LB.copy(store_v, (1, nkv, cap, d), hip)
+        ck.realize(), cv.realize()
+        if packed:
+            buf = LB.copy(qkv, (1, 1, row), hip)
+            kc = hip_ops.kv_append(ck, length, buf, cos, sin, pos, False, x_offset=nq, x_row_stride=row)
+            vc = hip_ops.kv_append(cv, length, buf, x_offset=nq + nk, x_row_stride=row)
+            out = hip_ops.attention_cached(buf, kc, vc, length + 1, scale, cos, sin, pos, False, q_offset=0, q_row_stride=row, n_heads=nh)
+        else:
+            kc = hip_ops.kv_append(ck, length, LB.copy(qkv[nq:nq + nk], (1, 1, nk), hip), cos, sin, pos, False)
+            vc = hip_ops.kv_append(cv, length, LB.copy(qkv[nq + nk:], (1, 1, nk), hip))
+            out = hip_ops.attention_cached(LB.copy(qkv[:nq], (1, 1, nq), hip), kc, vc, length + 1, scale, cos, sin, pos, False)
+        assert tuple(out.dims()) == (1, 1, nq)
+        return out.data_vec(), ck.data_vec(), cv.data_vec()
+
+    for a, b2 in zip(run(True), run(False)):
+        np.testing.assert_array_equal(a, b2)
+    with pytest.raises(ug_amd.UgError, match="mismatched shapes"):
+        hip_ops.kv_append(LB.copy(store_k, (1, nkv, cap, d), hip), length, LB.copy(qkv, (1, 1, row), hip), x_offset=nq + nk + 4, x_row_stride=row).data_vec()
 
 
 # ---- safetensors: upload in the stored dtype, convert on the device ----------------------------------------------------

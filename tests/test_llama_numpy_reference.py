@@ -102,10 +102,10 @@ class NumpyLlama:
 
 
 @pytest.mark.parametrize("interleaved", [False, True])
-@pytest.mark.parametrize("custom_softmax,fused", [(False, 0), (True, 0), (True, 1), (True, 2)])
+@pytest.mark.parametrize("custom_softmax,fused", [(False, 0), (True, 0), (True, 1), (True, 2), (True, 3)])
 def test_llama_restatement_matches_numpy_f64(cpu, cpu_ops, interleaved, custom_softmax, fused):
     """fused > 0 routes attention through the optional Ops hooks (1: causal_softmax, rope_append,
-    attention_decode_flat; 2: kv_append, attention_cached), whose defaults (used by the CPU ops) are
+    attention_decode_flat; 2: kv_append, attention_cached; 3: also gate_up, linear_add), whose defaults (used by the CPU ops) are
     the same ops composed one by one: the graph changes shape, the values must not."""
     cfg = ug_amd.LlamaConfig(hidden_size=128, intermediate_size=320, max_position_embeddings=64, num_attention_heads=4, num_key_value_heads=2,
                              num_hidden_layers=2, vocab_size=512, rope_interleaved=interleaved)

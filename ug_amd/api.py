@@ -669,21 +669,45 @@ class LlamaOps(_Handle):
         _chk(host_lib().ugh_llama_kv_cache_capacity(_p(self.h), C.c_size_t(max_positions), C.c_size_t(head_dim), C.byref(out)))
         return out.value
 
-    def kv_append(self, cache, length, x, cos=None, sin=None, pos=None, interleaved=False):
+    def kv_append(self, cache, length, x, cos=None, sin=None, pos=None, interleaved=False, x_offset=0, x_row_stride=0):
         """cache [b, n, cap, d] holding `length` rows receives x [b, t, n * d] as rows length .. length + t - 1
-        (rotated when a table is given): in place when cap > length, by concatenation when cap == length."""
+        (rotated when a table is given): in place when cap > length, by concatenation when cap == length.
+        x_offset / x_row_stride: x as a column range of wider rows (a packed q|k|v projection)."""
         rope = cos is not None
         lb = self._op("ugh_llama_kv_append", cache, C.c_size_t(length), _p(x.h), _p(cos.h) if rope else None, _p(sin.h) if rope else None,
-                      _p(pos.h) if rope else None, int(interleaved))
+                      _p(pos.h) if rope else None, int(interleaved), C.c_size_t(x_offset), C.c_size_t(x_row_stride))
         lb._keep += [x] + ([cos, sin, pos] if rope else [])
         return lb
 
-    def attention_cached(self, q, k, v, s, scale, cos=None, sin=None, pos=None, interleaved=False):
-        """Causal attention of q [b, t, nh * d] over the first s rows of k, v [b, nkv, cap, d] -> [b, t, nh * d]."""
+    def attention_cached(self, q, k, v, s, scale, cos=None, sin=None, pos=None, interleaved=False, q_offset=0, q_row_stride=0, n_heads=0):
+        """Causal attention of q [b, t, nh * d] over the first s rows of k, v [b, nkv, cap, d] -> [b, t, nh * d].
+        q_offset / q_row_stride / n_heads: q as a column range of wider rows (a packed q|k|v projection)."""
         rope = cos is not None
         lb = self._op("ugh_llama_attention_cached", q, _p(k.h), _p(v.h), C.c_size_t(s), C.c_float(scale), _p(cos.h) if rope else None,
-                      _p(sin.h) if rope else None, _p(pos.h) if rope else None, int(interleaved))
+                      _p(sin.h) if rope else None, _p(pos.h) if rope else None, int(interleaved), C.c_size_t(q_offset), C.c_size_t(q_row_stride), C.c_size_t(n_heads))
         lb._keep += [k, v] + ([cos, sin, pos] if rope else [])
+        return lb
+
+    def packed_projections(self):
+        return bool(host_lib().ugh_llama_packed_projections(_p(self.h)))
+
+    def linear_packed(self, x, ws):
+        """x [b, t, k] against up to three [n_i, k] matrices -> [b, t, sum n_i], results side by side."""
+        arr = (C.c_void_p * len(ws))(*[w.h for w in ws])
+        lb = self._op("ugh_llama_linear_packed", x, C.c_size_t(len(ws)), arr)
+        lb._keep += list(ws)
+        return lb
+
+    def gate_up(self, x, w_gate, w_up):
+        """silu(x gate^T) * (x up^T)"""
+        lb = self._op("ugh_llama_gate_up", x, _p(w_gate.h), _p(w_up.h))
+        lb._keep += [w_gate, w_up]
+        return lb
+
+    def linear_add(self, x, w, residual):
+        """x w^T + residual"""
+        lb = self._op("ugh_llama_linear_add", x, _p(w.h), _p(residual.h))
+        lb._keep += [w, residual]
         return lb
 
 

@@ -35,7 +35,7 @@ def _run(cmd):
 def build_ughip():
     os.makedirs(LIB, exist_ok=True)
     src = os.path.join(CSRC, "ughip")
-    files = [os.path.join(src, f) for f in ("runtime.cpp", "lower_hip.cpp", "llama_ops.hip", "matmul.hip", "gemm_tiled.hip", "attention.hip", "convert.hip")]
+    files = [os.path.join(src, f) for f in ("runtime.cpp", "lower_hip.cpp", "llama_ops.hip", "matmul.hip", "gemm_tiled.hip", "attention.hip", "fused_linear.hip", "convert.hip")]
     _run([os.path.join(ROCM, "bin", "hipcc")] + HIP_FLAGS + ["-shared", "-I" + INC, "-I" + src] + files +
          ["-L" + os.path.join(ROCM, "lib"), "-lhiprtc", "-Wl,-rpath," + os.path.join(ROCM, "lib"), "-o", os.path.join(LIB, "libughip.so")])
 

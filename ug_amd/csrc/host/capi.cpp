@@ -460,17 +460,35 @@ int ugh_llama_attention_decode_flat(void* ops, void* q, void* k, void* v, float 
 int ugh_llama_kv_cache_capacity(void* ops, size_t max_positions, size_t head_dim, size_t* out) {
   return guard([&] { *out = ops_of(ops).kv_cache_capacity(max_positions, head_dim); });
 }
-int ugh_llama_kv_append(void* ops, void* cache, size_t len, void* x, void* cos, void* sin, void* pos, int interleaved, void** out) {
+int ugh_llama_kv_append(void* ops, void* cache, size_t len, void* x, void* cos, void* sin, void* pos, int interleaved, size_t x_offset, size_t x_row_stride,
+                        void** out) {
   return guard([&] {
-    if (cos) *out = box(ops_of(ops).kv_append(lb_of(cache), len, lb_of(x), &lb_of(cos), &lb_of(sin), &lb_of(pos), interleaved != 0));
-    else *out = box(ops_of(ops).kv_append(lb_of(cache), len, lb_of(x), nullptr, nullptr, nullptr, false));
+    if (cos) *out = box(ops_of(ops).kv_append(lb_of(cache), len, lb_of(x), &lb_of(cos), &lb_of(sin), &lb_of(pos), interleaved != 0, x_offset, x_row_stride));
+    else *out = box(ops_of(ops).kv_append(lb_of(cache), len, lb_of(x), nullptr, nullptr, nullptr, false, x_offset, x_row_stride));
   });
 }
-int ugh_llama_attention_cached(void* ops, void* q, void* k, void* v, size_t s, float scale, void* cos, void* sin, void* pos, int interleaved, void** out) {
+int ugh_llama_attention_cached(void* ops, void* q, void* k, void* v, size_t s, float scale, void* cos, void* sin, void* pos, int interleaved, size_t q_offset,
+                               size_t q_row_stride, size_t n_heads, void** out) {
   return guard([&] {
-    if (cos) *out = box(ops_of(ops).attention_cached(lb_of(q), lb_of(k), lb_of(v), s, scale, &lb_of(cos), &lb_of(sin), &lb_of(pos), interleaved != 0));
-    else *out = box(ops_of(ops).attention_cached(lb_of(q), lb_of(k), lb_of(v), s, scale, nullptr, nullptr, nullptr, false));
+    if (cos)
+      *out = box(ops_of(ops).attention_cached(lb_of(q), lb_of(k), lb_of(v), s, scale, &lb_of(cos), &lb_of(sin), &lb_of(pos), interleaved != 0, q_offset, q_row_stride,
+                                              n_heads));
+    else *out = box(ops_of(ops).attention_cached(lb_of(q), lb_of(k), lb_of(v), s, scale, nullptr, nullptr, nullptr, false, q_offset, q_row_stride, n_heads));
   });
+}
+int ugh_llama_packed_projections(void* ops) { return ops_of(ops).packed_projections() ? 1 : 0; }
+int ugh_llama_linear_packed(void* ops, void* x, size_t n_mats, void** ws, void** out) {
+  return guard([&] {
+    std::vector<ug::LazyBuffer> w;
+    for (size_t i = 0; i < n_mats; ++i) w.push_back(lb_of(ws[i]));
+    *out = box(ops_of(ops).linear_packed(lb_of(x), w));
+  });
+}
+int ugh_llama_gate_up(void* ops, void* x, void* w_gate, void* w_up, void** out) {
+  return guard([&] { *out = box(ops_of(ops).gate_up(lb_of(x), lb_of(w_gate), lb_of(w_up))); });
+}
+int ugh_llama_linear_add(void* ops, void* x, void* w, void* residual, void** out) {
+  return guard([&] { *out = box(ops_of(ops).linear_add(lb_of(x), lb_of(w), lb_of(residual))); });
 }
 int ugh_llama_rms_norm(void* src, void* alpha, float eps, void** out) {
   return guard([&] { *out = box(ug_llama::rms_norm(lb_of(src), lb_of(alpha), eps)); });

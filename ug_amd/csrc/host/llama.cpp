@@ -168,11 +168,16 @@ struct HipOps : Ops {
     return head_dim == 32 || head_dim == 64 || head_dim == 128 ? max_positions : 0;
   }
 
-  LB kv_append(const LB& cache, size_t len, const LB& x, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const override {
+  bool packed_projections() const override { return true; }
+
+  LB kv_append(const LB& cache, size_t len, const LB& x, const LB* cos, const LB* sin, const LB* pos, bool interleaved, size_t x_offset,
+               size_t x_row_stride) const override {
     if (cache.rank() != 4 || x.rank() != 3) bail("kv_append: expected cache [b, n, cap, d] and x [b, t, n * d]");
     size_t b = cache.dims()[0], n = cache.dims()[1], cap = cache.dims()[2], d = cache.dims()[3], t = x.dims()[1];
-    if (x.dims()[0] != b || x.dims()[2] != n * d) bail("kv_append: mismatched shapes " + cache.shape().str() + " " + x.shape().str());
-    if (cap == len || d % 4 != 0) return Ops::kv_append(cache, len, x, cos, sin, pos, interleaved);
+    const bool packed = x_offset != 0 || x_row_stride != 0;
+    if (x.dims()[0] != b || (packed ? x_row_stride != x.dims()[2] || x_offset + n * d > x_row_stride : x.dims()[2] != n * d))
+      bail("kv_append: mismatched shapes " + cache.shape().str() + " " + x.shape().str());
+    if (cap == len || d % 4 != 0) return Ops::kv_append(cache, len, x, cos, sin, pos, interleaved, x_offset, x_row_stride);
     if (len + t > cap) bail("kv_append: " + std::to_string(len + t) + " rows exceed the cache capacity " + std::to_string(cap));
     ughip_device* dev = hip_dev(x);
     const bool with_rope = cos != nullptr;
@@ -180,7 +185,8 @@ struct HipOps : Ops {
     // in-place op: arguments first, the cache last (schedule.rs:404-413)
     auto f = [=](const std::vector<Slice*>& vs) {
       if (vs.size() != (with_rope ? 5u : 2u)) bail("kv_append: unexpected number of slices");
-      hip_check(ughip_kv_append(dev, hip_raw_slice(*vs.back()), hip_raw_slice(*vs[0]), b, n, cap, len, t, d, with_rope ? hip_raw_slice(*vs[1]) : nullptr,
+      hip_check(ughip_kv_append(dev, hip_raw_slice(*vs.back()), hip_raw_slice(*vs[0]), x_offset, x_row_stride, b, n, cap, len, t, d,
+                                with_rope ? hip_raw_slice(*vs[1]) : nullptr,
                                 with_rope ? hip_raw_slice(*vs[2]) : nullptr, with_rope ? hip_raw_slice(*vs[3]) : nullptr, il),
                 "kv_append");
     };
@@ -193,22 +199,25 @@ struct HipOps : Ops {
     return cache.custom_ip(f, args);
   }
 
-  LB attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float scale, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const override {
+  LB attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float scale, const LB* cos, const LB* sin, const LB* pos, bool interleaved,
+                      size_t q_offset, size_t q_row_stride, size_t n_heads) const override {
     if (q.rank() != 3 || k.rank() != 4 || v.rank() != 4) bail("attention_cached: expected q [b, t, nh * d] and k, v [b, nkv, cap, d]");
     size_t b = q.dims()[0], t = q.dims()[1], nkv = k.dims()[1], cap = k.dims()[2], d = k.dims()[3];
-    if (k.dims() != v.dims() || k.dims()[0] != b || d == 0 || q.dims()[2] % d != 0 || s > cap || t > s)
+    const bool packed = q_offset != 0 || q_row_stride != 0;
+    if (k.dims() != v.dims() || k.dims()[0] != b || d == 0 || s > cap || t > s || (packed ? n_heads == 0 || q_row_stride != q.dims()[2] || q_offset + n_heads * d > q_row_stride
+                                                                                              : q.dims()[2] % d != 0 || (n_heads != 0 && n_heads * d != q.dims()[2])))
       bail("attention_cached: mismatched shapes " + q.shape().str() + " " + k.shape().str() + " with " + std::to_string(s) + " keys");
-    size_t nh = q.dims()[2] / d;
+    size_t nh = packed ? n_heads : q.dims()[2] / d;
     const bool one = t == 1 && d >= 16 && d <= 256 && (d & (d - 1)) == 0 && s <= 12000;
     const bool many = t > 1 && (d == 32 || d == 64 || d == 128);
-    if (!one && !many) return Ops::attention_cached(q, k, v, s, scale, cos, sin, pos, interleaved);
+    if (!one && !many) return Ops::attention_cached(q, k, v, s, scale, cos, sin, pos, interleaved, q_offset, q_row_stride, n_heads);
     ughip_device* dev = hip_dev(q);
     const bool with_rope = cos != nullptr;
     int il = interleaved ? 1 : 0;
     auto f = [=](const std::vector<Slice*>& vs) {
       if (vs.size() != (with_rope ? 7u : 4u)) bail("attention_cached: unexpected number of slices");
       ughip_slice* dst = hip_raw_slice(*vs.back());
-      hip_check(ughip_attention_cached(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), dst, b, nh, nkv, t, s, cap, d, scale,
+      hip_check(ughip_attention_cached(dev, hip_raw_slice(*vs[0]), q_offset, q_row_stride, hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), dst, b, nh, nkv, t, s, cap, d, scale,
                                        with_rope ? hip_raw_slice(*vs[3]) : nullptr, with_rope ? hip_raw_slice(*vs[4]) : nullptr,
                                        with_rope ? hip_raw_slice(*vs[5]) : nullptr, il),
                 "attention_cached");
@@ -219,7 +228,60 @@ struct HipOps : Ops {
       args.push_back(*sin);
       args.push_back(*pos);
     }
-    return LB::custom(f, args, q.shape(), q.dtype(), q.device());
+    return LB::custom(f, args, Shape({b, t, nh * d}), q.dtype(), q.device());
+  }
+
+  // One input row of f32 against row-major [n, k] matrices: the shapes the fused GEMV kernels take.
+  static bool one_f32_row(const LB& x, const std::vector<const LB*>& ws) {
+    if (x.rank() != 3 || x.dims()[0] * x.dims()[1] != 1 || x.dtype() != DType::F32 || x.dims()[2] % 4 != 0) return false;
+    for (const LB* w : ws)
+      if (w->rank() != 2 || w->dims()[1] != x.dims()[2] || w->dtype() != DType::F32) return false;
+    return true;
+  }
+
+  LB linear_packed(const LB& x, const std::vector<LB>& ws) const override {
+    std::vector<const LB*> wp;
+    for (const LB& w : ws) wp.push_back(&w);
+    if (ws.empty() || ws.size() > 3 || !one_f32_row(x, wp)) return Ops::linear_packed(x, ws);
+    std::vector<size_t> ns;
+    size_t total = 0, k = x.dims()[2];
+    for (const LB& w : ws) {
+      ns.push_back(w.dims()[0]);
+      total += w.dims()[0];
+    }
+    ughip_device* dev = hip_dev(x);
+    size_t n_mats = ws.size();
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != n_mats + 2) bail("linear_packed: unexpected number of slices");
+      const ughip_slice* w[3] = {nullptr, nullptr, nullptr};
+      for (size_t i = 0; i < n_mats; ++i) w[i] = hip_raw_slice(*vs[1 + i]);
+      hip_check(ughip_gemv_multi(dev, hip_raw_slice(*vs[0]), n_mats, w, ns.data(), k, hip_raw_slice(*vs.back())), "linear_packed");
+    };
+    std::vector<LB> args = {x};
+    for (const LB& w : ws) args.push_back(w);
+    return LB::custom(f, args, Shape({1, 1, total}), x.dtype(), x.device());
+  }
+
+  LB gate_up(const LB& x, const LB& w_gate, const LB& w_up) const override {
+    if (!one_f32_row(x, {&w_gate, &w_up}) || w_gate.dims() != w_up.dims()) return Ops::gate_up(x, w_gate, w_up);
+    size_t n = w_gate.dims()[0], k = x.dims()[2];
+    ughip_device* dev = hip_dev(x);
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != 4) bail("gate_up: expected 4 slices");
+      hip_check(ughip_gemv_gate_up(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), hip_raw_slice(*vs[3]), n, k), "gate_up");
+    };
+    return LB::custom(f, {x, w_gate, w_up}, Shape({1, 1, n}), x.dtype(), x.device());
+  }
+
+  LB linear_add(const LB& x, const LB& w, const LB& residual) const override {
+    if (!one_f32_row(x, {&w}) || residual.dtype() != DType::F32 || residual.elem_count() != w.dims()[0]) return Ops::linear_add(x, w, residual);
+    size_t n = w.dims()[0], k = x.dims()[2];
+    ughip_device* dev = hip_dev(x);
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != 4) bail("linear_add: expected 4 slices");
+      hip_check(ughip_gemv_add(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), hip_raw_slice(*vs[3]), n, k), "linear_add");
+    };
+    return LB::custom(f, {x, w, residual}, residual.shape(), x.dtype(), x.device());
   }
 };
 
@@ -293,7 +355,9 @@ LB Ops::attention_decode_flat(const LB& q, const LB& k, const LB& v, float scale
 }
 
 // model.rs:207-230 for t new positions, op by op (a cache that holds exactly `len` rows).
-LB Ops::kv_append(const LB& cache, size_t len, const LB& x, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const {
+LB Ops::kv_append(const LB& cache, size_t len, const LB& x, const LB* cos, const LB* sin, const LB* pos, bool interleaved, size_t x_offset,
+                  size_t x_row_stride) const {
+  if (x_offset != 0 || x_row_stride != 0) bail("kv_append: rows packed into a wider buffer need a device kernel");
   if (cache.rank() != 4 || x.rank() != 3) bail("kv_append: expected cache [b, n, cap, d] and x [b, t, n * d]");
   if (cache.dims()[2] != len) bail("kv_append: this device appends by concatenation and needs a cache of exactly " + std::to_string(len) + " rows, got " + cache.shape().str());
   size_t n = cache.dims()[1], d = cache.dims()[3];
@@ -303,7 +367,10 @@ LB Ops::kv_append(const LB& cache, size_t len, const LB& x, const LB* cos, const
 }
 
 // model.rs:207-210, 231-245, op by op.
-LB Ops::attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float scale, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const {
+LB Ops::attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float scale, const LB* cos, const LB* sin, const LB* pos, bool interleaved,
+                         size_t q_offset, size_t q_row_stride, size_t n_heads) const {
+  if (q_offset != 0 || q_row_stride != 0) bail("attention_cached: rows packed into a wider buffer need a device kernel");
+  (void)n_heads;
   if (q.rank() != 3 || k.rank() != 4 || v.rank() != 4) bail("attention_cached: expected q [b, t, nh * d] and k, v [b, nkv, s, d]");
   size_t t = q.dims()[1], d = k.dims()[3], nh = q.dims()[2] / d, nkv = k.dims()[1];
   if (k.dims()[2] != s) bail("attention_cached: this device needs caches of exactly " + std::to_string(s) + " rows, got " + k.shape().str());
@@ -318,6 +385,20 @@ LB Ops::attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float 
   att = t == 1 ? custom_softmax(att) : causal_softmax(att);
   return att.matmul(vr).transpose(2, 1).merge_dims(-2);
 }
+
+// model.rs:206-208 side by side.
+LB Ops::linear_packed(const LB& x, const std::vector<LB>& ws) const {
+  if (ws.empty()) bail("linear_packed: no matrices");
+  LB out = x.matmul_t(ws[0]);
+  for (size_t i = 1; i < ws.size(); ++i) out = cat(out, x.matmul_t(ws[i]), x.rank() - 1);
+  return out;
+}
+
+// model.rs:160-168 up to the down projection.
+LB Ops::gate_up(const LB& x, const LB& w_gate, const LB& w_up) const { return silu(x.matmul_t(w_gate)).binary(BinaryOp::Mul, x.matmul_t(w_up)); }
+
+// model.rs:366-372: a projection, then the residual.
+LB Ops::linear_add(const LB& x, const LB& w, const LB& residual) const { return x.matmul_t(w).binary(BinaryOp::Add, residual); }
 
 std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16) {
   return std::make_shared<SyntheticWeights>(seed, std, round_bf16);
@@ -497,10 +578,20 @@ Model::Model(const Config& cfg, bool custom_softmax, WeightSource& w, const Devi
 }
 
 // model.rs:203-248
-LB Model::attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache) const {
+LB Model::attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache, const LB* residual) const {
   if (xs.rank() != 3) bail("attention: expected [b, t, hidden]");
   size_t seq_len = xs.dims()[1];
   size_t nh = cfg_.num_attention_heads, nkv = cfg_.num_key_value_heads, hd = cfg_.head_dim();
+  auto finish = [&](const LB& out) { return residual ? ops_->linear_add(out, l.o_proj, *residual) : out.matmul_t(l.o_proj); };
+  if (fused_attention_ >= 3 && seq_len == 1 && xs.dims()[0] == 1 && cache.capacity && ops_->packed_projections()) {
+    // one position: q | k | v come out of one launch side by side and are read where they lie
+    const size_t nq = nh * hd, nk = nkv * hd, row = nq + 2 * nk, len = cache.len;
+    LB qkv = ops_->linear_packed(xs, {l.q_proj, l.k_proj, l.v_proj});
+    LB kc = ops_->kv_append(cache.prev_k, len, qkv, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, nq, row);
+    LB vc = ops_->kv_append(cache.prev_v, len, qkv, nullptr, nullptr, nullptr, false, nq + nk, row);
+    cache.len = len + 1;
+    return finish(ops_->attention_cached(qkv, kc, vc, cache.len, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, 0, row, nh));
+  }
   LB q = xs.matmul_t(l.q_proj);
   LB k = xs.matmul_t(l.k_proj);
   LB v = xs.matmul_t(l.v_proj);
@@ -515,16 +606,14 @@ LB Model::attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache) c
       cache.prev_v = vc;
     }  // else: kc and vc are this step's in-place writes of the storage prev_k / prev_v keep naming
     cache.len = len + seq_len;
-    LB out = ops_->attention_cached(q, kc, vc, cache.len, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved);
-    return out.matmul_t(l.o_proj);
+    return finish(ops_->attention_cached(q, kc, vc, cache.len, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved));
   }
   if (fused_attention_ && seq_len == 1) {
     // one new position: rows go from the projections into the caches and the attention kernel
     // without the split/transpose copies, and the result comes back in the layout o_proj reads
     cache.prev_k = ops_->rope_append(cache.prev_k, k, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved);
     cache.prev_v = ops_->rope_append(cache.prev_v, v, nullptr, nullptr, nullptr, false);
-    LB out = ops_->attention_decode_flat(q, cache.prev_k, cache.prev_v, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved);
-    return out.matmul_t(l.o_proj);
+    return finish(ops_->attention_decode_flat(q, cache.prev_k, cache.prev_v, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved));
   }
   q = q.split_dim(2, nh, hd).transpose(2, 1);
   k = k.split_dim(2, nkv, hd).transpose(2, 1);
@@ -557,11 +646,12 @@ LB Model::attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache) c
     out = att.matmul(vr);
   }
   out = out.transpose(2, 1).merge_dims(-2);
-  return out.matmul_t(l.o_proj);
+  return finish(out);
 }
 
 // model.rs:160-168
-LB Model::mlp(const Layer& l, const LB& xs) const {
+LB Model::mlp(const Layer& l, const LB& xs, const LB* residual) const {
+  if (residual) return ops_->linear_add(ops_->gate_up(xs, l.gate_proj, l.up_proj), l.down_proj, *residual);
   LB xs1 = xs.matmul_t(l.gate_proj);
   LB xs2 = xs.matmul_t(l.up_proj);
   xs1 = silu(xs1);
@@ -581,11 +671,16 @@ LB Model::fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const 
     const Layer& l = layers_[i];
     LB residual = xs;
     LB h = rms_norm(xs, l.rms1, eps);
-    h = attention(l, h, pos, cache[i]);
+    if (fused_attention_ >= 3) {
+      h = attention(l, h, pos, cache[i], &residual);
+      xs = mlp(l, rms_norm(h, l.rms2, eps), &h);
+      continue;
+    }
+    h = attention(l, h, pos, cache[i], nullptr);
     h = h.binary(BinaryOp::Add, residual);
     residual = h;
     LB m = rms_norm(h, l.rms2, eps);
-    m = mlp(l, m);
+    m = mlp(l, m, nullptr);
     xs = m.binary(BinaryOp::Add, residual);
   }
   xs = rms_norm(xs, ln_f_, eps);

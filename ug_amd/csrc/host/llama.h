@@ -47,12 +47,30 @@ struct Ops {
   // and is rotated at table rows pos[0] + i when a table is given.  Returns the cache with rows
   // len .. len + t - 1 written: the same storage when cap > len (in place), otherwise (cap == len,
   // the default) a new buffer [b, n, len + t, d] built with rope and cat.
-  virtual LB kv_append(const LB& cache, size_t len, const LB& x, const LB* cos, const LB* sin, const LB* pos, bool interleaved) const;
+  // x may be a column range of wider rows (a packed q|k|v projection): row i then starts at
+  // element x_offset + i * x_row_stride of x (x_row_stride 0 = dense rows); only devices with
+  // packed_projections() take that form.
+  virtual LB kv_append(const LB& cache, size_t len, const LB& x, const LB* cos, const LB* sin, const LB* pos, bool interleaved, size_t x_offset = 0,
+                       size_t x_row_stride = 0) const;
   // Causal attention of q [b, t, nh * d] (rotated first when a table is given) over the first s rows
   // of k and v [b, nkv, cap, d]; query i sees keys 0 .. s - t + i.  Returns [b, t, nh * d].  The
   // default composes model.rs:207-210, 231-245 and needs cap == s and, for t > 1, s == t.
+  // q_offset / q_row_stride / n_heads: q as a column range of wider rows, as for kv_append
+  // (n_heads = 0: taken from q's last dim).
   virtual LB attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float scale, const LB* cos, const LB* sin, const LB* pos,
-                              bool interleaved) const;
+                              bool interleaved, size_t q_offset = 0, size_t q_row_stride = 0, size_t n_heads = 0) const;
+
+  // Projections with their neighbours folded in.  The defaults compose matmul_t with the lazy
+  // graph's own element-wise ops, exactly as model.rs:160-168, 206-208, 366-372 do.
+  // packed_projections(): linear_packed gives q|k|v side by side in one buffer and kv_append /
+  // attention_cached read their part of it in place.
+  virtual bool packed_projections() const { return false; }
+  // x [b, t, k] against up to three [n_i, k] matrices -> [b, t, n_0 + n_1 + n_2].
+  virtual LB linear_packed(const LB& x, const std::vector<LB>& ws) const;
+  // silu(x gate^T) * (x up^T)
+  virtual LB gate_up(const LB& x, const LB& w_gate, const LB& w_up) const;
+  // x w^T + residual
+  virtual LB linear_add(const LB& x, const LB& w, const LB& residual) const;
 };
 
 // The HIP implementation (counterpart of ug-llama/src/cuda_ops.rs).
@@ -121,6 +139,9 @@ class Model {
   // 2: Ops::kv_append + Ops::attention_cached for any number of positions; with a device that
   //    preallocates (Ops::kv_cache_capacity) the caches are written in place and scores never
   //    reach memory.
+  // 3: 2, and the projections through Ops::linear_packed (q|k|v), Ops::gate_up and
+  //    Ops::linear_add (o_proj / down_proj with the residual): 8 schedule items per layer and
+  //    decode step on a device that fuses them.
   void set_fused_attention(int level) { fused_attention_ = level; }
   int fused_attention() const { return fused_attention_; }
   // Caches of the kind fwd() expects at the current fusion level.
@@ -136,8 +157,9 @@ class Model {
     LB q_proj, k_proj, v_proj, o_proj;
     LB gate_proj, up_proj, down_proj;
   };
-  LB attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache) const;
-  LB mlp(const Layer& l, const LB& xs) const;
+  // residual != nullptr: the result includes the residual add (fusion level 3)
+  LB attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache, const LB* residual) const;
+  LB mlp(const Layer& l, const LB& xs, const LB* residual) const;
   Config cfg_;
   bool custom_softmax_;
   int fused_attention_ = 0;

@@ -122,8 +122,8 @@ __device__ __forceinline__ float att_block_reduce(float v, float* lds16) {
 }
 
 __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
-                                                                       float* __restrict__ dst, int nh, int nkv, int s, size_t kv_head_stride, int d,
-                                                                       float scale, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                                       float* __restrict__ dst, int nh, int nkv, int s, size_t kv_head_stride,
+                                                                       size_t q_batch_stride, int d, float scale, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                                                        const int* __restrict__ pos, size_t table_len, int interleaved) {
   extern __shared__ __attribute__((aligned(16))) float sc[];  // s scores, then ATT_WAVES * 64 float4 of reduction space
   __shared__ float lds16[ATT_WAVES];
@@ -132,7 +132,8 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
   const int lpk = d >> 2, kpb = ATT_THREADS / lpk;  // lanes per key, keys per step
   const int c4 = tid % lpk, slot = tid / lpk;
   const int bh = blockIdx.x, b = bh / nh, h = bh % nh, kvh = h / (nh / nkv);
-  const float4* q4 = reinterpret_cast<const float4*>(q + (size_t)bh * d);
+  const float* qh = q + (size_t)b * q_batch_stride + (size_t)h * d;  // q_batch_stride = nh * d unless q is part of a wider row
+  const float4* q4 = reinterpret_cast<const float4*>(qh);
   const float4* k4 = reinterpret_cast<const float4*>(k + ((size_t)b * nkv + kvh) * kv_head_stride);
   const float4* v4 = reinterpret_cast<const float4*>(v + ((size_t)b * nkv + kvh) * kv_head_stride);
 
@@ -145,7 +146,7 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
       const bool ok = p >= 0 && ics < table_len;
       const float c = ok ? cos_t[ics] : NAN, sn = ok ? sin_t[ics] : NAN;
       const int i1 = interleaved ? 2 * tid : tid, i2 = interleaved ? 2 * tid + 1 : tid + half;
-      const float x1 = q[(size_t)bh * d + i1], x2 = q[(size_t)bh * d + i2];
+      const float x1 = qh[i1], x2 = qh[i2];
       qs[i1] = x1 * c - x2 * sn;
       qs[i2] = x1 * sn + x2 * c;
     }
@@ -273,10 +274,11 @@ __global__ void __launch_bounds__(256) rope_append_kernel(const float* __restric
 }
 
 // ---- cache append in place ------------------------------------------------------------------------
-// cache [b, n, cap, d], x [b, t, n * d]: cache[b, h, s_old + i, :] = x[b, i, h * d .. (h + 1) * d),
-// rotated at table row pos[0] + i when a table is given.  One thread per float4 of x (d % 4 == 0).
-__global__ void __launch_bounds__(256) kv_append_kernel(float* __restrict__ cache, const float* __restrict__ x, size_t n4, int t, int n, int d, size_t cap,
-                                                        int s_old, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+// cache [b, n, cap, d], x [b, t, n * d] (rows x_row_stride apart): cache[b, h, s_old + i, :] =
+// x[b, i, h * d .. (h + 1) * d), rotated at table row pos[0] + i when a table is given.  One thread
+// per float4 of x (d % 4 == 0).
+__global__ void __launch_bounds__(256) kv_append_kernel(float* __restrict__ cache, const float* __restrict__ x, size_t x_row_stride, size_t n4, int t, int n,
+                                                        int d, size_t cap, int s_old, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                                         const int* __restrict__ pos, size_t table_len, int interleaved) {
   const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (g >= n4) return;
@@ -287,7 +289,7 @@ __global__ void __launch_bounds__(256) kv_append_kernel(float* __restrict__ cach
   rest /= n;
   const int i = (int)(rest % t);
   const size_t b = rest / t;
-  const float* xr = x + ((b * t + i) * n + h) * (size_t)d;
+  const float* xr = x + (b * t + i) * x_row_stride + (size_t)h * d;  // x_row_stride = n * d unless x is part of a wider row
   float4 out;
   if (!cos_t) {
     out = reinterpret_cast<const float4*>(xr)[c4];
@@ -313,7 +315,7 @@ __global__ void __launch_bounds__(256) kv_append_kernel(float* __restrict__ cach
 }
 
 // ---- causal attention over a cache, many query positions ------------------------------------------
-// q, dst: [b, t, nh * D]; k, v: [b, nkv, cap, D] with rows 0 .. s-1 valid.  Query i sits at position
+// q, dst: [b, t, nh * D] (q rows q_row_stride apart); k, v: [b, nkv, cap, D] with rows 0 .. s-1 valid.  Query i sits at position
 // s - t + i and sees keys 0 .. s - t + i (model.rs:231-244 with the mask of cpu_ops.rs:33-56 moved to
 // that offset).  Scores never reach memory: a group of 4 waves owns 32 queries of one head, its waves
 // take every fourth block of 32 keys and keep a running (max, sum, output) per query, merged at the
@@ -332,8 +334,8 @@ typedef float att_f32x16 __attribute__((ext_vector_type(16)));
 
 template <int D, int GROUPS>
 __global__ void __launch_bounds__(256 * GROUPS) attention_prefill_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
-                                                                float* __restrict__ dst, int nh, int nkv, int t, int s, size_t cap, float scale,
-                                                                const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                                float* __restrict__ dst, int nh, int nkv, int t, int s, size_t cap,
+                                                                size_t q_row_stride, float scale, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                                                 const int* __restrict__ pos, size_t table_len, int interleaved) {
   constexpr int H = D / 2, DB = D / 32;  // floats of q / k per lane; 32-wide blocks of the head dimension
   __shared__ float merge_ml_all[GROUPS][3][2][64];
@@ -373,7 +375,7 @@ __global__ void __launch_bounds__(256 * GROUPS) attention_prefill_kernel(const f
   // this lane's half of its (rotated) query row
   float qr[H];
   {
-    const float* qrow = q + ((size_t)b * t + qi) * ((size_t)nh * D) + (size_t)head * D;
+    const float* qrow = q + ((size_t)b * t + qi) * q_row_stride + (size_t)head * D;  // nh * D unless q is part of a wider row
     if (!cos_t) {
 #pragma unroll
       for (int j = 0; j < H; j += 4) {
@@ -579,9 +581,9 @@ int ughip_attention_decode(ughip_device* dev, const ughip_slice* q, const ughip_
 
 namespace {
 // One query position per head against s keys of caches whose heads are cap rows apart.
-int attention_decode_launch(ughip_device* dev, const ughip_slice* q, const ughip_slice* k, const ughip_slice* v, ughip_slice* dst, size_t b, size_t n_heads,
-                            size_t n_kv_heads, size_t s, size_t cap, size_t d, float scale, const ughip_slice* cos, const ughip_slice* sin,
-                            const ughip_slice* pos, int interleaved) {
+int attention_decode_launch(ughip_device* dev, const ughip_slice* q, size_t q_offset, size_t q_row_stride, const ughip_slice* k, const ughip_slice* v,
+                            ughip_slice* dst, size_t b, size_t n_heads, size_t n_kv_heads, size_t s, size_t cap, size_t d, float scale, const ughip_slice* cos,
+                            const ughip_slice* sin, const ughip_slice* pos, int interleaved) {
   if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
   const bool rope = cos || sin || pos;
   if (rope)
@@ -592,7 +594,10 @@ int attention_decode_launch(ughip_device* dev, const ughip_slice* q, const ughip
   if (s == 0) return set_error(UGHIP_ERR_INVALID, "attention_decode: empty key sequence");
   if (s > cap) return set_error(UGHIP_ERR_INVALID, "attention_decode: %zu keys exceed the cache capacity %zu", s, cap);
   if (s > 12000) return set_error(UGHIP_ERR_INVALID, "attention_decode: %zu keys exceed the 12000 this kernel holds in LDS", s);
-  if (int rc = check_f32(q, b * n_heads * d, "attention_decode q")) return rc;
+  if (q_row_stride == 0) q_row_stride = n_heads * d;
+  if (q_row_stride < n_heads * d || (q_offset | q_row_stride) % 4 != 0)
+    return set_error(UGHIP_ERR_INVALID, "attention_decode: q offset %zu / row stride %zu do not fit rows of %zu", q_offset, q_row_stride, n_heads * d);
+  if (int rc = check_f32(q, b ? q_offset + (b - 1) * q_row_stride + n_heads * d : 0, "attention_decode q")) return rc;
   if (int rc = check_f32(k, b * n_kv_heads * cap * d, "attention_decode k")) return rc;
   if (int rc = check_f32(v, b * n_kv_heads * cap * d, "attention_decode v")) return rc;
   if (int rc = check_f32(dst, b * n_heads * d, "attention_decode dst")) return rc;
@@ -602,8 +607,8 @@ int attention_decode_launch(ughip_device* dev, const ughip_slice* q, const ughip
   if (int rc = device_activate(dev)) return rc;
   const size_t lds = (s + 3 + ATT_WAVES * 64 * 4) * sizeof(float);  // scores, alignment slack, one float4 per lane slot of every wave
   attention_decode_kernel<<<(unsigned)(b * n_heads), ATT_THREADS, lds, dev->stream>>>(
-      static_cast<const float*>(q->ptr), static_cast<const float*>(k->ptr), static_cast<const float*>(v->ptr), static_cast<float*>(dst->ptr), (int)n_heads,
-      (int)n_kv_heads, (int)s, cap * d, (int)d, scale, rope ? static_cast<const float*>(cos->ptr) : nullptr,
+      static_cast<const float*>(q->ptr) + q_offset, static_cast<const float*>(k->ptr), static_cast<const float*>(v->ptr), static_cast<float*>(dst->ptr),
+      (int)n_heads, (int)n_kv_heads, (int)s, cap * d, q_row_stride, (int)d, scale, rope ? static_cast<const float*>(cos->ptr) : nullptr,
       rope ? static_cast<const float*>(sin->ptr) : nullptr, rope ? static_cast<const int*>(pos->ptr) : nullptr,
       rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved);
   UGHIP_HIPCHK(hipGetLastError());
@@ -614,7 +619,7 @@ int attention_decode_launch(ughip_device* dev, const ughip_slice* q, const ughip
 int ughip_attention_decode_rope(ughip_device* dev, const ughip_slice* q, const ughip_slice* k, const ughip_slice* v, ughip_slice* dst, size_t b,
                                 size_t n_heads, size_t n_kv_heads, size_t s, size_t d, float scale, const ughip_slice* cos, const ughip_slice* sin,
                                 const ughip_slice* pos, int interleaved) {
-  return attention_decode_launch(dev, q, k, v, dst, b, n_heads, n_kv_heads, s, s, d, scale, cos, sin, pos, interleaved);
+  return attention_decode_launch(dev, q, 0, 0, k, v, dst, b, n_heads, n_kv_heads, s, s, d, scale, cos, sin, pos, interleaved);
 }
 
 int ughip_rope_append(ughip_device* dev, const ughip_slice* cache, const ughip_slice* x, ughip_slice* dst, size_t bh, size_t s_old, size_t d,
@@ -644,8 +649,8 @@ int ughip_rope_append(ughip_device* dev, const ughip_slice* cache, const ughip_s
   return UGHIP_OK;
 }
 
-int ughip_kv_append(ughip_device* dev, ughip_slice* cache, const ughip_slice* x, size_t b, size_t n, size_t cap, size_t s_old, size_t t, size_t d,
-                    const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos, int interleaved) {
+int ughip_kv_append(ughip_device* dev, ughip_slice* cache, const ughip_slice* x, size_t x_offset, size_t x_row_stride, size_t b, size_t n, size_t cap,
+                    size_t s_old, size_t t, size_t d, const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos, int interleaved) {
   if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
   if (d == 0 || d % 4 != 0) return set_error(UGHIP_ERR_INVALID, "kv_append: head size %zu is not a multiple of 4", d);
   const bool rope = cos || sin || pos;
@@ -655,7 +660,10 @@ int ughip_kv_append(ughip_device* dev, ughip_slice* cache, const ughip_slice* x,
   }
   if (s_old + t > cap) return set_error(UGHIP_ERR_BOUNDS, "kv_append: rows %zu..%zu do not fit a cache of %zu rows", s_old, s_old + t, cap);
   if (int rc = check_f32(cache, b * n * cap * d, "kv_append cache")) return rc;
-  if (int rc = check_f32(x, b * t * n * d, "kv_append x")) return rc;
+  if (x_row_stride == 0) x_row_stride = n * d;
+  if (x_row_stride < n * d || (x_offset | x_row_stride) % 4 != 0)
+    return set_error(UGHIP_ERR_INVALID, "kv_append: x offset %zu / row stride %zu do not fit rows of %zu", x_offset, x_row_stride, n * d);
+  if (int rc = check_f32(x, b * t ? x_offset + (b * t - 1) * x_row_stride + n * d : 0, "kv_append x")) return rc;
   if (cache == x) return set_error(UGHIP_ERR_INVALID, "kv_append: x aliases the cache");
   const size_t n4 = b * t * n * d / 4;
   if (n4 == 0) return UGHIP_OK;
@@ -663,17 +671,17 @@ int ughip_kv_append(ughip_device* dev, ughip_slice* cache, const ughip_slice* x,
     return set_error(UGHIP_ERR_INVALID, "kv_append: shape too large");
   if (int rc = device_activate(dev)) return rc;
   kv_append_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, dev->stream>>>(
-      static_cast<float*>(cache->ptr), static_cast<const float*>(x->ptr), n4, (int)t, (int)n, (int)d, cap, (int)s_old,
+      static_cast<float*>(cache->ptr), static_cast<const float*>(x->ptr) + x_offset, x_row_stride, n4, (int)t, (int)n, (int)d, cap, (int)s_old,
       rope ? static_cast<const float*>(cos->ptr) : nullptr, rope ? static_cast<const float*>(sin->ptr) : nullptr,
       rope ? static_cast<const int*>(pos->ptr) : nullptr, rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
 }
 
-int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, const ughip_slice* k, const ughip_slice* v, ughip_slice* dst, size_t b, size_t n_heads,
-                           size_t n_kv_heads, size_t t, size_t s, size_t cap, size_t d, float scale, const ughip_slice* cos, const ughip_slice* sin,
-                           const ughip_slice* pos, int interleaved) {
-  if (t == 1) return attention_decode_launch(dev, q, k, v, dst, b, n_heads, n_kv_heads, s, cap, d, scale, cos, sin, pos, interleaved);
+int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_offset, size_t q_row_stride, const ughip_slice* k, const ughip_slice* v,
+                           ughip_slice* dst, size_t b, size_t n_heads, size_t n_kv_heads, size_t t, size_t s, size_t cap, size_t d, float scale,
+                           const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos, int interleaved) {
+  if (t == 1) return attention_decode_launch(dev, q, q_offset, q_row_stride, k, v, dst, b, n_heads, n_kv_heads, s, cap, d, scale, cos, sin, pos, interleaved);
   if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
   const bool rope = cos || sin || pos;
   if (rope)
@@ -684,7 +692,10 @@ int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, const ughip_
     return set_error(UGHIP_ERR_UNSUPPORTED, "attention_cached: head size %zu (32, 64 and 128 are built for more than one query position)", d);
   if (t == 0 || s < t) return set_error(UGHIP_ERR_INVALID, "attention_cached: %zu query positions need at least as many keys, got %zu", t, s);
   if (s > cap) return set_error(UGHIP_ERR_INVALID, "attention_cached: %zu keys exceed the cache capacity %zu", s, cap);
-  if (int rc = check_f32(q, b * t * n_heads * d, "attention_cached q")) return rc;
+  if (q_row_stride == 0) q_row_stride = n_heads * d;
+  if (q_row_stride < n_heads * d || (q_offset | q_row_stride) % 4 != 0)
+    return set_error(UGHIP_ERR_INVALID, "attention_cached: q offset %zu / row stride %zu do not fit rows of %zu", q_offset, q_row_stride, n_heads * d);
+  if (int rc = check_f32(q, b ? q_offset + (b * t - 1) * q_row_stride + n_heads * d : 0, "attention_cached q")) return rc;
   if (int rc = check_f32(k, b * n_kv_heads * cap * d, "attention_cached k")) return rc;
   if (int rc = check_f32(v, b * n_kv_heads * cap * d, "attention_cached v")) return rc;
   if (int rc = check_f32(dst, b * t * n_heads * d, "attention_cached dst")) return rc;
@@ -697,7 +708,7 @@ int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, const ughip_
   const float* sp = rope ? static_cast<const float*>(sin->ptr) : nullptr;
   const int* pp = rope ? static_cast<const int*>(pos->ptr) : nullptr;
   const size_t tl = rope ? (cos->len < sin->len ? cos->len : sin->len) : 0;
-  const float* qp = static_cast<const float*>(q->ptr);
+  const float* qp = static_cast<const float*>(q->ptr) + q_offset;
   const float* kp = static_cast<const float*>(k->ptr);
   const float* vp = static_cast<const float*>(v->ptr);
   float* op = static_cast<float*>(dst->ptr);
@@ -706,11 +717,11 @@ int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, const ughip_
   // workgroup would give every CU two workgroups anyway; d = 128 needs the whole register file for 4 waves.
   const dim3 paired((n_qb + 1) / 2, (unsigned)(b * n_heads)), single(n_qb, (unsigned)(b * n_heads));
   const bool pair = d <= 64 && (size_t)n_qb * b * n_heads >= 512;
-  if (d == 32 && pair) attention_prefill_kernel<32, 2><<<paired, 512, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, scale, cp, sp, pp, tl, interleaved);
-  else if (d == 32) attention_prefill_kernel<32, 1><<<single, 256, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, scale, cp, sp, pp, tl, interleaved);
-  else if (d == 64 && pair) attention_prefill_kernel<64, 2><<<paired, 512, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, scale, cp, sp, pp, tl, interleaved);
-  else if (d == 64) attention_prefill_kernel<64, 1><<<single, 256, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, scale, cp, sp, pp, tl, interleaved);
-  else attention_prefill_kernel<128, 1><<<single, 256, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, scale, cp, sp, pp, tl, interleaved);
+  if (d == 32 && pair) attention_prefill_kernel<32, 2><<<paired, 512, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, q_row_stride, scale, cp, sp, pp, tl, interleaved);
+  else if (d == 32) attention_prefill_kernel<32, 1><<<single, 256, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, q_row_stride, scale, cp, sp, pp, tl, interleaved);
+  else if (d == 64 && pair) attention_prefill_kernel<64, 2><<<paired, 512, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, q_row_stride, scale, cp, sp, pp, tl, interleaved);
+  else if (d == 64) attention_prefill_kernel<64, 1><<<single, 256, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, q_row_stride, scale, cp, sp, pp, tl, interleaved);
+  else attention_prefill_kernel<128, 1><<<single, 256, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, q_row_stride, scale, cp, sp, pp, tl, interleaved);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
 }

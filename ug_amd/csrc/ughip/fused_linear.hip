@@ -1,0 +1,247 @@
+// Row-vector projections of a decode step with their neighbours folded in (f32, one input row):
+//
+//   ughip_gemv_multi    y = [x W_0^T | x W_1^T | x W_2^T]: up to three matrices over the same x in one
+//                       launch, results side by side (the q / k / v projections of
+//                       ug-llama/src/model.rs:206-208)
+//   ughip_gemv_gate_up  y = silu(x G^T) * (x U^T), silu(g) = g / (1 + exp(-g))
+//                       (model.rs:160-168 up to the down projection, written as in model.rs:99-109)
+//   ughip_gemv_add      y = x W^T + r   (o_proj / down_proj followed by the residual add, model.rs:366-372)
+//
+// One token's projections are 6-46 MB matrix streams behind 2-3 us launches; these entry points
+// remove launches and the small vectors that would travel between them, nothing else: every
+// product is the same fixed-order f32 sum a separate ughip_matmul computes, the epilogues are
+// the same f32 operations the lazy graph would run on the rounded products.
+//
+// KS waves share one output column, each walking every KS-th 64-lane slab of k with four 128-bit
+// loads in flight per lane and matrix; a workgroup of 4 waves covers 4 / KS columns.
+#include <hip/hip_runtime.h>
+
+#include <cstdlib>
+
+#include "internal.h"
+#include "ughip.h"
+
+using namespace ughip;
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+enum { MODE_MULTI = 0, MODE_GATE_UP = 1, MODE_ADD = 2 };
+
+struct FusedArgs {
+  const float* x;
+  const float* w[3];
+  float* y[3];
+  int col_end[3];  // MODE_MULTI: matrix i owns the columns col_end[i-1] .. col_end[i] - 1 of the grid
+  int n_cols;      // columns of the grid
+  int k;
+  const float* residual;
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+__device__ __forceinline__ float dot4(const f32x4& w, const f32x4& x, float acc) {
+  acc += w.x * x.x;
+  acc += w.y * x.y;
+  acc += w.z * x.z;
+  acc += w.w * x.w;
+  return acc;
+}
+
+template <int KS, int MODE>
+__global__ void __launch_bounds__(256) fused_gemv(FusedArgs a) {
+  __shared__ float part[4][2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = blockIdx.x * (4 / KS) + wave / KS, ks = wave % KS;
+  const bool live = col < a.n_cols;
+  // which matrix and which of its rows this column is
+  const float* __restrict__ W0 = nullptr;
+  const float* __restrict__ W1 = nullptr;
+  float* __restrict__ Y = nullptr;
+  if (live) {
+    int m = 0, first = 0;
+    if (MODE == MODE_MULTI) {
+      if (col >= a.col_end[0]) m = 1, first = a.col_end[0];
+      if (col >= a.col_end[1]) m = 2, first = a.col_end[1];
+    }
+    const int row = col - first;
+    W0 = a.w[m] + (size_t)row * a.k;
+    if (MODE == MODE_GATE_UP) W1 = a.w[1] + (size_t)row * a.k;
+    Y = a.y[m] + row;
+  }
+  float acc0 = 0.f, acc1 = 0.f;
+  if (live) {
+    const float* __restrict__ X = a.x;
+    constexpr int stride = 64 * 4 * KS;
+    int k = (ks * 64 + lane) * 4;
+    for (; k + 3 * stride < a.k; k += 4 * stride) {
+      const f32x4 w0 = *reinterpret_cast<const f32x4*>(W0 + k), w1 = *reinterpret_cast<const f32x4*>(W0 + k + stride);
+      const f32x4 w2 = *reinterpret_cast<const f32x4*>(W0 + k + 2 * stride), w3 = *reinterpret_cast<const f32x4*>(W0 + k + 3 * stride);
+      f32x4 u0, u1, u2, u3;
+      if (MODE == MODE_GATE_UP) {
+        u0 = *reinterpret_cast<const f32x4*>(W1 + k), u1 = *reinterpret_cast<const f32x4*>(W1 + k + stride);
+        u2 = *reinterpret_cast<const f32x4*>(W1 + k + 2 * stride), u3 = *reinterpret_cast<const f32x4*>(W1 + k + 3 * stride);
+      }
+      const f32x4 x0 = *reinterpret_cast<const f32x4*>(X + k), x1 = *reinterpret_cast<const f32x4*>(X + k + stride);
+      const f32x4 x2 = *reinterpret_cast<const f32x4*>(X + k + 2 * stride), x3 = *reinterpret_cast<const f32x4*>(X + k + 3 * stride);
+      acc0 = dot4(w0, x0, acc0);
+      acc0 = dot4(w1, x1, acc0);
+      acc0 = dot4(w2, x2, acc0);
+      acc0 = dot4(w3, x3, acc0);
+      if (MODE == MODE_GATE_UP) {
+        acc1 = dot4(u0, x0, acc1);
+        acc1 = dot4(u1, x1, acc1);
+        acc1 = dot4(u2, x2, acc1);
+        acc1 = dot4(u3, x3, acc1);
+      }
+    }
+    for (; k < a.k; k += stride) {
+      const f32x4 x0 = *reinterpret_cast<const f32x4*>(X + k);
+      acc0 = dot4(*reinterpret_cast<const f32x4*>(W0 + k), x0, acc0);
+      if (MODE == MODE_GATE_UP) acc1 = dot4(*reinterpret_cast<const f32x4*>(W1 + k), x0, acc1);
+    }
+  }
+  acc0 = wave_sum(acc0);
+  if (MODE == MODE_GATE_UP) acc1 = wave_sum(acc1);
+  if (KS > 1) {
+    if (lane == 0) {
+      part[wave][0] = acc0;
+      part[wave][1] = acc1;
+    }
+    __syncthreads();
+    if (ks != 0) return;
+    acc0 = part[wave][0];
+    acc1 = part[wave][1];
+#pragma unroll
+    for (int j = 1; j < KS; ++j) {
+      acc0 += part[wave + j][0];
+      acc1 += part[wave + j][1];
+    }
+  }
+  if (!live || lane != 0) return;
+  if (MODE == MODE_GATE_UP) *Y = acc0 / (1.f + expf(-acc0)) * acc1;
+  else if (MODE == MODE_ADD) *Y = acc0 + a.residual[col];
+  else *Y = acc0;
+}
+
+int pick_ks(size_t cols, size_t k) {
+  // enough waves to hide HBM latency: about 8192 over the chip
+  int ks = cols <= 2048 ? 4 : cols <= 6144 ? 2 : 1;
+  if (const char* e = getenv("UGHIP_GEMV_KS")) ks = atoi(e);  // tuning aid: 1, 2 or 4
+  if (ks != 1 && ks != 2 && ks != 4) ks = 1;
+  while (ks > 1 && k < (size_t)64 * 4 * ks) ks >>= 1;
+  return ks;
+}
+
+template <int MODE>
+void launch(hipStream_t st, const FusedArgs& a) {
+  const int ks = pick_ks((size_t)a.n_cols * (MODE == MODE_GATE_UP ? 2 : 1), (size_t)a.k);
+  const unsigned per_wg = 4 / ks;
+  const unsigned grid = ((unsigned)a.n_cols + per_wg - 1) / per_wg;
+  if (ks == 4) fused_gemv<4, MODE><<<grid, 256, 0, st>>>(a);
+  else if (ks == 2) fused_gemv<2, MODE><<<grid, 256, 0, st>>>(a);
+  else fused_gemv<1, MODE><<<grid, 256, 0, st>>>(a);
+}
+
+int check(const ughip_device* dev, const ughip_slice* s, size_t need, const char* what) {
+  if (!s) return set_error(UGHIP_ERR_INVALID, "%s: null slice", what);
+  if (s->dev != dev) return set_error(UGHIP_ERR_INVALID, "%s: slice lives on another device", what);
+  if (s->dtype != UGHIP_F32) return set_error(UGHIP_ERR_UNSUPPORTED, "%s: dtype %s, this entry point is built for F32", what, dtype_name(s->dtype));
+  if (s->len < need) return set_error(UGHIP_ERR_BOUNDS, "%s: slice has %zu elements, op needs %zu", what, s->len, need);
+  return UGHIP_OK;
+}
+
+int check_k(size_t k, const char* what) {
+  if (k == 0 || k % 4 != 0) return set_error(UGHIP_ERR_UNSUPPORTED, "%s: k = %zu is not a positive multiple of 4", what, k);
+  if (k > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "%s: k = %zu is too large", what, k);
+  return UGHIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ughip_gemv_multi(ughip_device* dev, const ughip_slice* x, size_t n_mats, const ughip_slice* const* w, const size_t* n, size_t k, ughip_slice* dst) {
+  if (!dev || !w || !n) return set_error(UGHIP_ERR_INVALID, "gemv_multi: null argument");
+  if (n_mats == 0 || n_mats > 3) return set_error(UGHIP_ERR_INVALID, "gemv_multi: %zu matrices, 1 to 3 are supported", n_mats);
+  if (int rc = check_k(k, "gemv_multi")) return rc;
+  if (int rc = check(dev, x, k, "gemv_multi x")) return rc;
+  size_t total = 0;
+  for (size_t i = 0; i < n_mats; ++i) total += n[i];
+  if (total > 0x7fffffffull / 4) return set_error(UGHIP_ERR_INVALID, "gemv_multi: too many columns");
+  if (int rc = check(dev, dst, total, "gemv_multi dst")) return rc;
+  if (dst == x) return set_error(UGHIP_ERR_INVALID, "gemv_multi: dst aliases x");
+  FusedArgs a{};
+  a.x = static_cast<const float*>(x->ptr);
+  a.k = (int)k;
+  size_t first = 0;
+  for (size_t i = 0; i < 3; ++i) {
+    if (i < n_mats) {
+      if (int rc = check(dev, w[i], n[i] * k, "gemv_multi w")) return rc;
+      if (dst == w[i]) return set_error(UGHIP_ERR_INVALID, "gemv_multi: dst aliases a matrix");
+      a.w[i] = static_cast<const float*>(w[i]->ptr);
+      a.y[i] = static_cast<float*>(dst->ptr) + first;
+      first += n[i];
+    }
+    a.col_end[i] = (int)first;
+  }
+  a.n_cols = (int)total;
+  if (total == 0) return UGHIP_OK;
+  if (int rc = device_activate(dev)) return rc;
+  launch<MODE_MULTI>(dev->stream, a);
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+int ughip_gemv_gate_up(ughip_device* dev, const ughip_slice* x, const ughip_slice* w_gate, const ughip_slice* w_up, ughip_slice* dst, size_t n, size_t k) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "gemv_gate_up: null device");
+  if (int rc = check_k(k, "gemv_gate_up")) return rc;
+  if (n > 0x7fffffffull / 4) return set_error(UGHIP_ERR_INVALID, "gemv_gate_up: too many columns");
+  if (int rc = check(dev, x, k, "gemv_gate_up x")) return rc;
+  if (int rc = check(dev, w_gate, n * k, "gemv_gate_up gate")) return rc;
+  if (int rc = check(dev, w_up, n * k, "gemv_gate_up up")) return rc;
+  if (int rc = check(dev, dst, n, "gemv_gate_up dst")) return rc;
+  if (dst == x || dst == w_gate || dst == w_up) return set_error(UGHIP_ERR_INVALID, "gemv_gate_up: dst aliases an input");
+  if (n == 0) return UGHIP_OK;
+  FusedArgs a{};
+  a.x = static_cast<const float*>(x->ptr);
+  a.w[0] = static_cast<const float*>(w_gate->ptr);
+  a.w[1] = static_cast<const float*>(w_up->ptr);
+  a.y[0] = static_cast<float*>(dst->ptr);
+  a.col_end[0] = a.col_end[1] = a.col_end[2] = a.n_cols = (int)n;
+  a.k = (int)k;
+  if (int rc = device_activate(dev)) return rc;
+  launch<MODE_GATE_UP>(dev->stream, a);
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+int ughip_gemv_add(ughip_device* dev, const ughip_slice* x, const ughip_slice* w, const ughip_slice* residual, ughip_slice* dst, size_t n, size_t k) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "gemv_add: null device");
+  if (int rc = check_k(k, "gemv_add")) return rc;
+  if (n > 0x7fffffffull / 4) return set_error(UGHIP_ERR_INVALID, "gemv_add: too many columns");
+  if (int rc = check(dev, x, k, "gemv_add x")) return rc;
+  if (int rc = check(dev, w, n * k, "gemv_add w")) return rc;
+  if (int rc = check(dev, residual, n, "gemv_add residual")) return rc;
+  if (int rc = check(dev, dst, n, "gemv_add dst")) return rc;
+  if (dst == x || dst == w || dst == residual) return set_error(UGHIP_ERR_INVALID, "gemv_add: dst aliases an input");
+  if (n == 0) return UGHIP_OK;
+  FusedArgs a{};
+  a.x = static_cast<const float*>(x->ptr);
+  a.w[0] = static_cast<const float*>(w->ptr);
+  a.y[0] = static_cast<float*>(dst->ptr);
+  a.col_end[0] = a.col_end[1] = a.col_end[2] = a.n_cols = (int)n;
+  a.k = (int)k;
+  a.residual = static_cast<const float*>(residual->ptr);
+  if (int rc = device_activate(dev)) return rc;
+  launch<MODE_ADD>(dev->stream, a);
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+}  // extern "C"
