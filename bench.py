@@ -300,6 +300,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--extras", action="store_true", help="(default) kept for older command lines")
     ap.add_argument("--llama", action="store_true", help="(default) kept for older command lines")
+    ap.add_argument("--llama-level", type=int, default=None, choices=[0, 1, 2, 3], help="run config 5 at this fusion level only (default: all four)")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-llama", action="store_true")
     ap.add_argument("--headline-only", action="store_true", help="only the config-2 kernel: no extras, no llama, no CPU baseline")
@@ -363,6 +364,8 @@ def main():
     if not (args.no_llama or args.headline_only):
         for key, fused in (("llama_decode_f32", 0), ("llama_decode_f32_fused_attention", 1), ("llama_decode_f32_inplace_cache", 2),
                            ("llama_decode_f32_fused_projections", 3)):
+            if args.llama_level is not None and fused != args.llama_level:
+                continue
             try:
                 line.setdefault("extras", {})[key] = llama_decode(dev, fused_attention=fused)
             except Exception as e:  # noqa: BLE001

@@ -291,6 +291,14 @@ int ughip_gemv_multi(ughip_device* dev, const ughip_slice* x, size_t n_mats,
 /* dst[c] = silu(x . gate[c]) * (x . up[c]), silu(g) = g / (1 + exp(-g)) (model.rs:99-109,160-168). */
 int ughip_gemv_gate_up(ughip_device* dev, const ughip_slice* x, const ughip_slice* w_gate,
                        const ughip_slice* w_up, ughip_slice* dst, size_t n, size_t k);
+/* The two above on rms_norm(x) = x / sqrt(mean(x^2) + eps) * alpha (ug-llama/src/model.rs:32-50)
+ * instead of x: the norms in front of attention, the MLP and the output head.  k <= 4096. */
+int ughip_rms_gemv_multi(ughip_device* dev, const ughip_slice* x, const ughip_slice* alpha, float eps,
+                         size_t n_mats, const ughip_slice* const* w, const size_t* n, size_t k,
+                         ughip_slice* dst);
+int ughip_rms_gemv_gate_up(ughip_device* dev, const ughip_slice* x, const ughip_slice* alpha,
+                           float eps, const ughip_slice* w_gate, const ughip_slice* w_up,
+                           ughip_slice* dst, size_t n, size_t k);
 /* dst[c] = x . w[c] + residual[c] (a projection followed by the residual add, model.rs:366-372). */
 int ughip_gemv_add(ughip_device* dev, const ughip_slice* x, const ughip_slice* w,
                    const ughip_slice* residual, ughip_slice* dst, size_t n, size_t k);

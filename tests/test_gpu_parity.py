@@ -907,6 +907,46 @@ def test_linear_add_fused(hip, cpu, hip_ops, cpu_ops, n, k):
         assert np.all(np.abs(got - sep) <= 2 * tol)
 
 
+@pytest.mark.parametrize("k", [2048, 4096, 260, 1000])
+def test_projections_with_the_norm_folded_in(hip, cpu, hip_ops, cpu_ops, k):
+    """linear_packed / gate_up on rms_norm(x): against rms_norm + matmul_t (+ SwiGLU) op by op on the oracle and against float64."""
+    print("rms projections", k, flush=True)
+    n, eps = 96, 1e-5
+    x, alpha = rng.normal(111, k, 2.0), rng.normal(112, k, 0.5)
+    ws = [rng.normal(113 + i, n * k, 0.05).reshape(n, k) for i in range(3)]
+
+    def packed(dev, ops):
+        return ops.linear_packed(LB.copy(x, (1, 1, k), dev), [LB.copy(w.ravel(), (n, k), dev) for w in ws], LB.copy(alpha, (k,), dev), eps).data_vec()
+
+    def gated(dev, ops):
+        return ops.gate_up(LB.copy(x, (1, 1, k), dev), LB.copy(ws[0].ravel(), (n, k), dev), LB.copy(ws[1].ravel(), (n, k), dev), LB.copy(alpha, (k,), dev), eps).data_vec()
+
+    x6 = x.astype(np.float64)
+    xn = x6 / np.sqrt((x6 * x6).mean() + eps) * alpha
+    wall = np.concatenate(ws, 0)
+    tol = 2 * _gemv_tol(xn.astype(np.float32), wall) + 1e-6 * np.abs(wall.astype(np.float64) @ xn)
+    got, want = packed(hip, hip_ops), packed(cpu, cpu_ops)
+    assert np.all(np.abs(got - wall.astype(np.float64) @ xn) <= tol)
+    assert np.all(np.abs(got - want) <= 2 * tol)
+    g, u = ws[0].astype(np.float64) @ xn, ws[1].astype(np.float64) @ xn
+    sig = 1.0 / (1.0 + np.exp(-g))
+    truth = g * sig * u
+    tol_g = 1.1 * tol[:n] * np.abs(u) + np.abs(g * sig) * tol[n:2 * n] + 4e-7 * np.abs(truth) + 1e-30
+    got, want = gated(hip, hip_ops), gated(cpu, cpu_ops)
+    assert np.all(np.abs(got - truth) <= tol_g)
+    assert np.all(np.abs(got - want) <= 2 * tol_g)
+
+
+def test_projections_with_the_norm_need_a_short_row(hip, hip_ops):
+    """Rows longer than the fused norm keeps in registers take the op-by-op composition."""
+    k, n = 4352, 8
+    x, alpha, w = rng.normal(116, k), rng.normal(117, k, 0.5), rng.normal(118, n * k, 0.05)
+    got = hip_ops.linear_packed(LB.copy(x, (1, 1, k), hip), [LB.copy(w, (n, k), hip)], LB.copy(alpha, (k,), hip), 1e-5).data_vec()
+    x6 = x.astype(np.float64)
+    truth = w.reshape(n, k).astype(np.float64) @ (x6 / np.sqrt((x6 * x6).mean() + 1e-5) * alpha)
+    np.testing.assert_allclose(got, truth, rtol=1e-4, atol=1e-5)
+
+
 def test_fused_projections_fall_back_for_several_rows(hip, cpu, hip_ops, cpu_ops):
     """More than one input row (prefill): the hooks answer with the op-by-op composition on any device."""
     t, k, n = 5, 64, 24

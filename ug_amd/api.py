@@ -691,17 +691,18 @@ class LlamaOps(_Handle):
     def packed_projections(self):
         return bool(host_lib().ugh_llama_packed_projections(_p(self.h)))
 
-    def linear_packed(self, x, ws):
-        """x [b, t, k] against up to three [n_i, k] matrices -> [b, t, sum n_i], results side by side."""
+    def linear_packed(self, x, ws, alpha=None, eps=0.0):
+        """x [b, t, k] against up to three [n_i, k] matrices -> [b, t, sum n_i], results side by side;
+        on rms_norm(x, alpha, eps) when alpha is given."""
         arr = (C.c_void_p * len(ws))(*[w.h for w in ws])
-        lb = self._op("ugh_llama_linear_packed", x, C.c_size_t(len(ws)), arr)
-        lb._keep += list(ws)
+        lb = self._op("ugh_llama_linear_packed", x, C.c_size_t(len(ws)), arr, _p(alpha.h) if alpha is not None else None, C.c_float(eps))
+        lb._keep += list(ws) + ([alpha] if alpha is not None else [])
         return lb
 
-    def gate_up(self, x, w_gate, w_up):
-        """silu(x gate^T) * (x up^T)"""
-        lb = self._op("ugh_llama_gate_up", x, _p(w_gate.h), _p(w_up.h))
-        lb._keep += [w_gate, w_up]
+    def gate_up(self, x, w_gate, w_up, alpha=None, eps=0.0):
+        """silu(x gate^T) * (x up^T); on rms_norm(x, alpha, eps) when alpha is given."""
+        lb = self._op("ugh_llama_gate_up", x, _p(w_gate.h), _p(w_up.h), _p(alpha.h) if alpha is not None else None, C.c_float(eps))
+        lb._keep += [w_gate, w_up] + ([alpha] if alpha is not None else [])
         return lb
 
     def linear_add(self, x, w, residual):

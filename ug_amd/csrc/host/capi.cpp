@@ -477,15 +477,15 @@ int ugh_llama_attention_cached(void* ops, void* q, void* k, void* v, size_t s, f
   });
 }
 int ugh_llama_packed_projections(void* ops) { return ops_of(ops).packed_projections() ? 1 : 0; }
-int ugh_llama_linear_packed(void* ops, void* x, size_t n_mats, void** ws, void** out) {
+int ugh_llama_linear_packed(void* ops, void* x, size_t n_mats, void** ws, void* alpha, float eps, void** out) {
   return guard([&] {
     std::vector<ug::LazyBuffer> w;
     for (size_t i = 0; i < n_mats; ++i) w.push_back(lb_of(ws[i]));
-    *out = box(ops_of(ops).linear_packed(lb_of(x), w));
+    *out = box(ops_of(ops).linear_packed(lb_of(x), w, alpha ? &lb_of(alpha) : nullptr, eps));
   });
 }
-int ugh_llama_gate_up(void* ops, void* x, void* w_gate, void* w_up, void** out) {
-  return guard([&] { *out = box(ops_of(ops).gate_up(lb_of(x), lb_of(w_gate), lb_of(w_up))); });
+int ugh_llama_gate_up(void* ops, void* x, void* w_gate, void* w_up, void* alpha, float eps, void** out) {
+  return guard([&] { *out = box(ops_of(ops).gate_up(lb_of(x), lb_of(w_gate), lb_of(w_up), alpha ? &lb_of(alpha) : nullptr, eps)); });
 }
 int ugh_llama_linear_add(void* ops, void* x, void* w, void* residual, void** out) {
   return guard([&] { *out = box(ops_of(ops).linear_add(lb_of(x), lb_of(w), lb_of(residual))); });

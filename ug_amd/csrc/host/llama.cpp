@@ -239,10 +239,15 @@ struct HipOps : Ops {
     return true;
   }
 
-  LB linear_packed(const LB& x, const std::vector<LB>& ws) const override {
+  // the fused norm keeps the row in registers
+  static bool rms_ok(const LB& x, const LB* alpha) {
+    return !alpha || (x.dims()[2] <= 4096 && alpha->dtype() == DType::F32 && alpha->elem_count() == x.dims()[2]);
+  }
+
+  LB linear_packed(const LB& x, const std::vector<LB>& ws, const LB* alpha, float eps) const override {
     std::vector<const LB*> wp;
     for (const LB& w : ws) wp.push_back(&w);
-    if (ws.empty() || ws.size() > 3 || !one_f32_row(x, wp)) return Ops::linear_packed(x, ws);
+    if (ws.empty() || ws.size() > 3 || !one_f32_row(x, wp) || !rms_ok(x, alpha)) return Ops::linear_packed(x, ws, alpha, eps);
     std::vector<size_t> ns;
     size_t total = 0, k = x.dims()[2];
     for (const LB& w : ws) {
@@ -251,26 +256,35 @@ struct HipOps : Ops {
     }
     ughip_device* dev = hip_dev(x);
     size_t n_mats = ws.size();
+    const bool norm = alpha != nullptr;
     auto f = [=](const std::vector<Slice*>& vs) {
-      if (vs.size() != n_mats + 2) bail("linear_packed: unexpected number of slices");
+      if (vs.size() != n_mats + 2 + (norm ? 1 : 0)) bail("linear_packed: unexpected number of slices");
       const ughip_slice* w[3] = {nullptr, nullptr, nullptr};
       for (size_t i = 0; i < n_mats; ++i) w[i] = hip_raw_slice(*vs[1 + i]);
-      hip_check(ughip_gemv_multi(dev, hip_raw_slice(*vs[0]), n_mats, w, ns.data(), k, hip_raw_slice(*vs.back())), "linear_packed");
+      hip_check(ughip_rms_gemv_multi(dev, hip_raw_slice(*vs[0]), norm ? hip_raw_slice(*vs[1 + n_mats]) : nullptr, eps, n_mats, w, ns.data(), k,
+                                     hip_raw_slice(*vs.back())),
+                "linear_packed");
     };
     std::vector<LB> args = {x};
     for (const LB& w : ws) args.push_back(w);
+    if (norm) args.push_back(*alpha);
     return LB::custom(f, args, Shape({1, 1, total}), x.dtype(), x.device());
   }
 
-  LB gate_up(const LB& x, const LB& w_gate, const LB& w_up) const override {
-    if (!one_f32_row(x, {&w_gate, &w_up}) || w_gate.dims() != w_up.dims()) return Ops::gate_up(x, w_gate, w_up);
+  LB gate_up(const LB& x, const LB& w_gate, const LB& w_up, const LB* alpha, float eps) const override {
+    if (!one_f32_row(x, {&w_gate, &w_up}) || w_gate.dims() != w_up.dims() || !rms_ok(x, alpha)) return Ops::gate_up(x, w_gate, w_up, alpha, eps);
     size_t n = w_gate.dims()[0], k = x.dims()[2];
     ughip_device* dev = hip_dev(x);
+    const bool norm = alpha != nullptr;
     auto f = [=](const std::vector<Slice*>& vs) {
-      if (vs.size() != 4) bail("gate_up: expected 4 slices");
-      hip_check(ughip_gemv_gate_up(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), hip_raw_slice(*vs[3]), n, k), "gate_up");
+      if (vs.size() != (norm ? 5u : 4u)) bail("gate_up: unexpected number of slices");
+      hip_check(ughip_rms_gemv_gate_up(dev, hip_raw_slice(*vs[0]), norm ? hip_raw_slice(*vs[3]) : nullptr, eps, hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]),
+                                       hip_raw_slice(*vs.back()), n, k),
+                "gate_up");
     };
-    return LB::custom(f, {x, w_gate, w_up}, Shape({1, 1, n}), x.dtype(), x.device());
+    std::vector<LB> args = {x, w_gate, w_up};
+    if (norm) args.push_back(*alpha);
+    return LB::custom(f, args, Shape({1, 1, n}), x.dtype(), x.device());
   }
 
   LB linear_add(const LB& x, const LB& w, const LB& residual) const override {
@@ -387,15 +401,19 @@ LB Ops::attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float 
 }
 
 // model.rs:206-208 side by side.
-LB Ops::linear_packed(const LB& x, const std::vector<LB>& ws) const {
+LB Ops::linear_packed(const LB& x0, const std::vector<LB>& ws, const LB* alpha, float eps) const {
   if (ws.empty()) bail("linear_packed: no matrices");
+  LB x = alpha ? rms_norm(x0, *alpha, eps) : x0;
   LB out = x.matmul_t(ws[0]);
   for (size_t i = 1; i < ws.size(); ++i) out = cat(out, x.matmul_t(ws[i]), x.rank() - 1);
   return out;
 }
 
 // model.rs:160-168 up to the down projection.
-LB Ops::gate_up(const LB& x, const LB& w_gate, const LB& w_up) const { return silu(x.matmul_t(w_gate)).binary(BinaryOp::Mul, x.matmul_t(w_up)); }
+LB Ops::gate_up(const LB& x0, const LB& w_gate, const LB& w_up, const LB* alpha, float eps) const {
+  LB x = alpha ? rms_norm(x0, *alpha, eps) : x0;
+  return silu(x.matmul_t(w_gate)).binary(BinaryOp::Mul, x.matmul_t(w_up));
+}
 
 // model.rs:366-372: a projection, then the residual.
 LB Ops::linear_add(const LB& x, const LB& w, const LB& residual) const { return x.matmul_t(w).binary(BinaryOp::Add, residual); }
@@ -578,20 +596,22 @@ Model::Model(const Config& cfg, bool custom_softmax, WeightSource& w, const Devi
 }
 
 // model.rs:203-248
-LB Model::attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache, const LB* residual) const {
-  if (xs.rank() != 3) bail("attention: expected [b, t, hidden]");
-  size_t seq_len = xs.dims()[1];
+LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache, const LB* residual, bool norm_first) const {
+  if (xs_in.rank() != 3) bail("attention: expected [b, t, hidden]");
+  size_t seq_len = xs_in.dims()[1];
   size_t nh = cfg_.num_attention_heads, nkv = cfg_.num_key_value_heads, hd = cfg_.head_dim();
+  const float eps = (float)cfg_.rms_norm_eps;
   auto finish = [&](const LB& out) { return residual ? ops_->linear_add(out, l.o_proj, *residual) : out.matmul_t(l.o_proj); };
-  if (fused_attention_ >= 3 && seq_len == 1 && xs.dims()[0] == 1 && cache.capacity && ops_->packed_projections()) {
-    // one position: q | k | v come out of one launch side by side and are read where they lie
+  if (fused_attention_ >= 3 && seq_len == 1 && xs_in.dims()[0] == 1 && cache.capacity && ops_->packed_projections()) {
+    // one position: q | k | v come out of one launch (with the norm in front) side by side and are read where they lie
     const size_t nq = nh * hd, nk = nkv * hd, row = nq + 2 * nk, len = cache.len;
-    LB qkv = ops_->linear_packed(xs, {l.q_proj, l.k_proj, l.v_proj});
+    LB qkv = ops_->linear_packed(xs_in, {l.q_proj, l.k_proj, l.v_proj}, norm_first ? &l.rms1 : nullptr, eps);
     LB kc = ops_->kv_append(cache.prev_k, len, qkv, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, nq, row);
     LB vc = ops_->kv_append(cache.prev_v, len, qkv, nullptr, nullptr, nullptr, false, nq + nk, row);
     cache.len = len + 1;
     return finish(ops_->attention_cached(qkv, kc, vc, cache.len, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, 0, row, nh));
   }
+  LB xs = norm_first ? rms_norm(xs_in, l.rms1, eps) : xs_in;
   LB q = xs.matmul_t(l.q_proj);
   LB k = xs.matmul_t(l.k_proj);
   LB v = xs.matmul_t(l.v_proj);
@@ -650,8 +670,9 @@ LB Model::attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache, c
 }
 
 // model.rs:160-168
-LB Model::mlp(const Layer& l, const LB& xs, const LB* residual) const {
-  if (residual) return ops_->linear_add(ops_->gate_up(xs, l.gate_proj, l.up_proj), l.down_proj, *residual);
+LB Model::mlp(const Layer& l, const LB& xs, const LB* residual, bool norm_first) const {
+  if (residual)
+    return ops_->linear_add(ops_->gate_up(xs, l.gate_proj, l.up_proj, norm_first ? &l.rms2 : nullptr, (float)cfg_.rms_norm_eps), l.down_proj, *residual);
   LB xs1 = xs.matmul_t(l.gate_proj);
   LB xs2 = xs.matmul_t(l.up_proj);
   xs1 = silu(xs1);
@@ -670,19 +691,21 @@ LB Model::fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const 
   for (size_t i = 0; i < layers_.size(); ++i) {
     const Layer& l = layers_[i];
     LB residual = xs;
-    LB h = rms_norm(xs, l.rms1, eps);
     if (fused_attention_ >= 3) {
-      h = attention(l, h, pos, cache[i], &residual);
-      xs = mlp(l, rms_norm(h, l.rms2, eps), &h);
+      // the norms travel with the projections behind them, the residual adds with the ones in front
+      LB h = attention(l, xs, pos, cache[i], &residual, true);
+      xs = mlp(l, h, &h, true);
       continue;
     }
-    h = attention(l, h, pos, cache[i], nullptr);
+    LB h = rms_norm(xs, l.rms1, eps);
+    h = attention(l, h, pos, cache[i], nullptr, false);
     h = h.binary(BinaryOp::Add, residual);
     residual = h;
     LB m = rms_norm(h, l.rms2, eps);
-    m = mlp(l, m, nullptr);
+    m = mlp(l, m, nullptr, false);
     xs = m.binary(BinaryOp::Add, residual);
   }
+  if (fused_attention_ >= 3) return ops_->linear_packed(xs, {embedding_}, &ln_f_, eps);
   xs = rms_norm(xs, ln_f_, eps);
   return xs.matmul_t(embedding_);
 }

@@ -65,10 +65,11 @@ struct Ops {
   // packed_projections(): linear_packed gives q|k|v side by side in one buffer and kv_append /
   // attention_cached read their part of it in place.
   virtual bool packed_projections() const { return false; }
-  // x [b, t, k] against up to three [n_i, k] matrices -> [b, t, n_0 + n_1 + n_2].
-  virtual LB linear_packed(const LB& x, const std::vector<LB>& ws) const;
-  // silu(x gate^T) * (x up^T)
-  virtual LB gate_up(const LB& x, const LB& w_gate, const LB& w_up) const;
+  // x [b, t, k] against up to three [n_i, k] matrices -> [b, t, n_0 + n_1 + n_2].  alpha != nullptr:
+  // on rms_norm(x, *alpha, eps) instead of x (the norm in front of the projection folded in).
+  virtual LB linear_packed(const LB& x, const std::vector<LB>& ws, const LB* alpha = nullptr, float eps = 0.f) const;
+  // silu(x gate^T) * (x up^T), x normalised first when alpha != nullptr
+  virtual LB gate_up(const LB& x, const LB& w_gate, const LB& w_up, const LB* alpha = nullptr, float eps = 0.f) const;
   // x w^T + residual
   virtual LB linear_add(const LB& x, const LB& w, const LB& residual) const;
 };
@@ -139,9 +140,9 @@ class Model {
   // 2: Ops::kv_append + Ops::attention_cached for any number of positions; with a device that
   //    preallocates (Ops::kv_cache_capacity) the caches are written in place and scores never
   //    reach memory.
-  // 3: 2, and the projections through Ops::linear_packed (q|k|v), Ops::gate_up and
-  //    Ops::linear_add (o_proj / down_proj with the residual): 8 schedule items per layer and
-  //    decode step on a device that fuses them.
+  // 3: 2, and the projections through Ops::linear_packed (norm + q|k|v, norm + output head),
+  //    Ops::gate_up (norm + gate, up, SwiGLU) and Ops::linear_add (o_proj / down_proj with the
+  //    residual): 7 schedule items per layer and decode step on a device that fuses them.
   void set_fused_attention(int level) { fused_attention_ = level; }
   int fused_attention() const { return fused_attention_; }
   // Caches of the kind fwd() expects at the current fusion level.
@@ -157,9 +158,10 @@ class Model {
     LB q_proj, k_proj, v_proj, o_proj;
     LB gate_proj, up_proj, down_proj;
   };
-  // residual != nullptr: the result includes the residual add (fusion level 3)
-  LB attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache, const LB* residual) const;
-  LB mlp(const Layer& l, const LB& xs, const LB* residual) const;
+  // residual != nullptr: the result includes the residual add; norm_first: xs still has to go
+  // through the layer's RMSNorm (fusion level 3 folds both into the projections)
+  LB attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache, const LB* residual, bool norm_first) const;
+  LB mlp(const Layer& l, const LB& xs, const LB* residual, bool norm_first) const;
   Config cfg_;
   bool custom_softmax_;
   int fused_attention_ = 0;

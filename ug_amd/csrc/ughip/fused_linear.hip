@@ -6,6 +6,8 @@
 //   ughip_gemv_gate_up  y = silu(x G^T) * (x U^T), silu(g) = g / (1 + exp(-g))
 //                       (model.rs:160-168 up to the down projection, written as in model.rs:99-109)
 //   ughip_gemv_add      y = x W^T + r   (o_proj / down_proj followed by the residual add, model.rs:366-372)
+//   ughip_rms_gemv_multi, ughip_rms_gemv_gate_up: the first two with RMSNorm (model.rs:32-50) applied to x
+//                       on the way in (the norms in front of attention, the MLP and the output head)
 //
 // One token's projections are 6-46 MB matrix streams behind 2-3 us launches; these entry points
 // remove launches and the small vectors that would travel between them, nothing else: every
@@ -37,6 +39,8 @@ struct FusedArgs {
   int n_cols;      // columns of the grid
   int k;
   const float* residual;
+  const float* alpha;  // RMS variants: y uses x / sqrt(mean(x^2) + eps) * alpha in place of x
+  float eps;
 };
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -129,6 +133,94 @@ __global__ void __launch_bounds__(256) fused_gemv(FusedArgs a) {
   else *Y = acc0;
 }
 
+// The same with RMSNorm (ug-llama/src/model.rs:32-50: x / sqrt(mean(x^2) + eps) * alpha) applied to x
+// first.  The row is short (k <= 256 * RMS_SLABS floats): every wave sums its squares itself, then
+// keeps the normalised slabs it multiplies in registers, so the matrix loads of a wave are all
+// in flight at once.
+constexpr int RMS_SLABS = 16;
+
+template <int KS, int MODE, int SLABS>
+__global__ void __launch_bounds__(256) fused_rms_gemv(FusedArgs a) {
+  constexpr int NVW = SLABS / KS;  // slabs of 256 floats per wave
+  __shared__ float part[4][2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = blockIdx.x * (4 / KS) + wave / KS, ks = wave % KS;
+  const bool live = col < a.n_cols;
+  const float* __restrict__ X = a.x;
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < SLABS; ++i) {
+    const int k = (i * 64 + lane) * 4;
+    if (k < a.k) {
+      const f32x4 x = *reinterpret_cast<const f32x4*>(X + k);
+      ss += x.x * x.x;
+      ss += x.y * x.y;
+      ss += x.z * x.z;
+      ss += x.w * x.w;
+    }
+  }
+  ss = wave_sum(ss);
+  const float m = sqrtf(ss * (1.f / (float)a.k) + a.eps);
+  f32x4 xv[NVW];
+#pragma unroll
+  for (int j = 0; j < NVW; ++j) {
+    const int k = ((j * KS + ks) * 64 + lane) * 4;
+    xv[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (k < a.k) {
+      const f32x4 x = *reinterpret_cast<const f32x4*>(X + k), al = *reinterpret_cast<const f32x4*>(a.alpha + k);
+      xv[j] = f32x4{x.x / m * al.x, x.y / m * al.y, x.z / m * al.z, x.w / m * al.w};
+    }
+  }
+  float acc0 = 0.f, acc1 = 0.f;
+  float* __restrict__ Y = nullptr;
+  if (live) {
+    int mtx = 0, first = 0;
+    if (MODE == MODE_MULTI) {
+      if (col >= a.col_end[0]) mtx = 1, first = a.col_end[0];
+      if (col >= a.col_end[1]) mtx = 2, first = a.col_end[1];
+    }
+    const int row = col - first;
+    const float* __restrict__ W0 = a.w[mtx] + (size_t)row * a.k;
+    const float* __restrict__ W1 = MODE == MODE_GATE_UP ? a.w[1] + (size_t)row * a.k : nullptr;
+    Y = a.y[mtx] + row;
+    f32x4 w0[NVW], w1[NVW];
+#pragma unroll
+    for (int j = 0; j < NVW; ++j) {
+      const int k = ((j * KS + ks) * 64 + lane) * 4;
+      w0[j] = w1[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (k < a.k) {
+        w0[j] = *reinterpret_cast<const f32x4*>(W0 + k);
+        if (MODE == MODE_GATE_UP) w1[j] = *reinterpret_cast<const f32x4*>(W1 + k);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NVW; ++j) {
+      acc0 = dot4(w0[j], xv[j], acc0);
+      if (MODE == MODE_GATE_UP) acc1 = dot4(w1[j], xv[j], acc1);
+    }
+  }
+  acc0 = wave_sum(acc0);
+  if (MODE == MODE_GATE_UP) acc1 = wave_sum(acc1);
+  if (KS > 1) {
+    if (lane == 0) {
+      part[wave][0] = acc0;
+      part[wave][1] = acc1;
+    }
+    __syncthreads();
+    if (ks != 0) return;
+    acc0 = part[wave][0];
+    acc1 = part[wave][1];
+#pragma unroll
+    for (int j = 1; j < KS; ++j) {
+      acc0 += part[wave + j][0];
+      acc1 += part[wave + j][1];
+    }
+  }
+  if (!live || lane != 0) return;
+  if (MODE == MODE_GATE_UP) *Y = acc0 / (1.f + expf(-acc0)) * acc1;
+  else *Y = acc0;
+}
+
 int pick_ks(size_t cols, size_t k) {
   // enough waves to hide HBM latency: about 8192 over the chip
   int ks = cols <= 2048 ? 4 : cols <= 6144 ? 2 : 1;
@@ -143,6 +235,15 @@ void launch(hipStream_t st, const FusedArgs& a) {
   const int ks = pick_ks((size_t)a.n_cols * (MODE == MODE_GATE_UP ? 2 : 1), (size_t)a.k);
   const unsigned per_wg = 4 / ks;
   const unsigned grid = ((unsigned)a.n_cols + per_wg - 1) / per_wg;
+  if (a.alpha) {
+    if (MODE == MODE_ADD) return;  // not built (the residual projections read attention / SwiGLU outputs, not a norm)
+    constexpr int M = MODE == MODE_ADD ? MODE_MULTI : MODE;
+    const bool small = a.k <= 256 * 8;
+    if (ks == 4) small ? fused_rms_gemv<4, M, 8><<<grid, 256, 0, st>>>(a) : fused_rms_gemv<4, M, 16><<<grid, 256, 0, st>>>(a);
+    else if (ks == 2) small ? fused_rms_gemv<2, M, 8><<<grid, 256, 0, st>>>(a) : fused_rms_gemv<2, M, 16><<<grid, 256, 0, st>>>(a);
+    else small ? fused_rms_gemv<1, M, 8><<<grid, 256, 0, st>>>(a) : fused_rms_gemv<1, M, 16><<<grid, 256, 0, st>>>(a);
+    return;
+  }
   if (ks == 4) fused_gemv<4, MODE><<<grid, 256, 0, st>>>(a);
   else if (ks == 2) fused_gemv<2, MODE><<<grid, 256, 0, st>>>(a);
   else fused_gemv<1, MODE><<<grid, 256, 0, st>>>(a);
@@ -166,8 +267,23 @@ int check_k(size_t k, const char* what) {
 
 extern "C" {
 
+namespace {
+// alpha == nullptr: no norm.  Otherwise the row has to fit the registers of the RMS kernels.
+int check_rms(const ughip_device* dev, const ughip_slice* alpha, size_t k, const char* what) {
+  if (!alpha) return UGHIP_OK;
+  if (k > (size_t)256 * RMS_SLABS) return set_error(UGHIP_ERR_UNSUPPORTED, "%s: rows of %zu elements, the fused norm is built for up to %d", what, k, 256 * RMS_SLABS);
+  return check(dev, alpha, k, what);
+}
+}  // namespace
+
 int ughip_gemv_multi(ughip_device* dev, const ughip_slice* x, size_t n_mats, const ughip_slice* const* w, const size_t* n, size_t k, ughip_slice* dst) {
+  return ughip_rms_gemv_multi(dev, x, nullptr, 0.f, n_mats, w, n, k, dst);
+}
+
+int ughip_rms_gemv_multi(ughip_device* dev, const ughip_slice* x, const ughip_slice* alpha, float eps, size_t n_mats, const ughip_slice* const* w,
+                         const size_t* n, size_t k, ughip_slice* dst) {
   if (!dev || !w || !n) return set_error(UGHIP_ERR_INVALID, "gemv_multi: null argument");
+  if (int rc = check_rms(dev, alpha, k, "gemv_multi alpha")) return rc;
   if (n_mats == 0 || n_mats > 3) return set_error(UGHIP_ERR_INVALID, "gemv_multi: %zu matrices, 1 to 3 are supported", n_mats);
   if (int rc = check_k(k, "gemv_multi")) return rc;
   if (int rc = check(dev, x, k, "gemv_multi x")) return rc;
@@ -179,6 +295,8 @@ int ughip_gemv_multi(ughip_device* dev, const ughip_slice* x, size_t n_mats, con
   FusedArgs a{};
   a.x = static_cast<const float*>(x->ptr);
   a.k = (int)k;
+  a.alpha = alpha ? static_cast<const float*>(alpha->ptr) : nullptr;
+  a.eps = eps;
   size_t first = 0;
   for (size_t i = 0; i < 3; ++i) {
     if (i < n_mats) {
@@ -199,7 +317,13 @@ int ughip_gemv_multi(ughip_device* dev, const ughip_slice* x, size_t n_mats, con
 }
 
 int ughip_gemv_gate_up(ughip_device* dev, const ughip_slice* x, const ughip_slice* w_gate, const ughip_slice* w_up, ughip_slice* dst, size_t n, size_t k) {
+  return ughip_rms_gemv_gate_up(dev, x, nullptr, 0.f, w_gate, w_up, dst, n, k);
+}
+
+int ughip_rms_gemv_gate_up(ughip_device* dev, const ughip_slice* x, const ughip_slice* alpha, float eps, const ughip_slice* w_gate, const ughip_slice* w_up,
+                           ughip_slice* dst, size_t n, size_t k) {
   if (!dev) return set_error(UGHIP_ERR_INVALID, "gemv_gate_up: null device");
+  if (int rc = check_rms(dev, alpha, k, "gemv_gate_up alpha")) return rc;
   if (int rc = check_k(k, "gemv_gate_up")) return rc;
   if (n > 0x7fffffffull / 4) return set_error(UGHIP_ERR_INVALID, "gemv_gate_up: too many columns");
   if (int rc = check(dev, x, k, "gemv_gate_up x")) return rc;
@@ -212,6 +336,8 @@ int ughip_gemv_gate_up(ughip_device* dev, const ughip_slice* x, const ughip_slic
   a.x = static_cast<const float*>(x->ptr);
   a.w[0] = static_cast<const float*>(w_gate->ptr);
   a.w[1] = static_cast<const float*>(w_up->ptr);
+  a.alpha = alpha ? static_cast<const float*>(alpha->ptr) : nullptr;
+  a.eps = eps;
   a.y[0] = static_cast<float*>(dst->ptr);
   a.col_end[0] = a.col_end[1] = a.col_end[2] = a.n_cols = (int)n;
   a.k = (int)k;
