@@ -134,45 +134,24 @@ __global__ void __launch_bounds__(256) fused_gemv(FusedArgs a) {
 }
 
 // The same with RMSNorm (ug-llama/src/model.rs:32-50: x / sqrt(mean(x^2) + eps) * alpha) applied to x
-// first.  The row is short (k <= 256 * RMS_SLABS floats): every wave sums its squares itself, then
-// keeps the normalised slabs it multiplies in registers, so the matrix loads of a wave are all
-// in flight at once.
+// first.  The row is short (k <= 256 * RMS_SLABS floats): a wave requests all of its matrix loads,
+// the workgroup normalises the row once into LDS in their shadow, then every wave multiplies.
 constexpr int RMS_SLABS = 16;
 
 template <int KS, int MODE, int SLABS>
 __global__ void __launch_bounds__(256) fused_rms_gemv(FusedArgs a) {
   constexpr int NVW = SLABS / KS;  // slabs of 256 floats per wave
   __shared__ float part[4][2];
+  __shared__ float ssum[4];
+  __shared__ f32x4 xs[SLABS * 64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = blockIdx.x * (4 / KS) + wave / KS, ks = wave % KS;
   const bool live = col < a.n_cols;
-  const float* __restrict__ X = a.x;
-  float ss = 0.f;
-#pragma unroll
-  for (int i = 0; i < SLABS; ++i) {
-    const int k = (i * 64 + lane) * 4;
-    if (k < a.k) {
-      const f32x4 x = *reinterpret_cast<const f32x4*>(X + k);
-      ss += x.x * x.x;
-      ss += x.y * x.y;
-      ss += x.z * x.z;
-      ss += x.w * x.w;
-    }
-  }
-  ss = wave_sum(ss);
-  const float m = sqrtf(ss * (1.f / (float)a.k) + a.eps);
-  f32x4 xv[NVW];
-#pragma unroll
-  for (int j = 0; j < NVW; ++j) {
-    const int k = ((j * KS + ks) * 64 + lane) * 4;
-    xv[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (k < a.k) {
-      const f32x4 x = *reinterpret_cast<const f32x4*>(X + k), al = *reinterpret_cast<const f32x4*>(a.alpha + k);
-      xv[j] = f32x4{x.x / m * al.x, x.y / m * al.y, x.z / m * al.z, x.w / m * al.w};
-    }
-  }
-  float acc0 = 0.f, acc1 = 0.f;
+  // the matrix rows are requested first: they are the long pole, the norm below runs in their shadow
   float* __restrict__ Y = nullptr;
+  f32x4 w0[NVW], w1[NVW];
+#pragma unroll
+  for (int j = 0; j < NVW; ++j) w0[j] = w1[j] = f32x4{0.f, 0.f, 0.f, 0.f};
   if (live) {
     int mtx = 0, first = 0;
     if (MODE == MODE_MULTI) {
@@ -183,20 +162,53 @@ __global__ void __launch_bounds__(256) fused_rms_gemv(FusedArgs a) {
     const float* __restrict__ W0 = a.w[mtx] + (size_t)row * a.k;
     const float* __restrict__ W1 = MODE == MODE_GATE_UP ? a.w[1] + (size_t)row * a.k : nullptr;
     Y = a.y[mtx] + row;
-    f32x4 w0[NVW], w1[NVW];
 #pragma unroll
     for (int j = 0; j < NVW; ++j) {
       const int k = ((j * KS + ks) * 64 + lane) * 4;
-      w0[j] = w1[j] = f32x4{0.f, 0.f, 0.f, 0.f};
       if (k < a.k) {
         w0[j] = *reinterpret_cast<const f32x4*>(W0 + k);
         if (MODE == MODE_GATE_UP) w1[j] = *reinterpret_cast<const f32x4*>(W1 + k);
       }
     }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // the workgroup normalises the row once, into LDS: thread t owns elements 4 t .. 4 t + 3 of every 1024
+  const float* __restrict__ X = a.x;
+  constexpr int PER_T = SLABS / 4;
+  f32x4 xl[PER_T];
+  float ss = 0.f;
 #pragma unroll
-    for (int j = 0; j < NVW; ++j) {
-      acc0 = dot4(w0[j], xv[j], acc0);
-      if (MODE == MODE_GATE_UP) acc1 = dot4(w1[j], xv[j], acc1);
+  for (int i = 0; i < PER_T; ++i) {
+    const int k = (i * 256 + (int)threadIdx.x) * 4;
+    xl[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (k < a.k) xl[i] = *reinterpret_cast<const f32x4*>(X + k);
+    ss += xl[i].x * xl[i].x;
+    ss += xl[i].y * xl[i].y;
+    ss += xl[i].z * xl[i].z;
+    ss += xl[i].w * xl[i].w;
+  }
+  ss = wave_sum(ss);
+  if (lane == 0) ssum[wave] = ss;
+  __syncthreads();
+  ss = (ssum[0] + ssum[1]) + (ssum[2] + ssum[3]);
+  const float m = sqrtf(ss * (1.f / (float)a.k) + a.eps);
+#pragma unroll
+  for (int i = 0; i < PER_T; ++i) {
+    const int k = (i * 256 + (int)threadIdx.x) * 4;
+    if (k < a.k) {
+      const f32x4 al = *reinterpret_cast<const f32x4*>(a.alpha + k);
+      xs[i * 256 + threadIdx.x] = f32x4{xl[i].x / m * al.x, xl[i].y / m * al.y, xl[i].z / m * al.z, xl[i].w / m * al.w};
+    }
+  }
+  __syncthreads();
+  float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+  for (int j = 0; j < NVW; ++j) {
+    const int k4 = (j * KS + ks) * 64 + lane;
+    if (k4 * 4 < a.k) {
+      const f32x4 xn = xs[k4];
+      acc0 = dot4(w0[j], xn, acc0);
+      if (MODE == MODE_GATE_UP) acc1 = dot4(w1[j], xn, acc1);
     }
   }
   acc0 = wave_sum(acc0);
