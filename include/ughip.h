@@ -303,6 +303,15 @@ int ughip_rms_gemv_gate_up(ughip_device* dev, const ughip_slice* x, const ughip_
 int ughip_gemv_add(ughip_device* dev, const ughip_slice* x, const ughip_slice* w,
                    const ughip_slice* residual, ughip_slice* dst, size_t n, size_t k);
 
+/* ---- greedy step on the device ----------------------------------------------------------------
+ * Row `row` of logits [rows, n] (F32): the index of its largest value (the lowest index among
+ * equal values -- what a host loop with `>` finds) goes to token[0] (I32; NULL: skipped) and to
+ * ids[slot]; the largest value and the largest of the rest go to vals[2 * slot], vals[2 * slot + 1].
+ * Lets a greedy decoder (the loop of ug-llama/src/main.rs:125-153 with argmax in place of sampling)
+ * queue step i + 1 behind step i without reading the logits back in between. */
+int ughip_argmax_row(ughip_device* dev, const ughip_slice* logits, size_t n, size_t row,
+                     ughip_slice* token, ughip_slice* ids, ughip_slice* vals, size_t slot);
+
 /* ---- element type conversion ------------------------------------------------------------------
  * dst[i] = (dtype of dst) src[i], same length, any pair of the five dtypes.  Replaces the host
  * loops of ug-core/src/safetensors.rs:141-271 (load_with_cast converts on the CPU, then uploads):

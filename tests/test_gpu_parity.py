@@ -993,6 +993,53 @@ def test_packed_rows_feed_cache_and_attention(hip, hip_ops):
         hip_ops.kv_append(LB.copy(store_k, (1, nkv, cap, d), hip), length, LB.copy(qkv, (1, 1, row), hip), x_offset=nq + nk + 4, x_row_stride=row).data_vec()
 
 
+# ---- greedy step on the device ------------------------------------------------------------------------------------------
+def _host_top2(row):
+    """The host loop of the read-back decoder: first index of the maximum, largest of the rest."""
+    best, second = 0, -np.inf
+    for i in range(1, row.size):
+        if row[i] > row[best]:
+            second, best = row[best], i
+        elif row[i] > second:
+            second = row[i]
+    return best, float(row[best]), float(second)
+
+
+@pytest.mark.parametrize("rows,n,row", [(1, 32000, 0), (3, 1000, 2), (2, 7, 1), (1, 1, 0), (1, 5000, 0)])
+def test_argmax_into(hip, hip_ops, rows, n, row):
+    assert hip_ops.device_argmax()
+    x = rng.normal(121, rows * n).reshape(rows, n)
+    if n > 100:
+        x[row, 17] = x[row, 90] = x[row].max() + 1.0          # a tie for the maximum: the lower index wins, the other is "the rest"
+    token = LB.copy(np.array([-1], np.int32), (1, 1), hip)
+    ids = LB.copy(np.full(4, -7, np.int32), (4,), hip)
+    vals = LB.copy(np.zeros(8, np.float32), (8,), hip)
+    for lb in (token, ids, vals):
+        lb.realize()
+    out = hip_ops.argmax_into(token, LB.copy(x.ravel(), (1, rows, n), hip), row, ids, vals, 2)
+    got = int(out.data_vec()[0])
+    best, bv, sv = _host_top2(x[row])
+    assert got == best and int(token.data_vec()[0]) == best
+    assert ids.data_vec().tolist() == [-7, -7, best, -7]
+    v = vals.data_vec()
+    assert v[4] == np.float32(bv) and (v[5] == np.float32(sv) or (n == 1 and v[5] == -np.inf))
+    assert np.all(v[:4] == 0) and np.all(v[6:] == 0)
+
+
+@pytest.mark.parametrize("level", [0, 3])
+def test_queued_greedy_decode_matches_the_read_back_loop(hip, hip_ops, level, monkeypatch):
+    """Tokens picked on the device and fed to the next step without a read-back: same ids and
+    margins as the loop that copies the logits to the host for every token."""
+    cfg = ug_amd.LlamaConfig(num_hidden_layers=2, max_position_embeddings=256)
+    prompt = rng.token_ids(10, 16, cfg.vocab_size)
+    model = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=0.02, fused_attention=level)
+    ids_q, st_q = model.generate(prompt, 12)
+    monkeypatch.setenv("UG_LLAMA_HOST_ARGMAX", "1")
+    ids_h, st_h = model.generate(prompt, 12)
+    assert ids_q.tolist() == ids_h.tolist()
+    np.testing.assert_array_equal(st_q["margins"], st_h["margins"])
+
+
 # ---- safetensors: upload in the stored dtype, convert on the device ----------------------------------------------------
 @pytest.mark.parametrize("dst", ["BF16", "F16", "F32", "I32", "I64"])
 @pytest.mark.parametrize("src", ["BF16", "F16", "F32", "I32", "I64"])

@@ -688,6 +688,15 @@ class LlamaOps(_Handle):
         lb._keep += [k, v] + ([cos, sin, pos] if rope else [])
         return lb
 
+    def device_argmax(self):
+        return bool(host_lib().ugh_llama_device_argmax(_p(self.h)))
+
+    def argmax_into(self, token, logits, row, ids, vals, slot):
+        """Index of the largest value of row `row` of logits -> token (in place), ids[slot]; the two largest values -> vals[2 slot ..]."""
+        lb = self._op("ugh_llama_argmax_into", token, _p(logits.h), C.c_size_t(row), _p(ids.h), _p(vals.h), C.c_size_t(slot))
+        lb._keep += [logits, ids, vals]
+        return lb
+
     def packed_projections(self):
         return bool(host_lib().ugh_llama_packed_projections(_p(self.h)))
 

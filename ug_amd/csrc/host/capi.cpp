@@ -476,6 +476,10 @@ int ugh_llama_attention_cached(void* ops, void* q, void* k, void* v, size_t s, f
     else *out = box(ops_of(ops).attention_cached(lb_of(q), lb_of(k), lb_of(v), s, scale, nullptr, nullptr, nullptr, false, q_offset, q_row_stride, n_heads));
   });
 }
+int ugh_llama_device_argmax(void* ops) { return ops_of(ops).device_argmax() ? 1 : 0; }
+int ugh_llama_argmax_into(void* ops, void* token, void* logits, size_t row, void* ids, void* vals, size_t slot, void** out) {
+  return guard([&] { *out = box(ops_of(ops).argmax_into(lb_of(token), lb_of(logits), row, lb_of(ids), lb_of(vals), slot)); });
+}
 int ugh_llama_packed_projections(void* ops) { return ops_of(ops).packed_projections() ? 1 : 0; }
 int ugh_llama_linear_packed(void* ops, void* x, size_t n_mats, void** ws, void* alpha, float eps, void** out) {
   return guard([&] {

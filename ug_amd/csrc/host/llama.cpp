@@ -297,6 +297,23 @@ struct HipOps : Ops {
     };
     return LB::custom(f, {x, w, residual}, residual.shape(), x.dtype(), x.device());
   }
+
+  bool device_argmax() const override { return true; }
+
+  LB argmax_into(const LB& token, const LB& logits, size_t row, const LB& ids, const LB& vals, size_t slot) const override {
+    if (logits.rank() < 2 || logits.dtype() != DType::F32 || token.dtype() != DType::I32 || token.elem_count() != 1 || ids.dtype() != DType::I32 ||
+        vals.dtype() != DType::F32)
+      bail("argmax_into: expected F32 logits [.., rows, n], an I32 token, I32 ids and F32 vals");
+    size_t n = logits.dims()[logits.rank() - 1];
+    if ((row + 1) * n > logits.elem_count() || slot >= ids.elem_count() || 2 * (slot + 1) > vals.elem_count()) bail("argmax_into: row or slot out of range");
+    ughip_device* dev = hip_dev(logits);
+    // in-place op: arguments first, the token buffer last (schedule.rs:404-413)
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != 4) bail("argmax_into: expected 4 slices");
+      hip_check(ughip_argmax_row(dev, hip_raw_slice(*vs[0]), n, row, hip_raw_slice(*vs[3]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), slot), "argmax_into");
+    };
+    return token.custom_ip(f, {logits, ids, vals});
+  }
 };
 
 }  // namespace
@@ -399,6 +416,8 @@ LB Ops::attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float 
   att = t == 1 ? custom_softmax(att) : causal_softmax(att);
   return att.matmul(vr).transpose(2, 1).merge_dims(-2);
 }
+
+LB Ops::argmax_into(const LB&, const LB&, size_t, const LB&, const LB&, size_t) const { bail("argmax_into: this device reads the logits back and picks the token on the host"); }
 
 // model.rs:206-208 side by side.
 LB Ops::linear_packed(const LB& x0, const std::vector<LB>& ws, const LB* alpha, float eps) const {
@@ -729,6 +748,116 @@ double ms_between(std::chrono::steady_clock::time_point a, std::chrono::steady_c
 
 }  // namespace
 
+namespace {
+
+// The same loop for a device that queues work and picks the token itself: the argmax of step i
+// writes the input buffer of step i + 1 on the device, so nothing is read back between steps and
+// the launches of step i + 1 are issued while step i still runs.  Inputs that have to come from
+// the host (prompt, positions) are uploaded before the first launch, because an upload waits for
+// the stream.  Ids and the two largest logits of every step are read once at the end.
+std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vector<int32_t>& prompt, size_t n_steps, GenerateStats* stats) {
+  using clock = std::chrono::steady_clock;
+  const DevicePtr& dev = model.device();
+  const Ops& ops = model.ops();
+  std::vector<Cache> cache = model.new_cache();
+  CompilationCache ccache;
+  const bool verbose = getenv("UG_LLAMA_VERBOSE") != nullptr;
+  model.rope().cos.realize();
+  model.rope().sin.realize();
+
+  const size_t total = n_steps + 1;
+  LB ids = LB::alloc_uninit(DType::I32, Shape({total}), dev), vals = LB::alloc_uninit(DType::F32, Shape({2 * total}), dev);
+  ids.maybe_allocate_uninit();
+  vals.maybe_allocate_uninit();
+  std::vector<LB> tokens(total + 1), pos(total);
+  tokens[0] = LB::copy(prompt.data(), DType::I32, prompt.size(), Shape({1, prompt.size()}), dev);
+  for (size_t i = 0; i < total; ++i) {
+    int32_t p32 = i == 0 ? 0 : (int32_t)(prompt.size() + i - 1);
+    pos[i] = LB::copy(&p32, DType::I32, 1, Shape({1, 1}), dev);
+    tokens[i + 1] = LB::alloc_uninit(DType::I32, Shape({1, 1}), dev);  // written by the argmax of step i
+    tokens[i + 1].maybe_allocate_uninit();
+  }
+
+  auto build = [&](size_t i, PreparedStep& st) {
+    auto t0 = clock::now();
+    st.t = i == 0 ? prompt.size() : 1;
+    st.tokens = tokens[i];
+    LB logits = model.fwd(st.tokens, pos[i], cache);
+    st.logits = ops.argmax_into(tokens[i + 1], logits, st.t - 1, ids, vals, i);
+    auto t1 = clock::now();
+    Schedule schedule = Schedule::create_one(st.logits);
+    auto t2 = clock::now();
+    st.compiled = std::make_unique<CompiledSchedule>(schedule.compile_with_cache(ccache));
+    st.compiled->allocate_all();
+    st.n_items = schedule.items().size();
+    st.build_ms = ms_between(t0, t1);
+    st.gen_ms = ms_between(t1, t2);
+    st.comp_ms = ms_between(t2, clock::now());
+  };
+
+  PreparedStep cur, done;
+  auto t_start = clock::now();
+  build(0, cur);
+  auto t_decode = t_start;
+  for (size_t step = 0; step <= n_steps; ++step) {
+    const bool more = step < n_steps;
+    PreparedStep next;
+    for (Cache& c : cache) {
+      c.prev_k.maybe_allocate_uninit();
+      c.prev_v.maybe_allocate_uninit();
+      c.prev_k.detach();
+      c.prev_v.detach();
+    }
+    auto t0 = clock::now();
+    auto t1 = t0;
+    if (more) {
+      std::exception_ptr run_err;
+      std::thread launcher([&] {
+        try {
+          cur.compiled->run();
+        } catch (...) {
+          run_err = std::current_exception();
+        }
+        t1 = clock::now();
+      });
+      try {
+        build(step + 1, next);
+        done = PreparedStep();  // buffers go back to the pool; the stream orders their reuse behind this step's kernels
+      } catch (...) {
+        launcher.join();
+        throw;
+      }
+      launcher.join();
+      if (run_err) std::rethrow_exception(run_err);
+    } else {
+      cur.compiled->run();
+      t1 = clock::now();
+    }
+    if (verbose)
+      fprintf(stderr, "step %zu: launches %.2fms, next build %.2fms gen %.2fms comp %.2fms, both %.2fms, items %zu (queued, no read-back)\n", step,
+              ms_between(t0, t1), next.build_ms, next.gen_ms, next.comp_ms, ms_between(t0, clock::now()), cur.n_items);
+    if (step == 0) {
+      dev->synchronize();  // separates the prompt's time from the decode steps'
+      t_decode = clock::now();
+      if (stats) stats->prefill_ms = ms_between(t_start, t_decode);
+    }
+    done = std::move(cur);
+    cur = std::move(next);
+  }
+  std::vector<int32_t> out(total);
+  ids.data_vec(out.data(), DType::I32);  // waits for the last step
+  if (stats) {
+    stats->decode_ms = ms_between(t_decode, clock::now());
+    std::vector<float> v(2 * total);
+    vals.data_vec(v.data(), DType::F32);
+    for (size_t i = 0; i < total; ++i) stats->top1_margin.push_back(v[2 * i] - v[2 * i + 1]);
+    stats->step_ms.assign(n_steps, n_steps ? stats->decode_ms / (double)n_steps : 0.0);  // steps overlap: only their mean is observable
+  }
+  return out;
+}
+
+}  // namespace
+
 // The loop of ug-llama/src/main.rs:118-170 (rebuild the graph, schedule, compile against the cache,
 // run, read the logits back, argmax) with one change of order: the graph of step i+1 depends on the
 // position but not on the token value, so it is built, scheduled and compiled while the device is
@@ -736,12 +865,15 @@ double ms_between(std::chrono::steady_clock::time_point a, std::chrono::steady_c
 // also overlaps the launches of step i), and the token id is uploaded into its input buffer once
 // known.  Every value computed is the same as in the reference's order.
 // UG_LLAMA_NO_OVERLAP=1 keeps everything on the calling thread.
+// UG_LLAMA_HOST_ARGMAX=1 keeps this read-back loop on a device that could pick the token itself.
 std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32_t>& prompt, size_t n_steps, GenerateStats* stats) {
   using clock = std::chrono::steady_clock;
   const Config& cfg = model.config();
   const DevicePtr& dev = model.device();
   if (prompt.empty()) bail("empty prompt");
   if (prompt.size() + n_steps > cfg.max_position_embeddings) bail("prompt + steps exceed max_position_embeddings");
+  if (dev->runs_async() && model.ops().device_argmax() && getenv("UG_LLAMA_HOST_ARGMAX") == nullptr && getenv("UG_LLAMA_NO_OVERLAP") == nullptr)
+    return generate_greedy_queued(model, prompt, n_steps, stats);
   std::vector<Cache> cache = model.new_cache();
   CompilationCache ccache;
   std::vector<int32_t> out;

@@ -72,6 +72,13 @@ struct Ops {
   virtual LB gate_up(const LB& x, const LB& w_gate, const LB& w_up, const LB* alpha = nullptr, float eps = 0.f) const;
   // x w^T + residual
   virtual LB linear_add(const LB& x, const LB& w, const LB& residual) const;
+
+  // Greedy step on the device (device_argmax() == true): the index of the largest value of row
+  // `row` of logits [b, rows, n] is written into `token` (I32, one element, in place: the result
+  // names the same storage) and recorded with the two largest values at ids[slot], vals[2 slot],
+  // vals[2 slot + 1].  A decoder can then queue the next step without reading the logits back.
+  virtual bool device_argmax() const { return false; }
+  virtual LB argmax_into(const LB& token, const LB& logits, size_t row, const LB& ids, const LB& vals, size_t slot) const;
 };
 
 // The HIP implementation (counterpart of ug-llama/src/cuda_ops.rs).
@@ -151,6 +158,7 @@ class Model {
   const Config& config() const { return cfg_; }
   const ug::DevicePtr& device() const { return dev_; }
   const Rope& rope() const { return rope_; }
+  const Ops& ops() const { return *ops_; }
 
  private:
   struct Layer {

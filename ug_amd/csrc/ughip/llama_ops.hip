@@ -292,6 +292,59 @@ int check_f32(const ughip_slice* s, size_t need, const char* what) {
 
 unsigned blocks_for(size_t n, unsigned per_block) { return (unsigned)((n + per_block - 1) / per_block); }
 
+// ---- greedy step ------------------------------------------------------------------------------------
+// Largest value of a row and its index (the lowest index among equal values), and the largest of
+// the rest: what the host loop of a greedy decoder computes from the logits it reads back.
+struct Top2 {
+  float best;
+  int idx;
+  float second;
+};
+
+__device__ __forceinline__ Top2 top2_merge(const Top2& a, const Top2& b) {
+  const bool a_wins = a.best > b.best || (a.best == b.best && a.idx < b.idx);
+  Top2 r;
+  r.best = a_wins ? a.best : b.best;
+  r.idx = a_wins ? a.idx : b.idx;
+  r.second = a_wins ? fmaxf(a.second, b.best) : fmaxf(b.second, a.best);
+  return r;
+}
+
+__global__ void __launch_bounds__(1024) argmax_row_kernel(const float* __restrict__ x, int n, int* __restrict__ token, int* __restrict__ ids,
+                                                          float* __restrict__ vals, size_t slot) {
+  __shared__ Top2 part[16];
+  Top2 t{-INFINITY, 0x7fffffff, -INFINITY};
+  for (int i = threadIdx.x; i < n; i += 1024) {
+    const float v = x[i];
+    if (v > t.best) {  // indices grow within a thread: an equal value never replaces an earlier one
+      t.second = t.best;
+      t.best = v;
+      t.idx = i;
+    } else if (v > t.second) {
+      t.second = v;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    Top2 u;
+    u.best = __shfl_xor(t.best, o, 64);
+    u.idx = __shfl_xor(t.idx, o, 64);
+    u.second = __shfl_xor(t.second, o, 64);
+    t = top2_merge(t, u);
+  }
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = t;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    Top2 r = part[0];
+    for (int w = 1; w < 16; ++w) r = top2_merge(r, part[w]);
+    if (r.idx == 0x7fffffff) r.idx = 0;  // a row of NaN / -inf only
+    if (token) token[0] = r.idx;
+    ids[slot] = r.idx;
+    vals[2 * slot] = r.best;
+    vals[2 * slot + 1] = r.second;
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -404,6 +457,21 @@ int ughip_cat(ughip_device* dev, const ughip_slice* lhs, const ughip_slice* rhs,
     cat_kernel<float4, 4><<<blocks_for(n / 4, 256), 256, 0, dev->stream>>>(l, r, o, n / 4, d2_l, d2_r);
   else
     cat_kernel<float, 1><<<blocks_for(n, 256), 256, 0, dev->stream>>>(l, r, o, n, d2_l, d2_r);
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+int ughip_argmax_row(ughip_device* dev, const ughip_slice* logits, size_t n, size_t row, ughip_slice* token, ughip_slice* ids, ughip_slice* vals, size_t slot) {
+  if (!dev || !logits || !ids || !vals) return set_error(UGHIP_ERR_INVALID, "argmax_row: null argument");
+  if (logits->dtype != UGHIP_F32 || vals->dtype != UGHIP_F32 || ids->dtype != UGHIP_I32 || (token && token->dtype != UGHIP_I32))
+    return set_error(UGHIP_ERR_INVALID, "argmax_row: expected F32 logits and values, I32 token and ids");
+  if (n == 0 || n > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "argmax_row: row length %zu", n);
+  if (logits->len < (row + 1) * n) return set_error(UGHIP_ERR_BOUNDS, "argmax_row: row %zu of %zu elements is outside a slice of %zu", row, n, logits->len);
+  if (ids->len <= slot || vals->len < 2 * (slot + 1) || (token && token->len < 1))
+    return set_error(UGHIP_ERR_BOUNDS, "argmax_row: slot %zu is outside the record slices", slot);
+  if (int rc = device_activate(dev)) return rc;
+  argmax_row_kernel<<<1, 1024, 0, dev->stream>>>(static_cast<const float*>(logits->ptr) + row * n, (int)n, token ? static_cast<int*>(token->ptr) : nullptr,
+                                                 static_cast<int*>(ids->ptr), static_cast<float*>(vals->ptr), slot);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
 }
