@@ -280,6 +280,17 @@ int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_off
                            size_t t, size_t s, size_t cap, size_t d, float scale, const ughip_slice* cos, const ughip_slice* sin,
                            const ughip_slice* pos, int interleaved);
 
+/* One decode position in one launch: ughip_kv_append of the k and v parts of a packed q|k|v row
+ * (qkv [b, row_stride], parts at q_offset / k_offset / v_offset) into row s_old of both caches,
+ * and ughip_attention_cached of the q part over rows 0 .. s_old.  The caches are read and
+ * written; dst [b, n_heads * d].  d a power of two in 16..256, s_old + 1 <= min(cap, 12000). */
+int ughip_attention_step(ughip_device* dev, const ughip_slice* qkv, size_t row_stride,
+                         size_t q_offset, size_t k_offset, size_t v_offset, ughip_slice* kcache,
+                         ughip_slice* vcache, ughip_slice* dst, size_t b, size_t n_heads,
+                         size_t n_kv_heads, size_t s_old, size_t cap, size_t d, float scale,
+                         const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos,
+                         int interleaved);
+
 /* ---- projections of one position with their neighbours folded in (f32, one input row) ----------
  * No counterpart in the reference's device trait: there each is a matmul (lib.rs:62-70) followed
  * by the small kernels of the lazy graph.  Every product is x (k elements) against the rows of a

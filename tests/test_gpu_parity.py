@@ -989,6 +989,24 @@ def test_packed_rows_feed_cache_and_attention(hip, hip_ops):
 
     for a, b2 in zip(run(True), run(False)):
         np.testing.assert_array_equal(a, b2)
+
+    # and both appends plus the attention as one launch
+    for il in (False, True):
+        for with_rope in (True, False):
+            def step(fused):
+                ck, cv = LB.copy(store_k, (1, nkv, cap, d), hip), LB.copy(store_v, (1, nkv, cap, d), hip)
+                ck.realize(), cv.realize()
+                buf = LB.copy(qkv, (1, 1, row), hip)
+                rp = (cos, sin, pos, il) if with_rope else ()
+                if fused:
+                    out = hip_ops.attention_step(buf, ck, cv, length, nh, scale, *rp)
+                else:
+                    kc = hip_ops.kv_append(ck, length, buf, *rp, x_offset=nq, x_row_stride=row)
+                    vc = hip_ops.kv_append(cv, length, buf, x_offset=nq + nk, x_row_stride=row)
+                    out = hip_ops.attention_cached(buf, kc, vc, length + 1, scale, *rp, q_offset=0, q_row_stride=row, n_heads=nh)
+                return out.data_vec(), ck.data_vec(), cv.data_vec()
+            for a, b2 in zip(step(True), step(False)):
+                np.testing.assert_array_equal(a, b2)
     with pytest.raises(ug_amd.UgError, match="mismatched shapes"):
         hip_ops.kv_append(LB.copy(store_k, (1, nkv, cap, d), hip), length, LB.copy(qkv, (1, 1, row), hip), x_offset=nq + nk + 4, x_row_stride=row).data_vec()
 

@@ -688,6 +688,15 @@ class LlamaOps(_Handle):
         lb._keep += [k, v] + ([cos, sin, pos] if rope else [])
         return lb
 
+    def attention_step(self, qkv, kcache, vcache, length, n_heads, scale, cos=None, sin=None, pos=None, interleaved=False):
+        """One decode position: the k | v parts of the packed row go into row `length` of the caches (which are
+        written), the q part attends to rows 0 .. length -> [b, 1, n_heads * d]."""
+        rope = cos is not None
+        lb = self._op("ugh_llama_attention_step", qkv, _p(kcache.h), _p(vcache.h), C.c_size_t(length), C.c_size_t(n_heads), C.c_float(scale),
+                      _p(cos.h) if rope else None, _p(sin.h) if rope else None, _p(pos.h) if rope else None, int(interleaved))
+        lb._keep += [kcache, vcache] + ([cos, sin, pos] if rope else [])
+        return lb
+
     def device_argmax(self):
         return bool(host_lib().ugh_llama_device_argmax(_p(self.h)))
 

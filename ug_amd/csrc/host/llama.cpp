@@ -298,6 +298,32 @@ struct HipOps : Ops {
     return LB::custom(f, {x, w, residual}, residual.shape(), x.dtype(), x.device());
   }
 
+  LB attention_step(const LB& qkv, const LB& kcache, const LB& vcache, size_t len, size_t n_heads, float scale, const LB* cos, const LB* sin, const LB* pos,
+                    bool interleaved) const override {
+    if (qkv.rank() != 3 || qkv.dims()[1] != 1 || kcache.rank() != 4 || kcache.dims() != vcache.dims()) bail("attention_step: expected qkv [b, 1, row] and caches [b, nkv, cap, d]");
+    size_t b = qkv.dims()[0], row = qkv.dims()[2], nkv = kcache.dims()[1], cap = kcache.dims()[2], d = kcache.dims()[3];
+    size_t nq = n_heads * d, nk = nkv * d;
+    if (kcache.dims()[0] != b || row != nq + 2 * nk || len >= cap)
+      bail("attention_step: mismatched shapes " + qkv.shape().str() + " " + kcache.shape().str() + " at position " + std::to_string(len));
+    ughip_device* dev = hip_dev(qkv);
+    const bool with_rope = cos != nullptr;
+    int il = interleaved ? 1 : 0;
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != (with_rope ? 7u : 4u)) bail("attention_step: unexpected number of slices");
+      hip_check(ughip_attention_step(dev, hip_raw_slice(*vs[0]), row, 0, nq, nq + nk, hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), hip_raw_slice(*vs.back()), b, n_heads,
+                                     nkv, len, cap, d, scale, with_rope ? hip_raw_slice(*vs[3]) : nullptr, with_rope ? hip_raw_slice(*vs[4]) : nullptr,
+                                     with_rope ? hip_raw_slice(*vs[5]) : nullptr, il),
+                "attention_step");
+    };
+    std::vector<LB> args = {qkv, kcache, vcache};
+    if (with_rope) {
+      args.push_back(*cos);
+      args.push_back(*sin);
+      args.push_back(*pos);
+    }
+    return LB::custom(f, args, Shape({b, 1, nq}), qkv.dtype(), qkv.device());
+  }
+
   bool device_argmax() const override { return true; }
 
   LB argmax_into(const LB& token, const LB& logits, size_t row, const LB& ids, const LB& vals, size_t slot) const override {
@@ -415,6 +441,10 @@ LB Ops::attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float 
   att = att.binary(BinaryOp::Mul, LB::cst(Const::f32(scale), Shape(), q.device()).broadcast(att.shape()));
   att = t == 1 ? custom_softmax(att) : causal_softmax(att);
   return att.matmul(vr).transpose(2, 1).merge_dims(-2);
+}
+
+LB Ops::attention_step(const LB&, const LB&, const LB&, size_t, size_t, float, const LB*, const LB*, const LB*, bool) const {
+  bail("attention_step: needs a device with packed projections and caches written in place");
 }
 
 LB Ops::argmax_into(const LB&, const LB&, size_t, const LB&, const LB&, size_t) const { bail("argmax_into: this device reads the logits back and picks the token on the host"); }
@@ -625,10 +655,13 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
     // one position: q | k | v come out of one launch (with the norm in front) side by side and are read where they lie
     const size_t nq = nh * hd, nk = nkv * hd, row = nq + 2 * nk, len = cache.len;
     LB qkv = ops_->linear_packed(xs_in, {l.q_proj, l.k_proj, l.v_proj}, norm_first ? &l.rms1 : nullptr, eps);
+    cache.len = len + 1;
+    const float scale = std::pow((float)hd, -0.5f);
+    if (hd >= 16 && hd <= 256 && (hd & (hd - 1)) == 0 && cache.len <= 12000)
+      return finish(ops_->attention_step(qkv, cache.prev_k, cache.prev_v, len, nh, scale, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved));
     LB kc = ops_->kv_append(cache.prev_k, len, qkv, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, nq, row);
     LB vc = ops_->kv_append(cache.prev_v, len, qkv, nullptr, nullptr, nullptr, false, nq + nk, row);
-    cache.len = len + 1;
-    return finish(ops_->attention_cached(qkv, kc, vc, cache.len, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, 0, row, nh));
+    return finish(ops_->attention_cached(qkv, kc, vc, cache.len, scale, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, 0, row, nh));
   }
   LB xs = norm_first ? rms_norm(xs_in, l.rms1, eps) : xs_in;
   LB q = xs.matmul_t(l.q_proj);

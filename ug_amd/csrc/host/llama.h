@@ -73,6 +73,13 @@ struct Ops {
   // x w^T + residual
   virtual LB linear_add(const LB& x, const LB& w, const LB& residual) const;
 
+  // One decode position in one launch (devices with packed_projections()): the k and v parts of
+  // the packed row qkv [b, 1, (nh + 2 nkv) d] go into row `len` of both caches (k rotated), the q
+  // part attends to rows 0 .. len.  The caches are WRITTEN although they are passed as arguments:
+  // they must be preallocated stores that nothing else in the same graph reads.
+  virtual LB attention_step(const LB& qkv, const LB& kcache, const LB& vcache, size_t len, size_t n_heads, float scale, const LB* cos, const LB* sin,
+                            const LB* pos, bool interleaved) const;
+
   // Greedy step on the device (device_argmax() == true): the index of the largest value of row
   // `row` of logits [b, rows, n] is written into `token` (I32, one element, in place: the result
   // names the same storage) and recorded with the two largest values at ids[slot], vals[2 slot],

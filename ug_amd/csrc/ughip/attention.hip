@@ -124,10 +124,14 @@ __device__ __forceinline__ float att_block_reduce(float v, float* lds16) {
 __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
                                                                        float* __restrict__ dst, int nh, int nkv, int s, size_t kv_head_stride,
                                                                        size_t q_batch_stride, int d, float scale, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-                                                                       const int* __restrict__ pos, size_t table_len, int interleaved) {
+                                                                       const int* __restrict__ pos, size_t table_len, int interleaved,
+                                                                       const float* __restrict__ k_new, const float* __restrict__ v_new, float* __restrict__ k_out,
+                                                                       float* __restrict__ v_out) {
   extern __shared__ __attribute__((aligned(16))) float sc[];  // s scores, then ATT_WAVES * 64 float4 of reduction space
   __shared__ float lds16[ATT_WAVES];
   __shared__ __attribute__((aligned(16))) float qs[256];
+  __shared__ __attribute__((aligned(16))) float kn[256];
+  __shared__ __attribute__((aligned(16))) float vn[256];
   const int tid = threadIdx.x;
   const int lpk = d >> 2, kpb = ATT_THREADS / lpk;  // lanes per key, keys per step
   const int c4 = tid % lpk, slot = tid / lpk;
@@ -137,24 +141,43 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
   const float4* k4 = reinterpret_cast<const float4*>(k + ((size_t)b * nkv + kvh) * kv_head_stride);
   const float4* v4 = reinterpret_cast<const float4*>(v + ((size_t)b * nkv + kvh) * kv_head_stride);
 
+  // k_new != nullptr: key / value row s-1 is not in the caches yet.  It comes from k_new / v_new
+  // (rows of the same packed buffer as q: q_batch_stride apart, head kvh at kvh * d), the key is
+  // rotated like q, and the first query head of every kv head stores both rows into the caches at
+  // row s-1 for the steps to come (nobody reads that cache row in this launch).
+  const float* knh = k_new ? k_new + (size_t)b * q_batch_stride + (size_t)kvh * d : nullptr;
+  const float* vnh = k_new ? v_new + (size_t)b * q_batch_stride + (size_t)kvh * d : nullptr;
   float4 qv;
   if (cos_t) {
     const int half = d >> 1;
-    if (tid < half) {
+    if (tid < 2 * half && (tid < half || k_new)) {
+      const int pr = tid < half ? tid : tid - half;
+      const float* src = tid < half ? qh : knh;
+      float* out = tid < half ? qs : kn;
       const long long p = pos[0];
-      const size_t ics = (size_t)p * half + tid;
+      const size_t ics = (size_t)p * half + pr;
       const bool ok = p >= 0 && ics < table_len;
       const float c = ok ? cos_t[ics] : NAN, sn = ok ? sin_t[ics] : NAN;
-      const int i1 = interleaved ? 2 * tid : tid, i2 = interleaved ? 2 * tid + 1 : tid + half;
-      const float x1 = qh[i1], x2 = qh[i2];
-      qs[i1] = x1 * c - x2 * sn;
-      qs[i2] = x1 * sn + x2 * c;
+      const int i1 = interleaved ? 2 * pr : pr, i2 = interleaved ? 2 * pr + 1 : pr + half;
+      const float x1 = src[i1], x2 = src[i2];
+      out[i1] = x1 * c - x2 * sn;
+      out[i2] = x1 * sn + x2 * c;
     }
+    if (k_new && tid >= 512 && tid < 512 + d) vn[tid - 512] = vnh[tid - 512];
     __syncthreads();
     qv = reinterpret_cast<const float4*>(qs)[c4];
   } else {
+    if (k_new && tid < d) kn[tid] = knh[tid];
+    if (k_new && tid >= 512 && tid < 512 + d) vn[tid - 512] = vnh[tid - 512];
+    if (k_new) __syncthreads();
     qv = q4[c4];
   }
+  if (k_out && h % (nh / nkv) == 0 && tid < 2 * lpk) {
+    const size_t row = (((size_t)b * nkv + kvh) * kv_head_stride + (size_t)(s - 1) * d) / 4;
+    if (tid < lpk) reinterpret_cast<float4*>(k_out)[row + tid] = reinterpret_cast<const float4*>(kn)[tid];
+    else reinterpret_cast<float4*>(v_out)[row + tid - lpk] = reinterpret_cast<const float4*>(vn)[tid - lpk];
+  }
+  const int j_new = k_new ? s - 1 : -1;
   // scores = (q . k_j) * scale, four key rows per lane group in flight
   float m = -INFINITY;
   for (int j0 = 0; j0 < s; j0 += 4 * kpb) {
@@ -164,7 +187,7 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
       const int j = j0 + u * kpb + slot;
       p[u] = 0.f;
       if (j < s) {
-        const float4 kv = k4[(size_t)j * lpk + c4];
+        const float4 kv = j == j_new ? reinterpret_cast<const float4*>(kn)[c4] : k4[(size_t)j * lpk + c4];
         p[u] = (qv.x * kv.x + qv.y * kv.y) + (qv.z * kv.z + qv.w * kv.w);
       }
     }
@@ -198,7 +221,7 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
     for (int u = 0; u < 4; ++u) {
       const int j = j0 + u * kpb;
       pj[u] = j < s ? sc[j] : 0.f;
-      vv[u] = j < s ? v4[(size_t)j * lpk + c4] : make_float4(0.f, 0.f, 0.f, 0.f);
+      vv[u] = j >= s ? make_float4(0.f, 0.f, 0.f, 0.f) : j == j_new ? reinterpret_cast<const float4*>(vn)[c4] : v4[(size_t)j * lpk + c4];
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -610,11 +633,48 @@ int attention_decode_launch(ughip_device* dev, const ughip_slice* q, size_t q_of
       static_cast<const float*>(q->ptr) + q_offset, static_cast<const float*>(k->ptr), static_cast<const float*>(v->ptr), static_cast<float*>(dst->ptr),
       (int)n_heads, (int)n_kv_heads, (int)s, cap * d, q_row_stride, (int)d, scale, rope ? static_cast<const float*>(cos->ptr) : nullptr,
       rope ? static_cast<const float*>(sin->ptr) : nullptr, rope ? static_cast<const int*>(pos->ptr) : nullptr,
-      rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved);
+      rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved, nullptr, nullptr, nullptr, nullptr);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
 }
 }  // namespace
+
+int ughip_attention_step(ughip_device* dev, const ughip_slice* qkv, size_t row_stride, size_t q_offset, size_t k_offset, size_t v_offset, ughip_slice* kcache,
+                         ughip_slice* vcache, ughip_slice* dst, size_t b, size_t n_heads, size_t n_kv_heads, size_t s_old, size_t cap, size_t d, float scale,
+                         const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos, int interleaved) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  const bool rope = cos || sin || pos;
+  if (rope)
+    if (int rc = check_rope_table(cos, sin, pos, d, "attention_step")) return rc;
+  if (n_kv_heads == 0 || n_heads % n_kv_heads != 0)
+    return set_error(UGHIP_ERR_INVALID, "attention_step: %zu heads are not a multiple of %zu kv heads", n_heads, n_kv_heads);
+  if (d < 16 || d > 256 || (d & (d - 1)) != 0) return set_error(UGHIP_ERR_INVALID, "attention_step: head size %zu is not a power of two in 16..256", d);
+  const size_t s = s_old + 1;
+  if (s > cap) return set_error(UGHIP_ERR_BOUNDS, "attention_step: position %zu does not fit a cache of %zu rows", s_old, cap);
+  if (s > 12000) return set_error(UGHIP_ERR_INVALID, "attention_step: %zu keys exceed the 12000 this kernel holds in LDS", s);
+  const size_t nq = n_heads * d, nk = n_kv_heads * d;
+  if (row_stride % 4 != 0 || (q_offset | k_offset | v_offset) % 4 != 0 || q_offset + nq > row_stride || k_offset + nk > row_stride || v_offset + nk > row_stride)
+    return set_error(UGHIP_ERR_INVALID, "attention_step: q/k/v at %zu/%zu/%zu do not fit rows of %zu", q_offset, k_offset, v_offset, row_stride);
+  if (int rc = check_f32(qkv, b * row_stride, "attention_step qkv")) return rc;
+  if (int rc = check_f32(kcache, b * n_kv_heads * cap * d, "attention_step k cache")) return rc;
+  if (int rc = check_f32(vcache, b * n_kv_heads * cap * d, "attention_step v cache")) return rc;
+  if (int rc = check_f32(dst, b * nq, "attention_step dst")) return rc;
+  if (dst == qkv || dst == kcache || dst == vcache || kcache == vcache || qkv == kcache || qkv == vcache)
+    return set_error(UGHIP_ERR_INVALID, "attention_step: aliased slices");
+  if (b * n_heads == 0) return UGHIP_OK;
+  if (b * n_heads > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "attention_step: too many heads");
+  if (int rc = device_activate(dev)) return rc;
+  const size_t lds = (s + 3 + ATT_WAVES * 64 * 4) * sizeof(float);
+  const float* base = static_cast<const float*>(qkv->ptr);
+  attention_decode_kernel<<<(unsigned)(b * n_heads), ATT_THREADS, lds, dev->stream>>>(
+      base + q_offset, static_cast<const float*>(kcache->ptr), static_cast<const float*>(vcache->ptr), static_cast<float*>(dst->ptr), (int)n_heads,
+      (int)n_kv_heads, (int)s, cap * d, row_stride, (int)d, scale, rope ? static_cast<const float*>(cos->ptr) : nullptr,
+      rope ? static_cast<const float*>(sin->ptr) : nullptr, rope ? static_cast<const int*>(pos->ptr) : nullptr,
+      rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved, base + k_offset, base + v_offset, static_cast<float*>(kcache->ptr),
+      static_cast<float*>(vcache->ptr));
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
 
 int ughip_attention_decode_rope(ughip_device* dev, const ughip_slice* q, const ughip_slice* k, const ughip_slice* v, ughip_slice* dst, size_t b,
                                 size_t n_heads, size_t n_kv_heads, size_t s, size_t d, float scale, const ughip_slice* cos, const ughip_slice* sin,
