@@ -108,6 +108,7 @@ __global__ void __launch_bounds__(256) causal_softmax_generic(const float* __res
 // With a rope table (cos_t != nullptr) q is rotated first, at table row pos[0] (rope: pairs
 // (i, i + d/2); rope_i: pairs (2i, 2i + 1); cpu_ops.rs:58-126 for t = 1).
 constexpr int ATT_THREADS = 1024, ATT_WAVES = ATT_THREADS / 64;
+typedef float att_f32x4 __attribute__((ext_vector_type(4)));
 
 template <bool IS_MAX>
 __device__ __forceinline__ float att_block_reduce(float v, float* lds16) {
@@ -147,6 +148,20 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
   // row s-1 for the steps to come (nobody reads that cache row in this launch).
   const float* knh = k_new ? k_new + (size_t)b * q_batch_stride + (size_t)kvh * d : nullptr;
   const float* vnh = k_new ? v_new + (size_t)b * q_batch_stride + (size_t)kvh * d : nullptr;
+  const int j_new = k_new ? s - 1 : -1;
+  // The cache rows of the first trip of both loops below (keys u * kpb + slot) are requested now:
+  // they do not depend on pos or on the rotation, whose loads they overlap.
+  // (native vectors: arrays of HIP's float4 struct are copied through memory)
+  att_f32x4 kpre[4], vpre[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    // unconditional loads (a branch here sends the arrays to scratch memory): rows this lane has
+    // no use for are read as row 0 and ignored below
+    const int j = u * kpb + slot;
+    const size_t jj = j < s && j != j_new ? (size_t)j : 0;
+    kpre[u] = reinterpret_cast<const att_f32x4*>(k4)[jj * lpk + c4];
+    vpre[u] = reinterpret_cast<const att_f32x4*>(v4)[jj * lpk + c4];
+  }
   float4 qv;
   if (cos_t) {
     const int half = d >> 1;
@@ -177,19 +192,23 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
     if (tid < lpk) reinterpret_cast<float4*>(k_out)[row + tid] = reinterpret_cast<const float4*>(kn)[tid];
     else reinterpret_cast<float4*>(v_out)[row + tid - lpk] = reinterpret_cast<const float4*>(vn)[tid - lpk];
   }
-  const int j_new = k_new ? s - 1 : -1;
   // scores = (q . k_j) * scale, four key rows per lane group in flight
   float m = -INFINITY;
-  for (int j0 = 0; j0 < s; j0 += 4 * kpb) {
+  auto load_rows = [&](const float4* base, int j0, att_f32x4 (&r)[4]) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + u * kpb + slot;
+      const size_t jj = j < s && j != j_new ? (size_t)j : 0;
+      r[u] = reinterpret_cast<const att_f32x4*>(base)[jj * lpk + c4];
+    }
+  };
+  auto score_trip = [&](int j0, const att_f32x4 (&kr)[4]) {
     float p[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int j = j0 + u * kpb + slot;
-      p[u] = 0.f;
-      if (j < s) {
-        const float4 kv = j == j_new ? reinterpret_cast<const float4*>(kn)[c4] : k4[(size_t)j * lpk + c4];
-        p[u] = (qv.x * kv.x + qv.y * kv.y) + (qv.z * kv.z + qv.w * kv.w);
-      }
+      const att_f32x4 kv = j == j_new ? reinterpret_cast<const att_f32x4*>(kn)[c4] : kr[u];
+      p[u] = (qv.x * kv.x + qv.y * kv.y) + (qv.z * kv.z + qv.w * kv.w);
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -202,6 +221,12 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
         m = fmaxf(m, pu);
       }
     }
+  };
+  score_trip(0, kpre);
+  for (int j0 = 4 * kpb; j0 < s; j0 += 4 * kpb) {
+    att_f32x4 kr[4];
+    load_rows(k4, j0, kr);
+    score_trip(j0, kr);
   }
   m = att_block_reduce<true>(m, lds16);  // the barriers inside also publish sc[]
   float sum = 0.f;
@@ -214,22 +239,23 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
 
   // out = sum_j p_j v_j / sum: slot walks the keys, c4 owns 4 output columns
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int j0 = slot; j0 < s; j0 += 4 * kpb) {
-    float4 vv[4];
-    float pj[4];
+  auto value_trip = [&](int j0, const att_f32x4 (&vr)[4]) {
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const int j = j0 + u * kpb;
-      pj[u] = j < s ? sc[j] : 0.f;
-      vv[u] = j >= s ? make_float4(0.f, 0.f, 0.f, 0.f) : j == j_new ? reinterpret_cast<const float4*>(vn)[c4] : v4[(size_t)j * lpk + c4];
+      const int j = j0 + u * kpb + slot;
+      const float pj = j < s ? sc[j] : 0.f;
+      const att_f32x4 vv = j == j_new ? reinterpret_cast<const att_f32x4*>(vn)[c4] : vr[u];
+      acc.x += pj * vv.x;
+      acc.y += pj * vv.y;
+      acc.z += pj * vv.z;
+      acc.w += pj * vv.w;
     }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      acc.x += pj[u] * vv[u].x;
-      acc.y += pj[u] * vv[u].y;
-      acc.z += pj[u] * vv[u].z;
-      acc.w += pj[u] * vv[u].w;
-    }
+  };
+  value_trip(0, vpre);
+  for (int j0 = 4 * kpb; j0 < s; j0 += 4 * kpb) {
+    att_f32x4 vr[4];
+    load_rows(v4, j0, vr);
+    value_trip(j0, vr);
   }
   // the slots of one wave (lanes lpk apart), then the waves in order
   for (int o = lpk; o < 64; o <<= 1) {

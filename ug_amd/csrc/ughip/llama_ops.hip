@@ -2,6 +2,8 @@
 // Semantics follow the CPU implementations in ug-llama/src/cpu_ops.rs:6-167; all f32.
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
+
 #include "internal.h"
 #include "ughip.h"
 
@@ -310,19 +312,44 @@ __device__ __forceinline__ Top2 top2_merge(const Top2& a, const Top2& b) {
   return r;
 }
 
+__device__ __forceinline__ void top2_take(Top2& t, float v, int i) {
+  if (v > t.best) {  // indices grow within a thread: an equal value never replaces an earlier one
+    t.second = t.best;
+    t.best = v;
+    t.idx = i;
+  } else if (v > t.second) {
+    t.second = v;
+  }
+}
+
+// VEC: the row starts on a 16-byte boundary; eight 128-bit loads per thread are in flight at once
+// (a 32000-wide row is one trip), the last n % 4 elements are taken one by one.
+template <bool VEC>
 __global__ void __launch_bounds__(1024) argmax_row_kernel(const float* __restrict__ x, int n, int* __restrict__ token, int* __restrict__ ids,
                                                           float* __restrict__ vals, size_t slot) {
   __shared__ Top2 part[16];
   Top2 t{-INFINITY, 0x7fffffff, -INFINITY};
-  for (int i = threadIdx.x; i < n; i += 1024) {
-    const float v = x[i];
-    if (v > t.best) {  // indices grow within a thread: an equal value never replaces an earlier one
-      t.second = t.best;
-      t.best = v;
-      t.idx = i;
-    } else if (v > t.second) {
-      t.second = v;
+  if (VEC) {
+    typedef float v4 __attribute__((ext_vector_type(4)));
+    const int n4 = n >> 2;
+    for (int i0 = threadIdx.x; i0 < n4; i0 += 8 * 1024) {
+      v4 r[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) r[u] = reinterpret_cast<const v4*>(x)[min(i0 + u * 1024, n4 - 1)];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int i = i0 + u * 1024;
+        if (i < n4) {
+          top2_take(t, r[u].x, 4 * i);
+          top2_take(t, r[u].y, 4 * i + 1);
+          top2_take(t, r[u].z, 4 * i + 2);
+          top2_take(t, r[u].w, 4 * i + 3);
+        }
+      }
     }
+    for (int i = 4 * n4 + threadIdx.x; i < n; i += 1024) top2_take(t, x[i], i);
+  } else {
+    for (int i = threadIdx.x; i < n; i += 1024) top2_take(t, x[i], i);
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
@@ -470,8 +497,12 @@ int ughip_argmax_row(ughip_device* dev, const ughip_slice* logits, size_t n, siz
   if (ids->len <= slot || vals->len < 2 * (slot + 1) || (token && token->len < 1))
     return set_error(UGHIP_ERR_BOUNDS, "argmax_row: slot %zu is outside the record slices", slot);
   if (int rc = device_activate(dev)) return rc;
-  argmax_row_kernel<<<1, 1024, 0, dev->stream>>>(static_cast<const float*>(logits->ptr) + row * n, (int)n, token ? static_cast<int*>(token->ptr) : nullptr,
-                                                 static_cast<int*>(ids->ptr), static_cast<float*>(vals->ptr), slot);
+  const float* x = static_cast<const float*>(logits->ptr) + row * n;
+  int* tp = token ? static_cast<int*>(token->ptr) : nullptr;
+  if ((reinterpret_cast<uintptr_t>(x) & 15) == 0 && n >= 4)
+    argmax_row_kernel<true><<<1, 1024, 0, dev->stream>>>(x, (int)n, tp, static_cast<int*>(ids->ptr), static_cast<float*>(vals->ptr), slot);
+  else
+    argmax_row_kernel<false><<<1, 1024, 0, dev->stream>>>(x, (int)n, tp, static_cast<int*>(ids->ptr), static_cast<float*>(vals->ptr), slot);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
 }
