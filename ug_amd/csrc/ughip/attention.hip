@@ -381,15 +381,38 @@ __global__ void __launch_bounds__(256) kv_append_kernel(float* __restrict__ cach
 //                 any data movement; A = V[that key][lane % 32 + 32 * block].
 typedef float att_f32x16 __attribute__((ext_vector_type(16)));
 
+// exp(x) for x <= 0 in six branch-free instructions: x log2(e) is formed as a rounded product t plus
+// its exact remainder r (two FMAs, log2(e) split in two), then 2^t (1 + r ln 2).  Within 2 ulp over the
+// range the exponentials of a softmax live in; anything below about -87 (ATT_MASKED included) gives 0.
+constexpr float ATT_MASKED = -1e30f;
+__device__ __forceinline__ float att_exp(float x) {
+  constexpr float L2E_HI = 1.44269502162933349609375f, L2E_LO = 1.925963033500011e-8f, LN2 = 0.693147182464599609375f;
+  const float t = x * L2E_HI;
+  float r = __builtin_fmaf(x, L2E_HI, -t);
+  r = __builtin_fmaf(x, L2E_LO, r);
+  const float y = __builtin_amdgcn_exp2f(t);
+  return __builtin_fmaf(y, r * LN2, y);
+}
+
 template <int D, int GROUPS>
 __global__ void __launch_bounds__(256 * GROUPS) attention_prefill_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
                                                                 float* __restrict__ dst, int nh, int nkv, int t, int s, size_t cap,
                                                                 size_t q_row_stride, float scale, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                                                 const int* __restrict__ pos, size_t table_len, int interleaved) {
   constexpr int H = D / 2, DB = D / 32;  // floats of q / k per lane; 32-wide blocks of the head dimension
-  __shared__ float merge_ml_all[GROUPS][3][2][64];
-  __shared__ float merge_o_all[GROUPS][3][DB * 16][64];
+  // K / V blocks reach the MFMA operand layout through a staging area private to each wave: rows
+  // are loaded from global memory whole (consecutive lanes, consecutive 16 bytes) and read back
+  // one row per lane.  Row pitches of D + 4 (128-bit reads of 16 rows) and D + 8 (32-bit reads of
+  // two rows 4 apart) floats keep both read patterns free of bank conflicts.
+  constexpr int NV = D / 8, KP = D + 4, VP = D + 8, STAGE = 32 * (KP + VP);
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  // the merge buffers take the staging area over once every wave is out of its loop
+  float (*merge_ml_all)[3][2][64] = reinterpret_cast<float (*)[3][2][64]>(smem);
+  float (*merge_o_all)[3][DB * 16][64] = reinterpret_cast<float (*)[3][DB * 16][64]>(smem + GROUPS * 3 * 2 * 64);
+  static_assert(GROUPS * (3 * 2 * 64 + 3 * DB * 16 * 64) <= 4 * GROUPS * STAGE, "merge buffers must fit the staging area");
   const int tid = threadIdx.x, lane = tid & 63, wave = (tid >> 6) & 3, group = tid >> 8;
+  float* const kst = smem + (size_t)(tid >> 6) * STAGE;
+  float* const vst = kst + 32 * KP;
   const int col = lane & 31, hh = lane >> 5;
   const int bh = blockIdx.y, b = bh / nh, head = bh % nh, kvh = head / (nh / nkv);
   // GROUPS == 2: a workgroup takes the query blocks x and n - 1 - x, one per group of 4 waves, so
@@ -403,23 +426,31 @@ __global__ void __launch_bounds__(256 * GROUPS) attention_prefill_kernel(const f
   const int qi = min(q0 + col, t - 1);        // rows past t repeat the last query and are not stored
   const int q_pos = s - t + qi;               // last key this query sees
   const int last_pos = s - t + min(q0 + 31, t - 1);
+  const int q_pos_min = s - t + min(q0, t - 1);  // the query of this block that sees the fewest keys
   const float* kb_ptr = k + ((size_t)b * nkv + kvh) * cap * D;
   const float* vb_ptr = v + ((size_t)b * nkv + kvh) * cap * D;
 
-  // K operand of a block: D/2 consecutive floats of key row key0 + col.  Rows past s repeat row s-1
-  // (they are masked, and a block index past the end is harmless).
-  auto load_k = [&](int kb, float (&kr)[H]) {
-    const float* krow = kb_ptr + (size_t)min(kb * 32 + col, s - 1) * D + hh * H;
+  // One block of 32 rows (rows past s repeat row s-1: they are masked, and a block index past
+  // the end is harmless) as NV 128-bit loads per lane, and its way into the staging area.
+  auto load_block = [&](const float* base, int kb, att_f32x4 (&raw)[NV]) {
 #pragma unroll
-    for (int j = 0; j < H; j += 4) {
-      const float4 x = *reinterpret_cast<const float4*>(krow + j);
-      kr[j] = x.x, kr[j + 1] = x.y, kr[j + 2] = x.z, kr[j + 3] = x.w;
+    for (int i = 0; i < NV; ++i) {
+      const int f4 = i * 64 + lane, row = f4 / (D / 4), c4 = f4 % (D / 4);
+      raw[i] = *reinterpret_cast<const att_f32x4*>(base + (size_t)min(kb * 32 + row, s - 1) * D + c4 * 4);
+    }
+  };
+  auto stage_block = [&](float* dst_rows, int pitch, const att_f32x4 (&raw)[NV]) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int f4 = i * 64 + lane, row = f4 / (D / 4), c4 = f4 % (D / 4);
+      *reinterpret_cast<att_f32x4*>(dst_rows + row * pitch + c4 * 4) = raw[i];
     }
   };
 
-  // the first K block is requested before the query row, whose table row hangs off a load of pos
-  float kn[H];
-  load_k(wave, kn);
+  // the first blocks are requested before the query row, whose table row hangs off a load of pos
+  att_f32x4 kraw[NV], vraw[NV];
+  load_block(kb_ptr, wave, kraw);
+  load_block(vb_ptr, wave, vraw);
 
   // this lane's half of its (rotated) query row
   float qr[H];
@@ -481,7 +512,7 @@ __global__ void __launch_bounds__(256 * GROUPS) attention_prefill_kernel(const f
     }
   }
 
-  float m_run = -INFINITY, l_half = 0.f;  // l_half: sum over the keys this half of the query's lanes holds
+  float m_run = ATT_MASKED, l_half = 0.f;  // l_half: sum over the keys this half of the query's lanes holds
   att_f32x16 o[DB];
 #pragma unroll
   for (int e = 0; e < DB; ++e)
@@ -489,54 +520,75 @@ __global__ void __launch_bounds__(256 * GROUPS) attention_prefill_kernel(const f
     for (int r = 0; r < 16; ++r) o[e][r] = 0.f;
 
   const int n_blocks = idle ? 0 : last_pos / 32 + 1;
-  // K of the next block is in flight while this one is multiplied; V of this block is requested at
-  // the top and first needed after the scores and their exponentials
+  // K and V of the next block are in flight (in registers) while this one is multiplied
   for (int kb = wave; kb < n_blocks; kb += 4) {
     const int key0 = kb * 32;
-    float kr[H], vr[DB][16];
-#pragma unroll
-    for (int j = 0; j < H; ++j) kr[j] = kn[j];
-    // V operand of MFMA r: row key0 + 8 (r / 4) + 4 hh + r % 4, column col + 32 e
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float* vrow = vb_ptr + (size_t)min(key0 + (r >> 2) * 8 + hh * 4 + (r & 3), s - 1) * D + col;
-#pragma unroll
-      for (int e = 0; e < DB; ++e) vr[e][r] = vrow[e * 32];
-    }
-    load_k(kb + 4, kn);
+    stage_block(kst, KP, kraw);
+    stage_block(vst, VP, vraw);
+    load_block(kb_ptr, kb + 4, kraw);
+    load_block(vb_ptr, kb + 4, vraw);
     __builtin_amdgcn_sched_barrier(0);  // keeps the loads up here instead of next to their uses
+    // K operand: D/2 consecutive floats of key row col
+    float kr[H];
+#pragma unroll
+    for (int j = 0; j < H; j += 4) {
+      const att_f32x4 x = *reinterpret_cast<const att_f32x4*>(kst + col * KP + hh * H + j);
+      kr[j] = x.x, kr[j + 1] = x.y, kr[j + 2] = x.z, kr[j + 3] = x.w;
+    }
     att_f32x16 sc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) sc[r] = 0.f;
 #pragma unroll
     for (int j = 0; j < H; ++j) sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kr[j], qr[j], sc, 0, 0, 0);
-    float mx = -INFINITY;
+    // V operand of MFMA r: row 8 (r / 4) + 4 hh + r % 4 of the block, column col + 32 e.  Requested
+    // while the score MFMAs run, first needed after the exponentials.
+    float vr[DB][16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int key = key0 + (r >> 2) * 8 + hh * 4 + (r & 3);
-      sc[r] = key <= q_pos ? sc[r] * scale : -INFINITY;
-      mx = fmaxf(mx, sc[r]);
+    for (int e = 0; e < DB; ++e)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) vr[e][r] = vst[((r >> 2) * 8 + hh * 4 + (r & 3)) * VP + e * 32 + col];
+    __builtin_amdgcn_sched_barrier(0);
+    // masked scores become ATT_MASKED, a finite stand-in for -inf that the exponential below maps to 0
+    float mx = ATT_MASKED;
+    if (key0 + 31 > q_pos_min) {  // wave-uniform: only blocks that touch the diagonal have anything to mask
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = key0 + (r >> 2) * 8 + hh * 4 + (r & 3);
+        sc[r] = key <= q_pos ? sc[r] * scale : ATT_MASKED;
+        mx = fmaxf(mx, sc[r]);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        sc[r] *= scale;
+        mx = fmaxf(mx, sc[r]);
+      }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m_run, mx);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // no key seen yet: every exp below is exp(-inf) = 0
-    const float alpha = expf(m_run - m_use);
+    const float m_use = m_new <= ATT_MASKED ? 0.f : m_new;  // no key seen yet: every exponential below is 0
+    const float alpha = att_exp(m_run - m_use);
     m_run = m_new;
     float psum = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      sc[r] = expf(sc[r] - m_use);
+      sc[r] = att_exp(sc[r] - m_use);
       psum += sc[r];
     }
     l_half = l_half * alpha + psum;
+    if (__any(alpha != 1.f)) {  // the running maximum settles after a few blocks
 #pragma unroll
-    for (int e = 0; e < DB; ++e) {
+      for (int e = 0; e < DB; ++e)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) o[e][r] *= alpha;
+        for (int r = 0; r < 16; ++r) o[e][r] *= alpha;
+    }
+#pragma unroll
+    for (int e = 0; e < DB; ++e)
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[e] = __builtin_amdgcn_mfma_f32_32x32x2f32(vr[e][r], sc[r], o[e], 0, 0, 0);
-    }
+    __builtin_amdgcn_wave_barrier();  // the next trip overwrites the staging area
   }
+  __syncthreads();  // every wave is done with its staging area: the merge buffers may take it over
 
   // merge the four waves' partial results in wave order
   if (wave != 0) {
@@ -553,7 +605,7 @@ __global__ void __launch_bounds__(256 * GROUPS) attention_prefill_kernel(const f
 #pragma unroll
   for (int w = 0; w < 3; ++w) m_tot = fmaxf(m_tot, merge_ml[w][0][lane]);
   // key 0 is visible to every query and belongs to wave 0's first block: m_tot is finite
-  float f = expf(m_run - m_tot);
+  float f = att_exp(m_run - m_tot);
   float l_tot = l_half * f;
 #pragma unroll
   for (int e = 0; e < DB; ++e)
@@ -561,7 +613,7 @@ __global__ void __launch_bounds__(256 * GROUPS) attention_prefill_kernel(const f
     for (int r = 0; r < 16; ++r) o[e][r] *= f;
 #pragma unroll
   for (int w = 0; w < 3; ++w) {
-    f = expf(merge_ml[w][0][lane] - m_tot);
+    f = att_exp(merge_ml[w][0][lane] - m_tot);
     l_tot += merge_ml[w][1][lane] * f;
 #pragma unroll
     for (int e = 0; e < DB; ++e)
@@ -803,11 +855,19 @@ int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_off
   // workgroup would give every CU two workgroups anyway; d = 128 needs the whole register file for 4 waves.
   const dim3 paired((n_qb + 1) / 2, (unsigned)(b * n_heads)), single(n_qb, (unsigned)(b * n_heads));
   const bool pair = d <= 64 && (size_t)n_qb * b * n_heads >= 512;
-  if (d == 32 && pair) attention_prefill_kernel<32, 2><<<paired, 512, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, q_row_stride, scale, cp, sp, pp, tl, interleaved);
-  else if (d == 32) attention_prefill_kernel<32, 1><<<single, 256, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, q_row_stride, scale, cp, sp, pp, tl, interleaved);
-  else if (d == 64 && pair) attention_prefill_kernel<64, 2><<<paired, 512, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, q_row_stride, scale, cp, sp, pp, tl, interleaved);
-  else if (d == 64) attention_prefill_kernel<64, 1><<<single, 256, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, q_row_stride, scale, cp, sp, pp, tl, interleaved);
-  else attention_prefill_kernel<128, 1><<<single, 256, 0, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, q_row_stride, scale, cp, sp, pp, tl, interleaved);
+  hipError_t err = hipSuccess;
+  auto go = [&](auto kernel, int dd, int groups, dim3 grid) {
+    const size_t lds = (size_t)4 * groups * 32 * (2 * dd + 12) * sizeof(float);  // per wave: 32 rows of d + 4 and of d + 8 floats
+    err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (err != hipSuccess) return;
+    kernel<<<grid, 256 * groups, lds, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, q_row_stride, scale, cp, sp, pp, tl, interleaved);
+  };
+  if (d == 32 && pair) go(attention_prefill_kernel<32, 2>, 32, 2, paired);
+  else if (d == 32) go(attention_prefill_kernel<32, 1>, 32, 1, single);
+  else if (d == 64 && pair) go(attention_prefill_kernel<64, 2>, 64, 2, paired);
+  else if (d == 64) go(attention_prefill_kernel<64, 1>, 64, 1, single);
+  else go(attention_prefill_kernel<128, 1>, 128, 1, single);
+  UGHIP_HIPCHK(err);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
 }
