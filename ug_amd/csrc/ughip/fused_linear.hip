@@ -83,31 +83,27 @@ __global__ void __launch_bounds__(256) fused_gemv(FusedArgs a) {
     const float* __restrict__ X = a.x;
     constexpr int stride = 64 * 4 * KS;
     int k = (ks * 64 + lane) * 4;
-    for (; k + 3 * stride < a.k; k += 4 * stride) {
-      const f32x4 w0 = *reinterpret_cast<const f32x4*>(W0 + k), w1 = *reinterpret_cast<const f32x4*>(W0 + k + stride);
-      const f32x4 w2 = *reinterpret_cast<const f32x4*>(W0 + k + 2 * stride), w3 = *reinterpret_cast<const f32x4*>(W0 + k + 3 * stride);
-      f32x4 u0, u1, u2, u3;
-      if (MODE == MODE_GATE_UP) {
-        u0 = *reinterpret_cast<const f32x4*>(W1 + k), u1 = *reinterpret_cast<const f32x4*>(W1 + k + stride);
-        u2 = *reinterpret_cast<const f32x4*>(W1 + k + 2 * stride), u3 = *reinterpret_cast<const f32x4*>(W1 + k + 3 * stride);
+    // four slabs per trip, all requested before the first is used; slabs past the end of the row
+    // are skipped lane by lane (a short row must not turn into a chain of single loads)
+    for (; k < a.k; k += 4 * stride) {
+      const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+      f32x4 w[4], u[4], x[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int ki = k + i * stride;
+        w[i] = u[i] = x[i] = zero;
+        if (ki < a.k) {
+          w[i] = *reinterpret_cast<const f32x4*>(W0 + ki);
+          if (MODE == MODE_GATE_UP) u[i] = *reinterpret_cast<const f32x4*>(W1 + ki);
+          x[i] = *reinterpret_cast<const f32x4*>(X + ki);
+        }
       }
-      const f32x4 x0 = *reinterpret_cast<const f32x4*>(X + k), x1 = *reinterpret_cast<const f32x4*>(X + k + stride);
-      const f32x4 x2 = *reinterpret_cast<const f32x4*>(X + k + 2 * stride), x3 = *reinterpret_cast<const f32x4*>(X + k + 3 * stride);
-      acc0 = dot4(w0, x0, acc0);
-      acc0 = dot4(w1, x1, acc0);
-      acc0 = dot4(w2, x2, acc0);
-      acc0 = dot4(w3, x3, acc0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc0 = dot4(w[i], x[i], acc0);
       if (MODE == MODE_GATE_UP) {
-        acc1 = dot4(u0, x0, acc1);
-        acc1 = dot4(u1, x1, acc1);
-        acc1 = dot4(u2, x2, acc1);
-        acc1 = dot4(u3, x3, acc1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc1 = dot4(u[i], x[i], acc1);
       }
-    }
-    for (; k < a.k; k += stride) {
-      const f32x4 x0 = *reinterpret_cast<const f32x4*>(X + k);
-      acc0 = dot4(*reinterpret_cast<const f32x4*>(W0 + k), x0, acc0);
-      if (MODE == MODE_GATE_UP) acc1 = dot4(*reinterpret_cast<const f32x4*>(W1 + k), x0, acc1);
     }
   }
   acc0 = wave_sum(acc0);
