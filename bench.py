@@ -102,6 +102,46 @@ def cpu_baseline(a, b, truth, budget_s=12.0):
             "host_cpus": os.cpu_count()}
 
 
+def cpu_extras(budget_s=4.0):
+    """The CPU oracle (restatement of ug's CPU backend) on configs 1 and 3, timed on this box's host
+    cores next to the GPU numbers: each a bounded sample of the same workload."""
+    from conftest import _oracle_lib
+    import ug_amd
+    from ug_amd import LazyBuffer as LB, Schedule, rng
+    lib = _oracle_lib()
+    h = C.c_void_p()
+    assert lib.ugo_cpu_device_new(C.byref(h)) == 0
+    cpu = ug_amd.Device(h.value)
+    out = {}
+
+    def sample(run):
+        run()
+        n, t0 = 0, time.perf_counter()
+        while True:
+            run()
+            n += 1
+            el = time.perf_counter() - t0
+            if el > budget_s:
+                return n, el
+
+    rows, cols = 32, 1024
+    sm = ug_amd.llama.softmax(LB.copy(rng.normal(1, rows * cols, 3.0), (rows, cols), cpu))
+    cs = Schedule.create_one(sm).compile()
+    n, el = sample(cs.run)
+    out["cpu_softmax_lazy_32x1024"] = {"us_per_softmax": round(el / n * 1e6, 1), "GB/s": round(8.0 * rows * cols * n / el / 1e9, 4), "cores": 1, "kind": "port",
+                                       "sample": f"{n} runs of the two kernels the reference's lowering emits (max and sum recomputed per element) in {el:.1f} s"}
+    b, m = 8, 1024
+    threads = min(16, os.cpu_count() or 1)   # a one-GPU box's share of host cores
+    os.environ.setdefault("RAYON_NUM_THREADS", str(threads))   # the oracle's matmul reads it, like the reference (utils.rs:3-20)
+    a, w = rng.uniform_pm1(4, b * m * m), rng.uniform_pm1(5, b * m * m)
+    mm = LB.copy(a, (b, m, m), cpu).matmul(LB.copy(w, (b, m, m), cpu))
+    cs = Schedule.create_one(mm).compile()
+    n, el = sample(cs.run)
+    out["cpu_bmm_f32_8x1024^3"] = {"TFLOP/s": round(2.0 * b * m * m * m * n / el / 1e12, 4), "ms": round(el / n * 1e3, 1), "cores": int(os.environ["RAYON_NUM_THREADS"]), "kind": "port",
+                                   "sample": f"{n} runs in {el:.1f} s; the reference multiplies with the gemm crate, the oracle with its own blocked loops"}
+    return out
+
+
 def extras(dev, steps, warmup, only=None):
     """Other single-GPU configs of BASELINE.json: GB/s or TFLOP/s with the roofline fraction."""
     out = {}
@@ -113,6 +153,8 @@ def extras(dev, steps, warmup, only=None):
         out.update(llama_pieces(dev, steps, warmup))
     if only in (None, "safetensors"):
         out.update(safetensors_load(dev))
+    if only in (None, "cpu"):
+        out.update(cpu_extras())
     return out
 
 
@@ -304,7 +346,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-llama", action="store_true")
     ap.add_argument("--headline-only", action="store_true", help="only the config-2 kernel: no extras, no llama, no CPU baseline")
-    ap.add_argument("--only", choices=["softmax", "bmm", "llama_pieces", "safetensors", "llama"], help="besides the headline, run just this group (profiler runs)")
+    ap.add_argument("--only", choices=["softmax", "bmm", "llama_pieces", "safetensors", "cpu", "llama"], help="besides the headline, run just this group (profiler runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true", help="also run a plain 2^24-element copy kernel (counter calibration)")
     args = ap.parse_args()
