@@ -427,7 +427,9 @@ int pick_split(int dtype, const MMArgs& p, size_t batch, int shape) {
   const size_t tiles = batch * (size_t)(p.M / kShapes[shape][0]) * (size_t)(p.N / kShapes[shape][1]);
   const int kt = p.K / bk;
   if (tiles >= 128 || kt < 8) return 1;
-  int want = (int)((256 + tiles - 1) / tiles);
+  // three workgroups per CU: measured on the projections of a 128-token prefill, short slabs overlap
+  // each other's pipeline fill better than one workgroup per CU with longer ones
+  int want = (int)((768 + tiles - 1) / tiles);
   want = std::min(want, kt / 4);  // at least 4 K tiles per slab
   return std::max(1, std::min(want, 32));
 }
