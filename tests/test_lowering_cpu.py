@@ -26,6 +26,38 @@ def test_c_abi_exports_every_declared_symbol():
     assert lib.ughip_use_grid() == 0
 
 
+def test_entry_points_refuse_a_null_device_without_touching_the_gpu():
+    """Argument checks come before any HIP call: every data entry point answers a null device (or null
+    slices) with an error code and a message, on a box without a GPU too."""
+    lib = ug_amd.ughip_lib()
+    z, n3 = C.c_size_t(0), (C.c_size_t * 3)(4, 4, 4)
+    f = C.c_float(1.0)
+    calls = {
+        "ughip_softmax_rows": (None, None, None, z, z),
+        "ughip_causal_mask": (None, None, None, z, z, z),
+        "ughip_rope": (None, None, None, None, None, None, z, z, z, 0),
+        "ughip_cat": (None, None, None, None, z, z, z),
+        "ughip_causal_softmax_rows": (None, None, None, z, z, z),
+        "ughip_attention_decode": (None, None, None, None, None, z, z, z, z, z, f),
+        "ughip_rope_append": (None, None, None, None, z, z, z, None, None, None, 0),
+        "ughip_kv_append": (None, None, None, z, z, z, z, z, z, z, z, None, None, None, 0),
+        "ughip_attention_cached": (None, None, z, z, None, None, None, z, z, z, C.c_size_t(2), z, z, C.c_size_t(64), f, None, None, None, 0),
+        "ughip_attention_step": (None, None, z, z, z, z, None, None, None, z, z, z, z, z, z, f, None, None, None, 0),
+        "ughip_gemv_multi": (None, None, C.c_size_t(1), None, n3, C.c_size_t(4), None),
+        "ughip_rms_gemv_multi": (None, None, None, f, C.c_size_t(1), None, n3, C.c_size_t(4), None),
+        "ughip_gemv_gate_up": (None, None, None, None, None, z, C.c_size_t(4)),
+        "ughip_rms_gemv_gate_up": (None, None, None, f, None, None, None, z, C.c_size_t(4)),
+        "ughip_gemv_add": (None, None, None, None, None, z, C.c_size_t(4)),
+        "ughip_argmax_row": (None, None, C.c_size_t(4), z, None, None, None, z),
+        "ughip_convert": (None, None, None),
+        "ughip_matmul": (None, None, None, None, z, z, z, z, z, None, None, z, None, None, z),
+    }
+    for name, args in calls.items():
+        rc = getattr(lib, name)(*args)
+        assert rc != 0, name
+        assert lib.ughip_last_error(), name
+
+
 def test_no_gpu_is_a_loud_error_not_a_fallback():
     lib = ug_amd.ughip_lib()
     dev = C.c_void_p()
