@@ -1044,16 +1044,17 @@ def test_argmax_into(hip, hip_ops, rows, n, row):
     assert np.all(v[:4] == 0) and np.all(v[6:] == 0)
 
 
-@pytest.mark.parametrize("level", [0, 3])
-def test_queued_greedy_decode_matches_the_read_back_loop(hip, hip_ops, level, monkeypatch):
+@pytest.mark.parametrize("level,n_steps", [(0, 12), (3, 12), (3, 400)])
+def test_queued_greedy_decode_matches_the_read_back_loop(hip, hip_ops, level, n_steps, monkeypatch):
     """Tokens picked on the device and fed to the next step without a read-back: same ids and
-    margins as the loop that copies the logits to the host for every token."""
-    cfg = ug_amd.LlamaConfig(num_hidden_layers=2, max_position_embeddings=256)
+    margins as the loop that copies the logits to the host for every token.  400 steps let the
+    launches run far ahead of the device and recycle every buffer of the pool many times."""
+    cfg = ug_amd.LlamaConfig(num_hidden_layers=2, max_position_embeddings=512)
     prompt = rng.token_ids(10, 16, cfg.vocab_size)
     model = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=0.02, fused_attention=level)
-    ids_q, st_q = model.generate(prompt, 12)
+    ids_q, st_q = model.generate(prompt, n_steps)
     monkeypatch.setenv("UG_LLAMA_HOST_ARGMAX", "1")
-    ids_h, st_h = model.generate(prompt, 12)
+    ids_h, st_h = model.generate(prompt, n_steps)
     assert ids_q.tolist() == ids_h.tolist()
     np.testing.assert_array_equal(st_q["margins"], st_h["margins"])
 
