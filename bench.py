@@ -239,6 +239,14 @@ def bmm(dev, steps, warmup):
     _, ms = timed(dev, lambda: dev.matmul(dst, sa, sw, (b, m, m, m), lay, lay), steps, warmup)
     tf = flop * steps / (ms * 1e-3) / 1e12
     out["bmm_bf16_8x1024^3"] = {"TFLOP/s": round(tf, 2), "frac_mfma_bf16": round(tf / MFMA_BF16_PEAK_TF, 4), "us": round(ms * 1e3 / steps, 1)}
+    # a large product with the rhs stored [n, k] (what matmul_t of the llama projections hands over): 256 tiles of 256 x 256
+    m = 4096
+    a, w = rng.uniform_pm1(4, m * m), rng.uniform_pm1(5, m * m)
+    sa, sw = dev.slice_from(rng.to_bf16_bits(a)), dev.slice_from(rng.to_bf16_bits(w))
+    dst = dev.allocate_uninit(ug_amd.BF16, m * m)
+    _, ms = timed(dev, lambda: dev.matmul(dst, sa, sw, (1, m, m, m), ((1, m, m), (m * m, m, 1), 0), ((1, m, m), (m * m, 1, m), 0)), steps, warmup)
+    tf = 2.0 * m * m * m * steps / (ms * 1e-3) / 1e12
+    out["mm_bf16_nt_4096^3"] = {"TFLOP/s": round(tf, 2), "frac_mfma_bf16": round(tf / MFMA_BF16_PEAK_TF, 4), "us": round(ms * 1e3 / steps, 1)}
     return out
 
 

@@ -333,6 +333,31 @@ def test_matmul_bf16_tile_multiples(hip, bmnk, rhs_nk):
     assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-12)
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("bmnk", [(1, 4096, 4096, 64), (1, 4096, 4096, 128), (4, 2048, 2048, 192), (1, 8192, 2048, 320), (16, 1024, 1024, 64)])
+def test_matmul_16bit_256x256_tiles(hip, bmnk, dtype):
+    """[n, k]-major rhs and at least 256 tiles of 256 x 256: the kernel whose loads write LDS directly
+    (1, 2, 3 and 5 K tiles: prologue only, both stages, the steady state)."""
+    b, m, n, k = bmnk
+    print("matmul 256x256", dtype, bmnk, flush=True)
+    rnd = rng.bf16_round if dtype == "bf16" else (lambda v: v.astype(np.float16).astype(np.float32))
+    a = rnd(rng.uniform_pm1(25, b * m * k)).reshape(b, m, k)
+    w = rnd(rng.uniform_pm1(26, b * k * n)).reshape(b, k, n)
+    got = _raw_matmul(hip, ug_amd.BF16 if dtype == "bf16" else ug_amd.F16, a, w, True)
+    exact = np.matmul(a.astype(np.float64), w.astype(np.float64))
+    half_ulp = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
+    bound = half_ulp * np.abs(exact) + k * np.finfo(np.float32).eps * np.matmul(np.abs(a).astype(np.float64), np.abs(w).astype(np.float64))
+    assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-7)
+    # the same product through the register-staged 256 x 128 kernel: same k order, bit for bit
+    import os
+    os.environ["UGHIP_GEMM_SHAPE"] = "0"
+    try:
+        other = _raw_matmul(hip, ug_amd.BF16 if dtype == "bf16" else ug_amd.F16, a, w, True)
+    finally:
+        del os.environ["UGHIP_GEMM_SHAPE"]
+    np.testing.assert_array_equal(got, other)
+
+
 # The m <= 8 shapes of decode: wave-per-column GEMV with 1, 2 or 4 waves per column, the short-k
 # variant (attention scores) and the [k, n]-major variant (attention output).
 GEMV_SHAPES = [(1, 1, 2048, 2048), (1, 1, 5000, 512), (1, 1, 7000, 256), (1, 3, 640, 320), (2, 8, 300, 1024), (32, 1, 129, 64), (32, 1, 77, 128),
