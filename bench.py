@@ -317,29 +317,33 @@ def llama_pieces(dev, steps, warmup):
     return out
 
 
-def llama_decode(dev, n_prompt=128, n_steps=128, fused_attention=0):
+def llama_decode(dev, n_prompt=128, n_steps=128, fused_attention=0, bf16_matrices=False):
     """Config 5: TinyLlama-1.1B shape, random-init f32 weights, prefill 128 then 128 greedy steps.
     Fresh buffers are not zero-filled here (every kernel of the model writes its whole output; the
     ids are the same either way, which the GPU tests check).  fused_attention: 0 = the reference's
     op-by-op graph; 1 = ughip_causal_softmax_rows / ughip_rope_append / ughip_attention_decode;
     2 = caches written in place (ughip_kv_append) and ughip_attention_cached for prefill and decode;
-    3 = 2 plus packed q|k|v, gate/up + SwiGLU and residual projections (ughip_gemv_multi / _gate_up / _add)."""
+    3 = 2 plus packed q|k|v, gate/up + SwiGLU and residual projections (ughip_gemv_multi / _gate_up / _add).
+    bf16_matrices: bf16-rounded weights, the projection matrices and the head kept and streamed as bf16
+    (activations, caches, norms f32): the numbers of the f32 model on the rounded weights from half the bytes."""
     import ug_amd
     from ug_amd import rng
     cfg = ug_amd.LlamaConfig()
     ops = ug_amd.LlamaOps.hip()
     dev.set_zero_fill(False)
     t0 = time.perf_counter()
-    model = ug_amd.LlamaModel(dev, ops, cfg, custom_softmax=True, seed=9, std=0.02, fused_attention=fused_attention)
+    model = ug_amd.LlamaModel(dev, ops, cfg, custom_softmax=True, seed=9, std=0.02, round_bf16=bf16_matrices, fused_attention=fused_attention,
+                              bf16_matrices=bf16_matrices)
     load_s = time.perf_counter() - t0
     prompt = rng.token_ids(10, n_prompt, cfg.vocab_size)
     model.generate(prompt, 4)          # compiles every kernel shape family once
     toks, st = model.generate(prompt, n_steps)
     dev.set_zero_fill(True)
-    weights_bytes = 4 * 1034512384
+    # streamed per token: every matrix once (2 or 4 bytes per weight); the 45 norm vectors stay f32
+    weights_bytes = (2 if bf16_matrices else 4) * 1034512384
     tok_s = n_steps / (st["decode_ms"] * 1e-3)
     return {"tok/s": round(tok_s, 2), "decode_ms_per_token": round(st["decode_ms"] / n_steps, 3), "prefill_ms": round(st["prefill_ms"], 1),
-            "frac_hbm_weights_only": round(tok_s * weights_bytes / 1e9 / HBM_PEAK_GBS, 4), "load_s": round(load_s, 1), "dtype": "f32", "zero_fill": False, "fused_attention": fused_attention,
+            "frac_hbm_weights_only": round(tok_s * weights_bytes / 1e9 / HBM_PEAK_GBS, 4), "load_s": round(load_s, 1), "dtype": "f32 activations, bf16 matrices" if bf16_matrices else "f32", "zero_fill": False, "fused_attention": fused_attention,
             "first_ids": toks[:8].tolist(), "min_top1_margin": float(st["margins"].min())}
 
 
@@ -351,6 +355,7 @@ def main():
     ap.add_argument("--extras", action="store_true", help="(default) kept for older command lines")
     ap.add_argument("--llama", action="store_true", help="(default) kept for older command lines")
     ap.add_argument("--llama-level", type=int, default=None, choices=[0, 1, 2, 3], help="run config 5 at this fusion level only (default: all four)")
+    ap.add_argument("--llama-bf16", action="store_true", help="with --llama-level 3: the run with bf16 matrices instead of the f32 one")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-llama", action="store_true")
     ap.add_argument("--headline-only", action="store_true", help="only the config-2 kernel: no extras, no llama, no CPU baseline")
@@ -412,12 +417,12 @@ def main():
         except Exception as e:  # noqa: BLE001
             line["extras"] = {"error": f"{type(e).__name__}: {e}"}
     if not (args.no_llama or args.headline_only):
-        for key, fused in (("llama_decode_f32", 0), ("llama_decode_f32_fused_attention", 1), ("llama_decode_f32_inplace_cache", 2),
-                           ("llama_decode_f32_fused_projections", 3)):
-            if args.llama_level is not None and fused != args.llama_level:
+        for key, fused, narrow in (("llama_decode_f32", 0, False), ("llama_decode_f32_fused_attention", 1, False), ("llama_decode_f32_inplace_cache", 2, False),
+                                   ("llama_decode_f32_fused_projections", 3, False), ("llama_decode_bf16_matrices", 3, True)):
+            if args.llama_level is not None and (fused != args.llama_level or narrow != args.llama_bf16):
                 continue
             try:
-                line.setdefault("extras", {})[key] = llama_decode(dev, fused_attention=fused)
+                line.setdefault("extras", {})[key] = llama_decode(dev, fused_attention=fused, bf16_matrices=narrow)
             except Exception as e:  # noqa: BLE001
                 line.setdefault("extras", {})[key] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(line), flush=True)

@@ -663,6 +663,29 @@ def test_llama_fused_attention_ids_match_unfused_cpu(hip, cpu, hip_ops, cpu_ops,
     np.testing.assert_allclose(st_h["margins"], st_c["margins"], rtol=1e-2, atol=1e-7)
 
 
+@pytest.mark.parametrize("width", ["small", "config5"])
+def test_llama_bf16_matrices_are_the_rounded_f32_model(hip, cpu, hip_ops, cpu_ops, width):
+    """Matrices kept and streamed as bf16 (fusion level 3): token for token and margin for margin the
+    f32 model on the same device whose weights hold the same (bf16-representable) values; ids equal to
+    the oracle's op-by-op f32 graph on those weights."""
+    if width == "small":
+        cfg = ug_amd.LlamaConfig(hidden_size=128, intermediate_size=320, max_position_embeddings=64, num_attention_heads=4, num_key_value_heads=2,
+                                 num_hidden_layers=2, vocab_size=512)
+        n_prompt, n_steps, std = 12, 10, 0.3
+    else:
+        cfg = ug_amd.LlamaConfig(num_hidden_layers=2, max_position_embeddings=256)
+        n_prompt, n_steps, std = 16, 6, 0.02
+    prompt = rng.token_ids(10, n_prompt, cfg.vocab_size)
+    wide = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=std, round_bf16=True, fused_attention=3).generate(prompt, n_steps)
+    toks, st = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=std, round_bf16=True, fused_attention=3, bf16_matrices=True).generate(prompt, n_steps)
+    print("bf16 matrices", toks.tolist(), flush=True)
+    assert toks.tolist() == wide[0].tolist()
+    assert np.array_equal(st["margins"], wide[1]["margins"])
+    toks_c, st_c = ug_amd.LlamaModel(cpu, cpu_ops, cfg, True, seed=9, std=std, round_bf16=True).generate(prompt, n_steps)
+    assert wide[0].tolist() == toks_c.tolist()
+    np.testing.assert_allclose(wide[1]["margins"], st_c["margins"], rtol=1e-2, atol=1e-7)
+
+
 def _rope_tables(dev, hd, max_pos=64):
     cfg = ug_amd.LlamaConfig(hidden_size=hd * 4, num_attention_heads=4, num_key_value_heads=2, max_position_embeddings=max_pos)
     cos, sin = ug_amd.llama.rope_tables(dev, cfg)
@@ -960,6 +983,86 @@ def test_projections_with_the_norm_folded_in(hip, cpu, hip_ops, cpu_ops, k):
     got, want = gated(hip, hip_ops), gated(cpu, cpu_ops)
     assert np.all(np.abs(got - truth) <= tol_g)
     assert np.all(np.abs(got - want) <= 2 * tol_g)
+
+
+@pytest.mark.parametrize("k,n", [(2048, 96), (5632, 33), (128, 64), (260, 9), (4096, 5)])
+def test_fused_projections_take_bf16_matrices(hip, hip_ops, k, n):
+    """Matrices stored as bf16 (x, the sums and the result stay f32): a bf16 widens exactly and the
+    sums run in the same order, so every hook gives bit for bit what it gives for f32 matrices
+    holding the same values."""
+    print("bf16 matrices", k, n, flush=True)
+    eps = 1e-5
+    x, alpha, r = rng.normal(121, k, 2.0), rng.normal(122, k, 0.5), rng.normal(123, n)
+    ws = [rng.bf16_round(rng.normal(124 + i, n * k, 0.05)) for i in range(3)]
+
+    def mats(bf16, idx):
+        return [LB.copy(rng.to_bf16_bits(ws[i]) if bf16 else ws[i], (n, k), hip) for i in idx]
+
+    def xs():
+        return LB.copy(x, (1, 1, k), hip)
+
+    for norm in (False, True):
+        extra = (LB.copy(alpha, (k,), hip), eps) if norm else ()
+        wide = hip_ops.linear_packed(xs(), mats(False, (0, 1, 2)), *extra).data_vec()
+        narrow = hip_ops.linear_packed(xs(), mats(True, (0, 1, 2)), *extra)
+        assert narrow.dtype == ug_amd.F32
+        assert np.array_equal(narrow.data_vec(), wide)
+        extra = (LB.copy(alpha, (k,), hip), eps) if norm else ()
+        wide = hip_ops.gate_up(xs(), *mats(False, (0, 1)), *extra).data_vec()
+        assert np.array_equal(hip_ops.gate_up(xs(), *mats(True, (0, 1)), *extra).data_vec(), wide)
+    res = LB.copy(r, (1, 1, n), hip)
+    wide = hip_ops.linear_add(xs(), mats(False, (2,))[0], res).data_vec()
+    assert np.array_equal(hip_ops.linear_add(xs(), mats(True, (2,))[0], LB.copy(r, (1, 1, n), hip)).data_vec(), wide)
+    # and against float64 on the rounded values
+    truth = ws[2].reshape(n, k).astype(np.float64) @ x.astype(np.float64) + r
+    assert np.all(np.abs(wide - truth) <= _gemv_tol(x, ws[2].reshape(n, k)) + 1e-6 * np.abs(truth))
+
+
+def test_bf16_matrices_meet_several_rows_through_a_cast(hip, hip_ops):
+    """Prefill shapes: a bf16 matrix is widened in front of matmul (one dtype per product,
+    ug-core/src/lib.rs:62-70) and the result is that of the f32 matrix with the same values."""
+    t, k, n = 5, 256, 48
+    x = rng.normal(131, t * k)
+    ws = [rng.bf16_round(rng.normal(132 + i, n * k, 0.05)) for i in range(2)]
+    r = rng.normal(135, t * n)
+
+    def run(bf16):
+        m = [LB.copy(rng.to_bf16_bits(w) if bf16 else w, (n, k), hip) for w in ws]
+        a = hip_ops.linear_packed(LB.copy(x, (1, t, k), hip), m).data_vec()
+        g = hip_ops.gate_up(LB.copy(x, (1, t, k), hip), m[0], m[1]).data_vec()
+        o = hip_ops.linear_add(LB.copy(x, (1, t, k), hip), m[1], LB.copy(r, (1, t, n), hip)).data_vec()
+        return a, g, o
+
+    for got, want in zip(run(True), run(False)):
+        assert np.array_equal(got, want)
+
+
+def test_fused_projections_refuse_mixed_or_other_matrix_dtypes(hip):
+    """Straight through the C ABI: one matrix dtype per call, F32 or BF16."""
+    lib, dev = ug_amd.ughip_lib(), C.c_void_p(hip.raw_hip())
+    k, n = 64, 8
+
+    def alloc(dtype, length):
+        out = C.c_void_p()
+        assert lib.ughip_alloc(dev, dtype, C.c_size_t(length), C.byref(out)) == 0
+        return out
+
+    x, dst = alloc(ug_amd.F32, k), alloc(ug_amd.F32, 2 * n)
+    wf, wb, wh = alloc(ug_amd.F32, n * k), alloc(ug_amd.BF16, n * k), alloc(ug_amd.F16, n * k)
+
+    def multi(ws):
+        arr = (C.c_void_p * len(ws))(*[w.value for w in ws])
+        ns = (C.c_size_t * len(ws))(*[n] * len(ws))
+        return lib.ughip_gemv_multi(dev, x, C.c_size_t(len(ws)), arr, ns, C.c_size_t(k), dst)
+
+    assert multi([wf, wb]) != 0 and b"share a dtype" in lib.ughip_last_error()
+    assert multi([wh]) != 0 and b"F32 or BF16" in lib.ughip_last_error()
+    assert lib.ughip_gemv_gate_up(dev, x, wb, wf, dst, C.c_size_t(n), C.c_size_t(k)) != 0 and b"share a dtype" in lib.ughip_last_error()
+    assert lib.ughip_gemv_add(dev, x, wh, dst, dst, C.c_size_t(n), C.c_size_t(k)) != 0
+    assert multi([wb, wb]) == 0, lib.ughip_last_error()
+    assert lib.ughip_synchronize(dev) == 0
+    for sl in (x, dst, wf, wb, wh):
+        lib.ughip_free(sl)
 
 
 def test_projections_with_the_norm_need_a_short_row(hip, hip_ops):

@@ -804,18 +804,20 @@ class LlamaModel(_Handle):
     """ug_llama::Model with random-init weights N(0, std) from the seeded generator."""
     _free = "ugh_llama_model_free"
 
-    def __init__(self, device, ops, cfg, custom_softmax=False, seed=9, std=0.02, round_bf16=False, fused_attention=False):
+    def __init__(self, device, ops, cfg, custom_softmax=False, seed=9, std=0.02, round_bf16=False, fused_attention=False, bf16_matrices=False):
         out = C.c_void_p()
         _chk(host_lib().ugh_llama_model_new(_p(device.h), _p(ops.h), C.byref(cfg), int(custom_softmax), C.c_uint64(seed), C.c_float(std),
                                             int(round_bf16), C.byref(out)))
         super().__init__(out.value)
         if fused_attention:
             _chk(host_lib().ugh_llama_model_set_fused_attention(_p(self.h), int(fused_attention)))
+        if bf16_matrices:
+            _chk(host_lib().ugh_llama_model_store_matrices_bf16(_p(self.h)))
         self._keep = [device, ops]
         self.cfg = cfg
 
     @classmethod
-    def from_safetensors(cls, device, ops, cfg, paths, custom_softmax=False, fused_attention=False):
+    def from_safetensors(cls, device, ops, cfg, paths, custom_softmax=False, fused_attention=False, bf16_matrices=False):
         """Weights by their HF names from safetensors file(s), cast to f32 (model.rs:299-346)."""
         if isinstance(paths, (str, bytes, os.PathLike)):
             paths = [paths]
@@ -828,6 +830,8 @@ class LlamaModel(_Handle):
         self.cfg = cfg
         if fused_attention:
             _chk(host_lib().ugh_llama_model_set_fused_attention(_p(self.h), int(fused_attention)))
+        if bf16_matrices:
+            _chk(host_lib().ugh_llama_model_store_matrices_bf16(_p(self.h)))
         return self
 
     def generate(self, prompt, n_steps):

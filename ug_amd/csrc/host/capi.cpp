@@ -554,6 +554,9 @@ void ugh_llama_model_free(void* m) { delete static_cast<ug_llama::Model*>(m); }
 int ugh_llama_model_set_fused_attention(void* m, int on) {
   return guard([&] { static_cast<ug_llama::Model*>(m)->set_fused_attention(on); });
 }
+int ugh_llama_model_store_matrices_bf16(void* m) {
+  return guard([&] { static_cast<ug_llama::Model*>(m)->store_matrices_bf16(); });
+}
 int ugh_llama_generate(void* m, const int32_t* prompt, size_t n_prompt, size_t n_steps, int32_t* out_tokens, double* prefill_ms,
                        double* decode_ms, float* margins) {
   return guard([&] {

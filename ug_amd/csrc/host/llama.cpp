@@ -231,11 +231,14 @@ struct HipOps : Ops {
     return LB::custom(f, args, Shape({b, t, nh * d}), q.dtype(), q.device());
   }
 
-  // One input row of f32 against row-major [n, k] matrices: the shapes the fused GEMV kernels take.
+  // One input row of f32 against row-major [n, k] matrices stored as f32 or bf16 (all alike): the
+  // shapes the fused GEMV kernels take.
   static bool one_f32_row(const LB& x, const std::vector<const LB*>& ws) {
     if (x.rank() != 3 || x.dims()[0] * x.dims()[1] != 1 || x.dtype() != DType::F32 || x.dims()[2] % 4 != 0) return false;
-    for (const LB* w : ws)
-      if (w->rank() != 2 || w->dims()[1] != x.dims()[2] || w->dtype() != DType::F32) return false;
+    for (const LB* w : ws) {
+      if (w->rank() != 2 || w->dims()[1] != x.dims()[2] || w->dtype() != ws[0]->dtype()) return false;
+      if (w->dtype() != DType::F32 && w->dtype() != DType::BF16) return false;
+    }
     return true;
   }
 
@@ -449,23 +452,29 @@ LB Ops::attention_step(const LB&, const LB&, const LB&, size_t, size_t, float, c
 
 LB Ops::argmax_into(const LB&, const LB&, size_t, const LB&, const LB&, size_t) const { bail("argmax_into: this device reads the logits back and picks the token on the host"); }
 
+namespace {
+// A matrix kept in bf16 meets activations of another dtype: matmul wants one dtype throughout
+// (ug-core/src/lib.rs:62-70), so the matrix is widened for this use (exact).
+LB like(const LB& w, const LB& x) { return w.dtype() == x.dtype() ? w : w.cast(x.dtype()); }
+}  // namespace
+
 // model.rs:206-208 side by side.
 LB Ops::linear_packed(const LB& x0, const std::vector<LB>& ws, const LB* alpha, float eps) const {
   if (ws.empty()) bail("linear_packed: no matrices");
   LB x = alpha ? rms_norm(x0, *alpha, eps) : x0;
-  LB out = x.matmul_t(ws[0]);
-  for (size_t i = 1; i < ws.size(); ++i) out = cat(out, x.matmul_t(ws[i]), x.rank() - 1);
+  LB out = x.matmul_t(like(ws[0], x));
+  for (size_t i = 1; i < ws.size(); ++i) out = cat(out, x.matmul_t(like(ws[i], x)), x.rank() - 1);
   return out;
 }
 
 // model.rs:160-168 up to the down projection.
 LB Ops::gate_up(const LB& x0, const LB& w_gate, const LB& w_up, const LB* alpha, float eps) const {
   LB x = alpha ? rms_norm(x0, *alpha, eps) : x0;
-  return silu(x.matmul_t(w_gate)).binary(BinaryOp::Mul, x.matmul_t(w_up));
+  return silu(x.matmul_t(like(w_gate, x))).binary(BinaryOp::Mul, x.matmul_t(like(w_up, x)));
 }
 
 // model.rs:366-372: a projection, then the residual.
-LB Ops::linear_add(const LB& x, const LB& w, const LB& residual) const { return x.matmul_t(w).binary(BinaryOp::Add, residual); }
+LB Ops::linear_add(const LB& x, const LB& w, const LB& residual) const { return x.matmul_t(like(w, x)).binary(BinaryOp::Add, residual); }
 
 std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16) {
   return std::make_shared<SyntheticWeights>(seed, std, round_bf16);
@@ -626,6 +635,7 @@ Model::Model(const Config& cfg, bool custom_softmax, WeightSource& w, const Devi
   if (!cfg.tie_word_embeddings) bail("tie_word_embeddings == false is not supported yet");
   size_t h = cfg.hidden_size, isz = cfg.intermediate_size, kv = cfg.head_dim() * cfg.num_key_value_heads;
   embedding_ = load_w(w, "model.embed_tokens.weight", {cfg.vocab_size, h}, dev);
+  head_ = embedding_;  // tied (model.rs:315-319)
   ln_f_ = load_w(w, "model.norm.weight", {h}, dev);
   for (size_t i = 0; i < cfg.num_hidden_layers; ++i) {
     std::string p = "model.layers." + std::to_string(i);
@@ -650,7 +660,7 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
   size_t seq_len = xs_in.dims()[1];
   size_t nh = cfg_.num_attention_heads, nkv = cfg_.num_key_value_heads, hd = cfg_.head_dim();
   const float eps = (float)cfg_.rms_norm_eps;
-  auto finish = [&](const LB& out) { return residual ? ops_->linear_add(out, l.o_proj, *residual) : out.matmul_t(l.o_proj); };
+  auto finish = [&](const LB& out) { return residual ? ops_->linear_add(out, l.o_proj, *residual) : out.matmul_t(like(l.o_proj, out)); };
   if (fused_attention_ >= 3 && seq_len == 1 && xs_in.dims()[0] == 1 && cache.capacity && ops_->packed_projections()) {
     // one position: q | k | v come out of one launch (with the norm in front) side by side and are read where they lie
     const size_t nq = nh * hd, nk = nkv * hd, row = nq + 2 * nk, len = cache.len;
@@ -664,9 +674,9 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
     return finish(ops_->attention_cached(qkv, kc, vc, cache.len, scale, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, 0, row, nh));
   }
   LB xs = norm_first ? rms_norm(xs_in, l.rms1, eps) : xs_in;
-  LB q = xs.matmul_t(l.q_proj);
-  LB k = xs.matmul_t(l.k_proj);
-  LB v = xs.matmul_t(l.v_proj);
+  LB q = xs.matmul_t(like(l.q_proj, xs));
+  LB k = xs.matmul_t(like(l.k_proj, xs));
+  LB v = xs.matmul_t(like(l.v_proj, xs));
   if (fused_attention_ >= 2) {
     // rows go from the projections into the caches (in place when they were preallocated) and
     // the attention kernel reads them there; the result comes back in the layout o_proj reads
@@ -725,10 +735,30 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
 LB Model::mlp(const Layer& l, const LB& xs, const LB* residual, bool norm_first) const {
   if (residual)
     return ops_->linear_add(ops_->gate_up(xs, l.gate_proj, l.up_proj, norm_first ? &l.rms2 : nullptr, (float)cfg_.rms_norm_eps), l.down_proj, *residual);
-  LB xs1 = xs.matmul_t(l.gate_proj);
-  LB xs2 = xs.matmul_t(l.up_proj);
+  LB xs1 = xs.matmul_t(like(l.gate_proj, xs));
+  LB xs2 = xs.matmul_t(like(l.up_proj, xs));
   xs1 = silu(xs1);
-  return xs1.binary(BinaryOp::Mul, xs2).matmul_t(l.down_proj);
+  return xs1.binary(BinaryOp::Mul, xs2).matmul_t(like(l.down_proj, xs));
+}
+
+void Model::store_matrices_bf16() {
+  if (bf16_matrices_) return;
+  auto narrow = [](LB& w) {
+    LB n = w.cast(DType::BF16);
+    n.realize();
+    n.detach();
+    w = n;
+  };
+  for (Layer& l : layers_)
+    for (LB* w : {&l.q_proj, &l.k_proj, &l.v_proj, &l.o_proj, &l.gate_proj, &l.up_proj, &l.down_proj}) narrow(*w);
+  narrow(head_);
+  // The lookup reads t rows and keeps an f32 table, the head streams all of the bf16 one; both hold
+  // the same values (one tied tensor, model.rs:315-319).
+  LB wide = head_.cast(DType::F32);
+  wide.realize();
+  wide.detach();
+  embedding_ = wide;
+  bf16_matrices_ = true;
 }
 
 std::vector<Cache> Model::new_cache() const {
@@ -757,9 +787,9 @@ LB Model::fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const 
     m = mlp(l, m, nullptr, false);
     xs = m.binary(BinaryOp::Add, residual);
   }
-  if (fused_attention_ >= 3) return ops_->linear_packed(xs, {embedding_}, &ln_f_, eps);
+  if (fused_attention_ >= 3) return ops_->linear_packed(xs, {head_}, &ln_f_, eps);
   xs = rms_norm(xs, ln_f_, eps);
-  return xs.matmul_t(embedding_);
+  return xs.matmul_t(like(head_, xs));
 }
 
 // One prefill call over the prompt, then `n_steps` greedy single-token steps (graph rebuilt per

@@ -159,6 +159,13 @@ class Model {
   //    residual): 7 schedule items per layer and decode step on a device that fuses them.
   void set_fused_attention(int level) { fused_attention_ = level; }
   int fused_attention() const { return fused_attention_; }
+  // Keep the projection matrices and the output head in bf16 (rounded to nearest even when they
+  // are not bf16 values already) and stream them in that form; activations stay f32.  The numbers
+  // are those of a model whose f32 weights hold the rounded values - what a bf16 checkpoint gives
+  // after load_with_cast(.., F32, ..) (model.rs:118,140,313) - because every use widens exactly:
+  // inside the fused one-row projections of level 3, through a cast in front of matmul elsewhere.
+  void store_matrices_bf16();
+  bool bf16_matrices() const { return bf16_matrices_; }
   // Caches of the kind fwd() expects at the current fusion level.
   std::vector<Cache> new_cache() const;
   LB fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const;
@@ -182,7 +189,8 @@ class Model {
   int fused_attention_ = 0;
   ug::DevicePtr dev_;
   std::shared_ptr<Ops> ops_;
-  LB embedding_, ln_f_;
+  LB embedding_, head_, ln_f_;
+  bool bf16_matrices_ = false;
   Rope rope_;
   std::vector<Layer> layers_;
 };

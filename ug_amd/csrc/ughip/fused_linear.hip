@@ -14,10 +14,17 @@
 // product is the same fixed-order f32 sum a separate ughip_matmul computes, the epilogues are
 // the same f32 operations the lazy graph would run on the rounded products.
 //
+// The matrices may be stored as BF16 (all of one call alike) while x, the sums and y stay F32: a
+// bf16 widens to f32 exactly, so the result is bit for bit the one the F32 kernel gives on the
+// same values, from half the bytes - decode streams every weight once per token and nothing else
+// of that size.  (ug's Device::matmul wants one dtype for all three operands, ug-core/src/lib.rs:62-70;
+// a checkpoint stored in bf16 is widened at load time, ug-core/src/safetensors.rs:120-271.)
+//
 // KS waves share one output column, each walking every KS-th 64-lane slab of k with four 128-bit
 // loads in flight per lane and matrix; a workgroup of 4 waves covers 4 / KS columns.
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
 #include <cstdlib>
 
 #include "internal.h"
@@ -28,12 +35,13 @@ using namespace ughip;
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 enum { MODE_MULTI = 0, MODE_GATE_UP = 1, MODE_ADD = 2 };
 
 struct FusedArgs {
   const float* x;
-  const float* w[3];
+  const void* w[3];  // [n_i, k] row-major, float or bf16 (the kernel's WT)
   float* y[3];
   int col_end[3];  // MODE_MULTI: matrix i owns the columns col_end[i-1] .. col_end[i] - 1 of the grid
   int n_cols;      // columns of the grid
@@ -49,6 +57,19 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Four consecutive matrix elements as f32.
+template <typename WT>
+__device__ __forceinline__ f32x4 load_w4(const WT* p);
+template <>
+__device__ __forceinline__ f32x4 load_w4<float>(const float* p) {
+  return *reinterpret_cast<const f32x4*>(p);
+}
+template <>
+__device__ __forceinline__ f32x4 load_w4<uint16_t>(const uint16_t* p) {
+  const u32x2 v = *reinterpret_cast<const u32x2*>(p);
+  return f32x4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u)};
+}
+
 __device__ __forceinline__ float dot4(const f32x4& w, const f32x4& x, float acc) {
   acc += w.x * x.x;
   acc += w.y * x.y;
@@ -57,15 +78,15 @@ __device__ __forceinline__ float dot4(const f32x4& w, const f32x4& x, float acc)
   return acc;
 }
 
-template <int KS, int MODE>
+template <typename WT, int KS, int MODE>
 __global__ void __launch_bounds__(256) fused_gemv(FusedArgs a) {
   __shared__ float part[4][2];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = blockIdx.x * (4 / KS) + wave / KS, ks = wave % KS;
   const bool live = col < a.n_cols;
   // which matrix and which of its rows this column is
-  const float* __restrict__ W0 = nullptr;
-  const float* __restrict__ W1 = nullptr;
+  const WT* __restrict__ W0 = nullptr;
+  const WT* __restrict__ W1 = nullptr;
   float* __restrict__ Y = nullptr;
   if (live) {
     int m = 0, first = 0;
@@ -74,8 +95,8 @@ __global__ void __launch_bounds__(256) fused_gemv(FusedArgs a) {
       if (col >= a.col_end[1]) m = 2, first = a.col_end[1];
     }
     const int row = col - first;
-    W0 = a.w[m] + (size_t)row * a.k;
-    if (MODE == MODE_GATE_UP) W1 = a.w[1] + (size_t)row * a.k;
+    W0 = static_cast<const WT*>(a.w[m]) + (size_t)row * a.k;
+    if (MODE == MODE_GATE_UP) W1 = static_cast<const WT*>(a.w[1]) + (size_t)row * a.k;
     Y = a.y[m] + row;
   }
   float acc0 = 0.f, acc1 = 0.f;
@@ -93,8 +114,8 @@ __global__ void __launch_bounds__(256) fused_gemv(FusedArgs a) {
         const int ki = k + i * stride;
         w[i] = u[i] = x[i] = zero;
         if (ki < a.k) {
-          w[i] = *reinterpret_cast<const f32x4*>(W0 + ki);
-          if (MODE == MODE_GATE_UP) u[i] = *reinterpret_cast<const f32x4*>(W1 + ki);
+          w[i] = load_w4<WT>(W0 + ki);
+          if (MODE == MODE_GATE_UP) u[i] = load_w4<WT>(W1 + ki);
           x[i] = *reinterpret_cast<const f32x4*>(X + ki);
         }
       }
@@ -134,16 +155,34 @@ __global__ void __launch_bounds__(256) fused_gemv(FusedArgs a) {
 // the workgroup normalises the row once into LDS in their shadow, then every wave multiplies.
 constexpr int RMS_SLABS = 16;
 
-template <int KS, int MODE, int SLABS>
+// FULL: the row has exactly 256 * SLABS elements, no slab needs a bounds check (the guards and
+// the zero fills behind them are most of the instructions of the general form, and at 4 cycles per
+// wave instruction these kernels are not far from being bound by them).
+template <typename WT, int KS, int MODE, int SLABS, bool FULL>
 __global__ void __launch_bounds__(256) fused_rms_gemv(FusedArgs a) {
   constexpr int NVW = SLABS / KS;  // slabs of 256 floats per wave
+  const int klen = FULL ? SLABS * 256 : a.k;
   __shared__ float part[4][2];
   __shared__ float ssum[4];
   __shared__ f32x4 xs[SLABS * 64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = blockIdx.x * (4 / KS) + wave / KS, ks = wave % KS;
   const bool live = col < a.n_cols;
-  // the matrix rows are requested first: they are the long pole, the norm below runs in their shadow
+  // Loads come back in the order they were issued.  The row and the norm weights (cache hits, thread t
+  // owns elements 4 t .. 4 t + 3 of every 1024) are requested first so that the norm below runs while
+  // the matrix rows, the long pole, are still on their way from memory.
+  const float* __restrict__ X = a.x;
+  constexpr int PER_T = SLABS / 4;
+  f32x4 xl[PER_T], al[PER_T];
+#pragma unroll
+  for (int i = 0; i < PER_T; ++i) {
+    const int k = (i * 256 + (int)threadIdx.x) * 4;
+    xl[i] = al[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (FULL || k < klen) {
+      xl[i] = *reinterpret_cast<const f32x4*>(X + k);
+      al[i] = *reinterpret_cast<const f32x4*>(a.alpha + k);
+    }
+  }
   float* __restrict__ Y = nullptr;
   f32x4 w0[NVW], w1[NVW];
 #pragma unroll
@@ -155,29 +194,23 @@ __global__ void __launch_bounds__(256) fused_rms_gemv(FusedArgs a) {
       if (col >= a.col_end[1]) mtx = 2, first = a.col_end[1];
     }
     const int row = col - first;
-    const float* __restrict__ W0 = a.w[mtx] + (size_t)row * a.k;
-    const float* __restrict__ W1 = MODE == MODE_GATE_UP ? a.w[1] + (size_t)row * a.k : nullptr;
+    const WT* __restrict__ W0 = static_cast<const WT*>(a.w[mtx]) + (size_t)row * klen;
+    const WT* __restrict__ W1 = MODE == MODE_GATE_UP ? static_cast<const WT*>(a.w[1]) + (size_t)row * klen : nullptr;
     Y = a.y[mtx] + row;
 #pragma unroll
     for (int j = 0; j < NVW; ++j) {
       const int k = ((j * KS + ks) * 64 + lane) * 4;
-      if (k < a.k) {
-        w0[j] = *reinterpret_cast<const f32x4*>(W0 + k);
-        if (MODE == MODE_GATE_UP) w1[j] = *reinterpret_cast<const f32x4*>(W1 + k);
+      if (FULL || k < klen) {
+        w0[j] = load_w4<WT>(W0 + k);
+        if (MODE == MODE_GATE_UP) w1[j] = load_w4<WT>(W1 + k);
       }
     }
   }
   __builtin_amdgcn_sched_barrier(0);
-  // the workgroup normalises the row once, into LDS: thread t owns elements 4 t .. 4 t + 3 of every 1024
-  const float* __restrict__ X = a.x;
-  constexpr int PER_T = SLABS / 4;
-  f32x4 xl[PER_T];
+  // the workgroup normalises the row once, into LDS
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < PER_T; ++i) {
-    const int k = (i * 256 + (int)threadIdx.x) * 4;
-    xl[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (k < a.k) xl[i] = *reinterpret_cast<const f32x4*>(X + k);
     ss += xl[i].x * xl[i].x;
     ss += xl[i].y * xl[i].y;
     ss += xl[i].z * xl[i].z;
@@ -187,21 +220,18 @@ __global__ void __launch_bounds__(256) fused_rms_gemv(FusedArgs a) {
   if (lane == 0) ssum[wave] = ss;
   __syncthreads();
   ss = (ssum[0] + ssum[1]) + (ssum[2] + ssum[3]);
-  const float m = sqrtf(ss * (1.f / (float)a.k) + a.eps);
+  const float inv = 1.f / sqrtf(ss * (1.f / (float)klen) + a.eps);  // one division per thread; x / m as x * (1 / m) is within an ulp
 #pragma unroll
   for (int i = 0; i < PER_T; ++i) {
     const int k = (i * 256 + (int)threadIdx.x) * 4;
-    if (k < a.k) {
-      const f32x4 al = *reinterpret_cast<const f32x4*>(a.alpha + k);
-      xs[i * 256 + threadIdx.x] = f32x4{xl[i].x / m * al.x, xl[i].y / m * al.y, xl[i].z / m * al.z, xl[i].w / m * al.w};
-    }
+    if (FULL || k < klen) xs[i * 256 + threadIdx.x] = f32x4{xl[i].x * inv * al[i].x, xl[i].y * inv * al[i].y, xl[i].z * inv * al[i].z, xl[i].w * inv * al[i].w};
   }
   __syncthreads();
   float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
   for (int j = 0; j < NVW; ++j) {
     const int k4 = (j * KS + ks) * 64 + lane;
-    if (k4 * 4 < a.k) {
+    if (FULL || k4 * 4 < klen) {
       const f32x4 xn = xs[k4];
       acc0 = dot4(w0[j], xn, acc0);
       if (MODE == MODE_GATE_UP) acc1 = dot4(w1[j], xn, acc1);
@@ -238,29 +268,55 @@ int pick_ks(size_t cols, size_t k) {
   return ks;
 }
 
-template <int MODE>
-void launch(hipStream_t st, const FusedArgs& a) {
+template <typename WT, int MODE>
+void launch_t(hipStream_t st, const FusedArgs& a) {
   const int ks = pick_ks((size_t)a.n_cols, (size_t)a.k);  // measured: gate/up (two rows per wave) also does best with the plain rule
   const unsigned per_wg = 4 / ks;
   const unsigned grid = ((unsigned)a.n_cols + per_wg - 1) / per_wg;
   if (a.alpha) {
     if (MODE == MODE_ADD) return;  // not built (the residual projections read attention / SwiGLU outputs, not a norm)
     constexpr int M = MODE == MODE_ADD ? MODE_MULTI : MODE;
-    const bool small = a.k <= 256 * 8;
-    if (ks == 4) small ? fused_rms_gemv<4, M, 8><<<grid, 256, 0, st>>>(a) : fused_rms_gemv<4, M, 16><<<grid, 256, 0, st>>>(a);
-    else if (ks == 2) small ? fused_rms_gemv<2, M, 8><<<grid, 256, 0, st>>>(a) : fused_rms_gemv<2, M, 16><<<grid, 256, 0, st>>>(a);
-    else small ? fused_rms_gemv<1, M, 8><<<grid, 256, 0, st>>>(a) : fused_rms_gemv<1, M, 16><<<grid, 256, 0, st>>>(a);
+    const bool small = a.k <= 256 * 8, full = a.k == 256 * 8 || a.k == 256 * 16;
+#define UGHIP_RMS_GO(KS_)                                                                             \
+  do {                                                                                                \
+    if (small && full) fused_rms_gemv<WT, KS_, M, 8, true><<<grid, 256, 0, st>>>(a);                  \
+    else if (small) fused_rms_gemv<WT, KS_, M, 8, false><<<grid, 256, 0, st>>>(a);                    \
+    else if (full) fused_rms_gemv<WT, KS_, M, 16, true><<<grid, 256, 0, st>>>(a);                     \
+    else fused_rms_gemv<WT, KS_, M, 16, false><<<grid, 256, 0, st>>>(a);                              \
+  } while (0)
+    if (ks == 4) UGHIP_RMS_GO(4);
+    else if (ks == 2) UGHIP_RMS_GO(2);
+    else UGHIP_RMS_GO(1);
+#undef UGHIP_RMS_GO
     return;
   }
-  if (ks == 4) fused_gemv<4, MODE><<<grid, 256, 0, st>>>(a);
-  else if (ks == 2) fused_gemv<2, MODE><<<grid, 256, 0, st>>>(a);
-  else fused_gemv<1, MODE><<<grid, 256, 0, st>>>(a);
+  if (ks == 4) fused_gemv<WT, 4, MODE><<<grid, 256, 0, st>>>(a);
+  else if (ks == 2) fused_gemv<WT, 2, MODE><<<grid, 256, 0, st>>>(a);
+  else fused_gemv<WT, 1, MODE><<<grid, 256, 0, st>>>(a);
+}
+
+template <int MODE>
+void launch(hipStream_t st, const FusedArgs& a, int w_dtype) {
+  if (w_dtype == UGHIP_BF16) launch_t<uint16_t, MODE>(st, a);
+  else launch_t<float, MODE>(st, a);
 }
 
 int check(const ughip_device* dev, const ughip_slice* s, size_t need, const char* what) {
   if (!s) return set_error(UGHIP_ERR_INVALID, "%s: null slice", what);
   if (s->dev != dev) return set_error(UGHIP_ERR_INVALID, "%s: slice lives on another device", what);
   if (s->dtype != UGHIP_F32) return set_error(UGHIP_ERR_UNSUPPORTED, "%s: dtype %s, this entry point is built for F32", what, dtype_name(s->dtype));
+  if (s->len < need) return set_error(UGHIP_ERR_BOUNDS, "%s: slice has %zu elements, op needs %zu", what, s->len, need);
+  return UGHIP_OK;
+}
+
+// A matrix: F32 or BF16, and every matrix of a call like the first (*dtype < 0: not seen yet).
+int check_w(const ughip_device* dev, const ughip_slice* s, size_t need, int* dtype, const char* what) {
+  if (!s) return set_error(UGHIP_ERR_INVALID, "%s: null slice", what);
+  if (s->dev != dev) return set_error(UGHIP_ERR_INVALID, "%s: slice lives on another device", what);
+  if (s->dtype != UGHIP_F32 && s->dtype != UGHIP_BF16)
+    return set_error(UGHIP_ERR_UNSUPPORTED, "%s: dtype %s, matrices are taken as F32 or BF16", what, dtype_name(s->dtype));
+  if (*dtype >= 0 && s->dtype != *dtype) return set_error(UGHIP_ERR_INVALID, "%s: the matrices of one call must share a dtype", what);
+  *dtype = s->dtype;
   if (s->len < need) return set_error(UGHIP_ERR_BOUNDS, "%s: slice has %zu elements, op needs %zu", what, s->len, need);
   return UGHIP_OK;
 }
@@ -306,11 +362,12 @@ int ughip_rms_gemv_multi(ughip_device* dev, const ughip_slice* x, const ughip_sl
   a.alpha = alpha ? static_cast<const float*>(alpha->ptr) : nullptr;
   a.eps = eps;
   size_t first = 0;
+  int wdt = -1;
   for (size_t i = 0; i < 3; ++i) {
     if (i < n_mats) {
-      if (int rc = check(dev, w[i], n[i] * k, "gemv_multi w")) return rc;
+      if (int rc = check_w(dev, w[i], n[i] * k, &wdt, "gemv_multi w")) return rc;
       if (dst == w[i]) return set_error(UGHIP_ERR_INVALID, "gemv_multi: dst aliases a matrix");
-      a.w[i] = static_cast<const float*>(w[i]->ptr);
+      a.w[i] = w[i]->ptr;
       a.y[i] = static_cast<float*>(dst->ptr) + first;
       first += n[i];
     }
@@ -319,7 +376,7 @@ int ughip_rms_gemv_multi(ughip_device* dev, const ughip_slice* x, const ughip_sl
   a.n_cols = (int)total;
   if (total == 0) return UGHIP_OK;
   if (int rc = device_activate(dev)) return rc;
-  launch<MODE_MULTI>(dev->stream, a);
+  launch<MODE_MULTI>(dev->stream, a, wdt);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
 }
@@ -335,22 +392,23 @@ int ughip_rms_gemv_gate_up(ughip_device* dev, const ughip_slice* x, const ughip_
   if (int rc = check_k(k, "gemv_gate_up")) return rc;
   if (n > 0x7fffffffull / 4) return set_error(UGHIP_ERR_INVALID, "gemv_gate_up: too many columns");
   if (int rc = check(dev, x, k, "gemv_gate_up x")) return rc;
-  if (int rc = check(dev, w_gate, n * k, "gemv_gate_up gate")) return rc;
-  if (int rc = check(dev, w_up, n * k, "gemv_gate_up up")) return rc;
+  int wdt = -1;
+  if (int rc = check_w(dev, w_gate, n * k, &wdt, "gemv_gate_up gate")) return rc;
+  if (int rc = check_w(dev, w_up, n * k, &wdt, "gemv_gate_up up")) return rc;
   if (int rc = check(dev, dst, n, "gemv_gate_up dst")) return rc;
   if (dst == x || dst == w_gate || dst == w_up) return set_error(UGHIP_ERR_INVALID, "gemv_gate_up: dst aliases an input");
   if (n == 0) return UGHIP_OK;
   FusedArgs a{};
   a.x = static_cast<const float*>(x->ptr);
-  a.w[0] = static_cast<const float*>(w_gate->ptr);
-  a.w[1] = static_cast<const float*>(w_up->ptr);
+  a.w[0] = w_gate->ptr;
+  a.w[1] = w_up->ptr;
   a.alpha = alpha ? static_cast<const float*>(alpha->ptr) : nullptr;
   a.eps = eps;
   a.y[0] = static_cast<float*>(dst->ptr);
   a.col_end[0] = a.col_end[1] = a.col_end[2] = a.n_cols = (int)n;
   a.k = (int)k;
   if (int rc = device_activate(dev)) return rc;
-  launch<MODE_GATE_UP>(dev->stream, a);
+  launch<MODE_GATE_UP>(dev->stream, a, wdt);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
 }
@@ -360,20 +418,21 @@ int ughip_gemv_add(ughip_device* dev, const ughip_slice* x, const ughip_slice* w
   if (int rc = check_k(k, "gemv_add")) return rc;
   if (n > 0x7fffffffull / 4) return set_error(UGHIP_ERR_INVALID, "gemv_add: too many columns");
   if (int rc = check(dev, x, k, "gemv_add x")) return rc;
-  if (int rc = check(dev, w, n * k, "gemv_add w")) return rc;
+  int wdt = -1;
+  if (int rc = check_w(dev, w, n * k, &wdt, "gemv_add w")) return rc;
   if (int rc = check(dev, residual, n, "gemv_add residual")) return rc;
   if (int rc = check(dev, dst, n, "gemv_add dst")) return rc;
   if (dst == x || dst == w || dst == residual) return set_error(UGHIP_ERR_INVALID, "gemv_add: dst aliases an input");
   if (n == 0) return UGHIP_OK;
   FusedArgs a{};
   a.x = static_cast<const float*>(x->ptr);
-  a.w[0] = static_cast<const float*>(w->ptr);
+  a.w[0] = w->ptr;
   a.y[0] = static_cast<float*>(dst->ptr);
   a.col_end[0] = a.col_end[1] = a.col_end[2] = a.n_cols = (int)n;
   a.k = (int)k;
   a.residual = static_cast<const float*>(residual->ptr);
   if (int rc = device_activate(dev)) return rc;
-  launch<MODE_ADD>(dev->stream, a);
+  launch<MODE_ADD>(dev->stream, a, wdt);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
 }
