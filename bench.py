@@ -139,6 +139,27 @@ def cpu_extras(budget_s=4.0):
     n, el = sample(cs.run)
     out["cpu_bmm_f32_8x1024^3"] = {"TFLOP/s": round(2.0 * b * m * m * m * n / el / 1e12, 4), "ms": round(el / n * 1e3, 1), "cores": int(os.environ["RAYON_NUM_THREADS"]), "kind": "port",
                                    "sample": f"{n} runs in {el:.1f} s; the reference multiplies with the gemm crate, the oracle with its own blocked loops"}
+    # config 5 at full width, two of the 22 layers: a decode step is the same two layers 11 times over
+    # plus the head, so the per-layer and the head time are fitted from a 1-layer and a 2-layer run
+    prompt = rng.token_ids(10, 8, 32000)
+    oh = C.c_void_p()
+    assert lib.ugo_llama_ops_cpu(C.byref(oh)) == 0
+    cpu_ops = ug_amd.LlamaOps(oh.value)
+    n_steps = 6
+    per_tok = {}
+    for layers in (1, 2):
+        cfg = ug_amd.LlamaConfig(num_hidden_layers=layers)
+        model = ug_amd.LlamaModel(cpu, cpu_ops, cfg, custom_softmax=True, seed=9, std=0.02)
+        model.generate(prompt, 1)     # compiles (gcc) every kernel once
+        _, st = model.generate(prompt, n_steps)
+        per_tok[layers] = st["decode_ms"] / n_steps
+        del model
+    layer_ms = per_tok[2] - per_tok[1]
+    full_ms = per_tok[1] + 21 * layer_ms
+    out["cpu_llama_decode_f32"] = {"tok/s": round(1e3 / full_ms, 3), "decode_ms_per_token": round(full_ms, 1), "ms_per_layer": round(layer_ms, 2),
+                                   "ms_1_layer_model": round(per_tok[1], 2), "ms_2_layer_model": round(per_tok[2], 2), "cores": int(os.environ["RAYON_NUM_THREADS"]),
+                                   "kind": "port", "sample": f"{n_steps} decode steps each of a 1-layer and a 2-layer model of config 5's width after an 8-token prompt; "
+                                   "22 layers = the 1-layer step + 21 x the difference (the fused kernels run on one thread as in the reference, the matmuls on all)"}
     return out
 
 
