@@ -136,7 +136,7 @@ def lb_set(dev):
 ALL = [lb_add, lb_mm, lb_cat, schedule_one_item, lb_copy, schedule_broadcast, lb_custom, lb_layout, lb_custom_in_place, lb_set]
 
 
-# ---- the BASELINE configs as lazy graphs ---------------------------------------------------------------
+# ---- the benchmark workloads as lazy graphs ---------------------------------------------------------------
 def softmax_graph(src):
     """ug-llama/src/model.rs:94-101 == config 1: max-reduce, subtract, exp, sum-reduce, divide."""
     return ug_amd.llama.softmax(src)

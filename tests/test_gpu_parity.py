@@ -124,7 +124,7 @@ def test_scheduler_grid_ssa_reduce_local(hip, oracle, cols):
     np.testing.assert_allclose(out.reshape(rows, cols), np.exp(x.astype(np.float64) - x[:, :1]) / cols, rtol=2e-6)
 
 
-# ---- BASELINE configs 1 and 2 at full size ----------------------------------------------------------------------
+# ---- row softmax [32,1024] and the 2^24-element fused reduce at full size ----------------------------------------------------------------------
 def test_config1_softmax_32x1024(hip, cpu):
     x = (rng.normal(1, 32 * 1024) * np.float32(3.0)).reshape(32, 1024)
     got = ug_amd.llama.softmax(LB.copy(x, (32, 1024), hip)).data_vec().reshape(32, 1024)
@@ -564,7 +564,7 @@ def test_small_llama_greedy_ids_match_cpu(hip, cpu, hip_ops, cpu_ops, custom_sof
 
 @pytest.mark.parametrize("round_bf16", [False, True])
 def test_llama_config5_width_greedy_ids_match_cpu(hip, cpu, hip_ops, cpu_ops, round_bf16):
-    """BASELINE config 5 at full width (hidden 2048, 32/4 heads, FFN 5632, vocab 32000, N(0,0.02)
+    """The TinyLlama-1.1B shape at full width (hidden 2048, 32/4 heads, FFN 5632, vocab 32000, N(0,0.02)
     weights, seed 9) but 2 layers and a short run, so the CPU oracle finishes in seconds; weights
     f32 or bf16-rounded (what the reference's load_with_cast(F32) makes of a bf16 checkpoint)."""
     cfg = ug_amd.LlamaConfig(num_hidden_layers=2, max_position_embeddings=256)

@@ -74,7 +74,7 @@ class SsaWire(C.Structure):
 
 
 class LlamaConfig(C.Structure):
-    """ug-llama/src/model.rs:10-24; defaults are BASELINE config 5."""
+    """ug-llama/src/model.rs:10-24; defaults are the TinyLlama-1.1B shape."""
     _fields_ = [("hidden_size", C.c_size_t), ("intermediate_size", C.c_size_t), ("max_position_embeddings", C.c_size_t),
                 ("num_attention_heads", C.c_size_t), ("num_key_value_heads", C.c_size_t), ("num_hidden_layers", C.c_size_t),
                 ("rms_norm_eps", C.c_double), ("rope_interleaved", C.c_int), ("rope_theta", C.c_float), ("vocab_size", C.c_size_t)]

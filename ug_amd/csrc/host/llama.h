@@ -195,7 +195,7 @@ class Model {
   std::vector<Layer> layers_;
 };
 
-// The harness of BASELINE config 5: one prefill call over `prompt`, then `n_steps` greedy
+// The greedy-decode harness (the loop of ug-llama/src/main.rs:118-170): one prefill call over `prompt`, then `n_steps` greedy
 // (argmax) single-token steps with the KV cache.  Returns the generated ids; timings in ms.
 struct GenerateStats {
   double prefill_ms = 0, decode_ms = 0;
