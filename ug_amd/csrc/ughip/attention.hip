@@ -15,21 +15,12 @@
 
 #include "internal.h"
 #include "ughip.h"
+#include "wave_ops.h"
 
 using namespace ughip;
 
 namespace {
 
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
-}
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
 
 // All threads of a 256-thread workgroup get the max / the sum of v.
 template <bool IS_MAX>
@@ -213,7 +204,15 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       float pu = p[u];
-      for (int o = lpk >> 1; o > 0; o >>= 1) pu += __shfl_xor(pu, o, 64);  // lpk is a power of two <= 64: stays inside the key's lanes
+      // sum over the lpk lanes of this key (a power of two <= 64); from 16 lanes up the last four
+      // steps are rotations within rows of 16
+      if (lpk >= 16) {
+        if (lpk > 32) pu += __shfl_xor(pu, 32, 64);
+        if (lpk > 16) pu += __shfl_xor(pu, 16, 64);
+        pu = row_sum16(pu);
+      } else {
+        for (int o = lpk >> 1; o > 0; o >>= 1) pu += __shfl_xor(pu, o, 64);
+      }
       pu *= scale;
       const int j = j0 + u * kpb + slot;
       if (j < s) {

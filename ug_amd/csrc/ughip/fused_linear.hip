@@ -29,6 +29,7 @@
 
 #include "internal.h"
 #include "ughip.h"
+#include "wave_ops.h"
 
 using namespace ughip;
 
@@ -50,21 +51,6 @@ struct FusedArgs {
   const float* alpha;  // RMS variants: y uses x / sqrt(mean(x^2) + eps) * alpha in place of x
   float eps;
 };
-
-// Butterfly sum over the 64 lanes, partners at distance 32, 16, 8, 4, 2, 1 in that order (the order
-// ughip_matmul's row-vector kernel uses, so sums agree to the bit).  After the step at distance d
-// lanes that differ in bit d hold the same value, which lets the last four steps use a rotation
-// within rows of 16 lanes (a register-to-register DPP move) in place of an exchange through LDS:
-// lane i + d mod 16 differs from lane i ^ d only in bits already summed over.
-__device__ __forceinline__ float wave_sum(float v) {
-  v += __shfl_xor(v, 32, 64);
-  v += __shfl_xor(v, 16, 64);
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));  // row_ror:8
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xf, 0xf, false));  // row_ror:4
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xf, 0xf, false));  // row_ror:2
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xf, 0xf, false));  // row_ror:1
-  return v;
-}
 
 // Four consecutive matrix elements as f32.
 template <typename WT>

@@ -6,21 +6,12 @@
 
 #include "internal.h"
 #include "ughip.h"
+#include "wave_ops.h"
 
 using namespace ughip;
 
 namespace {
 
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
-}
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
 
 // Reduction across the NW waves of a workgroup through LDS; every thread gets the result.
 template <int NW, bool IS_MAX>

@@ -11,6 +11,7 @@
 #include "gemm.h"
 #include "internal.h"
 #include "ughip.h"
+#include "wave_ops.h"
 
 using namespace ughip;
 
@@ -136,11 +137,6 @@ __global__ void __launch_bounds__(256) gemm_half_any(MMArgs p) {
 // ---- GEMV kernels for the m <= 8 rows of decode ---------------------------------------------------
 // All of them stream the big operand from HBM exactly once with 128-bit loads (x comes from L2),
 // accumulate in f32 and reduce in a fixed order, so results do not change from run to run.
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
 
 template <typename T>
 struct Vec;
