@@ -231,7 +231,7 @@ int ughip_causal_softmax_rows(ughip_device* dev, const ughip_slice* src, ughip_s
                               size_t bh, size_t s1, size_t s2);
 /* Attention of one query position, f32: q [b, n_heads, d], k and v [b, n_kv_heads, s, d]
  * (query head h reads kv head h / (n_heads / n_kv_heads), i.e. model.rs:80-92's repeat),
- * dst [b, n_heads, d] = softmax(q k^T * scale) v.  d a power of two in 16..256, s <= 12000. */
+ * dst [b, n_heads, d] = softmax(q k^T * scale) v.  d a power of two in 16..256. */
 int ughip_attention_decode(ughip_device* dev, const ughip_slice* q, const ughip_slice* k,
                            const ughip_slice* v, ughip_slice* dst, size_t b, size_t n_heads,
                            size_t n_kv_heads, size_t s, size_t d, float scale);
@@ -283,7 +283,7 @@ int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_off
 /* One decode position in one launch: ughip_kv_append of the k and v parts of a packed q|k|v row
  * (qkv [b, row_stride], parts at q_offset / k_offset / v_offset) into row s_old of both caches,
  * and ughip_attention_cached of the q part over rows 0 .. s_old.  The caches are read and
- * written; dst [b, n_heads * d].  d a power of two in 16..256, s_old + 1 <= min(cap, 12000). */
+ * written; dst [b, n_heads * d].  d a power of two in 16..256, s_old + 1 <= cap. */
 int ughip_attention_step(ughip_device* dev, const ughip_slice* qkv, size_t row_stride,
                          size_t q_offset, size_t k_offset, size_t v_offset, ughip_slice* kcache,
                          ughip_slice* vcache, ughip_slice* dst, size_t b, size_t n_heads,

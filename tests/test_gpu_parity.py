@@ -601,7 +601,7 @@ def test_causal_softmax_fused(hip, cpu, hip_ops, cpu_ops, shape):
 
 
 @pytest.mark.parametrize("b,nh,nkv,s,d", [(1, 32, 4, 1, 64), (1, 32, 4, 5, 64), (1, 32, 4, 129, 64), (2, 8, 2, 700, 64), (1, 8, 8, 33, 128), (3, 4, 1, 17, 16),
-                                          (1, 2, 1, 2100, 256), (1, 32, 4, 2047, 64)])
+                                          (1, 2, 1, 2100, 256), (1, 32, 4, 2047, 64), (1, 4, 2, 13001, 64), (1, 2, 2, 300, 32)])
 def test_attention_decode_fused(hip, cpu, hip_ops, cpu_ops, b, nh, nkv, s, d):
     print("attention decode", (b, nh, nkv, s, d), flush=True)
     q = rng.normal(62, b * nh * d)

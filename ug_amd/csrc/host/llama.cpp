@@ -208,7 +208,7 @@ struct HipOps : Ops {
                                                                                               : q.dims()[2] % d != 0 || (n_heads != 0 && n_heads * d != q.dims()[2])))
       bail("attention_cached: mismatched shapes " + q.shape().str() + " " + k.shape().str() + " with " + std::to_string(s) + " keys");
     size_t nh = packed ? n_heads : q.dims()[2] / d;
-    const bool one = t == 1 && d >= 16 && d <= 256 && (d & (d - 1)) == 0 && s <= 12000;
+    const bool one = t == 1 && d >= 16 && d <= 256 && (d & (d - 1)) == 0;
     const bool many = t > 1 && (d == 32 || d == 64 || d == 128);
     if (!one && !many) return Ops::attention_cached(q, k, v, s, scale, cos, sin, pos, interleaved, q_offset, q_row_stride, n_heads);
     ughip_device* dev = hip_dev(q);
@@ -667,7 +667,7 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
     LB qkv = ops_->linear_packed(xs_in, {l.q_proj, l.k_proj, l.v_proj}, norm_first ? &l.rms1 : nullptr, eps);
     cache.len = len + 1;
     const float scale = std::pow((float)hd, -0.5f);
-    if (hd >= 16 && hd <= 256 && (hd & (hd - 1)) == 0 && cache.len <= 12000)
+    if (hd >= 16 && hd <= 256 && (hd & (hd - 1)) == 0)
       return finish(ops_->attention_step(qkv, cache.prev_k, cache.prev_v, len, nh, scale, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved));
     LB kc = ops_->kv_append(cache.prev_k, len, qkv, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, nq, row);
     LB vc = ops_->kv_append(cache.prev_v, len, qkv, nullptr, nullptr, nullptr, false, nq + nk, row);

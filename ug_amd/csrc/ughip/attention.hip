@@ -93,25 +93,14 @@ __global__ void __launch_bounds__(256) causal_softmax_generic(const float* __res
 // One workgroup of 1024 threads per query head.  q: [b, nh, d]; k, v: [b, nkv, s, d] (heads
 // kv_head_stride elements apart: s * d, or capacity * d for a preallocated cache); dst: [b, nh, d].
 // LPK = d / 4 lanes share one key row (one 128-bit load each, a row is one contiguous 4*d bytes);
-// 1024 / LPK keys are in flight per step and four steps per loop trip, because at batch 1 this
-// kernel is a chain of L2 round trips, not a bandwidth problem.  Scores and probabilities live in
-// LDS (s floats).
+// 1024 / LPK keys are in flight per step and four steps per loop trip, keys and values together,
+// because at batch 1 this kernel is a chain of memory round trips and barriers, not a bandwidth
+// problem: softmax runs in one pass with a running maximum per wave, and the only workgroup-wide
+// exchange is the merge of the 16 waves at the end.
 // With a rope table (cos_t != nullptr) q is rotated first, at table row pos[0] (rope: pairs
 // (i, i + d/2); rope_i: pairs (2i, 2i + 1); cpu_ops.rs:58-126 for t = 1).
 constexpr int ATT_THREADS = 1024, ATT_WAVES = ATT_THREADS / 64;
 typedef float att_f32x4 __attribute__((ext_vector_type(4)));
-
-template <bool IS_MAX>
-__device__ __forceinline__ float att_block_reduce(float v, float* lds16) {
-  v = IS_MAX ? wave_max(v) : wave_sum(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) lds16[threadIdx.x >> 6] = v;
-  __syncthreads();
-  float r = lds16[0];
-#pragma unroll
-  for (int i = 1; i < ATT_WAVES; ++i) r = IS_MAX ? fmaxf(r, lds16[i]) : r + lds16[i];
-  return r;
-}
 
 __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
                                                                        float* __restrict__ dst, int nh, int nkv, int s, size_t kv_head_stride,
@@ -119,8 +108,8 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
                                                                        const int* __restrict__ pos, size_t table_len, int interleaved,
                                                                        const float* __restrict__ k_new, const float* __restrict__ v_new, float* __restrict__ k_out,
                                                                        float* __restrict__ v_out) {
-  extern __shared__ __attribute__((aligned(16))) float sc[];  // s scores, then ATT_WAVES * 64 float4 of reduction space
-  __shared__ float lds16[ATT_WAVES];
+  __shared__ __attribute__((aligned(16))) float sc[ATT_WAVES * 64 * 4];  // one float4 per lane slot of every wave for the final merge
+  __shared__ float wave_m[ATT_WAVES], wave_l[ATT_WAVES];
   __shared__ __attribute__((aligned(16))) float qs[256];
   __shared__ __attribute__((aligned(16))) float kn[256];
   __shared__ __attribute__((aligned(16))) float vn[256];
@@ -183,8 +172,12 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
     if (tid < lpk) reinterpret_cast<float4*>(k_out)[row + tid] = reinterpret_cast<const float4*>(kn)[tid];
     else reinterpret_cast<float4*>(v_out)[row + tid - lpk] = reinterpret_cast<const float4*>(vn)[tid - lpk];
   }
-  // scores = (q . k_j) * scale, four key rows per lane group in flight
-  float m = -INFINITY;
+  // One pass over the keys, four key rows and four value rows per lane group in flight.  Every wave
+  // keeps a running maximum m_run, the sum l_run of exp(score - m_run) and the weighted value rows
+  // acc of the keys it has seen (rescaled when the maximum moves); the 16 waves are merged once at
+  // the end.  Scores and probabilities never leave registers.
+  float m_run = -INFINITY, l_run = 0.f;
+  att_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   auto load_rows = [&](const float4* base, int j0, att_f32x4 (&r)[4]) {
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -193,7 +186,7 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
       r[u] = reinterpret_cast<const att_f32x4*>(base)[jj * lpk + c4];
     }
   };
-  auto score_trip = [&](int j0, const att_f32x4 (&kr)[4]) {
+  auto trip = [&](int j0, const att_f32x4 (&kr)[4], const att_f32x4 (&vr)[4]) {
     float p[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -201,6 +194,7 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
       const att_f32x4 kv = j == j_new ? reinterpret_cast<const att_f32x4*>(kn)[c4] : kr[u];
       p[u] = (qv.x * kv.x + qv.y * kv.y) + (qv.z * kv.z + qv.w * kv.w);
     }
+    float mt = -INFINITY;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       float pu = p[u];
@@ -213,70 +207,60 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
       } else {
         for (int o = lpk >> 1; o > 0; o >>= 1) pu += __shfl_xor(pu, o, 64);
       }
-      pu *= scale;
-      const int j = j0 + u * kpb + slot;
-      if (j < s) {
-        if (c4 == 0) sc[j] = pu;
-        m = fmaxf(m, pu);
-      }
+      p[u] = j0 + u * kpb + slot < s ? pu * scale : -INFINITY;
+      mt = fmaxf(mt, p[u]);
     }
-  };
-  score_trip(0, kpre);
-  for (int j0 = 4 * kpb; j0 < s; j0 += 4 * kpb) {
-    att_f32x4 kr[4];
-    load_rows(k4, j0, kr);
-    score_trip(j0, kr);
-  }
-  m = att_block_reduce<true>(m, lds16);  // the barriers inside also publish sc[]
-  float sum = 0.f;
-  for (int j = tid; j < s; j += ATT_THREADS) {
-    const float e = expf(sc[j] - m);
-    sc[j] = e;
-    sum += e;
-  }
-  sum = att_block_reduce<false>(sum, lds16);
-
-  // out = sum_j p_j v_j / sum: slot walks the keys, c4 owns 4 output columns
-  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  auto value_trip = [&](int j0, const att_f32x4 (&vr)[4]) {
+    const float m_new = fmaxf(m_run, wave_max(mt));
+    if (m_new == -INFINITY) return;  // this wave has not seen a key yet (wave-uniform)
+    const float alpha = expf(m_run - m_new);  // 0 on the wave's first keys (m_run = -inf)
+    acc *= alpha;
+    float lt = 0.f;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int j = j0 + u * kpb + slot;
-      const float pj = j < s ? sc[j] : 0.f;
+      const float e = expf(p[u] - m_new);  // 0 for the keys past the end
       const att_f32x4 vv = j == j_new ? reinterpret_cast<const att_f32x4*>(vn)[c4] : vr[u];
-      acc.x += pj * vv.x;
-      acc.y += pj * vv.y;
-      acc.z += pj * vv.z;
-      acc.w += pj * vv.w;
+      acc += e * vv;
+      if (c4 == 0) lt += e;  // a key's lanes all hold its e: count it once
     }
+    l_run = l_run * alpha + wave_sum(lt);
+    m_run = m_new;
   };
-  value_trip(0, vpre);
+  trip(0, kpre, vpre);
   for (int j0 = 4 * kpb; j0 < s; j0 += 4 * kpb) {
-    att_f32x4 vr[4];
+    att_f32x4 kr[4], vr[4];
+    load_rows(k4, j0, kr);
     load_rows(v4, j0, vr);
-    value_trip(j0, vr);
+    trip(j0, kr, vr);
   }
-  // the slots of one wave (lanes lpk apart), then the waves in order
+  // the slots of one wave (lanes lpk apart) ...
   for (int o = lpk; o < 64; o <<= 1) {
     acc.x += __shfl_xor(acc.x, o, 64);
     acc.y += __shfl_xor(acc.y, o, 64);
     acc.z += __shfl_xor(acc.z, o, 64);
     acc.w += __shfl_xor(acc.w, o, 64);
   }
-  float4* red = reinterpret_cast<float4*>(sc + s + ((4 - (s & 3)) & 3));  // 16-byte aligned space after the scores
+  // ... then the waves in order, each weighted by exp(its maximum - the overall one)
+  att_f32x4* red = reinterpret_cast<att_f32x4*>(sc);
   const int lane = tid & 63, wave = tid >> 6;
   if (lane < lpk) red[wave * 64 + lane] = acc;
+  if (lane == 0) {
+    wave_m[wave] = m_run;
+    wave_l[wave] = l_run;
+  }
   __syncthreads();
   if (tid < lpk) {
-    float4 o = red[tid];
-    for (int w = 1; w < ATT_WAVES; ++w) {
-      const float4 t = red[w * 64 + tid];
-      o.x += t.x;
-      o.y += t.y;
-      o.z += t.z;
-      o.w += t.w;
+    float mx = wave_m[0];  // key 0 belongs to wave 0: finite unless the data is not
+#pragma unroll
+    for (int w = 1; w < ATT_WAVES; ++w) mx = fmaxf(mx, wave_m[w]);
+    att_f32x4 o = {0.f, 0.f, 0.f, 0.f};
+    float sum = 0.f;
+    for (int w = 0; w < ATT_WAVES; ++w) {
+      const float f = expf(wave_m[w] - mx);  // 0 for a wave without keys
+      o += f * red[w * 64 + tid];
+      sum += f * wave_l[w];
     }
-    reinterpret_cast<float4*>(dst + (size_t)bh * d)[tid] = make_float4(o.x / sum, o.y / sum, o.z / sum, o.w / sum);
+    reinterpret_cast<att_f32x4*>(dst + (size_t)bh * d)[tid] = o / sum;
   }
 }
 
@@ -693,7 +677,7 @@ int attention_decode_launch(ughip_device* dev, const ughip_slice* q, size_t q_of
   if (d < 16 || d > 256 || (d & (d - 1)) != 0) return set_error(UGHIP_ERR_INVALID, "attention_decode: head size %zu is not a power of two in 16..256", d);
   if (s == 0) return set_error(UGHIP_ERR_INVALID, "attention_decode: empty key sequence");
   if (s > cap) return set_error(UGHIP_ERR_INVALID, "attention_decode: %zu keys exceed the cache capacity %zu", s, cap);
-  if (s > 12000) return set_error(UGHIP_ERR_INVALID, "attention_decode: %zu keys exceed the 12000 this kernel holds in LDS", s);
+  if (s > 0x7fffffffull / 4) return set_error(UGHIP_ERR_INVALID, "attention_decode: too many keys");
   if (q_row_stride == 0) q_row_stride = n_heads * d;
   if (q_row_stride < n_heads * d || (q_offset | q_row_stride) % 4 != 0)
     return set_error(UGHIP_ERR_INVALID, "attention_decode: q offset %zu / row stride %zu do not fit rows of %zu", q_offset, q_row_stride, n_heads * d);
@@ -705,8 +689,7 @@ int attention_decode_launch(ughip_device* dev, const ughip_slice* q, size_t q_of
   if (b * n_heads == 0) return UGHIP_OK;
   if (b * n_heads > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "attention_decode: too many heads");
   if (int rc = device_activate(dev)) return rc;
-  const size_t lds = (s + 3 + ATT_WAVES * 64 * 4) * sizeof(float);  // scores, alignment slack, one float4 per lane slot of every wave
-  attention_decode_kernel<<<(unsigned)(b * n_heads), ATT_THREADS, lds, dev->stream>>>(
+  attention_decode_kernel<<<(unsigned)(b * n_heads), ATT_THREADS, 0, dev->stream>>>(
       static_cast<const float*>(q->ptr) + q_offset, static_cast<const float*>(k->ptr), static_cast<const float*>(v->ptr), static_cast<float*>(dst->ptr),
       (int)n_heads, (int)n_kv_heads, (int)s, cap * d, q_row_stride, (int)d, scale, rope ? static_cast<const float*>(cos->ptr) : nullptr,
       rope ? static_cast<const float*>(sin->ptr) : nullptr, rope ? static_cast<const int*>(pos->ptr) : nullptr,
@@ -728,7 +711,7 @@ int ughip_attention_step(ughip_device* dev, const ughip_slice* qkv, size_t row_s
   if (d < 16 || d > 256 || (d & (d - 1)) != 0) return set_error(UGHIP_ERR_INVALID, "attention_step: head size %zu is not a power of two in 16..256", d);
   const size_t s = s_old + 1;
   if (s > cap) return set_error(UGHIP_ERR_BOUNDS, "attention_step: position %zu does not fit a cache of %zu rows", s_old, cap);
-  if (s > 12000) return set_error(UGHIP_ERR_INVALID, "attention_step: %zu keys exceed the 12000 this kernel holds in LDS", s);
+  if (s > 0x7fffffffull / 4) return set_error(UGHIP_ERR_INVALID, "attention_step: too many keys");
   const size_t nq = n_heads * d, nk = n_kv_heads * d;
   if (row_stride % 4 != 0 || (q_offset | k_offset | v_offset) % 4 != 0 || q_offset + nq > row_stride || k_offset + nk > row_stride || v_offset + nk > row_stride)
     return set_error(UGHIP_ERR_INVALID, "attention_step: q/k/v at %zu/%zu/%zu do not fit rows of %zu", q_offset, k_offset, v_offset, row_stride);
@@ -741,9 +724,8 @@ int ughip_attention_step(ughip_device* dev, const ughip_slice* qkv, size_t row_s
   if (b * n_heads == 0) return UGHIP_OK;
   if (b * n_heads > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "attention_step: too many heads");
   if (int rc = device_activate(dev)) return rc;
-  const size_t lds = (s + 3 + ATT_WAVES * 64 * 4) * sizeof(float);
   const float* base = static_cast<const float*>(qkv->ptr);
-  attention_decode_kernel<<<(unsigned)(b * n_heads), ATT_THREADS, lds, dev->stream>>>(
+  attention_decode_kernel<<<(unsigned)(b * n_heads), ATT_THREADS, 0, dev->stream>>>(
       base + q_offset, static_cast<const float*>(kcache->ptr), static_cast<const float*>(vcache->ptr), static_cast<float*>(dst->ptr), (int)n_heads,
       (int)n_kv_heads, (int)s, cap * d, row_stride, (int)d, scale, rope ? static_cast<const float*>(cos->ptr) : nullptr,
       rope ? static_cast<const float*>(sin->ptr) : nullptr, rope ? static_cast<const int*>(pos->ptr) : nullptr,
