@@ -190,6 +190,22 @@ int ughip_func_get_info(const ughip_func* f, ughip_func_info* out);
 int ughip_codegen(const ughip_ssa* ssa, const char* name, char* buf, size_t buf_len,
                   size_t* out_len, ughip_func_info* info);
 
+/* The same kernel translated statement by statement, for its own launch configuration: a serial
+ * loop nest stays one thread's loop nest, as in the text ug-cuda/src/code_gen.rs:68-186 produces
+ * and ug-pyo3 hands out as `Kernel.cuda_code(name)` (ug-pyo3/src/lib.rs:396-401).  The entry point
+ * is `extern "C" __global__ void <name>(...)` with one pointer per kernel argument; `name` must be
+ * a C identifier.  Slow by construction; ughip_compile is the fast path. */
+int ughip_codegen_as_written(const ughip_ssa* ssa, const char* name, char* buf, size_t buf_len,
+                             size_t* out_len);
+/* Device::compile_cu (ug-cuda/src/runtime.rs:179-186) as ug-pyo3 exposes it
+ * (ug-pyo3/src/lib.rs:438-456): build HIP source text with hiprtc and take kernel `entry` with a
+ * fixed launch configuration.  The kernel takes n_args pointers, one per slice passed to ughip_run;
+ * arg_dtypes are checked against the slices, lengths are not (the library does not know what the
+ * source indexes), and no slice may appear twice in one call. */
+int ughip_compile_source(ughip_device* dev, const char* source, const char* entry, size_t n_args,
+                         const int* arg_dtypes, unsigned grid_dim, unsigned block_dim,
+                         unsigned shared_mem_bytes, ughip_func** out);
+
 /* hiprtc only, no device needed: does `source` build for `arch` ("gfx950")?  Lets the CPU-side
  * test-suite check that every generated kernel compiles. */
 int ughip_rtc_check(const char* source, const char* arch, size_t* code_size);

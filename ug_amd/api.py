@@ -15,6 +15,13 @@ UNARY = {"id": 0, "exp": 1, "sin": 2, "cos": 3, "neg": 4, "sqrt": 5}
 BINARY = {"add": 0, "sub": 1, "mul": 2, "div": 3, "mod": 4, "min": 5, "max": 6}
 REDUCE = {"sum": 0, "max": 1, "min": 2}
 STRATEGY = {0: "literal", 1: "elementwise", 2: "row_block", 3: "row_thread", 4: "grid_reduce"}
+# ssa::Instr discriminants and selectors on the wire (include/ughip.h, order of ug-core/src/lang.rs:690-709)
+(I_DEFINE_ACC, I_DEFINE_GLOBAL, I_DEFINE_LOCAL, I_SPECIAL, I_CONST, I_UNARY, I_BINARY, I_RANGE, I_LOAD, I_ASSIGN, I_END_RANGE, I_IF, I_END_IF,
+ I_STORE, I_BARRIER, I_REDUCE_LOCAL) = range(16)
+SPECIAL_THREAD_IDX, SPECIAL_BLOCK_IDX = 0, 1
+R_SUM, R_MAX, R_MIN = 0, 1, 2
+U_ID, U_EXP, U_SIN, U_COS, U_NEG, U_SQRT, U_CAST = range(7)
+B_ADD, B_SUB, B_MUL, B_DIV, B_MOD, B_MIN, B_MAX = range(7)
 
 
 class UgError(RuntimeError):

@@ -185,6 +185,227 @@ void ugh_ssa_set_launch(void* kernel, uint32_t grid, uint32_t block, uint32_t sh
 }
 void ugh_ssa_free(void* kernel) { delete static_cast<ssa::Kernel*>(kernel); }
 
+// ---- op-level kernels and the other pieces ug-pyo3 exposes (ug-pyo3/src/lib.rs) -------------------
+namespace {
+size_t copy_out(const std::string& s, char* buf, size_t buf_len) {
+  if (buf && buf_len) {
+    size_t n = std::min(buf_len - 1, s.size());
+    memcpy(buf, s.data(), n);
+    buf[n] = 0;
+  }
+  return s.size();
+}
+const char* unary_name(int op) {
+  static const char* n[] = {"Id", "Exp", "Sin", "Cos", "Neg", "Sqrt", "Cast"};
+  return op >= 0 && op <= UGHIP_U_CAST ? n[op] : "?";
+}
+const char* binary_name(int op) {
+  static const char* n[] = {"Add", "Sub", "Mul", "Div", "Mod", "Min", "Max"};
+  return op >= 0 && op <= UGHIP_B_MAX ? n[op] : "?";
+}
+const char* reduce_name(int op) {
+  static const char* n[] = {"Sum", "Max", "Min"};
+  return op >= 0 && op <= UGHIP_R_MIN ? n[op] : "?";
+}
+std::string a_str(const ughip_a& a) {
+  if (!a.is_const) return "Var(" + std::to_string(a.var) + ")";
+  if (is_float((DType)a.dtype)) {
+    char b[64];
+    snprintf(b, sizeof b, "%g", (double)a.f);
+    return std::string("Const(") + dtype_str((DType)a.dtype) + "(" + b + "))";
+  }
+  return std::string("Const(") + dtype_str((DType)a.dtype) + "(" + std::to_string((long long)a.i) + "))";
+}
+// One line per instruction, numbered like the reference's Debug impl (lang.rs:816-823).
+std::string ssa_str(const ssa::Kernel& k) {
+  std::string out;
+  for (size_t i = 0; i < k.instrs.size(); ++i) {
+    const ssa::Instr& in = k.instrs[i];
+    char head[16];
+    snprintf(head, sizeof head, "%03zu ", i);
+    std::string l = head;
+    const char* dt = dtype_str((DType)in.dtype);
+    switch (in.op) {
+      case UGHIP_I_DEFINE_ACC: l += "DefineAcc(" + a_str(in.a) + ")"; break;
+      case UGHIP_I_DEFINE_GLOBAL: l += "DefineGlobal { index: " + std::to_string(in.n) + ", dtype: " + dt + " }"; break;
+      case UGHIP_I_DEFINE_LOCAL: l += "DefineLocal { size: " + std::to_string(in.n) + ", dtype: " + dt + " }"; break;
+      case UGHIP_I_SPECIAL: l += in.sub == UGHIP_SPECIAL_THREAD_IDX ? "Special(ThreadIdx)" : "Special(BlockIdx)"; break;
+      case UGHIP_I_CONST: l += a_str(in.a); break;
+      case UGHIP_I_UNARY: l += std::string("Unary { op: ") + unary_name(in.sub) + ", arg: " + a_str(in.a) + ", dtype: " + dt + " }"; break;
+      case UGHIP_I_BINARY:
+        l += std::string("Binary { op: ") + binary_name(in.sub) + ", lhs: " + a_str(in.a) + ", rhs: " + a_str(in.b) + ", dtype: " + dt + " }";
+        break;
+      case UGHIP_I_RANGE:
+        l += "Range { lo: " + a_str(in.a) + ", up: " + a_str(in.b) + ", step: " + std::to_string(in.n) + ", end_idx: " + std::to_string(in.v) + " }";
+        break;
+      case UGHIP_I_LOAD: l += "Load { src: " + std::to_string(in.v) + ", offset: " + a_str(in.a) + ", dtype: " + dt + " }"; break;
+      case UGHIP_I_ASSIGN: l += "Assign { dst: " + std::to_string(in.v) + ", src: " + a_str(in.a) + " }"; break;
+      case UGHIP_I_END_RANGE: l += "EndRange { start_idx: " + std::to_string(in.v) + " }"; break;
+      case UGHIP_I_IF: l += "If { cond: " + a_str(in.a) + ", end_idx: " + std::to_string(in.v) + " }"; break;
+      case UGHIP_I_END_IF: l += "EndIf"; break;
+      case UGHIP_I_STORE:
+        l += "Store { dst: " + std::to_string(in.v) + ", offset: " + a_str(in.a) + ", value: " + a_str(in.b) + ", dtype: " + dt + " }";
+        break;
+      case UGHIP_I_BARRIER: l += "Barrier"; break;
+      case UGHIP_I_REDUCE_LOCAL: l += std::string("ReduceLocal { op: ") + reduce_name(in.sub) + ", arg: " + a_str(in.a) + ", dtype: " + dt + " }"; break;
+      default: l += "?"; break;
+    }
+    out += l + "\n";
+  }
+  return out;
+}
+std::string ast_str(const op::Ast& a) {
+  const op::AstInner& in = *a.inner;
+  switch (in.kind) {
+    case op::AstInner::Load: return "Load(arg " + std::to_string(in.load_src.v) + ", " + a.shape.str() + ")";
+    case op::AstInner::Const: {
+      ughip_a c{};
+      c.is_const = 1;
+      c.dtype = (uint8_t)in.cst.dtype;
+      c.i = in.cst.i;
+      c.f = in.cst.f;
+      return a_str(c);
+    }
+    case op::AstInner::Unary: return std::string(unary_name((int)in.unary_op)) + "(" + ast_str(in.arg) + ")";
+    case op::AstInner::Binary: return std::string(binary_name((int)in.binary_op)) + "(" + ast_str(in.arg) + ", " + ast_str(in.rhs) + ")";
+    case op::AstInner::Reduce:
+      return std::string("Reduce") + reduce_name((int)in.reduce_op) + "(" + ast_str(in.arg) + ", axis " + std::to_string(in.reduce_dim) + ")";
+    default: return "Layout(" + ast_str(in.arg) + " -> " + a.shape.str() + ")";
+  }
+}
+// ssa::Kernel::flops_mem_per_thread (lang.rs:755-811)
+void flops_mem(const ssa::Kernel& k, size_t* flops, size_t* mem) {
+  size_t fl = 0, mm = 0, mult = 1;
+  std::vector<size_t> mults;
+  auto bound = [&](const ughip_a& a, const char* what) -> int64_t {
+    if (a.is_const) {
+      if (a.dtype != UGHIP_I32 && a.dtype != UGHIP_I64) bail(std::string("range ") + what + " is not a const i32/i64");
+      return a.i;
+    }
+    const ssa::Instr& d = k.instrs.at(a.var);
+    if (d.op != UGHIP_I_CONST || (d.a.dtype != UGHIP_I32 && d.a.dtype != UGHIP_I64)) bail(std::string("range ") + what + " is not a const");
+    return d.a.i;
+  };
+  for (const ssa::Instr& in : k.instrs) {
+    switch (in.op) {
+      case UGHIP_I_LOAD:
+      case UGHIP_I_STORE: mm += mult * size_in_bytes((DType)in.dtype); break;
+      case UGHIP_I_RANGE: {
+        mults.push_back(mult);
+        int64_t lo = bound(in.a, "lo"), up = bound(in.b, "up");
+        mult *= (size_t)std::max<int64_t>(up - lo, 0) / (in.n ? in.n : 1);
+        break;
+      }
+      case UGHIP_I_END_RANGE:
+        if (mults.empty()) bail("unexpected EndRange");
+        mult = mults.back();
+        mults.pop_back();
+        break;
+      case UGHIP_I_UNARY:
+      case UGHIP_I_BINARY: fl += mult; break;
+      default: break;
+    }
+  }
+  *flops = fl;
+  *mem = mm;
+}
+}  // namespace
+
+int ugh_op_arg_new(int is_ptr, int dtype, void** out) {
+  return guard([&] {
+    Arg a = Arg::ptr((DType)dtype);
+    a.is_ptr = is_ptr != 0;
+    *out = new Arg(a);
+  });
+}
+void ugh_op_arg_free(void* a) { delete static_cast<Arg*>(a); }
+size_t ugh_op_arg_str(void* a, char* buf, size_t buf_len) {
+  const Arg& x = *static_cast<Arg*>(a);
+  return copy_out(std::string("Arg { id: ") + std::to_string(x.id.v) + ", type_: " + (x.is_ptr ? "Ptr(" : "Value(") + dtype_str(x.dtype) + ") }", buf, buf_len);
+}
+void ugh_op_ast_free(void* a) { delete static_cast<op::Ast*>(a); }
+// ug-pyo3/src/lib.rs:205-214
+int ugh_op_load(void* arg, const size_t* dims, size_t rank, void** out) {
+  return guard([&] {
+    const Arg& a = *static_cast<Arg*>(arg);
+    if (!a.is_ptr) bail(std::string("unexpected dtype for load Value(") + dtype_str(a.dtype) + ")");
+    *out = new op::Ast(op::load(a.id, Layout::from_shape(shape_of(dims, rank)), a.dtype));
+  });
+}
+int ugh_op_cst_i32(int32_t v, void** out) {
+  return guard([&] { *out = new op::Ast(op::cst(Const::i32(v))); });
+}
+int ugh_op_cst_f32(float v, void** out) {
+  return guard([&] { *out = new op::Ast(op::cst(Const::f32(v))); });
+}
+int ugh_op_unary(void* a, int op, void** out) {
+  return guard([&] { *out = new op::Ast(op::unary((UnaryOp)op, *static_cast<op::Ast*>(a))); });
+}
+int ugh_op_binary(int op, void* lhs, void* rhs, void** out) {
+  return guard([&] { *out = new op::Ast(op::binary((BinaryOp)op, *static_cast<op::Ast*>(lhs), *static_cast<op::Ast*>(rhs))); });
+}
+int ugh_op_reduce(int op, void* a, size_t axis, void** out) {
+  return guard([&] { *out = new op::Ast(op::reduce((ReduceOp)op, *static_cast<op::Ast*>(a), axis)); });
+}
+int ugh_op_broadcast(void* a, const size_t* dims, size_t rank, void** out) {
+  return guard([&] { *out = new op::Ast(op::broadcast(*static_cast<op::Ast*>(a), shape_of(dims, rank))); });
+}
+size_t ugh_op_ast_rank(void* a) { return static_cast<op::Ast*>(a)->shape.rank(); }
+void ugh_op_ast_dims(void* a, size_t* out) {
+  const auto& d = static_cast<op::Ast*>(a)->shape.dims();
+  for (size_t i = 0; i < d.size(); ++i) out[i] = d[i];
+}
+int ugh_op_ast_dtype(void* a) { return (int)static_cast<op::Ast*>(a)->dtype; }
+// ug-pyo3/src/lib.rs:230-237
+int ugh_op_store(void* arg, const size_t* dims, size_t rank, void* value, void** out) {
+  return guard([&] {
+    op::Store st;
+    st.dst = static_cast<Arg*>(arg)->id;
+    st.layout = Layout::from_shape(shape_of(dims, rank));
+    st.value = *static_cast<op::Ast*>(value);
+    *out = new op::Store(std::move(st));
+  });
+}
+void ugh_op_store_free(void* s) { delete static_cast<op::Store*>(s); }
+// ug-pyo3/src/lib.rs:244-265
+int ugh_op_kernel_new(const char* name, void** args, size_t n_args, void** stores, size_t n_stores, void** out) {
+  return guard([&] {
+    op::Kernel k;
+    k.name = name ? name : "";
+    for (size_t i = 0; i < n_args; ++i) k.args.push_back(*static_cast<Arg*>(args[i]));
+    for (size_t i = 0; i < n_stores; ++i) k.ops.push_back(*static_cast<op::Store*>(stores[i]));
+    *out = new op::Kernel(std::move(k));
+  });
+}
+void ugh_op_kernel_free(void* k) { delete static_cast<op::Kernel*>(k); }
+int ugh_op_kernel_lower(void* k, void** out) {
+  return guard([&] { *out = new ssa::Kernel(static_cast<op::Kernel*>(k)->lower(op::Opts{})); });
+}
+size_t ugh_op_kernel_str(void* k, char* buf, size_t buf_len) {
+  const op::Kernel& kk = *static_cast<op::Kernel*>(k);
+  std::string s = "Kernel { name: \"" + kk.name + "\", args: [";
+  for (size_t i = 0; i < kk.args.size(); ++i) s += (i ? ", " : "") + std::to_string(kk.args[i].id.v);
+  s += "], ops: [";
+  for (size_t i = 0; i < kk.ops.size(); ++i)
+    s += std::string(i ? ", " : "") + "Store { dst: " + std::to_string(kk.ops[i].dst.v) + ", shape: " + kk.ops[i].layout.shape().str() + ", value: " + ast_str(kk.ops[i].value) + " }";
+  return copy_out(s + "] }", buf, buf_len);
+}
+size_t ugh_ssa_str(void* kernel, char* buf, size_t buf_len) { return copy_out(ssa_str(*static_cast<ssa::Kernel*>(kernel)), buf, buf_len); }
+int ugh_ssa_flops_mem(void* kernel, size_t* flops, size_t* mem) {
+  return guard([&] { flops_mem(*static_cast<ssa::Kernel*>(kernel), flops, mem); });
+}
+// Device::compile_cu as ug-pyo3 exposes it (ug-pyo3/src/lib.rs:438-456), for HIP source text.
+int ugh_hip_compile_source(void* d, const char* source, const char* entry, size_t n_args, const int* arg_dtypes, uint32_t grid, uint32_t block,
+                           uint32_t shared, void** out) {
+  return guard([&] {
+    HipDevice* hd = dynamic_cast<HipDevice*>(dev_of(d).get());
+    if (!hd) bail("compile_hip needs the HIP device");
+    ughip_func* f = nullptr;
+    if (ughip_compile_source(hd->raw(), source, entry, n_args, arg_dtypes, grid, block, shared, &f)) bail(ughip_last_error());
+    *out = new std::shared_ptr<Func>(std::make_shared<HipFunc>(f));
+  });
+}
+
 // ---- lazy buffers ---------------------------------------------------------------------------------
 int ugh_lb_cst(void* d, int dtype, double v, const size_t* dims, size_t rank, void** out) {
   return guard([&] { *out = box(LazyBuffer::cst(const_of(dtype, v), shape_of(dims, rank), dev_of(d))); });

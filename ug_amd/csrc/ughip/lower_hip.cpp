@@ -188,7 +188,7 @@ struct Item {
 
 class Lowering {
  public:
-  Lowering(const ughip_ssa& s, const std::string& entry) : s_(s), I_(s.instrs), n_((int)s.n_instrs), entry_(entry) {}
+  Lowering(const ughip_ssa& s, const std::string& entry, bool as_written) : s_(s), I_(s.instrs), n_((int)s.n_instrs), entry_(entry), as_written_(as_written) {}
 
   Lowered run() {
     validate();
@@ -215,7 +215,7 @@ class Lowering {
       emit_literal(1, 1);  // valid source, never launched
       return out_;
     }
-    if (gpu_style) {
+    if (gpu_style || as_written_) {
       emit_literal(s_.grid_dim ? s_.grid_dim : 1, s_.block_dim ? s_.block_dim : 1);
       return out_;
     }
@@ -230,6 +230,7 @@ class Lowering {
   const ughip_instr* I_;
   int n_;
   std::string entry_;
+  bool as_written_ = false;
   Lowered out_;
 
   std::vector<VType> vt_;
@@ -1314,9 +1315,9 @@ class Lowering {
 
 }  // namespace
 
-Lowered lower_ssa(const ughip_ssa& ssa, const std::string& entry) {
+Lowered lower_ssa(const ughip_ssa& ssa, const std::string& entry, bool as_written) {
   if (!ssa.instrs || (!ssa.args && ssa.n_args)) throw std::runtime_error("ssa lowering: null instrs/args");
-  Lowering l(ssa, entry);
+  Lowering l(ssa, entry, as_written);
   return l.run();
 }
 

@@ -28,8 +28,10 @@ struct Lowered {
   bool empty_launch = false;       // a loop of the nest has zero trips: nothing to run
 };
 
-// Throws std::runtime_error on malformed SSA.
-Lowered lower_ssa(const ughip_ssa& ssa, const std::string& entry);
+// Throws std::runtime_error on malformed SSA.  as_written: translate statement by statement for
+// the kernel's own launch configuration (a serial loop nest stays one thread's loop nest, what
+// ug-cuda/src/code_gen.rs:68-186 emits) instead of re-parallelising it.
+Lowered lower_ssa(const ughip_ssa& ssa, const std::string& entry, bool as_written = false);
 
 const char* dtype_c_name(int dtype);
 size_t dtype_size(int dtype);

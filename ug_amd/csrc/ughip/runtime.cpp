@@ -247,10 +247,10 @@ static std::string sanitize_name(const char* name) {
   return s;
 }
 
-static int lower_checked(const ughip_ssa* ssa, const char* name, Lowered* out) {
+static int lower_checked(const ughip_ssa* ssa, const char* name, Lowered* out, bool as_written = false) {
   if (!ssa) return set_error(UGHIP_ERR_INVALID, "null ssa");
   try {
-    *out = lower_ssa(*ssa, sanitize_name(name));
+    *out = lower_ssa(*ssa, as_written && name && *name ? std::string(name) : sanitize_name(name), as_written);
   } catch (const std::exception& e) {
     return set_error(UGHIP_ERR_COMPILE, "%s", e.what());
   }
@@ -272,6 +272,24 @@ int ughip_codegen(const ughip_ssa* ssa, const char* name, char* buf, size_t buf_
     info->block_dim = low.block;
     info->lds_bytes = low.lds_bytes;
     info->scratch_bytes = low.scratch_part_bytes;
+  }
+  return UGHIP_OK;
+}
+
+int ughip_codegen_as_written(const ughip_ssa* ssa, const char* name, char* buf, size_t buf_len, size_t* out_len) {
+  Lowered low;
+  if (name) {
+    if (!*name) return set_error(UGHIP_ERR_INVALID, "codegen: empty kernel name");
+    for (const char* c = name; *c; ++c)
+      if (!(*c == '_' || (*c >= 'a' && *c <= 'z') || (*c >= 'A' && *c <= 'Z') || (c != name && *c >= '0' && *c <= '9')))
+        return set_error(UGHIP_ERR_INVALID, "codegen: '%s' is not a valid kernel name", name);
+  }
+  if (int rc = lower_checked(ssa, name, &low, true)) return rc;
+  if (out_len) *out_len = low.source.size();
+  if (buf && buf_len) {
+    size_t n = std::min(buf_len - 1, low.source.size());
+    memcpy(buf, low.source.data(), n);
+    buf[n] = 0;
   }
   return UGHIP_OK;
 }
@@ -331,6 +349,52 @@ int ughip_compile(ughip_device* dev, const ughip_ssa* ssa, const char* name, ugh
     f->function2 = it->second.function2;
   }
   if (f->low.scratch_part_bytes) HIPCHK(hipMalloc(&f->scratch_part, f->low.scratch_part_bytes));
+  ughip_device_retain(dev);
+  *out = f.release();
+  return UGHIP_OK;
+}
+
+int ughip_compile_source(ughip_device* dev, const char* source, const char* entry, size_t n_args, const int* arg_dtypes, unsigned grid_dim,
+                         unsigned block_dim, unsigned shared_mem_bytes, ughip_func** out) {
+  if (!dev || !out || !source || !entry || (n_args && !arg_dtypes)) return set_error(UGHIP_ERR_INVALID, "compile_source: null argument");
+  if (n_args > 64) return set_error(UGHIP_ERR_INVALID, "compile_source: %zu arguments, at most 64 are supported", n_args);
+  if (block_dim == 0 || block_dim > 1024) return set_error(UGHIP_ERR_INVALID, "compile_source: block_dim %u is not in 1..1024", block_dim);
+  if (shared_mem_bytes > 160 * 1024) return set_error(UGHIP_ERR_INVALID, "compile_source: %u bytes of LDS, a workgroup has 160 KiB", shared_mem_bytes);
+  for (size_t a = 0; a < n_args; ++a)
+    if (arg_dtypes[a] < 0 || arg_dtypes[a] > UGHIP_I64) return set_error(UGHIP_ERR_INVALID, "compile_source: unknown dtype %d for argument %zu", arg_dtypes[a], a);
+  if (int rc = device_activate(dev)) return rc;
+  std::unique_ptr<ughip_func> f(new ughip_func);
+  f->dev = dev;
+  Lowered& low = f->low;
+  low.source = source;
+  low.entry = entry;
+  low.strategy = UGHIP_STRAT_LITERAL;
+  low.grid = grid_dim;
+  low.block = block_dim;
+  low.lds_bytes = shared_mem_bytes;
+  low.arg_dtype.assign(arg_dtypes, arg_dtypes + n_args);
+  low.min_len.assign(n_args, -1);     // what the source indexes is not known here
+  low.arg_written.assign(n_args, 1);  // nor what it writes: no slice may be passed twice
+  low.empty_launch = grid_dim == 0;
+  {
+    std::lock_guard<std::mutex> g(dev->mu);
+    const std::string key = low.source + "\n// entry " + low.entry;
+    auto it = dev->modules.find(key);
+    if (it == dev->modules.end()) {
+      std::vector<char> code;
+      if (int rc = rtc_compile(low.source, dev->arch, &code)) return rc;
+      CachedModule cm;
+      HIPCHK(hipModuleLoadData(&cm.module, code.data()));
+      hipError_t e = hipModuleGetFunction(&cm.function, cm.module, low.entry.c_str());
+      if (e != hipSuccess) {
+        hipModuleUnload(cm.module);
+        return set_error(UGHIP_ERR_COMPILE, "compile_source: no kernel '%s' in the source (declare it extern \"C\" __global__): %s", low.entry.c_str(),
+                         hipGetErrorString(e));
+      }
+      it = dev->modules.emplace(key, cm).first;
+    }
+    f->function = it->second.function;
+  }
   ughip_device_retain(dev);
   *out = f.release();
   return UGHIP_OK;
