@@ -214,7 +214,13 @@ int ughip_rtc_check(const char* source, const char* arch, size_t* code_size);
 /* dst[b,m,n] = lhs[b,m,k] x rhs[b,k,n], beta = 0, f32 accumulate.  `rank` (2..4) strides
  * per operand, in elements, as in ug::Layout (layout.rs:577-583); batch strides follow
  * the rules of cpu_runtime.rs:527-549 and ug-cuda/src/gemm.rs:59-74.  dtype triple must
- * match: F32, F16 or BF16 (ug-cuda/src/gemm.rs:303-330); integers are UGHIP_ERR_UNSUPPORTED. */
+ * match: F32, F16 or BF16 (ug-cuda/src/gemm.rs:303-330); integers are UGHIP_ERR_UNSUPPORTED.
+ * One addition to the reference's contract: dst and lhs F32 with rhs BF16 (weights kept as a
+ * checkpoint stores them, where the reference widens them at load time,
+ * ug-core/src/safetensors.rs:120-271).  The rhs is widened on its way into LDS, so the result is
+ * bit for bit that of the F32 product on the widened values.  Built for an [n, k]-major rhs
+ * (strides (1, k)) with m % 128 == 0, n % 64 == 0, k % 32 == 0; other shapes are
+ * UGHIP_ERR_UNSUPPORTED (convert the rhs with ughip_convert first). */
 int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs,
                  const ughip_slice* rhs, size_t b, size_t m, size_t n, size_t k, size_t rank,
                  const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset,

@@ -358,6 +358,40 @@ def test_matmul_16bit_256x256_tiles(hip, bmnk, dtype):
     np.testing.assert_array_equal(got, other)
 
 
+@pytest.mark.parametrize("bmnk", [(1, 128, 2048, 2048), (1, 128, 256, 2048), (1, 256, 5632, 2048), (1, 128, 2048, 5632), (2, 512, 384, 96), (1, 1024, 1024, 32)])
+def test_matmul_f32_with_a_bf16_rhs(hip, bmnk):
+    """An F32 product reading an [n, k]-major rhs stored as bf16 (split-K prefill shapes and plain ones):
+    bit for bit the F32 product on the widened values."""
+    b, m, n, k = bmnk
+    print("matmul f32 x bf16", bmnk, flush=True)
+    a = rng.uniform_pm1(27, b * m * k).reshape(b, m, k)
+    w = rng.bf16_round(rng.uniform_pm1(28, b * k * n)).reshape(b, k, n)
+    wide = _raw_matmul(hip, ug_amd.F32, a, w, True)
+    sa = hip.slice_from(np.ascontiguousarray(a))
+    sw = hip.slice_from(rng.to_bf16_bits(np.ascontiguousarray(np.swapaxes(w, 1, 2))))
+    dst = hip.allocate_uninit(ug_amd.F32, b * m * n)
+    hip.matmul(dst, sa, sw, (b, m, n, k), ((b, m, k), (m * k, k, 1), 0), ((b, k, n), (k * n, 1, k), 0))
+    np.testing.assert_array_equal(dst.to_vec().reshape(b, m, n), wide)
+    exact = np.matmul(a.astype(np.float64), w.astype(np.float64))
+    bound = k * np.finfo(np.float32).eps * np.matmul(np.abs(a).astype(np.float64), np.abs(w).astype(np.float64))
+    assert np.all(np.abs(wide - exact) <= bound + 1e-7)
+
+
+def test_matmul_f32_with_a_bf16_rhs_limits(hip):
+    m, n, k = 128, 64, 64
+    sa, dst = hip.slice_from(np.zeros(m * k, np.float32)), hip.allocate_uninit(ug_amd.F32, m * n)
+    sw = hip.slice_from(np.zeros(n * k, np.uint16))
+    lhs = ((1, m, k), (m * k, k, 1), 0)
+    with pytest.raises(ug_amd.UgError, match=r"\[n, k\]-major"):      # [k, n]-major rhs
+        hip.matmul(dst, sa, sw, (1, m, n, k), lhs, ((1, k, n), (k * n, n, 1), 0))
+    with pytest.raises(ug_amd.UgError, match="multiples of 128, 64, 32"):     # one row of x: the fused projections' job
+        hip.matmul(dst, sa, sw, (1, 1, n, k), ((1, 1, k), (k, k, 1), 0), ((1, k, n), (k * n, 1, k), 0))
+    with pytest.raises(ug_amd.UgError, match="incorrect dtypes"):              # the other way round is not a thing
+        hip.matmul(dst, sw, sa, (1, m, n, k), lhs, ((1, k, n), (k * n, 1, k), 0))
+    hip.matmul(dst, sa, sw, (1, m, n, k), lhs, ((1, k, n), (k * n, 1, k), 0))
+    assert not dst.to_vec().any()
+
+
 # The m <= 8 shapes of decode: wave-per-column GEMV with 1, 2 or 4 waves per column, the short-k
 # variant (attention scores) and the [k, n]-major variant (attention output).
 GEMV_SHAPES = [(1, 1, 2048, 2048), (1, 1, 5000, 512), (1, 1, 7000, 256), (1, 3, 640, 320), (2, 8, 300, 1024), (32, 1, 129, 64), (32, 1, 77, 128),
@@ -1035,6 +1069,34 @@ def test_bf16_matrices_meet_several_rows_through_a_cast(hip, hip_ops):
 
     for got, want in zip(run(True), run(False)):
         assert np.array_equal(got, want)
+
+
+def test_linear_hook_reads_bf16_matrices_in_place(hip, hip_ops):
+    """Ops::linear: 128-row blocks of f32 against a bf16 matrix go to the mixed product, other row counts
+    widen the matrix first; both are the f32 result on the same values."""
+    k, n = 256, 192
+    w = rng.bf16_round(rng.normal(137, n * k, 0.05))
+    for t in (128, 384, 5):
+        x = rng.normal(138, t * k)
+        wide = hip_ops.linear(LB.copy(x, (1, t, k), hip), LB.copy(w, (n, k), hip)).data_vec()
+        got = hip_ops.linear(LB.copy(x, (1, t, k), hip), LB.copy(rng.to_bf16_bits(w), (n, k), hip))
+        assert tuple(got.dims()) == (1, t, n) and got.dtype == ug_amd.F32
+        np.testing.assert_array_equal(got.data_vec(), wide)
+        truth = x.reshape(t, k).astype(np.float64) @ w.reshape(n, k).astype(np.float64).T
+        np.testing.assert_allclose(wide.reshape(t, n), truth, rtol=1e-4, atol=1e-5)
+
+
+def test_llama_bf16_matrices_prefill_of_128_tokens(hip, hip_ops):
+    """A 128-token prompt sends every projection of the prefill through the mixed product: ids and margins
+    of the f32 model on the same weights."""
+    cfg = ug_amd.LlamaConfig(hidden_size=256, intermediate_size=512, max_position_embeddings=256, num_attention_heads=4, num_key_value_heads=2,
+                             num_hidden_layers=2, vocab_size=1024)
+    prompt = rng.token_ids(11, 128, cfg.vocab_size)
+    wide = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=0.2, round_bf16=True, fused_attention=3).generate(prompt, 6)
+    toks, st = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=0.2, round_bf16=True, fused_attention=3, bf16_matrices=True).generate(prompt, 6)
+    print("bf16 prefill 128", toks.tolist(), flush=True)
+    assert toks.tolist() == wide[0].tolist()
+    np.testing.assert_array_equal(st["margins"], wide[1]["margins"])
 
 
 def test_fused_projections_refuse_mixed_or_other_matrix_dtypes(hip):

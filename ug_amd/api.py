@@ -730,6 +730,12 @@ class LlamaOps(_Handle):
         lb._keep += [w_gate, w_up] + ([alpha] if alpha is not None else [])
         return lb
 
+    def linear(self, x, w):
+        """x w^T for a matrix that may be stored as bf16 under f32 rows."""
+        lb = self._op("ugh_llama_linear", x, _p(w.h))
+        lb._keep += [w]
+        return lb
+
     def linear_add(self, x, w, residual):
         """x w^T + residual"""
         lb = self._op("ugh_llama_linear_add", x, _p(w.h), _p(residual.h))

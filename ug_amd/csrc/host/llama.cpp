@@ -247,6 +247,25 @@ struct HipOps : Ops {
     return !alpha || (x.dims()[2] <= 4096 && alpha->dtype() == DType::F32 && alpha->elem_count() == x.dims()[2]);
   }
 
+  // f32 rows against a matrix stored as bf16: ughip_matmul reads it as it is where the tiled kernel
+  // applies (any number of 128-row blocks of x); other shapes widen it first.
+  LB linear(const LB& x, const LB& w) const override {
+    const size_t rows = x.rank() ? x.elem_count() / x.dims().back() : 0;
+    if (x.dtype() != DType::F32 || w.dtype() != DType::BF16 || w.rank() != 2 || x.rank() < 2 || w.dims()[1] != x.dims().back() || rows == 0 ||
+        rows % 128 != 0 || w.dims()[0] % 64 != 0 || w.dims()[1] % 32 != 0)
+      return Ops::linear(x, w);
+    const size_t n = w.dims()[0], k = w.dims()[1];
+    ughip_device* dev = hip_dev(x);
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != 3) bail("linear: expected 3 slices");
+      const size_t ld[3] = {1, rows, k}, ls[3] = {rows * k, k, 1}, rd[3] = {1, k, n}, rs[3] = {n * k, 1, k};
+      hip_check(ughip_matmul(dev, hip_raw_slice(*vs[2]), hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), 1, rows, n, k, 3, ld, ls, 0, rd, rs, 0), "linear");
+    };
+    std::vector<size_t> dims = x.dims();
+    dims.back() = n;
+    return LB::custom(f, {x, w}, Shape(dims), DType::F32, x.device());
+  }
+
   LB linear_packed(const LB& x, const std::vector<LB>& ws, const LB* alpha, float eps) const override {
     std::vector<const LB*> wp;
     for (const LB& w : ws) wp.push_back(&w);
@@ -452,29 +471,27 @@ LB Ops::attention_step(const LB&, const LB&, const LB&, size_t, size_t, float, c
 
 LB Ops::argmax_into(const LB&, const LB&, size_t, const LB&, const LB&, size_t) const { bail("argmax_into: this device reads the logits back and picks the token on the host"); }
 
-namespace {
 // A matrix kept in bf16 meets activations of another dtype: matmul wants one dtype throughout
 // (ug-core/src/lib.rs:62-70), so the matrix is widened for this use (exact).
-LB like(const LB& w, const LB& x) { return w.dtype() == x.dtype() ? w : w.cast(x.dtype()); }
-}  // namespace
+LB Ops::linear(const LB& x, const LB& w) const { return x.matmul_t(w.dtype() == x.dtype() ? w : w.cast(x.dtype())); }
 
 // model.rs:206-208 side by side.
 LB Ops::linear_packed(const LB& x0, const std::vector<LB>& ws, const LB* alpha, float eps) const {
   if (ws.empty()) bail("linear_packed: no matrices");
   LB x = alpha ? rms_norm(x0, *alpha, eps) : x0;
-  LB out = x.matmul_t(like(ws[0], x));
-  for (size_t i = 1; i < ws.size(); ++i) out = cat(out, x.matmul_t(like(ws[i], x)), x.rank() - 1);
+  LB out = linear(x, ws[0]);
+  for (size_t i = 1; i < ws.size(); ++i) out = cat(out, linear(x, ws[i]), x.rank() - 1);
   return out;
 }
 
 // model.rs:160-168 up to the down projection.
 LB Ops::gate_up(const LB& x0, const LB& w_gate, const LB& w_up, const LB* alpha, float eps) const {
   LB x = alpha ? rms_norm(x0, *alpha, eps) : x0;
-  return silu(x.matmul_t(like(w_gate, x))).binary(BinaryOp::Mul, x.matmul_t(like(w_up, x)));
+  return silu(linear(x, w_gate)).binary(BinaryOp::Mul, linear(x, w_up));
 }
 
 // model.rs:366-372: a projection, then the residual.
-LB Ops::linear_add(const LB& x, const LB& w, const LB& residual) const { return x.matmul_t(like(w, x)).binary(BinaryOp::Add, residual); }
+LB Ops::linear_add(const LB& x, const LB& w, const LB& residual) const { return linear(x, w).binary(BinaryOp::Add, residual); }
 
 std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16) {
   return std::make_shared<SyntheticWeights>(seed, std, round_bf16);
@@ -660,7 +677,7 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
   size_t seq_len = xs_in.dims()[1];
   size_t nh = cfg_.num_attention_heads, nkv = cfg_.num_key_value_heads, hd = cfg_.head_dim();
   const float eps = (float)cfg_.rms_norm_eps;
-  auto finish = [&](const LB& out) { return residual ? ops_->linear_add(out, l.o_proj, *residual) : out.matmul_t(like(l.o_proj, out)); };
+  auto finish = [&](const LB& out) { return residual ? ops_->linear_add(out, l.o_proj, *residual) : ops_->linear(out, l.o_proj); };
   if (fused_attention_ >= 3 && seq_len == 1 && xs_in.dims()[0] == 1 && cache.capacity && ops_->packed_projections()) {
     // one position: q | k | v come out of one launch (with the norm in front) side by side and are read where they lie
     const size_t nq = nh * hd, nk = nkv * hd, row = nq + 2 * nk, len = cache.len;
@@ -674,9 +691,9 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
     return finish(ops_->attention_cached(qkv, kc, vc, cache.len, scale, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, 0, row, nh));
   }
   LB xs = norm_first ? rms_norm(xs_in, l.rms1, eps) : xs_in;
-  LB q = xs.matmul_t(like(l.q_proj, xs));
-  LB k = xs.matmul_t(like(l.k_proj, xs));
-  LB v = xs.matmul_t(like(l.v_proj, xs));
+  LB q = ops_->linear(xs, l.q_proj);
+  LB k = ops_->linear(xs, l.k_proj);
+  LB v = ops_->linear(xs, l.v_proj);
   if (fused_attention_ >= 2) {
     // rows go from the projections into the caches (in place when they were preallocated) and
     // the attention kernel reads them there; the result comes back in the layout o_proj reads
@@ -735,10 +752,10 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
 LB Model::mlp(const Layer& l, const LB& xs, const LB* residual, bool norm_first) const {
   if (residual)
     return ops_->linear_add(ops_->gate_up(xs, l.gate_proj, l.up_proj, norm_first ? &l.rms2 : nullptr, (float)cfg_.rms_norm_eps), l.down_proj, *residual);
-  LB xs1 = xs.matmul_t(like(l.gate_proj, xs));
-  LB xs2 = xs.matmul_t(like(l.up_proj, xs));
+  LB xs1 = ops_->linear(xs, l.gate_proj);
+  LB xs2 = ops_->linear(xs, l.up_proj);
   xs1 = silu(xs1);
-  return xs1.binary(BinaryOp::Mul, xs2).matmul_t(like(l.down_proj, xs));
+  return ops_->linear(xs1.binary(BinaryOp::Mul, xs2), l.down_proj);
 }
 
 void Model::store_matrices_bf16() {
@@ -789,7 +806,7 @@ LB Model::fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const 
   }
   if (fused_attention_ >= 3) return ops_->linear_packed(xs, {head_}, &ln_f_, eps);
   xs = rms_norm(xs, ln_f_, eps);
-  return xs.matmul_t(like(head_, xs));
+  return ops_->linear(xs, head_);
 }
 
 // One prefill call over the prompt, then `n_steps` greedy single-token steps (graph rebuilt per

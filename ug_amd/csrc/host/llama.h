@@ -60,6 +60,11 @@ struct Ops {
   virtual LB attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float scale, const LB* cos, const LB* sin, const LB* pos,
                               bool interleaved, size_t q_offset = 0, size_t q_row_stride = 0, size_t n_heads = 0) const;
 
+  // x [.., k] against a matrix w [n, k] that may be stored in another dtype than x (bf16 weights under
+  // f32 activations).  The default widens w with a cast in front of matmul_t (model.rs:147-158 with
+  // the one dtype Device::matmul wants, ug-core/src/lib.rs:62-70).
+  virtual LB linear(const LB& x, const LB& w) const;
+
   // Projections with their neighbours folded in.  The defaults compose matmul_t with the lazy
   // graph's own element-wise ops, exactly as model.rs:160-168, 206-208, 366-372 do.
   // packed_projections(): linear_packed gives q|k|v side by side in one buffer and kv_append /

@@ -18,9 +18,10 @@ struct MMArgs {
 
 // Tuned kernel: 256x128, 128x128 or 128x64 tiles that divide M x N, K % 64 == 0 (bf16) /
 // K % 32 == 0 (f32), lhs rows contiguous, rhs either [k, n] row-major or [n, k] row-major.
-bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch);
+// rhs_bf16: the rhs is stored as bf16 under an f32 product ([n, k] row-major only) and widened on its way into LDS.
+bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf16 = false);
 // Bytes of f32 scratch the launch needs (split-K partial tiles for skinny products; 0 for most).
 size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch);
-hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, float* workspace);
+hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, float* workspace, bool rhs_bf16 = false);
 
 }  // namespace ughip

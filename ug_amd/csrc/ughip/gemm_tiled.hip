@@ -73,8 +73,22 @@ struct Staged {
   u32x4 b[4];
 };
 
-template <typename T, bool B_NK, int BM, int BN, int NT>
-__device__ __forceinline__ void load_tiles(const T* __restrict__ A, const T* __restrict__ B, const MMArgs& p, int kt, int tid, Staged<BM, NT>& r) {
+// B_NK: 0 = rhs [k, n] row-major, 1 = rhs [n, k] row-major, 2 = [n, k] row-major stored as bf16 under an
+// f32 product (BT = uint16_t): a chunk of 4 elements is 8 bytes in memory and is widened on its way
+// into LDS (exact), so the product is bit for bit the f32 one on the widened values.
+template <typename T, int B_NK>
+struct RhsElt {
+  typedef T type;
+};
+template <>
+struct RhsElt<float, 2> {
+  typedef uint16_t type;
+};
+
+__device__ __forceinline__ u32x4 widen_bf16x4(const u32x4& r) { return u32x4{r.x << 16, r.x & 0xffff0000u, r.y << 16, r.y & 0xffff0000u}; }
+
+template <typename T, int B_NK, int BM, int BN, int NT, typename BT>
+__device__ __forceinline__ void load_tiles(const T* __restrict__ A, const BT* __restrict__ B, const MMArgs& p, int kt, int tid, Staged<BM, NT>& r) {
   constexpr int RP = NT / 8;  // rows per pass
   constexpr int BK = Elt<T>::BK, VE = Elt<T>::VE;
   constexpr bool IS_16BIT = sizeof(T) == 2;
@@ -84,14 +98,22 @@ __device__ __forceinline__ void load_tiles(const T* __restrict__ A, const T* __r
 #pragma unroll
   for (int i = 0; i < BM / RP; ++i) r.a[i] = *reinterpret_cast<const u32x4*>(Ap + i * a_step);
   if (B_NK) {
-    const T* Bp = B + (size_t)(tid >> 3) * p.b_cs + k0 + (tid & 7) * VE;
+    const BT* Bp = B + (size_t)(tid >> 3) * p.b_cs + k0 + (tid & 7) * VE;
     const size_t b_step = (size_t)RP * p.b_cs;
 #pragma unroll
-    for (int i = 0; i < BN / RP; ++i) r.b[i] = *reinterpret_cast<const u32x4*>(Bp + i * b_step);
+    for (int i = 0; i < BN / RP; ++i) {
+      if (B_NK == 2) {
+        const u32x2 v = *reinterpret_cast<const u32x2*>(Bp + i * b_step);
+        r.b[i].x = v.x;
+        r.b[i].y = v.y;
+      } else {
+        r.b[i] = *reinterpret_cast<const u32x4*>(Bp + i * b_step);
+      }
+    }
   } else if (tid < 2 * BN) {
     // 4 (k) x 8 (n) bf16 block or 4 (k) x 4 (n) f32 block per thread; 2 * BN threads cover the tile
     const int kg = IS_16BIT ? (tid & 15) : (tid & 7), ng = IS_16BIT ? (tid >> 4) : (tid >> 3);
-    const T* Bp = B + (k0 + kg * 4) * (size_t)p.b_rs + ng * VE;
+    const T* Bp = reinterpret_cast<const T*>(B) + (k0 + kg * 4) * (size_t)p.b_rs + ng * VE;
 #pragma unroll
     for (int i = 0; i < 4; ++i) r.b[i] = *reinterpret_cast<const u32x4*>(Bp + i * (size_t)p.b_rs);
   }
@@ -99,7 +121,7 @@ __device__ __forceinline__ void load_tiles(const T* __restrict__ A, const T* __r
 
 // Staging stores of one prefetched tile, split into four parts (PART = 0..3) so that they can be
 // spread between the MFMAs of a K tile.  PART < 0 issues all of them.
-template <typename T, bool B_NK, int BM, int BN, int NT, int PART>
+template <typename T, int B_NK, int BM, int BN, int NT, int PART>
 __device__ __forceinline__ void store_tiles(u32x4* __restrict__ S, int tid, const Staged<BM, NT>& r) {
   constexpr bool IS_16BIT = sizeof(T) == 2;
   constexpr int RP = NT / 8, NA = BM / RP;
@@ -112,7 +134,7 @@ __device__ __forceinline__ void store_tiles(u32x4* __restrict__ S, int tid, cons
     u32x4* Sb = Sa + BM * CHUNKS;
 #pragma unroll
     for (int i = 0; i < BN / RP; ++i)
-      if (PART < 0 || ((NA + i) & 3) == PART) Sb[i * RP * CHUNKS] = r.b[i];
+      if (PART < 0 || ((NA + i) & 3) == PART) Sb[i * RP * CHUNKS] = B_NK == 2 ? widen_bf16x4(r.b[i]) : r.b[i];
   } else if (tid < 2 * BN) {
     if (IS_16BIT) {
       const int kg = tid & 15, ng = tid >> 4;
@@ -193,7 +215,7 @@ __device__ __forceinline__ void interleave_step() {
 }
 
 // Staging stores of part PART (see store_tiles): A stores i with i % 4 == PART, then B's.
-template <typename T, bool B_NK, int BM, int BN, int NT>
+template <typename T, int B_NK, int BM, int BN, int NT>
 constexpr int stores_in_part(int part) {
   const int rp = NT / 8, na = BM / rp;
   int n = 0;
@@ -217,8 +239,8 @@ constexpr int stores_in_part(int part) {
 // The loads are unconditional (LOAD is a compile-time switch): a load under a run-time branch makes
 // the compiler wait for every outstanding load before the staging stores, which would undo the
 // two-tile lead.
-template <typename T, bool B_NK, int BM, int BN, int NT, int MI, int NJ, bool LOAD, int WRITE>
-__device__ __forceinline__ void k_phase(const T* __restrict__ A, const T* __restrict__ B, const MMArgs& p, const u32x4* __restrict__ cur, u32x4* __restrict__ nxt,
+template <typename T, int B_NK, int BM, int BN, int NT, int MI, int NJ, bool LOAD, int WRITE>
+__device__ __forceinline__ void k_phase(const T* __restrict__ A, const typename RhsElt<T, B_NK>::type* __restrict__ B, const MMArgs& p, const u32x4* __restrict__ cur, u32x4* __restrict__ nxt,
                                         bool do_write, const Staged<BM, NT>& wr, int load_kt, Staged<BM, NT>& ld, int tid, int lane, int wm, int wn,
                                         floatx16 (&acc)[MI][NJ]) {
   constexpr int N_MFMA = MI * NJ * (sizeof(T) == 4 ? 4 : 1), N_READ = MI + NJ;
@@ -260,7 +282,7 @@ __device__ __forceinline__ void k_phase(const T* __restrict__ A, const T* __rest
 // [s * kt_per, (s + 1) * kt_per)), each writes its f32 partial tile to ws[s][batch][m][n], and
 // gemm_split_reduce adds the slabs in index order.  For skinny products (few output tiles, long K:
 // the projections of a 128-token prefill) this is what puts every CU to work.
-template <typename T, bool B_NK, int BM, int BN, int NT, bool SPLIT>
+template <typename T, int B_NK, int BM, int BN, int NT, bool SPLIT>
 __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p, int tiles_m, int tiles_n, int remap, int nsplit, int kt_per, float* __restrict__ ws) {
   extern __shared__ u32x4 lds[];
   constexpr int BK = Elt<T>::BK;
@@ -281,8 +303,9 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p, int tiles_m, int tile
   const int kt0 = SPLIT ? slab * kt_per : 0;
   const size_t k_off = (size_t)kt0 * BK;
   const T* __restrict__ A = static_cast<const T*>(p.a) + (size_t)batch * p.a_bs + (size_t)m0 * p.a_rs + k_off;
-  const T* __restrict__ B =
-      static_cast<const T*>(p.b) + (size_t)batch * p.b_bs + (B_NK ? (size_t)n0 * p.b_cs + k_off : (size_t)n0 + k_off * (size_t)p.b_rs);
+  typedef typename RhsElt<T, B_NK>::type BT;
+  const BT* __restrict__ B =
+      static_cast<const BT*>(p.b) + (size_t)batch * p.b_bs + (B_NK ? (size_t)n0 * p.b_cs + k_off : (size_t)n0 + k_off * (size_t)p.b_rs);
   const int KT = SPLIT ? min(kt_per, p.K / BK - kt0) : p.K / BK;
   const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
 
@@ -481,7 +504,7 @@ __global__ void __launch_bounds__(256) gemm_split_reduce(const float* __restrict
   o[3] = (T)s.w;
 }
 
-template <typename T, bool B_NK, int BM, int BN, int NT, bool SPLIT>
+template <typename T, int B_NK, int BM, int BN, int NT, bool SPLIT>
 hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch, int nsplit, float* ws) {
   constexpr int LDS_BYTES = 2 * (BM + BN) * CHUNKS * 16;
   constexpr int BK = Elt<T>::BK;
@@ -526,7 +549,7 @@ hipError_t launch_dma256(hipStream_t stream, const MMArgs& p, size_t batch) {
   return hipGetLastError();
 }
 
-template <typename T, bool B_NK, bool SPLIT>
+template <typename T, int B_NK, bool SPLIT>
 hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int shape, int nsplit, float* ws) {
   switch (shape) {
     case 0:
@@ -534,7 +557,7 @@ hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int s
                                          : launch<T, B_NK, 256, 128, 512, SPLIT>(stream, p, batch, nsplit, ws);
     case 1: return launch<T, B_NK, 128, 128, 256, SPLIT>(stream, p, batch, nsplit, ws);
     case 3:
-      if constexpr (sizeof(T) == 2 && B_NK && !SPLIT) return launch_dma256<T>(stream, p, batch);
+      if constexpr (sizeof(T) == 2 && B_NK == 1 && !SPLIT) return launch_dma256<T>(stream, p, batch);
       [[fallthrough]];
     default: return launch<T, B_NK, 128, 64, 256, SPLIT>(stream, p, batch, nsplit, ws);
   }
@@ -585,8 +608,9 @@ int pick_split(int dtype, const MMArgs& p, size_t batch, int shape) {
 
 }  // namespace
 
-bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch) {
+bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf16) {
   if (dtype != UGHIP_F32 && dtype != UGHIP_BF16 && dtype != UGHIP_F16) return false;
+  if (rhs_bf16 && (dtype != UGHIP_F32 || p.b_rs != 1 || p.b_cs == 1)) return false;  // widening is built for an [n, k]-major rhs under an f32 product
   const int ve = dtype == UGHIP_F32 ? 4 : 8, bk = dtype == UGHIP_F32 ? 32 : 64;
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.K % bk || batch == 0) return false;
   if (p.a_cs != 1 || p.a_rs % ve || p.a_bs % ve || p.b_bs % ve || p.c_bs % ve) return false;
@@ -607,19 +631,22 @@ size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch) {
   return nsplit > 1 ? (size_t)nsplit * batch * (size_t)p.M * p.N * sizeof(float) : 0;
 }
 
-hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, float* workspace) {
+hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, float* workspace, bool rhs_bf16) {
   const bool nt = p.b_rs == 1 && p.b_cs != 1;
+  if (rhs_bf16 && (dtype != UGHIP_F32 || !nt)) return hipErrorInvalidValue;
   const int s = pick_shape(p, batch, dtype);
   if (s < 0) return hipErrorInvalidValue;
   const int nsplit = s == 3 ? 1 : pick_split(dtype, p, batch, s);
   if (nsplit > 1) {
     if (!workspace) return hipErrorInvalidValue;
+    if (rhs_bf16) return launch_shape<float, 2, true>(stream, p, batch, s, nsplit, workspace);
     if (dtype == UGHIP_F32)
       return nt ? launch_shape<float, true, true>(stream, p, batch, s, nsplit, workspace) : launch_shape<float, false, true>(stream, p, batch, s, nsplit, workspace);
     if (dtype == UGHIP_F16)
       return nt ? launch_shape<_Float16, true, true>(stream, p, batch, s, nsplit, workspace) : launch_shape<_Float16, false, true>(stream, p, batch, s, nsplit, workspace);
     return nt ? launch_shape<__bf16, true, true>(stream, p, batch, s, nsplit, workspace) : launch_shape<__bf16, false, true>(stream, p, batch, s, nsplit, workspace);
   }
+  if (rhs_bf16) return launch_shape<float, 2, false>(stream, p, batch, s, 1, nullptr);
   if (dtype == UGHIP_F32)
     return nt ? launch_shape<float, true, false>(stream, p, batch, s, 1, nullptr) : launch_shape<float, false, false>(stream, p, batch, s, 1, nullptr);
   if (dtype == UGHIP_F16)

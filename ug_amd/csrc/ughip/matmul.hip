@@ -394,7 +394,10 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
   if (!dev || !dst || !lhs || !rhs) return set_error(UGHIP_ERR_INVALID, "matmul: null argument");
   if (rank < 2 || rank > 4 || !lhs_dims || !lhs_strides || !rhs_dims || !rhs_strides)
     return set_error(UGHIP_ERR_INVALID, "matmul: rank %zu layouts are not supported", rank);
-  if (dst->dtype != lhs->dtype || dst->dtype != rhs->dtype || (dst->dtype != UGHIP_F32 && dst->dtype != UGHIP_BF16 && dst->dtype != UGHIP_F16)) {
+  // One dtype for all three (lib.rs:62-70), with one addition: an F32 product may read a BF16 rhs (weights
+  // kept as a checkpoint stores them); it is widened on the way in, which is exact.
+  const bool mixed = dst->dtype == UGHIP_F32 && lhs->dtype == UGHIP_F32 && rhs->dtype == UGHIP_BF16;
+  if (!mixed && (dst->dtype != lhs->dtype || dst->dtype != rhs->dtype || (dst->dtype != UGHIP_F32 && dst->dtype != UGHIP_BF16 && dst->dtype != UGHIP_F16))) {
     int code = (dst->dtype == lhs->dtype && dst->dtype == rhs->dtype) ? UGHIP_ERR_UNSUPPORTED : UGHIP_ERR_INVALID;
     return set_error(code, "incorrect dtypes for matmul, dst: %s, lhs: %s, rhs: %s", dtype_name(dst->dtype), dtype_name(lhs->dtype),
                      dtype_name(rhs->dtype));
@@ -422,7 +425,7 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
   if (int rc = device_activate(dev)) return rc;
   const size_t esz = dst->dtype == UGHIP_F32 ? 4 : 2;
   p.a = static_cast<const char*>(lhs->ptr) + lhs_offset * esz;
-  p.b = static_cast<const char*>(rhs->ptr) + rhs_offset * esz;
+  p.b = static_cast<const char*>(rhs->ptr) + rhs_offset * (mixed ? 2 : esz);
   p.c = dst->ptr;
   const bool f32 = dst->dtype == UGHIP_F32;
   hipStream_t st = dev->stream;
@@ -434,16 +437,23 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
   const bool rhs_vec_ok = (b == 1 || p.b_bs % lv == 0) && rhs_offset % vec == 0;
   const bool gemv_nt_ok = small_m && lhs_vec_ok && rhs_vec_ok && k % vec == 0 && p.b_rs == 1 && (n == 1 || p.b_cs % lv == 0);
   const bool gemv_nn_ok = small_m && f32 && rhs_vec_ok && n % 4 == 0 && p.b_cs == 1 && (k == 1 || p.b_rs % 4 == 0);
-  if (gemv_nt_ok) {
+  if (mixed) {
+    if (!gemm_tiled_supported(UGHIP_F32, p, b, true) || rhs_offset % 8 != 0)
+      return set_error(UGHIP_ERR_UNSUPPORTED,
+                       "matmul: an F32 product with a BF16 rhs is built for an [n, k]-major rhs and m, n, k in multiples of 128, 64, 32 "
+                       "(got m %zu, n %zu, k %zu, rhs strides %lld, %lld)",
+                       m, n, k, p.b_rs, p.b_cs);
+  }
+  if (!mixed && gemv_nt_ok) {
     if (f32) launch_gemv_nt_any<float>(st, p, b);
     else if (dst->dtype == UGHIP_F16) launch_gemv_nt_any<_Float16>(st, p, b);
     else launch_gemv_nt_any<__bf16>(st, p, b);
-  } else if (gemv_nn_ok) {
+  } else if (!mixed && gemv_nn_ok) {
     dim3 grid((unsigned)((n + 63) / 64), 1, (unsigned)b);
     if (m == 1) gemv_nn_f32<1><<<grid, 1024, 0, st>>>(p);
     else if (m <= 4) gemv_nn_f32<4><<<grid, 1024, 0, st>>>(p);
     else gemv_nn_f32<8><<<grid, 1024, 0, st>>>(p);
-  } else if (gemm_tiled_supported(dst->dtype, p, b)) {
+  } else if (gemm_tiled_supported(dst->dtype, p, b, mixed)) {
     const size_t ws_bytes = gemm_tiled_workspace_bytes(dst->dtype, p, b);
     if (ws_bytes > dev->gemm_ws_bytes) {
       std::lock_guard<std::mutex> g(dev->mu);
@@ -455,7 +465,7 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
       UGHIP_HIPCHK(hipMalloc(&dev->gemm_ws, want));
       dev->gemm_ws_bytes = want;
     }
-    UGHIP_HIPCHK(gemm_tiled_launch(st, dst->dtype, p, b, ws_bytes ? static_cast<float*>(dev->gemm_ws) : nullptr));
+    UGHIP_HIPCHK(gemm_tiled_launch(st, dst->dtype, p, b, ws_bytes ? static_cast<float*>(dev->gemm_ws) : nullptr, mixed));
     return UGHIP_OK;
   } else {
     dim3 grid((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64), (unsigned)b);
