@@ -288,7 +288,9 @@ def _raw_matmul(hip, dtype, a, w, rhs_nk):
     b, m, k = a.shape
     n = w.shape[2]
     enc = rng.to_bf16_bits if dtype == ug_amd.BF16 else (lambda v: v.astype(np.float16)) if dtype == ug_amd.F16 else (lambda v: v)
-    dst = hip.allocate_uninit(dtype, b * m * n)
+    guard = 4 * n
+    fill = np.full(b * m * n + guard, 7.0, np.float32)
+    dst = hip.slice_from(enc(fill))
     sa = hip.slice_from(enc(np.ascontiguousarray(a)))
     if rhs_nk:
         sw = hip.slice_from(enc(np.ascontiguousarray(np.swapaxes(w, 1, 2))))
@@ -298,15 +300,20 @@ def _raw_matmul(hip, dtype, a, w, rhs_nk):
         rhs = ((b, k, n), (k * n, n, 1), 0)
     hip.matmul(dst, sa, sw, (b, m, n, k), ((b, m, k), (m * k, k, 1), 0), rhs)
     out = dst.to_vec()
-    return (rng.from_bf16_bits(out) if dtype == ug_amd.BF16 else out.astype(np.float32)).reshape(b, m, n)
+    out = rng.from_bf16_bits(out) if dtype == ug_amd.BF16 else out.astype(np.float32)
+    assert np.all(out[b * m * n:] == 7.0), "matmul wrote past the end of its result"
+    return out[:b * m * n].reshape(b, m, n)
 
 
-# Shapes that are whole multiples of a 256x128, 128x128 or 128x64 tile (K a multiple of 32 f32 / 64
-# bf16) take the tuned MFMA kernel; neighbours one element off take the generic one.  Both are held
-# to the same bound.
+# N a whole multiple of a tile width and K a multiple of 32 (f32) / 64 (bf16) take the tuned MFMA kernel, with
+# any number of rows from 9 up (a last tile that hangs over the end of the lhs reads its last row again and
+# stores nothing for the rows that do not exist; split-K included: 100 x 2048 x 2048 is a prompt of 100 tokens);
+# neighbours one column off take the generic one.  All are held to the same bound, and a sentinel behind the
+# result checks that nothing is written past the last row.
 @pytest.mark.parametrize("rhs_nk", [False, True])
 @pytest.mark.parametrize("bmnk", [(2, 256, 128, 96), (1, 512, 384, 160), (3, 256, 256, 32), (1, 255, 128, 96), (1, 256, 129, 96),
-                                  (1, 128, 128, 64), (2, 128, 64, 96), (1, 384, 192, 64), (40, 256, 128, 32), (32, 512, 64, 512)])
+                                  (1, 128, 128, 64), (2, 128, 64, 96), (1, 384, 192, 64), (40, 256, 128, 32), (32, 512, 64, 512),
+                                  (1, 100, 2048, 2048), (2, 300, 256, 64), (1, 37, 5632, 256), (3, 9, 64, 32), (1, 129, 128, 96)])
 def test_matmul_f32_tile_multiples(hip, bmnk, rhs_nk):
     b, m, n, k = bmnk
     print("matmul f32", bmnk, "rhs_nk", rhs_nk, flush=True)
@@ -320,7 +327,8 @@ def test_matmul_f32_tile_multiples(hip, bmnk, rhs_nk):
 
 @pytest.mark.parametrize("rhs_nk", [False, True])
 @pytest.mark.parametrize("bmnk", [(2, 256, 128, 192), (1, 512, 384, 64), (3, 256, 256, 320), (1, 256, 128, 96), (1, 248, 128, 128),
-                                  (1, 128, 128, 64), (2, 128, 64, 128), (1, 384, 192, 192), (40, 256, 128, 64)])
+                                  (1, 128, 128, 64), (2, 128, 64, 128), (1, 384, 192, 192), (40, 256, 128, 64), (1, 100, 2048, 2048), (2, 300, 256, 64),
+                                  (3, 9, 64, 64)])
 def test_matmul_bf16_tile_multiples(hip, bmnk, rhs_nk):
     b, m, n, k = bmnk
     print("matmul bf16", bmnk, "rhs_nk", rhs_nk, flush=True)
@@ -358,7 +366,8 @@ def test_matmul_16bit_256x256_tiles(hip, bmnk, dtype):
     np.testing.assert_array_equal(got, other)
 
 
-@pytest.mark.parametrize("bmnk", [(1, 128, 2048, 2048), (1, 128, 256, 2048), (1, 256, 5632, 2048), (1, 128, 2048, 5632), (2, 512, 384, 96), (1, 1024, 1024, 32)])
+@pytest.mark.parametrize("bmnk", [(1, 128, 2048, 2048), (1, 128, 256, 2048), (1, 256, 5632, 2048), (1, 128, 2048, 5632), (2, 512, 384, 96), (1, 1024, 1024, 32),
+                                  (1, 100, 2048, 2048), (2, 130, 128, 64), (1, 9, 64, 32)])
 def test_matmul_f32_with_a_bf16_rhs(hip, bmnk):
     """An F32 product reading an [n, k]-major rhs stored as bf16 (split-K prefill shapes and plain ones):
     bit for bit the F32 product on the widened values."""
@@ -384,8 +393,8 @@ def test_matmul_f32_with_a_bf16_rhs_limits(hip):
     lhs = ((1, m, k), (m * k, k, 1), 0)
     with pytest.raises(ug_amd.UgError, match=r"\[n, k\]-major"):      # [k, n]-major rhs
         hip.matmul(dst, sa, sw, (1, m, n, k), lhs, ((1, k, n), (k * n, n, 1), 0))
-    with pytest.raises(ug_amd.UgError, match="multiples of 128, 64, 32"):     # one row of x: the fused projections' job
-        hip.matmul(dst, sa, sw, (1, 1, n, k), ((1, 1, k), (k, k, 1), 0), ((1, k, n), (k * n, 1, k), 0))
+    with pytest.raises(ug_amd.UgError, match="multiples of 64, 32"):           # a column count no tile divides
+        hip.matmul(dst, sa, sw, (1, m, n - 1, k), lhs, ((1, k, n - 1), (k * (n - 1), 1, k), 0))
     with pytest.raises(ug_amd.UgError, match="incorrect dtypes"):              # the other way round is not a thing
         hip.matmul(dst, sw, sa, (1, m, n, k), lhs, ((1, k, n), (k * n, 1, k), 0))
     hip.matmul(dst, sa, sw, (1, m, n, k), lhs, ((1, k, n), (k * n, 1, k), 0))
@@ -1072,11 +1081,11 @@ def test_bf16_matrices_meet_several_rows_through_a_cast(hip, hip_ops):
 
 
 def test_linear_hook_reads_bf16_matrices_in_place(hip, hip_ops):
-    """Ops::linear: 128-row blocks of f32 against a bf16 matrix go to the mixed product, other row counts
-    widen the matrix first; both are the f32 result on the same values."""
+    """Ops::linear: 9 or more rows of f32 against a bf16 matrix go to the mixed product, one row to the fused
+    projection, 2 to 8 rows widen the matrix first; all are the f32 result on the same values."""
     k, n = 256, 192
     w = rng.bf16_round(rng.normal(137, n * k, 0.05))
-    for t in (128, 384, 5):
+    for t in (128, 384, 5, 100, 1):
         x = rng.normal(138, t * k)
         wide = hip_ops.linear(LB.copy(x, (1, t, k), hip), LB.copy(w, (n, k), hip)).data_vec()
         got = hip_ops.linear(LB.copy(x, (1, t, k), hip), LB.copy(rng.to_bf16_bits(w), (n, k), hip))

@@ -247,12 +247,15 @@ struct HipOps : Ops {
     return !alpha || (x.dims()[2] <= 4096 && alpha->dtype() == DType::F32 && alpha->elem_count() == x.dims()[2]);
   }
 
-  // f32 rows against a matrix stored as bf16: ughip_matmul reads it as it is where the tiled kernel
-  // applies (any number of 128-row blocks of x); other shapes widen it first.
+  // f32 rows against a matrix stored as bf16: one row is a fused projection without neighbours; from 9
+  // rows up (where an f32 matrix takes the tiled kernel too) ughip_matmul reads the matrix as it is;
+  // the row counts in between and the shapes no tile divides widen it first.  Each way the numbers
+  // are those of the f32 matrix with the same values.
   LB linear(const LB& x, const LB& w) const override {
     const size_t rows = x.rank() ? x.elem_count() / x.dims().back() : 0;
-    if (x.dtype() != DType::F32 || w.dtype() != DType::BF16 || w.rank() != 2 || x.rank() < 2 || w.dims()[1] != x.dims().back() || rows == 0 ||
-        rows % 128 != 0 || w.dims()[0] % 64 != 0 || w.dims()[1] % 32 != 0)
+    if (x.dtype() == DType::F32 && w.dtype() == DType::BF16 && rows == 1 && x.rank() == 3 && one_f32_row(x, {&w})) return linear_packed(x, {w}, nullptr, 0.f);
+    if (x.dtype() != DType::F32 || w.dtype() != DType::BF16 || w.rank() != 2 || x.rank() < 2 || w.dims()[1] != x.dims().back() || rows <= 8 ||
+        w.dims()[0] % 64 != 0 || w.dims()[1] % 32 != 0)
       return Ops::linear(x, w);
     const size_t n = w.dims()[0], k = w.dims()[1];
     ughip_device* dev = hip_dev(x);

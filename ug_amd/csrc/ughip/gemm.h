@@ -16,8 +16,9 @@ struct MMArgs {
   long long a_bs, b_bs, c_bs;
 };
 
-// Tuned kernel: 256x128, 128x128 or 128x64 tiles that divide M x N, K % 64 == 0 (bf16) /
-// K % 32 == 0 (f32), lhs rows contiguous, rhs either [k, n] row-major or [n, k] row-major.
+// Tuned kernel: 256x128, 128x128 or 128x64 tiles whose width divides N (the 128-row tiles take any M:
+// the last one may hang over the end of the lhs), K % 64 == 0 (bf16) / K % 32 == 0 (f32), lhs rows
+// contiguous, rhs either [k, n] row-major or [n, k] row-major.
 // rhs_bf16: the rhs is stored as bf16 under an f32 product ([n, k] row-major only) and widened on its way into LDS.
 bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf16 = false);
 // Bytes of f32 scratch the launch needs (split-K partial tiles for skinny products; 0 for most).

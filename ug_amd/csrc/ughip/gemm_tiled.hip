@@ -87,7 +87,9 @@ struct RhsElt<float, 2> {
 
 __device__ __forceinline__ u32x4 widen_bf16x4(const u32x4& r) { return u32x4{r.x << 16, r.x & 0xffff0000u, r.y << 16, r.y & 0xffff0000u}; }
 
-template <typename T, int B_NK, int BM, int BN, int NT, typename BT>
+// RAGGED: the tile hangs over the last row of the lhs; p.M is then the number of rows of THIS tile that
+// exist, and rows past them read the last one (their products are never stored).
+template <typename T, int B_NK, int BM, int BN, int NT, bool RAGGED = false, typename BT>
 __device__ __forceinline__ void load_tiles(const T* __restrict__ A, const BT* __restrict__ B, const MMArgs& p, int kt, int tid, Staged<BM, NT>& r) {
   constexpr int RP = NT / 8;  // rows per pass
   constexpr int BK = Elt<T>::BK, VE = Elt<T>::VE;
@@ -96,7 +98,14 @@ __device__ __forceinline__ void load_tiles(const T* __restrict__ A, const BT* __
   const T* Ap = A + (size_t)(tid >> 3) * p.a_rs + k0 + (tid & 7) * VE;  // row tid/8 (+RP per pass), chunk tid%8
   const size_t a_step = (size_t)RP * p.a_rs;
 #pragma unroll
-  for (int i = 0; i < BM / RP; ++i) r.a[i] = *reinterpret_cast<const u32x4*>(Ap + i * a_step);
+  for (int i = 0; i < BM / RP; ++i) {
+    if (RAGGED) {
+      const int row = min((tid >> 3) + i * RP, p.M - 1);
+      r.a[i] = *reinterpret_cast<const u32x4*>(A + (size_t)row * p.a_rs + k0 + (tid & 7) * VE);
+    } else {
+      r.a[i] = *reinterpret_cast<const u32x4*>(Ap + i * a_step);
+    }
+  }
   if (B_NK) {
     const BT* Bp = B + (size_t)(tid >> 3) * p.b_cs + k0 + (tid & 7) * VE;
     const size_t b_step = (size_t)RP * p.b_cs;
@@ -239,7 +248,7 @@ constexpr int stores_in_part(int part) {
 // The loads are unconditional (LOAD is a compile-time switch): a load under a run-time branch makes
 // the compiler wait for every outstanding load before the staging stores, which would undo the
 // two-tile lead.
-template <typename T, int B_NK, int BM, int BN, int NT, int MI, int NJ, bool LOAD, int WRITE>
+template <typename T, int B_NK, int BM, int BN, int NT, int MI, int NJ, bool LOAD, int WRITE, bool RAGGED = false>
 __device__ __forceinline__ void k_phase(const T* __restrict__ A, const typename RhsElt<T, B_NK>::type* __restrict__ B, const MMArgs& p, const u32x4* __restrict__ cur, u32x4* __restrict__ nxt,
                                         bool do_write, const Staged<BM, NT>& wr, int load_kt, Staged<BM, NT>& ld, int tid, int lane, int wm, int wn,
                                         floatx16 (&acc)[MI][NJ]) {
@@ -250,7 +259,7 @@ __device__ __forceinline__ void k_phase(const T* __restrict__ A, const typename 
   load_frags<BM, MI, NJ>(cur, lane, wm, wn, 0, f0);
   __builtin_amdgcn_sched_barrier(0);
   // step 0
-  if (LOAD) load_tiles<T, B_NK, BM, BN, NT>(A, B, p, load_kt, tid, ld);
+  if (LOAD) load_tiles<T, B_NK, BM, BN, NT, RAGGED>(A, B, p, load_kt, tid, ld);
   load_frags<BM, MI, NJ>(cur, lane, wm, wn, 1, f1);
   mma_frags<T, MI, NJ>(f0, acc);
   if (WRITE == 1 || (WRITE == 2 && do_write)) store_tiles<T, B_NK, BM, BN, NT, 0>(nxt, tid, wr);
@@ -282,8 +291,8 @@ __device__ __forceinline__ void k_phase(const T* __restrict__ A, const typename 
 // [s * kt_per, (s + 1) * kt_per)), each writes its f32 partial tile to ws[s][batch][m][n], and
 // gemm_split_reduce adds the slabs in index order.  For skinny products (few output tiles, long K:
 // the projections of a 128-token prefill) this is what puts every CU to work.
-template <typename T, int B_NK, int BM, int BN, int NT, bool SPLIT>
-__global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p, int tiles_m, int tiles_n, int remap, int nsplit, int kt_per, float* __restrict__ ws) {
+template <typename T, int B_NK, int BM, int BN, int NT, bool SPLIT, bool RAGGED = false>
+__global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p_in, int tiles_m, int tiles_n, int remap, int nsplit, int kt_per, float* __restrict__ ws) {
   extern __shared__ u32x4 lds[];
   constexpr int BK = Elt<T>::BK;
   constexpr int WM = BM / (NT / 128), WN = BN / 2, MI = WM / 32, NJ = WN / 32;
@@ -300,6 +309,9 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p, int tiles_m, int tile
   const int batch = bid / tpb;
   const int t_in = bid - batch * tpb;
   const int m0 = (t_in / tiles_n) * BM, n0 = (t_in % tiles_n) * BN;
+  // p: the problem as this tile sees it -- with RAGGED, M counts the rows of this tile that exist
+  MMArgs p = p_in;
+  if (RAGGED) p.M = min(BM, p_in.M - m0);
   const int kt0 = SPLIT ? slab * kt_per : 0;
   const size_t k_off = (size_t)kt0 * BK;
   const T* __restrict__ A = static_cast<const T*>(p.a) + (size_t)batch * p.a_bs + (size_t)m0 * p.a_rs + k_off;
@@ -322,39 +334,40 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p, int tiles_m, int tile
   Staged<BM, NT> r0, r1;
   u32x4* lds0 = lds;
   u32x4* lds1 = lds + STAGE;
-  load_tiles<T, B_NK, BM, BN, NT>(A, B, p, 0, tid, r0);
-  if (KT > 1) load_tiles<T, B_NK, BM, BN, NT>(A, B, p, 1, tid, r1);
+  load_tiles<T, B_NK, BM, BN, NT, RAGGED>(A, B, p, 0, tid, r0);
+  if (KT > 1) load_tiles<T, B_NK, BM, BN, NT, RAGGED>(A, B, p, 1, tid, r1);
   store_tiles<T, B_NK, BM, BN, NT, -1>(lds0, tid, r0);
   __syncthreads();
   int kt = 0;
   // steady state: both phases store and load unconditionally (tiles kt+2 and kt+3 exist)
   for (; kt + 3 < KT; kt += 2) {
     // stage 1 was last read in the previous odd phase, a barrier ago
-    k_phase<T, B_NK, BM, BN, NT, MI, NJ, true, 1>(A, B, p, lds0, lds1, true, r1, kt + 2, r0, tid, lane, wm, wn, acc);
+    k_phase<T, B_NK, BM, BN, NT, MI, NJ, true, 1, RAGGED>(A, B, p, lds0, lds1, true, r1, kt + 2, r0, tid, lane, wm, wn, acc);
     __syncthreads();
-    k_phase<T, B_NK, BM, BN, NT, MI, NJ, true, 1>(A, B, p, lds1, lds0, true, r0, kt + 3, r1, tid, lane, wm, wn, acc);
+    k_phase<T, B_NK, BM, BN, NT, MI, NJ, true, 1, RAGGED>(A, B, p, lds1, lds0, true, r0, kt + 3, r1, tid, lane, wm, wn, acc);
     __syncthreads();
   }
   // the last two or three tiles: tile kt+2, if there is one, still has to be fetched (past the end
   // the last tile is loaded again and never stored)
   for (; kt + 1 < KT; kt += 2) {
-    k_phase<T, B_NK, BM, BN, NT, MI, NJ, true, 1>(A, B, p, lds0, lds1, true, r1, min(kt + 2, KT - 1), r0, tid, lane, wm, wn, acc);
+    k_phase<T, B_NK, BM, BN, NT, MI, NJ, true, 1, RAGGED>(A, B, p, lds0, lds1, true, r1, min(kt + 2, KT - 1), r0, tid, lane, wm, wn, acc);
     __syncthreads();
-    k_phase<T, B_NK, BM, BN, NT, MI, NJ, false, 2>(A, B, p, lds1, lds0, kt + 2 < KT, r0, 0, r1, tid, lane, wm, wn, acc);
+    k_phase<T, B_NK, BM, BN, NT, MI, NJ, false, 2, RAGGED>(A, B, p, lds1, lds0, kt + 2 < KT, r0, 0, r1, tid, lane, wm, wn, acc);
     __syncthreads();
   }
-  if (kt < KT) k_phase<T, B_NK, BM, BN, NT, MI, NJ, false, 0>(A, B, p, lds0, lds1, false, r1, 0, r0, tid, lane, wm, wn, acc);  // odd tile count: the last tile
+  if (kt < KT) k_phase<T, B_NK, BM, BN, NT, MI, NJ, false, 0, RAGGED>(A, B, p, lds0, lds1, false, r1, 0, r0, tid, lane, wm, wn, acc);  // odd tile count: the last tile
 
   // accumulator register r of lane l: row (r/4)*8 + (l/32)*4 + r%4, column l%32
   if (SPLIT) {
-    float* __restrict__ W = ws + ((size_t)slab * (gridDim.x / (nsplit * tpb)) + batch) * (size_t)p.M * p.N + (size_t)m0 * p.N + n0;
+    float* __restrict__ W = ws + ((size_t)slab * (gridDim.x / (nsplit * tpb)) + batch) * (size_t)p_in.M * p.N + (size_t)m0 * p.N + n0;
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         float* Wt = W + (size_t)(wm + i * 32 + (lane >> 5) * 4) * p.N + wn + j * 32 + (lane & 31);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) Wt[(size_t)((r >> 2) * 8 + (r & 3)) * p.N] = acc[i][j][r];
+        for (int r = 0; r < 16; ++r)
+          if (!RAGGED || wm + i * 32 + (lane >> 5) * 4 + (r >> 2) * 8 + (r & 3) < p.M) Wt[(size_t)((r >> 2) * 8 + (r & 3)) * p.N] = acc[i][j][r];
       }
   } else {
     T* __restrict__ C = static_cast<T*>(p.c) + (size_t)batch * p.c_bs + (size_t)m0 * p.N + n0;
@@ -364,7 +377,8 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p, int tiles_m, int tile
       for (int j = 0; j < NJ; ++j) {
         T* Ct = C + (size_t)(wm + i * 32 + (lane >> 5) * 4) * p.N + wn + j * 32 + (lane & 31);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) Ct[(size_t)((r >> 2) * 8 + (r & 3)) * p.N] = (T)acc[i][j][r];
+        for (int r = 0; r < 16; ++r)
+          if (!RAGGED || wm + i * 32 + (lane >> 5) * 4 + (r >> 2) * 8 + (r & 3) < p.M) Ct[(size_t)((r >> 2) * 8 + (r & 3)) * p.N] = (T)acc[i][j][r];
       }
   }
 }
@@ -504,18 +518,18 @@ __global__ void __launch_bounds__(256) gemm_split_reduce(const float* __restrict
   o[3] = (T)s.w;
 }
 
-template <typename T, int B_NK, int BM, int BN, int NT, bool SPLIT>
+template <typename T, int B_NK, int BM, int BN, int NT, bool SPLIT, bool RAGGED = false>
 hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch, int nsplit, float* ws) {
   constexpr int LDS_BYTES = 2 * (BM + BN) * CHUNKS * 16;
   constexpr int BK = Elt<T>::BK;
   static bool configured = false;
-  auto kernel = gemm_tiled<T, B_NK, BM, BN, NT, SPLIT>;
+  auto kernel = gemm_tiled<T, B_NK, BM, BN, NT, SPLIT, RAGGED>;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if (e != hipSuccess) return e;
     configured = true;
   }
-  const int tiles_m = p.M / BM, tiles_n = p.N / BN;
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = p.N / BN;
   const int kt = p.K / BK, kt_per = SPLIT ? (kt + nsplit - 1) / nsplit : kt;
   if (SPLIT) nsplit = (kt + kt_per - 1) / kt_per;  // no empty slab
   const size_t total = batch * (size_t)tiles_m * tiles_n * (SPLIT ? nsplit : 1);
@@ -555,11 +569,13 @@ hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int s
     case 0:
       return getenv("UGHIP_GEMM_4WAVES") ? launch<T, B_NK, 256, 128, 256, SPLIT>(stream, p, batch, nsplit, ws)
                                          : launch<T, B_NK, 256, 128, 512, SPLIT>(stream, p, batch, nsplit, ws);
-    case 1: return launch<T, B_NK, 128, 128, 256, SPLIT>(stream, p, batch, nsplit, ws);
+    case 1:
+      return p.M % 128 ? launch<T, B_NK, 128, 128, 256, SPLIT, true>(stream, p, batch, nsplit, ws) : launch<T, B_NK, 128, 128, 256, SPLIT>(stream, p, batch, nsplit, ws);
     case 3:
       if constexpr (sizeof(T) == 2 && B_NK == 1 && !SPLIT) return launch_dma256<T>(stream, p, batch);
       [[fallthrough]];
-    default: return launch<T, B_NK, 128, 64, 256, SPLIT>(stream, p, batch, nsplit, ws);
+    default:
+      return p.M % 128 ? launch<T, B_NK, 128, 64, 256, SPLIT, true>(stream, p, batch, nsplit, ws) : launch<T, B_NK, 128, 64, 256, SPLIT>(stream, p, batch, nsplit, ws);
   }
 }
 
@@ -576,15 +592,16 @@ int pick_shape(const MMArgs& p, size_t batch, int dtype) {
   if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
     const int s = atoi(e);
     if (s == 3 && can3) return 3;
-    if (s >= 0 && s < 3 && p.M % kShapes[s][0] == 0 && p.N % kShapes[s][1] == 0) return s;
+    if (s >= 0 && s < 3 && (p.M % kShapes[s][0] == 0 || kShapes[s][0] == 128) && p.N % kShapes[s][1] == 0) return s;
   }
   // half the LDS traffic per flop of 256 x 128, once it alone gives every CU a workgroup
   if (can3 && batch * (size_t)(p.M / 256) * (size_t)(p.N / 256) >= 256) return 3;
   int best = -1;
   size_t best_tiles = 0;
   for (int s = 0; s < 3; ++s) {
-    if (p.M % kShapes[s][0] || p.N % kShapes[s][1]) continue;
-    const size_t tiles = batch * (size_t)(p.M / kShapes[s][0]) * (size_t)(p.N / kShapes[s][1]);
+    // the 128-row tiles also take an lhs whose last tile is partly empty (any M >= 9: fewer rows are the GEMV kernels' job)
+    if ((p.M % kShapes[s][0] && kShapes[s][0] != 128) || p.N % kShapes[s][1]) continue;
+    const size_t tiles = batch * (size_t)((p.M + kShapes[s][0] - 1) / kShapes[s][0]) * (size_t)(p.N / kShapes[s][1]);
     if (tiles >= 256) return s;
     if (tiles > best_tiles) best = s, best_tiles = tiles;
   }
@@ -596,7 +613,7 @@ int pick_shape(const MMArgs& p, size_t batch, int dtype) {
 int pick_split(int dtype, const MMArgs& p, size_t batch, int shape) {
   if (const char* e = getenv("UGHIP_GEMM_SPLIT")) return std::max(1, atoi(e));  // tuning aid
   const int bk = dtype == UGHIP_F32 ? 32 : 64;
-  const size_t tiles = batch * (size_t)(p.M / kShapes[shape][0]) * (size_t)(p.N / kShapes[shape][1]);
+  const size_t tiles = batch * (size_t)((p.M + kShapes[shape][0] - 1) / kShapes[shape][0]) * (size_t)(p.N / kShapes[shape][1]);
   const int kt = p.K / bk;
   if (tiles >= 128 || kt < 8) return 1;
   // three workgroups per CU: measured on the projections of a 128-token prefill, short slabs overlap
@@ -621,7 +638,7 @@ bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf1
   if (!aligned16(p.a) || !aligned16(p.b) || !aligned16(p.c)) return false;
   const int s = pick_shape(p, batch, dtype);
   if (s < 0) return false;
-  return batch * (size_t)(p.M / kShapes[s][0]) * (size_t)(p.N / kShapes[s][1]) < (1u << 24);
+  return batch * (size_t)((p.M + kShapes[s][0] - 1) / kShapes[s][0]) * (size_t)(p.N / kShapes[s][1]) < (1u << 24);
 }
 
 size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch) {
