@@ -115,6 +115,24 @@ def test_strategy_selection(cpu):
     src, info = k[1].hip_code(k[0])
     assert info["strategy"] == "grid_reduce" and info["grid_dim"] >= 256 and info["scratch_bytes"] > 0
     rtc_ok(src)
+    # its first stage streams the operands once, with loads that do not claim cache lines; nothing else does
+    first, fin = src.split('extern "C" __global__')[1:]
+    assert first.count("__builtin_nontemporal_load(") == 3 and "__builtin_nontemporal_load" not in fin
+    for n, kk in kernels_of(cases.softmax((4096, 1024)), cpu):
+        assert "__builtin_nontemporal_load" not in kk.hip_code(n)[0]
+
+
+@pytest.mark.parametrize("dtype", [ug_amd.F32, ug_amd.I32, ug_amd.I64])
+def test_grid_reduce_compiles_for_every_accumulator_type(cpu, dtype):
+    """Cooperative reductions exist for 32- and 64-bit accumulators (a 16-bit sum depends on its order too much to
+    be split; those kernels keep one thread per output)."""
+    def build(dev):
+        # only scheduled and lowered here; narrow as in config 2: a reduce keeps its dim at full length (lazy_buffer.rs:453-467)
+        return LB.copy(np.zeros(1 << 22, np.float32), (1 << 22,), dev).cast(dtype).reduce("max", 0).narrow(0, 0, 1)
+    ks = kernels_of(build, cpu)
+    src, info = ks[-1][1].hip_code("wide_max")
+    assert info["strategy"] == "grid_reduce" and "__builtin_nontemporal_load(" in src
+    rtc_ok(src)
 
 
 def test_gpu_style_ssa_is_translated_literally():
