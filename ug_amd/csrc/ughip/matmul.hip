@@ -183,8 +183,9 @@ __global__ void __launch_bounds__(256) gemv_nt(MMArgs p) {
     constexpr int stride = 64 * VE * KS;
     int k = (ks * 64 + lane) * VE;
     for (; k + 3 * stride < p.K; k += 4 * stride) {
-      const V w0 = *reinterpret_cast<const V*>(W + k), w1 = *reinterpret_cast<const V*>(W + k + stride);
-      const V w2 = *reinterpret_cast<const V*>(W + k + 2 * stride), w3 = *reinterpret_cast<const V*>(W + k + 3 * stride);
+      // every matrix element is read once per launch: loads that do not claim cache lines
+      const V w0 = __builtin_nontemporal_load(reinterpret_cast<const V*>(W + k)), w1 = __builtin_nontemporal_load(reinterpret_cast<const V*>(W + k + stride));
+      const V w2 = __builtin_nontemporal_load(reinterpret_cast<const V*>(W + k + 2 * stride)), w3 = __builtin_nontemporal_load(reinterpret_cast<const V*>(W + k + 3 * stride));
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         if (r < p.M) {
