@@ -172,10 +172,11 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
     if (tid < lpk) reinterpret_cast<float4*>(k_out)[row + tid] = reinterpret_cast<const float4*>(kn)[tid];
     else reinterpret_cast<float4*>(v_out)[row + tid - lpk] = reinterpret_cast<const float4*>(vn)[tid - lpk];
   }
-  // One pass over the keys, four key rows and four value rows per lane group in flight.  Every wave
-  // keeps a running maximum m_run, the sum l_run of exp(score - m_run) and the weighted value rows
-  // acc of the keys it has seen (rescaled when the maximum moves); the 16 waves are merged once at
-  // the end.  Scores and probabilities never leave registers.
+  // One pass over the keys, four key rows and four value rows per lane group in flight.  Every lane
+  // group keeps a running maximum m_run, the sum l_run of exp(score - m_run) and the weighted value
+  // rows acc of the keys it has seen (rescaled when the maximum moves): inside the loop nothing
+  // crosses the group, so a long cache costs arithmetic, not exchanges.  The groups of a wave and
+  // then the 16 waves are merged once at the end.  Scores and probabilities never leave registers.
   float m_run = -INFINITY, l_run = 0.f;
   att_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   auto load_rows = [&](const float4* base, int j0, att_f32x4 (&r)[4]) {
@@ -210,20 +211,20 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
       p[u] = j0 + u * kpb + slot < s ? pu * scale : -INFINITY;
       mt = fmaxf(mt, p[u]);
     }
-    const float m_new = fmaxf(m_run, wave_max(mt));
-    if (m_new == -INFINITY) return;  // this wave has not seen a key yet (wave-uniform)
-    const float alpha = expf(m_run - m_new);  // 0 on the wave's first keys (m_run = -inf)
+    const float m_new = fmaxf(m_run, mt);
+    // a group that has not seen a key yet keeps its zeros (exp(-inf - -inf) would be NaN)
+    const float alpha = m_new == -INFINITY ? 0.f : expf(m_run - m_new);  // 0 on the group's first keys (m_run = -inf)
     acc *= alpha;
     float lt = 0.f;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int j = j0 + u * kpb + slot;
-      const float e = expf(p[u] - m_new);  // 0 for the keys past the end
+      const float e = m_new == -INFINITY ? 0.f : expf(p[u] - m_new);  // 0 for the keys past the end
       const att_f32x4 vv = j == j_new ? reinterpret_cast<const att_f32x4*>(vn)[c4] : vr[u];
       acc += e * vv;
-      if (c4 == 0) lt += e;  // a key's lanes all hold its e: count it once
+      lt += e;  // the lanes of a group all hold the same e and the same sums
     }
-    l_run = l_run * alpha + wave_sum(lt);
+    l_run = l_run * alpha + lt;
     m_run = m_new;
   };
   trip(0, kpre, vpre);
@@ -233,8 +234,17 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
     load_rows(v4, j0, vr);
     trip(j0, kr, vr);
   }
-  // the slots of one wave (lanes lpk apart) ...
+  // the groups of one wave (lanes lpk apart): bring them to the wave's maximum, then add up ...
+  {
+    float m_w = m_run;
+    for (int o = lpk; o < 64; o <<= 1) m_w = fmaxf(m_w, __shfl_xor(m_w, o, 64));
+    const float f = m_run == -INFINITY ? 0.f : expf(m_run - m_w);  // m_w is finite wherever m_run is
+    acc *= f;
+    l_run *= f;
+    m_run = m_w;
+  }
   for (int o = lpk; o < 64; o <<= 1) {
+    l_run += __shfl_xor(l_run, o, 64);
     acc.x += __shfl_xor(acc.x, o, 64);
     acc.y += __shfl_xor(acc.y, o, 64);
     acc.z += __shfl_xor(acc.z, o, 64);
