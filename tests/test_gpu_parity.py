@@ -729,6 +729,36 @@ def test_llama_bf16_matrices_are_the_rounded_f32_model(hip, cpu, hip_ops, cpu_op
     np.testing.assert_allclose(wide[1]["margins"], st_c["margins"], rtol=1e-2, atol=1e-7)
 
 
+@pytest.mark.parametrize("b,nh,nkv,s,d", [(1, 8, 2, 1, 64), (1, 8, 2, 5, 64), (2, 4, 4, 700, 64), (1, 4, 1, 3000, 128), (1, 2, 2, 300, 32)])
+def test_attention_decode_key_ranges(hip, hip_ops, b, nh, nkv, s, d):
+    """The keys of a head split over 2, 8 or 64 workgroups and merged (what caches of 1024 rows and more get by
+    themselves), ranges without a key included: the single-workgroup result to rounding, and float64."""
+    import os
+    print("attention decode ranges", (b, nh, nkv, s, d), flush=True)
+    q, k, v = rng.normal(151, b * nh * d), rng.normal(152, b * nkv * s * d), rng.normal(153, b * nkv * s * d)
+    scale = float(np.float32(d) ** np.float32(-0.5))
+
+    def run(n):
+        os.environ["UGHIP_ATT_SPLIT"] = str(n)
+        try:
+            return hip_ops.attention_decode(LB.copy(q, (b, nh, 1, d), hip), LB.copy(k, (b, nkv, s, d), hip), LB.copy(v, (b, nkv, s, d), hip), scale).data_vec()
+        finally:
+            del os.environ["UGHIP_ATT_SPLIT"]
+
+    one = run(1)
+    q6, k6, v6 = q.reshape(b, nh, d).astype(np.float64), k.reshape(b, nkv, s, d).astype(np.float64), v.reshape(b, nkv, s, d).astype(np.float64)
+    sc = np.einsum("bhd,bhsd->bhs", q6, np.repeat(k6, nh // nkv, 1)) * scale
+    p = np.exp(sc - sc.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    truth = np.einsum("bhs,bhsd->bhd", p, np.repeat(v6, nh // nkv, 1)).ravel()
+    tol = 1e-5 * np.abs(truth).max() + 1e-5 * np.abs(truth)
+    assert np.all(np.abs(one - truth) <= tol)
+    for n in (2, 8, 64):
+        got = run(n)
+        assert np.all(np.abs(got - truth) <= tol), n
+        np.testing.assert_allclose(got, one, rtol=2e-5, atol=2e-6 * np.abs(truth).max())
+
+
 def _rope_tables(dev, hd, max_pos=64):
     cfg = ug_amd.LlamaConfig(hidden_size=hd * 4, num_attention_heads=4, num_key_value_heads=2, max_position_embeddings=max_pos)
     cos, sin = ug_amd.llama.rope_tables(dev, cfg)
@@ -1159,10 +1189,12 @@ def test_fused_projections_fall_back_for_several_rows(hip, cpu, hip_ops, cpu_ops
         np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-6)
 
 
-def test_packed_rows_feed_cache_and_attention(hip, hip_ops):
+@pytest.mark.parametrize("cap,length", [(32, 5), (2048, 1500)])
+def test_packed_rows_feed_cache_and_attention(hip, hip_ops, cap, length):
     """q | k | v side by side in one buffer, read in place by kv_append and attention_cached: same
-    results as the three parts handed over separately."""
-    nh, nkv, d, cap, length = 8, 2, 64, 32, 5
+    results as the three parts handed over separately (a short cache, and one long enough for the keys
+    of a head to be split over several workgroups)."""
+    nh, nkv, d = 8, 2, 64
     nq, nk = nh * d, nkv * d
     row = nq + 2 * nk
     qkv = rng.normal(105, row)

@@ -107,7 +107,7 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
                                                                        size_t q_batch_stride, int d, float scale, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                                                        const int* __restrict__ pos, size_t table_len, int interleaved,
                                                                        const float* __restrict__ k_new, const float* __restrict__ v_new, float* __restrict__ k_out,
-                                                                       float* __restrict__ v_out) {
+                                                                       float* __restrict__ v_out, int nsplit, float* __restrict__ part) {
   __shared__ __attribute__((aligned(16))) float sc[ATT_WAVES * 64 * 4];  // one float4 per lane slot of every wave for the final merge
   __shared__ float wave_m[ATT_WAVES], wave_l[ATT_WAVES];
   __shared__ __attribute__((aligned(16))) float qs[256];
@@ -116,7 +116,13 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
   const int tid = threadIdx.x;
   const int lpk = d >> 2, kpb = ATT_THREADS / lpk;  // lanes per key, keys per step
   const int c4 = tid % lpk, slot = tid / lpk;
-  const int bh = blockIdx.x, b = bh / nh, h = bh % nh, kvh = h / (nh / nkv);
+  // nsplit > 1 (long caches): nsplit workgroups share a head, each takes a range of keys [j_lo, j_hi)
+  // that is a whole number of loop trips and leaves its (maximum, sum, unnormalised row) in `part`
+  // for attention_merge_kernel; one workgroup streams about 100 GB/s, so 32 heads alone cannot keep
+  // up with a cache of thousands of rows.
+  const int bh = blockIdx.x / nsplit, split = blockIdx.x % nsplit, b = bh / nh, h = bh % nh, kvh = h / (nh / nkv);
+  const int chunk = nsplit == 1 ? s : (((s + nsplit - 1) / nsplit + 4 * kpb - 1) / (4 * kpb)) * (4 * kpb);
+  const int j_lo = min(s, split * chunk), j_hi = min(s, j_lo + chunk);
   const float* qh = q + (size_t)b * q_batch_stride + (size_t)h * d;  // q_batch_stride = nh * d unless q is part of a wider row
   const float4* q4 = reinterpret_cast<const float4*>(qh);
   const float4* k4 = reinterpret_cast<const float4*>(k + ((size_t)b * nkv + kvh) * kv_head_stride);
@@ -137,8 +143,8 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
   for (int u = 0; u < 4; ++u) {
     // unconditional loads (a branch here sends the arrays to scratch memory): rows this lane has
     // no use for are read as row 0 and ignored below
-    const int j = u * kpb + slot;
-    const size_t jj = j < s && j != j_new ? (size_t)j : 0;
+    const int j = j_lo + u * kpb + slot;
+    const size_t jj = j < j_hi && j != j_new ? (size_t)j : 0;
     kpre[u] = reinterpret_cast<const att_f32x4*>(k4)[jj * lpk + c4];
     vpre[u] = reinterpret_cast<const att_f32x4*>(v4)[jj * lpk + c4];
   }
@@ -167,7 +173,7 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
     if (k_new) __syncthreads();
     qv = q4[c4];
   }
-  if (k_out && h % (nh / nkv) == 0 && tid < 2 * lpk) {
+  if (k_out && h % (nh / nkv) == 0 && split == 0 && tid < 2 * lpk) {
     const size_t row = (((size_t)b * nkv + kvh) * kv_head_stride + (size_t)(s - 1) * d) / 4;
     if (tid < lpk) reinterpret_cast<float4*>(k_out)[row + tid] = reinterpret_cast<const float4*>(kn)[tid];
     else reinterpret_cast<float4*>(v_out)[row + tid - lpk] = reinterpret_cast<const float4*>(vn)[tid - lpk];
@@ -183,7 +189,7 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int j = j0 + u * kpb + slot;
-      const size_t jj = j < s && j != j_new ? (size_t)j : 0;
+      const size_t jj = j < j_hi && j != j_new ? (size_t)j : 0;
       r[u] = reinterpret_cast<const att_f32x4*>(base)[jj * lpk + c4];
     }
   };
@@ -208,7 +214,7 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
       } else {
         for (int o = lpk >> 1; o > 0; o >>= 1) pu += __shfl_xor(pu, o, 64);
       }
-      p[u] = j0 + u * kpb + slot < s ? pu * scale : -INFINITY;
+      p[u] = j0 + u * kpb + slot < j_hi ? pu * scale : -INFINITY;
       mt = fmaxf(mt, p[u]);
     }
     const float m_new = fmaxf(m_run, mt);
@@ -227,8 +233,8 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
     l_run = l_run * alpha + lt;
     m_run = m_new;
   };
-  trip(0, kpre, vpre);
-  for (int j0 = 4 * kpb; j0 < s; j0 += 4 * kpb) {
+  trip(j_lo, kpre, vpre);
+  for (int j0 = j_lo + 4 * kpb; j0 < j_hi; j0 += 4 * kpb) {
     att_f32x4 kr[4], vr[4];
     load_rows(k4, j0, kr);
     load_rows(v4, j0, vr);
@@ -260,18 +266,45 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
   }
   __syncthreads();
   if (tid < lpk) {
-    float mx = wave_m[0];  // key 0 belongs to wave 0: finite unless the data is not
+    float mx = wave_m[0];  // the first key of the range belongs to wave 0: finite unless the range is empty or the data is not
 #pragma unroll
     for (int w = 1; w < ATT_WAVES; ++w) mx = fmaxf(mx, wave_m[w]);
     att_f32x4 o = {0.f, 0.f, 0.f, 0.f};
     float sum = 0.f;
     for (int w = 0; w < ATT_WAVES; ++w) {
-      const float f = expf(wave_m[w] - mx);  // 0 for a wave without keys
+      const float f = wave_m[w] == -INFINITY ? 0.f : expf(wave_m[w] - mx);  // 0 for a wave without keys
       o += f * red[w * 64 + tid];
       sum += f * wave_l[w];
     }
-    reinterpret_cast<att_f32x4*>(dst + (size_t)bh * d)[tid] = o / sum;
+    if (nsplit == 1) {
+      reinterpret_cast<att_f32x4*>(dst + (size_t)bh * d)[tid] = o / sum;
+    } else {
+      float* pp = part + ((size_t)bh * nsplit + split) * (size_t)(d + 4);
+      if (tid == 0) {
+        pp[0] = mx;
+        pp[1] = sum;
+      }
+      reinterpret_cast<att_f32x4*>(pp + 4)[tid] = o;
+    }
   }
+}
+
+// The ranges of one head put together: out = sum_i exp(m_i - M) o_i / sum_i exp(m_i - M) l_i, in range order.
+__global__ void __launch_bounds__(64) attention_merge_kernel(const float* __restrict__ part, float* __restrict__ dst, int nsplit, int d) {
+  const int bh = blockIdx.x, t = threadIdx.x;
+  if (t >= (d >> 2)) return;
+  const float* pp = part + (size_t)bh * nsplit * (size_t)(d + 4);
+  float mx = -INFINITY;
+  for (int i = 0; i < nsplit; ++i) mx = fmaxf(mx, pp[(size_t)i * (d + 4)]);
+  att_f32x4 o = {0.f, 0.f, 0.f, 0.f};
+  float sum = 0.f;
+  for (int i = 0; i < nsplit; ++i) {
+    const float* pi = pp + (size_t)i * (d + 4);
+    const float f = pi[0] == -INFINITY ? 0.f : expf(pi[0] - mx);  // 0 for a range without keys
+    o += f * reinterpret_cast<const att_f32x4*>(pi + 4)[t];
+    sum += f * pi[1];
+  }
+  reinterpret_cast<att_f32x4*>(dst + (size_t)bh * d)[t] = o / sum;
 }
 
 // ---- cache append for one new position ------------------------------------------------------------
@@ -675,6 +708,30 @@ int ughip_attention_decode(ughip_device* dev, const ughip_slice* q, const ughip_
 
 namespace {
 // One query position per head against s keys of caches whose heads are cap rows apart.
+// Key ranges per head for `s` keys: one below 1024 (a merge launch costs what ~800 keys cost), then enough
+// ranges to give every CU a workgroup.  UGHIP_ATT_SPLIT forces a count (tests, tuning).
+int decode_ranges(size_t s, size_t heads) {
+  int n = s >= 1024 ? (int)std::max<size_t>(1, std::min<size_t>(8, 256 / std::max<size_t>(heads, 1))) : 1;
+  if (const char* e = getenv("UGHIP_ATT_SPLIT")) n = atoi(e);
+  return std::max(1, std::min(n, 64));
+}
+
+// Scratch for the partial rows, grown on demand like the matmul's.
+int decode_scratch(ughip_device* dev, size_t bytes, float** out) {
+  if (bytes > dev->att_ws_bytes) {
+    std::lock_guard<std::mutex> g(dev->mu);
+    UGHIP_HIPCHK(hipStreamSynchronize(dev->stream));  // earlier launches may still read the old block
+    if (dev->att_ws) hipFree(dev->att_ws);
+    dev->att_ws = nullptr;
+    dev->att_ws_bytes = 0;
+    const size_t want = std::max<size_t>(bytes, (size_t)1 << 20);
+    UGHIP_HIPCHK(hipMalloc(&dev->att_ws, want));
+    dev->att_ws_bytes = want;
+  }
+  *out = static_cast<float*>(dev->att_ws);
+  return UGHIP_OK;
+}
+
 int attention_decode_launch(ughip_device* dev, const ughip_slice* q, size_t q_offset, size_t q_row_stride, const ughip_slice* k, const ughip_slice* v,
                             ughip_slice* dst, size_t b, size_t n_heads, size_t n_kv_heads, size_t s, size_t cap, size_t d, float scale, const ughip_slice* cos,
                             const ughip_slice* sin, const ughip_slice* pos, int interleaved) {
@@ -699,12 +756,20 @@ int attention_decode_launch(ughip_device* dev, const ughip_slice* q, size_t q_of
   if (b * n_heads == 0) return UGHIP_OK;
   if (b * n_heads > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "attention_decode: too many heads");
   if (int rc = device_activate(dev)) return rc;
-  attention_decode_kernel<<<(unsigned)(b * n_heads), ATT_THREADS, 0, dev->stream>>>(
+  const int nsplit = decode_ranges(s, b * n_heads);
+  float* part = nullptr;
+  if (nsplit > 1)
+    if (int rc = decode_scratch(dev, b * n_heads * nsplit * (d + 4) * sizeof(float), &part)) return rc;
+  attention_decode_kernel<<<(unsigned)(b * n_heads * nsplit), ATT_THREADS, 0, dev->stream>>>(
       static_cast<const float*>(q->ptr) + q_offset, static_cast<const float*>(k->ptr), static_cast<const float*>(v->ptr), static_cast<float*>(dst->ptr),
       (int)n_heads, (int)n_kv_heads, (int)s, cap * d, q_row_stride, (int)d, scale, rope ? static_cast<const float*>(cos->ptr) : nullptr,
       rope ? static_cast<const float*>(sin->ptr) : nullptr, rope ? static_cast<const int*>(pos->ptr) : nullptr,
-      rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved, nullptr, nullptr, nullptr, nullptr);
+      rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved, nullptr, nullptr, nullptr, nullptr, nsplit, part);
   UGHIP_HIPCHK(hipGetLastError());
+  if (nsplit > 1) {
+    attention_merge_kernel<<<(unsigned)(b * n_heads), 64, 0, dev->stream>>>(part, static_cast<float*>(dst->ptr), nsplit, (int)d);
+    UGHIP_HIPCHK(hipGetLastError());
+  }
   return UGHIP_OK;
 }
 }  // namespace
@@ -735,13 +800,21 @@ int ughip_attention_step(ughip_device* dev, const ughip_slice* qkv, size_t row_s
   if (b * n_heads > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "attention_step: too many heads");
   if (int rc = device_activate(dev)) return rc;
   const float* base = static_cast<const float*>(qkv->ptr);
-  attention_decode_kernel<<<(unsigned)(b * n_heads), ATT_THREADS, 0, dev->stream>>>(
+  const int nsplit = decode_ranges(s, b * n_heads);
+  float* part = nullptr;
+  if (nsplit > 1)
+    if (int rc = decode_scratch(dev, b * n_heads * nsplit * (d + 4) * sizeof(float), &part)) return rc;
+  attention_decode_kernel<<<(unsigned)(b * n_heads * nsplit), ATT_THREADS, 0, dev->stream>>>(
       base + q_offset, static_cast<const float*>(kcache->ptr), static_cast<const float*>(vcache->ptr), static_cast<float*>(dst->ptr), (int)n_heads,
       (int)n_kv_heads, (int)s, cap * d, row_stride, (int)d, scale, rope ? static_cast<const float*>(cos->ptr) : nullptr,
       rope ? static_cast<const float*>(sin->ptr) : nullptr, rope ? static_cast<const int*>(pos->ptr) : nullptr,
       rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved, base + k_offset, base + v_offset, static_cast<float*>(kcache->ptr),
-      static_cast<float*>(vcache->ptr));
+      static_cast<float*>(vcache->ptr), nsplit, part);
   UGHIP_HIPCHK(hipGetLastError());
+  if (nsplit > 1) {
+    attention_merge_kernel<<<(unsigned)(b * n_heads), 64, 0, dev->stream>>>(part, static_cast<float*>(dst->ptr), nsplit, (int)d);
+    UGHIP_HIPCHK(hipGetLastError());
+  }
   return UGHIP_OK;
 }
 

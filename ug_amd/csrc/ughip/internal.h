@@ -32,6 +32,9 @@ struct ughip_device {
   // device's one stream, freed with the device.
   void* gemm_ws = nullptr;
   size_t gemm_ws_bytes = 0;
+  // Partial rows of single-query attention over a long cache (one per head and key range); same life cycle.
+  void* att_ws = nullptr;
+  size_t att_ws_bytes = 0;
 };
 
 struct ughip_slice {
