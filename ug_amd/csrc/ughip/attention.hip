@@ -732,6 +732,27 @@ int decode_scratch(ughip_device* dev, size_t bytes, float** out) {
   return UGHIP_OK;
 }
 
+// The launch both entry points share: one workgroup per head and key range, then the merge when a head has several.
+int decode_run(ughip_device* dev, size_t heads, const float* q, const float* k, const float* v, float* dst, size_t n_heads, size_t n_kv_heads, size_t s,
+               size_t kv_head_stride, size_t q_batch_stride, size_t d, float scale, const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos,
+               int interleaved, const float* k_new, const float* v_new, float* k_out, float* v_out) {
+  const bool rope = cos != nullptr;
+  const int nsplit = decode_ranges(s, heads);
+  float* part = nullptr;
+  if (nsplit > 1)
+    if (int rc = decode_scratch(dev, heads * nsplit * (d + 4) * sizeof(float), &part)) return rc;
+  attention_decode_kernel<<<(unsigned)(heads * nsplit), ATT_THREADS, 0, dev->stream>>>(
+      q, k, v, dst, (int)n_heads, (int)n_kv_heads, (int)s, kv_head_stride, q_batch_stride, (int)d, scale, rope ? static_cast<const float*>(cos->ptr) : nullptr,
+      rope ? static_cast<const float*>(sin->ptr) : nullptr, rope ? static_cast<const int*>(pos->ptr) : nullptr,
+      rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved, k_new, v_new, k_out, v_out, nsplit, part);
+  UGHIP_HIPCHK(hipGetLastError());
+  if (nsplit > 1) {
+    attention_merge_kernel<<<(unsigned)heads, 64, 0, dev->stream>>>(part, dst, nsplit, (int)d);
+    UGHIP_HIPCHK(hipGetLastError());
+  }
+  return UGHIP_OK;
+}
+
 int attention_decode_launch(ughip_device* dev, const ughip_slice* q, size_t q_offset, size_t q_row_stride, const ughip_slice* k, const ughip_slice* v,
                             ughip_slice* dst, size_t b, size_t n_heads, size_t n_kv_heads, size_t s, size_t cap, size_t d, float scale, const ughip_slice* cos,
                             const ughip_slice* sin, const ughip_slice* pos, int interleaved) {
@@ -756,21 +777,9 @@ int attention_decode_launch(ughip_device* dev, const ughip_slice* q, size_t q_of
   if (b * n_heads == 0) return UGHIP_OK;
   if (b * n_heads > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "attention_decode: too many heads");
   if (int rc = device_activate(dev)) return rc;
-  const int nsplit = decode_ranges(s, b * n_heads);
-  float* part = nullptr;
-  if (nsplit > 1)
-    if (int rc = decode_scratch(dev, b * n_heads * nsplit * (d + 4) * sizeof(float), &part)) return rc;
-  attention_decode_kernel<<<(unsigned)(b * n_heads * nsplit), ATT_THREADS, 0, dev->stream>>>(
-      static_cast<const float*>(q->ptr) + q_offset, static_cast<const float*>(k->ptr), static_cast<const float*>(v->ptr), static_cast<float*>(dst->ptr),
-      (int)n_heads, (int)n_kv_heads, (int)s, cap * d, q_row_stride, (int)d, scale, rope ? static_cast<const float*>(cos->ptr) : nullptr,
-      rope ? static_cast<const float*>(sin->ptr) : nullptr, rope ? static_cast<const int*>(pos->ptr) : nullptr,
-      rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved, nullptr, nullptr, nullptr, nullptr, nsplit, part);
-  UGHIP_HIPCHK(hipGetLastError());
-  if (nsplit > 1) {
-    attention_merge_kernel<<<(unsigned)(b * n_heads), 64, 0, dev->stream>>>(part, static_cast<float*>(dst->ptr), nsplit, (int)d);
-    UGHIP_HIPCHK(hipGetLastError());
-  }
-  return UGHIP_OK;
+  return decode_run(dev, b * n_heads, static_cast<const float*>(q->ptr) + q_offset, static_cast<const float*>(k->ptr), static_cast<const float*>(v->ptr),
+                    static_cast<float*>(dst->ptr), n_heads, n_kv_heads, s, cap * d, q_row_stride, d, scale, rope ? cos : nullptr, rope ? sin : nullptr,
+                    rope ? pos : nullptr, interleaved, nullptr, nullptr, nullptr, nullptr);
 }
 }  // namespace
 
@@ -800,22 +809,9 @@ int ughip_attention_step(ughip_device* dev, const ughip_slice* qkv, size_t row_s
   if (b * n_heads > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "attention_step: too many heads");
   if (int rc = device_activate(dev)) return rc;
   const float* base = static_cast<const float*>(qkv->ptr);
-  const int nsplit = decode_ranges(s, b * n_heads);
-  float* part = nullptr;
-  if (nsplit > 1)
-    if (int rc = decode_scratch(dev, b * n_heads * nsplit * (d + 4) * sizeof(float), &part)) return rc;
-  attention_decode_kernel<<<(unsigned)(b * n_heads * nsplit), ATT_THREADS, 0, dev->stream>>>(
-      base + q_offset, static_cast<const float*>(kcache->ptr), static_cast<const float*>(vcache->ptr), static_cast<float*>(dst->ptr), (int)n_heads,
-      (int)n_kv_heads, (int)s, cap * d, row_stride, (int)d, scale, rope ? static_cast<const float*>(cos->ptr) : nullptr,
-      rope ? static_cast<const float*>(sin->ptr) : nullptr, rope ? static_cast<const int*>(pos->ptr) : nullptr,
-      rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved, base + k_offset, base + v_offset, static_cast<float*>(kcache->ptr),
-      static_cast<float*>(vcache->ptr), nsplit, part);
-  UGHIP_HIPCHK(hipGetLastError());
-  if (nsplit > 1) {
-    attention_merge_kernel<<<(unsigned)(b * n_heads), 64, 0, dev->stream>>>(part, static_cast<float*>(dst->ptr), nsplit, (int)d);
-    UGHIP_HIPCHK(hipGetLastError());
-  }
-  return UGHIP_OK;
+  return decode_run(dev, b * n_heads, base + q_offset, static_cast<const float*>(kcache->ptr), static_cast<const float*>(vcache->ptr), static_cast<float*>(dst->ptr),
+                    n_heads, n_kv_heads, s, cap * d, row_stride, d, scale, rope ? cos : nullptr, rope ? sin : nullptr, rope ? pos : nullptr, interleaved,
+                    base + k_offset, base + v_offset, static_cast<float*>(kcache->ptr), static_cast<float*>(vcache->ptr));
 }
 
 int ughip_attention_decode_rope(ughip_device* dev, const ughip_slice* q, const ughip_slice* k, const ughip_slice* v, ughip_slice* dst, size_t b,
