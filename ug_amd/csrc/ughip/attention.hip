@@ -721,7 +721,7 @@ int decode_scratch(ughip_device* dev, size_t bytes, float** out) {
   if (bytes > dev->att_ws_bytes) {
     std::lock_guard<std::mutex> g(dev->mu);
     UGHIP_HIPCHK(hipStreamSynchronize(dev->stream));  // earlier launches may still read the old block
-    if (dev->att_ws) hipFree(dev->att_ws);
+    if (dev->att_ws) (void)hipFree(dev->att_ws);
     dev->att_ws = nullptr;
     dev->att_ws_bytes = 0;
     const size_t want = std::max<size_t>(bytes, (size_t)1 << 20);

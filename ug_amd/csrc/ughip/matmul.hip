@@ -459,7 +459,7 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
     if (ws_bytes > dev->gemm_ws_bytes) {
       std::lock_guard<std::mutex> g(dev->mu);
       UGHIP_HIPCHK(hipStreamSynchronize(st));  // earlier launches may still read the old block
-      if (dev->gemm_ws) hipFree(dev->gemm_ws);
+      if (dev->gemm_ws) (void)hipFree(dev->gemm_ws);
       dev->gemm_ws = nullptr;
       dev->gemm_ws_bytes = 0;
       const size_t want = std::max<size_t>(ws_bytes, (size_t)32 << 20);
