@@ -219,8 +219,8 @@ int ughip_rtc_check(const char* source, const char* arch, size_t* code_size);
  * checkpoint stores them, where the reference widens them at load time,
  * ug-core/src/safetensors.rs:120-271).  The rhs is widened on its way into LDS, so the result is
  * bit for bit that of the F32 product on the widened values.  Built for an [n, k]-major rhs
- * (strides (1, k)) with n % 64 == 0, k % 32 == 0; other shapes are UGHIP_ERR_UNSUPPORTED
- * (convert the rhs with ughip_convert first). */
+ * (strides (1, k)) with k % 32 == 0; other layouts are UGHIP_ERR_UNSUPPORTED (convert the rhs
+ * with ughip_convert first). */
 int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs,
                  const ughip_slice* rhs, size_t b, size_t m, size_t n, size_t k, size_t rank,
                  const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset,

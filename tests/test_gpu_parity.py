@@ -305,15 +305,16 @@ def _raw_matmul(hip, dtype, a, w, rhs_nk):
     return out[:b * m * n].reshape(b, m, n)
 
 
-# N a whole multiple of a tile width and K a multiple of 32 (f32) / 64 (bf16) take the tuned MFMA kernel, with
-# any number of rows from 9 up (a last tile that hangs over the end of the lhs reads its last row again and
-# stores nothing for the rows that do not exist; split-K included: 100 x 2048 x 2048 is a prompt of 100 tokens);
-# neighbours one column off take the generic one.  All are held to the same bound, and a sentinel behind the
+# K a multiple of 32 (f32) / 64 (bf16) takes the tuned MFMA kernel, with any number of rows from 9 up and, for an
+# [n, k]-major rhs, any number of columns (a last tile that hangs over the end reads the last row again and
+# stores nothing for what does not exist; split-K included: 100 x 2048 x 2048 is a prompt of 100 tokens,
+# 128 x 32001 x 64 a vocabulary with one added token); a [k, n]-major rhs one column off takes the generic one.  All are held to the same bound, and a sentinel behind the
 # result checks that nothing is written past the last row.
 @pytest.mark.parametrize("rhs_nk", [False, True])
 @pytest.mark.parametrize("bmnk", [(2, 256, 128, 96), (1, 512, 384, 160), (3, 256, 256, 32), (1, 255, 128, 96), (1, 256, 129, 96),
                                   (1, 128, 128, 64), (2, 128, 64, 96), (1, 384, 192, 64), (40, 256, 128, 32), (32, 512, 64, 512),
-                                  (1, 100, 2048, 2048), (2, 300, 256, 64), (1, 37, 5632, 256), (3, 9, 64, 32), (1, 129, 128, 96)])
+                                  (1, 100, 2048, 2048), (2, 300, 256, 64), (1, 37, 5632, 256), (3, 9, 64, 32), (1, 129, 128, 96),
+                                  (1, 128, 1001, 256), (1, 37, 77, 64), (3, 200, 190, 32), (1, 128, 32001, 64)])
 def test_matmul_f32_tile_multiples(hip, bmnk, rhs_nk):
     b, m, n, k = bmnk
     print("matmul f32", bmnk, "rhs_nk", rhs_nk, flush=True)
@@ -328,7 +329,7 @@ def test_matmul_f32_tile_multiples(hip, bmnk, rhs_nk):
 @pytest.mark.parametrize("rhs_nk", [False, True])
 @pytest.mark.parametrize("bmnk", [(2, 256, 128, 192), (1, 512, 384, 64), (3, 256, 256, 320), (1, 256, 128, 96), (1, 248, 128, 128),
                                   (1, 128, 128, 64), (2, 128, 64, 128), (1, 384, 192, 192), (40, 256, 128, 64), (1, 100, 2048, 2048), (2, 300, 256, 64),
-                                  (3, 9, 64, 64)])
+                                  (3, 9, 64, 64), (1, 128, 1001, 256), (3, 200, 190, 64)])
 def test_matmul_bf16_tile_multiples(hip, bmnk, rhs_nk):
     b, m, n, k = bmnk
     print("matmul bf16", bmnk, "rhs_nk", rhs_nk, flush=True)
@@ -367,7 +368,7 @@ def test_matmul_16bit_256x256_tiles(hip, bmnk, dtype):
 
 
 @pytest.mark.parametrize("bmnk", [(1, 128, 2048, 2048), (1, 128, 256, 2048), (1, 256, 5632, 2048), (1, 128, 2048, 5632), (2, 512, 384, 96), (1, 1024, 1024, 32),
-                                  (1, 100, 2048, 2048), (2, 130, 128, 64), (1, 9, 64, 32)])
+                                  (1, 100, 2048, 2048), (2, 130, 128, 64), (1, 9, 64, 32), (1, 128, 1001, 256), (1, 37, 77, 64), (3, 200, 190, 32)])
 def test_matmul_f32_with_a_bf16_rhs(hip, bmnk):
     """An F32 product reading an [n, k]-major rhs stored as bf16 (split-K prefill shapes and plain ones):
     bit for bit the F32 product on the widened values."""
@@ -393,8 +394,8 @@ def test_matmul_f32_with_a_bf16_rhs_limits(hip):
     lhs = ((1, m, k), (m * k, k, 1), 0)
     with pytest.raises(ug_amd.UgError, match=r"\[n, k\]-major"):      # [k, n]-major rhs
         hip.matmul(dst, sa, sw, (1, m, n, k), lhs, ((1, k, n), (k * n, n, 1), 0))
-    with pytest.raises(ug_amd.UgError, match="multiples of 64, 32"):           # a column count no tile divides
-        hip.matmul(dst, sa, sw, (1, m, n - 1, k), lhs, ((1, k, n - 1), (k * (n - 1), 1, k), 0))
+    with pytest.raises(ug_amd.UgError, match="multiple of 32"):                # a k the tiles do not divide
+        hip.matmul(dst, sa, sw, (1, m, n, k - 8), ((1, m, k - 8), (m * (k - 8), k - 8, 1), 0), ((1, k - 8, n), ((k - 8) * n, 1, k - 8), 0))
     with pytest.raises(ug_amd.UgError, match="incorrect dtypes"):              # the other way round is not a thing
         hip.matmul(dst, sw, sa, (1, m, n, k), lhs, ((1, k, n), (k * n, 1, k), 0))
     hip.matmul(dst, sa, sw, (1, m, n, k), lhs, ((1, k, n), (k * n, 1, k), 0))

@@ -255,7 +255,7 @@ struct HipOps : Ops {
     const size_t rows = x.rank() ? x.elem_count() / x.dims().back() : 0;
     if (x.dtype() == DType::F32 && w.dtype() == DType::BF16 && rows == 1 && x.rank() == 3 && one_f32_row(x, {&w})) return linear_packed(x, {w}, nullptr, 0.f);
     if (x.dtype() != DType::F32 || w.dtype() != DType::BF16 || w.rank() != 2 || x.rank() < 2 || w.dims()[1] != x.dims().back() || rows <= 8 ||
-        w.dims()[0] % 64 != 0 || w.dims()[1] % 32 != 0)
+        w.dims()[1] % 32 != 0)
       return Ops::linear(x, w);
     const size_t n = w.dims()[0], k = w.dims()[1];
     ughip_device* dev = hip_dev(x);

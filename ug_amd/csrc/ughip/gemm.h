@@ -14,11 +14,13 @@ struct MMArgs {
   long long a_rs, a_cs;  // lhs strides of (m, k), in elements
   long long b_rs, b_cs;  // rhs strides of (k, n), in elements
   long long a_bs, b_bs, c_bs;
+  int n_tile = 0;  // set inside the tiled kernel: columns of the workgroup's tile that exist (a last tile may hang over N)
 };
 
-// Tuned kernel: 256x128, 128x128 or 128x64 tiles whose width divides N (the 128-row tiles take any M:
-// the last one may hang over the end of the lhs), K % 64 == 0 (bf16) / K % 32 == 0 (f32), lhs rows
-// contiguous, rhs either [k, n] row-major or [n, k] row-major.
+// Tuned kernel: 256x128, 128x128 or 128x64 tiles, K % 64 == 0 (bf16) / K % 32 == 0 (f32), lhs rows
+// contiguous, rhs either [k, n] row-major or [n, k] row-major.  The 128-row tiles take any M, and with
+// an [n, k]-major rhs any N: a last tile may hang over the end, it reads the last row again and
+// stores only what exists.
 // rhs_bf16: the rhs is stored as bf16 under an f32 product ([n, k] row-major only) and widened on its way into LDS.
 bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf16 = false);
 // Bytes of f32 scratch the launch needs (split-K partial tiles for skinny products; 0 for most).

@@ -87,8 +87,9 @@ struct RhsElt<float, 2> {
 
 __device__ __forceinline__ u32x4 widen_bf16x4(const u32x4& r) { return u32x4{r.x << 16, r.x & 0xffff0000u, r.y << 16, r.y & 0xffff0000u}; }
 
-// RAGGED: the tile hangs over the last row of the lhs; p.M is then the number of rows of THIS tile that
-// exist, and rows past them read the last one (their products are never stored).
+// RAGGED: the tile may hang over the last row of the lhs or (B_NK != 0) of the rhs; p.M and p.n_tile are then
+// the rows and columns of THIS tile that exist, and rows past them read the last one (their products are
+// never stored).
 template <typename T, int B_NK, int BM, int BN, int NT, bool RAGGED = false, typename BT>
 __device__ __forceinline__ void load_tiles(const T* __restrict__ A, const BT* __restrict__ B, const MMArgs& p, int kt, int tid, Staged<BM, NT>& r) {
   constexpr int RP = NT / 8;  // rows per pass
@@ -111,7 +112,17 @@ __device__ __forceinline__ void load_tiles(const T* __restrict__ A, const BT* __
     const size_t b_step = (size_t)RP * p.b_cs;
 #pragma unroll
     for (int i = 0; i < BN / RP; ++i) {
-      if (B_NK == 2) {
+      if (RAGGED) {
+        const int row = min((tid >> 3) + i * RP, p.n_tile - 1);
+        const BT* q = B + (size_t)row * p.b_cs + k0 + (tid & 7) * VE;
+        if (B_NK == 2) {
+          const u32x2 v = *reinterpret_cast<const u32x2*>(q);
+          r.b[i].x = v.x;
+          r.b[i].y = v.y;
+        } else {
+          r.b[i] = *reinterpret_cast<const u32x4*>(q);
+        }
+      } else if (B_NK == 2) {
         const u32x2 v = *reinterpret_cast<const u32x2*>(Bp + i * b_step);
         r.b[i].x = v.x;
         r.b[i].y = v.y;
@@ -311,7 +322,10 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p_in, int tiles_m, int t
   const int m0 = (t_in / tiles_n) * BM, n0 = (t_in % tiles_n) * BN;
   // p: the problem as this tile sees it -- with RAGGED, M counts the rows of this tile that exist
   MMArgs p = p_in;
-  if (RAGGED) p.M = min(BM, p_in.M - m0);
+  if (RAGGED) {
+    p.M = min(BM, p_in.M - m0);
+    p.n_tile = min(BN, p_in.N - n0);
+  }
   const int kt0 = SPLIT ? slab * kt_per : 0;
   const size_t k_off = (size_t)kt0 * BK;
   const T* __restrict__ A = static_cast<const T*>(p.a) + (size_t)batch * p.a_bs + (size_t)m0 * p.a_rs + k_off;
@@ -367,7 +381,8 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p_in, int tiles_m, int t
         float* Wt = W + (size_t)(wm + i * 32 + (lane >> 5) * 4) * p.N + wn + j * 32 + (lane & 31);
 #pragma unroll
         for (int r = 0; r < 16; ++r)
-          if (!RAGGED || wm + i * 32 + (lane >> 5) * 4 + (r >> 2) * 8 + (r & 3) < p.M) Wt[(size_t)((r >> 2) * 8 + (r & 3)) * p.N] = acc[i][j][r];
+          if (!RAGGED || (wm + i * 32 + (lane >> 5) * 4 + (r >> 2) * 8 + (r & 3) < p.M && wn + j * 32 + (lane & 31) < p.n_tile))
+            Wt[(size_t)((r >> 2) * 8 + (r & 3)) * p.N] = acc[i][j][r];
       }
   } else {
     T* __restrict__ C = static_cast<T*>(p.c) + (size_t)batch * p.c_bs + (size_t)m0 * p.N + n0;
@@ -378,7 +393,8 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p_in, int tiles_m, int t
         T* Ct = C + (size_t)(wm + i * 32 + (lane >> 5) * 4) * p.N + wn + j * 32 + (lane & 31);
 #pragma unroll
         for (int r = 0; r < 16; ++r)
-          if (!RAGGED || wm + i * 32 + (lane >> 5) * 4 + (r >> 2) * 8 + (r & 3) < p.M) Ct[(size_t)((r >> 2) * 8 + (r & 3)) * p.N] = (T)acc[i][j][r];
+          if (!RAGGED || (wm + i * 32 + (lane >> 5) * 4 + (r >> 2) * 8 + (r & 3) < p.M && wn + j * 32 + (lane & 31) < p.n_tile))
+            Ct[(size_t)((r >> 2) * 8 + (r & 3)) * p.N] = (T)acc[i][j][r];
       }
   }
 }
@@ -529,7 +545,7 @@ hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch, int nsplit,
     if (e != hipSuccess) return e;
     configured = true;
   }
-  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = p.N / BN;
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const int kt = p.K / BK, kt_per = SPLIT ? (kt + nsplit - 1) / nsplit : kt;
   if (SPLIT) nsplit = (kt + kt_per - 1) / kt_per;  // no empty slab
   const size_t total = batch * (size_t)tiles_m * tiles_n * (SPLIT ? nsplit : 1);
@@ -570,12 +586,14 @@ hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int s
       return getenv("UGHIP_GEMM_4WAVES") ? launch<T, B_NK, 256, 128, 256, SPLIT>(stream, p, batch, nsplit, ws)
                                          : launch<T, B_NK, 256, 128, 512, SPLIT>(stream, p, batch, nsplit, ws);
     case 1:
-      return p.M % 128 ? launch<T, B_NK, 128, 128, 256, SPLIT, true>(stream, p, batch, nsplit, ws) : launch<T, B_NK, 128, 128, 256, SPLIT>(stream, p, batch, nsplit, ws);
+      return p.M % 128 || p.N % 128 ? launch<T, B_NK, 128, 128, 256, SPLIT, true>(stream, p, batch, nsplit, ws)
+                                    : launch<T, B_NK, 128, 128, 256, SPLIT>(stream, p, batch, nsplit, ws);
     case 3:
       if constexpr (sizeof(T) == 2 && B_NK == 1 && !SPLIT) return launch_dma256<T>(stream, p, batch);
       [[fallthrough]];
     default:
-      return p.M % 128 ? launch<T, B_NK, 128, 64, 256, SPLIT, true>(stream, p, batch, nsplit, ws) : launch<T, B_NK, 128, 64, 256, SPLIT>(stream, p, batch, nsplit, ws);
+      return p.M % 128 || p.N % 64 ? launch<T, B_NK, 128, 64, 256, SPLIT, true>(stream, p, batch, nsplit, ws)
+                                   : launch<T, B_NK, 128, 64, 256, SPLIT>(stream, p, batch, nsplit, ws);
   }
 }
 
@@ -587,21 +605,24 @@ constexpr int kShapes[4][2] = {{256, 128}, {128, 128}, {128, 64}, {256, 256}};
 // the dividing tile with the most workgroups.  -1: no tile divides M x N.
 int pick_shape(const MMArgs& p, size_t batch, int dtype) {
   // shape 3 (256 x 256, loads that write LDS directly): 16-bit types with an [n, k]-major rhs
-  const bool can3 = dtype != UGHIP_F32 && p.b_rs == 1 && p.b_cs != 1 && p.M % 256 == 0 && p.N % 256 == 0;
+  const bool rhs_nk = p.b_rs == 1 && p.b_cs != 1;
+  const bool can3 = dtype != UGHIP_F32 && rhs_nk && p.M % 256 == 0 && p.N % 256 == 0;
   // UGHIP_GEMM_SHAPE=0..3 forces a tile shape (tuning aid); ignored when it does not fit the problem.
   if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
     const int s = atoi(e);
     if (s == 3 && can3) return 3;
-    if (s >= 0 && s < 3 && (p.M % kShapes[s][0] == 0 || kShapes[s][0] == 128) && p.N % kShapes[s][1] == 0) return s;
+    if (s >= 0 && s < 3 && (p.M % kShapes[s][0] == 0 || kShapes[s][0] == 128) && (p.N % kShapes[s][1] == 0 || (kShapes[s][0] == 128 && rhs_nk))) return s;
   }
   // half the LDS traffic per flop of 256 x 128, once it alone gives every CU a workgroup
   if (can3 && batch * (size_t)(p.M / 256) * (size_t)(p.N / 256) >= 256) return 3;
   int best = -1;
   size_t best_tiles = 0;
   for (int s = 0; s < 3; ++s) {
-    // the 128-row tiles also take an lhs whose last tile is partly empty (any M >= 9: fewer rows are the GEMV kernels' job)
-    if ((p.M % kShapes[s][0] && kShapes[s][0] != 128) || p.N % kShapes[s][1]) continue;
-    const size_t tiles = batch * (size_t)((p.M + kShapes[s][0] - 1) / kShapes[s][0]) * (size_t)(p.N / kShapes[s][1]);
+    // the 128-row tiles also take an lhs whose last tile is partly empty (any M >= 9: fewer rows are the GEMV kernels'
+    // job) and, with an [n, k]-major rhs, an N they do not divide
+    const bool ragged_ok = kShapes[s][0] == 128;
+    if ((p.M % kShapes[s][0] && !ragged_ok) || (p.N % kShapes[s][1] && !(ragged_ok && rhs_nk))) continue;
+    const size_t tiles = batch * (size_t)((p.M + kShapes[s][0] - 1) / kShapes[s][0]) * (size_t)((p.N + kShapes[s][1] - 1) / kShapes[s][1]);
     if (tiles >= 256) return s;
     if (tiles > best_tiles) best = s, best_tiles = tiles;
   }
@@ -613,9 +634,10 @@ int pick_shape(const MMArgs& p, size_t batch, int dtype) {
 int pick_split(int dtype, const MMArgs& p, size_t batch, int shape) {
   if (const char* e = getenv("UGHIP_GEMM_SPLIT")) return std::max(1, atoi(e));  // tuning aid
   const int bk = dtype == UGHIP_F32 ? 32 : 64;
-  const size_t tiles = batch * (size_t)((p.M + kShapes[shape][0] - 1) / kShapes[shape][0]) * (size_t)(p.N / kShapes[shape][1]);
+  const size_t tiles = batch * (size_t)((p.M + kShapes[shape][0] - 1) / kShapes[shape][0]) * (size_t)((p.N + kShapes[shape][1] - 1) / kShapes[shape][1]);
   const int kt = p.K / bk;
   if (tiles >= 128 || kt < 8) return 1;
+  if ((batch * (size_t)p.M * (size_t)p.N) % 4 != 0) return 1;  // the fold of the partial tiles works on groups of 4 elements
   // three workgroups per CU: measured on the projections of a 128-token prefill, short slabs overlap
   // each other's pipeline fill better than one workgroup per CU with longer ones
   int want = (int)((768 + tiles - 1) / tiles);
@@ -630,7 +652,7 @@ bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf1
   if (rhs_bf16 && (dtype != UGHIP_F32 || p.b_rs != 1 || p.b_cs == 1)) return false;  // widening is built for an [n, k]-major rhs under an f32 product
   const int ve = dtype == UGHIP_F32 ? 4 : 8, bk = dtype == UGHIP_F32 ? 32 : 64;
   if (p.M <= 0 || p.N <= 0 || p.K <= 0 || p.K % bk || batch == 0) return false;
-  if (p.a_cs != 1 || p.a_rs % ve || p.a_bs % ve || p.b_bs % ve || p.c_bs % ve) return false;
+  if (p.a_cs != 1 || p.a_rs % ve || (batch > 1 && (p.a_bs % ve || p.b_bs % ve))) return false;  // 128-bit loads; the result is stored element by element
   const bool nn = p.b_cs == 1, nt = p.b_rs == 1;
   if (nn == nt) return false;
   if (nn && p.b_rs % ve) return false;
@@ -638,7 +660,7 @@ bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf1
   if (!aligned16(p.a) || !aligned16(p.b) || !aligned16(p.c)) return false;
   const int s = pick_shape(p, batch, dtype);
   if (s < 0) return false;
-  return batch * (size_t)((p.M + kShapes[s][0] - 1) / kShapes[s][0]) * (size_t)(p.N / kShapes[s][1]) < (1u << 24);
+  return batch * (size_t)((p.M + kShapes[s][0] - 1) / kShapes[s][0]) * (size_t)((p.N + kShapes[s][1] - 1) / kShapes[s][1]) < (1u << 24);
 }
 
 size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch) {

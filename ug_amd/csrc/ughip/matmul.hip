@@ -441,8 +441,8 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
   if (mixed) {
     if (!gemm_tiled_supported(UGHIP_F32, p, b, true) || rhs_offset % 8 != 0)
       return set_error(UGHIP_ERR_UNSUPPORTED,
-                       "matmul: an F32 product with a BF16 rhs is built for an [n, k]-major rhs with n, k in multiples of 64, 32 "
-                       "(got m %zu, n %zu, k %zu, rhs strides %lld, %lld)",
+                       "matmul: an F32 product with a BF16 rhs is built for an [n, k]-major rhs with k a multiple of 32 and rows that "
+                       "start on 8-byte boundaries (got m %zu, n %zu, k %zu, rhs strides %lld, %lld)",
                        m, n, k, p.b_rs, p.b_cs);
   }
   if (!mixed && gemv_nt_ok) {
