@@ -365,7 +365,7 @@ def llama_decode(dev, n_prompt=128, n_steps=128, fused_attention=0, bf16_matrice
     tok_s = n_steps / (st["decode_ms"] * 1e-3)
     return {"tok/s": round(tok_s, 2), "decode_ms_per_token": round(st["decode_ms"] / n_steps, 3), "prefill_ms": round(st["prefill_ms"], 1),
             "frac_hbm_weights_only": round(tok_s * weights_bytes / 1e9 / HBM_PEAK_GBS, 4), "load_s": round(load_s, 1), "dtype": "f32 activations, bf16 matrices" if bf16_matrices else "f32", "zero_fill": False, "fused_attention": fused_attention,
-            "first_ids": toks[:8].tolist(), "min_top1_margin": float(st["margins"].min())}
+            "prompt_tokens": n_prompt, "decode_steps": n_steps, "first_ids": toks[:8].tolist(), "min_top1_margin": float(st["margins"].min())}
 
 
 def main():
@@ -443,12 +443,16 @@ def main():
         except Exception as e:  # noqa: BLE001
             line["extras"] = {"error": f"{type(e).__name__}: {e}"}
     if not (args.no_llama or args.headline_only):
-        for key, fused, narrow in (("llama_decode_f32", 0, False), ("llama_decode_f32_fused_attention", 1, False), ("llama_decode_f32_inplace_cache", 2, False),
-                                   ("llama_decode_f32_fused_projections", 3, False), ("llama_decode_bf16_matrices", 3, True)):
+        # the last entry: the same model decoding behind a 1900-token prompt (caches near their 2048 rows)
+        for key, fused, narrow, n_prompt, n_steps in (("llama_decode_f32", 0, False, 128, 128), ("llama_decode_f32_fused_attention", 1, False, 128, 128),
+                                                      ("llama_decode_f32_inplace_cache", 2, False, 128, 128),
+                                                      ("llama_decode_f32_fused_projections", 3, False, 128, 128),
+                                                      ("llama_decode_bf16_matrices", 3, True, 128, 128),
+                                                      ("llama_decode_bf16_matrices_prompt1900", 3, True, 1900, 64)):
             if args.llama_level is not None and (fused != args.llama_level or narrow != args.llama_bf16):
                 continue
             try:
-                line.setdefault("extras", {})[key] = llama_decode(dev, fused_attention=fused, bf16_matrices=narrow)
+                line.setdefault("extras", {})[key] = llama_decode(dev, n_prompt=n_prompt, n_steps=n_steps, fused_attention=fused, bf16_matrices=narrow)
             except Exception as e:  # noqa: BLE001
                 line.setdefault("extras", {})[key] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(line), flush=True)
