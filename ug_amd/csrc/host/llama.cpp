@@ -694,6 +694,16 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
     return finish(ops_->attention_cached(qkv, kc, vc, cache.len, scale, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, 0, row, nh));
   }
   LB xs = norm_first ? rms_norm(xs_in, l.rms1, eps) : xs_in;
+  if (fused_attention_ >= 3 && cache.capacity && l.qkv_stacked.valid()) {
+    // several positions: one product gives q | k | v side by side and everything behind it reads its
+    // column range of the wide rows in place (a preallocated cache implies a head size the kernels take)
+    const size_t nq = nh * hd, nk = nkv * hd, row = nq + 2 * nk, len = cache.len;
+    LB qkv = ops_->linear(xs, l.qkv_stacked);
+    LB kc = ops_->kv_append(cache.prev_k, len, qkv, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, nq, row);
+    LB vc = ops_->kv_append(cache.prev_v, len, qkv, nullptr, nullptr, nullptr, false, nq + nk, row);
+    cache.len = len + seq_len;
+    return finish(ops_->attention_cached(qkv, kc, vc, cache.len, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, 0, row, nh));
+  }
   LB q = ops_->linear(xs, l.q_proj);
   LB k = ops_->linear(xs, l.k_proj);
   LB v = ops_->linear(xs, l.v_proj);
@@ -753,12 +763,41 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
 
 // model.rs:160-168
 LB Model::mlp(const Layer& l, const LB& xs, const LB* residual, bool norm_first) const {
+  if (residual && l.gate_up_stacked.valid() && xs.rank() == 3 && xs.dims()[0] * xs.dims()[1] > 1) {
+    // several positions: gate and up in one product, SwiGLU on the two halves of its rows
+    const size_t isz = cfg_.intermediate_size;
+    LB x = norm_first ? rms_norm(xs, l.rms2, (float)cfg_.rms_norm_eps) : xs;
+    LB gu = ops_->linear(x, l.gate_up_stacked);
+    LB act = silu(gu.narrow(2, 0, isz)).binary(BinaryOp::Mul, gu.narrow(2, isz, isz));
+    return ops_->linear_add(act, l.down_proj, *residual);
+  }
   if (residual)
     return ops_->linear_add(ops_->gate_up(xs, l.gate_proj, l.up_proj, norm_first ? &l.rms2 : nullptr, (float)cfg_.rms_norm_eps), l.down_proj, *residual);
   LB xs1 = ops_->linear(xs, l.gate_proj);
   LB xs2 = ops_->linear(xs, l.up_proj);
   xs1 = silu(xs1);
   return ops_->linear(xs1.binary(BinaryOp::Mul, xs2), l.down_proj);
+}
+
+void Model::set_fused_attention(int level) {
+  fused_attention_ = level;
+  if (level >= 3 && ops_->packed_projections()) stack_matrices();
+}
+
+void Model::stack_matrices() {
+  for (Layer& l : layers_) {
+    if (l.qkv_stacked.valid() && l.qkv_stacked.dtype() == l.q_proj.dtype()) continue;
+    // cat is an allocation written in place (lazy_buffer.rs:722-766), which every schedule would run again:
+    // the copy through Id is an ordinary buffer that stays realised
+    auto stacked = [](const std::vector<LB>& parts) {
+      LB s = LB::cat(parts, 0).unary(UnaryOp::Id);
+      s.realize();
+      s.detach();
+      return s;
+    };
+    l.qkv_stacked = stacked({l.q_proj, l.k_proj, l.v_proj});
+    l.gate_up_stacked = stacked({l.gate_proj, l.up_proj});
+  }
 }
 
 void Model::store_matrices_bf16() {
@@ -772,6 +811,7 @@ void Model::store_matrices_bf16() {
   for (Layer& l : layers_)
     for (LB* w : {&l.q_proj, &l.k_proj, &l.v_proj, &l.o_proj, &l.gate_proj, &l.up_proj, &l.down_proj}) narrow(*w);
   narrow(head_);
+  if (!layers_.empty() && layers_[0].qkv_stacked.valid()) stack_matrices();  // the stacked copies follow the dtype
   // The lookup reads t rows and keeps an f32 table, the head streams all of the bf16 one; both hold
   // the same values (one tied tensor, model.rs:315-319).
   LB wide = head_.cast(DType::F32);

@@ -162,7 +162,12 @@ class Model {
   // 3: 2, and the projections through Ops::linear_packed (norm + q|k|v, norm + output head),
   //    Ops::gate_up (norm + gate, up, SwiGLU) and Ops::linear_add (o_proj / down_proj with the
   //    residual): 7 schedule items per layer and decode step on a device that fuses them.
-  void set_fused_attention(int level) { fused_attention_ = level; }
+  //    With more than one position (prefill) level 3 multiplies by q|k|v and gate|up stacked into one
+  //    matrix each -- 4 products per layer instead of 7 -- and the cache appends, the attention kernel
+  //    and SwiGLU read their column ranges of the wide results in place.  The stacked copies are made
+  //    the first time level 3 is set on a device with packed projections and kept beside the
+  //    separate matrices, which the one-position kernels stream (1.3 x the matrix bytes resident).
+  void set_fused_attention(int level);
   int fused_attention() const { return fused_attention_; }
   // Keep the projection matrices and the output head in bf16 (rounded to nearest even when they
   // are not bf16 values already) and stream them in that form; activations stay f32.  The numbers
@@ -184,7 +189,9 @@ class Model {
     LB rms1, rms2;
     LB q_proj, k_proj, v_proj, o_proj;
     LB gate_proj, up_proj, down_proj;
+    LB qkv_stacked, gate_up_stacked;  // [q; k; v] and [gate; up] by rows; invalid until level 3 asks for them
   };
+  void stack_matrices();
   // residual != nullptr: the result includes the residual add; norm_first: xs still has to go
   // through the layer's RMSNorm (fusion level 3 folds both into the projections)
   LB attention(const Layer& l, const LB& xs, const LB& pos, Cache& cache, const LB* residual, bool norm_first) const;

@@ -636,7 +636,7 @@ int pick_split(int dtype, const MMArgs& p, size_t batch, int shape) {
   const int bk = dtype == UGHIP_F32 ? 32 : 64;
   const size_t tiles = batch * (size_t)((p.M + kShapes[shape][0] - 1) / kShapes[shape][0]) * (size_t)((p.N + kShapes[shape][1] - 1) / kShapes[shape][1]);
   const int kt = p.K / bk;
-  if (tiles >= 128 || kt < 8) return 1;
+  if (tiles >= 256 || kt < 8) return 1;
   if ((batch * (size_t)p.M * (size_t)p.N) % 4 != 0) return 1;  // the fold of the partial tiles works on groups of 4 elements
   // three workgroups per CU: measured on the projections of a 128-token prefill, short slabs overlap
   // each other's pipeline fill better than one workgroup per CU with longer ones
