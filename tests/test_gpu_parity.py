@@ -1190,6 +1190,40 @@ def test_fused_projections_fall_back_for_several_rows(hip, cpu, hip_ops, cpu_ops
         np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-6)
 
 
+@pytest.mark.parametrize("t,length,d", [(5, 0, 64), (7, 9, 64), (130, 0, 64), (4, 3, 32), (3, 2, 128)])
+def test_packed_rows_of_several_positions(hip, hip_ops, t, length, d):
+    """Prefill form of the packed rows: t positions of q | k | v side by side (what one product with the stacked
+    matrix gives), read in place by kv_append and attention_cached: the results of the three parts handed over
+    separately, bit for bit."""
+    nh, nkv, cap = 4, 2, 256
+    nq, nk = nh * d, nkv * d
+    row = nq + 2 * nk
+    qkv = rng.normal(161, t * row).reshape(t, row)
+    store_k, store_v = rng.normal(162, nkv * cap * d), rng.normal(163, nkv * cap * d)
+    cos, sin = _rope_tables(hip, d, max_pos=cap)
+    pos = LB.copy(np.array([length], np.int32), (1, 1), hip)
+    scale = float(np.float32(d) ** np.float32(-0.5))
+
+    def run(packed):
+        ck, cv = LB.copy(store_k, (1, nkv, cap, d), hip), LB.copy(store_v, (1, nkv, cap, d), hip)
+        ck.realize(), cv.realize()
+        if packed:
+            buf = LB.copy(qkv.ravel(), (1, t, row), hip)
+            kc = hip_ops.kv_append(ck, length, buf, cos, sin, pos, False, x_offset=nq, x_row_stride=row)
+            vc = hip_ops.kv_append(cv, length, buf, x_offset=nq + nk, x_row_stride=row)
+            out = hip_ops.attention_cached(buf, kc, vc, length + t, scale, cos, sin, pos, False, q_offset=0, q_row_stride=row, n_heads=nh)
+        else:
+            part = lambda a, b: LB.copy(np.ascontiguousarray(qkv[:, a:b]).ravel(), (1, t, b - a), hip)   # noqa: E731
+            kc = hip_ops.kv_append(ck, length, part(nq, nq + nk), cos, sin, pos, False)
+            vc = hip_ops.kv_append(cv, length, part(nq + nk, row))
+            out = hip_ops.attention_cached(part(0, nq), kc, vc, length + t, scale, cos, sin, pos, False)
+        assert tuple(out.dims()) == (1, t, nq)
+        return out.data_vec(), ck.data_vec(), cv.data_vec()
+
+    for a, b2 in zip(run(True), run(False)):
+        np.testing.assert_array_equal(a, b2)
+
+
 @pytest.mark.parametrize("cap,length", [(32, 5), (2048, 1500)])
 def test_packed_rows_feed_cache_and_attention(hip, hip_ops, cap, length):
     """q | k | v side by side in one buffer, read in place by kv_append and attention_cached: same
