@@ -125,6 +125,11 @@ typedef struct ughip_func ughip_func;     /* ug_cuda::runtime::Func    (runtime.
 typedef struct ughip_event ughip_event;
 
 const char* ughip_last_error(void);
+/* Tuning and test aid with no counterpart in the reference (cuBLAS picks its kernels out of sight,
+ * ug-cuda/src/gemm.rs:130-290): the hand-written kernel the calling thread's last ughip_matmul
+ * launched, e.g. "gemm_tiled<f32,NN,256x128,512t>", "gemm_tiled<bf16,NT,128x64,256t,ragged,splitK=12>",
+ * "gemv_nt<f32>", "gemm_any<f16>".  Thread-local; "" before the first product. */
+const char* ughip_last_kernel(void);
 
 /* ---- device: Device::new / Clone / synchronize (runtime.rs:158-177,243-246) ---------- */
 int ughip_device_create(int ordinal, ughip_device** out);

@@ -1,0 +1,371 @@
+"""BASELINE.json's configs at their stated sizes on the HIP device: config 3 (batched matmul 8 x 1024^3, f32 and
+bf16), config 4 (the llama layer pieces at T = 512, hidden 2048, 32 heads x 64) and config 5 (22 layers, a prompt
+of 128 ids, 128 greedy steps).  The oracle runs where it finishes in seconds; beyond that the expectation is a
+float64 numpy statement of the same formula (with the forward-error bound written out) or, for config 5, the
+fixture the oracle wrote at full depth (tests/golden/llama_config5_greedy.json).  Every test names the kernel it
+means to reach and asserts that this is the one that ran."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import ug_amd
+from ug_amd import F32, LazyBuffer as LB, rng
+
+pytestmark = pytest.mark.gpu
+
+EPS32 = float(np.finfo(np.float32).eps)
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _matmul(hip, dtype, a, w, rhs_nk):
+    """a [b, m, k], w [b, k, n] (f32 values); rhs_nk hands the rhs over stored [b, n, k].  Returns (f32 result, kernel name)."""
+    b, m, k = a.shape
+    n = w.shape[2]
+    enc = rng.to_bf16_bits if dtype == ug_amd.BF16 else (lambda v: v)
+    sa = hip.slice_from(enc(np.ascontiguousarray(a)))
+    if rhs_nk:
+        sw = hip.slice_from(enc(np.ascontiguousarray(np.swapaxes(w, 1, 2))))
+        rhs = ((b, k, n), (k * n, 1, k), 0)
+    else:
+        sw = hip.slice_from(enc(np.ascontiguousarray(w)))
+        rhs = ((b, k, n), (k * n, n, 1), 0)
+    dst = hip.allocate_uninit(dtype, b * m * n)
+    hip.matmul(dst, sa, sw, (b, m, n, k), ((b, m, k), (m * k, k, 1), 0), rhs)
+    kernel = ug_amd.last_kernel()
+    out = dst.to_vec()
+    out = rng.from_bf16_bits(out) if dtype == ug_amd.BF16 else out
+    return out.reshape(b, m, n), kernel
+
+
+def _f64_product(a, w):
+    exact = np.matmul(a.astype(np.float64), w.astype(np.float64))
+    mag = np.matmul(np.abs(a).astype(np.float64), np.abs(w).astype(np.float64))
+    return exact, mag
+
+
+# ---- config 3: A [8, 1024, 1024] x B [8, 1024, 1024], U(-1, 1) from seeds 4 / 5 ---------------------------------------
+def _config3_operands(round_bf16):
+    b, m = 8, 1024
+    a, w = rng.uniform_pm1(4, b * m * m), rng.uniform_pm1(5, b * m * m)
+    if round_bf16:
+        a, w = rng.bf16_round(a), rng.bf16_round(w)
+    return a.reshape(b, m, m), w.reshape(b, m, m)
+
+
+@pytest.mark.parametrize("rhs_nk", [False, True], ids=["NN", "NT"])
+def test_config3_bmm_f32(hip, cpu, rhs_nk):
+    """f32 8 x 1024^3: against the float64 product within k eps sum|a||b| (the forward bound of any f32 summation
+    order), and, for the row-major rhs BASELINE names, against the oracle's matmul (two f32 orders: twice the bound)."""
+    a, w = _config3_operands(False)
+    got, kernel = _matmul(hip, F32, a, w, rhs_nk)
+    print("config 3 f32", "NT" if rhs_nk else "NN", kernel, flush=True)
+    assert kernel == f"gemm_tiled<f32,{'NT' if rhs_nk else 'NN'},256x128,512t>"
+    exact, mag = _f64_product(a, w)
+    bound = 1024 * EPS32 * mag
+    assert np.all(np.abs(got - exact) <= bound + 1e-12)
+    # typical error is far inside the worst-case bound: the rms error of a 1024-term f32 sum is about sqrt(k) eps |terms|
+    assert float(np.sqrt(np.mean((got - exact) ** 2))) <= 32 * EPS32 * float(np.sqrt(np.mean(mag ** 2)))
+    if not rhs_nk:
+        want = LB.copy(a, a.shape, cpu).matmul(LB.copy(w, w.shape, cpu)).data_vec().reshape(got.shape)
+        assert np.all(np.abs(got - want) <= 2 * bound + 1e-12)
+        # through the lazy graph on the HIP device: the same kernel, the same bits
+        lazy = LB.copy(a, a.shape, hip).matmul(LB.copy(w, w.shape, hip)).data_vec().reshape(got.shape)
+        assert ug_amd.last_kernel() == kernel
+        np.testing.assert_array_equal(lazy, got)
+
+
+@pytest.mark.parametrize("rhs_nk", [False, True], ids=["NN", "NT"])
+def test_config3_bmm_bf16(hip, rhs_nk):
+    """bf16 8 x 1024^3 (RNE-rounded copies of the f32 operands): no reference result exists (cpu_runtime.rs:345-356
+    refuses BF16), so the expectation is the exact product of the rounded operands, f32 accumulation (k eps sum|a||b|)
+    and one rounding to bf16 (2^-8 relative) -- inside BASELINE's 1e-2."""
+    a, w = _config3_operands(True)
+    got, kernel = _matmul(hip, ug_amd.BF16, a, w, rhs_nk)
+    print("config 3 bf16", "NT" if rhs_nk else "NN", kernel, flush=True)
+    assert kernel.startswith("gemm_") and ("bf16,NT" if rhs_nk else "bf16,NN") in kernel, kernel
+    exact, mag = _f64_product(a, w)
+    bound = 2.0 ** -8 * np.abs(exact) + 1024 * EPS32 * mag
+    assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-12)
+    scale = float(np.abs(exact).max())
+    assert float(np.abs(got - exact).max()) <= 1e-2 * scale
+
+
+@pytest.mark.parametrize("dtype_name", ["f32", "bf16"])
+@pytest.mark.parametrize("rhs_nk", [False, True], ids=["NN", "NT"])
+@pytest.mark.parametrize("bmnk,split", [((2, 256, 128, 96 * 2), 0), ((1, 512, 256, 64), 0), ((1, 256, 128, 1024), 4), ((3, 256, 384, 128), 0)])
+def test_matmul_256x128_tile_forced(hip, monkeypatch, bmnk, split, rhs_nk, dtype_name):
+    """The 256 x 128, 8-wave tile on problems small enough for an exact check: forced through UGHIP_GEMM_SHAPE=0
+    (the dispatcher only picks it from 256 tiles up), with and without a K split."""
+    b, m, n, k = bmnk
+    monkeypatch.setenv("UGHIP_GEMM_SHAPE", "0")
+    if split:
+        monkeypatch.setenv("UGHIP_GEMM_SPLIT", str(split))
+    dtype = F32 if dtype_name == "f32" else ug_amd.BF16
+    a = rng.uniform_pm1(71, b * m * k).reshape(b, m, k)
+    w = rng.uniform_pm1(72, b * k * n).reshape(b, k, n)
+    if dtype_name == "bf16":
+        a, w = rng.bf16_round(a.ravel()).reshape(a.shape), rng.bf16_round(w.ravel()).reshape(w.shape)
+    got, kernel = _matmul(hip, dtype, a, w, rhs_nk)
+    print("forced 256x128", dtype_name, bmnk, "NT" if rhs_nk else "NN", kernel, flush=True)
+    assert f"{dtype_name},{'NT' if rhs_nk else 'NN'},256x128,512t" in kernel and (f"splitK={split}" in kernel) == bool(split), kernel
+    exact, mag = _f64_product(a, w)
+    bound = k * EPS32 * mag + (2.0 ** -8 * np.abs(exact) if dtype_name == "bf16" else 0.0)
+    assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-12)
+    # small integers: every partial sum is exact in f32, so the result is the integer product bit for bit
+    ai, wi = np.floor(a * 4), np.floor(w * 4)
+    want = np.matmul(ai.astype(np.float64), wi.astype(np.float64)).astype(np.float32)
+    if dtype_name == "bf16":
+        want = rng.bf16_round(want.ravel()).reshape(want.shape)
+    goti, _ = _matmul(hip, dtype, ai, wi, rhs_nk)
+    np.testing.assert_array_equal(goti, want)
+
+
+# ---- config 4: the llama layer pieces at T = 512 ----------------------------------------------------------------------
+T, HIDDEN, HEADS, HD = 512, 2048, 32, 64
+
+
+def test_config4_rms_norm_512x2048(hip):
+    """x [1, 512, 2048] N(0, 1), alpha N(0, 0.02), eps 1e-5 (model.rs:65-78): float64 statement, 1e-5 relative.  The
+    oracle's own kernel recomputes the sum per element (2.1 G iterations); it checks the first rows."""
+    x = rng.normal(6, T * HIDDEN).reshape(1, T, HIDDEN)
+    alpha = rng.normal(106, HIDDEN, 0.02)
+    lb = ug_amd.llama.rms_norm(LB.copy(x, x.shape, hip), LB.copy(alpha, alpha.shape, hip), 1e-5)
+    got = lb.data_vec().reshape(x.shape)
+    x64 = x.astype(np.float64)
+    want = x64 / np.sqrt((x64 * x64).mean(-1, keepdims=True) + np.float64(np.float32(1e-5))) * alpha.astype(np.float64)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5 * float(np.abs(want).max()) * 1e-2)
+
+
+def test_config4_rms_norm_rows_against_the_oracle(hip, cpu):
+    x = rng.normal(6, T * HIDDEN).reshape(1, T, HIDDEN)[:, :8]
+    alpha = rng.normal(106, HIDDEN, 0.02)
+    got = ug_amd.llama.rms_norm(LB.copy(x, x.shape, hip), LB.copy(alpha, alpha.shape, hip), 1e-5).data_vec()
+    want = ug_amd.llama.rms_norm(LB.copy(x, x.shape, cpu), LB.copy(alpha, alpha.shape, cpu), 1e-5).data_vec()
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-9)
+
+
+def _rope_f64(x, cos, sin, pos0, interleaved):
+    """x [bh, t, d] float64; cos/sin [max_pos, d/2] (cpu_ops.rs:58-126)."""
+    bh, t, d = x.shape
+    c, s = cos[pos0:pos0 + t].astype(np.float64), sin[pos0:pos0 + t].astype(np.float64)
+    out = np.empty_like(x)
+    if interleaved:
+        x1, x2 = x[..., 0::2], x[..., 1::2]
+        out[..., 0::2] = x1 * c - x2 * s
+        out[..., 1::2] = x1 * s + x2 * c
+    else:
+        x1, x2 = x[..., :d // 2], x[..., d // 2:]
+        out[..., :d // 2] = x1 * c - x2 * s
+        out[..., d // 2:] = x1 * s + x2 * c
+    return out
+
+
+@pytest.mark.parametrize("interleaved", [False, True], ids=["rope", "rope_i"])
+@pytest.mark.parametrize("heads,pos0", [(HEADS, 0), (4, 0), (HEADS, 1500)])
+def test_config4_rope(hip, cpu, hip_ops, cpu_ops, interleaved, heads, pos0):
+    """q [1, 32, 512, 64] and k [1, 4, 512, 64], tables from Rope::new's rule (model.rs:277-296): bit for bit the
+    oracle's op (same table, one multiply-add pair per element), and the float64 statement within 2 eps of the
+    operand magnitudes."""
+    cfg = ug_amd.LlamaConfig()
+    x = rng.normal(7, heads * T * HD).reshape(1, heads, T, HD)
+    res = {}
+    for name, dev, ops in (("hip", hip, hip_ops), ("cpu", cpu, cpu_ops)):
+        cos, sin = ug_amd.llama.rope_tables(dev, cfg)
+        pos = LB.copy(np.array([pos0], np.int32), (1,), dev)
+        f = ops.rope_i if interleaved else ops.rope
+        res[name] = (f(LB.copy(x, x.shape, dev), cos, sin, pos).data_vec().reshape(x.shape), cos.data_vec().reshape(-1, HD // 2), sin.data_vec().reshape(-1, HD // 2))
+    # the tables themselves (powf on the host, an f32 product, cosf / sinf on the device): 1e-5 relative at angles up to 2047 rad
+    np.testing.assert_allclose(res["hip"][1], res["cpu"][1], rtol=0, atol=1e-5)
+    np.testing.assert_allclose(res["hip"][2], res["cpu"][2], rtol=0, atol=1e-5)
+    want = _rope_f64(x.reshape(heads, T, HD).astype(np.float64), res["hip"][1], res["hip"][2], pos0, interleaved).reshape(x.shape)
+    mag = np.abs(x).reshape(heads, T, HD)
+    pair = (np.maximum(mag[..., 0::2], mag[..., 1::2]).repeat(2, -1) if interleaved else np.tile(np.maximum(mag[..., :HD // 2], mag[..., HD // 2:]), 2)).reshape(x.shape)
+    assert np.all(np.abs(res["hip"][0] - want) <= 4 * EPS32 * pair + 1e-30)
+    # against the oracle's op on the oracle's tables: the tables differ by at most 1e-5, the products follow
+    np.testing.assert_allclose(res["hip"][0], res["cpu"][0], rtol=0, atol=2.5e-5 * float(pair.max()))
+
+
+def test_config4_mask_and_softmax_1x32x512x512(hip, cpu, hip_ops, cpu_ops):
+    """Scores [1, 32, 512, 512]: causal_mask, custom_softmax, the two composed, the one-kernel fusion and the lazy
+    softmax of model.rs:94-101 -- mask bit for bit, softmax 1e-5 relative against the oracle's op and against float64."""
+    shape = (1, HEADS, T, T)
+    x = rng.normal(8, int(np.prod(shape))).reshape(shape)
+    keep = np.arange(T)[None, :] <= np.arange(T)[:, None]
+    got_mask = hip_ops.causal_mask(LB.copy(x, shape, hip)).data_vec().reshape(shape)
+    np.testing.assert_array_equal(got_mask, np.where(keep, x, np.float32(-np.inf)))
+    np.testing.assert_array_equal(got_mask, cpu_ops.causal_mask(LB.copy(x, shape, cpu)).data_vec().reshape(shape))
+
+    def sm64(v):
+        v = v.astype(np.float64)
+        e = np.exp(v - v.max(-1, keepdims=True))
+        return e / e.sum(-1, keepdims=True)
+
+    want_plain, want_causal = sm64(x), sm64(np.where(keep, x, -np.inf))
+    got = hip_ops.custom_softmax(LB.copy(x, shape, hip)).data_vec().reshape(shape)
+    np.testing.assert_allclose(got, want_plain, rtol=1e-5, atol=1e-30)
+    np.testing.assert_allclose(got, cpu_ops.custom_softmax(LB.copy(x, shape, cpu)).data_vec().reshape(shape), rtol=1e-5, atol=1e-30)
+    lazy = ug_amd.llama.softmax(LB.copy(x, shape, hip)).data_vec().reshape(shape)
+    np.testing.assert_allclose(lazy, want_plain, rtol=1e-5, atol=1e-30)
+    composed = hip_ops.custom_softmax(hip_ops.causal_mask(LB.copy(x, shape, hip))).data_vec().reshape(shape)
+    np.testing.assert_allclose(composed, want_causal, rtol=1e-5, atol=1e-30)
+    fused = hip_ops.causal_softmax(LB.copy(x, shape, hip)).data_vec().reshape(shape)
+    np.testing.assert_allclose(fused, want_causal, rtol=1e-5, atol=1e-30)
+    assert not fused[..., ~keep].any()
+    lazy_causal = ug_amd.llama.softmax(hip_ops.causal_mask(LB.copy(x, shape, hip))).data_vec().reshape(shape)
+    np.testing.assert_allclose(lazy_causal, want_causal, rtol=1e-5, atol=1e-30)
+
+
+def test_config4_lazy_softmax_rows_against_the_oracle(hip, cpu):
+    """The lazy two-kernel softmax against the oracle's own two kernels (which recompute max and sum per element:
+    4.3 G iterations at full size, so 8 of the 16384 rows)."""
+    x = rng.normal(8, HEADS * T * T).reshape(1, HEADS, T, T)[:, :1, :8]
+    got = ug_amd.llama.softmax(LB.copy(x, x.shape, hip)).data_vec()
+    want = ug_amd.llama.softmax(LB.copy(x, x.shape, cpu)).data_vec()
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-30)
+
+
+def test_config4_qk_t_and_att_v(hip, cpu):
+    """q k^T (b = 32, 512 x 512 x 64, rhs [n, k]-major) and att v (b = 32, 512 x 64 x 512, rhs row-major), f32, through the
+    lazy graph as model.rs:231-245 builds them: float64 product within k eps sum|a||b|, and the oracle's matmul within twice that."""
+    q = rng.normal(7, HEADS * T * HD).reshape(1, HEADS, T, HD)
+    k = rng.normal(208, HEADS * T * HD).reshape(1, HEADS, T, HD)
+    v = rng.normal(308, HEADS * T * HD).reshape(1, HEADS, T, HD)
+    s = rng.normal(8, HEADS * T * T).reshape(1, HEADS, T, T)
+    got = LB.copy(q, q.shape, hip).matmul_t(LB.copy(k, k.shape, hip)).data_vec().reshape(1, HEADS, T, T)
+    kernel = ug_amd.last_kernel()
+    print("config 4 q k^T", kernel, flush=True)
+    assert kernel == "gemm_tiled<f32,NT,256x128,512t>"
+    exact, mag = _f64_product(q, np.swapaxes(k, -1, -2))
+    assert np.all(np.abs(got - exact) <= HD * EPS32 * mag + 1e-12)
+    want = LB.copy(q, q.shape, cpu).matmul_t(LB.copy(k, k.shape, cpu)).data_vec().reshape(got.shape)
+    assert np.all(np.abs(got - want) <= 2 * HD * EPS32 * mag + 1e-12)
+
+    got = LB.copy(s, s.shape, hip).matmul(LB.copy(v, v.shape, hip)).data_vec().reshape(1, HEADS, T, HD)
+    kernel = ug_amd.last_kernel()
+    print("config 4 att v", kernel, flush=True)
+    assert kernel.startswith("gemm_tiled<f32,NN,"), kernel
+    exact, mag = _f64_product(s, v)
+    assert np.all(np.abs(got - exact) <= T * EPS32 * mag + 1e-12)
+    want = LB.copy(s, s.shape, cpu).matmul(LB.copy(v, v.shape, cpu)).data_vec().reshape(got.shape)
+    assert np.all(np.abs(got - want) <= 2 * T * EPS32 * mag + 1e-12)
+
+
+def test_config4_attention_chain_and_cached_t512(hip, cpu, hip_ops, cpu_ops):
+    """The whole config-4 chain at T = 512 on the HIP device -- rope(q), rope(k), GQA repeat, q k^T, scale, mask, softmax,
+    att v, as model.rs:207-245 composes them -- and ughip_attention_cached over preallocated caches, both against a
+    float64 statement of causal attention (and so against each other)."""
+    nkv, cap = 4, 2048
+    cfg = ug_amd.LlamaConfig()
+    scale = float(np.float32(HD) ** np.float32(-0.5))
+    qf = rng.normal(7, T * HEADS * HD).reshape(1, T, HEADS * HD)
+    kx = rng.normal(208, T * nkv * HD).reshape(1, T, nkv * HD)
+    vx = rng.normal(308, T * nkv * HD).reshape(1, T, nkv * HD)
+    cos, sin = ug_amd.llama.rope_tables(hip, cfg)
+    cos_h, sin_h = cos.data_vec().reshape(-1, HD // 2), sin.data_vec().reshape(-1, HD // 2)
+    pos = LB.copy(np.zeros(1, np.int32), (1,), hip)
+
+    def heads_first(x, n):
+        return np.ascontiguousarray(x.reshape(T, n, HD).transpose(1, 0, 2))
+
+    q64 = _rope_f64(heads_first(qf, HEADS).astype(np.float64), cos_h, sin_h, 0, False)
+    k64 = _rope_f64(heads_first(kx, nkv).astype(np.float64), cos_h, sin_h, 0, False)
+    v64 = heads_first(vx, nkv).astype(np.float64)
+    keep = np.arange(T)[None, :] <= np.arange(T)[:, None]
+    truth = np.empty((HEADS, T, HD))
+    for h in range(HEADS):
+        sc = q64[h] @ k64[h // (HEADS // nkv)].T * scale
+        sc = np.where(keep, sc, -np.inf)
+        e = np.exp(sc - sc.max(-1, keepdims=True))
+        truth[h] = (e / e.sum(-1, keepdims=True)) @ v64[h // (HEADS // nkv)]
+    truth = truth.transpose(1, 0, 2).reshape(1, T, HEADS * HD)
+    tol = 2e-5 * float(np.abs(truth).max())
+
+    # the reference's op-by-op chain on the HIP device
+    ll = ug_amd.llama
+    q = hip_ops.rope(LB.copy(qf, qf.shape, hip).split_dim(2, HEADS, HD).transpose(2, 1), cos, sin, pos)
+    k = hip_ops.rope(LB.copy(kx, kx.shape, hip).split_dim(2, nkv, HD).transpose(2, 1), cos, sin, pos)
+    v = LB.copy(vx, vx.shape, hip).split_dim(2, nkv, HD).transpose(2, 1)
+    k, v = ll.repeat(k, 1, HEADS // nkv), ll.repeat(v, 1, HEADS // nkv)
+    att = q.matmul_t(k).binary("mul", LB.cst(scale, (), hip).broadcast((1, HEADS, T, T)))
+    att = hip_ops.custom_softmax(hip_ops.causal_mask(att))
+    chain = att.matmul(v).transpose(2, 1).merge_dims(2).data_vec().reshape(1, T, HEADS * HD)
+    np.testing.assert_allclose(chain, truth, rtol=0, atol=tol)
+
+    # one kernel over preallocated caches (rows past T never read)
+    kc = np.zeros((1, nkv, cap, HD), np.float32)
+    vc = np.full((1, nkv, cap, HD), np.nan, np.float32)
+    kc[0, :, :T] = heads_first(kx, nkv)
+    vc[0, :, :T] = heads_first(vx, nkv)
+    kc[0, :, T:] = np.nan
+    kc_l = hip_ops.kv_append(LB.copy(kc, kc.shape, hip), 0, LB.copy(kx, kx.shape, hip), cos, sin, pos, False)
+    got = hip_ops.attention_cached(LB.copy(qf, qf.shape, hip), kc_l, LB.copy(vc, vc.shape, hip), T, scale, cos, sin, pos, False).data_vec().reshape(truth.shape)
+    np.testing.assert_allclose(got, truth, rtol=0, atol=tol)
+    np.testing.assert_allclose(got, chain, rtol=0, atol=tol)
+
+
+# ---- config 5: 22 layers, 128 prompt ids, 128 greedy steps ------------------------------------------------------------
+# Logits of this random-init model are about 0.1 in size and follow from 22 layers of f32 sums in two different
+# orders (gcc's and the GPU's); LOGIT_TOL bounds their measured difference with a wide margin (observed: below 2e-6).
+# Ids must agree wherever the oracle's own gap between its two best logits is larger than TIE_MARGIN = 2 LOGIT_TOL;
+# inside that band the two devices hold a tie and either id is a correct greedy choice.
+LOGIT_TOL = 2e-5
+TIE_MARGIN = 2 * LOGIT_TOL
+
+
+def _config5_fixture():
+    with open(os.path.join(HERE, "golden", "llama_config5_greedy.json")) as f:
+        return json.load(f)
+
+
+@pytest.mark.parametrize("variant", ["f32_level0", "f32_level3", "bf16_rounded_level0", "bf16_matrices_level3"])
+def test_config5_full_depth_greedy_ids(hip, hip_ops, variant):
+    """BASELINE config 5 as stated against the oracle's run of the reference's op-by-op graph (the fixture):
+    free-running ids equal up to the first position where the oracle itself holds a near-tie, and -- fed the
+    oracle's ids, so that every position sees the same inputs -- the same id at every position outside the tie band,
+    top logits within LOGIT_TOL and margins within 2 LOGIT_TOL."""
+    fx = _config5_fixture()
+    run = fx["runs"]["f32" if variant.startswith("f32") else "bf16_rounded"]
+    ids_o, top_o, mar_o = np.array(run["ids"], np.int32), np.array(run["top1"]), np.array(run["margin"])
+    n_steps = fx["steps"]
+    cfg = ug_amd.LlamaConfig(num_hidden_layers=fx["config"]["num_hidden_layers"])
+    prompt = rng.token_ids(fx["prompt"]["seed"], fx["prompt"]["n"], cfg.vocab_size)
+    level = 3 if variant.endswith("level3") else 0
+    hip.set_zero_fill(False)
+    try:
+        model = ug_amd.LlamaModel(hip, hip_ops, cfg, custom_softmax=True, seed=fx["weights"]["seed"], std=fx["weights"]["std"], round_bf16=not variant.startswith("f32"),
+                                  fused_attention=level, bf16_matrices=variant.startswith("bf16_matrices"))
+        free, st_free = model.generate(prompt, n_steps)
+        forced, st = model.generate(prompt, n_steps, forced=ids_o[:-1])
+    finally:
+        hip.set_zero_fill(True)
+    clear = mar_o > TIE_MARGIN
+    differs = np.flatnonzero(free != ids_o)
+    first = int(differs[0]) if differs.size else None
+    print(f"config 5 {variant}: free-running ids equal at {int((free == ids_o).sum())}/{ids_o.size} positions, first difference {first}; "
+          f"fed the oracle's ids: equal at {int((forced == ids_o).sum())}/{ids_o.size}, {int(clear.sum())} positions outside the tie band, "
+          f"max |top1 - oracle| {float(np.abs(st['top1'] - top_o).max()):.3g}, max |margin - oracle| {float(np.abs(st['margins'] - mar_o).max()):.3g}, "
+          f"oracle margins min {mar_o.min():.3g} median {np.median(mar_o):.3g}", flush=True)
+    for i in range(ids_o.size):
+        print(f"  pos {i:3d} oracle id {ids_o[i]:5d} margin {mar_o[i]:.3e} | hip (same inputs) id {forced[i]:5d} margin {st['margins'][i]:.3e} | hip free id {free[i]:5d}", flush=True)
+    assert np.all(forced[clear] == ids_o[clear])
+    np.testing.assert_allclose(st["top1"], top_o, rtol=0, atol=LOGIT_TOL)
+    np.testing.assert_allclose(st["margins"], mar_o, rtol=0, atol=2 * LOGIT_TOL)
+    if first is not None:
+        assert mar_o[first] <= TIE_MARGIN, f"free-running ids part at position {first} where the oracle's margin is {mar_o[first]}"
+    assert clear.sum() >= ids_o.size // 2, "most positions should lie outside the tie band for the id comparison to mean something"
+
+
+def test_generate_refuses_ids_outside_the_vocabulary(hip, hip_ops):
+    cfg = ug_amd.LlamaConfig(hidden_size=128, intermediate_size=320, max_position_embeddings=64, num_attention_heads=4, num_key_value_heads=2,
+                             num_hidden_layers=1, vocab_size=512)
+    model = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=0.3)
+    with pytest.raises(ug_amd.UgError, match="outside the vocabulary"):
+        model.generate(np.array([1, 512, 3], np.int32), 2)
+    with pytest.raises(ug_amd.UgError, match="outside the vocabulary"):
+        model.generate(np.array([1, -1], np.int32), 2)
+    with pytest.raises(ug_amd.UgError, match="outside the vocabulary"):
+        model.generate(np.array([1, 2], np.int32), 2, forced=np.array([5, 9999], np.int32))
+    toks, _ = model.generate(np.array([1, 511], np.int32), 2)
+    assert toks.size == 3

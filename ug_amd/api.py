@@ -50,6 +50,7 @@ def ughip_lib():
     if _ughip is None:
         lib = _load("libughip.so")
         lib.ughip_last_error.restype = C.c_char_p
+        lib.ughip_last_kernel.restype = C.c_char_p
         lib.ughip_slice_len.restype = C.c_size_t
         lib.ughip_slice_ptr.restype = C.c_void_p
         lib.ughip_func_source.restype = C.c_size_t
@@ -111,7 +112,7 @@ def host_lib():
         for f in ("ugh_slice_len", "ugh_lb_rank", "ugh_lb_elem_count", "ugh_schedule_n_items", "ugh_schedule_item_n_args",
                   "ugh_compiled_n_funcs", "ugh_cache_size"):
             getattr(lib, f).restype = C.c_size_t
-        for f in ("ugh_cache_new", "ugh_device_raw_hip", "ugh_func_raw_hip", "ugh_compiled_func_raw_hip"):
+        for f in ("ugh_cache_new", "ugh_device_raw_hip", "ugh_func_raw_hip", "ugh_compiled_func_raw_hip", "ugh_slice_raw_hip"):
             getattr(lib, f).restype = C.c_void_p
         for f in ("ugh_device_free", "ugh_slice_free", "ugh_func_free", "ugh_ssa_free", "ugh_lb_free", "ugh_schedule_free", "ugh_cache_free",
                   "ugh_compiled_free", "ugh_llama_ops_free", "ugh_llama_model_free", "ugh_lb_dims", "ugh_ssa_set_launch"):
@@ -158,6 +159,10 @@ class Slice(_Handle):
     @property
     def dtype(self):
         return host_lib().ugh_slice_dtype(_p(self.h))
+
+    def raw(self):
+        """The ughip_slice* of a HIP slice, for direct calls into libughip.so (0 on other devices)."""
+        return host_lib().ugh_slice_raw_hip(_p(self.h)) or 0
 
     def copy_host_to_device(self, src, dtype=None):
         src = np.ascontiguousarray(src)
@@ -322,6 +327,11 @@ class Device(_Handle):
 
     def raw_hip(self):
         return host_lib().ugh_device_raw_hip(_p(self.h))
+
+
+def last_kernel():
+    """The hand-written kernel this thread's last Device.matmul launched (ughip_last_kernel)."""
+    return ughip_lib().ughip_last_kernel().decode()
 
 
 def hip_device(ordinal=0):
@@ -847,13 +857,22 @@ class LlamaModel(_Handle):
             _chk(host_lib().ugh_llama_model_store_matrices_bf16(_p(self.h)))
         return self
 
-    def generate(self, prompt, n_steps):
+    def generate(self, prompt, n_steps, forced=None):
         """Prefill over `prompt`, then n_steps greedy single-token steps.  Returns
-        (n_steps + 1 token ids, {"prefill_ms", "decode_ms", "margins"})."""
+        (n_steps + 1 token ids, {"prefill_ms", "decode_ms", "margins", "top1"}).
+        forced (n_steps ids): decode step i is fed forced[i - 1] instead of the id picked one step earlier."""
         prompt = np.ascontiguousarray(prompt, dtype=np.int32)
         toks = np.zeros(n_steps + 1, dtype=np.int32)
         margins = np.zeros(n_steps + 1, dtype=np.float32)
+        top1 = np.zeros(n_steps + 1, dtype=np.float32)
         pre, dec = C.c_double(), C.c_double()
-        _chk(host_lib().ugh_llama_generate(_p(self.h), prompt.ctypes.data_as(C.c_void_p), C.c_size_t(prompt.size), C.c_size_t(n_steps),
-                                           toks.ctypes.data_as(C.c_void_p), C.byref(pre), C.byref(dec), margins.ctypes.data_as(C.c_void_p)))
-        return toks, {"prefill_ms": pre.value, "decode_ms": dec.value, "margins": margins}
+        fp = None
+        if forced is not None:
+            forced = np.ascontiguousarray(forced, dtype=np.int32)
+            if forced.size != n_steps:
+                raise ValueError(f"forced: expected {n_steps} ids, got {forced.size}")
+            fp = forced.ctypes.data_as(C.c_void_p)
+        _chk(host_lib().ugh_llama_generate_ex(_p(self.h), prompt.ctypes.data_as(C.c_void_p), C.c_size_t(prompt.size), C.c_size_t(n_steps), fp,
+                                              toks.ctypes.data_as(C.c_void_p), C.byref(pre), C.byref(dec), margins.ctypes.data_as(C.c_void_p),
+                                              top1.ctypes.data_as(C.c_void_p)))
+        return toks, {"prefill_ms": pre.value, "decode_ms": dec.value, "margins": margins, "top1": top1}

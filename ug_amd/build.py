@@ -32,11 +32,31 @@ def _run(cmd):
         raise RuntimeError("build step failed: " + " ".join(cmd))
 
 
-def build_ughip():
+UGHIP_SOURCES = ("runtime.cpp", "lower_hip.cpp", "llama_ops.hip", "matmul.hip", "gemm_tiled.hip", "attention.hip", "fused_linear.hip", "convert.hip")
+
+
+def build_ughip(only_changed=False):
+    """One object per source file, compiled side by side, then one link.  only_changed (a developer's
+    shortcut, `python -m ug_amd.build ughip-changed`): keep objects newer than their source and every header."""
+    from concurrent.futures import ThreadPoolExecutor
     os.makedirs(LIB, exist_ok=True)
     src = os.path.join(CSRC, "ughip")
-    files = [os.path.join(src, f) for f in ("runtime.cpp", "lower_hip.cpp", "llama_ops.hip", "matmul.hip", "gemm_tiled.hip", "attention.hip", "fused_linear.hip", "convert.hip")]
-    _run([os.path.join(ROCM, "bin", "hipcc")] + HIP_FLAGS + ["-shared", "-I" + INC, "-I" + src] + files +
+    obj_dir = os.path.join(LIB, "obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    headers = [os.path.join(src, f) for f in os.listdir(src) if f.endswith(".h")] + [os.path.join(INC, f) for f in os.listdir(INC)]
+    newest_header = max(os.path.getmtime(h) for h in headers)
+    jobs, objs = [], []
+    for f in UGHIP_SOURCES:
+        o = os.path.join(obj_dir, f.rsplit(".", 1)[0] + ".o")
+        objs.append(o)
+        path = os.path.join(src, f)
+        if only_changed and os.path.exists(o) and os.path.getmtime(o) > max(os.path.getmtime(path), newest_header):
+            continue
+        jobs.append([hipcc] + HIP_FLAGS + ["-c", "-I" + INC, "-I" + src, path, "-o", o])
+    with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as pool:
+        list(pool.map(_run, jobs))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs +
          ["-L" + os.path.join(ROCM, "lib"), "-lhiprtc", "-Wl,-rpath," + os.path.join(ROCM, "lib"), "-o", os.path.join(LIB, "libughip.so")])
 
 
@@ -62,4 +82,4 @@ def build_all():
 if __name__ == "__main__":
     what = sys.argv[1:] or ["all"]
     for w in what:
-        {"all": build_all, "ughip": build_ughip, "host": build_host, "oracle": build_oracle}[w]()
+        {"all": build_all, "ughip": build_ughip, "ughip-changed": lambda: build_ughip(True), "host": build_host, "oracle": build_oracle}[w]()

@@ -100,6 +100,11 @@ int ugh_device_convert(void* d, void* dst, void* src, int* done) {
   return guard([&] { *done = dev_of(d)->convert(*static_cast<Slice*>(dst), *static_cast<Slice*>(src)) ? 1 : 0; });
 }
 void ugh_slice_free(void* s) { delete static_cast<Slice*>(s); }
+// The ughip_slice behind a slice of the HIP device (null for any other device): for callers that go to the C ABI directly.
+void* ugh_slice_raw_hip(void* s) {
+  HipSlice* h = s ? dynamic_cast<HipSlice*>(static_cast<Slice*>(s)) : nullptr;
+  return h ? h->raw() : nullptr;
+}
 size_t ugh_slice_len(void* s) { return static_cast<Slice*>(s)->len(); }
 int ugh_slice_dtype(void* s) { return (int)static_cast<Slice*>(s)->dtype(); }
 int ugh_slice_h2d(void* s, const void* src, int dtype, size_t len) {
@@ -791,6 +796,20 @@ int ugh_llama_generate(void* m, const int32_t* prompt, size_t n_prompt, size_t n
     if (prefill_ms) *prefill_ms = st.prefill_ms;
     if (decode_ms) *decode_ms = st.decode_ms;
     if (margins) std::memcpy(margins, st.top1_margin.data(), st.top1_margin.size() * sizeof(float));
+  });
+}
+int ugh_llama_generate_ex(void* m, const int32_t* prompt, size_t n_prompt, size_t n_steps, const int32_t* forced, int32_t* out_tokens, double* prefill_ms,
+                          double* decode_ms, float* margins, float* top1_values) {
+  return guard([&] {
+    ug_llama::GenerateStats st;
+    std::vector<int32_t> p(prompt, prompt + n_prompt), f;
+    if (forced) f.assign(forced, forced + n_steps);
+    std::vector<int32_t> toks = ug_llama::generate_greedy(*static_cast<ug_llama::Model*>(m), p, n_steps, &st, forced ? &f : nullptr);
+    std::memcpy(out_tokens, toks.data(), toks.size() * sizeof(int32_t));
+    if (prefill_ms) *prefill_ms = st.prefill_ms;
+    if (decode_ms) *decode_ms = st.decode_ms;
+    if (margins) std::memcpy(margins, st.top1_margin.data(), st.top1_margin.size() * sizeof(float));
+    if (top1_values) std::memcpy(top1_values, st.top1_value.data(), st.top1_value.size() * sizeof(float));
   });
 }
 int ugh_synthetic_weights(uint64_t seed, float std, int round_bf16, const char* name, size_t n, float* out) {

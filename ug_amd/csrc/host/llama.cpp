@@ -878,7 +878,8 @@ namespace {
 // the launches of step i + 1 are issued while step i still runs.  Inputs that have to come from
 // the host (prompt, positions) are uploaded before the first launch, because an upload waits for
 // the stream.  Ids and the two largest logits of every step are read once at the end.
-std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vector<int32_t>& prompt, size_t n_steps, GenerateStats* stats) {
+std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vector<int32_t>& prompt, size_t n_steps, GenerateStats* stats,
+                                            const std::vector<int32_t>* forced) {
   using clock = std::chrono::steady_clock;
   const DevicePtr& dev = model.device();
   const Ops& ops = model.ops();
@@ -897,8 +898,17 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
   for (size_t i = 0; i < total; ++i) {
     int32_t p32 = i == 0 ? 0 : (int32_t)(prompt.size() + i - 1);
     pos[i] = LB::copy(&p32, DType::I32, 1, Shape({1, 1}), dev);
-    tokens[i + 1] = LB::alloc_uninit(DType::I32, Shape({1, 1}), dev);  // written by the argmax of step i
-    tokens[i + 1].maybe_allocate_uninit();
+    if (forced && i < n_steps) {
+      tokens[i + 1] = LB::copy(&(*forced)[i], DType::I32, 1, Shape({1, 1}), dev);  // the input of step i + 1 is given
+    } else {
+      tokens[i + 1] = LB::alloc_uninit(DType::I32, Shape({1, 1}), dev);  // written by the argmax of step i
+      tokens[i + 1].maybe_allocate_uninit();
+    }
+  }
+  LB picked;  // with forced inputs the argmax still runs and is recorded, but writes its id here
+  if (forced) {
+    picked = LB::alloc_uninit(DType::I32, Shape({1, 1}), dev);
+    picked.maybe_allocate_uninit();
   }
 
   auto build = [&](size_t i, PreparedStep& st) {
@@ -906,7 +916,7 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
     st.t = i == 0 ? prompt.size() : 1;
     st.tokens = tokens[i];
     LB logits = model.fwd(st.tokens, pos[i], cache);
-    st.logits = ops.argmax_into(tokens[i + 1], logits, st.t - 1, ids, vals, i);
+    st.logits = ops.argmax_into(forced ? picked : tokens[i + 1], logits, st.t - 1, ids, vals, i);
     auto t1 = clock::now();
     Schedule schedule = Schedule::create_one(st.logits);
     auto t2 = clock::now();
@@ -973,7 +983,10 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
     stats->decode_ms = ms_between(t_decode, clock::now());
     std::vector<float> v(2 * total);
     vals.data_vec(v.data(), DType::F32);
-    for (size_t i = 0; i < total; ++i) stats->top1_margin.push_back(v[2 * i] - v[2 * i + 1]);
+    for (size_t i = 0; i < total; ++i) {
+      stats->top1_margin.push_back(v[2 * i] - v[2 * i + 1]);
+      stats->top1_value.push_back(v[2 * i]);
+    }
     stats->step_ms.assign(n_steps, n_steps ? stats->decode_ms / (double)n_steps : 0.0);  // steps overlap: only their mean is observable
   }
   return out;
@@ -989,14 +1002,25 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
 // known.  Every value computed is the same as in the reference's order.
 // UG_LLAMA_NO_OVERLAP=1 keeps everything on the calling thread.
 // UG_LLAMA_HOST_ARGMAX=1 keeps this read-back loop on a device that could pick the token itself.
-std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32_t>& prompt, size_t n_steps, GenerateStats* stats) {
+std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32_t>& prompt, size_t n_steps, GenerateStats* stats,
+                                     const std::vector<int32_t>* forced) {
   using clock = std::chrono::steady_clock;
   const Config& cfg = model.config();
   const DevicePtr& dev = model.device();
   if (prompt.empty()) bail("empty prompt");
   if (prompt.size() + n_steps > cfg.max_position_embeddings) bail("prompt + steps exceed max_position_embeddings");
+  if (forced && forced->size() != n_steps) bail("forced ids: expected one per decode step (" + std::to_string(n_steps) + "), got " + std::to_string(forced->size()));
+  // The embedding gather forms its source offset from the id on the device, where nothing can check it
+  // (ids picked by the argmax are in range by construction; these come from the caller).
+  auto check_ids = [&](const std::vector<int32_t>& ids, const char* what) {
+    for (size_t i = 0; i < ids.size(); ++i)
+      if (ids[i] < 0 || (size_t)ids[i] >= cfg.vocab_size)
+        bail(std::string(what) + " id " + std::to_string(ids[i]) + " at index " + std::to_string(i) + " is outside the vocabulary of " + std::to_string(cfg.vocab_size));
+  };
+  check_ids(prompt, "prompt");
+  if (forced) check_ids(*forced, "forced");
   if (dev->runs_async() && model.ops().device_argmax() && getenv("UG_LLAMA_HOST_ARGMAX") == nullptr && getenv("UG_LLAMA_NO_OVERLAP") == nullptr)
-    return generate_greedy_queued(model, prompt, n_steps, stats);
+    return generate_greedy_queued(model, prompt, n_steps, stats, forced);
   std::vector<Cache> cache = model.new_cache();
   CompilationCache ccache;
   std::vector<int32_t> out;
@@ -1098,7 +1122,7 @@ std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32
       }
     }
     if (more) {
-      int32_t id = (int32_t)best;
+      int32_t id = forced ? (*forced)[step] : (int32_t)best;
       next.tokens.data()->slice->copy_host_to_device(&id, DType::I32, 1);
     }
     auto t4 = clock::now();
@@ -1117,6 +1141,7 @@ std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32
         stats->step_ms.push_back(ms);
       }
       stats->top1_margin.push_back(last[best] - second);
+      stats->top1_value.push_back(last[best]);
     }
     pos_v += cur.t;
     out.push_back((int32_t)best);

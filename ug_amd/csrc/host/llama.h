@@ -213,7 +213,12 @@ struct GenerateStats {
   double prefill_ms = 0, decode_ms = 0;
   std::vector<double> step_ms;
   std::vector<float> top1_margin;  // logit gap between the best and second-best token per step
+  std::vector<float> top1_value;   // the best token's logit per step
 };
-std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32_t>& prompt, size_t n_steps, GenerateStats* stats);
+// forced != nullptr (n_steps ids): decode step i is fed (*forced)[i - 1] instead of the id picked at step i - 1, so that two
+// devices can be compared position by position on identical inputs; the ids returned are still each step's argmax.
+// Ids outside [0, vocab_size) in `prompt` or `forced` are refused (they would index the embedding table out of bounds).
+std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32_t>& prompt, size_t n_steps, GenerateStats* stats,
+                                     const std::vector<int32_t>* forced = nullptr);
 
 }  // namespace ug_llama

@@ -18,9 +18,12 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
+#include <cstdio>
 #include <cstdlib>
 
 #include "gemm.h"
+#include "internal.h"
 #include "ughip.h"
 
 namespace ughip {
@@ -534,17 +537,24 @@ __global__ void __launch_bounds__(256) gemm_split_reduce(const float* __restrict
   o[3] = (T)s.w;
 }
 
+// Raises the kernel's dynamic LDS limit once per device (`done`: one bit per device ordinal; devices past 63 pay the call every launch).
+hipError_t allow_lds(const void* kernel, int lds_bytes, std::atomic<unsigned long long>& done) {
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev)) return e;
+  const unsigned long long bit = dev < 64 ? 1ull << dev : 0;
+  if (bit && (done.load(std::memory_order_relaxed) & bit)) return hipSuccess;
+  if (hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes)) return e;
+  done.fetch_or(bit, std::memory_order_relaxed);
+  return hipSuccess;
+}
+
 template <typename T, int B_NK, int BM, int BN, int NT, bool SPLIT, bool RAGGED = false>
 hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch, int nsplit, float* ws) {
   constexpr int LDS_BYTES = 2 * (BM + BN) * CHUNKS * 16;
   constexpr int BK = Elt<T>::BK;
-  static bool configured = false;
+  static std::atomic<unsigned long long> configured{0};  // one bit per device: the attribute is per device
   auto kernel = gemm_tiled<T, B_NK, BM, BN, NT, SPLIT, RAGGED>;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  if (hipError_t e = allow_lds(reinterpret_cast<const void*>(kernel), LDS_BYTES, configured)) return e;
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const int kt = p.K / BK, kt_per = SPLIT ? (kt + nsplit - 1) / nsplit : kt;
   if (SPLIT) nsplit = (kt + kt_per - 1) / kt_per;  // no empty slab
@@ -566,13 +576,9 @@ template <typename T>
 hipError_t launch_dma256(hipStream_t stream, const MMArgs& p, size_t batch) {
   constexpr int BM = 256, BN = 256, NT = 512, STAGES = 2;
   constexpr int LDS_BYTES = STAGES * (BM + BN) * CHUNKS * 16;
-  static bool configured = false;
+  static std::atomic<unsigned long long> configured{0};
   auto kernel = gemm_tiled_dma<T, BM, BN, NT, STAGES>;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  if (hipError_t e = allow_lds(reinterpret_cast<const void*>(kernel), LDS_BYTES, configured)) return e;
   const int tiles_m = p.M / BM, tiles_n = p.N / BN;
   const size_t total = batch * (size_t)tiles_m * tiles_n;
   kernel<<<dim3((unsigned)total), dim3(NT), LDS_BYTES, stream>>>(p, tiles_m, tiles_n, total % 8 == 0 ? 1 : 0);
@@ -676,6 +682,16 @@ hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, siz
   const int s = pick_shape(p, batch, dtype);
   if (s < 0) return hipErrorInvalidValue;
   const int nsplit = s == 3 ? 1 : pick_split(dtype, p, batch, s);
+  {
+    const char* tn = rhs_bf16 ? "f32xbf16" : dtype == UGHIP_F32 ? "f32" : dtype == UGHIP_F16 ? "f16" : "bf16";
+    const bool ragged = s != 0 && s != 3 && (p.M % kShapes[s][0] || p.N % kShapes[s][1]);
+    char split[32] = "";
+    if (nsplit > 1) snprintf(split, sizeof split, ",splitK=%d", nsplit);
+    if (s == 3) note_kernel("gemm_tiled_dma<%s,NT,256x256,512t>", tn);
+    else
+      note_kernel("gemm_tiled<%s,%s,%dx%d,%dt%s%s>", tn, nt ? "NT" : "NN", kShapes[s][0], kShapes[s][1], s == 0 && !getenv("UGHIP_GEMM_4WAVES") ? 512 : 256,
+                  ragged ? ",ragged" : "", split);
+  }
   if (nsplit > 1) {
     if (!workspace) return hipErrorInvalidValue;
     if (rhs_bf16) return launch_shape<float, 2, true>(stream, p, batch, s, nsplit, workspace);

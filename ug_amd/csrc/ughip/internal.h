@@ -48,6 +48,8 @@ namespace ughip {
 
 // Records the thread-local message returned by ughip_last_error() and returns `code`.
 int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+// Records what ughip_last_kernel() returns: the hand-written kernel the calling thread launched last.
+void note_kernel(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 int device_activate(ughip_device* d);
 const char* dtype_name(int dt);
 

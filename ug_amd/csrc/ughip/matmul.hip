@@ -445,11 +445,14 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
                        "start on 8-byte boundaries (got m %zu, n %zu, k %zu, rhs strides %lld, %lld)",
                        m, n, k, p.b_rs, p.b_cs);
   }
+  const char* tn = f32 ? "f32" : dst->dtype == UGHIP_F16 ? "f16" : "bf16";
   if (!mixed && gemv_nt_ok) {
+    note_kernel("gemv_nt<%s>", tn);
     if (f32) launch_gemv_nt_any<float>(st, p, b);
     else if (dst->dtype == UGHIP_F16) launch_gemv_nt_any<_Float16>(st, p, b);
     else launch_gemv_nt_any<__bf16>(st, p, b);
   } else if (!mixed && gemv_nn_ok) {
+    note_kernel("gemv_nn<f32>");
     dim3 grid((unsigned)((n + 63) / 64), 1, (unsigned)b);
     if (m == 1) gemv_nn_f32<1><<<grid, 1024, 0, st>>>(p);
     else if (m <= 4) gemv_nn_f32<4><<<grid, 1024, 0, st>>>(p);
@@ -471,6 +474,7 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
   } else {
     dim3 grid((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64), (unsigned)b);
     if (grid.y > 65535 || b > 65535) return set_error(UGHIP_ERR_INVALID, "matmul: m or batch too large for this kernel");
+    note_kernel("gemm_any<%s>", tn);
     if (f32) gemm_f32_any<<<grid, 256, 0, st>>>(p);
     else if (dst->dtype == UGHIP_F16) gemm_half_any<_Float16><<<grid, 256, 0, st>>>(p);
     else gemm_half_any<__bf16><<<grid, 256, 0, st>>>(p);

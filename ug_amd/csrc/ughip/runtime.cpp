@@ -30,6 +30,17 @@ int set_error(int code, const char* fmt, ...) {
   return code;
 }
 
+static thread_local std::string g_last_kernel;
+
+void note_kernel(const char* fmt, ...) {
+  char buf[256];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_last_kernel = buf;
+}
+
 }  // namespace ughip
 
 using namespace ughip;
@@ -76,6 +87,7 @@ static size_t size_class(size_t bytes) {
 extern "C" {
 
 const char* ughip_last_error(void) { return g_last_error.c_str(); }
+const char* ughip_last_kernel(void) { return g_last_kernel.c_str(); }
 
 int ughip_use_grid(void) { return 0; }
 
@@ -158,6 +170,7 @@ int ughip_alloc(ughip_device* dev, int dtype, size_t len, ughip_slice** out) {
   s->dev = dev;
   s->dtype = dtype;
   s->len = len;
+  if (len > SIZE_MAX / dtype_size(dtype)) return set_error(UGHIP_ERR_INVALID, "alloc: %zu elements of %s overflow size_t", len, dtype_name(dtype));
   size_t bytes = len * dtype_size(dtype);
   if (bytes) {
     size_t cls = size_class(bytes);
@@ -189,7 +202,17 @@ int ughip_alloc(ughip_device* dev, int dtype, size_t len, ughip_slice** out) {
       std::lock_guard<std::mutex> g(dev->mu);
       dev->live_bytes += cls;
     }
-    if (dev->zero_fill) HIPCHK(hipMemsetAsync(s->ptr, 0, bytes, dev->stream));
+    if (dev->zero_fill) {
+      hipError_t e = hipMemsetAsync(s->ptr, 0, bytes, dev->stream);
+      if (e != hipSuccess) {
+        // the block goes back to the pool and out of the live count, as ughip_free would do
+        std::lock_guard<std::mutex> g(dev->mu);
+        dev->pool[cls].push_back(s->ptr);
+        dev->pool_bytes += cls;
+        dev->live_bytes -= cls;
+        return set_error(UGHIP_ERR_HIP, "hipMemsetAsync(%zu): %s", bytes, hipGetErrorString(e));
+      }
+    }
   }
   ughip_device_retain(dev);
   *out = s.release();
@@ -342,8 +365,12 @@ int ughip_compile(ughip_device* dev, const ughip_ssa* ssa, const char* name, ugh
       if (int rc = rtc_compile(f->low.source, dev->arch, &code)) return rc;
       CachedModule cm;
       HIPCHK(hipModuleLoadData(&cm.module, code.data()));
-      HIPCHK(hipModuleGetFunction(&cm.function, cm.module, f->low.entry.c_str()));
-      if (!f->low.entry2.empty()) HIPCHK(hipModuleGetFunction(&cm.function2, cm.module, f->low.entry2.c_str()));
+      hipError_t e = hipModuleGetFunction(&cm.function, cm.module, f->low.entry.c_str());
+      if (e == hipSuccess && !f->low.entry2.empty()) e = hipModuleGetFunction(&cm.function2, cm.module, f->low.entry2.c_str());
+      if (e != hipSuccess) {
+        hipModuleUnload(cm.module);
+        return set_error(UGHIP_ERR_HIP, "hipModuleGetFunction(%s): %s", f->low.entry.c_str(), hipGetErrorString(e));
+      }
       it = dev->modules.emplace(f->low.source, cm).first;
     }
     f->function = it->second.function;
