@@ -527,6 +527,21 @@ def test_matmul_errors(hip):
         hip.matmul(dst, a, b, (1, 2, 2, 4), ((2, 4), (4, 1), 0), ((4, 2), (2, 1), 0))
 
 
+def test_a_failed_call_does_not_surface_at_the_next_launch(hip):
+    """hipModuleGetFunction failing inside ughip_compile_source stays behind as the thread's last HIP error; the check
+    after the next kernel launch (hipGetLastError) must not report it against that launch."""
+    lib = ug_amd.ughip_lib()
+    src = b'extern "C" __global__ void present(float* x) { x[0] = 1.f; }'
+    out = C.c_void_p()
+    dt = (C.c_int * 1)(int(F32))
+    rc = lib.ughip_compile_source(C.c_void_p(hip.raw_hip()), src, b"absent", C.c_size_t(1), dt, C.c_uint(1), C.c_uint(64), C.c_uint(0), C.byref(out))
+    assert rc != 0 and b"no kernel 'absent'" in lib.ughip_last_error()
+    b, m, n, k = 1, 128, 256, 2048   # a split-K product: tile kernel and fold, both checked with hipGetLastError
+    a = np.floor(rng.uniform_pm1(33, b * m * k) * 4).reshape(b, m, k)
+    w = np.floor(rng.uniform_pm1(34, b * k * n) * 4).reshape(b, k, n)
+    np.testing.assert_array_equal(_raw_matmul(hip, F32, a, w, True), (a.astype(np.float64) @ w.astype(np.float64)).astype(np.float32))
+
+
 # ---- error behaviour at the boundary ------------------------------------------------------------------------------------------
 def test_run_checks_bounds_aliasing_and_dtypes(hip):
     k = SsaKernel.sample("simple_add", 6)

@@ -27,6 +27,10 @@ int set_error(int code, const char* fmt, ...) {
   vsnprintf(buf, sizeof buf, fmt, ap);
   va_end(ap);
   g_last_error = buf;
+  // A failed HIP call also stays behind as the thread's "last error", and the next hipGetLastError() -- the
+  // check after a <<<>>> launch -- would report it against a launch that went fine.  The failure is on record
+  // here, so the runtime's copy is dropped.
+  (void)hipGetLastError();
   return code;
 }
 
@@ -187,6 +191,7 @@ int ughip_alloc(ughip_device* dev, int dtype, size_t len, ughip_slice** out) {
       hipError_t e = hipMalloc(&s->ptr, cls);
       if (e != hipSuccess) {
         // Give cached blocks back to the driver and retry once.
+        (void)hipGetLastError();  // the retry may succeed: the failed attempt must not surface at a later launch check
         std::lock_guard<std::mutex> g(dev->mu);
         hipStreamSynchronize(dev->stream);
         for (auto& kv : dev->pool)
