@@ -231,6 +231,21 @@ int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs,
                  const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset,
                  const size_t* rhs_dims, const size_t* rhs_strides, size_t rhs_offset);
 
+/* ughip_matmul for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and
+ * the same bits as ughip_matmul, but it calls no hipMalloc / hipFree: products that split K (skinny
+ * shapes with a long k, e.g. the projections of a 128-token prefill) put their f32 partial tiles into a
+ * static device array of UGHIP_MATMUL_NOALLOC_SCRATCH_BYTES that each GPU holds until the process ends,
+ * instead of the grown-on-demand block ughip_matmul keeps per device.  A product whose partial tiles
+ * need more is refused with UGHIP_ERR_UNSUPPORTED (the message gives both sizes).  All calls on one GPU
+ * share that GPU's array: calls that overlap on one GPU (two threads, two streams) race; calls of one
+ * thread are ordered by the device's stream.  Nothing in the array has to start at zero. */
+#define UGHIP_MATMUL_NOALLOC_SCRATCH_BYTES (64u << 20)
+int ughip_matmul_noalloc(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs,
+                         const ughip_slice* rhs, size_t b, size_t m, size_t n, size_t k, size_t rank,
+                         const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset,
+                         const size_t* rhs_dims, const size_t* rhs_strides, size_t rhs_offset);
+
 /* ---- ug-llama custom ops (ug-llama/src/main.rs:22-28; oracle cpu_ops.rs:6-167) ------- */
 /* rope / rope_i (cuda_ops.rs:17-104): src, dst are [bh, t*d] f32, cos/sin [max_pos, d/2]
  * f32, pos i32 (only pos[0] is read, cpu_ops.rs:67,100). */

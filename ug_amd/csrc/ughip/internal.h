@@ -32,6 +32,8 @@ struct ughip_device {
   // device's one stream, freed with the device.
   void* gemm_ws = nullptr;
   size_t gemm_ws_bytes = 0;
+  // This device's address of the static array behind ughip_matmul_noalloc (hipGetSymbolAddress at device creation).
+  void* static_scratch = nullptr;
   // Partial rows of single-query attention over a long cache (one per head and key range); same life cycle.
   void* att_ws = nullptr;
   size_t att_ws_bytes = 0;
@@ -51,6 +53,7 @@ int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3
 // Records what ughip_last_kernel() returns: the hand-written kernel the calling thread launched last.
 void note_kernel(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 int device_activate(ughip_device* d);
+int matmul_scratch_setup(ughip_device* dev);  // matmul.hip
 const char* dtype_name(int dt);
 
 }  // namespace ughip

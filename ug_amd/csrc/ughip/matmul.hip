@@ -389,9 +389,26 @@ bool batch_stride(size_t rank, const size_t* dims, const size_t* strides, size_t
 
 }  // namespace
 
-extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs, const ughip_slice* rhs, size_t b, size_t m, size_t n,
-                            size_t k, size_t rank, const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset, const size_t* rhs_dims,
-                            const size_t* rhs_strides, size_t rhs_offset) {
+// Partial tiles of ughip_matmul_noalloc's split-K products.  Every GPU the library runs on holds its own
+// copy of this array at its own address for the life of the process.  In host code the name `scratch` is
+// only a handle for hipGetSymbolAddress -- never a device address: kernels, copies and fills get the
+// per-device pointer that matmul_scratch_setup() stored in the device.
+static __device__ __align__(256) float scratch[UGHIP_MATMUL_NOALLOC_SCRATCH_BYTES / sizeof(float)];
+
+namespace ughip {
+// Called once per device from ughip_device_create, with that device current.
+int matmul_scratch_setup(ughip_device* dev) {
+  void* ptr = nullptr;
+  hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !ptr) return set_error(UGHIP_ERR_HIP, "hipGetSymbolAddress(matmul scratch) on device %d: %s", dev->ordinal, hipGetErrorString(e));
+  dev->static_scratch = ptr;
+  return UGHIP_OK;
+}
+}  // namespace ughip
+
+static int matmul_impl(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs, const ughip_slice* rhs, size_t b, size_t m, size_t n, size_t k,
+                       size_t rank, const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset, const size_t* rhs_dims, const size_t* rhs_strides,
+                       size_t rhs_offset, bool no_alloc) {
   if (!dev || !dst || !lhs || !rhs) return set_error(UGHIP_ERR_INVALID, "matmul: null argument");
   if (rank < 2 || rank > 4 || !lhs_dims || !lhs_strides || !rhs_dims || !rhs_strides)
     return set_error(UGHIP_ERR_INVALID, "matmul: rank %zu layouts are not supported", rank);
@@ -459,6 +476,18 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
     else gemv_nn_f32<8><<<grid, 1024, 0, st>>>(p);
   } else if (gemm_tiled_supported(dst->dtype, p, b, mixed)) {
     const size_t ws_bytes = gemm_tiled_workspace_bytes(dst->dtype, p, b);
+    if (no_alloc) {
+      // the partial tiles go to the device's copy of the static array; every slab writes its whole tile before
+      // the fold reads it, so nothing has to be cleared between calls
+      if (ws_bytes > (size_t)UGHIP_MATMUL_NOALLOC_SCRATCH_BYTES)
+        return set_error(UGHIP_ERR_UNSUPPORTED,
+                         "matmul_noalloc: this product splits K and needs %zu bytes for its partial tiles, the static scratch holds %zu "
+                         "(b %zu, m %zu, n %zu, k %zu); use ughip_matmul",
+                         ws_bytes, (size_t)UGHIP_MATMUL_NOALLOC_SCRATCH_BYTES, b, m, n, k);
+      if (ws_bytes && !dev->static_scratch) return set_error(UGHIP_ERR_HIP, "matmul_noalloc: the static scratch of device %d was not set up", dev->ordinal);
+      UGHIP_HIPCHK(gemm_tiled_launch(st, dst->dtype, p, b, ws_bytes ? static_cast<float*>(dev->static_scratch) : nullptr, mixed));
+      return UGHIP_OK;
+    }
     if (ws_bytes > dev->gemm_ws_bytes) {
       std::lock_guard<std::mutex> g(dev->mu);
       UGHIP_HIPCHK(hipStreamSynchronize(st));  // earlier launches may still read the old block
@@ -481,4 +510,16 @@ extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_sli
   }
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
+}
+
+extern "C" int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs, const ughip_slice* rhs, size_t b, size_t m, size_t n,
+                            size_t k, size_t rank, const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset, const size_t* rhs_dims,
+                            const size_t* rhs_strides, size_t rhs_offset) {
+  return matmul_impl(dev, dst, lhs, rhs, b, m, n, k, rank, lhs_dims, lhs_strides, lhs_offset, rhs_dims, rhs_strides, rhs_offset, false);
+}
+
+extern "C" int ughip_matmul_noalloc(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs, const ughip_slice* rhs, size_t b, size_t m, size_t n,
+                                    size_t k, size_t rank, const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset,
+                                    const size_t* rhs_dims, const size_t* rhs_strides, size_t rhs_offset) {
+  return matmul_impl(dev, dst, lhs, rhs, b, m, n, k, rank, lhs_dims, lhs_strides, lhs_offset, rhs_dims, rhs_strides, rhs_offset, true);
 }

@@ -112,6 +112,10 @@ int ughip_device_create(int ordinal, ughip_device** out) {
   size_t colon = d->arch.find(':');
   if (colon != std::string::npos) d->arch.resize(colon);
   HIPCHK(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking));
+  if (int rc = matmul_scratch_setup(d.get())) {
+    hipStreamDestroy(d->stream);
+    return rc;
+  }
   *out = d.release();
   return UGHIP_OK;
 }
