@@ -172,6 +172,10 @@ int ughip_func_release(ughip_func* f);
  * no-op (runtime.rs:269-277).  Fails with UGHIP_ERR_BOUNDS if a slice is shorter than the
  * largest offset the kernel can form. */
 int ughip_run(ughip_device* dev, ughip_func* f, ughip_slice* const* args, size_t n_args);
+/* Timing aid with no counterpart in the reference: a func lowered to two kernels (a grid-wide reduction:
+ * partial sums, then the fold) launches only its first (part 1) or second (part 2) kernel, with the checks of
+ * ughip_run.  Part 2 alone reads whatever partials the last part 1 left; a single-kernel func has no part 2. */
+int ughip_run_part(ughip_device* dev, ughip_func* f, ughip_slice* const* args, size_t n_args, int part);
 /* HIP source the SSA was lowered to (counterpart of `Kernel.cuda_code()`,
  * ug-pyo3/src/lib.rs:396-401).  Returns the length excluding NUL; copies at most buf_len. */
 size_t ughip_func_source(const ughip_func* f, char* buf, size_t buf_len);

@@ -15,13 +15,11 @@ def pytest_configure(config):
 
 def _oracle_lib():
     """The CPU oracle (oracle/): test infrastructure only -- never imported by the product."""
-    import ug_amd  # noqa: F401  (loads libug_host.so first; the oracle links against it)
-    path = os.path.join(ROOT, "oracle", "_build", "libug_oracle.so")
-    if not os.path.exists(path):
-        pytest.fail(f"{path} missing: run `python -m ug_amd.build` first")
-    lib = C.CDLL(path, mode=C.RTLD_GLOBAL)
-    lib.ugo_last_error.restype = C.c_char_p
-    return lib
+    from oracle.load import oracle_lib
+    try:
+        return oracle_lib()
+    except RuntimeError as e:
+        pytest.fail(str(e))
 
 
 @pytest.fixture(scope="session")
@@ -32,18 +30,14 @@ def oracle():
 @pytest.fixture(scope="session")
 def cpu(oracle):
     """ug::CpuDevice restatement, usable wherever a ug_amd.Device is."""
-    import ug_amd
-    out = C.c_void_p()
-    assert oracle.ugo_cpu_device_new(C.byref(out)) == 0, oracle.ugo_last_error()
-    return ug_amd.Device(out.value)
+    from oracle.load import cpu_device
+    return cpu_device()
 
 
 @pytest.fixture(scope="session")
 def cpu_ops(oracle):
-    import ug_amd
-    out = C.c_void_p()
-    assert oracle.ugo_llama_ops_cpu(C.byref(out)) == 0, oracle.ugo_last_error()
-    return ug_amd.LlamaOps(out.value)
+    from oracle.load import cpu_llama_ops
+    return cpu_llama_ops()
 
 
 @pytest.fixture(scope="session")

@@ -142,9 +142,4 @@ def softmax_graph(src):
     return ug_amd.llama.softmax(src)
 
 
-def fused_reduce_graph(a, b, dev):
-    """Config 2: ((a*b) + (a*0.5)).reduce(Sum, 0).narrow(0, 0, 1); the tensor operand stays on the
-    left so the result keeps its shape (op::binary takes the lhs shape, lang.rs:507-520)."""
-    n = a.dims()[0]
-    half = LB.cst(0.5, (n,), dev)
-    return a.binary("mul", b).binary("add", a.binary("mul", half)).reduce("sum", 0).narrow(0, 0, 1)
+from ug_amd.graphs import fused_reduce_graph  # noqa: E402,F401  (config 2; shared with bench.py and smoke())

@@ -1,13 +1,13 @@
 """The safetensors reader and load_with_cast (ug_amd/csrc/host/ug/safetensors.cpp, after
 ug-core/src/safetensors.rs) on the CPU oracle device, where every conversion runs on the host.
-Files come from two independent writers: the `safetensors` package and tests/st_files.py."""
+Files come from two independent writers: the `safetensors` package and ug_amd/st_writer.py."""
 import os
 import struct
 
 import numpy as np
 import pytest
 
-import st_files
+from ug_amd import st_writer as st_files
 import ug_amd
 from ug_amd import rng
 

@@ -470,7 +470,8 @@ int ughip_func_get_info(const ughip_func* f, ughip_func_info* out) {
   return UGHIP_OK;
 }
 
-int ughip_run(ughip_device* dev, ughip_func* f, ughip_slice* const* args, size_t n_args) {
+// which: 0 = every launch of the func, 1 / 2 = only its first / second kernel (timing aid).
+static int run_impl(ughip_device* dev, ughip_func* f, ughip_slice* const* args, size_t n_args, int which) {
   if (!dev || !f) return set_error(UGHIP_ERR_INVALID, "null device/func");
   if (f->dev != dev) return set_error(UGHIP_ERR_INVALID, "func was compiled for another device");
   const Lowered& low = f->low;
@@ -497,9 +498,17 @@ int ughip_run(ughip_device* dev, ughip_func* f, ughip_slice* const* args, size_t
   if (low.scratch_part_bytes) params[np++] = &f->scratch_part;
   if (!low.kparams.empty()) params[np++] = const_cast<int*>(low.kparams.data());
   if (int rc = device_activate(dev)) return rc;
-  HIPCHK(hipModuleLaunchKernel(f->function, low.grid, 1, 1, low.block, 1, 1, low.lds_bytes, dev->stream, params, nullptr));
-  if (f->function2) HIPCHK(hipModuleLaunchKernel(f->function2, low.grid2, 1, 1, low.block2, 1, 1, 0, dev->stream, params, nullptr));
+  if (which != 2) HIPCHK(hipModuleLaunchKernel(f->function, low.grid, 1, 1, low.block, 1, 1, low.lds_bytes, dev->stream, params, nullptr));
+  if (f->function2 && which != 1) HIPCHK(hipModuleLaunchKernel(f->function2, low.grid2, 1, 1, low.block2, 1, 1, 0, dev->stream, params, nullptr));
   return UGHIP_OK;
+}
+
+int ughip_run(ughip_device* dev, ughip_func* f, ughip_slice* const* args, size_t n_args) { return run_impl(dev, f, args, n_args, 0); }
+
+int ughip_run_part(ughip_device* dev, ughip_func* f, ughip_slice* const* args, size_t n_args, int part) {
+  if (part != 1 && part != 2) return set_error(UGHIP_ERR_INVALID, "run_part: part is 1 or 2, got %d", part);
+  if (f && part == 2 && !f->function2) return set_error(UGHIP_ERR_INVALID, "run_part: %s is a single kernel", f->low.entry.c_str());
+  return run_impl(dev, f, args, n_args, part);
 }
 
 // ---- events --------------------------------------------------------------------------------------

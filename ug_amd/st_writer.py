@@ -1,4 +1,4 @@
-"""Writers for safetensors files used by the tests (the format is 8 bytes of little-endian header
+"""Writer for safetensors files (synthetic checkpoints for the tests and the benchmark; the format is 8 bytes of little-endian header
 length, a JSON header, then the raw tensor bytes): a hand-written one that can store bf16, which
 numpy has no type for, next to the `safetensors` package's own writer where that is enough."""
 import json
