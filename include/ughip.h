@@ -252,7 +252,12 @@ int ughip_matmul_noalloc(ughip_device* dev, ughip_slice* dst, const ughip_slice*
 
 /* ---- ug-llama custom ops (ug-llama/src/main.rs:22-28; oracle cpu_ops.rs:6-167) ------- */
 /* rope / rope_i (cuda_ops.rs:17-104): src, dst are [bh, t*d] f32, cos/sin [max_pos, d/2]
- * f32, pos i32 (only pos[0] is read, cpu_ops.rs:67,100). */
+ * f32, pos i32 (only pos[0] is read, cpu_ops.rs:67,100).
+ * pos lives on the device, so the host cannot check it against the table: a position whose table row
+ * pos[0] + i_t lies outside cos/sin is never read (no out-of-bounds access) and the rotated values of that
+ * row come out as NaN, here and in every fused entry point below that takes (cos, sin, pos) -- where the
+ * reference's slice index would panic (cpu_ops.rs:76-77,112-113).  Callers that know the position on the
+ * host check it there (the llama graph refuses a step past its cache / table when it is built). */
 int ughip_rope(ughip_device* dev, const ughip_slice* src, const ughip_slice* cos,
                const ughip_slice* sin, const ughip_slice* pos, ughip_slice* dst, size_t bh,
                size_t t, size_t d, int interleaved);

@@ -575,6 +575,43 @@ def test_run_checks_bounds_aliasing_and_dtypes(hip):
         s.copy_host_to_device(np.zeros(4, np.int32))
 
 
+def test_a_store_guarded_by_an_if_is_not_held_to_the_rounded_up_grid(hip):
+    """A GPU-style kernel over 100 elements launched as 2 x 64 threads, its store under `If(max(100 - i, 0))`: the
+    bounds check counts what the guard lets through, not the 128 offsets the grid could form."""
+    from ug_amd.api import A, Instr
+    I32_ = int(I32)
+
+    def var(i):
+        return A(0, I32_, 0, i, 0, 0.0, 0)
+
+    def ci(v):
+        return A(1, I32_, 0, 0, v, 0.0, 0)
+
+    def cf(v):
+        return A(1, int(F32), 0, 0, 0, v, 0)
+
+    def ins(op, dtype=0, sub=0, v=0, n=0, a=None, b=None):
+        return Instr(op, dtype, sub, v, n, a or A(), b or A())
+
+    prog = [
+        ins(1, int(F32), n=0),                              # 0 DefineGlobal{0, F32}
+        ins(3, I32_, sub=0),                                # 1 ThreadIdx
+        ins(3, I32_, sub=1),                                # 2 BlockIdx
+        ins(6, I32_, sub=2, a=var(2), b=ci(64)),            # 3 bi * 64
+        ins(6, I32_, sub=0, a=var(3), b=var(1)),            # 4 i = bi * 64 + ti
+        ins(6, I32_, sub=1, a=ci(100), b=var(4)),           # 5 100 - i
+        ins(6, I32_, sub=6, a=var(5), b=ci(0)),             # 6 max(100 - i, 0): non-zero iff i < 100
+        ins(11, v=9, a=var(6)),                             # 7 If
+        ins(13, int(F32), v=0, a=var(4), b=cf(3.0)),        # 8 Store dst[i] = 3
+        ins(12),                                            # 9 EndIf
+    ]
+    k = SsaKernel.from_instrs(prog, grid=2, block=64)
+    func = hip.compile(k, "guarded_store")
+    dst = hip.slice_from(np.zeros(100, np.float32))
+    hip.run(func, [dst])
+    assert np.all(dst.to_vec() == 3.0)
+
+
 def test_more_than_five_args_work_on_hip(hip):
     xs = [LB.copy(f32([i, 2 * i]), (2,), hip) for i in range(7)]
     acc = xs[0]

@@ -177,6 +177,8 @@ struct HipOps : Ops {
     const bool packed = x_offset != 0 || x_row_stride != 0;
     if (x.dims()[0] != b || (packed ? x_row_stride != x.dims()[2] || x_offset + n * d > x_row_stride : x.dims()[2] != n * d))
       bail("kv_append: mismatched shapes " + cache.shape().str() + " " + x.shape().str());
+    // a cache with exactly the rows written so far is the reference's growing representation (model.rs:226-230);
+    // one that was preallocated and is full is refused below, not quietly reallocated
     if (cap == len || d % 4 != 0) return Ops::kv_append(cache, len, x, cos, sin, pos, interleaved, x_offset, x_row_stride);
     if (len + t > cap) bail("kv_append: " + std::to_string(len + t) + " rows exceed the cache capacity " + std::to_string(cap));
     ughip_device* dev = hip_dev(x);
@@ -681,6 +683,12 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
   size_t nh = cfg_.num_attention_heads, nkv = cfg_.num_key_value_heads, hd = cfg_.head_dim();
   const float eps = (float)cfg_.rms_norm_eps;
   auto finish = [&](const LB& out) { return residual ? ops_->linear_add(out, l.o_proj, *residual) : ops_->linear(out, l.o_proj); };
+  // A preallocated cache is full when its rows are used up: stop here, at graph-build time, like the reference's
+  // slice index would (the kernels behind this cannot report an error, and positions past the rotary table
+  // would read outside it).
+  if (cache.capacity && cache.len + seq_len > cache.capacity)
+    bail("attention: " + std::to_string(cache.len) + " cached + " + std::to_string(seq_len) + " new positions exceed the cache's " + std::to_string(cache.capacity) +
+         " rows (max_position_embeddings)");
   if (fused_attention_ >= 3 && seq_len == 1 && xs_in.dims()[0] == 1 && cache.capacity && ops_->packed_projections()) {
     // one position: q | k | v come out of one launch (with the norm in front) side by side and are read where they lie
     const size_t nq = nh * hd, nk = nkv * hd, row = nq + 2 * nk, len = cache.len;

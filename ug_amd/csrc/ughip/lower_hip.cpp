@@ -239,6 +239,7 @@ class Lowering {
   std::vector<int> loop_id_;   // per instr: loop id if Range, else -1
   std::vector<int> encl_;      // per instr: innermost enclosing loop id (Range belongs to its parent)
   std::vector<int> arg_of_;    // per instr: kernel-arg index if DefineGlobal
+  std::vector<bool> guarded_;  // per instr: inside an If
   std::vector<uint64_t> dep_;  // per var: loops it depends on
   std::vector<Itv> itv_;
   std::vector<Aff> aff_;
@@ -275,6 +276,7 @@ class Lowering {
     loop_id_.assign(n_, -1);
     encl_.assign(n_, -1);
     arg_of_.assign(n_, -1);
+    guarded_.assign(n_, false);
     std::vector<int> stack;     // open loop ids / -2 for If
     std::vector<int> if_stack;  // instr index of open Ifs
     size_t n_globals = 0;
@@ -287,6 +289,7 @@ class Lowering {
           break;
         }
       encl_[i] = cur;
+      guarded_[i] = !if_stack.empty();
       if (in.dtype < 0 || in.dtype > UGHIP_I64) fail("bad dtype at " + std::to_string(i));
       switch (in.op) {
         case UGHIP_I_DEFINE_ACC:
@@ -529,6 +532,10 @@ class Lowering {
       }
       if (dead(i)) continue;
       if (in.op == UGHIP_I_STORE) live_store = true;
+      // An access under an If may be exactly what the guard keeps in range (a grid rounded up to the block size with
+      // `if (i < n)` around the store): the interval of its offset says nothing about what is touched, so it adds
+      // no requirement (the unguarded accesses of the same argument still do).
+      if (guarded_[i]) continue;
       Itv o = itv_of(in.a);
       if (!o.known || o.lo < 0)
         out_.min_len[a] = -1;
