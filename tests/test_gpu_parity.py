@@ -353,16 +353,21 @@ def test_matmul_bf16_tile_multiples(hip, bmnk, rhs_nk):
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "f16"])
-@pytest.mark.parametrize("bmnk", [(1, 4096, 4096, 64), (1, 4096, 4096, 128), (4, 2048, 2048, 192), (1, 8192, 2048, 320), (16, 1024, 1024, 64)])
-def test_matmul_16bit_256x256_tiles(hip, bmnk, dtype):
-    """[n, k]-major rhs and at least 256 tiles of 256 x 256: the kernel whose loads write LDS directly
-    (1, 2, 3 and 5 K tiles: prologue only, both stages, the steady state)."""
+@pytest.mark.parametrize("rhs_nk", [True, False], ids=["NT", "NN"])
+@pytest.mark.parametrize("bmnk,bn", [((1, 4096, 4096, 256), 256), ((4, 2048, 2048, 320), 256), ((1, 8192, 2048, 384), 256), ((16, 1024, 1024, 448), 256),
+                                     ((8, 1024, 1024, 256), 128), ((1, 4096, 2048, 320), 128), ((2, 2048, 2048, 576), 128)])
+def test_matmul_16bit_one_wave_per_simd_tiles(hip, bmnk, bn, rhs_nk, dtype):
+    """Products whose 256 x 256 (or only whose 256 x 128) tiles fill the chip: the 4-wave kernel whose loads write LDS
+    directly, for both rhs layouts (a [k, n]-major rhs goes through transposing LDS reads).  4, 5, 6, 7 and 9 K tiles:
+    prologue and tail only, then 1, 2, 3 and 5 rounds of the steady-state loop."""
     b, m, n, k = bmnk
-    print("matmul 256x256", dtype, bmnk, flush=True)
+    print("matmul one-wave-per-SIMD", dtype, bmnk, "NT" if rhs_nk else "NN", flush=True)
     rnd = rng.bf16_round if dtype == "bf16" else (lambda v: v.astype(np.float16).astype(np.float32))
+    dt = ug_amd.BF16 if dtype == "bf16" else ug_amd.F16
     a = rnd(rng.uniform_pm1(25, b * m * k)).reshape(b, m, k)
     w = rnd(rng.uniform_pm1(26, b * k * n)).reshape(b, k, n)
-    got = _raw_matmul(hip, ug_amd.BF16 if dtype == "bf16" else ug_amd.F16, a, w, True)
+    got = _raw_matmul(hip, dt, a, w, rhs_nk)
+    assert ug_amd.last_kernel() == f"gemm_dma4<{dtype},{'NT' if rhs_nk else 'NN'},256x{bn},256t>"
     exact = np.matmul(a.astype(np.float64), w.astype(np.float64))
     half_ulp = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
     bound = half_ulp * np.abs(exact) + k * np.finfo(np.float32).eps * np.matmul(np.abs(a).astype(np.float64), np.abs(w).astype(np.float64))
@@ -371,10 +376,35 @@ def test_matmul_16bit_256x256_tiles(hip, bmnk, dtype):
     import os
     os.environ["UGHIP_GEMM_SHAPE"] = "0"
     try:
-        other = _raw_matmul(hip, ug_amd.BF16 if dtype == "bf16" else ug_amd.F16, a, w, True)
+        other = _raw_matmul(hip, dt, a, w, rhs_nk)
+        assert ug_amd.last_kernel().startswith("gemm_tiled<")
     finally:
         del os.environ["UGHIP_GEMM_SHAPE"]
     np.testing.assert_array_equal(got, other)
+    # small integers: every partial sum is exact, so the result is the integer product bit for bit
+    ai, wi = np.floor(a * 4), np.floor(w * 4)
+    want = np.matmul(ai.astype(np.float64), wi.astype(np.float64)).astype(np.float32)
+    want = rng.bf16_round(want.ravel()).reshape(want.shape) if dtype == "bf16" else want.astype(np.float16).astype(np.float32)
+    np.testing.assert_array_equal(_raw_matmul(hip, dt, ai, wi, rhs_nk), want)
+
+
+def test_matmul_16bit_one_wave_per_simd_forced_and_limits(hip, monkeypatch):
+    """UGHIP_GEMM_SHAPE=3 / 4 force the kernel onto problems it would leave to others (few tiles); shapes it cannot
+    take (K below 4 tiles, rows the tile does not divide) fall through to the register-staged kernel."""
+    a = rng.bf16_round(rng.uniform_pm1(27, 2 * 512 * 256)).reshape(2, 512, 256)
+    w = rng.bf16_round(rng.uniform_pm1(28, 2 * 256 * 256)).reshape(2, 256, 256)
+    plain = _raw_matmul(hip, ug_amd.BF16, a, w, False)
+    assert ug_amd.last_kernel().startswith("gemm_tiled<")
+    for shape, bn in (("3", 256), ("4", 128)):
+        monkeypatch.setenv("UGHIP_GEMM_SHAPE", shape)
+        for rhs_nk in (True, False):
+            got = _raw_matmul(hip, ug_amd.BF16, a, w, rhs_nk)
+            assert ug_amd.last_kernel() == f"gemm_dma4<bf16,{'NT' if rhs_nk else 'NN'},256x{bn},256t>"
+            np.testing.assert_array_equal(got, plain)
+        _raw_matmul(hip, ug_amd.BF16, a[:, :, :192], w[:, :192], True)      # 3 K tiles
+        assert ug_amd.last_kernel().startswith("gemm_tiled<")
+        _raw_matmul(hip, ug_amd.BF16, a[:, :384], w, True)                    # 384 rows
+        assert ug_amd.last_kernel().startswith("gemm_tiled<")
 
 
 @pytest.mark.parametrize("bmnk", [(1, 128, 2048, 2048), (1, 128, 256, 2048), (1, 256, 5632, 2048), (1, 128, 2048, 5632), (2, 512, 384, 96), (1, 1024, 1024, 32),

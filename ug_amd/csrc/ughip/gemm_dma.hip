@@ -1,0 +1,324 @@
+// 16-bit MFMA GEMM for gfx950 with one wave per SIMD: C[b] = A[b] x B[b], f32 accumulate, bf16 or f16.
+//
+//   block tile 256 x BN (BN = 256 or 128), K tile 64, 4 waves laid out 2 x 2, each owning 128 x BN/2 of the result:
+//   16 (8) accumulators of 32 x 32 live in the 256 accumulation registers a lone wave per SIMD can have, which leaves
+//   the architectural registers to two sets of operand fragments -- 8 (6) fragment reads feed 16 (8) MFMAs
+//   global -> LDS with global_load_lds_dwordx4 (no staging registers), two 64 KiB stages; the loads of tile t+2 are
+//   spread, one in front of every other MFMA, over the quarter of tile t that follows the barrier which frees their
+//   stage and over the first quarter of tile t+1: a wave alone on its SIMD has nobody to hide a burst of 16 loads
+//   behind, and with them spread the matrix pipe never waits for the issue of a memory instruction
+//   rhs [n, k]-major: operand fragments are 128-bit LDS reads of k-contiguous rows (XOR-swizzled chunks, conflict free);
+//   rhs [k, n]-major: the tile stays [k][n] in LDS and ds_read_b64_tr_b16 hands every lane 4 consecutive k of its own
+//   column, so no transposing pass through registers is needed
+//   the MFMA operands are swapped (B fragment first): a lane then holds 4 consecutive columns of one result row, the
+//   epilogue packs them and goes through LDS so that the result leaves in 16-byte pieces of whole rows
+//
+// What bounds it: power.  With U(-1, 1) operands the chip runs this kernel at about 1.4 GHz of its 2.4 GHz (shader
+// clock against the 100 MHz reference, read in the kernel), and the matrix pipes are busy 92 % of those cycles.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <type_traits>
+
+#include "gemm.h"
+#include "internal.h"
+#include "ughip.h"
+
+namespace ughip {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ floatx16 mma(__bf16, const u32x4& a, const u32x4& b, const floatx16& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ floatx16 mma(_Float16, const u32x4& a, const u32x4& b, const floatx16& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+
+// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | (((N >> 4) & 3) << 14) | (7 << 4) | (15 << 8));
+}
+__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc07f); }
+
+// Every lane's 16 bytes at base + voff go to LDS at lds_byte_addr + lane * 16.  The compiler does not see the load
+// (it would wait for all of them before any LDS read): the waits are explicit.
+__device__ __forceinline__ void dma16(const void* base, unsigned voff, unsigned lds_byte_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
+}
+
+constexpr int BK = 64, BM = 256;
+
+// k-contiguous operand tile ([rows][64] 16-bit): 128-byte rows of 8 chunks, chunk' = chunk ^ ((row / 2) & 7)
+__device__ __forceinline__ int kc_idx(int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); }  // in 16-byte units
+
+// n-contiguous rhs tile ([64 k][BN n] 16-bit): rows of BN / 32 segments of 64 bytes, segment' = segment ^ (k & mask)
+template <int BN>
+__device__ __forceinline__ int kn_byte(int k, int n) {
+  return k * (BN * 2) + (((n >> 5) ^ (k & (BN / 32 - 1))) << 6) + (n & 31) * 2;
+}
+
+template <typename T, int BN, bool B_KN>
+__global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tiles_n) {
+  extern __shared__ u32x4 lds[];
+  constexpr int NJ = BN / 64;                          // 32-column fragments per wave
+  constexpr int NM = 4 * NJ;                           // MFMAs per k16 step
+  constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2, STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int NDA = 8, NDB = BN / 32, ND = NDA + NDB;  // DMA instructions per wave and K tile
+  constexpr int H = ND / 2;                            // ... per step that carries them
+  constexpr int R = 4 + NJ;                            // fragment reads per step
+  static_assert(R == H, "reads and DMAs of a step alternate one for one");
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  // Block ids go round-robin over the 8 XCDs: id -> (id % 8) * (grid / 8) + id / 8 hands every XCD a contiguous run of
+  // tiles, and tiles are numbered in super-rows of 4 tile rows, column by column inside, so that such a run is a 4-row
+  // block: its workgroups share few A and B panels in their XCD's L2.
+  int bid = blockIdx.x;
+  if ((gridDim.x & 7) == 0) bid = (bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3);
+  const int tpb = tiles_m * tiles_n;
+  const int batch = bid / tpb;
+  const int t_in = bid - batch * tpb;
+  int tm, tn;
+  if ((tiles_m & 3) == 0) {
+    const int sr = t_in / (4 * tiles_n), rem = t_in - sr * 4 * tiles_n;
+    tm = sr * 4 + (rem & 3);
+    tn = rem >> 2;
+  } else {
+    tm = t_in / tiles_n;
+    tn = t_in - tm * tiles_n;
+  }
+  const int m0 = tm * BM, n0 = tn * BN;
+  const long long lda = p.a_rs, ldb = B_KN ? p.b_rs : p.b_cs;
+  const char* Ab = reinterpret_cast<const char*>(static_cast<const T*>(p.a) + (size_t)batch * p.a_bs + (size_t)m0 * lda);
+  const char* Bb = reinterpret_cast<const char*>(static_cast<const T*>(p.b) + (size_t)batch * p.b_bs + (B_KN ? (size_t)n0 : (size_t)n0 * ldb));
+  const int KT = p.K / BK;
+  const int wm = (wave >> 1) * 128, wn = (wave & 1) * (BN / 2);
+  const unsigned lds_addr = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
+
+  // per-lane byte offsets of this wave's DMA instructions (the same for every K tile; the scalar base moves)
+  unsigned voff[ND];
+#pragma unroll
+  for (int i = 0; i < NDA; ++i) {
+    const int row = (i * 4 + wave) * 8 + (lane >> 3), cp = lane & 7;
+    voff[i] = (unsigned)(row * lda * 2 + ((cp ^ ((row >> 1) & 7)) << 4));
+  }
+#pragma unroll
+  for (int i = 0; i < NDB; ++i) {
+    const int g = i * 4 + wave;
+    if (!B_KN) {
+      const int row = g * 8 + (lane >> 3), cp = lane & 7;
+      voff[NDA + i] = (unsigned)(row * ldb * 2 + ((cp ^ ((row >> 1) & 7)) << 4));
+    } else {
+      // one instruction fills 1 KB = 512 / BN rows of k; the lane at LDS position (k, 16-byte chunk c') fetches the
+      // chunk whose 64-byte segment the swizzle maps there
+      constexpr int CPR = BN / 8;  // 16-byte chunks per row
+      const int k = g * (64 / CPR) + lane / CPR, cpos = lane % CPR;
+      const int seg = (cpos >> 2) ^ (k & (BN / 32 - 1));
+      voff[NDA + i] = (unsigned)(k * ldb * 2 + (((seg << 2) | (cpos & 3)) << 4));
+    }
+  }
+  const long long a_step = BK * 2, b_step = B_KN ? (long long)BK * ldb * 2 : BK * 2;
+  auto dma = [&](int tile, int idx) {  // idx: compile-time after unrolling
+    const unsigned st = lds_addr + (tile & 1) * STAGE_BYTES;
+    if (idx < NDA) dma16(Ab + tile * a_step, voff[idx], st + (idx * 4 + wave) * 1024);
+    else dma16(Bb + tile * b_step, voff[idx], st + A_BYTES + ((idx - NDA) * 4 + wave) * 1024);
+  };
+
+  floatx16 acc[4][NJ];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // operand fragments of one k16 step, two sets: lane l feeds row / column l % 32, k = 8 (l / 32) .. + 7
+  u32x4 fa[2][4], fb[2][NJ];
+  auto read_frag = [&](int stage, int s, int idx, int set) {  // idx < 4: A fragment idx, else B fragment idx - 4
+    if (idx < 4) {
+      fa[set][idx] = lds[stage * (STAGE_BYTES / 16) + kc_idx(wm + idx * 32 + (lane & 31), 2 * s + (lane >> 5))];
+    } else if (!B_KN) {
+      fb[set][idx - 4] = lds[stage * (STAGE_BYTES / 16) + A_BYTES / 16 + kc_idx(wn + (idx - 4) * 32 + (lane & 31), 2 * s + (lane >> 5))];
+    } else {
+      // A transposing read returns to lane i of a 16-lane group the 4 values at column i % 4 of the rows that lanes
+      // i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12 name.  Lane q + 4 e names row kbase + e, columns 4 q .. 4 q + 3 of its
+      // group's 16, so lane i receives k = kbase .. kbase + 3 of column i; two reads give the 8 consecutive k of the
+      // MFMA operand.  Groups 0, 1 hold k 0..7 of columns 0..15 and 16..31, groups 2, 3 hold k 8..15.
+      typedef __attribute__((address_space(3))) s16x4 lds_v4;
+      const int g = lane >> 4, li = lane & 15, q = li & 3, e = li >> 2;
+      const char __attribute__((address_space(3)))* Bs = (const char __attribute__((address_space(3)))*)lds + stage * STAGE_BYTES + A_BYTES;
+      const int n = wn + (idx - 4) * 32 + 16 * (g & 1) + 4 * q, k0 = s * 16 + 8 * (g >> 1) + e;
+      const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4*)(Bs + kn_byte<BN>(k0, n))));
+      const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4*)(Bs + kn_byte<BN>(k0 + 4, n))));
+      fb[set][idx - 4] = u32x4{lo.x, lo.y, hi.x, hi.y};
+    }
+  };
+
+  // prologue: tiles 0 and 1 requested and landed
+#pragma unroll
+  for (int i = 0; i < ND; ++i) dma(0, i);
+#pragma unroll
+  for (int i = 0; i < ND; ++i) dma(1, i);
+  wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int i = 0; i < R; ++i) read_frag(0, 0, i, 0);
+
+  // One K tile = 4 steps of NM MFMAs.  The memory instructions of a step -- the R fragment reads of the next step,
+  // then (D3: in step 3, D0: in step 0) one half of the DMAs that refill the stage everybody left at the barrier of
+  // step 3 -- are dealt evenly in front of the MFMAs.  RN: there is a next tile to read fragments from.
+  auto tile = [&](int kt, auto d0, auto d3, auto rn) {
+    constexpr bool D0 = decltype(d0)::value, D3 = decltype(d3)::value, RN = decltype(rn)::value;
+    const int cur = kt & 1, nxt = cur ^ 1;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int fc = s & 1, fn = fc ^ 1;
+      if (s == 3) {
+        // this wave's share of tile kt+1 has landed and its reads of stage cur are done; then everyone's
+        wait_vmcnt<0>();
+        wait_lgkmcnt0();
+        __builtin_amdgcn_s_barrier();
+      }
+      const bool reads = s < 3 || RN, dmas = (s == 3 && D3) || (s == 0 && D0);
+      const int n_ops = (reads ? R : 0) + (dmas ? H : 0);
+#pragma unroll
+      for (int g = 0; g < NM; ++g) {
+#pragma unroll
+        for (int t = 0; t < R + H; ++t) {
+          if (t < n_ops && t * NM / n_ops == g) {
+            // in a step with both kinds they alternate: read, DMA, read, DMA, ...
+            const bool both = reads && dmas;
+            const bool is_read = both ? (t & 1) == 0 && t / 2 < R : reads;
+            const int ri = both ? t / 2 : t, di = both ? ((t & 1) ? t / 2 : 0) : t;
+            if (is_read) read_frag(s < 3 ? cur : nxt, s < 3 ? s + 1 : 0, ri, fn);
+            else if (s == 3) dma(kt + 2, di);
+            else dma(kt + 1, H + di);
+          }
+        }
+        const int i = g / NJ, j = g % NJ;
+        acc[i][j] = mma(T(), fb[fc][j], fa[fc][i], acc[i][j]);  // operands swapped: rows of the block are columns of C
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  };
+  using Y = std::true_type;
+  using N_ = std::false_type;
+  tile(0, N_(), Y(), Y());  // tile 1 went out whole in the prologue
+  for (int kt = 1; kt < KT - 2; ++kt) tile(kt, Y(), Y(), Y());
+  tile(KT - 2, Y(), N_(), Y());
+  tile(KT - 1, N_(), N_(), N_());
+
+  // Epilogue through LDS (nobody reads a stage after the last barrier, no load is in flight).  Accumulator register r of
+  // lane l of block (i, j): column of C  wn + 32 j + 8 (r / 4) + 4 (l / 32) + r % 4,  row  wm + 32 i + l % 32: four
+  // consecutive columns per register quad.  Row pitch BN * 2 + 8 bytes: 32 lanes of consecutive rows hit 64 banks once.
+  constexpr int PITCH = BN * 2 + 8;
+  char __attribute__((address_space(3)))* Cs = (char __attribute__((address_space(3)))*)lds;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int rq = 0; rq < 4; ++rq) {
+        typedef T tx4 __attribute__((ext_vector_type(4)));
+        tx4 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (T)acc[i][j][rq * 4 + e];
+        const int row = wm + i * 32 + (lane & 31), col = wn + j * 32 + rq * 8 + (lane >> 5) * 4;
+        *(u32x2 __attribute__((address_space(3)))*)(Cs + row * PITCH + col * 2) = __builtin_bit_cast(u32x2, v);
+      }
+  __syncthreads();
+  constexpr int CPR = BN / 8, RPP = 256 / CPR;  // 16-byte chunks per row, rows per pass of the workgroup
+  T* __restrict__ C = static_cast<T*>(p.c) + (size_t)batch * p.c_bs + (size_t)m0 * p.N + n0;
+  const int c = tid % CPR, r0 = tid / CPR;
+#pragma unroll 4
+  for (int pass = 0; pass < BM / RPP; ++pass) {
+    const int row = pass * RPP + r0;
+    const u32x2 lo = *(const u32x2 __attribute__((address_space(3)))*)(Cs + row * PITCH + c * 16);
+    const u32x2 hi = *(const u32x2 __attribute__((address_space(3)))*)(Cs + row * PITCH + c * 16 + 8);
+    *reinterpret_cast<u32x4*>(C + (size_t)row * p.N + c * 8) = u32x4{lo.x, lo.y, hi.x, hi.y};
+  }
+}
+
+template <typename T, int BN, bool B_KN>
+hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch) {
+  constexpr int STAGES = 2 * (BM + BN) * BK * 2, EPI = BM * (BN * 2 + 8);
+  constexpr int LDS_BYTES = STAGES > EPI ? STAGES : EPI;
+  static std::atomic<unsigned long long> configured{0};  // one bit per device: the attribute is per device
+  auto kernel = gemm_dma4<T, BN, B_KN>;
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev)) return e;
+  const unsigned long long bit = dev < 64 ? 1ull << dev : 0;
+  if (!bit || !(configured.load(std::memory_order_relaxed) & bit)) {
+    if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES)) return e;
+    configured.fetch_or(bit, std::memory_order_relaxed);
+  }
+  const int tiles_m = p.M / BM, tiles_n = p.N / BN;
+  const size_t total = batch * (size_t)tiles_m * tiles_n;
+  kernel<<<dim3((unsigned)total), dim3(256), LDS_BYTES, stream>>>(p, tiles_m, tiles_n);
+  return hipGetLastError();
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace
+
+bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int bn) {
+  if (dtype != UGHIP_BF16 && dtype != UGHIP_F16) return false;
+  if (bn != 256 && bn != 128) return false;
+  if (p.M <= 0 || p.N <= 0 || p.M % BM || p.N % bn || p.K % BK || p.K < 4 * BK || batch == 0) return false;
+  if (p.a_cs != 1 || p.a_rs % 8 || (batch > 1 && (p.a_bs % 8 || p.b_bs % 8 || p.c_bs % 8))) return false;
+  const bool nn = p.b_cs == 1 && p.b_rs != 1, nt = p.b_rs == 1 && p.b_cs != 1;
+  if (nn == nt) return false;
+  const long long ldb = nn ? p.b_rs : p.b_cs;
+  if (ldb % 8) return false;
+  // per-lane offsets are 32-bit: the furthest row of a tile has to stay below 4 GiB from the tile's first byte
+  if ((unsigned long long)p.a_rs * 2 * BM >= (1ull << 32) || (unsigned long long)ldb * 2 * (nn ? BK : bn) >= (1ull << 32)) return false;
+  if (!aligned16(p.a) || !aligned16(p.b) || !aligned16(p.c)) return false;
+  return batch * (size_t)(p.M / BM) * (size_t)(p.N / bn) < (1u << 24);
+}
+
+// Which tile this kernel should take the problem with: 256 when 256 x 256 tiles fill the chip, 128 when only 256 x 128
+// tiles do (8 x 1024^3: 128 against 256 tiles), 0 when another kernel is the better choice (few tiles: the K-splitting
+// register-staged kernel; a last round of workgroups that would leave most CUs idle).
+// UGHIP_GEMM_SHAPE=3 / 4 forces 256 / 128 where the kernel applies, 0..2 keeps it out (tuning aid).
+int gemm_dma_pick(int dtype, const MMArgs& p, size_t batch) {
+  if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
+    const int s = atoi(e);
+    if (s == 3) return gemm_dma_supported(dtype, p, batch, 256) ? 256 : 0;
+    if (s == 4) return gemm_dma_supported(dtype, p, batch, 128) ? 128 : 0;
+    return 0;
+  }
+  for (int bn : {256, 128}) {
+    if (!gemm_dma_supported(dtype, p, batch, bn)) continue;
+    const size_t tiles = batch * (size_t)(p.M / BM) * (size_t)(p.N / bn), rounds = (tiles + 255) / 256;
+    if (tiles >= 200 && tiles * 5 >= rounds * 256 * 4) return bn;  // the last round at least 80 % of the average
+  }
+  return 0;
+}
+
+hipError_t gemm_dma_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, int bn) {
+  if (!gemm_dma_supported(dtype, p, batch, bn)) return hipErrorInvalidValue;
+  const bool nn = p.b_cs == 1 && p.b_rs != 1;
+  const char* tn = dtype == UGHIP_F16 ? "f16" : "bf16";
+  note_kernel("gemm_dma4<%s,%s,256x%d,256t>", tn, nn ? "NN" : "NT", bn);
+#define UGHIP_DMA_CASE(T)                                                                        \
+  if (bn == 256) return nn ? launch<T, 256, true>(stream, p, batch) : launch<T, 256, false>(stream, p, batch); \
+  return nn ? launch<T, 128, true>(stream, p, batch) : launch<T, 128, false>(stream, p, batch);
+  if (dtype == UGHIP_F16) {
+    UGHIP_DMA_CASE(_Float16)
+  }
+  UGHIP_DMA_CASE(__bf16)
+#undef UGHIP_DMA_CASE
+}
+
+}  // namespace ughip

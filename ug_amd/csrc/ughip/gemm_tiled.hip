@@ -10,7 +10,7 @@
 //   a row-major B ([k, n]) is transposed in registers on its way to LDS so that both MFMA
 //   operands read 128 bits of consecutive k (v_perm_b32 for bf16; free for f32)
 //   tiles are handed to workgroups XCD by XCD so that the tiles of one batch element share an L2
-//   16-bit types with an [n, k]-major rhs and >= 256 tiles of 256x256: gemm_tiled_dma below
+//   16-bit products whose 256 x 256 or 256 x 128 tiles fill the chip go to gemm_dma.hip instead (matmul.hip decides)
 //
 // bf16, f16: v_mfma_f32_32x32x16_{bf16,f16} (lane l feeds row/col l%32, k = 8*(l/32)..+7).
 // f32:  v_mfma_f32_32x32x2_f32   (lane l feeds row/col l%32, k = l/32); the 4 floats of a 128-bit
@@ -402,127 +402,6 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p_in, int tiles_m, int t
   }
 }
 
-// ---- variant with loads that write LDS directly ([n, k]-major rhs, no K split) --------------------------
-// global_load_lds_dwordx4: every lane names its own 16 global bytes, the wave's 64 x 16 bytes land
-// at M0 + lane * 16 in LDS.  No prefetch registers, no staging stores: a wave instruction fills 8
-// rows of a stage, the swizzle moves to the global side (lane at LDS chunk position c' fetches chunk
-// c' ^ swz(row), a permutation inside the 128-byte row, so coalescing is unchanged).  The compiler
-// does not see these loads (inline asm), so it neither waits for them before unrelated LDS reads nor
-// counts them: the waits are explicit.  The registers this frees pay for a 256 x 256 tile (8 waves of
-// 128 x 64: 128 accumulator registers), which halves the LDS bytes moved per flop; with its 64 KiB
-// stages two fit, so tile kt+1 is in flight while tile kt is multiplied (STAGES = 3 keeps two in
-// flight for smaller tiles: measured no faster than the register-staged kernel at 256 x 128).
-__device__ __forceinline__ void dma16(const void* g, unsigned lds_byte_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_byte_addr), "v"(g) : "memory");
-}
-
-// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  __builtin_amdgcn_s_waitcnt((N & 15) | (((N >> 4) & 3) << 14) | (7 << 4) | (15 << 8));
-}
-
-template <typename T, int BM, int BN, int NT>
-__device__ __forceinline__ void dma_tile(const T* __restrict__ A, const T* __restrict__ B, const MMArgs& p, int kt, unsigned stage_addr, int wave, int lane) {
-  constexpr int NWV = NT / 64, BK = Elt<T>::BK, VE = Elt<T>::VE;
-  const int r8 = lane >> 3, cp = lane & 7;  // row inside the group of 8 rows, chunk position in LDS
-  const size_t k0 = (size_t)kt * BK;
-#pragma unroll
-  for (int i = 0; i < BM / 8 / NWV; ++i) {
-    const int g = i * NWV + wave, row = g * 8 + r8;
-    dma16(A + (size_t)row * p.a_rs + k0 + (cp ^ lds_swz(row)) * VE, __builtin_amdgcn_readfirstlane(stage_addr + g * 8 * 128));
-  }
-#pragma unroll
-  for (int i = 0; i < BN / 8 / NWV; ++i) {
-    const int g = i * NWV + wave, row = g * 8 + r8;
-    dma16(B + (size_t)row * p.b_cs + k0 + (cp ^ lds_swz(row)) * VE, __builtin_amdgcn_readfirstlane(stage_addr + (BM + g * 8) * 128));
-  }
-}
-
-template <typename T, int BM, int MI, int NJ>
-__device__ __forceinline__ void compute_phase(const u32x4* __restrict__ cur, int lane, int wm, int wn, floatx16 (&acc)[MI][NJ]) {
-  constexpr int N_MFMA = MI * NJ * (sizeof(T) == 4 ? 4 : 1), N_READ = MI + NJ;
-  Frags<MI, NJ> f0, f1;
-  load_frags<BM, MI, NJ>(cur, lane, wm, wn, 0, f0);
-  __builtin_amdgcn_sched_barrier(0);
-  load_frags<BM, MI, NJ>(cur, lane, wm, wn, 1, f1);
-  mma_frags<T, MI, NJ>(f0, acc);
-  interleave_step<N_MFMA, N_READ, 0, 0>();
-  __builtin_amdgcn_sched_barrier(0);
-  load_frags<BM, MI, NJ>(cur, lane, wm, wn, 2, f0);
-  mma_frags<T, MI, NJ>(f1, acc);
-  interleave_step<N_MFMA, N_READ, 0, 0>();
-  __builtin_amdgcn_sched_barrier(0);
-  load_frags<BM, MI, NJ>(cur, lane, wm, wn, 3, f1);
-  mma_frags<T, MI, NJ>(f0, acc);
-  interleave_step<N_MFMA, N_READ, 0, 0>();
-  __builtin_amdgcn_sched_barrier(0);
-  mma_frags<T, MI, NJ>(f1, acc);
-}
-
-template <typename T, int BM, int BN, int NT, int STAGES>
-__global__ void __launch_bounds__(NT) gemm_tiled_dma(MMArgs p, int tiles_m, int tiles_n, int remap) {
-  extern __shared__ u32x4 lds[];
-  constexpr int BK = Elt<T>::BK;
-  constexpr int WM = BM / (NT / 128), WN = BN / 2, MI = WM / 32, NJ = WN / 32;
-  constexpr int STAGE = (BM + BN) * CHUNKS;             // in 16-byte units
-  constexpr int N_DMA = (BM + BN) / 8 / (NT / 64);       // wave instructions per tile
-  constexpr int AHEAD = STAGES - 1;                      // tiles requested ahead of the one being multiplied
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  int bid = blockIdx.x;
-  if (remap) bid = (bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3);
-  const int tpb = tiles_m * tiles_n;
-  const int batch = bid / tpb;
-  const int t_in = bid - batch * tpb;
-  const int m0 = (t_in / tiles_n) * BM, n0 = (t_in % tiles_n) * BN;
-  const T* __restrict__ A = static_cast<const T*>(p.a) + (size_t)batch * p.a_bs + (size_t)m0 * p.a_rs;
-  const T* __restrict__ B = static_cast<const T*>(p.b) + (size_t)batch * p.b_bs + (size_t)n0 * p.b_cs;
-  const int KT = p.K / BK;
-  const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
-  const unsigned lds_addr = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
-
-  floatx16 acc[MI][NJ];
-#pragma unroll
-  for (int i = 0; i < MI; ++i)
-#pragma unroll
-    for (int j = 0; j < NJ; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-  dma_tile<T, BM, BN, NT>(A, B, p, 0, lds_addr, wave, lane);
-  if (AHEAD == 2 && KT > 1) {
-    dma_tile<T, BM, BN, NT>(A, B, p, 1, lds_addr + STAGE * 16, wave, lane);
-    wait_vmcnt<N_DMA>();
-  } else {
-    wait_vmcnt<0>();
-  }
-  __builtin_amdgcn_s_barrier();
-  int stage = 0;
-  for (int kt = 0; kt < KT; ++kt) {
-    // the stage read one phase ago takes the tile AHEAD phases from now
-    const int into = stage == 0 ? STAGES - 1 : stage - 1;
-    if (kt + AHEAD < KT) dma_tile<T, BM, BN, NT>(A, B, p, kt + AHEAD, lds_addr + into * STAGE * 16, wave, lane);
-    compute_phase<T, BM, MI, NJ>(lds + stage * STAGE, lane, wm, wn, acc);
-    if (kt + 1 < KT) {
-      // tile kt+1 has to be in LDS; with three stages tile kt+2 may stay in flight
-      if (AHEAD == 2 && kt + 2 < KT) wait_vmcnt<N_DMA>();
-      else wait_vmcnt<0>();
-      __builtin_amdgcn_s_barrier();
-    }
-    stage = stage == STAGES - 1 ? 0 : stage + 1;
-  }
-
-  T* __restrict__ C = static_cast<T*>(p.c) + (size_t)batch * p.c_bs + (size_t)m0 * p.N + n0;
-#pragma unroll
-  for (int i = 0; i < MI; ++i)
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      T* Ct = C + (size_t)(wm + i * 32 + (lane >> 5) * 4) * p.N + wn + j * 32 + (lane & 31);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) Ct[(size_t)((r >> 2) * 8 + (r & 3)) * p.N] = (T)acc[i][j][r];
-    }
-}
-
 // c[i] = (T)(ws[0][i] + ws[1][i] + ... in slab order); n4 groups of 4 elements.
 template <typename T>
 __global__ void __launch_bounds__(256) gemm_split_reduce(const float* __restrict__ ws, T* __restrict__ c, size_t n4, size_t slab_elems, int nsplit) {
@@ -570,21 +449,6 @@ hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch, int nsplit,
   return hipSuccess;
 }
 
-// 256 x 256 tile, 8 waves of 128 x 64, two LDS stages filled by loads that write LDS directly:
-// 16-bit types, [n, k]-major rhs, no K split.
-template <typename T>
-hipError_t launch_dma256(hipStream_t stream, const MMArgs& p, size_t batch) {
-  constexpr int BM = 256, BN = 256, NT = 512, STAGES = 2;
-  constexpr int LDS_BYTES = STAGES * (BM + BN) * CHUNKS * 16;
-  static std::atomic<unsigned long long> configured{0};
-  auto kernel = gemm_tiled_dma<T, BM, BN, NT, STAGES>;
-  if (hipError_t e = allow_lds(reinterpret_cast<const void*>(kernel), LDS_BYTES, configured)) return e;
-  const int tiles_m = p.M / BM, tiles_n = p.N / BN;
-  const size_t total = batch * (size_t)tiles_m * tiles_n;
-  kernel<<<dim3((unsigned)total), dim3(NT), LDS_BYTES, stream>>>(p, tiles_m, tiles_n, total % 8 == 0 ? 1 : 0);
-  return hipGetLastError();
-}
-
 template <typename T, int B_NK, bool SPLIT>
 hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int shape, int nsplit, float* ws) {
   switch (shape) {
@@ -594,9 +458,6 @@ hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int s
     case 1:
       return p.M % 128 || p.N % 128 ? launch<T, B_NK, 128, 128, 256, SPLIT, true>(stream, p, batch, nsplit, ws)
                                     : launch<T, B_NK, 128, 128, 256, SPLIT>(stream, p, batch, nsplit, ws);
-    case 3:
-      if constexpr (sizeof(T) == 2 && B_NK == 1 && !SPLIT) return launch_dma256<T>(stream, p, batch);
-      [[fallthrough]];
     default:
       return p.M % 128 || p.N % 64 ? launch<T, B_NK, 128, 64, 256, SPLIT, true>(stream, p, batch, nsplit, ws)
                                    : launch<T, B_NK, 128, 64, 256, SPLIT>(stream, p, batch, nsplit, ws);
@@ -605,22 +466,17 @@ hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int s
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-constexpr int kShapes[4][2] = {{256, 128}, {128, 128}, {128, 64}, {256, 256}};
+constexpr int kShapes[3][2] = {{256, 128}, {128, 128}, {128, 64}};
 
 // The largest tile that divides the problem and still gives every CU a workgroup; failing that,
 // the dividing tile with the most workgroups.  -1: no tile divides M x N.
 int pick_shape(const MMArgs& p, size_t batch, int dtype) {
-  // shape 3 (256 x 256, loads that write LDS directly): 16-bit types with an [n, k]-major rhs
   const bool rhs_nk = p.b_rs == 1 && p.b_cs != 1;
-  const bool can3 = dtype != UGHIP_F32 && rhs_nk && p.M % 256 == 0 && p.N % 256 == 0;
-  // UGHIP_GEMM_SHAPE=0..3 forces a tile shape (tuning aid); ignored when it does not fit the problem.
+  // UGHIP_GEMM_SHAPE=0..2 forces a tile shape (tuning aid); ignored when it does not fit the problem.
   if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
     const int s = atoi(e);
-    if (s == 3 && can3) return 3;
     if (s >= 0 && s < 3 && (p.M % kShapes[s][0] == 0 || kShapes[s][0] == 128) && (p.N % kShapes[s][1] == 0 || (kShapes[s][0] == 128 && rhs_nk))) return s;
   }
-  // half the LDS traffic per flop of 256 x 128, once it alone gives every CU a workgroup
-  if (can3 && batch * (size_t)(p.M / 256) * (size_t)(p.N / 256) >= 256) return 3;
   int best = -1;
   size_t best_tiles = 0;
   for (int s = 0; s < 3; ++s) {
@@ -671,7 +527,7 @@ bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf1
 
 size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch) {
   const int s = pick_shape(p, batch, dtype);
-  if (s < 0 || s == 3) return 0;
+  if (s < 0) return 0;
   const int nsplit = pick_split(dtype, p, batch, s);
   return nsplit > 1 ? (size_t)nsplit * batch * (size_t)p.M * p.N * sizeof(float) : 0;
 }
@@ -681,15 +537,13 @@ hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, siz
   if (rhs_bf16 && (dtype != UGHIP_F32 || !nt)) return hipErrorInvalidValue;
   const int s = pick_shape(p, batch, dtype);
   if (s < 0) return hipErrorInvalidValue;
-  const int nsplit = s == 3 ? 1 : pick_split(dtype, p, batch, s);
+  const int nsplit = pick_split(dtype, p, batch, s);
   {
     const char* tn = rhs_bf16 ? "f32xbf16" : dtype == UGHIP_F32 ? "f32" : dtype == UGHIP_F16 ? "f16" : "bf16";
     const bool ragged = s != 0 && s != 3 && (p.M % kShapes[s][0] || p.N % kShapes[s][1]);
     char split[32] = "";
     if (nsplit > 1) snprintf(split, sizeof split, ",splitK=%d", nsplit);
-    if (s == 3) note_kernel("gemm_tiled_dma<%s,NT,256x256,512t>", tn);
-    else
-      note_kernel("gemm_tiled<%s,%s,%dx%d,%dt%s%s>", tn, nt ? "NT" : "NN", kShapes[s][0], kShapes[s][1], s == 0 && !getenv("UGHIP_GEMM_4WAVES") ? 512 : 256,
+    note_kernel("gemm_tiled<%s,%s,%dx%d,%dt%s%s>", tn, nt ? "NT" : "NN", kShapes[s][0], kShapes[s][1], s == 0 && !getenv("UGHIP_GEMM_4WAVES") ? 512 : 256,
                   ragged ? ",ragged" : "", split);
   }
   if (nsplit > 1) {

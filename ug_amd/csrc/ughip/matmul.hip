@@ -474,6 +474,9 @@ static int matmul_impl(ughip_device* dev, ughip_slice* dst, const ughip_slice* l
     if (m == 1) gemv_nn_f32<1><<<grid, 1024, 0, st>>>(p);
     else if (m <= 4) gemv_nn_f32<4><<<grid, 1024, 0, st>>>(p);
     else gemv_nn_f32<8><<<grid, 1024, 0, st>>>(p);
+  } else if (const int bn = mixed ? 0 : gemm_dma_pick(dst->dtype, p, b)) {
+    UGHIP_HIPCHK(gemm_dma_launch(st, dst->dtype, p, b, bn));
+    return UGHIP_OK;
   } else if (gemm_tiled_supported(dst->dtype, p, b, mixed)) {
     const size_t ws_bytes = gemm_tiled_workspace_bytes(dst->dtype, p, b);
     if (no_alloc) {
