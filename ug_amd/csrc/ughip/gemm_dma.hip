@@ -164,12 +164,12 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
     }
   };
 
-  // prologue: tiles 0 and 1 requested and landed
+  // prologue: tiles 0 and 1 requested, tile 0 landed (tile 1 is waited for at the barrier of tile 0's last step)
 #pragma unroll
   for (int i = 0; i < ND; ++i) dma(0, i);
 #pragma unroll
   for (int i = 0; i < ND; ++i) dma(1, i);
-  wait_vmcnt<0>();
+  wait_vmcnt<ND>();
   __builtin_amdgcn_s_barrier();
 #pragma unroll
   for (int i = 0; i < R; ++i) read_frag(0, 0, i, 0);
