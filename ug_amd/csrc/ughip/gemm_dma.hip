@@ -14,7 +14,8 @@
 //   epilogue packs them and goes through LDS so that the result leaves in 16-byte pieces of whole rows
 //
 // What bounds it: power.  With U(-1, 1) operands the chip runs this kernel at about 1.4 GHz of its 2.4 GHz (shader
-// clock against the 100 MHz reference, read in the kernel), and the matrix pipes are busy 92 % of those cycles.
+// clock against the 100 MHz reference, read in the kernel), and the matrix pipes are busy 80-90 % of those cycles
+// (SQ_VALU_MFMA_BUSY_CYCLES against SQ_WAVE_CYCLES: 83 % of a wave's whole residency at 4096^3).
 #include <hip/hip_runtime.h>
 
 #include <atomic>
