@@ -380,6 +380,25 @@ extern "C" {
         n: usize,
         k: usize,
     ) -> c_int;
+    pub fn ughip_linear_add_rows(
+        dev: *mut UghipDevice,
+        x: *const UghipSlice,
+        w: *const UghipSlice,
+        residual: *const UghipSlice,
+        dst: *mut UghipSlice,
+        m: usize,
+        n: usize,
+        k: usize,
+    ) -> c_int;
+    pub fn ughip_linear_swiglu_rows(
+        dev: *mut UghipDevice,
+        x: *const UghipSlice,
+        w: *const UghipSlice,
+        dst: *mut UghipSlice,
+        m: usize,
+        n: usize,
+        k: usize,
+    ) -> c_int;
     pub fn ughip_argmax_row(
         dev: *mut UghipDevice,
         logits: *const UghipSlice,

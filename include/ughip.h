@@ -371,6 +371,20 @@ int ughip_rms_gemv_gate_up(ughip_device* dev, const ughip_slice* x, const ughip_
 int ughip_gemv_add(ughip_device* dev, const ughip_slice* x, const ughip_slice* w,
                    const ughip_slice* residual, ughip_slice* dst, size_t n, size_t k);
 
+/* ---- the same two for several positions (m >= 9 rows; a prefill) -------------------------------
+ * x is [m, k] F32 with contiguous rows, w a row-major [n, k] matrix stored as F32 or BF16, k % 32 == 0, n % 8 == 0.
+ * The product is the tiled MFMA kernel's; skinny products split K over workgroups, and the fold of their
+ * partial tiles (which a plain ughip_matmul of these shapes runs anyway) applies the neighbour on its way out,
+ * so the residual add / SwiGLU of model.rs:99-109,160-168,366-372 costs no launch and no round trip.
+ * ughip_linear_add_rows: dst[m, n] = x w^T + residual[m, n]; dst may be residual itself (every element is read,
+ * then written, by one thread).
+ * ughip_linear_swiglu_rows: w is [2n, k], gate rows first then up rows: dst[m, n] = silu(x gate^T) * (x up^T).
+ * Shapes the tiled kernel does not take are refused with UGHIP_ERR_UNSUPPORTED (run the pieces instead). */
+int ughip_linear_add_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w,
+                          const ughip_slice* residual, ughip_slice* dst, size_t m, size_t n, size_t k);
+int ughip_linear_swiglu_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w,
+                             ughip_slice* dst, size_t m, size_t n, size_t k);
+
 /* ---- greedy step on the device ----------------------------------------------------------------
  * Row `row` of logits [rows, n] (F32): the index of its largest value (the lowest index among
  * equal values -- what a host loop with `>` finds) goes to token[0] (I32; NULL: skipped) and to

@@ -1203,6 +1203,82 @@ def test_bf16_matrices_meet_several_rows_through_a_cast(hip, hip_ops):
         assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("t,k,n", [(128, 2048, 2048), (128, 5632, 2048), (100, 256, 192), (37, 64, 48), (9, 32, 16), (300, 512, 1000)])
+@pytest.mark.parametrize("bf16", [False, True])
+def test_projections_of_several_rows_with_the_neighbour_in_the_fold(hip, cpu, hip_ops, cpu_ops, monkeypatch, t, k, n, bf16):
+    """Prefill shapes: linear_add and gate_up_stacked over 9 or more rows fold the residual add / SwiGLU into the fold of
+    the split-K partial tiles.  Against the oracle's op-by-op composition (matmul_t, add / silu, mul), against float64, and
+    against the same hooks with the folding switched off: where both split K alike, the residual form is bit for bit the
+    two kernels' result."""
+    print("rows with folded neighbour", t, k, n, "bf16" if bf16 else "f32", flush=True)
+    x = rng.normal(141, t * k)
+    w = rng.bf16_round(rng.normal(142, n * k, 0.05))
+    wgu = rng.bf16_round(rng.normal(143, 2 * n * k, 0.05))
+    r = rng.normal(144, t * n)
+    enc = rng.to_bf16_bits if bf16 else (lambda v: v)
+
+    def run(dev, ops, raw):
+        e = enc if raw else (lambda v: v)
+        o = ops.linear_add(LB.copy(x, (1, t, k), dev), LB.copy(e(w), (n, k), dev), LB.copy(r, (1, t, n), dev))
+        g = ops.gate_up_stacked(LB.copy(x, (1, t, k), dev), LB.copy(e(wgu), (2 * n, k), dev))
+        assert tuple(o.dims()) == (1, t, n) and tuple(g.dims()) == (1, t, n)
+        return o.data_vec().reshape(t, n), g.data_vec().reshape(t, n)
+
+    o_hip, g_hip = run(hip, hip_ops, True)
+    o_cpu, g_cpu = run(cpu, cpu_ops, False)
+    x64, w64, gu64 = x.reshape(t, k).astype(np.float64), w.reshape(n, k).astype(np.float64), wgu.reshape(2 * n, k).astype(np.float64)
+    o64 = x64 @ w64.T + r.reshape(t, n)
+    gg, uu = x64 @ gu64[:n].T, x64 @ gu64[n:].T
+    g64 = gg / (1.0 + np.exp(-gg)) * uu
+    eps = float(np.finfo(np.float32).eps)
+    o_bound = k * eps * (np.abs(x64) @ np.abs(w64).T) + 2 * eps * np.abs(o64) + 1e-7
+    assert np.all(np.abs(o_hip - o64) <= o_bound) and np.all(np.abs(o_cpu - o64) <= o_bound)
+    g_bound = k * eps * ((np.abs(x64) @ np.abs(gu64[:n]).T) * (np.abs(uu) * 1.3) + (np.abs(x64) @ np.abs(gu64[n:]).T) * np.abs(gg / (1.0 + np.exp(-gg)))) + 8 * eps * np.abs(g64) + 1e-7
+    assert np.all(np.abs(g_hip - g64) <= g_bound) and np.all(np.abs(g_cpu - g64) <= g_bound)
+    monkeypatch.setenv("UG_LLAMA_NO_FOLD_EPILOGUES", "1")
+    o_two, g_two = run(hip, hip_ops, True)
+    if t == 128:       # the prefill shapes split K the same way with and without the neighbour: the same sums in the same order
+        np.testing.assert_array_equal(o_hip, o_two)
+        np.testing.assert_allclose(g_hip, g_two, rtol=4 * eps, atol=1e-30)
+    else:              # a product that is not split on its own is, with a neighbour to fold in, summed in another order
+        assert np.all(np.abs(o_hip - o_two) <= 2 * o_bound) and np.all(np.abs(g_hip - g_two) <= 2 * g_bound)
+
+
+def test_projections_of_several_rows_limits(hip):
+    """The C entry points refuse what the tiled kernel does not take instead of computing something else, and accept the
+    residual as the destination."""
+    import ctypes as C
+    lib, dev = ug_amd.ughip_lib(), C.c_void_p(hip.raw_hip())
+    z = C.c_size_t
+
+    def alloc(dtype, length):
+        sl = C.c_void_p()
+        assert lib.ughip_alloc(dev, dtype, z(length), C.byref(sl)) == 0
+        return sl
+
+    m, n, k = 16, 64, 64
+    x, w, r, d = alloc(ug_amd.F32, m * k), alloc(ug_amd.F32, 2 * n * k), alloc(ug_amd.F32, m * n), alloc(ug_amd.F32, m * n)
+    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(m), z(n), z(k)) == 0, lib.ughip_last_error()
+    assert lib.ughip_linear_swiglu_rows(dev, x, w, d, z(m), z(n), z(k)) == 0, lib.ughip_last_error()
+    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(8), z(n), z(k)) != 0 and b"m >= 9" in lib.ughip_last_error()          # the row-vector kernels' job
+    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(m), z(n), z(48)) != 0 and b"k % 32" in lib.ughip_last_error()
+    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(m), z(60), z(k)) != 0 and b"n % 8" in lib.ughip_last_error()
+    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(m + 1), z(n), z(k)) != 0 and b"too short" in lib.ughip_last_error()
+    assert lib.ughip_linear_add_rows(dev, x, w, r, x, z(m), z(n), z(k)) != 0 and b"aliases" in lib.ughip_last_error()
+    assert lib.ughip_linear_add_rows(dev, x, w, None, d, z(m), z(n), z(k)) != 0 and b"null" in lib.ughip_last_error()
+    h = alloc(ug_amd.F16, 2 * n * k)
+    assert lib.ughip_linear_swiglu_rows(dev, x, h, d, z(m), z(n), z(k)) != 0 and b"F32 or BF16" in lib.ughip_last_error()
+    # dst == residual: x w^T accumulates onto the residual in place
+    xs, ws, rs = rng.normal(151, m * k), rng.normal(152, n * k, 0.1), rng.normal(153, m * n)
+    sx, sw, sr = hip.slice_from(xs), hip.slice_from(ws), hip.slice_from(rs)
+    raw = lambda s_: C.c_void_p(s_.raw())
+    assert lib.ughip_linear_add_rows(dev, raw(sx), raw(sw), raw(sr), raw(sr), z(m), z(n), z(k)) == 0, lib.ughip_last_error()
+    want = xs.reshape(m, k).astype(np.float64) @ ws.reshape(n, k).astype(np.float64).T + rs.reshape(m, n)
+    np.testing.assert_allclose(sr.to_vec().reshape(m, n), want, rtol=1e-5, atol=1e-5)
+    for sl in (x, w, r, d, h):
+        lib.ughip_free(sl)
+
+
 def test_linear_hook_reads_bf16_matrices_in_place(hip, hip_ops):
     """Ops::linear: 9 or more rows of f32 against a bf16 matrix go to the mixed product, one row to the fused
     projection, 2 to 8 rows widen the matrix first; all are the f32 result on the same values."""

@@ -740,6 +740,12 @@ class LlamaOps(_Handle):
         lb._keep += [w_gate, w_up] + ([alpha] if alpha is not None else [])
         return lb
 
+    def gate_up_stacked(self, x, w_gate_up):
+        """silu(x gate^T) * (x up^T) against one [2n, k] matrix holding the gate rows, then the up rows."""
+        lb = self._op("ugh_llama_gate_up_stacked", x, _p(w_gate_up.h))
+        lb._keep += [w_gate_up]
+        return lb
+
     def linear(self, x, w):
         """x w^T for a matrix that may be stored as bf16 under f32 rows."""
         lb = self._op("ugh_llama_linear", x, _p(w.h))

@@ -724,6 +724,9 @@ int ugh_llama_linear_packed(void* ops, void* x, size_t n_mats, void** ws, void* 
 int ugh_llama_gate_up(void* ops, void* x, void* w_gate, void* w_up, void* alpha, float eps, void** out) {
   return guard([&] { *out = box(ops_of(ops).gate_up(lb_of(x), lb_of(w_gate), lb_of(w_up), alpha ? &lb_of(alpha) : nullptr, eps)); });
 }
+int ugh_llama_gate_up_stacked(void* ops, void* x, void* w, void** out) {
+  return guard([&] { *out = box(ops_of(ops).gate_up_stacked(lb_of(x), lb_of(w))); });
+}
 int ugh_llama_linear(void* ops, void* x, void* w, void** out) {
   return guard([&] { *out = box(ops_of(ops).linear(*static_cast<LazyBuffer*>(x), *static_cast<LazyBuffer*>(w))); });
 }

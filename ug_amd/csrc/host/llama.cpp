@@ -314,7 +314,38 @@ struct HipOps : Ops {
     return LB::custom(f, args, Shape({1, 1, n}), x.dtype(), x.device());
   }
 
+  // Several positions of f32 rows against a row-major [n, k] matrix (f32 or bf16) in shapes the tiled kernel takes:
+  // the fold of its partial tiles can apply the neighbouring op.
+  static bool many_f32_rows(const LB& x, const LB& w, size_t n_multiple) {
+    if (x.rank() < 2 || w.rank() != 2 || x.dtype() != DType::F32 || (w.dtype() != DType::F32 && w.dtype() != DType::BF16)) return false;
+    const size_t k = x.dims().back(), rows = x.elem_count() / (k ? k : 1);
+    return k != 0 && w.dims()[1] == k && rows >= 9 && k % 32 == 0 && w.dims()[0] % n_multiple == 0;
+  }
+
+  LB gate_up_stacked(const LB& x, const LB& w) const override {
+    if (!many_f32_rows(x, w, 16) || getenv("UG_LLAMA_NO_FOLD_EPILOGUES")) return Ops::gate_up_stacked(x, w);
+    const size_t k = x.dims().back(), rows = x.elem_count() / k, n = w.dims()[0] / 2;
+    ughip_device* dev = hip_dev(x);
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != 3) bail("gate_up_stacked: expected 3 slices");
+      hip_check(ughip_linear_swiglu_rows(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), rows, n, k), "gate_up_stacked");
+    };
+    std::vector<size_t> dims = x.dims();
+    dims.back() = n;
+    return LB::custom(f, {x, w}, Shape(dims), DType::F32, x.device());
+  }
+
   LB linear_add(const LB& x, const LB& w, const LB& residual) const override {
+    if (many_f32_rows(x, w, 8) && residual.dtype() == DType::F32 && residual.elem_count() == x.elem_count() / x.dims().back() * w.dims()[0] &&
+        !getenv("UG_LLAMA_NO_FOLD_EPILOGUES")) {
+      const size_t k = x.dims().back(), rows = x.elem_count() / k, n = w.dims()[0];
+      ughip_device* dev = hip_dev(x);
+      auto f = [=](const std::vector<Slice*>& vs) {
+        if (vs.size() != 4) bail("linear_add: expected 4 slices");
+        hip_check(ughip_linear_add_rows(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), hip_raw_slice(*vs[3]), rows, n, k), "linear_add");
+      };
+      return LB::custom(f, {x, w, residual}, residual.shape(), DType::F32, x.device());
+    }
     if (!one_f32_row(x, {&w}) || residual.dtype() != DType::F32 || residual.elem_count() != w.dims()[0]) return Ops::linear_add(x, w, residual);
     size_t n = w.dims()[0], k = x.dims()[2];
     ughip_device* dev = hip_dev(x);
@@ -493,6 +524,13 @@ LB Ops::linear_packed(const LB& x0, const std::vector<LB>& ws, const LB* alpha, 
 LB Ops::gate_up(const LB& x0, const LB& w_gate, const LB& w_up, const LB* alpha, float eps) const {
   LB x = alpha ? rms_norm(x0, *alpha, eps) : x0;
   return silu(linear(x, w_gate)).binary(BinaryOp::Mul, linear(x, w_up));
+}
+
+// the same from the stacked matrix: SwiGLU on the two halves of the product's rows
+LB Ops::gate_up_stacked(const LB& x, const LB& w_gate_up) const {
+  const size_t n = w_gate_up.dims()[0] / 2, last = x.rank() - 1;
+  LB gu = linear(x, w_gate_up);
+  return silu(gu.narrow(last, 0, n)).binary(BinaryOp::Mul, gu.narrow(last, n, n));
 }
 
 // model.rs:366-372: a projection, then the residual.
@@ -773,11 +811,8 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
 LB Model::mlp(const Layer& l, const LB& xs, const LB* residual, bool norm_first) const {
   if (residual && l.gate_up_stacked.valid() && xs.rank() == 3 && xs.dims()[0] * xs.dims()[1] > 1) {
     // several positions: gate and up in one product, SwiGLU on the two halves of its rows
-    const size_t isz = cfg_.intermediate_size;
     LB x = norm_first ? rms_norm(xs, l.rms2, (float)cfg_.rms_norm_eps) : xs;
-    LB gu = ops_->linear(x, l.gate_up_stacked);
-    LB act = silu(gu.narrow(2, 0, isz)).binary(BinaryOp::Mul, gu.narrow(2, isz, isz));
-    return ops_->linear_add(act, l.down_proj, *residual);
+    return ops_->linear_add(ops_->gate_up_stacked(x, l.gate_up_stacked), l.down_proj, *residual);
   }
   if (residual)
     return ops_->linear_add(ops_->gate_up(xs, l.gate_proj, l.up_proj, norm_first ? &l.rms2 : nullptr, (float)cfg_.rms_norm_eps), l.down_proj, *residual);
@@ -919,7 +954,9 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
     picked.maybe_allocate_uninit();
   }
 
-  auto build = [&](size_t i, PreparedStep& st) {
+  // run_now: every item is launched as soon as it is compiled (the prompt's step: its first kernels execute while the
+  // rest of its 300 items are still being looked up)
+  auto build = [&](size_t i, PreparedStep& st, bool run_now) {
     auto t0 = clock::now();
     st.t = i == 0 ? prompt.size() : 1;
     st.tokens = tokens[i];
@@ -928,8 +965,12 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
     auto t1 = clock::now();
     Schedule schedule = Schedule::create_one(st.logits);
     auto t2 = clock::now();
-    st.compiled = std::make_unique<CompiledSchedule>(schedule.compile_with_cache(ccache));
-    st.compiled->allocate_all();
+    if (run_now) {
+      st.compiled = std::make_unique<CompiledSchedule>(schedule.compile_and_run(ccache));
+    } else {
+      st.compiled = std::make_unique<CompiledSchedule>(schedule.compile_with_cache(ccache));
+      st.compiled->allocate_all();
+    }
     st.n_items = schedule.items().size();
     st.build_ms = ms_between(t0, t1);
     st.gen_ms = ms_between(t1, t2);
@@ -938,7 +979,11 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
 
   PreparedStep cur, done;
   auto t_start = clock::now();
-  build(0, cur);
+  for (Cache& c : cache) {
+    c.prev_k.maybe_allocate_uninit();
+    c.prev_v.maybe_allocate_uninit();
+  }
+  build(0, cur, true);
   auto t_decode = t_start;
   for (size_t step = 0; step <= n_steps; ++step) {
     const bool more = step < n_steps;
@@ -955,14 +1000,14 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
       std::exception_ptr run_err;
       std::thread launcher([&] {
         try {
-          cur.compiled->run();
+          if (step != 0) cur.compiled->run();  // step 0 was launched while it was compiled
         } catch (...) {
           run_err = std::current_exception();
         }
         t1 = clock::now();
       });
       try {
-        build(step + 1, next);
+        build(step + 1, next, false);
         done = PreparedStep();  // buffers go back to the pool; the stream orders their reuse behind this step's kernels
       } catch (...) {
         launcher.join();
@@ -971,12 +1016,12 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
       launcher.join();
       if (run_err) std::rethrow_exception(run_err);
     } else {
-      cur.compiled->run();
+      if (step != 0) cur.compiled->run();
       t1 = clock::now();
     }
     if (verbose)
-      fprintf(stderr, "step %zu: launches %.2fms, next build %.2fms gen %.2fms comp %.2fms, both %.2fms, items %zu (queued, no read-back)\n", step,
-              ms_between(t0, t1), next.build_ms, next.gen_ms, next.comp_ms, ms_between(t0, clock::now()), cur.n_items);
+      fprintf(stderr, "step %zu: own build %.2fms gen %.2fms comp %.2fms; launches %.2fms, next build %.2fms gen %.2fms comp %.2fms, both %.2fms, items %zu (queued, no read-back)\n", step,
+              cur.build_ms, cur.gen_ms, cur.comp_ms, ms_between(t0, t1), next.build_ms, next.gen_ms, next.comp_ms, ms_between(t0, clock::now()), cur.n_items);
     if (step == 0) {
       dev->synchronize();  // separates the prompt's time from the decode steps'
       t_decode = clock::now();

@@ -75,6 +75,8 @@ struct Ops {
   virtual LB linear_packed(const LB& x, const std::vector<LB>& ws, const LB* alpha = nullptr, float eps = 0.f) const;
   // silu(x gate^T) * (x up^T), x normalised first when alpha != nullptr
   virtual LB gate_up(const LB& x, const LB& w_gate, const LB& w_up, const LB* alpha = nullptr, float eps = 0.f) const;
+  // the same against one [2n, k] matrix holding the gate rows, then the up rows (several positions: one product)
+  virtual LB gate_up_stacked(const LB& x, const LB& w_gate_up) const;
   // x w^T + residual
   virtual LB linear_add(const LB& x, const LB& w, const LB& residual) const;
 

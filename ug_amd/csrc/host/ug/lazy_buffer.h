@@ -158,6 +158,7 @@ struct CompiledSchedule {
   std::vector<CompiledFunc> funcs;
   DevicePtr device;
   void run() const;
+  void run_one(const CompiledFunc& f) const;
   // Allocates every buffer run() would allocate lazily (schedule.rs:247-250, 268-270), so that a
   // later run() only dispatches.
   void allocate_all() const;
@@ -174,9 +175,13 @@ class Schedule {
     return compile_with_cache(c);
   }
   CompiledSchedule compile_with_cache(CompilationCache& cache) const;
+  // The same, and every item is dispatched as soon as it is compiled: on a device that queues work the first kernels
+  // execute while the later items are still being looked up.  The result is as after compile_with_cache + run().
+  CompiledSchedule compile_and_run(CompilationCache& cache) const;
   const LazyBuffer& get_arg_id(ArgId id) const;
 
  private:
+  CompiledFunc compile_item(const ScheduleItem& item, CompilationCache& cache) const;
   std::vector<ScheduleItem> items_;
   std::map<size_t, LazyBuffer> per_arg_id_;
   DevicePtr device_;

@@ -251,7 +251,23 @@ const LazyBuffer& Schedule::get_arg_id(ArgId id) const {
 CompiledSchedule Schedule::compile_with_cache(CompilationCache& cache) const {
   CompiledSchedule out;
   out.device = device_;
+  for (const ScheduleItem& item : items_) out.funcs.push_back(compile_item(item, cache));
+  return out;
+}
+
+CompiledSchedule Schedule::compile_and_run(CompilationCache& cache) const {
+  CompiledSchedule out;
+  out.device = device_;
+  out.funcs.reserve(items_.size());
   for (const ScheduleItem& item : items_) {
+    out.funcs.push_back(compile_item(item, cache));
+    out.run_one(out.funcs.back());
+  }
+  return out;
+}
+
+CompiledFunc Schedule::compile_item(const ScheduleItem& item, CompilationCache& cache) const {
+  {
     CompiledFunc call;
     switch (item.kind) {
       case ScheduleItem::MatMul:
@@ -310,9 +326,8 @@ CompiledSchedule Schedule::compile_with_cache(CompilationCache& cache) const {
         break;
       }
     }
-    out.funcs.push_back(std::move(call));
+    return call;
   }
-  return out;
 }
 
 void CompiledSchedule::allocate_all() const {
@@ -329,8 +344,12 @@ void CompiledSchedule::allocate_all() const {
 
 // schedule.rs:234-305
 void CompiledSchedule::run() const {
-  std::vector<Slice*> bs;
-  for (const CompiledFunc& f : funcs) {
+  for (const CompiledFunc& f : funcs) run_one(f);
+}
+
+void CompiledSchedule::run_one(const CompiledFunc& f) const {
+  thread_local std::vector<Slice*> bs;
+  {
     switch (f.kind) {
       case CompiledFunc::Kernel:
       case CompiledFunc::Custom: {

@@ -23,9 +23,16 @@ struct MMArgs {
 // stores only what exists.
 // rhs_bf16: the rhs is stored as bf16 under an f32 product ([n, k] row-major only) and widened on its way into LDS.
 bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf16 = false);
-// Bytes of f32 scratch the launch needs (split-K partial tiles for skinny products; 0 for most).
-size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch);
-hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, float* workspace, bool rhs_bf16 = false);
+// What the fold of the partial tiles does on its way out (f32 products only).  With an epilogue the product always goes
+// through the scratch block, even unsplit, and p.c is the epilogue's output.
+struct GemmEpilogue {
+  enum Kind { ADD = 1, SWIGLU = 2 } kind;
+  const float* residual;  // ADD: c[m, n] = product + residual[m, n].  SWIGLU: c[m, n / 2] = silu(product[:, :n/2]) * product[:, n/2:]
+};
+// Bytes of f32 scratch the launch needs (split-K partial tiles for skinny products; 0 for most without an epilogue).
+size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch, const GemmEpilogue* epi = nullptr);
+hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, float* workspace, bool rhs_bf16 = false,
+                             const GemmEpilogue* epi = nullptr);
 
 // 16-bit types, one wave per SIMD: 256 x bn tiles (bn = 256 or 128), 4 waves of 128 x bn/2 with the accumulators in the
 // accumulation registers, loads that write LDS directly, rhs [n, k]- or [k, n]-major (gemm_dma.hip).  M % 256 == 0,

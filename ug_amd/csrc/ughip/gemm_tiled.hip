@@ -21,6 +21,7 @@
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
+#include <type_traits>
 
 #include "gemm.h"
 #include "internal.h"
@@ -403,12 +404,32 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p_in, int tiles_m, int t
 }
 
 // c[i] = (T)(ws[0][i] + ws[1][i] + ... in slab order); n4 groups of 4 elements.
-template <typename T>
-__global__ void __launch_bounds__(256) gemm_split_reduce(const float* __restrict__ ws, T* __restrict__ c, size_t n4, size_t slab_elems, int nsplit) {
+// EPI = GemmEpilogue::ADD: + residual[i].  EPI = GemmEpilogue::SWIGLU: the rows of the product are n wide and c's rows n / 2:
+// c[r][j] = silu(sum[r][j]) * sum[r][n / 2 + j]; n4 then counts groups of 4 elements of c (x / (1 + exp(-x)), the form the lazy graph
+// of ug-llama/src/model.rs:44-52 computes).
+template <typename T, int EPI>
+__global__ void __launch_bounds__(256) gemm_split_reduce(const float* __restrict__ ws, T* __restrict__ c, size_t n4, size_t slab_elems, int nsplit,
+                                                         const float* __restrict__ residual, int n) {
   const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (g >= n4) return;
-  f32x4 s = reinterpret_cast<const f32x4*>(ws)[g];
-  for (int k = 1; k < nsplit; ++k) s += reinterpret_cast<const f32x4*>(ws + (size_t)k * slab_elems)[g];
+  f32x4 s;
+  if constexpr (EPI == GemmEpilogue::SWIGLU) {
+    const size_t half4 = (size_t)n / 8, r = g / half4, j4 = g % half4;  // groups of 4 per row of c
+    const size_t gate = r * ((size_t)n / 4) + j4, up = gate + half4;
+    f32x4 a = reinterpret_cast<const f32x4*>(ws)[gate], b = reinterpret_cast<const f32x4*>(ws)[up];
+    for (int k = 1; k < nsplit; ++k) {
+      a += reinterpret_cast<const f32x4*>(ws + (size_t)k * slab_elems)[gate];
+      b += reinterpret_cast<const f32x4*>(ws + (size_t)k * slab_elems)[up];
+    }
+    s.x = a.x / (1.f + expf(-a.x)) * b.x;
+    s.y = a.y / (1.f + expf(-a.y)) * b.y;
+    s.z = a.z / (1.f + expf(-a.z)) * b.z;
+    s.w = a.w / (1.f + expf(-a.w)) * b.w;
+  } else {
+    s = reinterpret_cast<const f32x4*>(ws)[g];
+    for (int k = 1; k < nsplit; ++k) s += reinterpret_cast<const f32x4*>(ws + (size_t)k * slab_elems)[g];
+    if constexpr (EPI == GemmEpilogue::ADD) s += reinterpret_cast<const f32x4*>(residual)[g];
+  }
   T* o = c + g * 4;
   o[0] = (T)s.x;
   o[1] = (T)s.y;
@@ -428,7 +449,7 @@ hipError_t allow_lds(const void* kernel, int lds_bytes, std::atomic<unsigned lon
 }
 
 template <typename T, int B_NK, int BM, int BN, int NT, bool SPLIT, bool RAGGED = false>
-hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch, int nsplit, float* ws) {
+hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch, int nsplit, float* ws, const GemmEpilogue* epi) {
   constexpr int LDS_BYTES = 2 * (BM + BN) * CHUNKS * 16;
   constexpr int BK = Elt<T>::BK;
   static std::atomic<unsigned long long> configured{0};  // one bit per device: the attribute is per device
@@ -443,24 +464,35 @@ hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch, int nsplit,
   if (hipError_t e = hipGetLastError()) return e;
   if (SPLIT) {
     const size_t elems = batch * (size_t)p.M * p.N;  // contiguous [batch, M, N] result: c_bs == M * N
-    gemm_split_reduce<T><<<dim3((unsigned)((elems / 4 + 255) / 256)), dim3(256), 0, stream>>>(ws, static_cast<T*>(p.c), elems / 4, elems, nsplit);
+    const dim3 grid((unsigned)((elems / 4 + 255) / 256)), half_grid((unsigned)((elems / 8 + 255) / 256));
+    if constexpr (std::is_same<T, float>::value) {
+      if (epi && epi->kind == GemmEpilogue::ADD)
+        gemm_split_reduce<T, GemmEpilogue::ADD><<<grid, dim3(256), 0, stream>>>(ws, static_cast<T*>(p.c), elems / 4, elems, nsplit, epi->residual, p.N);
+      else if (epi)
+        gemm_split_reduce<T, GemmEpilogue::SWIGLU><<<half_grid, dim3(256), 0, stream>>>(ws, static_cast<T*>(p.c), elems / 8, elems, nsplit, nullptr, p.N);
+      else
+        gemm_split_reduce<T, 0><<<grid, dim3(256), 0, stream>>>(ws, static_cast<T*>(p.c), elems / 4, elems, nsplit, nullptr, p.N);
+    } else {
+      if (epi) return hipErrorInvalidValue;
+      gemm_split_reduce<T, 0><<<grid, dim3(256), 0, stream>>>(ws, static_cast<T*>(p.c), elems / 4, elems, nsplit, nullptr, p.N);
+    }
     return hipGetLastError();
   }
   return hipSuccess;
 }
 
 template <typename T, int B_NK, bool SPLIT>
-hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int shape, int nsplit, float* ws) {
+hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int shape, int nsplit, float* ws, const GemmEpilogue* epi = nullptr) {
   switch (shape) {
     case 0:
-      return getenv("UGHIP_GEMM_4WAVES") ? launch<T, B_NK, 256, 128, 256, SPLIT>(stream, p, batch, nsplit, ws)
-                                         : launch<T, B_NK, 256, 128, 512, SPLIT>(stream, p, batch, nsplit, ws);
+      return getenv("UGHIP_GEMM_4WAVES") ? launch<T, B_NK, 256, 128, 256, SPLIT>(stream, p, batch, nsplit, ws, epi)
+                                         : launch<T, B_NK, 256, 128, 512, SPLIT>(stream, p, batch, nsplit, ws, epi);
     case 1:
-      return p.M % 128 || p.N % 128 ? launch<T, B_NK, 128, 128, 256, SPLIT, true>(stream, p, batch, nsplit, ws)
-                                    : launch<T, B_NK, 128, 128, 256, SPLIT>(stream, p, batch, nsplit, ws);
+      return p.M % 128 || p.N % 128 ? launch<T, B_NK, 128, 128, 256, SPLIT, true>(stream, p, batch, nsplit, ws, epi)
+                                    : launch<T, B_NK, 128, 128, 256, SPLIT>(stream, p, batch, nsplit, ws, epi);
     default:
-      return p.M % 128 || p.N % 64 ? launch<T, B_NK, 128, 64, 256, SPLIT, true>(stream, p, batch, nsplit, ws)
-                                   : launch<T, B_NK, 128, 64, 256, SPLIT>(stream, p, batch, nsplit, ws);
+      return p.M % 128 || p.N % 64 ? launch<T, B_NK, 128, 64, 256, SPLIT, true>(stream, p, batch, nsplit, ws, epi)
+                                   : launch<T, B_NK, 128, 64, 256, SPLIT>(stream, p, batch, nsplit, ws, epi);
   }
 }
 
@@ -493,18 +525,30 @@ int pick_shape(const MMArgs& p, size_t batch, int dtype) {
 
 // How many K slabs per output tile: only when the tiles alone leave most CUs idle and K is long
 // enough that every slab still has a few tiles to pipeline.
-int pick_split(int dtype, const MMArgs& p, size_t batch, int shape) {
+int pick_split(int dtype, const MMArgs& p, size_t batch, int shape, bool always_fold = false) {
   if (const char* e = getenv("UGHIP_GEMM_SPLIT")) return std::max(1, atoi(e));  // tuning aid
   const int bk = dtype == UGHIP_F32 ? 32 : 64;
   const size_t tiles = batch * (size_t)((p.M + kShapes[shape][0] - 1) / kShapes[shape][0]) * (size_t)((p.N + kShapes[shape][1] - 1) / kShapes[shape][1]);
   const int kt = p.K / bk;
   if (tiles >= 256 || kt < 8) return 1;
   if ((batch * (size_t)p.M * (size_t)p.N) % 4 != 0) return 1;  // the fold of the partial tiles works on groups of 4 elements
-  // three workgroups per CU: measured on the projections of a 128-token prefill, short slabs overlap
-  // each other's pipeline fill better than one workgroup per CU with longer ones
-  int want = (int)((768 + tiles - 1) / tiles);
-  want = std::min(want, kt / 4);  // at least 4 K tiles per slab
-  return std::max(1, std::min(want, 32));
+  // A launch takes as long as its busiest CU: with ns slabs per tile the tiles * ns workgroups go round the 256 CUs
+  // ceil(tiles * ns / 256) times, each multiplying ceil(kt / ns) K tiles, and the fold moves every slab twice.  The
+  // times of the prefill products (128 rows against 2048..11264 x 2048..5632) follow this to 10 %: 32 tiles take 8
+  // slabs (one workgroup per CU), 40 take 6, 176 take 4.
+  const int max_split = std::min(32, kt / 4);  // at least 4 K tiles per slab
+  // one K tile of a workgroup alone on its CU; a [k, n]-major rhs is transposed on its way to LDS
+  const double tile_us = (dtype == UGHIP_F32 ? 1.03 : 0.4) * (p.b_cs == 1 ? 1.35 : 1.0) * (kShapes[shape][0] * kShapes[shape][1]) / 8192.0;
+  const double slab_us = 2.0 * (double)batch * p.M * p.N * 4 / 5e6, fold_us = 5.0;
+  int best = 1;
+  double best_cost = (double)((tiles + 255) / 256) * kt * tile_us + (always_fold ? slab_us + fold_us : 0.0);  // an epilogue folds even one slab
+  for (int ns = 2; ns <= max_split; ++ns) {
+    const int kt_per = (kt + ns - 1) / ns;
+    if ((kt + kt_per - 1) / kt_per != ns) continue;  // the launch would drop the empty slabs: same as a smaller ns
+    const double cost = (double)((tiles * ns + 255) / 256) * kt_per * tile_us + ns * slab_us + fold_us;
+    if (cost < best_cost) best = ns, best_cost = cost;
+  }
+  return best;
 }
 
 }  // namespace
@@ -525,32 +569,33 @@ bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf1
   return batch * (size_t)((p.M + kShapes[s][0] - 1) / kShapes[s][0]) * (size_t)((p.N + kShapes[s][1] - 1) / kShapes[s][1]) < (1u << 24);
 }
 
-size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch) {
+size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch, const GemmEpilogue* epi) {
   const int s = pick_shape(p, batch, dtype);
   if (s < 0) return 0;
-  const int nsplit = pick_split(dtype, p, batch, s);
-  return nsplit > 1 ? (size_t)nsplit * batch * (size_t)p.M * p.N * sizeof(float) : 0;
+  const int nsplit = pick_split(dtype, p, batch, s, epi != nullptr);
+  return nsplit > 1 || epi ? (size_t)nsplit * batch * (size_t)p.M * p.N * sizeof(float) : 0;
 }
 
-hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, float* workspace, bool rhs_bf16) {
+hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, float* workspace, bool rhs_bf16, const GemmEpilogue* epi) {
   const bool nt = p.b_rs == 1 && p.b_cs != 1;
   if (rhs_bf16 && (dtype != UGHIP_F32 || !nt)) return hipErrorInvalidValue;
+  if (epi && (dtype != UGHIP_F32 || (batch * (size_t)p.M * (size_t)p.N) % 8 != 0 || p.N % 8 != 0)) return hipErrorInvalidValue;
   const int s = pick_shape(p, batch, dtype);
   if (s < 0) return hipErrorInvalidValue;
-  const int nsplit = pick_split(dtype, p, batch, s);
+  const int nsplit = pick_split(dtype, p, batch, s, epi != nullptr);
   {
     const char* tn = rhs_bf16 ? "f32xbf16" : dtype == UGHIP_F32 ? "f32" : dtype == UGHIP_F16 ? "f16" : "bf16";
     const bool ragged = s != 0 && s != 3 && (p.M % kShapes[s][0] || p.N % kShapes[s][1]);
     char split[32] = "";
-    if (nsplit > 1) snprintf(split, sizeof split, ",splitK=%d", nsplit);
+    if (nsplit > 1 || epi) snprintf(split, sizeof split, ",splitK=%d%s", nsplit, !epi ? "" : epi->kind == GemmEpilogue::ADD ? ",+residual" : ",swiglu");
     note_kernel("gemm_tiled<%s,%s,%dx%d,%dt%s%s>", tn, nt ? "NT" : "NN", kShapes[s][0], kShapes[s][1], s == 0 && !getenv("UGHIP_GEMM_4WAVES") ? 512 : 256,
                   ragged ? ",ragged" : "", split);
   }
-  if (nsplit > 1) {
+  if (nsplit > 1 || epi) {
     if (!workspace) return hipErrorInvalidValue;
-    if (rhs_bf16) return launch_shape<float, 2, true>(stream, p, batch, s, nsplit, workspace);
+    if (rhs_bf16) return launch_shape<float, 2, true>(stream, p, batch, s, nsplit, workspace, epi);
     if (dtype == UGHIP_F32)
-      return nt ? launch_shape<float, true, true>(stream, p, batch, s, nsplit, workspace) : launch_shape<float, false, true>(stream, p, batch, s, nsplit, workspace);
+      return nt ? launch_shape<float, true, true>(stream, p, batch, s, nsplit, workspace, epi) : launch_shape<float, false, true>(stream, p, batch, s, nsplit, workspace, epi);
     if (dtype == UGHIP_F16)
       return nt ? launch_shape<_Float16, true, true>(stream, p, batch, s, nsplit, workspace) : launch_shape<_Float16, false, true>(stream, p, batch, s, nsplit, workspace);
     return nt ? launch_shape<__bf16, true, true>(stream, p, batch, s, nsplit, workspace) : launch_shape<__bf16, false, true>(stream, p, batch, s, nsplit, workspace);

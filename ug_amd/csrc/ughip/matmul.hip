@@ -406,6 +406,20 @@ int matmul_scratch_setup(ughip_device* dev) {
 }
 }  // namespace ughip
 
+// The per-device block the split-K partial tiles go to, grown (never shrunk) to `bytes`.
+static int grow_gemm_ws(ughip_device* dev, size_t bytes) {
+  if (bytes <= dev->gemm_ws_bytes) return UGHIP_OK;
+  std::lock_guard<std::mutex> g(dev->mu);
+  UGHIP_HIPCHK(hipStreamSynchronize(dev->stream));  // earlier launches may still read the old block
+  if (dev->gemm_ws) (void)hipFree(dev->gemm_ws);
+  dev->gemm_ws = nullptr;
+  dev->gemm_ws_bytes = 0;
+  const size_t want = std::max<size_t>(bytes, (size_t)32 << 20);
+  UGHIP_HIPCHK(hipMalloc(&dev->gemm_ws, want));
+  dev->gemm_ws_bytes = want;
+  return UGHIP_OK;
+}
+
 static int matmul_impl(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs, const ughip_slice* rhs, size_t b, size_t m, size_t n, size_t k,
                        size_t rank, const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset, const size_t* rhs_dims, const size_t* rhs_strides,
                        size_t rhs_offset, bool no_alloc) {
@@ -491,16 +505,7 @@ static int matmul_impl(ughip_device* dev, ughip_slice* dst, const ughip_slice* l
       UGHIP_HIPCHK(gemm_tiled_launch(st, dst->dtype, p, b, ws_bytes ? static_cast<float*>(dev->static_scratch) : nullptr, mixed));
       return UGHIP_OK;
     }
-    if (ws_bytes > dev->gemm_ws_bytes) {
-      std::lock_guard<std::mutex> g(dev->mu);
-      UGHIP_HIPCHK(hipStreamSynchronize(st));  // earlier launches may still read the old block
-      if (dev->gemm_ws) (void)hipFree(dev->gemm_ws);
-      dev->gemm_ws = nullptr;
-      dev->gemm_ws_bytes = 0;
-      const size_t want = std::max<size_t>(ws_bytes, (size_t)32 << 20);
-      UGHIP_HIPCHK(hipMalloc(&dev->gemm_ws, want));
-      dev->gemm_ws_bytes = want;
-    }
+    if (int rc = grow_gemm_ws(dev, ws_bytes)) return rc;
     UGHIP_HIPCHK(gemm_tiled_launch(st, dst->dtype, p, b, ws_bytes ? static_cast<float*>(dev->gemm_ws) : nullptr, mixed));
     return UGHIP_OK;
   } else {
@@ -525,4 +530,44 @@ extern "C" int ughip_matmul_noalloc(ughip_device* dev, ughip_slice* dst, const u
                                     size_t k, size_t rank, const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset,
                                     const size_t* rhs_dims, const size_t* rhs_strides, size_t rhs_offset) {
   return matmul_impl(dev, dst, lhs, rhs, b, m, n, k, rank, lhs_dims, lhs_strides, lhs_offset, rhs_dims, rhs_strides, rhs_offset, true);
+}
+
+// x [m, k] f32 against a row-major [rows, k] matrix (f32 or bf16) through the tiled kernel, the fold applying `epi`.
+static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x, const ughip_slice* w, const ughip_slice* residual, ughip_slice* dst, size_t m,
+                       size_t rows, size_t k, GemmEpilogue::Kind kind) {
+  if (!dev || !x || !w || !dst || (kind == GemmEpilogue::ADD && !residual)) return set_error(UGHIP_ERR_INVALID, "%s: null argument", what);
+  if (x->dtype != UGHIP_F32 || dst->dtype != UGHIP_F32 || (residual && residual->dtype != UGHIP_F32) || (w->dtype != UGHIP_F32 && w->dtype != UGHIP_BF16))
+    return set_error(UGHIP_ERR_INVALID, "%s: x, residual and dst are F32, the matrix F32 or BF16 (got x %s, w %s, dst %s)", what, dtype_name(x->dtype),
+                     dtype_name(w->dtype), dtype_name(dst->dtype));
+  if (dst == x || dst == w) return set_error(UGHIP_ERR_INVALID, "%s: dst aliases an operand", what);
+  if (m > 0x7fffffffull || rows > 0x7fffffffull || k > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "%s: shape too large", what);
+  const size_t out_cols = kind == GemmEpilogue::SWIGLU ? rows / 2 : rows;
+  if (x->len < m * k || w->len < rows * k || dst->len < m * out_cols || (residual && residual->len < m * rows))
+    return set_error(UGHIP_ERR_BOUNDS, "%s: a buffer is too short for m %zu, n %zu, k %zu", what, m, out_cols, k);
+  if (m == 0 || rows == 0) return UGHIP_OK;
+  MMArgs p;
+  p.M = (int)m, p.N = (int)rows, p.K = (int)k;
+  p.a_rs = (long long)k, p.a_cs = 1, p.b_rs = 1, p.b_cs = (long long)k;
+  p.a_bs = (long long)(m * k), p.b_bs = (long long)(rows * k), p.c_bs = (long long)(m * rows);
+  p.a = x->ptr, p.b = w->ptr, p.c = dst->ptr;
+  const bool mixed = w->dtype == UGHIP_BF16;
+  if (m < 9 || rows % 8 != 0 || (kind == GemmEpilogue::SWIGLU && rows % 16 != 0) || !gemm_tiled_supported(UGHIP_F32, p, 1, mixed))
+    return set_error(UGHIP_ERR_UNSUPPORTED, "%s: built for m >= 9 rows, k %% 32 == 0, n %% 8 == 0 and 16-byte aligned buffers (got m %zu, n %zu, k %zu)", what, m,
+                     out_cols, k);
+  if (int rc = device_activate(dev)) return rc;
+  const GemmEpilogue epi{kind, residual ? static_cast<const float*>(residual->ptr) : nullptr};
+  const size_t ws_bytes = gemm_tiled_workspace_bytes(UGHIP_F32, p, 1, &epi);
+  if (int rc = grow_gemm_ws(dev, ws_bytes)) return rc;
+  UGHIP_HIPCHK(gemm_tiled_launch(dev->stream, UGHIP_F32, p, 1, static_cast<float*>(dev->gemm_ws), mixed, &epi));
+  return UGHIP_OK;
+}
+
+extern "C" int ughip_linear_add_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w, const ughip_slice* residual, ughip_slice* dst, size_t m,
+                                     size_t n, size_t k) {
+  return linear_rows(dev, "linear_add_rows", x, w, residual, dst, m, n, k, GemmEpilogue::ADD);
+}
+
+extern "C" int ughip_linear_swiglu_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w, ughip_slice* dst, size_t m, size_t n, size_t k) {
+  if (n > 0x3fffffffull) return set_error(UGHIP_ERR_INVALID, "linear_swiglu_rows: shape too large");
+  return linear_rows(dev, "linear_swiglu_rows", x, w, nullptr, dst, m, 2 * n, k, GemmEpilogue::SWIGLU);
 }
