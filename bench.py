@@ -231,10 +231,112 @@ def extras(dev, steps, warmup, only=None):
         out.update(llama_pieces(dev, steps, warmup))
     if only in (None, "hbm_large"):
         out.update(hbm_large(dev, steps, warmup))
+    if only in (None, "floors"):
+        out.update(launch_and_barrier_floors(dev))
     if only in (None, "safetensors"):
         out.update(safetensors_load(dev))
     if only in (None, "cpu"):
         out.update(cpu_extras())
+    return out
+
+
+FLOOR_CHAIN_SRC = r"""
+extern "C" __global__ void bench_chain_step(const float* x, float* y) {
+  const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+  y[i] = x[i] + 1.0f;
+}
+"""
+
+# `iters` barriers inside one launch.  Arrivals go to 16 counters (workgroup % 16), every workgroup polls all 16;
+# between barriers every workgroup hands a value to its neighbour through memory (stored and loaded at agent scope),
+# so a barrier that lets someone through early shows up in stale[0].  A poll gives up after 2^22 rounds (gave_up[0]).
+FLOOR_BARRIER_SRC = r"""
+#define G 16
+#define PAD 64
+#define ITERS %d
+__device__ __forceinline__ bool grid_barrier(unsigned* counters, unsigned target, unsigned* gave_up) {
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __builtin_amdgcn_s_waitcnt(0);
+    __hip_atomic_fetch_add(&counters[(blockIdx.x %% G) * PAD], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  bool ok = true;
+  if (threadIdx.x < G) {
+    unsigned spins = 0;
+    while (__hip_atomic_load(&counters[threadIdx.x * PAD], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+      __builtin_amdgcn_s_sleep(1);
+      if (++spins > (1u << 22) || __hip_atomic_load(gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) { ok = false; break; }
+    }
+    if (!ok) __hip_atomic_store(gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  return ok;
+}
+extern "C" __global__ void __launch_bounds__(256) bench_grid_barrier(unsigned* counters, float* data, unsigned* gave_up, unsigned* stale) {
+  const unsigned n = gridDim.x;
+  const unsigned hits = threadIdx.x < G ? (n - threadIdx.x + G - 1) / G : 0;  // workgroups that arrive at this thread's counter
+  for (unsigned it = 0; it < ITERS; ++it) {
+    if (threadIdx.x == 0) __hip_atomic_store(&data[blockIdx.x * 16], (float)(it + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!grid_barrier(counters, hits * (it + 1), gave_up)) return;
+    if (threadIdx.x == 0 && __hip_atomic_load(&data[((blockIdx.x + 1) %% n) * 16], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (float)(it + 1)) atomicAdd(stale, 1u);
+  }
+}
+"""
+
+
+def launch_and_barrier_floors(dev):
+    """What one dependent step costs on this box, the two ways a decode step can be cut into steps: (a) a chain of
+    launches on one stream, each reading what the one before wrote; (b) a grid-wide barrier with a value handed over
+    through memory inside one resident kernel, at 64 / 256 / 512 workgroups.  Both kernels are built from source
+    through ughip_compile_source and run through ughip_run."""
+    import ug_amd
+    lib, raw = ug_amd.ughip_lib(), C.c_void_p(dev.raw_hip())
+    out = {}
+
+    def compile_src(src, entry, dtypes, grid, block):
+        f = C.c_void_p()
+        dts = (C.c_int * len(dtypes))(*dtypes)
+        assert lib.ughip_compile_source(raw, src.encode(), entry.encode(), C.c_size_t(len(dtypes)), dts, C.c_uint(grid), C.c_uint(block), C.c_uint(0), C.byref(f)) == 0, lib.ughip_last_error()
+        return f
+
+    def run(f, slices):
+        arr = (C.c_void_p * len(slices))(*[C.c_void_p(s_.raw()) for s_ in slices])
+        assert lib.ughip_run(raw, f, arr, C.c_size_t(len(slices))) == 0, lib.ughip_last_error()
+
+    # One thread issues a launch every ~3 us: the chain of tiny steps measures that rate (the GPU side of a small dependent
+    # kernel, 1.2-2 us, is in the kernel traces under profiles/).
+    for name, grid in (("launch_chain_8_workgroups", 8),):
+        n = grid * 256
+        a, b = dev.slice_from(np.zeros(n, np.float32)), dev.slice_from(np.zeros(n, np.float32))
+        f = compile_src(FLOOR_CHAIN_SRC, "bench_chain_step", [ug_amd.F32, ug_amd.F32], grid, 256)
+        ab = (C.c_void_p * 2)(C.c_void_p(a.raw()), C.c_void_p(b.raw()))
+        ba = (C.c_void_p * 2)(C.c_void_p(b.raw()), C.c_void_p(a.raw()))
+        go, two = lib.ughip_run, C.c_size_t(2)
+
+        def burst():      # 100 launches with as little interpreter work between them as ctypes allows
+            for _ in range(50):
+                go(raw, f, ab, two)
+                go(raw, f, ba, two)
+        reps = 20
+        wall, ms = timed(dev, burst, reps, 2)
+        got = a.to_vec()
+        if not np.all(got == 100.0 * (reps + 2)):
+            raise RuntimeError(f"{name}: the chain lost a step ({got[:4]})")
+        out[name] = {"us_per_dependent_launch": round(ms * 1e3 / (100 * reps), 2), "host_us_per_launch": round(wall * 1e6 / (100 * reps), 2),
+                     "bytes_per_launch": 8 * n, "verified": True}
+        lib.ughip_func_release(f)
+    iters = 2000
+    for wgs in (64, 256, 512):
+        counters = dev.slice_from(np.zeros(16 * 64, np.int32))
+        data = dev.slice_from(np.zeros(wgs * 16, np.float32))
+        gave_up, stale = dev.slice_from(np.zeros(1, np.int32)), dev.slice_from(np.zeros(1, np.int32))
+        f = compile_src(FLOOR_BARRIER_SRC % iters, "bench_grid_barrier", [ug_amd.I32, ug_amd.F32, ug_amd.I32, ug_amd.I32], wgs, 256)
+        _, ms = timed(dev, lambda: run(f, [counters, data, gave_up, stale]), 1, 0)
+        g, st = int(gave_up.to_vec()[0]), int(stale.to_vec()[0])
+        if g or st or not np.all(data.to_vec()[::16] == float(iters)):
+            raise RuntimeError(f"grid barrier at {wgs} workgroups: gave up {g}, stale reads {st}")
+        out[f"grid_barrier_{wgs}_workgroups"] = {"us_per_barrier_and_handoff": round(ms * 1e3 / iters, 2), "barriers": iters, "counters": 16, "verified": True}
+        lib.ughip_func_release(f)
     return out
 
 
@@ -617,7 +719,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-llama", action="store_true")
     ap.add_argument("--headline-only", action="store_true", help="only the config-2 kernel: no extras, no llama, no CPU baseline")
-    ap.add_argument("--only", choices=["softmax", "bmm", "llama_pieces", "hbm_large", "safetensors", "cpu", "llama"], help="besides the headline, run just this group (profiler runs)")
+    ap.add_argument("--only", choices=["softmax", "bmm", "llama_pieces", "hbm_large", "floors", "safetensors", "cpu", "llama"], help="besides the headline, run just this group (profiler runs)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true", help="also run a plain 2^24-element copy kernel (counter calibration)")
     args = ap.parse_args()
