@@ -459,6 +459,23 @@ def bmm(dev, steps, warmup):
         _, ms = timed(dev, run, steps, warmup)
         tf = 2.0 * m * m * m * steps / (ms * 1e-3) / 1e12
         out[key] = {"TFLOP/s": round(tf, 2), "frac_mfma_bf16": round(tf / MFMA_BF16_PEAK_TF, 4), "us": round(ms * 1e3 / steps, 1), "kernel": kernel, "verified": chk}
+    # The products of a 128-token prompt (f32 rows against bf16 matrices stored [n, k]): the f32 matrix pipe on the widened
+    # matrix against three bf16 terms per row element on the bf16 pipe.  TFLOP/s counts 2 m n k either way.
+    t = 128
+    for label, n, k in (("qkv", 2560, 2048), ("gate_up", 11264, 2048), ("down", 2048, 5632), ("head", 32000, 2048)):
+        xh = rng.normal(21, t * k)
+        wh = rng.bf16_round(rng.normal(22, n * k, 0.05))
+        x, w = LB.copy(xh, (1, t, k), dev), LB.copy(rng.to_bf16_bits(wh), (n, k), dev)
+        for name, ops in (("f32_pipe", ug_amd.LlamaOps.hip()), ("bf16x3", ug_amd.LlamaOps.hip(bf16x3=True))):
+            key = f"prefill_{label}_128x{n}x{k}_{name}"
+            lb = ops.linear(x, w)
+            cs = Schedule.create_one(lb).compile()
+            cs.run()
+            kernel = ug_amd.last_kernel()
+            chk = check_product_rows(key, lb.data_vec().reshape(1, t, n), xh.reshape(1, t, k), np.swapaxes(wh.reshape(1, n, k), 1, 2), k, False, rows=(0, 1, 63, 64, 127))
+            _, ms = timed(dev, cs.run, steps, warmup)
+            tf = 2.0 * t * n * k * steps / (ms * 1e-3) / 1e12
+            out[key] = {"TFLOP/s": round(tf, 2), "frac_mfma_f32": round(tf / MFMA_F32_PEAK_TF, 4), "us": round(ms * 1e3 / steps, 1), "kernel": kernel, "verified": chk}
     return out
 
 
@@ -676,7 +693,7 @@ def config5_ids_check(toks, st, n_prompt, n_steps, bf16_rounded):
     return {"checked": True, "ids_equal": int(ids_o.size - diff.size), "of": int(ids_o.size), "first_difference": first, "max_abs_top1_diff": top_err, "tie_band": tie}
 
 
-def llama_decode(dev, n_prompt=128, n_steps=128, fused_attention=0, bf16_matrices=False):
+def llama_decode(dev, n_prompt=128, n_steps=128, fused_attention=0, bf16_matrices=False, bf16x3=False):
     """Config 5: TinyLlama-1.1B shape, random-init f32 weights, prefill 128 then 128 greedy steps.
     Fresh buffers are not zero-filled here (every kernel of the model writes its whole output; the
     ids are the same either way, which the GPU tests check).  fused_attention: 0 = the reference's
@@ -684,11 +701,13 @@ def llama_decode(dev, n_prompt=128, n_steps=128, fused_attention=0, bf16_matrice
     2 = caches written in place (ughip_kv_append) and ughip_attention_cached for prefill and decode;
     3 = 2 plus packed q|k|v, gate/up + SwiGLU and residual projections (ughip_gemv_multi / _gate_up / _add).
     bf16_matrices: bf16-rounded weights, the projection matrices and the head kept and streamed as bf16
-    (activations, caches, norms f32): the numbers of the f32 model on the rounded weights from half the bytes."""
+    (activations, caches, norms f32): the numbers of the f32 model on the rounded weights from half the bytes.
+    bf16x3: with bf16 matrices, products over nine or more rows (the prompt) split every row element into three bf16
+    terms and run on the bf16 matrix pipe (UGHIP_PRODUCT_BF16X3): exact product terms, f32 sums in another order."""
     import ug_amd
     from ug_amd import rng
     cfg = ug_amd.LlamaConfig()
-    ops = ug_amd.LlamaOps.hip()
+    ops = ug_amd.LlamaOps.hip(bf16x3=bf16x3)
     dev.set_zero_fill(False)
     t0 = time.perf_counter()
     model = ug_amd.LlamaModel(dev, ops, cfg, custom_softmax=True, seed=9, std=0.02, round_bf16=bf16_matrices, fused_attention=fused_attention,
@@ -704,7 +723,7 @@ def llama_decode(dev, n_prompt=128, n_steps=128, fused_attention=0, bf16_matrice
     tok_s = n_steps / (st["decode_ms"] * 1e-3)
     return {"tok/s": round(tok_s, 2), "decode_ms_per_token": round(st["decode_ms"] / n_steps, 3), "prefill_ms": round(st["prefill_ms"], 1),
             "frac_hbm_weights_only": round(tok_s * weights_bytes / 1e9 / HBM_PEAK_GBS, 4), "load_s": round(load_s, 1), "dtype": "f32 activations, bf16 matrices" if bf16_matrices else "f32", "zero_fill": False, "fused_attention": fused_attention,
-            "prompt_tokens": n_prompt, "decode_steps": n_steps, "first_ids": toks[:8].tolist(), "min_top1_margin": float(st["margins"].min()), "ids_vs_oracle_fixture": check}
+            "prefill_product": "bf16x3" if bf16x3 else "f32", "prompt_tokens": n_prompt, "decode_steps": n_steps, "first_ids": toks[:8].tolist(), "min_top1_margin": float(st["margins"].min()), "ids_vs_oracle_fixture": check}
 
 
 def main():
@@ -790,15 +809,18 @@ def main():
             line["extras"] = {"error": f"{type(e).__name__}: {e}"}
     if not (args.no_llama or args.headline_only):
         # the last entry: the same model decoding behind a 1900-token prompt (caches near their 2048 rows)
-        for key, fused, narrow, n_prompt, n_steps in (("llama_decode_f32", 0, False, 128, 128), ("llama_decode_f32_fused_attention", 1, False, 128, 128),
-                                                      ("llama_decode_f32_inplace_cache", 2, False, 128, 128),
-                                                      ("llama_decode_f32_fused_projections", 3, False, 128, 128),
-                                                      ("llama_decode_bf16_matrices", 3, True, 128, 128),
-                                                      ("llama_decode_bf16_matrices_prompt1900", 3, True, 1900, 64)):
+        # the x3 entries: the prompt's products as three bf16 terms per row element on the bf16 matrix pipe (decode steps are unchanged)
+        for key, fused, narrow, n_prompt, n_steps, x3 in (("llama_decode_f32", 0, False, 128, 128, False), ("llama_decode_f32_fused_attention", 1, False, 128, 128, False),
+                                                          ("llama_decode_f32_inplace_cache", 2, False, 128, 128, False),
+                                                          ("llama_decode_f32_fused_projections", 3, False, 128, 128, False),
+                                                          ("llama_decode_bf16_matrices", 3, True, 128, 128, False),
+                                                          ("llama_decode_bf16_matrices_prefill_bf16x3", 3, True, 128, 128, True),
+                                                          ("llama_decode_bf16_matrices_prompt1900", 3, True, 1900, 64, False),
+                                                          ("llama_decode_bf16_matrices_prompt1900_prefill_bf16x3", 3, True, 1900, 64, True)):
             if args.llama_level is not None and (fused != args.llama_level or narrow != args.llama_bf16):
                 continue
             try:
-                line.setdefault("extras", {})[key] = llama_decode(dev, n_prompt=n_prompt, n_steps=n_steps, fused_attention=fused, bf16_matrices=narrow)
+                line.setdefault("extras", {})[key] = llama_decode(dev, n_prompt=n_prompt, n_steps=n_steps, fused_attention=fused, bf16_matrices=narrow, bf16x3=x3)
             except Exception as e:  # noqa: BLE001
                 line.setdefault("extras", {})[key] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(line), flush=True)

@@ -81,6 +81,8 @@ pub const UGHIP_I32: c_int = 3;
 pub const UGHIP_I64: c_int = 4;
 
 /// Size of the static device array behind `ughip_matmul_noalloc`.
+pub const UGHIP_PRODUCT_F32: c_int = 0;
+pub const UGHIP_PRODUCT_BF16X3: c_int = 1;
 pub const UGHIP_MATMUL_NOALLOC_SCRATCH_BYTES: usize = 64 << 20;
 
 extern "C" {
@@ -380,6 +382,16 @@ extern "C" {
         n: usize,
         k: usize,
     ) -> c_int;
+    pub fn ughip_linear_rows(
+        dev: *mut UghipDevice,
+        x: *const UghipSlice,
+        w: *const UghipSlice,
+        dst: *mut UghipSlice,
+        m: usize,
+        n: usize,
+        k: usize,
+        product: c_int,
+    ) -> c_int;
     pub fn ughip_linear_add_rows(
         dev: *mut UghipDevice,
         x: *const UghipSlice,
@@ -389,6 +401,7 @@ extern "C" {
         m: usize,
         n: usize,
         k: usize,
+        product: c_int,
     ) -> c_int;
     pub fn ughip_linear_swiglu_rows(
         dev: *mut UghipDevice,
@@ -398,6 +411,7 @@ extern "C" {
         m: usize,
         n: usize,
         k: usize,
+        product: c_int,
     ) -> c_int;
     pub fn ughip_argmax_row(
         dev: *mut UghipDevice,

@@ -371,19 +371,33 @@ int ughip_rms_gemv_gate_up(ughip_device* dev, const ughip_slice* x, const ughip_
 int ughip_gemv_add(ughip_device* dev, const ughip_slice* x, const ughip_slice* w,
                    const ughip_slice* residual, ughip_slice* dst, size_t n, size_t k);
 
-/* ---- the same two for several positions (m >= 9 rows; a prefill) -------------------------------
+/* ---- the same for several positions (m >= 9 rows; a prefill) ------------------------------------
  * x is [m, k] F32 with contiguous rows, w a row-major [n, k] matrix stored as F32 or BF16, k % 32 == 0, n % 8 == 0.
  * The product is the tiled MFMA kernel's; skinny products split K over workgroups, and the fold of their
  * partial tiles (which a plain ughip_matmul of these shapes runs anyway) applies the neighbour on its way out,
  * so the residual add / SwiGLU of model.rs:99-109,160-168,366-372 costs no launch and no round trip.
+ * `product` says how F32 rows meet a BF16 matrix:
+ *   UGHIP_PRODUCT_F32     the matrix is widened on its way in and the f32 matrix pipe multiplies: bit for bit the F32
+ *                         product on the same values (also the only choice for an F32 matrix);
+ *   UGHIP_PRODUCT_BF16X3  every x is split into three bf16 terms, x = hi + mid + lo exactly to 2^-25 |x| (each term the
+ *                         nearest-even bf16 of what the terms before it left), and the bf16 matrix pipe multiplies the
+ *                         three planes by the matrix as it is stored: every product term is exact in f32, the sums are f32
+ *                         sums in another order than the f32 pipe's, and three bf16 MFMAs replace eight times their work in
+ *                         f32 ones.  Same accuracy class as the F32 product (k eps bound), not bit-identical to it.
+ *                         Needs k % 64 == 0 and a BF16 matrix.
+ * ughip_linear_rows: dst[m, n] = x w^T.
  * ughip_linear_add_rows: dst[m, n] = x w^T + residual[m, n]; dst may be residual itself (every element is read,
  * then written, by one thread).
  * ughip_linear_swiglu_rows: w is [2n, k], gate rows first then up rows: dst[m, n] = silu(x gate^T) * (x up^T).
  * Shapes the tiled kernel does not take are refused with UGHIP_ERR_UNSUPPORTED (run the pieces instead). */
+enum { UGHIP_PRODUCT_F32 = 0, UGHIP_PRODUCT_BF16X3 = 1 };
+int ughip_linear_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w, ughip_slice* dst,
+                      size_t m, size_t n, size_t k, int product);
 int ughip_linear_add_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w,
-                          const ughip_slice* residual, ughip_slice* dst, size_t m, size_t n, size_t k);
+                          const ughip_slice* residual, ughip_slice* dst, size_t m, size_t n, size_t k,
+                          int product);
 int ughip_linear_swiglu_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w,
-                             ughip_slice* dst, size_t m, size_t n, size_t k);
+                             ughip_slice* dst, size_t m, size_t n, size_t k, int product);
 
 /* ---- greedy step on the device ----------------------------------------------------------------
  * Row `row` of logits [rows, n] (F32): the index of its largest value (the lowest index among

@@ -319,7 +319,7 @@ def _config5_fixture():
         return json.load(f)
 
 
-@pytest.mark.parametrize("variant", ["f32_level0", "f32_level3", "bf16_rounded_level0", "bf16_matrices_level3"])
+@pytest.mark.parametrize("variant", ["f32_level0", "f32_level3", "bf16_rounded_level0", "bf16_matrices_level3", "bf16_matrices_level3_x3"])
 def test_config5_full_depth_greedy_ids(hip, hip_ops, variant):
     """BASELINE config 5 as stated against the oracle's run of the reference's op-by-op graph (the fixture):
     free-running ids equal up to the first position where the oracle itself holds a near-tie, and -- fed the
@@ -331,7 +331,9 @@ def test_config5_full_depth_greedy_ids(hip, hip_ops, variant):
     n_steps = fx["steps"]
     cfg = ug_amd.LlamaConfig(num_hidden_layers=fx["config"]["num_hidden_layers"])
     prompt = rng.token_ids(fx["prompt"]["seed"], fx["prompt"]["n"], cfg.vocab_size)
-    level = 3 if variant.endswith("level3") else 0
+    level = 3 if "level3" in variant else 0
+    if variant.endswith("_x3"):       # the prompt's products as three bf16 terms per row element on the bf16 matrix pipe
+        hip_ops = ug_amd.LlamaOps.hip(bf16x3=True)
     hip.set_zero_fill(False)
     try:
         model = ug_amd.LlamaModel(hip, hip_ops, cfg, custom_softmax=True, seed=fx["weights"]["seed"], std=fx["weights"]["std"], round_bf16=not variant.startswith("f32"),

@@ -1244,6 +1244,60 @@ def test_projections_of_several_rows_with_the_neighbour_in_the_fold(hip, cpu, hi
         assert np.all(np.abs(o_hip - o_two) <= 2 * o_bound) and np.all(np.abs(g_hip - g_two) <= 2 * g_bound)
 
 
+@pytest.mark.parametrize("t,k,n", [(128, 2048, 2048), (128, 5632, 2048), (128, 2048, 2560), (100, 256, 192), (37, 64, 48), (9, 64, 16), (300, 512, 1000)])
+def test_projections_of_several_rows_as_three_bf16_terms(hip, t, k, n):
+    """UGHIP_PRODUCT_BF16X3: every f32 row element is split into three bf16 terms and the bf16 matrix pipe multiplies them
+    by the BF16 matrix as stored.  The product terms are exact, so the result has the f32 product's accuracy (the k eps
+    bound against float64) without being bit-identical to it; small integers, whose sums are exact in any order, come
+    out exactly; and the split itself loses nothing that f32 holds (x with all 24 mantissa bits set against the identity)."""
+    print("three bf16 terms", t, k, n, flush=True)
+    x3_ops = ug_amd.LlamaOps.hip(bf16x3=True)
+    f32_ops = ug_amd.LlamaOps.hip()
+    x = rng.normal(161, t * k)
+    w = rng.bf16_round(rng.normal(162, n * k, 0.05))
+    wgu = rng.bf16_round(rng.normal(163, 2 * n * k, 0.05))
+    r = rng.normal(164, t * n)
+    bits = rng.to_bf16_bits
+
+    def run(ops):
+        xs = lambda: LB.copy(x, (1, t, k), hip)
+        lin = ops.linear(xs(), LB.copy(bits(w), (n, k), hip)).data_vec().reshape(t, n)
+        kern = ug_amd.last_kernel()
+        add = ops.linear_add(xs(), LB.copy(bits(w), (n, k), hip), LB.copy(r, (1, t, n), hip)).data_vec().reshape(t, n)
+        glu = ops.gate_up_stacked(xs(), LB.copy(bits(wgu), (2 * n, k), hip)).data_vec().reshape(t, n)
+        return lin, add, glu, kern
+
+    lin3, add3, glu3, kern3 = run(x3_ops)
+    lin1, add1, glu1, kern1 = run(f32_ops)
+    assert kern3.startswith("gemm_tiled<bf16,NT,") and "f32 out" in kern3, kern3
+    assert kern1.startswith("gemm_tiled<f32xbf16,NT,"), kern1
+    x64, w64, gu64 = x.reshape(t, k).astype(np.float64), w.reshape(n, k).astype(np.float64), wgu.reshape(2 * n, k).astype(np.float64)
+    eps = float(np.finfo(np.float32).eps)
+    lin64 = x64 @ w64.T
+    bound = k * eps * (np.abs(x64) @ np.abs(w64).T) + 1e-7
+    for got in (lin3, lin1):
+        assert np.all(np.abs(got - lin64) <= bound)
+    assert np.all(np.abs(add3 - (lin64 + r.reshape(t, n))) <= bound + 2 * eps * np.abs(lin64 + r.reshape(t, n)))
+    gg, uu = x64 @ gu64[:n].T, x64 @ gu64[n:].T
+    g64 = gg / (1.0 + np.exp(-gg)) * uu
+    g_bound = k * eps * ((np.abs(x64) @ np.abs(gu64[:n]).T) * (np.abs(uu) * 1.3) + (np.abs(x64) @ np.abs(gu64[n:]).T) * np.abs(gg / (1.0 + np.exp(-gg)))) + 8 * eps * np.abs(g64) + 1e-7
+    assert np.all(np.abs(glu3 - g64) <= g_bound)
+    # the two products agree far inside the bound, and are not the same computation
+    assert np.max(np.abs(lin3 - lin1)) <= 0.25 * np.max(bound)
+    # small integers: every partial sum is exact on either pipe
+    xi, wi = np.floor(x * 4).astype(np.float32), np.floor(w * 40).astype(np.float32)
+    want = (xi.reshape(t, k).astype(np.float64) @ wi.reshape(n, k).astype(np.float64).T).astype(np.float32)
+    got = x3_ops.linear(LB.copy(xi, (1, t, k), hip), LB.copy(bits(wi), (n, k), hip)).data_vec().reshape(t, n)
+    np.testing.assert_array_equal(got, want)
+    # all 24 mantissa bits survive the split: x against rows of the identity comes back bit for bit
+    if n >= k:
+        full = (np.float32(1.0) + np.arange(t * k, dtype=np.float32).reshape(t, k) % 8388607 * np.float32(2.0 ** -23)) * rng.normal(165, t * k).reshape(t, k).astype(np.float32)
+        eye = np.zeros((n, k), np.float32)
+        eye[np.arange(k), np.arange(k)] = 1.0
+        back = x3_ops.linear(LB.copy(full.ravel(), (1, t, k), hip), LB.copy(bits(eye.ravel()), (n, k), hip)).data_vec().reshape(t, n)
+        np.testing.assert_array_equal(back[:, :k], full)
+
+
 def test_projections_of_several_rows_limits(hip):
     """The C entry points refuse what the tiled kernel does not take instead of computing something else, and accept the
     residual as the destination."""
@@ -1258,24 +1312,31 @@ def test_projections_of_several_rows_limits(hip):
 
     m, n, k = 16, 64, 64
     x, w, r, d = alloc(ug_amd.F32, m * k), alloc(ug_amd.F32, 2 * n * k), alloc(ug_amd.F32, m * n), alloc(ug_amd.F32, m * n)
-    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(m), z(n), z(k)) == 0, lib.ughip_last_error()
-    assert lib.ughip_linear_swiglu_rows(dev, x, w, d, z(m), z(n), z(k)) == 0, lib.ughip_last_error()
-    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(8), z(n), z(k)) != 0 and b"m >= 9" in lib.ughip_last_error()          # the row-vector kernels' job
-    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(m), z(n), z(48)) != 0 and b"k % 32" in lib.ughip_last_error()
-    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(m), z(60), z(k)) != 0 and b"n % 8" in lib.ughip_last_error()
-    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(m + 1), z(n), z(k)) != 0 and b"too short" in lib.ughip_last_error()
-    assert lib.ughip_linear_add_rows(dev, x, w, r, x, z(m), z(n), z(k)) != 0 and b"aliases" in lib.ughip_last_error()
-    assert lib.ughip_linear_add_rows(dev, x, w, None, d, z(m), z(n), z(k)) != 0 and b"null" in lib.ughip_last_error()
+    f32p, x3p = C.c_int(0), C.c_int(1)
+    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(m), z(n), z(k), f32p) == 0, lib.ughip_last_error()
+    assert lib.ughip_linear_swiglu_rows(dev, x, w, d, z(m), z(n), z(k), f32p) == 0, lib.ughip_last_error()
+    assert lib.ughip_linear_rows(dev, x, w, d, z(m), z(n), z(k), f32p) == 0, lib.ughip_last_error()
+    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(8), z(n), z(k), f32p) != 0 and b"m >= 9" in lib.ughip_last_error()          # the row-vector kernels' job
+    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(m), z(n), z(48), f32p) != 0 and b"k % 32" in lib.ughip_last_error()
+    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(m), z(60), z(k), f32p) != 0 and b"n % 8" in lib.ughip_last_error()
+    assert lib.ughip_linear_add_rows(dev, x, w, r, d, z(m + 1), z(n), z(k), f32p) != 0 and b"too short" in lib.ughip_last_error()
+    assert lib.ughip_linear_add_rows(dev, x, w, r, x, z(m), z(n), z(k), f32p) != 0 and b"aliases" in lib.ughip_last_error()
+    assert lib.ughip_linear_add_rows(dev, x, w, None, d, z(m), z(n), z(k), f32p) != 0 and b"null" in lib.ughip_last_error()
     h = alloc(ug_amd.F16, 2 * n * k)
-    assert lib.ughip_linear_swiglu_rows(dev, x, h, d, z(m), z(n), z(k)) != 0 and b"F32 or BF16" in lib.ughip_last_error()
+    assert lib.ughip_linear_swiglu_rows(dev, x, h, d, z(m), z(n), z(k), f32p) != 0 and b"F32 or BF16" in lib.ughip_last_error()
+    assert lib.ughip_linear_rows(dev, x, w, d, z(m), z(n), z(k), x3p) != 0 and b"needs a BF16 matrix" in lib.ughip_last_error()   # the matrix here is F32
+    assert lib.ughip_linear_rows(dev, x, w, d, z(m), z(n), z(k), C.c_int(7)) != 0 and b"unknown product" in lib.ughip_last_error()
+    wb = alloc(ug_amd.BF16, 2 * n * 96)
+    assert lib.ughip_linear_rows(dev, x, wb, d, z(m), z(n), z(32), x3p) != 0 and b"k % 64" in lib.ughip_last_error()
+    assert lib.ughip_linear_rows(dev, x, wb, d, z(m), z(n), z(k), x3p) == 0, lib.ughip_last_error()
     # dst == residual: x w^T accumulates onto the residual in place
     xs, ws, rs = rng.normal(151, m * k), rng.normal(152, n * k, 0.1), rng.normal(153, m * n)
     sx, sw, sr = hip.slice_from(xs), hip.slice_from(ws), hip.slice_from(rs)
     raw = lambda s_: C.c_void_p(s_.raw())
-    assert lib.ughip_linear_add_rows(dev, raw(sx), raw(sw), raw(sr), raw(sr), z(m), z(n), z(k)) == 0, lib.ughip_last_error()
+    assert lib.ughip_linear_add_rows(dev, raw(sx), raw(sw), raw(sr), raw(sr), z(m), z(n), z(k), f32p) == 0, lib.ughip_last_error()
     want = xs.reshape(m, k).astype(np.float64) @ ws.reshape(n, k).astype(np.float64).T + rs.reshape(m, n)
     np.testing.assert_allclose(sr.to_vec().reshape(m, n), want, rtol=1e-5, atol=1e-5)
-    for sl in (x, w, r, d, h):
+    for sl in (x, w, r, d, h, wb):
         lib.ughip_free(sl)
 
 

@@ -645,6 +645,9 @@ using OpsPtr = std::shared_ptr<ug_llama::Ops>;
 int ugh_llama_ops_hip(void** out) {
   return guard([&] { *out = new OpsPtr(ug_llama::hip_ops()); });
 }
+int ugh_llama_ops_hip_ex(int bf16x3, void** out) {
+  return guard([&] { *out = new OpsPtr(ug_llama::hip_ops(bf16x3 != 0)); });
+}
 void ugh_llama_ops_free(void* o) { delete static_cast<OpsPtr*>(o); }
 static ug_llama::Ops& ops_of(void* o) {
   if (!o) bail("null ops");

@@ -29,6 +29,9 @@ ughip_device* hip_dev(const LB& lb) {
 }
 
 struct HipOps : Ops {
+  explicit HipOps(bool bf16x3 = false) : bf16x3_(bf16x3) {}
+  bool bf16x3_;
+
   LB rope_any(const LB& src, const LB& cos, const LB& sin, const LB& pos, int interleaved) const {
     if (src.rank() != 4) bail("rope: expected a rank-4 tensor, got " + src.shape().str());
     size_t b = src.dims()[0], h = src.dims()[1], t = src.dims()[2], d = src.dims()[3];
@@ -261,8 +264,13 @@ struct HipOps : Ops {
       return Ops::linear(x, w);
     const size_t n = w.dims()[0], k = w.dims()[1];
     ughip_device* dev = hip_dev(x);
+    const bool x3 = product_for(w, k) == UGHIP_PRODUCT_BF16X3 && n % 8 == 0;
     auto f = [=](const std::vector<Slice*>& vs) {
       if (vs.size() != 3) bail("linear: expected 3 slices");
+      if (x3) {
+        hip_check(ughip_linear_rows(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), rows, n, k, UGHIP_PRODUCT_BF16X3), "linear");
+        return;
+      }
       const size_t ld[3] = {1, rows, k}, ls[3] = {rows * k, k, 1}, rd[3] = {1, k, n}, rs[3] = {n * k, 1, k};
       hip_check(ughip_matmul(dev, hip_raw_slice(*vs[2]), hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), 1, rows, n, k, 3, ld, ls, 0, rd, rs, 0), "linear");
     };
@@ -314,6 +322,10 @@ struct HipOps : Ops {
     return LB::custom(f, args, Shape({1, 1, n}), x.dtype(), x.device());
   }
 
+  // How nine or more f32 rows meet this matrix: three bf16 terms per row element on the bf16 matrix pipe when that was
+  // asked for and the matrix is bf16 with k a multiple of 64, else the f32 pipe.
+  int product_for(const LB& w, size_t k) const { return bf16x3_ && w.dtype() == DType::BF16 && k % 64 == 0 ? UGHIP_PRODUCT_BF16X3 : UGHIP_PRODUCT_F32; }
+
   // Several positions of f32 rows against a row-major [n, k] matrix (f32 or bf16) in shapes the tiled kernel takes:
   // the fold of its partial tiles can apply the neighbouring op.
   static bool many_f32_rows(const LB& x, const LB& w, size_t n_multiple) {
@@ -326,9 +338,10 @@ struct HipOps : Ops {
     if (!many_f32_rows(x, w, 16) || getenv("UG_LLAMA_NO_FOLD_EPILOGUES")) return Ops::gate_up_stacked(x, w);
     const size_t k = x.dims().back(), rows = x.elem_count() / k, n = w.dims()[0] / 2;
     ughip_device* dev = hip_dev(x);
+    const int product = product_for(w, k);
     auto f = [=](const std::vector<Slice*>& vs) {
       if (vs.size() != 3) bail("gate_up_stacked: expected 3 slices");
-      hip_check(ughip_linear_swiglu_rows(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), rows, n, k), "gate_up_stacked");
+      hip_check(ughip_linear_swiglu_rows(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), rows, n, k, product), "gate_up_stacked");
     };
     std::vector<size_t> dims = x.dims();
     dims.back() = n;
@@ -340,9 +353,10 @@ struct HipOps : Ops {
         !getenv("UG_LLAMA_NO_FOLD_EPILOGUES")) {
       const size_t k = x.dims().back(), rows = x.elem_count() / k, n = w.dims()[0];
       ughip_device* dev = hip_dev(x);
+      const int product = product_for(w, k);
       auto f = [=](const std::vector<Slice*>& vs) {
         if (vs.size() != 4) bail("linear_add: expected 4 slices");
-        hip_check(ughip_linear_add_rows(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), hip_raw_slice(*vs[3]), rows, n, k), "linear_add");
+        hip_check(ughip_linear_add_rows(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), hip_raw_slice(*vs[3]), rows, n, k, product), "linear_add");
       };
       return LB::custom(f, {x, w, residual}, residual.shape(), DType::F32, x.device());
     }
@@ -402,7 +416,7 @@ struct HipOps : Ops {
 
 }  // namespace
 
-std::shared_ptr<Ops> hip_ops() { return std::make_shared<HipOps>(); }
+std::shared_ptr<Ops> hip_ops(bool bf16x3) { return std::make_shared<HipOps>(bf16x3); }
 
 // ---- synthetic weights -----------------------------------------------------------------------------
 namespace {

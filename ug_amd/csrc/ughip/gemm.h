@@ -15,6 +15,11 @@ struct MMArgs {
   long long b_rs, b_cs;  // rhs strides of (k, n), in elements
   long long a_bs, b_bs, c_bs;
   int n_tile = 0;  // set inside the tiled kernel: columns of the workgroup's tile that exist (a last tile may hang over N)
+  // [n, k]-major rhs only: b_k_div > 1 -- K tile t of the lhs meets K tile t / b_k_div of the rhs (an lhs whose K tiles come in
+  // groups of b_k_div planes of the same columns against one matrix: the rhs tile is fetched once from memory and hit in
+  // cache for the other planes); 0 or 1 = tile for tile.  b_kt0 is set inside the tiled kernel: the first K tile of the
+  // workgroup's slab.
+  int b_k_div = 0, b_kt0 = 0;
 };
 
 // Tuned kernel: 256x128, 128x128 or 128x64 tiles, K % 64 == 0 (bf16) / K % 32 == 0 (f32), lhs rows
@@ -26,8 +31,9 @@ bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf1
 // What the fold of the partial tiles does on its way out (f32 products only).  With an epilogue the product always goes
 // through the scratch block, even unsplit, and p.c is the epilogue's output.
 struct GemmEpilogue {
-  enum Kind { ADD = 1, SWIGLU = 2 } kind;
+  enum Kind { NONE = 0, ADD = 1, SWIGLU = 2 } kind;
   const float* residual;  // ADD: c[m, n] = product + residual[m, n].  SWIGLU: c[m, n / 2] = silu(product[:, :n/2]) * product[:, n/2:]
+  bool out_f32 = false;   // a 16-bit product whose fold writes f32 (p.c is then a float buffer)
 };
 // Bytes of f32 scratch the launch needs (split-K partial tiles for skinny products; 0 for most without an epilogue).
 size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch, const GemmEpilogue* epi = nullptr);

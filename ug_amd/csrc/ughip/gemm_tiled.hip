@@ -112,13 +112,14 @@ __device__ __forceinline__ void load_tiles(const T* __restrict__ A, const BT* __
     }
   }
   if (B_NK) {
-    const BT* Bp = B + (size_t)(tid >> 3) * p.b_cs + k0 + (tid & 7) * VE;
+    const size_t k0b = p.b_k_div > 1 ? (size_t)((p.b_kt0 + kt) / p.b_k_div) * BK : k0;
+    const BT* Bp = B + (size_t)(tid >> 3) * p.b_cs + k0b + (tid & 7) * VE;
     const size_t b_step = (size_t)RP * p.b_cs;
 #pragma unroll
     for (int i = 0; i < BN / RP; ++i) {
       if (RAGGED) {
         const int row = min((tid >> 3) + i * RP, p.n_tile - 1);
-        const BT* q = B + (size_t)row * p.b_cs + k0 + (tid & 7) * VE;
+        const BT* q = B + (size_t)row * p.b_cs + k0b + (tid & 7) * VE;
         if (B_NK == 2) {
           const u32x2 v = *reinterpret_cast<const u32x2*>(q);
           r.b[i].x = v.x;
@@ -334,8 +335,10 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p_in, int tiles_m, int t
   const size_t k_off = (size_t)kt0 * BK;
   const T* __restrict__ A = static_cast<const T*>(p.a) + (size_t)batch * p.a_bs + (size_t)m0 * p.a_rs + k_off;
   typedef typename RhsElt<T, B_NK>::type BT;
+  const size_t k_off_b = B_NK && p.b_k_div > 1 ? 0 : k_off;  // an rhs that meets several lhs tiles per tile is addressed from its first K tile
+  p.b_kt0 = kt0;
   const BT* __restrict__ B =
-      static_cast<const BT*>(p.b) + (size_t)batch * p.b_bs + (B_NK ? (size_t)n0 * p.b_cs + k_off : (size_t)n0 + k_off * (size_t)p.b_rs);
+      static_cast<const BT*>(p.b) + (size_t)batch * p.b_bs + (B_NK ? (size_t)n0 * p.b_cs + k_off_b : (size_t)n0 + k_off_b * (size_t)p.b_rs);
   const int KT = SPLIT ? min(kt_per, p.K / BK - kt0) : p.K / BK;
   const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
 
@@ -465,13 +468,14 @@ hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch, int nsplit,
   if (SPLIT) {
     const size_t elems = batch * (size_t)p.M * p.N;  // contiguous [batch, M, N] result: c_bs == M * N
     const dim3 grid((unsigned)((elems / 4 + 255) / 256)), half_grid((unsigned)((elems / 8 + 255) / 256));
-    if constexpr (std::is_same<T, float>::value) {
+    if (std::is_same<T, float>::value || (epi && epi->out_f32)) {
+      float* c = static_cast<float*>(p.c);
       if (epi && epi->kind == GemmEpilogue::ADD)
-        gemm_split_reduce<T, GemmEpilogue::ADD><<<grid, dim3(256), 0, stream>>>(ws, static_cast<T*>(p.c), elems / 4, elems, nsplit, epi->residual, p.N);
-      else if (epi)
-        gemm_split_reduce<T, GemmEpilogue::SWIGLU><<<half_grid, dim3(256), 0, stream>>>(ws, static_cast<T*>(p.c), elems / 8, elems, nsplit, nullptr, p.N);
+        gemm_split_reduce<float, GemmEpilogue::ADD><<<grid, dim3(256), 0, stream>>>(ws, c, elems / 4, elems, nsplit, epi->residual, p.N);
+      else if (epi && epi->kind == GemmEpilogue::SWIGLU)
+        gemm_split_reduce<float, GemmEpilogue::SWIGLU><<<half_grid, dim3(256), 0, stream>>>(ws, c, elems / 8, elems, nsplit, nullptr, p.N);
       else
-        gemm_split_reduce<T, 0><<<grid, dim3(256), 0, stream>>>(ws, static_cast<T*>(p.c), elems / 4, elems, nsplit, nullptr, p.N);
+        gemm_split_reduce<float, 0><<<grid, dim3(256), 0, stream>>>(ws, c, elems / 4, elems, nsplit, nullptr, p.N);
     } else {
       if (epi) return hipErrorInvalidValue;
       gemm_split_reduce<T, 0><<<grid, dim3(256), 0, stream>>>(ws, static_cast<T*>(p.c), elems / 4, elems, nsplit, nullptr, p.N);
@@ -579,15 +583,19 @@ size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch, cons
 hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, float* workspace, bool rhs_bf16, const GemmEpilogue* epi) {
   const bool nt = p.b_rs == 1 && p.b_cs != 1;
   if (rhs_bf16 && (dtype != UGHIP_F32 || !nt)) return hipErrorInvalidValue;
-  if (epi && (dtype != UGHIP_F32 || (batch * (size_t)p.M * (size_t)p.N) % 8 != 0 || p.N % 8 != 0)) return hipErrorInvalidValue;
+  // an epilogue writes f32: an f32 product, or a bf16 one ([n, k]-major rhs) whose fold is told to
+  if (epi && ((dtype != UGHIP_F32 && !(dtype == UGHIP_BF16 && epi->out_f32 && nt)) || (batch * (size_t)p.M * (size_t)p.N) % 8 != 0 || p.N % 8 != 0)) return hipErrorInvalidValue;
+  if (p.b_k_div > 1 && !nt) return hipErrorInvalidValue;
   const int s = pick_shape(p, batch, dtype);
   if (s < 0) return hipErrorInvalidValue;
   const int nsplit = pick_split(dtype, p, batch, s, epi != nullptr);
   {
     const char* tn = rhs_bf16 ? "f32xbf16" : dtype == UGHIP_F32 ? "f32" : dtype == UGHIP_F16 ? "f16" : "bf16";
     const bool ragged = s != 0 && s != 3 && (p.M % kShapes[s][0] || p.N % kShapes[s][1]);
-    char split[32] = "";
-    if (nsplit > 1 || epi) snprintf(split, sizeof split, ",splitK=%d%s", nsplit, !epi ? "" : epi->kind == GemmEpilogue::ADD ? ",+residual" : ",swiglu");
+    char split[48] = "";
+    if (nsplit > 1 || epi)
+      snprintf(split, sizeof split, ",splitK=%d%s%s", nsplit, !epi ? "" : epi->kind == GemmEpilogue::ADD ? ",+residual" : epi->kind == GemmEpilogue::SWIGLU ? ",swiglu" : "",
+               epi && epi->out_f32 ? ",f32 out" : "");
     note_kernel("gemm_tiled<%s,%s,%dx%d,%dt%s%s>", tn, nt ? "NT" : "NN", kShapes[s][0], kShapes[s][1], s == 0 && !getenv("UGHIP_GEMM_4WAVES") ? 512 : 256,
                   ragged ? ",ragged" : "", split);
   }
@@ -598,7 +606,7 @@ hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, siz
       return nt ? launch_shape<float, true, true>(stream, p, batch, s, nsplit, workspace, epi) : launch_shape<float, false, true>(stream, p, batch, s, nsplit, workspace, epi);
     if (dtype == UGHIP_F16)
       return nt ? launch_shape<_Float16, true, true>(stream, p, batch, s, nsplit, workspace) : launch_shape<_Float16, false, true>(stream, p, batch, s, nsplit, workspace);
-    return nt ? launch_shape<__bf16, true, true>(stream, p, batch, s, nsplit, workspace) : launch_shape<__bf16, false, true>(stream, p, batch, s, nsplit, workspace);
+    return nt ? launch_shape<__bf16, true, true>(stream, p, batch, s, nsplit, workspace, epi) : launch_shape<__bf16, false, true>(stream, p, batch, s, nsplit, workspace);
   }
   if (rhs_bf16) return launch_shape<float, 2, false>(stream, p, batch, s, 1, nullptr);
   if (dtype == UGHIP_F32)

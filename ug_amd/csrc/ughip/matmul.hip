@@ -532,42 +532,95 @@ extern "C" int ughip_matmul_noalloc(ughip_device* dev, ughip_slice* dst, const u
   return matmul_impl(dev, dst, lhs, rhs, b, m, n, k, rank, lhs_dims, lhs_strides, lhs_offset, rhs_dims, rhs_strides, rhs_offset, true);
 }
 
-// x [m, k] f32 against a row-major [rows, k] matrix (f32 or bf16) through the tiled kernel, the fold applying `epi`.
+// x = hi + mid + lo with every term a bf16 (round to nearest even of what the terms before left): 24 mantissa bits in
+// three pieces, so |x - (hi + mid + lo)| <= 2^-25 |x|.  x3 row r holds, for every 64 columns c0 .. c0 + 63 of x, the
+// three planes side by side: [hi(c0..) | mid(c0..) | lo(c0..)], i.e. K tile t of x3 is plane t % 3 of K tile t / 3 of x,
+// and the three of them meet the same K tile of the matrix one after the other.
+__device__ __forceinline__ uint16_t bf16_rne(float f) {
+  const uint32_t x = __float_as_uint(f);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);  // NaN stays NaN
+  return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
+}
+__global__ void __launch_bounds__(256) split3_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ x3, size_t n4, int k) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n4) return;
+  const size_t e = g * 4, row = e / (size_t)k, col = e % (size_t)k;
+  const float4 v = reinterpret_cast<const float4*>(x)[g];
+  const float in[4] = {v.x, v.y, v.z, v.w};
+  uint16_t hi[4], mid[4], lo[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    hi[i] = bf16_rne(in[i]);
+    const float r1 = in[i] - __uint_as_float((uint32_t)hi[i] << 16);  // exact: hi shares the leading bits of x
+    mid[i] = bf16_rne(r1);
+    const float r2 = r1 - __uint_as_float((uint32_t)mid[i] << 16);
+    lo[i] = bf16_rne(r2);
+  }
+  uint16_t* o = x3 + row * 3 * (size_t)k + (col / 64) * 192 + col % 64;
+  *reinterpret_cast<ushort4*>(o) = make_ushort4(hi[0], hi[1], hi[2], hi[3]);
+  *reinterpret_cast<ushort4*>(o + 64) = make_ushort4(mid[0], mid[1], mid[2], mid[3]);
+  *reinterpret_cast<ushort4*>(o + 128) = make_ushort4(lo[0], lo[1], lo[2], lo[3]);
+}
+
+// x [m, k] f32 against a row-major [rows, k] matrix (f32 or bf16) through the tiled kernel, the fold applying `kind`.
+// product == UGHIP_PRODUCT_BF16X3 (bf16 matrix): the rows are split into three bf16 planes first and the product runs on
+// the bf16 matrix pipe over a K of 3 k, every K tile of the matrix meeting the three planes of its columns in turn.
 static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x, const ughip_slice* w, const ughip_slice* residual, ughip_slice* dst, size_t m,
-                       size_t rows, size_t k, GemmEpilogue::Kind kind) {
+                       size_t rows, size_t k, GemmEpilogue::Kind kind, int product) {
   if (!dev || !x || !w || !dst || (kind == GemmEpilogue::ADD && !residual)) return set_error(UGHIP_ERR_INVALID, "%s: null argument", what);
   if (x->dtype != UGHIP_F32 || dst->dtype != UGHIP_F32 || (residual && residual->dtype != UGHIP_F32) || (w->dtype != UGHIP_F32 && w->dtype != UGHIP_BF16))
     return set_error(UGHIP_ERR_INVALID, "%s: x, residual and dst are F32, the matrix F32 or BF16 (got x %s, w %s, dst %s)", what, dtype_name(x->dtype),
                      dtype_name(w->dtype), dtype_name(dst->dtype));
+  if (product != UGHIP_PRODUCT_F32 && product != UGHIP_PRODUCT_BF16X3) return set_error(UGHIP_ERR_INVALID, "%s: unknown product %d", what, product);
+  if (product == UGHIP_PRODUCT_BF16X3 && w->dtype != UGHIP_BF16)
+    return set_error(UGHIP_ERR_INVALID, "%s: the three-term bf16 product needs a BF16 matrix (an F32 one would have to be split as well), got %s", what, dtype_name(w->dtype));
   if (dst == x || dst == w) return set_error(UGHIP_ERR_INVALID, "%s: dst aliases an operand", what);
-  if (m > 0x7fffffffull || rows > 0x7fffffffull || k > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "%s: shape too large", what);
+  if (m > 0x7fffffffull || rows > 0x7fffffffull || k > 0x7fffffffull / 3) return set_error(UGHIP_ERR_INVALID, "%s: shape too large", what);
   const size_t out_cols = kind == GemmEpilogue::SWIGLU ? rows / 2 : rows;
   if (x->len < m * k || w->len < rows * k || dst->len < m * out_cols || (residual && residual->len < m * rows))
     return set_error(UGHIP_ERR_BOUNDS, "%s: a buffer is too short for m %zu, n %zu, k %zu", what, m, out_cols, k);
   if (m == 0 || rows == 0) return UGHIP_OK;
+  const bool x3 = product == UGHIP_PRODUCT_BF16X3;
   MMArgs p;
-  p.M = (int)m, p.N = (int)rows, p.K = (int)k;
-  p.a_rs = (long long)k, p.a_cs = 1, p.b_rs = 1, p.b_cs = (long long)k;
-  p.a_bs = (long long)(m * k), p.b_bs = (long long)(rows * k), p.c_bs = (long long)(m * rows);
+  p.M = (int)m, p.N = (int)rows, p.K = (int)(x3 ? 3 * k : k);
+  p.a_rs = (long long)(x3 ? 3 * k : k), p.a_cs = 1, p.b_rs = 1, p.b_cs = (long long)k;
+  p.a_bs = (long long)(m * (x3 ? 3 * k : k)), p.b_bs = (long long)(rows * k), p.c_bs = (long long)(m * rows);
   p.a = x->ptr, p.b = w->ptr, p.c = dst->ptr;
-  const bool mixed = w->dtype == UGHIP_BF16;
-  if (m < 9 || rows % 8 != 0 || (kind == GemmEpilogue::SWIGLU && rows % 16 != 0) || !gemm_tiled_supported(UGHIP_F32, p, 1, mixed))
-    return set_error(UGHIP_ERR_UNSUPPORTED, "%s: built for m >= 9 rows, k %% 32 == 0, n %% 8 == 0 and 16-byte aligned buffers (got m %zu, n %zu, k %zu)", what, m,
-                     out_cols, k);
+  if (x3) p.b_k_div = 3;
+  const bool mixed = !x3 && w->dtype == UGHIP_BF16;
+  const int dtype = x3 ? UGHIP_BF16 : UGHIP_F32;
+  // (x3: p.a is checked for alignment below with the f32 rows standing in; the planes live in the 256-byte aligned scratch block)
+  if (m < 9 || rows % 8 != 0 || (kind == GemmEpilogue::SWIGLU && rows % 16 != 0) || (x3 && k % 64 != 0) || !gemm_tiled_supported(dtype, p, 1, mixed))
+    return set_error(UGHIP_ERR_UNSUPPORTED, "%s: built for m >= 9 rows, k %% 32 == 0 (k %% 64 == 0 for the three-term bf16 product), n %% 8 == 0 and 16-byte aligned buffers (got m %zu, n %zu, k %zu)",
+                     what, m, out_cols, k);
   if (int rc = device_activate(dev)) return rc;
-  const GemmEpilogue epi{kind, residual ? static_cast<const float*>(residual->ptr) : nullptr};
-  const size_t ws_bytes = gemm_tiled_workspace_bytes(UGHIP_F32, p, 1, &epi);
-  if (int rc = grow_gemm_ws(dev, ws_bytes)) return rc;
-  UGHIP_HIPCHK(gemm_tiled_launch(dev->stream, UGHIP_F32, p, 1, static_cast<float*>(dev->gemm_ws), mixed, &epi));
+  GemmEpilogue epi{kind, residual ? static_cast<const float*>(residual->ptr) : nullptr};
+  epi.out_f32 = x3;
+  const size_t ws_bytes = (gemm_tiled_workspace_bytes(dtype, p, 1, &epi) + 255) & ~(size_t)255;
+  const size_t x3_bytes = x3 ? m * 3 * k * sizeof(uint16_t) : 0;
+  if (int rc = grow_gemm_ws(dev, ws_bytes + x3_bytes)) return rc;
+  if (x3) {
+    uint16_t* planes = reinterpret_cast<uint16_t*>(static_cast<char*>(dev->gemm_ws) + ws_bytes);
+    const size_t n4 = m * k / 4;
+    split3_bf16_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, dev->stream>>>(static_cast<const float*>(x->ptr), planes, n4, (int)k);
+    UGHIP_HIPCHK(hipGetLastError());
+    p.a = planes;
+  }
+  UGHIP_HIPCHK(gemm_tiled_launch(dev->stream, dtype, p, 1, static_cast<float*>(dev->gemm_ws), mixed, &epi));
   return UGHIP_OK;
 }
 
-extern "C" int ughip_linear_add_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w, const ughip_slice* residual, ughip_slice* dst, size_t m,
-                                     size_t n, size_t k) {
-  return linear_rows(dev, "linear_add_rows", x, w, residual, dst, m, n, k, GemmEpilogue::ADD);
+extern "C" int ughip_linear_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w, ughip_slice* dst, size_t m, size_t n, size_t k, int product) {
+  return linear_rows(dev, "linear_rows", x, w, nullptr, dst, m, n, k, GemmEpilogue::NONE, product);
 }
 
-extern "C" int ughip_linear_swiglu_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w, ughip_slice* dst, size_t m, size_t n, size_t k) {
+extern "C" int ughip_linear_add_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w, const ughip_slice* residual, ughip_slice* dst, size_t m,
+                                     size_t n, size_t k, int product) {
+  return linear_rows(dev, "linear_add_rows", x, w, residual, dst, m, n, k, GemmEpilogue::ADD, product);
+}
+
+extern "C" int ughip_linear_swiglu_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w, ughip_slice* dst, size_t m, size_t n, size_t k,
+                                        int product) {
   if (n > 0x3fffffffull) return set_error(UGHIP_ERR_INVALID, "linear_swiglu_rows: shape too large");
-  return linear_rows(dev, "linear_swiglu_rows", x, w, nullptr, dst, m, 2 * n, k, GemmEpilogue::SWIGLU);
+  return linear_rows(dev, "linear_swiglu_rows", x, w, nullptr, dst, m, 2 * n, k, GemmEpilogue::SWIGLU, product);
 }
