@@ -504,54 +504,67 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 
 constexpr int kShapes[3][2] = {{256, 128}, {128, 128}, {128, 64}};
 
-// The largest tile that divides the problem and still gives every CU a workgroup; failing that,
-// the dividing tile with the most workgroups.  -1: no tile divides M x N.
-int pick_shape(const MMArgs& p, size_t batch, int dtype) {
-  const bool rhs_nk = p.b_rs == 1 && p.b_cs != 1;
-  // UGHIP_GEMM_SHAPE=0..2 forces a tile shape (tuning aid); ignored when it does not fit the problem.
-  if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
-    const int s = atoi(e);
-    if (s >= 0 && s < 3 && (p.M % kShapes[s][0] == 0 || kShapes[s][0] == 128) && (p.N % kShapes[s][1] == 0 || (kShapes[s][0] == 128 && rhs_nk))) return s;
-  }
-  int best = -1;
-  size_t best_tiles = 0;
-  for (int s = 0; s < 3; ++s) {
-    // the 128-row tiles also take an lhs whose last tile is partly empty (any M >= 9: fewer rows are the GEMV kernels'
-    // job) and, with an [n, k]-major rhs, an N they do not divide
-    const bool ragged_ok = kShapes[s][0] == 128;
-    if ((p.M % kShapes[s][0] && !ragged_ok) || (p.N % kShapes[s][1] && !(ragged_ok && rhs_nk))) continue;
-    const size_t tiles = batch * (size_t)((p.M + kShapes[s][0] - 1) / kShapes[s][0]) * (size_t)((p.N + kShapes[s][1] - 1) / kShapes[s][1]);
-    if (tiles >= 256) return s;
-    if (tiles > best_tiles) best = s, best_tiles = tiles;
-  }
-  return best;
+// Which of the three tiles a problem can take: the 128-row tiles also take an lhs whose last tile is partly empty (any
+// M >= 9: fewer rows are the GEMV kernels' job) and, with an [n, k]-major rhs, an N they do not divide.
+bool shape_fits(const MMArgs& p, int s) {
+  const bool rhs_nk = p.b_rs == 1 && p.b_cs != 1, ragged_ok = kShapes[s][0] == 128;
+  return !((p.M % kShapes[s][0] && !ragged_ok) || (p.N % kShapes[s][1] && !(ragged_ok && rhs_nk)));
+}
+size_t tile_count(const MMArgs& p, size_t batch, int s) {
+  return batch * (size_t)((p.M + kShapes[s][0] - 1) / kShapes[s][0]) * (size_t)((p.N + kShapes[s][1] - 1) / kShapes[s][1]);
 }
 
-// How many K slabs per output tile: only when the tiles alone leave most CUs idle and K is long
-// enough that every slab still has a few tiles to pipeline.
-int pick_split(int dtype, const MMArgs& p, size_t batch, int shape, bool always_fold = false) {
-  if (const char* e = getenv("UGHIP_GEMM_SPLIT")) return std::max(1, atoi(e));  // tuning aid
+// How many K slabs per output tile, and what the launch then costs (us).  A launch takes as long as its busiest CU:
+// with ns slabs per tile the tiles * ns workgroups go round the 256 CUs ceil(tiles * ns / 256) times, each multiplying
+// ceil(kt / ns) K tiles, and the fold moves every slab twice behind a launch of its own.  The times of the prefill
+// products (128 rows against 2048..32000 x 2048..5632, f32 and three-term bf16) follow this to 10 %: 32 tiles take 8
+// slabs (one workgroup per CU), 40 take 6, 176 take 4.
+struct Split {
+  int nsplit;
+  double cost_us;
+};
+Split pick_split(int dtype, const MMArgs& p, size_t batch, int shape, bool always_fold = false) {
   const int bk = dtype == UGHIP_F32 ? 32 : 64;
-  const size_t tiles = batch * (size_t)((p.M + kShapes[shape][0] - 1) / kShapes[shape][0]) * (size_t)((p.N + kShapes[shape][1] - 1) / kShapes[shape][1]);
+  const size_t tiles = tile_count(p, batch, shape);
   const int kt = p.K / bk;
-  if (tiles >= 256 || kt < 8) return 1;
-  if ((batch * (size_t)p.M * (size_t)p.N) % 4 != 0) return 1;  // the fold of the partial tiles works on groups of 4 elements
-  // A launch takes as long as its busiest CU: with ns slabs per tile the tiles * ns workgroups go round the 256 CUs
-  // ceil(tiles * ns / 256) times, each multiplying ceil(kt / ns) K tiles, and the fold moves every slab twice.  The
-  // times of the prefill products (128 rows against 2048..11264 x 2048..5632) follow this to 10 %: 32 tiles take 8
-  // slabs (one workgroup per CU), 40 take 6, 176 take 4.
-  const int max_split = std::min(32, kt / 4);  // at least 4 K tiles per slab
-  // one K tile of a workgroup alone on its CU; a [k, n]-major rhs is transposed on its way to LDS
-  const double tile_us = (dtype == UGHIP_F32 ? 1.03 : 0.4) * (p.b_cs == 1 ? 1.35 : 1.0) * (kShapes[shape][0] * kShapes[shape][1]) / 8192.0;
+  // one K tile of a workgroup alone on its CU: f32 scales with the tile, the 16-bit 128x128 tile is better fed than two
+  // 128x64 ones; a [k, n]-major rhs is transposed on its way to LDS
+  const double area = (kShapes[shape][0] * kShapes[shape][1]) / 8192.0;
+  const double tile_us = (dtype == UGHIP_F32 ? 1.03 * area : area <= 1.0 ? 0.4 : 0.325 * area) * (p.b_cs == 1 ? 1.35 : 1.0);
   const double slab_us = 2.0 * (double)batch * p.M * p.N * 4 / 5e6, fold_us = 5.0;
-  int best = 1;
-  double best_cost = (double)((tiles + 255) / 256) * kt * tile_us + (always_fold ? slab_us + fold_us : 0.0);  // an epilogue folds even one slab
+  Split best{1, (double)((tiles + 255) / 256) * kt * tile_us + (always_fold ? slab_us + fold_us : 0.0)};  // an epilogue folds even one slab
+  if (const char* e = getenv("UGHIP_GEMM_SPLIT")) return Split{std::max(1, atoi(e)), best.cost_us};  // tuning aid
+  // only when the tiles alone leave CUs idle and K is long enough that every slab still has a few tiles to pipeline; the
+  // fold of the partial tiles works on groups of 4 elements
+  if (tiles >= 256 || kt < 8 || (batch * (size_t)p.M * (size_t)p.N) % 4 != 0) return best;
+  const int max_split = std::min(32, kt / 4);  // at least 4 K tiles per slab
   for (int ns = 2; ns <= max_split; ++ns) {
     const int kt_per = (kt + ns - 1) / ns;
     if ((kt + kt_per - 1) / kt_per != ns) continue;  // the launch would drop the empty slabs: same as a smaller ns
     const double cost = (double)((tiles * ns + 255) / 256) * kt_per * tile_us + ns * slab_us + fold_us;
-    if (cost < best_cost) best = ns, best_cost = cost;
+    if (cost < best.cost_us) best = Split{ns, cost};
   }
+  return best;
+}
+
+// The largest tile that fits the problem and still gives every CU a workgroup; with fewer tiles than that, whichever
+// of 128x128 and 128x64 the cost model above makes cheaper (128x64 on a tie: more workgroups).  -1: no tile fits M x N.
+int pick_shape(const MMArgs& p, size_t batch, int dtype, bool always_fold = false) {
+  // UGHIP_GEMM_SHAPE=0..2 forces a tile shape (tuning aid); ignored when it does not fit the problem.
+  if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
+    const int s = atoi(e);
+    if (s >= 0 && s < 3 && shape_fits(p, s)) return s;
+  }
+  if (shape_fits(p, 0) && tile_count(p, batch, 0) >= 256) return 0;
+  if (shape_fits(p, 1) && tile_count(p, batch, 1) >= 256) return 1;
+  int best = -1;
+  double best_cost = 0;
+  for (int s = 2; s >= 1; --s) {
+    if (!shape_fits(p, s)) continue;
+    const double cost = pick_split(dtype, p, batch, s, always_fold).cost_us;
+    if (best < 0 || cost < best_cost * 0.97) best = s, best_cost = cost;
+  }
+  if (best < 0 && shape_fits(p, 0)) best = 0;
   return best;
 }
 
@@ -574,9 +587,9 @@ bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf1
 }
 
 size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch, const GemmEpilogue* epi) {
-  const int s = pick_shape(p, batch, dtype);
+  const int s = pick_shape(p, batch, dtype, epi != nullptr);
   if (s < 0) return 0;
-  const int nsplit = pick_split(dtype, p, batch, s, epi != nullptr);
+  const int nsplit = pick_split(dtype, p, batch, s, epi != nullptr).nsplit;
   return nsplit > 1 || epi ? (size_t)nsplit * batch * (size_t)p.M * p.N * sizeof(float) : 0;
 }
 
@@ -586,9 +599,9 @@ hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, siz
   // an epilogue writes f32: an f32 product, or a bf16 one ([n, k]-major rhs) whose fold is told to
   if (epi && ((dtype != UGHIP_F32 && !(dtype == UGHIP_BF16 && epi->out_f32 && nt)) || (batch * (size_t)p.M * (size_t)p.N) % 8 != 0 || p.N % 8 != 0)) return hipErrorInvalidValue;
   if (p.b_k_div > 1 && !nt) return hipErrorInvalidValue;
-  const int s = pick_shape(p, batch, dtype);
+  const int s = pick_shape(p, batch, dtype, epi != nullptr);
   if (s < 0) return hipErrorInvalidValue;
-  const int nsplit = pick_split(dtype, p, batch, s, epi != nullptr);
+  const int nsplit = pick_split(dtype, p, batch, s, epi != nullptr).nsplit;
   {
     const char* tn = rhs_bf16 ? "f32xbf16" : dtype == UGHIP_F32 ? "f32" : dtype == UGHIP_F16 ? "f16" : "bf16";
     const bool ragged = s != 0 && s != 3 && (p.M % kShapes[s][0] || p.N % kShapes[s][1]);
