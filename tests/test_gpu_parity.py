@@ -1298,6 +1298,55 @@ def test_projections_of_several_rows_as_three_bf16_terms(hip, t, k, n):
         np.testing.assert_array_equal(back[:, :k], full)
 
 
+def test_projections_of_several_rows_random_shapes(hip):
+    """Straight through the C ABI over 30 seeded shapes (rows the tiles do not divide, column counts that leave a last
+    tile partly empty, one to sixteen K tiles), both products, the three forms: against float64 with the k eps bound, and
+    nothing written past the result (a guard region behind dst keeps its fill)."""
+    import ctypes as C
+    lib, dev = ug_amd.ughip_lib(), C.c_void_p(hip.raw_hip())
+    z, raw = C.c_size_t, (lambda s_: C.c_void_p(s_.raw()))
+    gen = np.random.default_rng(20240607)
+    eps = float(np.finfo(np.float32).eps)
+    for case in range(30):
+        m = int(gen.integers(9, 300))
+        n = 8 * int(gen.integers(1, 96)) if case % 3 else 16 * int(gen.integers(1, 48))
+        k = 64 * int(gen.integers(1, 17))
+        product = int(gen.integers(0, 2))
+        form = case % 3                      # 0 plain, 1 + residual, 2 SwiGLU (n output columns from 2n matrix rows)
+        rows = 2 * n if form == 2 else n
+        print("rows product", case, (m, n, k), ["f32 pipe", "bf16 x3"][product], ["plain", "+residual", "swiglu"][form], flush=True)
+        x = rng.normal(300 + case, m * k)
+        w = rng.bf16_round(rng.normal(400 + case, rows * k, 0.05))
+        r = rng.normal(500 + case, m * n)
+        guard = 64
+        sx, sw = hip.slice_from(x), hip.slice_from(rng.to_bf16_bits(w))
+        sr = hip.slice_from(r)
+        sd = hip.slice_from(np.full(m * n + guard, 7.0, np.float32))
+        if form == 0:
+            rc = lib.ughip_linear_rows(dev, raw(sx), raw(sw), raw(sd), z(m), z(n), z(k), C.c_int(product))
+        elif form == 1:
+            rc = lib.ughip_linear_add_rows(dev, raw(sx), raw(sw), raw(sr), raw(sd), z(m), z(n), z(k), C.c_int(product))
+        else:
+            rc = lib.ughip_linear_swiglu_rows(dev, raw(sx), raw(sw), raw(sd), z(m), z(n), z(k), C.c_int(product))
+        assert rc == 0, lib.ughip_last_error()
+        got = sd.to_vec()
+        assert np.all(got[m * n:] == 7.0), "wrote past the end of the result"
+        got = got[:m * n].reshape(m, n)
+        x64, w64 = x.reshape(m, k).astype(np.float64), w.reshape(rows, k).astype(np.float64)
+        full, mag = x64 @ w64.T, np.abs(x64) @ np.abs(w64).T
+        if form == 0:
+            want, bound = full, k * eps * mag
+        elif form == 1:
+            want = full + r.reshape(m, n)
+            bound = k * eps * mag + 2 * eps * np.abs(want)
+        else:
+            gg, uu = full[:, :n], full[:, n:]
+            silu = gg / (1.0 + np.exp(-gg))
+            want = silu * uu
+            bound = k * eps * (mag[:, :n] * np.abs(uu) * 1.3 + mag[:, n:] * np.abs(silu)) + 8 * eps * np.abs(want)
+        assert np.all(np.abs(got - want) <= bound + 1e-7), (case, float(np.abs(got - want).max()))
+
+
 def test_projections_of_several_rows_limits(hip):
     """The C entry points refuse what the tiled kernel does not take instead of computing something else, and accept the
     residual as the destination."""
