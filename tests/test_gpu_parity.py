@@ -1417,6 +1417,24 @@ def test_llama_bf16_matrices_prefill_of_128_tokens(hip, hip_ops):
     np.testing.assert_array_equal(st["margins"], wide[1]["margins"])
 
 
+@pytest.mark.parametrize("n_prompt", [9, 37, 100, 128, 200])
+def test_llama_prompt_products_as_three_bf16_terms(hip, cpu, hip_ops, cpu_ops, n_prompt):
+    """bf16 matrices with the prompt's products as three bf16 terms per row element (prompt lengths the tiles divide and
+    do not): the oracle's ids on the same bf16-rounded weights, margins to 1e-2 relative like the f32-pipe model's, and
+    the ids of the f32-pipe model on this device."""
+    cfg = ug_amd.LlamaConfig(hidden_size=256, intermediate_size=512, max_position_embeddings=256, num_attention_heads=4, num_key_value_heads=2,
+                             num_hidden_layers=2, vocab_size=1024)
+    prompt = rng.token_ids(12, n_prompt, cfg.vocab_size)
+    x3_ops = ug_amd.LlamaOps.hip(bf16x3=True)
+    toks, st = ug_amd.LlamaModel(hip, x3_ops, cfg, True, seed=9, std=0.2, round_bf16=True, fused_attention=3, bf16_matrices=True).generate(prompt, 6)
+    pipe = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=0.2, round_bf16=True, fused_attention=3, bf16_matrices=True).generate(prompt, 6)
+    toks_c, st_c = ug_amd.LlamaModel(cpu, cpu_ops, cfg, True, seed=9, std=0.2, round_bf16=True).generate(prompt, 6)
+    print("three bf16 terms, prompt of", n_prompt, toks.tolist(), "min margin", float(st_c["margins"].min()), flush=True)
+    assert toks.tolist() == toks_c.tolist() == pipe[0].tolist()
+    np.testing.assert_allclose(st["margins"], st_c["margins"], rtol=1e-2, atol=1e-6)
+    np.testing.assert_allclose(st["margins"], pipe[1]["margins"], rtol=1e-3, atol=1e-6)
+
+
 def test_fused_projections_refuse_mixed_or_other_matrix_dtypes(hip):
     """Straight through the C ABI: one matrix dtype per call, F32 or BF16."""
     lib, dev = ug_amd.ughip_lib(), C.c_void_p(hip.raw_hip())
