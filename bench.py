@@ -221,22 +221,19 @@ def cpu_extras(budget_s=3.0):
 
 
 def extras(dev, steps, warmup, only=None):
-    """Other single-GPU configs of BASELINE.json: GB/s or TFLOP/s with the roofline fraction."""
+    """Other single-GPU configs of BASELINE.json: GB/s or TFLOP/s with the roofline fraction.  A group that fails (a check
+    that does not hold, a launch error) is reported under `<group>_error` and does not take the other groups down."""
     out = {}
-    if only in (None, "softmax"):
-        out.update(softmax_sweep(dev, steps, warmup))
-    if only in (None, "bmm"):
-        out.update(bmm(dev, steps, warmup))
-    if only in (None, "llama_pieces"):
-        out.update(llama_pieces(dev, steps, warmup))
-    if only in (None, "hbm_large"):
-        out.update(hbm_large(dev, steps, warmup))
-    if only in (None, "floors"):
-        out.update(launch_and_barrier_floors(dev))
-    if only in (None, "safetensors"):
-        out.update(safetensors_load(dev))
-    if only in (None, "cpu"):
-        out.update(cpu_extras())
+    groups = (("softmax", lambda: softmax_sweep(dev, steps, warmup)), ("bmm", lambda: bmm(dev, steps, warmup)),
+              ("llama_pieces", lambda: llama_pieces(dev, steps, warmup)), ("hbm_large", lambda: hbm_large(dev, steps, warmup)),
+              ("floors", lambda: launch_and_barrier_floors(dev)), ("safetensors", lambda: safetensors_load(dev)), ("cpu", cpu_extras))
+    for name, run in groups:
+        if only not in (None, name):
+            continue
+        try:
+            out.update(run())
+        except Exception as e:  # noqa: BLE001
+            out[f"{name}_error"] = f"{type(e).__name__}: {e}"
     return out
 
 
