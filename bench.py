@@ -456,6 +456,20 @@ def bmm(dev, steps, warmup):
         _, ms = timed(dev, run, steps, warmup)
         tf = 2.0 * m * m * m * steps / (ms * 1e-3) / 1e12
         out[key] = {"TFLOP/s": round(tf, 2), "frac_mfma_bf16": round(tf / MFMA_BF16_PEAK_TF, 4), "us": round(ms * 1e3 / steps, 1), "kernel": kernel, "verified": chk}
+    # the same kernel where the fixed cost (launch, first tile, the result's way out: ~9 us) is 1 % of the run
+    m = 8192
+    a, w = rng.uniform_pm1(4, m * m), rng.uniform_pm1(5, m * m)
+    ab, wb = rng.bf16_round(a).reshape(1, m, m), rng.bf16_round(w).reshape(1, m, m)
+    sa, sw = dev.slice_from(rng.to_bf16_bits(a)), dev.slice_from(rng.to_bf16_bits(w))
+    dst = dev.allocate_uninit(ug_amd.BF16, m * m)
+    run = lambda: dev.matmul(dst, sa, sw, (1, m, m, m), ((1, m, m), (m * m, m, 1), 0), ((1, m, m), (m * m, 1, m), 0))  # noqa: E731
+    run()
+    chk = check_product_rows("mm_bf16_nt_8192^3", rng.from_bf16_bits(dst.to_vec()).reshape(1, m, m), ab, np.swapaxes(wb, 1, 2), m, True, rows=(0, 257, 4097, 8191))
+    kernel = ug_amd.last_kernel()
+    _, ms = timed(dev, run, 20, 3)
+    tf = 2.0 * m * m * m * 20 / (ms * 1e-3) / 1e12
+    out["mm_bf16_nt_8192^3"] = {"TFLOP/s": round(tf, 2), "frac_mfma_bf16": round(tf / MFMA_BF16_PEAK_TF, 4), "us": round(ms * 1e3 / 20, 1), "kernel": kernel, "verified": chk}
+    del sa, sw, dst
     # The products of a 128-token prompt (f32 rows against bf16 matrices stored [n, k]): the f32 matrix pipe on the widened
     # matrix against three bf16 terms per row element on the bf16 pipe.  TFLOP/s counts 2 m n k either way.
     t = 128
