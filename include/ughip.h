@@ -348,10 +348,10 @@ int ughip_attention_step(ughip_device* dev, const ughip_slice* qkv, size_t row_s
  * No counterpart in the reference's device trait: there each is a matmul (lib.rs:62-70) followed
  * by the small kernels of the lazy graph.  Every product is x (k elements) against the rows of a
  * row-major [n, k] matrix, k % 4 == 0, summed in a fixed order.  x, alpha, residual and dst are F32;
- * the matrices are F32 or BF16 (all of one call alike).  A BF16 matrix gives bit for bit the result
- * of the same values stored as F32 (a bf16 widens exactly) from half the bytes: the form a decoder
- * keeps a bf16 checkpoint in, where the reference widens it at load time
- * (ug-core/src/safetensors.rs:120-271).
+ * the matrices are F32 or BF16 (all of one call alike).  A BF16 matrix gives the result of the same
+ * values stored as F32 (a bf16 widens exactly; the f32 sums may run in another order, both within
+ * the k * eps bound of the exact product) from half the bytes: the form a decoder keeps a bf16
+ * checkpoint in, where the reference widens it at load time (ug-core/src/safetensors.rs:120-271).
  * ughip_gemv_multi: dst[0 .. n0+n1+n2) = [x W_0^T | x W_1^T | x W_2^T] for n_mats <= 3 matrices
  * (the q, k, v projections of ug-llama/src/model.rs:206-208 in one launch). */
 int ughip_gemv_multi(ughip_device* dev, const ughip_slice* x, size_t n_mats,

@@ -801,9 +801,9 @@ def test_llama_fused_attention_ids_match_unfused_cpu(hip, cpu, hip_ops, cpu_ops,
 
 @pytest.mark.parametrize("width", ["small", "config5"])
 def test_llama_bf16_matrices_are_the_rounded_f32_model(hip, cpu, hip_ops, cpu_ops, width):
-    """Matrices kept and streamed as bf16 (fusion level 3): token for token and margin for margin the
-    f32 model on the same device whose weights hold the same (bf16-representable) values; ids equal to
-    the oracle's op-by-op f32 graph on those weights."""
+    """Matrices kept and streamed as bf16 (fusion level 3): token for token the f32 model on the same device whose
+    weights hold the same (bf16-representable) values, margins equal where both run the same kernels and to 1e-3
+    where the bf16 rows have a kernel of their own; ids equal to the oracle's op-by-op f32 graph on those weights."""
     if width == "small":
         cfg = ug_amd.LlamaConfig(hidden_size=128, intermediate_size=320, max_position_embeddings=64, num_attention_heads=4, num_key_value_heads=2,
                                  num_hidden_layers=2, vocab_size=512)
@@ -816,7 +816,10 @@ def test_llama_bf16_matrices_are_the_rounded_f32_model(hip, cpu, hip_ops, cpu_op
     toks, st = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=std, round_bf16=True, fused_attention=3, bf16_matrices=True).generate(prompt, n_steps)
     print("bf16 matrices", toks.tolist(), flush=True)
     assert toks.tolist() == wide[0].tolist()
-    assert np.array_equal(st["margins"], wide[1]["margins"])
+    if width == "small":
+        assert np.array_equal(st["margins"], wide[1]["margins"])   # rows of 128 elements: the same kernels, the same order of the sums
+    else:
+        np.testing.assert_allclose(st["margins"], wide[1]["margins"], rtol=1e-3, atol=1e-7)   # rows of 2048: the bf16 kernels' own order
     toks_c, st_c = ug_amd.LlamaModel(cpu, cpu_ops, cfg, True, seed=9, std=std, round_bf16=True).generate(prompt, n_steps)
     assert wide[0].tolist() == toks_c.tolist()
     np.testing.assert_allclose(wide[1]["margins"], st_c["margins"], rtol=1e-2, atol=1e-7)
@@ -1151,15 +1154,18 @@ def test_projections_with_the_norm_folded_in(hip, cpu, hip_ops, cpu_ops, k):
     assert np.all(np.abs(got - want) <= 2 * tol_g)
 
 
-@pytest.mark.parametrize("k,n", [(2048, 96), (5632, 33), (128, 64), (260, 9), (4096, 5)])
+@pytest.mark.parametrize("k,n", [(2048, 96), (5632, 33), (128, 64), (260, 9), (4096, 5), (1000, 7), (8192, 6), (512, 3), (6152, 11), (8200, 4)])
 def test_fused_projections_take_bf16_matrices(hip, hip_ops, k, n):
-    """Matrices stored as bf16 (x, the sums and the result stay f32): a bf16 widens exactly and the
-    sums run in the same order, so every hook gives bit for bit what it gives for f32 matrices
-    holding the same values."""
+    """Matrices stored as bf16 (x, the sums and the result stay f32): a bf16 widens exactly, so every hook gives what it
+    gives for f32 matrices holding the same values -- within the k * eps bound of the float64 product where the bf16 rows
+    go through the kernel with eight consecutive elements per lane (rows of 512 .. 8192 elements, a multiple of 8), bit
+    for bit elsewhere (same kernel, same order of the sums)."""
     print("bf16 matrices", k, n, flush=True)
     eps = 1e-5
+    own_order = k % 8 == 0 and 512 <= k <= 8192
     x, alpha, r = rng.normal(121, k, 2.0), rng.normal(122, k, 0.5), rng.normal(123, n)
     ws = [rng.bf16_round(rng.normal(124 + i, n * k, 0.05)) for i in range(3)]
+    wall = np.concatenate([w.reshape(n, k) for w in ws], 0)
 
     def mats(bf16, idx):
         return [LB.copy(rng.to_bf16_bits(ws[i]) if bf16 else ws[i], (n, k), hip) for i in idx]
@@ -1167,21 +1173,35 @@ def test_fused_projections_take_bf16_matrices(hip, hip_ops, k, n):
     def xs():
         return LB.copy(x, (1, 1, k), hip)
 
+    def same(narrow, wide, truth, tol):
+        assert np.all(np.abs(wide - truth) <= tol), float((np.abs(wide - truth) / tol).max())
+        assert np.all(np.abs(narrow - truth) <= tol), float((np.abs(narrow - truth) / tol).max())
+        if not own_order:
+            assert np.array_equal(narrow, wide)
+
+    x6 = x.astype(np.float64)
     for norm in (False, True):
+        if norm and k > 4096:
+            continue   # the fused norm is built for rows of up to 4096 elements
+        xin = x6 / np.sqrt((x6 * x6).mean() + eps) * alpha if norm else x6
+        truth = wall.astype(np.float64) @ xin
+        tol = (2 if norm else 1) * _gemv_tol(xin.astype(np.float32), wall) + 1e-6 * np.abs(truth)
         extra = (LB.copy(alpha, (k,), hip), eps) if norm else ()
         wide = hip_ops.linear_packed(xs(), mats(False, (0, 1, 2)), *extra).data_vec()
         narrow = hip_ops.linear_packed(xs(), mats(True, (0, 1, 2)), *extra)
         assert narrow.dtype == ug_amd.F32
-        assert np.array_equal(narrow.data_vec(), wide)
+        same(narrow.data_vec(), wide, truth, tol)
         extra = (LB.copy(alpha, (k,), hip), eps) if norm else ()
+        g, u = truth[:n], truth[n:2 * n]
+        sig = 1.0 / (1.0 + np.exp(-g))
+        tol_g = 1.1 * tol[:n] * np.abs(u) + np.abs(g * sig) * tol[n:2 * n] + 4e-7 * np.abs(g * sig * u) + 1e-30
         wide = hip_ops.gate_up(xs(), *mats(False, (0, 1)), *extra).data_vec()
-        assert np.array_equal(hip_ops.gate_up(xs(), *mats(True, (0, 1)), *extra).data_vec(), wide)
+        same(hip_ops.gate_up(xs(), *mats(True, (0, 1)), *extra).data_vec(), wide, g * sig * u, tol_g)
     res = LB.copy(r, (1, 1, n), hip)
+    truth = ws[2].reshape(n, k).astype(np.float64) @ x6 + r
     wide = hip_ops.linear_add(xs(), mats(False, (2,))[0], res).data_vec()
-    assert np.array_equal(hip_ops.linear_add(xs(), mats(True, (2,))[0], LB.copy(r, (1, 1, n), hip)).data_vec(), wide)
-    # and against float64 on the rounded values
-    truth = ws[2].reshape(n, k).astype(np.float64) @ x.astype(np.float64) + r
-    assert np.all(np.abs(wide - truth) <= _gemv_tol(x, ws[2].reshape(n, k)) + 1e-6 * np.abs(truth))
+    same(hip_ops.linear_add(xs(), mats(True, (2,))[0], LB.copy(r, (1, 1, n), hip)).data_vec(), wide, truth,
+         _gemv_tol(x, ws[2].reshape(n, k)) + 1e-6 * np.abs(truth))
 
 
 def test_bf16_matrices_meet_several_rows_through_a_cast(hip, hip_ops):
@@ -1405,8 +1425,8 @@ def test_linear_hook_reads_bf16_matrices_in_place(hip, hip_ops):
 
 
 def test_llama_bf16_matrices_prefill_of_128_tokens(hip, hip_ops):
-    """A 128-token prompt sends every projection of the prefill through the mixed product: ids and margins
-    of the f32 model on the same weights."""
+    """A 128-token prompt sends every projection of the prefill through the mixed product: ids of the f32 model on the
+    same weights, margins to 1e-4."""
     cfg = ug_amd.LlamaConfig(hidden_size=256, intermediate_size=512, max_position_embeddings=256, num_attention_heads=4, num_key_value_heads=2,
                              num_hidden_layers=2, vocab_size=1024)
     prompt = rng.token_ids(11, 128, cfg.vocab_size)
@@ -1414,7 +1434,8 @@ def test_llama_bf16_matrices_prefill_of_128_tokens(hip, hip_ops):
     toks, st = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=0.2, round_bf16=True, fused_attention=3, bf16_matrices=True).generate(prompt, 6)
     print("bf16 prefill 128", toks.tolist(), flush=True)
     assert toks.tolist() == wide[0].tolist()
-    np.testing.assert_array_equal(st["margins"], wide[1]["margins"])
+    # the prompt's products are the f32 model's bit for bit; the decode steps' down projection (rows of 512 elements) sums in the bf16 kernels' own order
+    np.testing.assert_allclose(st["margins"], wide[1]["margins"], rtol=1e-4, atol=1e-6)
 
 
 @pytest.mark.parametrize("n_prompt", [9, 37, 100, 128, 200])
