@@ -883,7 +883,7 @@ std::vector<Cache> Model::new_cache() const {
 }
 
 // model.rs:259-269, 365-373
-LB Model::fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const {
+LB Model::fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache, const std::function<void(const LB&)>* after_layer) const {
   if (cache.size() != layers_.size()) bail("cache/layer count mismatch");
   LB xs = index_select(embedding_, tokens);
   float eps = (float)cfg_.rms_norm_eps;
@@ -894,15 +894,16 @@ LB Model::fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const 
       // the norms travel with the projections behind them, the residual adds with the ones in front
       LB h = attention(l, xs, pos, cache[i], &residual, true);
       xs = mlp(l, h, &h, true);
-      continue;
+    } else {
+      LB h = rms_norm(xs, l.rms1, eps);
+      h = attention(l, h, pos, cache[i], nullptr, false);
+      h = h.binary(BinaryOp::Add, residual);
+      residual = h;
+      LB m = rms_norm(h, l.rms2, eps);
+      m = mlp(l, m, nullptr, false);
+      xs = m.binary(BinaryOp::Add, residual);
     }
-    LB h = rms_norm(xs, l.rms1, eps);
-    h = attention(l, h, pos, cache[i], nullptr, false);
-    h = h.binary(BinaryOp::Add, residual);
-    residual = h;
-    LB m = rms_norm(h, l.rms2, eps);
-    m = mlp(l, m, nullptr, false);
-    xs = m.binary(BinaryOp::Add, residual);
+    if (after_layer) (*after_layer)(xs);
   }
   if (fused_attention_ >= 3) return ops_->linear_packed(xs, {head_}, &ln_f_, eps);
   xs = rms_norm(xs, ln_f_, eps);
@@ -919,6 +920,7 @@ struct PreparedStep {
   LB tokens, logits;
   size_t t = 0, n_items = 0;
   std::unique_ptr<CompiledSchedule> compiled;
+  std::vector<std::unique_ptr<CompiledSchedule>> layers;  // a step launched layer by layer: what ran before `compiled`
   double build_ms = 0, gen_ms = 0, comp_ms = 0;
 };
 
@@ -970,11 +972,20 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
 
   // run_now: every item is launched as soon as it is compiled (the prompt's step: its first kernels execute while the
   // rest of its 300 items are still being looked up)
+  const bool by_layer = getenv("UG_LLAMA_NO_LAYER_STEPS") == nullptr;
   auto build = [&](size_t i, PreparedStep& st, bool run_now) {
     auto t0 = clock::now();
     st.t = i == 0 ? prompt.size() : 1;
     st.tokens = tokens[i];
-    LB logits = model.fwd(st.tokens, pos[i], cache);
+    st.n_items = 0;
+    // run_now: the hidden state behind every layer is realised as soon as its graph exists, so the device starts on
+    // layer 0 after a twentieth of the host work of the step (a prompt of 128 tokens: 0.5 ms of graph and schedule)
+    const std::function<void(const LB&)> realise_layer = [&](const LB& x) {
+      Schedule part = Schedule::create_one(x);
+      st.layers.push_back(std::make_unique<CompiledSchedule>(part.compile_and_run(ccache)));
+      st.n_items += part.items().size();
+    };
+    LB logits = model.fwd(st.tokens, pos[i], cache, run_now && by_layer ? &realise_layer : nullptr);
     st.logits = ops.argmax_into(forced ? picked : tokens[i + 1], logits, st.t - 1, ids, vals, i);
     auto t1 = clock::now();
     Schedule schedule = Schedule::create_one(st.logits);
@@ -985,7 +996,7 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
       st.compiled = std::make_unique<CompiledSchedule>(schedule.compile_with_cache(ccache));
       st.compiled->allocate_all();
     }
-    st.n_items = schedule.items().size();
+    st.n_items += schedule.items().size();
     st.build_ms = ms_between(t0, t1);
     st.gen_ms = ms_between(t1, t2);
     st.comp_ms = ms_between(t2, clock::now());

@@ -2,6 +2,7 @@
 // ops a device has to bring (`trait Device` of ug-llama/src/main.rs:22-28).
 #pragma once
 #include <cstdint>
+#include <functional>
 #include <memory>
 #include <string>
 #include <vector>
@@ -182,7 +183,9 @@ class Model {
   bool bf16_matrices() const { return bf16_matrices_; }
   // Caches of the kind fwd() expects at the current fusion level.
   std::vector<Cache> new_cache() const;
-  LB fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache) const;
+  // after_layer, when given, is called with the hidden state behind every layer: a caller that realises it there
+  // (schedule, compile, launch) has the device working on layer i while the graph of layer i + 1 is still being built.
+  LB fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache, const std::function<void(const LB&)>* after_layer = nullptr) const;
   const Config& config() const { return cfg_; }
   const ug::DevicePtr& device() const { return dev_; }
   const Rope& rope() const { return rope_; }
