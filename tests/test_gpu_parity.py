@@ -1154,7 +1154,7 @@ def test_projections_with_the_norm_folded_in(hip, cpu, hip_ops, cpu_ops, k):
     assert np.all(np.abs(got - want) <= 2 * tol_g)
 
 
-@pytest.mark.parametrize("k,n", [(2048, 96), (5632, 33), (128, 64), (260, 9), (4096, 5), (1000, 7), (8192, 6), (512, 3), (6152, 11), (8200, 4)])
+@pytest.mark.parametrize("k,n", [(2048, 96), (5632, 33), (128, 64), (260, 9), (4096, 5), (1000, 7), (8192, 6), (512, 3), (6152, 11), (8200, 4), (512, 16391)])
 def test_fused_projections_take_bf16_matrices(hip, hip_ops, k, n):
     """Matrices stored as bf16 (x, the sums and the result stay f32): a bf16 widens exactly, so every hook gives what it
     gives for f32 matrices holding the same values -- within the k * eps bound of the float64 product where the bf16 rows
