@@ -290,6 +290,25 @@ extern "C" {
         pos: *const UghipSlice,
         interleaved: c_int,
     ) -> c_int;
+    pub fn ughip_kv_append_pair(
+        dev: *mut UghipDevice,
+        kcache: *mut UghipSlice,
+        vcache: *mut UghipSlice,
+        x: *const UghipSlice,
+        k_offset: usize,
+        v_offset: usize,
+        x_row_stride: usize,
+        b: usize,
+        n: usize,
+        cap: usize,
+        s_old: usize,
+        t: usize,
+        d: usize,
+        cos: *const UghipSlice,
+        sin: *const UghipSlice,
+        pos: *const UghipSlice,
+        interleaved: c_int,
+    ) -> c_int;
     pub fn ughip_attention_cached(
         dev: *mut UghipDevice,
         q: *const UghipSlice,

@@ -318,6 +318,15 @@ int ughip_kv_append(ughip_device* dev, ughip_slice* cache, const ughip_slice* x,
                     size_t d,
                     const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos,
                     int interleaved);
+/* Both appends of a layer in one launch: the k part (rotated when cos/sin/pos are given) and the v part
+ * (copied) of packed rows x [b, t, x_row_stride], at elements k_offset and v_offset of every row, go into
+ * rows s_old .. s_old + t - 1 of kcache and vcache [b, n, cap, d]: ughip_kv_append called twice
+ * (model.rs:226-230 for keys and values), bit for bit.  Offsets and stride are multiples of 4. */
+int ughip_kv_append_pair(ughip_device* dev, ughip_slice* kcache, ughip_slice* vcache,
+                         const ughip_slice* x, size_t k_offset, size_t v_offset, size_t x_row_stride,
+                         size_t b, size_t n, size_t cap, size_t s_old, size_t t, size_t d,
+                         const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos,
+                         int interleaved);
 /* Causal attention of t query positions over such caches, f32, without materialising the
  * [heads, t, s] scores (the chain model.rs:231-245: repeat, q k^T, scale, causal_mask, softmax,
  * x v, transpose, in one launch): q and dst [b, t, n_heads * d] (projection layout), k and v

@@ -1033,6 +1033,84 @@ def test_attention_cached(hip, cpu, hip_ops, cpu_ops, interleaved, b, nh, nkv, t
         assert np.all(np.abs(got - want) <= 2 * tol), float(np.abs(got - want).max())
 
 
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("b,nh,nkv,t,length,cap,d,with_rope", [
+    (1, 8, 2, 37, 0, 64, 64, True),       # a prompt into empty caches
+    (1, 32, 4, 128, 0, 256, 64, True),    # config 5's prompt shape
+    (2, 4, 4, 5, 11, 32, 32, True),       # a second chunk of positions behind cached ones, two sequences
+    (1, 4, 1, 9, 3, 16, 128, False),      # no rotation
+    (1, 6, 2, 4, 2, 8, 48, True),         # a head size without a multi-query kernel: the composition (and its refusal below)
+    (1, 8, 2, 1, 5, 16, 64, True),        # one position: the composition again
+])
+def test_attention_steps_appends_and_attends(hip, hip_ops, interleaved, b, nh, nkv, t, length, cap, d, with_rope):
+    """Ops::attention_steps over packed q|k|v rows: the caches end up as after two kv_append calls (bit for bit) and the
+    result is attention_cached's over them (bit for bit: the same kernels behind one schedule item and one launch fewer)."""
+    print("attention steps", (b, nh, nkv, t, length, cap, d, with_rope, interleaved), flush=True)
+    nq, nk = nh * d, nkv * d
+    row = nq + 2 * nk
+    x = rng.normal(86, b * t * row)
+    k0, v0 = rng.normal(87, b * nkv * cap * d), rng.normal(88, b * nkv * cap * d)
+    scale = float(np.float32(d) ** np.float32(-0.5))
+
+    def fresh():
+        kc, vc = LB.copy(k0, (b, nkv, cap, d), hip), LB.copy(v0, (b, nkv, cap, d), hip)
+        kc.realize()
+        vc.realize()
+        rope = []
+        if with_rope:
+            cos, sin = _rope_tables(hip, d, max_pos=cap + 8)
+            rope = [cos, sin, LB.copy(np.array([length], np.int32), (1, 1), hip), interleaved]
+        return LB.copy(x, (b, t, row), hip), kc, vc, rope
+
+    qkv, kc, vc, rope = fresh()
+    if d == 48:
+        with pytest.raises(ug_amd.UgError):
+            hip_ops.attention_steps(qkv, kc, vc, length, nh, scale, *rope).data_vec()    # the op-by-op chain has no packed rows
+        return
+    got = hip_ops.attention_steps(qkv, kc, vc, length, nh, scale, *rope)
+    assert tuple(got.dims()) == (b, t, nq)
+    got = got.data_vec()
+    got_k, got_v = kc.data_vec(), vc.data_vec()
+    qkv2, kc2, vc2, rope2 = fresh()
+    k_new = hip_ops.kv_append(kc2, length, qkv2, *(rope2 if with_rope else [None, None, None, False]), nq, row)
+    v_new = hip_ops.kv_append(vc2, length, qkv2, None, None, None, False, nq + nk, row)
+    want = hip_ops.attention_cached(qkv2, k_new, v_new, length + t, scale, *(rope2 if with_rope else [None, None, None, False]), 0, row, nh).data_vec()
+    np.testing.assert_array_equal(got_k, kc2.data_vec())
+    np.testing.assert_array_equal(got_v, vc2.data_vec())
+    np.testing.assert_array_equal(got, want)
+    # and the appended rows against float64
+    rows = x.reshape(b, t, row)
+    kr = rows[:, :, nq:nq + nk].reshape(b, t, nkv, d)
+    if with_rope:
+        kr = _rope_rows_f64(kr.astype(np.float64), rope[0].data_vec(), rope[1].data_vec(), length, interleaved)
+    np.testing.assert_allclose(got_k.reshape(b, nkv, cap, d)[:, :, length:length + t], np.asarray(kr).transpose(0, 2, 1, 3), rtol=1e-5, atol=1e-6)
+    np.testing.assert_array_equal(got_v.reshape(b, nkv, cap, d)[:, :, length:length + t], rows[:, :, nq + nk:].reshape(b, t, nkv, d).transpose(0, 2, 1, 3))
+    np.testing.assert_array_equal(got_k.reshape(b, nkv, cap, d)[:, :, length + t:], k0.reshape(b, nkv, cap, d)[:, :, length + t:])
+
+
+def test_kv_append_pair_limits(hip):
+    """Refusals of ughip_kv_append_pair straight through the C ABI."""
+    import ctypes as C
+    lib, dev = ug_amd.ughip_lib(), C.c_void_p(hip.raw_hip())
+    z = C.c_size_t
+    kc, vc = hip.allocate_uninit(ug_amd.F32, 2 * 8 * 16), hip.allocate_uninit(ug_amd.F32, 2 * 8 * 16)
+    x = hip.allocate_uninit(ug_amd.F32, 3 * 96)
+    raw = lambda s_: C.c_void_p(s_.raw())
+
+    def call(k=kc, v=vc, k_off=32, v_off=64, stride=96, cap=8, s_old=0, t=3):
+        return lib.ughip_kv_append_pair(dev, raw(k), raw(v), raw(x), z(k_off), z(v_off), z(stride), z(1), z(2), z(cap), z(s_old), z(t), z(16), None, None, None, 0)
+
+    assert call() == 0, lib.ughip_last_error()
+    assert call(s_old=6) != 0 and b"do not fit a cache" in lib.ughip_last_error()
+    assert call(v_off=80) != 0 and b"do not fit rows" in lib.ughip_last_error()       # the v part would run past the row
+    assert call(k_off=30) != 0 and b"do not fit rows" in lib.ughip_last_error()       # not a multiple of 4
+    assert call(stride=0) != 0
+    assert call(v=kc) != 0 and b"three different slices" in lib.ughip_last_error()
+    assert call(cap=16) != 0                                                          # caches too small for 16 rows
+    assert call(t=4) != 0                                                             # x holds 3 rows
+    assert lib.ughip_synchronize(dev) == 0
+
+
 def test_attention_cached_errors(hip, cpu, hip_ops, cpu_ops):
     def lb(shape, dev=hip):
         return LB.copy(np.zeros(int(np.prod(shape)), np.float32), shape, dev)

@@ -716,6 +716,15 @@ class LlamaOps(_Handle):
         lb._keep += [kcache, vcache] + ([cos, sin, pos] if rope else [])
         return lb
 
+
+    def attention_steps(self, qkv, kcache, vcache, length, n_heads, scale, cos=None, sin=None, pos=None, interleaved=False):
+        """t positions: the k | v parts of the packed rows go into rows length .. length + t - 1 of the caches (which
+        are written), query i attends to rows 0 .. length + i -> [b, t, n_heads * d]."""
+        rope = cos is not None
+        lb = self._op("ugh_llama_attention_steps", qkv, _p(kcache.h), _p(vcache.h), C.c_size_t(length), C.c_size_t(n_heads), C.c_float(scale),
+                      _p(cos.h) if rope else None, _p(sin.h) if rope else None, _p(pos.h) if rope else None, int(interleaved))
+        lb._keep += [kcache, vcache] + ([cos, sin, pos] if rope else [])
+        return lb
     def device_argmax(self):
         return bool(host_lib().ugh_llama_device_argmax(_p(self.h)))
 

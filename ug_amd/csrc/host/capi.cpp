@@ -712,6 +712,13 @@ int ugh_llama_attention_step(void* ops, void* qkv, void* kcache, void* vcache, s
     else *out = box(ops_of(ops).attention_step(lb_of(qkv), lb_of(kcache), lb_of(vcache), len, n_heads, scale, nullptr, nullptr, nullptr, false));
   });
 }
+int ugh_llama_attention_steps(void* ops, void* qkv, void* kcache, void* vcache, size_t len, size_t n_heads, float scale, void* cos, void* sin, void* pos,
+                              int interleaved, void** out) {
+  return guard([&] {
+    if (cos) *out = box(ops_of(ops).attention_steps(lb_of(qkv), lb_of(kcache), lb_of(vcache), len, n_heads, scale, &lb_of(cos), &lb_of(sin), &lb_of(pos), interleaved != 0));
+    else *out = box(ops_of(ops).attention_steps(lb_of(qkv), lb_of(kcache), lb_of(vcache), len, n_heads, scale, nullptr, nullptr, nullptr, false));
+  });
+}
 int ugh_llama_device_argmax(void* ops) { return ops_of(ops).device_argmax() ? 1 : 0; }
 int ugh_llama_argmax_into(void* ops, void* token, void* logits, size_t row, void* ids, void* vals, size_t slot, void** out) {
   return guard([&] { *out = box(ops_of(ops).argmax_into(lb_of(token), lb_of(logits), row, lb_of(ids), lb_of(vals), slot)); });

@@ -396,6 +396,38 @@ struct HipOps : Ops {
     return LB::custom(f, args, Shape({b, 1, nq}), qkv.dtype(), qkv.device());
   }
 
+  LB attention_steps(const LB& qkv, const LB& kcache, const LB& vcache, size_t len, size_t n_heads, float scale, const LB* cos, const LB* sin, const LB* pos,
+                     bool interleaved) const override {
+    if (qkv.rank() != 3 || kcache.rank() != 4 || kcache.dims() != vcache.dims()) bail("attention_steps: expected qkv [b, t, row] and caches [b, nkv, cap, d]");
+    size_t b = qkv.dims()[0], t = qkv.dims()[1], row = qkv.dims()[2], nkv = kcache.dims()[1], cap = kcache.dims()[2], d = kcache.dims()[3];
+    size_t nq = n_heads * d, nk = nkv * d;
+    if (kcache.dims()[0] != b || row != nq + 2 * nk)
+      bail("attention_steps: mismatched shapes " + qkv.shape().str() + " " + kcache.shape().str());
+    if (len + t > cap) bail("attention_steps: " + std::to_string(len + t) + " rows exceed the cache capacity " + std::to_string(cap));
+    // one position has a launch of its own kind, and head sizes without a multi-query kernel take the composition
+    if (t < 2 || !(d == 32 || d == 64 || d == 128) || qkv.dtype() != DType::F32 || getenv("UG_LLAMA_NO_APPEND_PAIR"))
+      return Ops::attention_steps(qkv, kcache, vcache, len, n_heads, scale, cos, sin, pos, interleaved);
+    ughip_device* dev = hip_dev(qkv);
+    const bool with_rope = cos != nullptr;
+    int il = interleaved ? 1 : 0;
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != (with_rope ? 7u : 4u)) bail("attention_steps: unexpected number of slices");
+      ughip_slice *x = hip_raw_slice(*vs[0]), *kc = hip_raw_slice(*vs[1]), *vc = hip_raw_slice(*vs[2]);
+      const ughip_slice* c = with_rope ? hip_raw_slice(*vs[3]) : nullptr;
+      const ughip_slice* sn = with_rope ? hip_raw_slice(*vs[4]) : nullptr;
+      const ughip_slice* p = with_rope ? hip_raw_slice(*vs[5]) : nullptr;
+      hip_check(ughip_kv_append_pair(dev, kc, vc, x, nq, nq + nk, row, b, nkv, cap, len, t, d, c, sn, p, il), "attention_steps");
+      hip_check(ughip_attention_cached(dev, x, 0, row, kc, vc, hip_raw_slice(*vs.back()), b, n_heads, nkv, t, len + t, cap, d, scale, c, sn, p, il), "attention_steps");
+    };
+    std::vector<LB> args = {qkv, kcache, vcache};
+    if (with_rope) {
+      args.push_back(*cos);
+      args.push_back(*sin);
+      args.push_back(*pos);
+    }
+    return LB::custom(f, args, Shape({b, t, nq}), qkv.dtype(), qkv.device());
+  }
+
   bool device_argmax() const override { return true; }
 
   LB argmax_into(const LB& token, const LB& logits, size_t row, const LB& ids, const LB& vals, size_t slot) const override {
@@ -517,6 +549,16 @@ LB Ops::attention_cached(const LB& q, const LB& k, const LB& v, size_t s, float 
 
 LB Ops::attention_step(const LB&, const LB&, const LB&, size_t, size_t, float, const LB*, const LB*, const LB*, bool) const {
   bail("attention_step: needs a device with packed projections and caches written in place");
+}
+
+LB Ops::attention_steps(const LB& qkv, const LB& kcache, const LB& vcache, size_t len, size_t n_heads, float scale, const LB* cos, const LB* sin, const LB* pos,
+                        bool interleaved) const {
+  if (qkv.rank() != 3 || kcache.rank() != 4 || kcache.dims() != vcache.dims()) bail("attention_steps: expected qkv [b, t, row] and caches [b, nkv, cap, d]");
+  const size_t t = qkv.dims()[1], row = qkv.dims()[2], nkv = kcache.dims()[1], d = kcache.dims()[3], nq = n_heads * d, nk = nkv * d;
+  if (row != nq + 2 * nk) bail("attention_steps: rows of " + std::to_string(row) + " elements are not q | k | v of " + std::to_string(n_heads) + " and " + std::to_string(nkv) + " heads");
+  LB kc = kv_append(kcache, len, qkv, cos, sin, pos, interleaved, nq, row);
+  LB vc = kv_append(vcache, len, qkv, nullptr, nullptr, nullptr, false, nq + nk, row);
+  return attention_cached(qkv, kc, vc, len + t, scale, cos, sin, pos, interleaved, 0, row, n_heads);
 }
 
 LB Ops::argmax_into(const LB&, const LB&, size_t, const LB&, const LB&, size_t) const { bail("argmax_into: this device reads the logits back and picks the token on the host"); }
@@ -757,12 +799,10 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
   if (fused_attention_ >= 3 && cache.capacity && l.qkv_stacked.valid()) {
     // several positions: one product gives q | k | v side by side and everything behind it reads its
     // column range of the wide rows in place (a preallocated cache implies a head size the kernels take)
-    const size_t nq = nh * hd, nk = nkv * hd, row = nq + 2 * nk, len = cache.len;
+    const size_t len = cache.len;
     LB qkv = ops_->linear(xs, l.qkv_stacked);
-    LB kc = ops_->kv_append(cache.prev_k, len, qkv, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, nq, row);
-    LB vc = ops_->kv_append(cache.prev_v, len, qkv, nullptr, nullptr, nullptr, false, nq + nk, row);
     cache.len = len + seq_len;
-    return finish(ops_->attention_cached(qkv, kc, vc, cache.len, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, 0, row, nh));
+    return finish(ops_->attention_steps(qkv, cache.prev_k, cache.prev_v, len, nh, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved));
   }
   LB q = ops_->linear(xs, l.q_proj);
   LB k = ops_->linear(xs, l.k_proj);

@@ -88,6 +88,13 @@ struct Ops {
   virtual LB attention_step(const LB& qkv, const LB& kcache, const LB& vcache, size_t len, size_t n_heads, float scale, const LB* cos, const LB* sin,
                             const LB* pos, bool interleaved) const;
 
+  // The same for t positions (a prompt): rows len .. len + t - 1 of both caches receive the k (rotated) and v parts
+  // of the packed rows qkv [b, t, (nh + 2 nkv) d], query i attends to rows 0 .. len + i.  The default composes
+  // kv_append (twice) and attention_cached; a device may fold the two appends into one launch and the three ops
+  // into one schedule item.  The caches are written, as in attention_step.
+  virtual LB attention_steps(const LB& qkv, const LB& kcache, const LB& vcache, size_t len, size_t n_heads, float scale, const LB* cos, const LB* sin,
+                             const LB* pos, bool interleaved) const;
+
   // Greedy step on the device (device_argmax() == true): the index of the largest value of row
   // `row` of logits [b, rows, n] is written into `token` (I32, one element, in place: the result
   // names the same storage) and recorded with the two largest values at ids[slot], vals[2 slot],

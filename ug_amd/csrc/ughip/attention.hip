@@ -352,11 +352,9 @@ __global__ void __launch_bounds__(256) rope_append_kernel(const float* __restric
 // cache [b, n, cap, d], x [b, t, n * d] (rows x_row_stride apart): cache[b, h, s_old + i, :] =
 // x[b, i, h * d .. (h + 1) * d), rotated at table row pos[0] + i when a table is given.  One thread
 // per float4 of x (d % 4 == 0).
-__global__ void __launch_bounds__(256) kv_append_kernel(float* __restrict__ cache, const float* __restrict__ x, size_t x_row_stride, size_t n4, int t, int n,
-                                                        int d, size_t cap, int s_old, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-                                                        const int* __restrict__ pos, size_t table_len, int interleaved) {
-  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (g >= n4) return;
+__device__ __forceinline__ void kv_append_body(size_t g, float* __restrict__ cache, const float* __restrict__ x, size_t x_row_stride, int t, int n, int d,
+                                               size_t cap, int s_old, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                               const int* __restrict__ pos, size_t table_len, int interleaved) {
   const int d4 = d >> 2;
   const int c4 = (int)(g % d4);
   size_t rest = g / d4;
@@ -387,6 +385,25 @@ __global__ void __launch_bounds__(256) kv_append_kernel(float* __restrict__ cach
     out = make_float4(o[0], o[1], o[2], o[3]);
   }
   reinterpret_cast<float4*>(cache + ((b * n + h) * cap + (size_t)s_old + i) * d)[c4] = out;
+}
+
+__global__ void __launch_bounds__(256) kv_append_kernel(float* __restrict__ cache, const float* __restrict__ x, size_t x_row_stride, size_t n4, int t, int n,
+                                                        int d, size_t cap, int s_old, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                        const int* __restrict__ pos, size_t table_len, int interleaved) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n4) return;
+  kv_append_body(g, cache, x, x_row_stride, t, n, d, cap, s_old, cos_t, sin_t, pos, table_len, interleaved);
+}
+
+// Keys (blockIdx.y == 0, rotated when a table is given) and values (blockIdx.y == 1, copied) of the same new positions in one launch.
+__global__ void __launch_bounds__(256) kv_append_pair_kernel(float* __restrict__ kcache, float* __restrict__ vcache, const float* __restrict__ xk,
+                                                             const float* __restrict__ xv, size_t x_row_stride, size_t n4, int t, int n, int d, size_t cap,
+                                                             int s_old, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                             const int* __restrict__ pos, size_t table_len, int interleaved) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n4) return;
+  if (blockIdx.y == 0) kv_append_body(g, kcache, xk, x_row_stride, t, n, d, cap, s_old, cos_t, sin_t, pos, table_len, interleaved);
+  else kv_append_body(g, vcache, xv, x_row_stride, t, n, d, cap, s_old, nullptr, nullptr, nullptr, 0, 0);
 }
 
 // ---- causal attention over a cache, many query positions ------------------------------------------
@@ -872,6 +889,37 @@ int ughip_kv_append(ughip_device* dev, ughip_slice* cache, const ughip_slice* x,
       static_cast<float*>(cache->ptr), static_cast<const float*>(x->ptr) + x_offset, x_row_stride, n4, (int)t, (int)n, (int)d, cap, (int)s_old,
       rope ? static_cast<const float*>(cos->ptr) : nullptr, rope ? static_cast<const float*>(sin->ptr) : nullptr,
       rope ? static_cast<const int*>(pos->ptr) : nullptr, rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved);
+  UGHIP_HIPCHK(hipGetLastError());
+  return UGHIP_OK;
+}
+
+int ughip_kv_append_pair(ughip_device* dev, ughip_slice* kcache, ughip_slice* vcache, const ughip_slice* x, size_t k_offset, size_t v_offset,
+                         size_t x_row_stride, size_t b, size_t n, size_t cap, size_t s_old, size_t t, size_t d, const ughip_slice* cos, const ughip_slice* sin,
+                         const ughip_slice* pos, int interleaved) {
+  if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
+  if (d == 0 || d % 4 != 0) return set_error(UGHIP_ERR_INVALID, "kv_append_pair: head size %zu is not a multiple of 4", d);
+  const bool rope = cos || sin || pos;
+  if (rope) {
+    if (d % 2 != 0) return set_error(UGHIP_ERR_INVALID, "kv_append_pair: odd head size %zu", d);
+    if (int rc = check_rope_table(cos, sin, pos, d, "kv_append_pair")) return rc;
+  }
+  if (s_old + t > cap) return set_error(UGHIP_ERR_BOUNDS, "kv_append_pair: rows %zu..%zu do not fit a cache of %zu rows", s_old, s_old + t, cap);
+  if (int rc = check_f32(kcache, b * n * cap * d, "kv_append_pair key cache")) return rc;
+  if (int rc = check_f32(vcache, b * n * cap * d, "kv_append_pair value cache")) return rc;
+  if (x_row_stride == 0 || x_row_stride < n * d || (k_offset | v_offset | x_row_stride) % 4 != 0 || k_offset + n * d > x_row_stride || v_offset + n * d > x_row_stride)
+    return set_error(UGHIP_ERR_INVALID, "kv_append_pair: offsets %zu, %zu / row stride %zu do not fit rows of %zu", k_offset, v_offset, x_row_stride, n * d);
+  if (int rc = check_f32(x, b * t * x_row_stride, "kv_append_pair x")) return rc;
+  if (kcache == x || vcache == x || kcache == vcache) return set_error(UGHIP_ERR_INVALID, "kv_append_pair: the caches and x must be three different slices");
+  const size_t n4 = b * t * n * d / 4;
+  if (n4 == 0) return UGHIP_OK;
+  if (cap > 0x7fffffffull || t > 0x7fffffffull || n > 0x7fffffffull || d > 0x7fffffffull || n4 > (size_t)0x7fffffff * 256)
+    return set_error(UGHIP_ERR_INVALID, "kv_append_pair: shape too large");
+  if (int rc = device_activate(dev)) return rc;
+  kv_append_pair_kernel<<<dim3((unsigned)((n4 + 255) / 256), 2), 256, 0, dev->stream>>>(
+      static_cast<float*>(kcache->ptr), static_cast<float*>(vcache->ptr), static_cast<const float*>(x->ptr) + k_offset, static_cast<const float*>(x->ptr) + v_offset,
+      x_row_stride, n4, (int)t, (int)n, (int)d, cap, (int)s_old, rope ? static_cast<const float*>(cos->ptr) : nullptr,
+      rope ? static_cast<const float*>(sin->ptr) : nullptr, rope ? static_cast<const int*>(pos->ptr) : nullptr,
+      rope ? (cos->len < sin->len ? cos->len : sin->len) : 0, interleaved);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
 }
