@@ -1282,6 +1282,46 @@ def test_fused_projections_take_bf16_matrices(hip, hip_ops, k, n):
          _gemv_tol(x, ws[2].reshape(n, k)) + 1e-6 * np.abs(truth))
 
 
+def test_fused_projections_bf16_random_shapes(hip, hip_ops):
+    """Seeded random row lengths (multiples of 8 from 512 to 8192, so every count of 2048-element chunks and ragged last
+    chunks), matrix counts and row counts that do not divide the rows a workgroup walks: all three hooks over bf16
+    matrices against float64."""
+    gen = np.random.default_rng(20240611)
+    eps = 1e-5
+    for case in range(24):
+        k = int(gen.integers(64, 1025)) * 8
+        ns = [int(gen.integers(1, 70)) for _ in range(int(gen.integers(1, 4)))]
+        norm = bool(gen.integers(0, 2)) and k <= 4096
+        print("bf16 random", case, k, ns, norm, flush=True)
+        x, alpha = rng.normal(300 + case, k, 2.0), rng.normal(400 + case, k, 0.5)
+        ws = [rng.bf16_round(rng.normal(500 + 3 * case + i, n * k, 0.05)).reshape(n, k) for i, n in enumerate(ns)]
+        x6 = x.astype(np.float64)
+        xin = x6 / np.sqrt((x6 * x6).mean() + eps) * alpha if norm else x6
+        wall = np.concatenate(ws, 0)
+        truth = wall.astype(np.float64) @ xin
+        tol = (2 if norm else 1) * _gemv_tol(xin.astype(np.float32), wall) + 1e-6 * np.abs(truth)
+        extra = (LB.copy(alpha, (k,), hip), eps) if norm else ()
+        mats = [LB.copy(rng.to_bf16_bits(w.ravel()), w.shape, hip) for w in ws]
+        got = hip_ops.linear_packed(LB.copy(x, (1, 1, k), hip), mats, *extra).data_vec()
+        assert got.shape == (sum(ns),)
+        assert np.all(np.abs(got - truth) <= tol), (case, float((np.abs(got - truth) / tol).max()))
+        # gate / up of the first matrix against itself shifted by one row (two matrices of the same shape)
+        n = ns[0]
+        up = np.roll(ws[0], 1, axis=0)
+        g, u = ws[0].astype(np.float64) @ xin, up.astype(np.float64) @ xin
+        tg = (2 if norm else 1) * _gemv_tol(xin.astype(np.float32), ws[0]) + 1e-6 * np.abs(g)
+        tu = (2 if norm else 1) * _gemv_tol(xin.astype(np.float32), up) + 1e-6 * np.abs(u)
+        sig = 1.0 / (1.0 + np.exp(-g))
+        tol_g = 1.1 * tg * np.abs(u) + np.abs(g * sig) * tu + 4e-7 * np.abs(g * sig * u) + 1e-30
+        extra = (LB.copy(alpha, (k,), hip), eps) if norm else ()
+        got = hip_ops.gate_up(LB.copy(x, (1, 1, k), hip), mats[0], LB.copy(rng.to_bf16_bits(up.ravel()), up.shape, hip), *extra).data_vec()
+        assert np.all(np.abs(got - g * sig * u) <= tol_g), (case, float((np.abs(got - g * sig * u) / tol_g).max()))
+        r = rng.normal(600 + case, n)
+        t_add = ws[0].astype(np.float64) @ x6 + r
+        got = hip_ops.linear_add(LB.copy(x, (1, 1, k), hip), mats[0], LB.copy(r, (1, 1, n), hip)).data_vec()
+        assert np.all(np.abs(got - t_add) <= _gemv_tol(x, ws[0]) + 1e-6 * np.abs(t_add)), case
+
+
 def test_bf16_matrices_meet_several_rows_through_a_cast(hip, hip_ops):
     """Prefill shapes: a bf16 matrix is widened in front of matmul (one dtype per product,
     ug-core/src/lib.rs:62-70) and the result is that of the f32 matrix with the same values."""
