@@ -366,7 +366,12 @@ def test_matmul_16bit_one_wave_per_simd_tiles(hip, bmnk, bn, rhs_nk, dtype):
     dt = ug_amd.BF16 if dtype == "bf16" else ug_amd.F16
     a = rnd(rng.uniform_pm1(25, b * m * k)).reshape(b, m, k)
     w = rnd(rng.uniform_pm1(26, b * k * n)).reshape(b, k, n)
-    got = _raw_matmul(hip, dt, a, w, rhs_nk)
+    import os
+    os.environ["UGHIP_GEMM_SHAPE"] = "3" if bn == 256 else "4"   # K this short is a toss-up between the kernels: the choice is tested below
+    try:
+        got = _raw_matmul(hip, dt, a, w, rhs_nk)
+    finally:
+        del os.environ["UGHIP_GEMM_SHAPE"]
     assert ug_amd.last_kernel() == f"gemm_dma4<{dtype},{'NT' if rhs_nk else 'NN'},256x{bn},256t>"
     exact = np.matmul(a.astype(np.float64), w.astype(np.float64))
     half_ulp = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
@@ -386,6 +391,27 @@ def test_matmul_16bit_one_wave_per_simd_tiles(hip, bmnk, bn, rhs_nk, dtype):
     want = np.matmul(ai.astype(np.float64), wi.astype(np.float64)).astype(np.float32)
     want = rng.bf16_round(want.ravel()).reshape(want.shape) if dtype == "bf16" else want.astype(np.float16).astype(np.float32)
     np.testing.assert_array_equal(_raw_matmul(hip, dt, ai, wi, rhs_nk), want)
+
+
+@pytest.mark.parametrize("bmnk,want", [
+    ((1, 4096, 4096, 1024), "gemm_dma4<bf16,NT,256x256,256t>"),      # 256 tiles of 256 x 256
+    ((8, 1024, 1024, 1024), "gemm_dma4<bf16,NT,256x128,256t>"),      # 128 such tiles: the narrower one fills the chip
+    ((1, 3072, 4096, 1024), "gemm_dma4<bf16,NT,256x256,256t>"),      # 192 tiles: three quarters of the chip at a higher clock
+    ((1, 2048, 2560, 2048), "gemm_dma4<bf16,NT,256x128,256t>"),      # 160 narrow tiles
+    ((1, 2048, 2048, 5632), "gemm_tiled<bf16,NT,128x128,256t>"),     # 128 narrow tiles and a long K: the register-staged kernel
+    ((1, 1024, 1024, 1024), "gemm_tiled<"),                          # a handful of tiles: K split
+])
+def test_matmul_16bit_kernel_choice(hip, bmnk, want):
+    """Which kernel a 16-bit product goes to (both are priced, the cheaper one runs), and that it is right there."""
+    b, m, n, k = bmnk
+    a = rng.bf16_round(rng.uniform_pm1(31, b * m * k)).reshape(b, m, k)
+    w = rng.bf16_round(rng.uniform_pm1(32, b * k * n)).reshape(b, k, n)
+    got = _raw_matmul(hip, ug_amd.BF16, a, w, True)
+    assert ug_amd.last_kernel().startswith(want), ug_amd.last_kernel()
+    rows = np.array([0, 1, m // 2 + 3, m - 1])
+    exact = np.matmul(a[:, rows].astype(np.float64), w.astype(np.float64))
+    bound = 2.0 ** -8 * np.abs(exact) + k * np.finfo(np.float32).eps * np.matmul(np.abs(a[:, rows]).astype(np.float64), np.abs(w).astype(np.float64))
+    assert np.all(np.abs(got[:, rows] - exact) <= bound * 1.001 + 1e-7)
 
 
 def test_matmul_16bit_one_wave_per_simd_forced_and_limits(hip, monkeypatch):

@@ -39,6 +39,9 @@ struct GemmEpilogue {
 size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch, const GemmEpilogue* epi = nullptr);
 hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, float* workspace, bool rhs_bf16 = false,
                              const GemmEpilogue* epi = nullptr);
+// What the launch above is expected to take (us), from the same per-tile figures that choose its tile and K split; a
+// negative value when the kernel does not take the problem.  Used to decide between this kernel and gemm_dma4.
+double gemm_tiled_cost_us(int dtype, const MMArgs& p, size_t batch);
 
 // 16-bit types, one wave per SIMD: 256 x bn tiles (bn = 256 or 128), 4 waves of 128 x bn/2 with the accumulators in the
 // accumulation registers, loads that write LDS directly, rhs [n, k]- or [k, n]-major (gemm_dma.hip).  M % 256 == 0,

@@ -288,10 +288,30 @@ bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int bn) {
   return batch * (size_t)(p.M / BM) * (size_t)(p.N / bn) < (1u << 24);
 }
 
-// Which tile this kernel should take the problem with: 256 when 256 x 256 tiles fill the chip, 128 when only 256 x 128
-// tiles do (8 x 1024^3: 128 against 256 tiles), 0 when another kernel is the better choice (few tiles: the K-splitting
-// register-staged kernel; a last round of workgroups that would leave most CUs idle).
+// Which tile this kernel should take the problem with (256 or 128), or 0 when the register-staged kernel is expected to
+// be faster.  Both are priced.  This kernel: a fixed cost (launch and first tile, 4 us, and the result's way out at the
+// rate of a stream) plus, per round of up to 256 workgroups, the K tiles at a time that grows with the share of the chip
+// that is busy -- the chip is power-bound under this kernel, a half-empty round runs at a higher clock: 0.9 + 0.6 x busy
+// us per K tile for 256 x 256, 0.62 + 0.2 x busy for 256 x 128, fitted to 4096^3 (108 us), 8 x 1024^3 (20), 3072 x 4096^2
+// (92 / 112), 5120^2 x 1024 (54 / 65), 2048 x 2560 x 2048 (40 / 29), 2816^3 (58 / 44), 1280 x 8192 x 2048 (46), 2048^2 x 5632
+// (97 / 72).  The other kernel: the model that chooses its own tiles.  Against "256 x 256 tiles when they number 200 or
+// more, else 256 x 128 under the same rule" this moves products with 130-250 tiles or a short last round to this kernel
+// (3072 x 4096^2: 131 -> 91 us, 5120^2 x 1024: 77 -> 54, 1280 x 8192 x 2048: 64 -> 47, 2048 x 2560 x 2048: 35 -> 29,
+// 2304^3: 39 -> 35) and leaves those with about 128 tiles where they were (2048^2 x 5632: 56 us against 72).
 // UGHIP_GEMM_SHAPE=3 / 4 forces 256 / 128 where the kernel applies, 0..2 keeps it out (tuning aid).
+double gemm_dma_cost_us(const MMArgs& p, size_t batch, int bn) {
+  const size_t tiles = batch * (size_t)(p.M / BM) * (size_t)(p.N / bn);
+  const int kt = p.K / BK;
+  const bool nn = p.b_cs == 1 && p.b_rs != 1;
+  const double t0 = bn == 256 ? 0.9 : 0.62, t1 = bn == 256 ? 0.6 : 0.2;
+  double us = 4.0 + (double)batch * p.M * p.N * 2 / 6.4e6;
+  for (size_t left = tiles; left > 0; left -= left < 256 ? left : 256) {
+    const double busy = (left < 256 ? (double)left : 256.0) / 256.0;
+    us += kt * (t0 + t1 * busy) * (nn ? 1.08 : 1.0);
+  }
+  return us;
+}
+
 int gemm_dma_pick(int dtype, const MMArgs& p, size_t batch) {
   if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
     const int s = atoi(e);
@@ -299,12 +319,16 @@ int gemm_dma_pick(int dtype, const MMArgs& p, size_t batch) {
     if (s == 4) return gemm_dma_supported(dtype, p, batch, 128) ? 128 : 0;
     return 0;
   }
+  int best = 0;
+  double best_us = 0;
   for (int bn : {256, 128}) {
     if (!gemm_dma_supported(dtype, p, batch, bn)) continue;
-    const size_t tiles = batch * (size_t)(p.M / BM) * (size_t)(p.N / bn), rounds = (tiles + 255) / 256;
-    if (tiles >= 200 && tiles * 5 >= rounds * 256 * 4) return bn;  // the last round at least 80 % of the average
+    const double us = gemm_dma_cost_us(p, batch, bn);
+    if (!best || us < best_us * 0.92) best = bn, best_us = us;  // the wider tile on a near tie: fewer operand bytes
   }
-  return 0;
+  if (!best) return 0;
+  const double other = gemm_tiled_cost_us(dtype, p, batch);
+  return other < 0 || best_us < other ? best : 0;
 }
 
 hipError_t gemm_dma_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, int bn) {
