@@ -429,8 +429,35 @@ def test_matmul_16bit_one_wave_per_simd_forced_and_limits(hip, monkeypatch):
             np.testing.assert_array_equal(got, plain)
         _raw_matmul(hip, ug_amd.BF16, a[:, :, :192], w[:, :192], True)      # 3 K tiles
         assert ug_amd.last_kernel().startswith("gemm_tiled<")
-        _raw_matmul(hip, ug_amd.BF16, a[:, :384], w, True)                    # 384 rows
+        _raw_matmul(hip, ug_amd.BF16, a, w[:, :, :252], True)                 # 252 columns: rows of the result are not whole 16-byte chunks
         assert ug_amd.last_kernel().startswith("gemm_tiled<")
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("rhs_nk", [True, False], ids=["NT", "NN"])
+@pytest.mark.parametrize("bmnk", [(1, 300, 264, 256), (2, 257, 136, 320), (1, 1900, 520, 256), (3, 9, 8, 256), (1, 511, 248, 448), (1, 700, 392, 576)])
+def test_matmul_16bit_one_wave_per_simd_ragged(hip, monkeypatch, bmnk, rhs_nk, dtype):
+    """Rows and columns the 256-wide tiles do not divide (any M, N a multiple of 8): the last tiles hang over the end,
+    read the last row again and store only what exists.  Both tile widths, forced; float64 bound, no write past the end
+    (the guard region of _raw_matmul), and bit for bit the register-staged kernel where that takes the shape."""
+    b, m, n, k = bmnk
+    print("matmul one-wave-per-SIMD ragged", dtype, bmnk, "NT" if rhs_nk else "NN", flush=True)
+    rnd = rng.bf16_round if dtype == "bf16" else (lambda v: v.astype(np.float16).astype(np.float32))
+    dt = ug_amd.BF16 if dtype == "bf16" else ug_amd.F16
+    a = rnd(rng.uniform_pm1(33, b * m * k)).reshape(b, m, k)
+    w = rnd(rng.uniform_pm1(34, b * k * n)).reshape(b, k, n)
+    exact = np.matmul(a.astype(np.float64), w.astype(np.float64))
+    half_ulp = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
+    bound = half_ulp * np.abs(exact) + k * np.finfo(np.float32).eps * np.matmul(np.abs(a).astype(np.float64), np.abs(w).astype(np.float64))
+    monkeypatch.setenv("UGHIP_GEMM_SHAPE", "1")
+    other = _raw_matmul(hip, dt, a, w, rhs_nk) if rhs_nk or n % 128 == 0 else None   # the 128-row tiles take any N only with an [n, k]-major rhs
+    for shape, bn in (("3", 256), ("4", 128)):
+        monkeypatch.setenv("UGHIP_GEMM_SHAPE", shape)
+        got = _raw_matmul(hip, dt, a, w, rhs_nk)
+        assert ug_amd.last_kernel() == f"gemm_dma4<{dtype},{'NT' if rhs_nk else 'NN'},256x{bn},256t>"
+        assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-7)
+        if other is not None:
+            np.testing.assert_array_equal(got, other)
 
 
 @pytest.mark.parametrize("bmnk", [(1, 128, 2048, 2048), (1, 128, 256, 2048), (1, 256, 5632, 2048), (1, 128, 2048, 5632), (2, 512, 384, 96), (1, 1024, 1024, 32),

@@ -44,8 +44,8 @@ hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, siz
 double gemm_tiled_cost_us(int dtype, const MMArgs& p, size_t batch);
 
 // 16-bit types, one wave per SIMD: 256 x bn tiles (bn = 256 or 128), 4 waves of 128 x bn/2 with the accumulators in the
-// accumulation registers, loads that write LDS directly, rhs [n, k]- or [k, n]-major (gemm_dma.hip).  M % 256 == 0,
-// N % bn == 0, K % 64 == 0 and K >= 256, 16-byte aligned rows, contiguous [batch, M, N] result.
+// accumulation registers, loads that write LDS directly, rhs [n, k]- or [k, n]-major (gemm_dma.hip).  Any M, N % 8 == 0,
+// K % 64 == 0 and K >= 256, 16-byte aligned rows, contiguous [batch, M, N] result.
 bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int bn);
 hipError_t gemm_dma_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, int bn);
 // The tile width (256 or 128) this kernel should take the problem with, 0 when another kernel should.

@@ -1,6 +1,7 @@
 // 16-bit MFMA GEMM for gfx950 with one wave per SIMD: C[b] = A[b] x B[b], f32 accumulate, bf16 or f16.
 //
-//   block tile 256 x BN (BN = 256 or 128), K tile 64, 4 waves laid out 2 x 2, each owning 128 x BN/2 of the result:
+//   block tile 256 x BN (BN = 256 or 128), K tile 64, 4 waves laid out 2 x 2, each owning 128 x BN/2 of the result
+//   (any M, N a multiple of 8: a last tile hangs over the end, reads the last row again and stores what exists):
 //   16 (8) accumulators of 32 x 32 live in the 256 accumulation registers a lone wave per SIMD can have, which leaves
 //   the architectural registers to two sets of operand fragments -- 8 (6) fragment reads feed 16 (8) MFMAs
 //   global -> LDS with global_load_lds_dwordx4 (no staging registers), two 64 KiB stages; the loads of tile t+2 are
@@ -108,24 +109,27 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
 
   // per-lane byte offsets of this wave's DMA instructions (the same for every K tile; the scalar base moves)
   unsigned voff[ND];
+  // a last tile may hang over the end of M or N: rows past the end fetch the last row again (their results are not
+  // stored), so every address stays inside the operands
+  const int m_last = p.M - 1 - m0, n_left = p.N - n0;
 #pragma unroll
   for (int i = 0; i < NDA; ++i) {
     const int row = (i * 4 + wave) * 8 + (lane >> 3), cp = lane & 7;
-    voff[i] = (unsigned)(row * lda * 2 + ((cp ^ ((row >> 1) & 7)) << 4));
+    voff[i] = (unsigned)(min(row, m_last) * lda * 2 + ((cp ^ ((row >> 1) & 7)) << 4));
   }
 #pragma unroll
   for (int i = 0; i < NDB; ++i) {
     const int g = i * 4 + wave;
     if (!B_KN) {
       const int row = g * 8 + (lane >> 3), cp = lane & 7;
-      voff[NDA + i] = (unsigned)(row * ldb * 2 + ((cp ^ ((row >> 1) & 7)) << 4));
+      voff[NDA + i] = (unsigned)(min(row, n_left - 1) * ldb * 2 + ((cp ^ ((row >> 1) & 7)) << 4));
     } else {
       // one instruction fills 1 KB = 512 / BN rows of k; the lane at LDS position (k, 16-byte chunk c') fetches the
       // chunk whose 64-byte segment the swizzle maps there
       constexpr int CPR = BN / 8;  // 16-byte chunks per row
       const int k = g * (64 / CPR) + lane / CPR, cpos = lane % CPR;
       const int seg = (cpos >> 2) ^ (k & (BN / 32 - 1));
-      voff[NDA + i] = (unsigned)(k * ldb * 2 + (((seg << 2) | (cpos & 3)) << 4));
+      voff[NDA + i] = (unsigned)(k * ldb * 2 + (min((seg << 2) | (cpos & 3), n_left / 8 - 1) << 4));  // N % 8 == 0: whole 16-byte chunks
     }
   }
   const long long a_step = BK * 2, b_step = B_KN ? (long long)BK * ldb * 2 : BK * 2;
@@ -246,7 +250,7 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
     const int row = pass * RPP + r0;
     const u32x2 lo = *(const u32x2 __attribute__((address_space(3)))*)(Cs + row * PITCH + c * 16);
     const u32x2 hi = *(const u32x2 __attribute__((address_space(3)))*)(Cs + row * PITCH + c * 16 + 8);
-    *reinterpret_cast<u32x4*>(C + (size_t)row * p.N + c * 8) = u32x4{lo.x, lo.y, hi.x, hi.y};
+    if (row <= m_last && c * 8 < n_left) *reinterpret_cast<u32x4*>(C + (size_t)row * p.N + c * 8) = u32x4{lo.x, lo.y, hi.x, hi.y};
   }
 }
 
@@ -263,7 +267,7 @@ hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch) {
     if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES)) return e;
     configured.fetch_or(bit, std::memory_order_relaxed);
   }
-  const int tiles_m = p.M / BM, tiles_n = p.N / BN;
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const size_t total = batch * (size_t)tiles_m * tiles_n;
   kernel<<<dim3((unsigned)total), dim3(256), LDS_BYTES, stream>>>(p, tiles_m, tiles_n);
   return hipGetLastError();
@@ -276,7 +280,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int bn) {
   if (dtype != UGHIP_BF16 && dtype != UGHIP_F16) return false;
   if (bn != 256 && bn != 128) return false;
-  if (p.M <= 0 || p.N <= 0 || p.M % BM || p.N % bn || p.K % BK || p.K < 4 * BK || batch == 0) return false;
+  if (p.M <= 0 || p.N <= 0 || p.N % 8 || p.K % BK || p.K < 4 * BK || batch == 0) return false;
   if (p.a_cs != 1 || p.a_rs % 8 || (batch > 1 && (p.a_bs % 8 || p.b_bs % 8 || p.c_bs % 8))) return false;
   const bool nn = p.b_cs == 1 && p.b_rs != 1, nt = p.b_rs == 1 && p.b_cs != 1;
   if (nn == nt) return false;
@@ -285,7 +289,7 @@ bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int bn) {
   // per-lane offsets are 32-bit: the furthest row of a tile has to stay below 4 GiB from the tile's first byte
   if ((unsigned long long)p.a_rs * 2 * BM >= (1ull << 32) || (unsigned long long)ldb * 2 * (nn ? BK : bn) >= (1ull << 32)) return false;
   if (!aligned16(p.a) || !aligned16(p.b) || !aligned16(p.c)) return false;
-  return batch * (size_t)(p.M / BM) * (size_t)(p.N / bn) < (1u << 24);
+  return batch * (size_t)((p.M + BM - 1) / BM) * (size_t)((p.N + bn - 1) / bn) < (1u << 24);
 }
 
 // Which tile this kernel should take the problem with (256 or 128), or 0 when the register-staged kernel is expected to
@@ -300,7 +304,7 @@ bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int bn) {
 // 2304^3: 39 -> 35) and leaves those with about 128 tiles where they were (2048^2 x 5632: 56 us against 72).
 // UGHIP_GEMM_SHAPE=3 / 4 forces 256 / 128 where the kernel applies, 0..2 keeps it out (tuning aid).
 double gemm_dma_cost_us(const MMArgs& p, size_t batch, int bn) {
-  const size_t tiles = batch * (size_t)(p.M / BM) * (size_t)(p.N / bn);
+  const size_t tiles = batch * (size_t)((p.M + BM - 1) / BM) * (size_t)((p.N + bn - 1) / bn);
   const int kt = p.K / BK;
   const bool nn = p.b_cs == 1 && p.b_rs != 1;
   const double t0 = bn == 256 ? 0.9 : 0.62, t1 = bn == 256 ? 0.6 : 0.2;

@@ -592,10 +592,11 @@ double gemm_tiled_cost_us(int dtype, const MMArgs& p, size_t batch) {
   const size_t tiles = tile_count(p, batch, s);
   const double launch_us = 4.0;
   if (tiles < 256) return launch_us + pick_split(dtype, p, batch, s).cost_us;
-  // many tiles: the last, partly filled round of workgroups takes about as long as its share of a full one (measured
-  // on 16-bit products of 2048..5120 rows: within 15 %)
+  // many tiles: a last, partly filled round of workgroups costs a third of a full one plus its share of the rest
+  // (16-bit products of 1900..5120 rows with 300, 320, 324, 384, 484 and 800 tiles: within 10 %)
   const double whole = pick_split(dtype, p, batch, s).cost_us / (double)((tiles + 255) / 256);
-  return launch_us + whole * (double)tiles / 256.0;
+  const size_t part = tiles % 256;
+  return launch_us + whole * ((double)(tiles / 256) + (part ? 0.35 + 0.65 * (double)part / 256.0 : 0.0));
 }
 
 size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch, const GemmEpilogue* epi) {
