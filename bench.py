@@ -456,6 +456,20 @@ def bmm(dev, steps, warmup):
         _, ms = timed(dev, run, steps, warmup)
         tf = 2.0 * m * m * m * steps / (ms * 1e-3) / 1e12
         out[key] = {"TFLOP/s": round(tf, 2), "frac_mfma_bf16": round(tf / MFMA_BF16_PEAK_TF, 4), "us": round(ms * 1e3 / steps, 1), "kernel": kernel, "verified": chk}
+    # rows the 256-row tiles do not divide (a prompt of 3000 tokens against a 4096 x 4096 matrix): the same kernel, its last tiles hang over the end
+    mr, nr = 3000, 4096
+    a, w = rng.uniform_pm1(4, mr * nr), rng.uniform_pm1(5, nr * nr)
+    ab, wb = rng.bf16_round(a).reshape(1, mr, nr), rng.bf16_round(w).reshape(1, nr, nr)
+    sa, sw = dev.slice_from(rng.to_bf16_bits(a)), dev.slice_from(rng.to_bf16_bits(w))
+    dst = dev.allocate_uninit(ug_amd.BF16, mr * nr)
+    run = lambda: dev.matmul(dst, sa, sw, (1, mr, nr, nr), ((1, mr, nr), (mr * nr, nr, 1), 0), ((1, nr, nr), (nr * nr, 1, nr), 0))  # noqa: E731
+    run()
+    chk = check_product_rows("mm_bf16_nt_3000x4096x4096", rng.from_bf16_bits(dst.to_vec()).reshape(1, mr, nr), ab, np.swapaxes(wb, 1, 2), nr, True, rows=(0, 255, 256, 2815, 2816, 2999))
+    kernel = ug_amd.last_kernel()
+    _, ms = timed(dev, run, steps, warmup)
+    tf = 2.0 * mr * nr * nr * steps / (ms * 1e-3) / 1e12
+    out["mm_bf16_nt_3000x4096x4096"] = {"TFLOP/s": round(tf, 2), "frac_mfma_bf16": round(tf / MFMA_BF16_PEAK_TF, 4), "us": round(ms * 1e3 / steps, 1), "kernel": kernel, "verified": chk}
+    del sa, sw, dst
     # the same kernel where the fixed cost (launch, first tile, the result's way out: ~9 us) is 1 % of the run
     m = 8192
     a, w = rng.uniform_pm1(4, m * m), rng.uniform_pm1(5, m * m)
