@@ -547,24 +547,29 @@ Split pick_split(int dtype, const MMArgs& p, size_t batch, int shape, bool alway
   return best;
 }
 
-// The largest tile that fits the problem and still gives every CU a workgroup; with fewer tiles than that, whichever
-// of 128x128 and 128x64 the cost model above makes cheaper (128x64 on a tie: more workgroups).  -1: no tile fits M x N.
+// The tile the cost model above makes cheapest among those that fit the problem.  Within 3 % of each other the smaller
+// tile wins when both leave CUs idle unsplit (fewer than 256 tiles: more workgroups to spread), the larger one otherwise
+// (fewer operand bytes per flop).  Counting rounds of 256 workgroups, not just "at least 256 tiles", is what sends
+// 3072 x 4096 x 4096 f32 to 128 x 128 (768 tiles, three full rounds: 889 us) instead of 256 x 128 (384 tiles, a round and
+// a half: 1000 us) and 2304^3 away from 324 tiles of 128 x 128 (303 -> 255 us).  -1: no tile fits M x N.
 int pick_shape(const MMArgs& p, size_t batch, int dtype, bool always_fold = false) {
   // UGHIP_GEMM_SHAPE=0..2 forces a tile shape (tuning aid); ignored when it does not fit the problem.
   if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
     const int s = atoi(e);
     if (s >= 0 && s < 3 && shape_fits(p, s)) return s;
   }
-  if (shape_fits(p, 0) && tile_count(p, batch, 0) >= 256) return 0;
-  if (shape_fits(p, 1) && tile_count(p, batch, 1) >= 256) return 1;
   int best = -1;
   double best_cost = 0;
-  for (int s = 2; s >= 1; --s) {
+  for (int s = 0; s < 3; ++s) {
     if (!shape_fits(p, s)) continue;
     const double cost = pick_split(dtype, p, batch, s, always_fold).cost_us;
-    if (best < 0 || cost < best_cost * 0.97) best = s, best_cost = cost;
+    if (best < 0) {
+      best = s, best_cost = cost;
+      continue;
+    }
+    const bool few = tile_count(p, batch, best) < 256 && tile_count(p, batch, s) < 256;
+    if (few ? cost <= best_cost * 1.03 : cost < best_cost * 0.97) best = s, best_cost = cost;
   }
-  if (best < 0 && shape_fits(p, 0)) best = 0;
   return best;
 }
 
