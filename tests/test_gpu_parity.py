@@ -355,7 +355,8 @@ def test_matmul_bf16_tile_multiples(hip, bmnk, rhs_nk):
 @pytest.mark.parametrize("dtype", ["bf16", "f16"])
 @pytest.mark.parametrize("rhs_nk", [True, False], ids=["NT", "NN"])
 @pytest.mark.parametrize("bmnk,bn", [((1, 4096, 4096, 256), 256), ((4, 2048, 2048, 320), 256), ((1, 8192, 2048, 384), 256), ((16, 1024, 1024, 448), 256),
-                                     ((8, 1024, 1024, 256), 128), ((1, 4096, 2048, 320), 128), ((2, 2048, 2048, 576), 128)])
+                                     ((8, 1024, 1024, 256), 128), ((1, 4096, 2048, 320), 128), ((2, 2048, 2048, 576), 128),
+                                     ((4, 1024, 1024, 256), 64), ((1, 2048, 2048, 448), 64), ((2, 1024, 2048, 576), 64)])
 def test_matmul_16bit_one_wave_per_simd_tiles(hip, bmnk, bn, rhs_nk, dtype):
     """Products whose 256 x 256 (or only whose 256 x 128) tiles fill the chip: the 4-wave kernel whose loads write LDS
     directly, for both rhs layouts (a [k, n]-major rhs goes through transposing LDS reads).  4, 5, 6, 7 and 9 K tiles:
@@ -367,12 +368,13 @@ def test_matmul_16bit_one_wave_per_simd_tiles(hip, bmnk, bn, rhs_nk, dtype):
     a = rnd(rng.uniform_pm1(25, b * m * k)).reshape(b, m, k)
     w = rnd(rng.uniform_pm1(26, b * k * n)).reshape(b, k, n)
     import os
-    os.environ["UGHIP_GEMM_SHAPE"] = "3" if bn == 256 else "4"   # K this short is a toss-up between the kernels: the choice is tested below
+    os.environ["UGHIP_GEMM_SHAPE"] = {256: "3", 128: "4", 64: "5"}[bn]   # K this short is a toss-up between the kernels: the choice is tested below
     try:
         got = _raw_matmul(hip, dt, a, w, rhs_nk)
     finally:
         del os.environ["UGHIP_GEMM_SHAPE"]
-    assert ug_amd.last_kernel() == f"gemm_dma4<{dtype},{'NT' if rhs_nk else 'NN'},256x{bn},256t>"
+    tile = {256: "256x256", 128: "256x128", 64: "128x128"}[bn]
+    assert ug_amd.last_kernel() == f"gemm_dma4<{dtype},{'NT' if rhs_nk else 'NN'},{tile},256t>"
     exact = np.matmul(a.astype(np.float64), w.astype(np.float64))
     half_ulp = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
     bound = half_ulp * np.abs(exact) + k * np.finfo(np.float32).eps * np.matmul(np.abs(a).astype(np.float64), np.abs(w).astype(np.float64))
@@ -397,7 +399,7 @@ def test_matmul_16bit_one_wave_per_simd_tiles(hip, bmnk, bn, rhs_nk, dtype):
     ((1, 4096, 4096, 1024), "gemm_dma4<bf16,NT,256x256,256t>"),      # 256 tiles of 256 x 256
     ((8, 1024, 1024, 1024), "gemm_dma4<bf16,NT,256x128,256t>"),      # 128 such tiles: the narrower one fills the chip
     ((1, 3072, 4096, 1024), "gemm_dma4<bf16,NT,256x256,256t>"),      # 192 tiles: three quarters of the chip at a higher clock
-    ((1, 2048, 2560, 2048), "gemm_dma4<bf16,NT,256x128,256t>"),      # 160 narrow tiles
+    ((1, 2048, 2560, 2048), "gemm_dma4<bf16,NT,128x128,256t>"),      # 160 tiles of 256 x 128 leave a third of the chip idle, 320 of 128 x 128 share the CUs two by two
     ((1, 2048, 2048, 5632), "gemm_tiled<bf16,NT,128x128,256t>"),     # 128 narrow tiles and a long K: the register-staged kernel
     ((1, 1024, 1024, 1024), "gemm_tiled<"),                          # a handful of tiles: K split
 ])
@@ -415,17 +417,19 @@ def test_matmul_16bit_kernel_choice(hip, bmnk, want):
 
 
 def test_matmul_16bit_one_wave_per_simd_forced_and_limits(hip, monkeypatch):
-    """UGHIP_GEMM_SHAPE=3 / 4 force the kernel onto problems it would leave to others (few tiles); shapes it cannot
-    take (K below 4 tiles, rows the tile does not divide) fall through to the register-staged kernel."""
+    """UGHIP_GEMM_SHAPE=3 / 4 / 5 force the kernel's three tiles onto a small problem (bit for bit the register-staged
+    kernel's result); shapes it cannot take (K below 4 tiles, a column count that is not a multiple of 8) fall through to
+    that kernel."""
     a = rng.bf16_round(rng.uniform_pm1(27, 2 * 512 * 256)).reshape(2, 512, 256)
     w = rng.bf16_round(rng.uniform_pm1(28, 2 * 256 * 256)).reshape(2, 256, 256)
+    monkeypatch.setenv("UGHIP_GEMM_SHAPE", "1")
     plain = _raw_matmul(hip, ug_amd.BF16, a, w, False)
     assert ug_amd.last_kernel().startswith("gemm_tiled<")
-    for shape, bn in (("3", 256), ("4", 128)):
+    for shape, tile in (("3", "256x256"), ("4", "256x128"), ("5", "128x128")):
         monkeypatch.setenv("UGHIP_GEMM_SHAPE", shape)
         for rhs_nk in (True, False):
             got = _raw_matmul(hip, ug_amd.BF16, a, w, rhs_nk)
-            assert ug_amd.last_kernel() == f"gemm_dma4<bf16,{'NT' if rhs_nk else 'NN'},256x{bn},256t>"
+            assert ug_amd.last_kernel() == f"gemm_dma4<bf16,{'NT' if rhs_nk else 'NN'},{tile},256t>"
             np.testing.assert_array_equal(got, plain)
         _raw_matmul(hip, ug_amd.BF16, a[:, :, :192], w[:, :192], True)      # 3 K tiles
         assert ug_amd.last_kernel().startswith("gemm_tiled<")
@@ -451,10 +455,10 @@ def test_matmul_16bit_one_wave_per_simd_ragged(hip, monkeypatch, bmnk, rhs_nk, d
     bound = half_ulp * np.abs(exact) + k * np.finfo(np.float32).eps * np.matmul(np.abs(a).astype(np.float64), np.abs(w).astype(np.float64))
     monkeypatch.setenv("UGHIP_GEMM_SHAPE", "1")
     other = _raw_matmul(hip, dt, a, w, rhs_nk) if rhs_nk or n % 128 == 0 else None   # the 128-row tiles take any N only with an [n, k]-major rhs
-    for shape, bn in (("3", 256), ("4", 128)):
+    for shape, tile in (("3", "256x256"), ("4", "256x128"), ("5", "128x128")):
         monkeypatch.setenv("UGHIP_GEMM_SHAPE", shape)
         got = _raw_matmul(hip, dt, a, w, rhs_nk)
-        assert ug_amd.last_kernel() == f"gemm_dma4<{dtype},{'NT' if rhs_nk else 'NN'},256x{bn},256t>"
+        assert ug_amd.last_kernel() == f"gemm_dma4<{dtype},{'NT' if rhs_nk else 'NN'},{tile},256t>"
         assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-7)
         if other is not None:
             np.testing.assert_array_equal(got, other)

@@ -43,12 +43,12 @@ hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, siz
 // negative value when the kernel does not take the problem.  Used to decide between this kernel and gemm_dma4.
 double gemm_tiled_cost_us(int dtype, const MMArgs& p, size_t batch);
 
-// 16-bit types, one wave per SIMD: 256 x bn tiles (bn = 256 or 128), 4 waves of 128 x bn/2 with the accumulators in the
-// accumulation registers, loads that write LDS directly, rhs [n, k]- or [k, n]-major (gemm_dma.hip).  Any M, N % 8 == 0,
-// K % 64 == 0 and K >= 256, 16-byte aligned rows, contiguous [batch, M, N] result.
-bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int bn);
-hipError_t gemm_dma_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, int bn);
-// The tile width (256 or 128) this kernel should take the problem with, 0 when another kernel should.
+// 16-bit types, one wave per SIMD: 256 x 256, 256 x 128 or 128 x 128 tiles (tile codes 256, 128, 64), 4 waves laid out
+// 2 x 2 with the accumulators in the accumulation registers, loads that write LDS directly, rhs [n, k]- or [k, n]-major
+// (gemm_dma.hip).  Any M, N % 8 == 0, K % 64 == 0 and K >= 256, 16-byte aligned rows, contiguous [batch, M, N] result.
+bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int tile);
+hipError_t gemm_dma_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, int tile);
+// The tile code this kernel should take the problem with, 0 when another kernel should.
 int gemm_dma_pick(int dtype, const MMArgs& p, size_t batch);
 
 }  // namespace ughip

@@ -1,9 +1,11 @@
 // 16-bit MFMA GEMM for gfx950 with one wave per SIMD: C[b] = A[b] x B[b], f32 accumulate, bf16 or f16.
 //
-//   block tile 256 x BN (BN = 256 or 128), K tile 64, 4 waves laid out 2 x 2, each owning 128 x BN/2 of the result
+//   block tile BM x BN (256 x 256, 256 x 128 or 128 x 128), K tile 64, 4 waves laid out 2 x 2, each owning BM/2 x BN/2 of the result
 //   (any M, N a multiple of 8: a last tile hangs over the end, reads the last row again and stores what exists):
-//   16 (8) accumulators of 32 x 32 live in the 256 accumulation registers a lone wave per SIMD can have, which leaves
-//   the architectural registers to two sets of operand fragments -- 8 (6) fragment reads feed 16 (8) MFMAs
+//   16 (8, 4) accumulators of 32 x 32 live in the accumulation registers -- all 256 of them for the largest tile, which
+//   a lone wave per SIMD can have -- and leave the architectural registers to two sets of operand fragments: 8 (6, 4)
+//   fragment reads feed 16 (8, 4) MFMAs, so the 128 x 128 tile is bound by its LDS reads like the register-staged
+//   kernel and is there for products whose larger tiles would leave CUs idle
 //   global -> LDS with global_load_lds_dwordx4 (no staging registers), two 64 KiB stages; the loads of tile t+2 are
 //   spread, one in front of every other MFMA, over the quarter of tile t that follows the barrier which frees their
 //   stage and over the first quarter of tile t+1: a wave alone on its SIMD has nobody to hide a burst of 16 loads
@@ -58,7 +60,7 @@ __device__ __forceinline__ void dma16(const void* base, unsigned voff, unsigned 
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
 }
 
-constexpr int BK = 64, BM = 256;
+constexpr int BK = 64;
 
 // k-contiguous operand tile ([rows][64] 16-bit): 128-byte rows of 8 chunks, chunk' = chunk ^ ((row / 2) & 7)
 __device__ __forceinline__ int kc_idx(int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); }  // in 16-byte units
@@ -69,15 +71,15 @@ __device__ __forceinline__ int kn_byte(int k, int n) {
   return k * (BN * 2) + (((n >> 5) ^ (k & (BN / 32 - 1))) << 6) + (n & 31) * 2;
 }
 
-template <typename T, int BN, bool B_KN>
+template <typename T, int BM, int BN, bool B_KN>
 __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tiles_n) {
   extern __shared__ u32x4 lds[];
-  constexpr int NJ = BN / 64;                          // 32-column fragments per wave
-  constexpr int NM = 4 * NJ;                           // MFMAs per k16 step
+  constexpr int NI = BM / 64, NJ = BN / 64;            // 32-row and 32-column fragments per wave
+  constexpr int NM = NI * NJ;                          // MFMAs per k16 step
   constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2, STAGE_BYTES = A_BYTES + B_BYTES;
-  constexpr int NDA = 8, NDB = BN / 32, ND = NDA + NDB;  // DMA instructions per wave and K tile
+  constexpr int NDA = BM / 32, NDB = BN / 32, ND = NDA + NDB;  // DMA instructions per wave and K tile
   constexpr int H = ND / 2;                            // ... per step that carries them
-  constexpr int R = 4 + NJ;                            // fragment reads per step
+  constexpr int R = NI + NJ;                           // fragment reads per step
   static_assert(R == H, "reads and DMAs of a step alternate one for one");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -104,7 +106,7 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
   const char* Ab = reinterpret_cast<const char*>(static_cast<const T*>(p.a) + (size_t)batch * p.a_bs + (size_t)m0 * lda);
   const char* Bb = reinterpret_cast<const char*>(static_cast<const T*>(p.b) + (size_t)batch * p.b_bs + (B_KN ? (size_t)n0 : (size_t)n0 * ldb));
   const int KT = p.K / BK;
-  const int wm = (wave >> 1) * 128, wn = (wave & 1) * (BN / 2);
+  const int wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
   const unsigned lds_addr = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
 
   // per-lane byte offsets of this wave's DMA instructions (the same for every K tile; the scalar base moves)
@@ -139,21 +141,21 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
     else dma16(Bb + tile * b_step, voff[idx], st + A_BYTES + ((idx - NDA) * 4 + wave) * 1024);
   };
 
-  floatx16 acc[4][NJ];
+  floatx16 acc[NI][NJ];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < NI; ++i)
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   // operand fragments of one k16 step, two sets: lane l feeds row / column l % 32, k = 8 (l / 32) .. + 7
-  u32x4 fa[2][4], fb[2][NJ];
-  auto read_frag = [&](int stage, int s, int idx, int set) {  // idx < 4: A fragment idx, else B fragment idx - 4
-    if (idx < 4) {
+  u32x4 fa[2][NI], fb[2][NJ];
+  auto read_frag = [&](int stage, int s, int idx, int set) {  // idx < NI: A fragment idx, else B fragment idx - NI
+    if (idx < NI) {
       fa[set][idx] = lds[stage * (STAGE_BYTES / 16) + kc_idx(wm + idx * 32 + (lane & 31), 2 * s + (lane >> 5))];
     } else if (!B_KN) {
-      fb[set][idx - 4] = lds[stage * (STAGE_BYTES / 16) + A_BYTES / 16 + kc_idx(wn + (idx - 4) * 32 + (lane & 31), 2 * s + (lane >> 5))];
+      fb[set][idx - NI] = lds[stage * (STAGE_BYTES / 16) + A_BYTES / 16 + kc_idx(wn + (idx - NI) * 32 + (lane & 31), 2 * s + (lane >> 5))];
     } else {
       // A transposing read returns to lane i of a 16-lane group the 4 values at column i % 4 of the rows that lanes
       // i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12 name.  Lane q + 4 e names row kbase + e, columns 4 q .. 4 q + 3 of its
@@ -162,10 +164,10 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
       typedef __attribute__((address_space(3))) s16x4 lds_v4;
       const int g = lane >> 4, li = lane & 15, q = li & 3, e = li >> 2;
       const char __attribute__((address_space(3)))* Bs = (const char __attribute__((address_space(3)))*)lds + stage * STAGE_BYTES + A_BYTES;
-      const int n = wn + (idx - 4) * 32 + 16 * (g & 1) + 4 * q, k0 = s * 16 + 8 * (g >> 1) + e;
+      const int n = wn + (idx - NI) * 32 + 16 * (g & 1) + 4 * q, k0 = s * 16 + 8 * (g >> 1) + e;
       const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4*)(Bs + kn_byte<BN>(k0, n))));
       const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4*)(Bs + kn_byte<BN>(k0 + 4, n))));
-      fb[set][idx - 4] = u32x4{lo.x, lo.y, hi.x, hi.y};
+      fb[set][idx - NI] = u32x4{lo.x, lo.y, hi.x, hi.y};
     }
   };
 
@@ -229,7 +231,7 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
   constexpr int PITCH = BN * 2 + 8;
   char __attribute__((address_space(3)))* Cs = (char __attribute__((address_space(3)))*)lds;
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < NI; ++i)
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
 #pragma unroll
@@ -254,12 +256,12 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
   }
 }
 
-template <typename T, int BN, bool B_KN>
+template <typename T, int BM, int BN, bool B_KN>
 hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch) {
   constexpr int STAGES = 2 * (BM + BN) * BK * 2, EPI = BM * (BN * 2 + 8);
   constexpr int LDS_BYTES = STAGES > EPI ? STAGES : EPI;
   static std::atomic<unsigned long long> configured{0};  // one bit per device: the attribute is per device
-  auto kernel = gemm_dma4<T, BN, B_KN>;
+  auto kernel = gemm_dma4<T, BM, BN, B_KN>;
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev)) return e;
   const unsigned long long bit = dev < 64 ? 1ull << dev : 0;
@@ -277,9 +279,21 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 
 }  // namespace
 
-bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int bn) {
+namespace {
+// tile codes of the entry points below: 256 = 256 x 256, 128 = 256 x 128, 64 = 128 x 128
+bool tile_dims(int tile, int* bm, int* bn) {
+  if (tile == 256) *bm = 256, *bn = 256;
+  else if (tile == 128) *bm = 256, *bn = 128;
+  else if (tile == 64) *bm = 128, *bn = 128;
+  else return false;
+  return true;
+}
+}  // namespace
+
+bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int tile) {
   if (dtype != UGHIP_BF16 && dtype != UGHIP_F16) return false;
-  if (bn != 256 && bn != 128) return false;
+  int bm, bn;
+  if (!tile_dims(tile, &bm, &bn)) return false;
   if (p.M <= 0 || p.N <= 0 || p.N % 8 || p.K % BK || p.K < 4 * BK || batch == 0) return false;
   if (p.a_cs != 1 || p.a_rs % 8 || (batch > 1 && (p.a_bs % 8 || p.b_bs % 8 || p.c_bs % 8))) return false;
   const bool nn = p.b_cs == 1 && p.b_rs != 1, nt = p.b_rs == 1 && p.b_cs != 1;
@@ -287,12 +301,12 @@ bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int bn) {
   const long long ldb = nn ? p.b_rs : p.b_cs;
   if (ldb % 8) return false;
   // per-lane offsets are 32-bit: the furthest row of a tile has to stay below 4 GiB from the tile's first byte
-  if ((unsigned long long)p.a_rs * 2 * BM >= (1ull << 32) || (unsigned long long)ldb * 2 * (nn ? BK : bn) >= (1ull << 32)) return false;
+  if ((unsigned long long)p.a_rs * 2 * bm >= (1ull << 32) || (unsigned long long)ldb * 2 * (nn ? BK : bn) >= (1ull << 32)) return false;
   if (!aligned16(p.a) || !aligned16(p.b) || !aligned16(p.c)) return false;
-  return batch * (size_t)((p.M + BM - 1) / BM) * (size_t)((p.N + bn - 1) / bn) < (1u << 24);
+  return batch * (size_t)((p.M + bm - 1) / bm) * (size_t)((p.N + bn - 1) / bn) < (1u << 24);
 }
 
-// Which tile this kernel should take the problem with (256 or 128), or 0 when the register-staged kernel is expected to
+// Which tile this kernel should take the problem with (a tile code), or 0 when the register-staged kernel is expected to
 // be faster.  Both are priced.  This kernel: a fixed cost (launch and first tile, 4 us, and the result's way out at the
 // rate of a stream) plus, per round of up to 256 workgroups, the K tiles at a time that grows with the share of the chip
 // that is busy -- the chip is power-bound under this kernel, a half-empty round runs at a higher clock: 0.9 + 0.6 x busy
@@ -301,17 +315,30 @@ bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int bn) {
 // (97 / 72).  The other kernel: the model that chooses its own tiles.  Against "256 x 256 tiles when they number 200 or
 // more, else 256 x 128 under the same rule" this moves products with 130-250 tiles or a short last round to this kernel
 // (3072 x 4096^2: 131 -> 91 us, 5120^2 x 1024: 77 -> 54, 1280 x 8192 x 2048: 64 -> 47, 2048 x 2560 x 2048: 35 -> 29,
-// 2304^3: 39 -> 35) and leaves those with about 128 tiles where they were (2048^2 x 5632: 56 us against 72).
-// UGHIP_GEMM_SHAPE=3 / 4 forces 256 / 128 where the kernel applies, 0..2 keeps it out (tuning aid).
-double gemm_dma_cost_us(const MMArgs& p, size_t batch, int bn) {
-  const size_t tiles = batch * (size_t)((p.M + BM - 1) / BM) * (size_t)((p.N + bn - 1) / bn);
+// 2304^3: 39 -> 35) and leaves those with about 128 tiles where they were (2048^2 x 5632: 56 us against 72).  The
+// 128 x 128 tile (two workgroups per CU) takes what neither fits: 2304^3 35 -> 31 us, 2048 x 2560 x 2048 29 -> 27.
+// UGHIP_GEMM_SHAPE=3 / 4 / 5 forces 256 x 256 / 256 x 128 / 128 x 128 where the kernel applies, 0..2 keeps it out (tuning aid).
+double gemm_dma_cost_us(const MMArgs& p, size_t batch, int tile) {
+  int bm, bn;
+  if (!tile_dims(tile, &bm, &bn)) return 1e30;
+  const size_t tiles = batch * (size_t)((p.M + bm - 1) / bm) * (size_t)((p.N + bn - 1) / bn);
   const int kt = p.K / BK;
   const bool nn = p.b_cs == 1 && p.b_rs != 1;
-  const double t0 = bn == 256 ? 0.9 : 0.62, t1 = bn == 256 ? 0.6 : 0.2;
   double us = 4.0 + (double)batch * p.M * p.N * 2 / 6.4e6;
+  const double layout = nn ? 1.08 : 1.0;
+  if (tile == 64) {
+    // two workgroups share a CU: a round is 512 tiles at 0.88 us per K tile; up to 256 tiles run one per CU at
+    // 0.47 + 0.16 x busy, the next 256 fill the second slots (2048^3 24.7 us, 2304^3 31.3, 2816^3 45.5, 5120^2 x 1024 61)
+    us += kt * 0.88 * (double)(tiles / 512) * layout;
+    const size_t left = tiles % 512;
+    if (left > 256) us += kt * (0.63 + 0.25 * (double)(left - 256) / 256.0) * layout;
+    else if (left) us += kt * (0.47 + 0.16 * (double)left / 256.0) * layout;
+    return us;
+  }
+  const double t0 = tile == 256 ? 0.9 : 0.62, t1 = tile == 256 ? 0.6 : 0.2;
   for (size_t left = tiles; left > 0; left -= left < 256 ? left : 256) {
     const double busy = (left < 256 ? (double)left : 256.0) / 256.0;
-    us += kt * (t0 + t1 * busy) * (nn ? 1.08 : 1.0);
+    us += kt * (t0 + t1 * busy) * layout;
   }
   return us;
 }
@@ -319,30 +346,34 @@ double gemm_dma_cost_us(const MMArgs& p, size_t batch, int bn) {
 int gemm_dma_pick(int dtype, const MMArgs& p, size_t batch) {
   if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
     const int s = atoi(e);
-    if (s == 3) return gemm_dma_supported(dtype, p, batch, 256) ? 256 : 0;
-    if (s == 4) return gemm_dma_supported(dtype, p, batch, 128) ? 128 : 0;
-    return 0;
+    const int forced = s == 3 ? 256 : s == 4 ? 128 : s == 5 ? 64 : 0;
+    return forced && gemm_dma_supported(dtype, p, batch, forced) ? forced : 0;
   }
   int best = 0;
   double best_us = 0;
-  for (int bn : {256, 128}) {
-    if (!gemm_dma_supported(dtype, p, batch, bn)) continue;
-    const double us = gemm_dma_cost_us(p, batch, bn);
-    if (!best || us < best_us * 0.92) best = bn, best_us = us;  // the wider tile on a near tie: fewer operand bytes
+  for (int tile : {256, 128, 64}) {
+    if (!gemm_dma_supported(dtype, p, batch, tile)) continue;
+    const double us = gemm_dma_cost_us(p, batch, tile);
+    if (!best || us < best_us * 0.97) best = tile, best_us = us;  // the larger tile on a near tie: fewer operand bytes
   }
   if (!best) return 0;
+  // the 128 x 128 tile runs at the register-staged kernel's pace (both are bound by their LDS reads): it has to be
+  // clearly cheaper to take the product from it
   const double other = gemm_tiled_cost_us(dtype, p, batch);
-  return other < 0 || best_us < other ? best : 0;
+  return other < 0 || best_us < other * (best == 64 ? 0.95 : 1.0) ? best : 0;
 }
 
-hipError_t gemm_dma_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, int bn) {
-  if (!gemm_dma_supported(dtype, p, batch, bn)) return hipErrorInvalidValue;
+hipError_t gemm_dma_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, int tile) {
+  if (!gemm_dma_supported(dtype, p, batch, tile)) return hipErrorInvalidValue;
+  int bm = 0, bn = 0;
+  tile_dims(tile, &bm, &bn);
   const bool nn = p.b_cs == 1 && p.b_rs != 1;
   const char* tn = dtype == UGHIP_F16 ? "f16" : "bf16";
-  note_kernel("gemm_dma4<%s,%s,256x%d,256t>", tn, nn ? "NN" : "NT", bn);
-#define UGHIP_DMA_CASE(T)                                                                        \
-  if (bn == 256) return nn ? launch<T, 256, true>(stream, p, batch) : launch<T, 256, false>(stream, p, batch); \
-  return nn ? launch<T, 128, true>(stream, p, batch) : launch<T, 128, false>(stream, p, batch);
+  note_kernel("gemm_dma4<%s,%s,%dx%d,256t>", tn, nn ? "NN" : "NT", bm, bn);
+#define UGHIP_DMA_CASE(T)                                                                                                  \
+  if (tile == 256) return nn ? launch<T, 256, 256, true>(stream, p, batch) : launch<T, 256, 256, false>(stream, p, batch); \
+  if (tile == 128) return nn ? launch<T, 256, 128, true>(stream, p, batch) : launch<T, 256, 128, false>(stream, p, batch); \
+  return nn ? launch<T, 128, 128, true>(stream, p, batch) : launch<T, 128, 128, false>(stream, p, batch);
   if (dtype == UGHIP_F16) {
     UGHIP_DMA_CASE(_Float16)
   }
