@@ -21,8 +21,10 @@
 // once per token and nothing else of that size.  (ug's Device::matmul wants one dtype for all three operands, ug-core/src/lib.rs:62-70;
 // a checkpoint stored in bf16 is widened at load time, ug-core/src/safetensors.rs:120-271.)
 //
-// KS waves share one output column, each walking every KS-th 64-lane slab of k with four 128-bit
-// loads in flight per lane and matrix; a workgroup of 4 waves covers 4 / KS columns.
+// F32 matrices (and BF16 rows the kernel below does not take): KS waves share one output column, each
+// walking every KS-th 64-lane slab of k with four 128-bit loads in flight per lane and matrix; a
+// workgroup of 4 waves covers 4 / KS columns.  BF16 matrices with rows of 512 .. 8192 elements:
+// fused_gemv_bf16_rows, x in registers and R rows per workgroup (described where it is defined).
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
