@@ -380,8 +380,9 @@ int ughip_rms_gemv_gate_up(ughip_device* dev, const ughip_slice* x, const ughip_
 int ughip_gemv_add(ughip_device* dev, const ughip_slice* x, const ughip_slice* w,
                    const ughip_slice* residual, ughip_slice* dst, size_t n, size_t k);
 
-/* ---- the same for several positions (m >= 9 rows; a prefill) ------------------------------------
- * x is [m, k] F32 with contiguous rows, w a row-major [n, k] matrix stored as F32 or BF16, k % 32 == 0, n % 8 == 0.
+/* ---- the same for several positions (a prefill) -------------------------------------------------
+ * x is [m, k] F32 with contiguous rows, w a row-major [n, k] matrix stored as F32 or BF16, k % 32 == 0, n % 8 == 0;
+ * m >= 9 with an F32 matrix (2 .. 8 rows are ughip_matmul's row-vector kernels), m >= 2 with a BF16 one.
  * The product is the tiled MFMA kernel's; skinny products split K over workgroups, and the fold of their
  * partial tiles (which a plain ughip_matmul of these shapes runs anyway) applies the neighbour on its way out,
  * so the residual add / SwiGLU of model.rs:99-109,160-168,366-372 costs no launch and no round trip.

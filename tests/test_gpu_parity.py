@@ -1379,10 +1379,12 @@ def test_fused_projections_bf16_random_shapes(hip, hip_ops):
         assert np.all(np.abs(got - t_add) <= _gemv_tol(x, ws[0]) + 1e-6 * np.abs(t_add)), case
 
 
-def test_bf16_matrices_meet_several_rows_through_a_cast(hip, hip_ops):
-    """Prefill shapes: a bf16 matrix is widened in front of matmul (one dtype per product,
-    ug-core/src/lib.rs:62-70) and the result is that of the f32 matrix with the same values."""
-    t, k, n = 5, 256, 48
+@pytest.mark.parametrize("t", [2, 5, 8])
+def test_bf16_matrices_meet_a_few_rows(hip, hip_ops, t):
+    """2 .. 8 positions: an f32 matrix takes the row-vector kernels, a bf16 one the tiled product that widens it on its way
+    into LDS (no widened copy of the matrix is made).  The results are those of the f32 matrix with the same values to the
+    rounding of another order of the sums, and both sit within the float64 bound."""
+    k, n = 256, 48
     x = rng.normal(131, t * k)
     ws = [rng.bf16_round(rng.normal(132 + i, n * k, 0.05)) for i in range(2)]
     r = rng.normal(135, t * n)
@@ -1394,8 +1396,18 @@ def test_bf16_matrices_meet_several_rows_through_a_cast(hip, hip_ops):
         o = hip_ops.linear_add(LB.copy(x, (1, t, k), hip), m[1], LB.copy(r, (1, t, n), hip)).data_vec()
         return a, g, o
 
-    for got, want in zip(run(True), run(False)):
-        assert np.array_equal(got, want)
+    x6 = x.reshape(t, k).astype(np.float64)
+    w6 = [w.reshape(n, k).astype(np.float64) for w in ws]
+    p0, p1 = x6 @ w6[0].T, x6 @ w6[1].T
+    tol0 = 2e-6 * (np.abs(x6) @ np.abs(w6[0]).T) + 1e-30
+    tol1 = 2e-6 * (np.abs(x6) @ np.abs(w6[1]).T) + 1e-30
+    sig = 1.0 / (1.0 + np.exp(-p0))
+    truths = (np.concatenate([p0, p1], 1).ravel(), (p0 * sig * p1).ravel(), (p1 + r.reshape(t, n)).ravel())
+    tols = (np.concatenate([tol0, tol1], 1).ravel(), (1.1 * tol0 * np.abs(p1) + np.abs(p0 * sig) * tol1 + 4e-7 * np.abs(p0 * sig * p1)).ravel() + 1e-30,
+            tol1.ravel() + 1.2e-7 * np.abs(truths[2]))
+    for got, want, truth, tol in zip(run(True), run(False), truths, tols):
+        assert np.all(np.abs(got - truth) <= tol), float((np.abs(got - truth) / tol).max())
+        assert np.all(np.abs(want - truth) <= tol), float((np.abs(want - truth) / tol).max())
 
 
 @pytest.mark.parametrize("t,k,n", [(128, 2048, 2048), (128, 5632, 2048), (100, 256, 192), (37, 64, 48), (9, 32, 16), (300, 512, 1000)])
@@ -1573,6 +1585,8 @@ def test_projections_of_several_rows_limits(hip):
     wb = alloc(ug_amd.BF16, 2 * n * 96)
     assert lib.ughip_linear_rows(dev, x, wb, d, z(m), z(n), z(32), x3p) != 0 and b"k % 64" in lib.ughip_last_error()
     assert lib.ughip_linear_rows(dev, x, wb, d, z(m), z(n), z(k), x3p) == 0, lib.ughip_last_error()
+    assert lib.ughip_linear_rows(dev, x, wb, d, z(2), z(n), z(k), f32p) == 0, lib.ughip_last_error()      # a BF16 matrix is taken from 2 rows on
+    assert lib.ughip_linear_rows(dev, x, wb, d, z(1), z(n), z(k), f32p) != 0 and b"m >= 2" in lib.ughip_last_error()
     # dst == residual: x w^T accumulates onto the residual in place
     xs, ws, rs = rng.normal(151, m * k), rng.normal(152, n * k, 0.1), rng.normal(153, m * n)
     sx, sw, sr = hip.slice_from(xs), hip.slice_from(ws), hip.slice_from(rs)
@@ -1585,8 +1599,8 @@ def test_projections_of_several_rows_limits(hip):
 
 
 def test_linear_hook_reads_bf16_matrices_in_place(hip, hip_ops):
-    """Ops::linear: 9 or more rows of f32 against a bf16 matrix go to the mixed product, one row to the fused
-    projection, 2 to 8 rows widen the matrix first; all are the f32 result on the same values."""
+    """Ops::linear: 2 or more rows of f32 against a bf16 matrix go to the mixed product, one row to the fused
+    projection; all are the f32 result on the same values (bit for bit where the f32 matrix takes the same kernel)."""
     k, n = 256, 192
     w = rng.bf16_round(rng.normal(137, n * k, 0.05))
     for t in (128, 384, 5, 100, 1):
@@ -1594,8 +1608,11 @@ def test_linear_hook_reads_bf16_matrices_in_place(hip, hip_ops):
         wide = hip_ops.linear(LB.copy(x, (1, t, k), hip), LB.copy(w, (n, k), hip)).data_vec()
         got = hip_ops.linear(LB.copy(x, (1, t, k), hip), LB.copy(rng.to_bf16_bits(w), (n, k), hip))
         assert tuple(got.dims()) == (1, t, n) and got.dtype == ug_amd.F32
-        np.testing.assert_array_equal(got.data_vec(), wide)
         truth = x.reshape(t, k).astype(np.float64) @ w.reshape(n, k).astype(np.float64).T
+        if t == 5:   # the f32 matrix meets 2 .. 8 rows in the row-vector kernel, the bf16 one in the tiled product: another order of the sums
+            np.testing.assert_allclose(got.data_vec().reshape(t, n), truth, rtol=1e-4, atol=1e-5)
+        else:
+            np.testing.assert_array_equal(got.data_vec(), wide)
         np.testing.assert_allclose(wide.reshape(t, n), truth, rtol=1e-4, atol=1e-5)
 
 

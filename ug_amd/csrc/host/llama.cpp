@@ -259,7 +259,7 @@ struct HipOps : Ops {
   LB linear(const LB& x, const LB& w) const override {
     const size_t rows = x.rank() ? x.elem_count() / x.dims().back() : 0;
     if (x.dtype() == DType::F32 && w.dtype() == DType::BF16 && rows == 1 && x.rank() == 3 && one_f32_row(x, {&w})) return linear_packed(x, {w}, nullptr, 0.f);
-    if (x.dtype() != DType::F32 || w.dtype() != DType::BF16 || w.rank() != 2 || x.rank() < 2 || w.dims()[1] != x.dims().back() || rows <= 8 ||
+    if (x.dtype() != DType::F32 || w.dtype() != DType::BF16 || w.rank() != 2 || x.rank() < 2 || w.dims()[1] != x.dims().back() || rows <= 1 ||
         w.dims()[1] % 32 != 0)
       return Ops::linear(x, w);
     const size_t n = w.dims()[0], k = w.dims()[1];
@@ -331,7 +331,9 @@ struct HipOps : Ops {
   static bool many_f32_rows(const LB& x, const LB& w, size_t n_multiple) {
     if (x.rank() < 2 || w.rank() != 2 || x.dtype() != DType::F32 || (w.dtype() != DType::F32 && w.dtype() != DType::BF16)) return false;
     const size_t k = x.dims().back(), rows = x.elem_count() / (k ? k : 1);
-    return k != 0 && w.dims()[1] == k && rows >= 9 && k % 32 == 0 && w.dims()[0] % n_multiple == 0;
+    // 2 .. 8 rows against an F32 matrix take the row-vector kernels; a BF16 matrix would have to be widened for those
+    // (three times its bytes moved), so it goes to the tiled product from 2 rows on
+    return k != 0 && w.dims()[1] == k && rows >= (w.dtype() == DType::BF16 ? 2u : 9u) && k % 32 == 0 && w.dims()[0] % n_multiple == 0;
   }
 
   LB gate_up_stacked(const LB& x, const LB& w) const override {

@@ -494,20 +494,25 @@ hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int s
     case 1:
       return p.M % 128 || p.N % 128 ? launch<T, B_NK, 128, 128, 256, SPLIT, true>(stream, p, batch, nsplit, ws, epi)
                                     : launch<T, B_NK, 128, 128, 256, SPLIT>(stream, p, batch, nsplit, ws, epi);
-    default:
+    case 2:
       return p.M % 128 || p.N % 64 ? launch<T, B_NK, 128, 64, 256, SPLIT, true>(stream, p, batch, nsplit, ws, epi)
                                    : launch<T, B_NK, 128, 64, 256, SPLIT>(stream, p, batch, nsplit, ws, epi);
+    default:
+      return p.M % 64 || p.N % 128 ? launch<T, B_NK, 64, 128, 256, SPLIT, true>(stream, p, batch, nsplit, ws, epi)
+                                   : launch<T, B_NK, 64, 128, 256, SPLIT>(stream, p, batch, nsplit, ws, epi);
   }
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-constexpr int kShapes[3][2] = {{256, 128}, {128, 128}, {128, 64}};
+constexpr int kNumShapes = 4;
+constexpr int kShapes[kNumShapes][2] = {{256, 128}, {128, 128}, {128, 64}, {64, 128}};
 
-// Which of the three tiles a problem can take: the 128-row tiles also take an lhs whose last tile is partly empty (any
-// M >= 9: fewer rows are the GEMV kernels' job) and, with an [n, k]-major rhs, an N they do not divide.
+// Which of the tiles a problem can take: the 128- and 64-row tiles also take an lhs whose last tile is partly empty (any
+// M >= 9: fewer rows are the GEMV kernels' job) and, with an [n, k]-major rhs, an N they do not divide.  The 64-row tile
+// is for prompts of up to 64 positions: half the rows of a 128-row tile would be multiplied for nothing.
 bool shape_fits(const MMArgs& p, int s) {
-  const bool rhs_nk = p.b_rs == 1 && p.b_cs != 1, ragged_ok = kShapes[s][0] == 128;
+  const bool rhs_nk = p.b_rs == 1 && p.b_cs != 1, ragged_ok = kShapes[s][0] <= 128;
   return !((p.M % kShapes[s][0] && !ragged_ok) || (p.N % kShapes[s][1] && !(ragged_ok && rhs_nk)));
 }
 size_t tile_count(const MMArgs& p, size_t batch, int s) {
@@ -555,19 +560,21 @@ Split pick_split(int dtype, const MMArgs& p, size_t batch, int shape, bool alway
 int pick_shape(const MMArgs& p, size_t batch, int dtype, bool always_fold = false) {
   // UGHIP_GEMM_SHAPE=0..2 forces a tile shape (tuning aid); ignored when it does not fit the problem.
   if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
-    const int s = atoi(e);
-    if (s >= 0 && s < 3 && shape_fits(p, s)) return s;
+    const int s = atoi(e) == 6 ? 3 : atoi(e);  // 3..5 name the other kernel's tiles: 6 is the 64-row tile here
+    if (s >= 0 && s < kNumShapes && (s < 3 || atoi(e) == 6) && shape_fits(p, s)) return s;
   }
   int best = -1;
   double best_cost = 0;
-  for (int s = 0; s < 3; ++s) {
+  for (int s = 0; s < kNumShapes; ++s) {
     if (!shape_fits(p, s)) continue;
     const double cost = pick_split(dtype, p, batch, s, always_fold).cost_us;
     if (best < 0) {
       best = s, best_cost = cost;
       continue;
     }
-    const bool few = tile_count(p, batch, best) < 256 && tile_count(p, batch, s) < 256;
+    // 64 x 128 against 128 x 64 (the same area): only when it is really cheaper, i.e. when the rows fit 64 -- two tile
+    // rows of 64 read every weight twice
+    const bool few = s != 3 && tile_count(p, batch, best) < 256 && tile_count(p, batch, s) < 256;
     if (few ? cost <= best_cost * 1.03 : cost < best_cost * 0.97) best = s, best_cost = cost;
   }
   return best;
@@ -622,7 +629,7 @@ hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, siz
   const int nsplit = pick_split(dtype, p, batch, s, epi != nullptr).nsplit;
   {
     const char* tn = rhs_bf16 ? "f32xbf16" : dtype == UGHIP_F32 ? "f32" : dtype == UGHIP_F16 ? "f16" : "bf16";
-    const bool ragged = s != 0 && s != 3 && (p.M % kShapes[s][0] || p.N % kShapes[s][1]);
+    const bool ragged = s != 0 && (p.M % kShapes[s][0] || p.N % kShapes[s][1]);
     char split[48] = "";
     if (nsplit > 1 || epi)
       snprintf(split, sizeof split, ",splitK=%d%s%s", nsplit, !epi ? "" : epi->kind == GemmEpilogue::ADD ? ",+residual" : epi->kind == GemmEpilogue::SWIGLU ? ",swiglu" : "",

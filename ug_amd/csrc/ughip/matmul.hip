@@ -590,8 +590,10 @@ static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x
   const bool mixed = !x3 && w->dtype == UGHIP_BF16;
   const int dtype = x3 ? UGHIP_BF16 : UGHIP_F32;
   // (x3: p.a is checked for alignment below with the f32 rows standing in; the planes live in the 256-byte aligned scratch block)
-  if (m < 9 || rows % 8 != 0 || (kind == GemmEpilogue::SWIGLU && rows % 16 != 0) || (x3 && k % 64 != 0) || !gemm_tiled_supported(dtype, p, 1, mixed))
-    return set_error(UGHIP_ERR_UNSUPPORTED, "%s: built for m >= 9 rows, k %% 32 == 0 (k %% 64 == 0 for the three-term bf16 product), n %% 8 == 0 and 16-byte aligned buffers (got m %zu, n %zu, k %zu)",
+  // an F32 matrix under 2 .. 8 rows is the row-vector kernels' job (ughip_matmul); those do not read a BF16 matrix
+  const size_t min_rows = w->dtype == UGHIP_BF16 ? 2 : 9;
+  if (m < min_rows || rows % 8 != 0 || (kind == GemmEpilogue::SWIGLU && rows % 16 != 0) || (x3 && k % 64 != 0) || !gemm_tiled_supported(dtype, p, 1, mixed))
+    return set_error(UGHIP_ERR_UNSUPPORTED, "%s: built for m >= 9 rows (m >= 2 with a BF16 matrix), k %% 32 == 0 (k %% 64 == 0 for the three-term bf16 product), n %% 8 == 0 and 16-byte aligned buffers (got m %zu, n %zu, k %zu)",
                      what, m, out_cols, k);
   if (int rc = device_activate(dev)) return rc;
   GemmEpilogue epi{kind, residual ? static_cast<const float*>(residual->ptr) : nullptr};
