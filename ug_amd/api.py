@@ -621,7 +621,7 @@ class LlamaOps(_Handle):
 
     @staticmethod
     def hip(bf16x3=False):
-        """bf16x3: nine or more f32 rows against a BF16 matrix are split into three bf16 terms each and multiplied on the
+        """bf16x3: two or more f32 rows against a BF16 matrix are split into three bf16 terms each and multiplied on the
         bf16 matrix pipe (UGHIP_PRODUCT_BF16X3) instead of widening the matrix for the f32 pipe."""
         out = C.c_void_p()
         _chk(host_lib().ugh_llama_ops_hip_ex(1 if bf16x3 else 0, C.byref(out)))

@@ -104,7 +104,7 @@ struct Ops {
 };
 
 // The HIP implementation (counterpart of ug-llama/src/cuda_ops.rs).
-// bf16x3: products of nine or more f32 rows with a BF16 matrix split the rows into three bf16 terms and run on the
+// bf16x3: products of two or more f32 rows with a BF16 matrix split the rows into three bf16 terms and run on the
 // bf16 matrix pipe (UGHIP_PRODUCT_BF16X3) instead of widening the matrix for the f32 pipe.
 std::shared_ptr<Ops> hip_ops(bool bf16x3 = false);
 
