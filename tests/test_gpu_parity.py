@@ -1410,7 +1410,7 @@ def test_bf16_matrices_meet_a_few_rows(hip, hip_ops, t):
         assert np.all(np.abs(want - truth) <= tol), float((np.abs(want - truth) / tol).max())
 
 
-@pytest.mark.parametrize("t,k,n", [(128, 2048, 2048), (128, 5632, 2048), (100, 256, 192), (37, 64, 48), (9, 32, 16), (300, 512, 1000)])
+@pytest.mark.parametrize("t,k,n", [(128, 2048, 2048), (128, 5632, 2048), (100, 256, 192), (37, 64, 48), (9, 32, 16), (300, 512, 1000), (64, 2048, 2048), (16, 512, 264)])
 @pytest.mark.parametrize("bf16", [False, True])
 def test_projections_of_several_rows_with_the_neighbour_in_the_fold(hip, cpu, hip_ops, cpu_ops, monkeypatch, t, k, n, bf16):
     """Prefill shapes: linear_add and gate_up_stacked over 9 or more rows fold the residual add / SwiGLU into the fold of
@@ -1451,7 +1451,8 @@ def test_projections_of_several_rows_with_the_neighbour_in_the_fold(hip, cpu, hi
         assert np.all(np.abs(o_hip - o_two) <= 2 * o_bound) and np.all(np.abs(g_hip - g_two) <= 2 * g_bound)
 
 
-@pytest.mark.parametrize("t,k,n", [(128, 2048, 2048), (128, 5632, 2048), (128, 2048, 2560), (100, 256, 192), (37, 64, 48), (9, 64, 16), (300, 512, 1000)])
+@pytest.mark.parametrize("t,k,n", [(128, 2048, 2048), (128, 5632, 2048), (128, 2048, 2560), (100, 256, 192), (37, 64, 48), (9, 64, 16), (300, 512, 1000),
+                                   (2, 2048, 2048), (5, 256, 48), (64, 2048, 5632), (33, 512, 136)])
 def test_projections_of_several_rows_as_three_bf16_terms(hip, t, k, n):
     """UGHIP_PRODUCT_BF16X3: every f32 row element is split into three bf16 terms and the bf16 matrix pipe multiplies them
     by the BF16 matrix as stored.  The product terms are exact, so the result has the f32 product's accuracy (the k eps
@@ -1630,7 +1631,7 @@ def test_llama_bf16_matrices_prefill_of_128_tokens(hip, hip_ops):
     np.testing.assert_allclose(st["margins"], wide[1]["margins"], rtol=1e-4, atol=1e-6)
 
 
-@pytest.mark.parametrize("n_prompt", [9, 37, 100, 128, 200])
+@pytest.mark.parametrize("n_prompt", [2, 5, 9, 37, 64, 100, 128, 200])
 def test_llama_prompt_products_as_three_bf16_terms(hip, cpu, hip_ops, cpu_ops, n_prompt):
     """bf16 matrices with the prompt's products as three bf16 terms per row element (prompt lengths the tiles divide and
     do not): the oracle's ids on the same bf16-rounded weights, margins to 1e-2 relative like the f32-pipe model's, and
