@@ -1475,8 +1475,27 @@ def test_projections_of_several_rows_as_three_bf16_terms(hip, t, k, n):
         glu = ops.gate_up_stacked(xs(), LB.copy(bits(wgu), (2 * n, k), hip)).data_vec().reshape(t, n)
         return lin, add, glu, kern
 
+    def run_c_abi():
+        """the three entry points with product = UGHIP_PRODUCT_BF16X3, straight through the C ABI"""
+        import ctypes as C
+        lib, dev, z = ug_amd.ughip_lib(), C.c_void_p(hip.raw_hip()), C.c_size_t
+        raw = lambda s_: C.c_void_p(s_.raw())
+        sx, sw, sgu, sr = hip.slice_from(x), hip.slice_from(bits(w)), hip.slice_from(bits(wgu)), hip.slice_from(r)
+        d = hip.allocate_uninit(ug_amd.F32, t * n)
+        assert lib.ughip_linear_rows(dev, raw(sx), raw(sw), raw(d), z(t), z(n), z(k), C.c_int(1)) == 0, lib.ughip_last_error()
+        kern = ug_amd.last_kernel()
+        lin = d.to_vec().reshape(t, n)
+        assert lib.ughip_linear_add_rows(dev, raw(sx), raw(sw), raw(sr), raw(d), z(t), z(n), z(k), C.c_int(1)) == 0, lib.ughip_last_error()
+        add = d.to_vec().reshape(t, n)
+        assert lib.ughip_linear_swiglu_rows(dev, raw(sx), raw(sgu), raw(d), z(t), z(n), z(k), C.c_int(1)) == 0, lib.ughip_last_error()
+        return lin, add, d.to_vec().reshape(t, n), kern
+
     lin3, add3, glu3, kern3 = run(x3_ops)
     lin1, add1, glu1, kern1 = run(f32_ops)
+    if t <= 64:
+        # up to 64 rows the hooks keep the f32 pipe (a 32- or 64-row tile there is as fast as the split, three planes and an f32 fold)
+        assert kern3.startswith("gemm_tiled<f32xbf16,NT,"), kern3
+        lin3, add3, glu3, kern3 = run_c_abi()
     assert kern3.startswith("gemm_tiled<bf16,NT,") and "f32 out" in kern3, kern3
     assert kern1.startswith("gemm_tiled<f32xbf16,NT,"), kern1
     x64, w64, gu64 = x.reshape(t, k).astype(np.float64), w.reshape(n, k).astype(np.float64), wgu.reshape(2 * n, k).astype(np.float64)

@@ -264,7 +264,7 @@ struct HipOps : Ops {
       return Ops::linear(x, w);
     const size_t n = w.dims()[0], k = w.dims()[1];
     ughip_device* dev = hip_dev(x);
-    const bool x3 = product_for(w, k) == UGHIP_PRODUCT_BF16X3 && n % 8 == 0;
+    const bool x3 = product_for(w, k, rows) == UGHIP_PRODUCT_BF16X3 && n % 8 == 0;
     auto f = [=](const std::vector<Slice*>& vs) {
       if (vs.size() != 3) bail("linear: expected 3 slices");
       if (x3) {
@@ -324,7 +324,11 @@ struct HipOps : Ops {
 
   // How nine or more f32 rows meet this matrix: three bf16 terms per row element on the bf16 matrix pipe when that was
   // asked for and the matrix is bf16 with k a multiple of 64, else the f32 pipe.
-  int product_for(const LB& w, size_t k) const { return bf16x3_ && w.dtype() == DType::BF16 && k % 64 == 0 ? UGHIP_PRODUCT_BF16X3 : UGHIP_PRODUCT_F32; }
+  // Up to 64 rows the f32 pipe on a 32- or 64-row tile is as fast as three bf16 terms (which cost a split and an f32
+  // fold per product): 1.95-2.1 ms against 2.2 for a prompt of 2 .. 32 tokens, the same at 64.
+  int product_for(const LB& w, size_t k, size_t rows) const {
+    return bf16x3_ && rows > 64 && w.dtype() == DType::BF16 && k % 64 == 0 ? UGHIP_PRODUCT_BF16X3 : UGHIP_PRODUCT_F32;
+  }
 
   // Several positions of f32 rows against a row-major [n, k] matrix (f32 or bf16) in shapes the tiled kernel takes:
   // the fold of its partial tiles can apply the neighbouring op.
@@ -340,7 +344,7 @@ struct HipOps : Ops {
     if (!many_f32_rows(x, w, 16) || getenv("UG_LLAMA_NO_FOLD_EPILOGUES")) return Ops::gate_up_stacked(x, w);
     const size_t k = x.dims().back(), rows = x.elem_count() / k, n = w.dims()[0] / 2;
     ughip_device* dev = hip_dev(x);
-    const int product = product_for(w, k);
+    const int product = product_for(w, k, rows);
     auto f = [=](const std::vector<Slice*>& vs) {
       if (vs.size() != 3) bail("gate_up_stacked: expected 3 slices");
       hip_check(ughip_linear_swiglu_rows(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), rows, n, k, product), "gate_up_stacked");
@@ -355,7 +359,7 @@ struct HipOps : Ops {
         !getenv("UG_LLAMA_NO_FOLD_EPILOGUES")) {
       const size_t k = x.dims().back(), rows = x.elem_count() / k, n = w.dims()[0];
       ughip_device* dev = hip_dev(x);
-      const int product = product_for(w, k);
+      const int product = product_for(w, k, rows);
       auto f = [=](const std::vector<Slice*>& vs) {
         if (vs.size() != 4) bail("linear_add: expected 4 slices");
         hip_check(ughip_linear_add_rows(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]), hip_raw_slice(*vs[3]), rows, n, k, product), "linear_add");

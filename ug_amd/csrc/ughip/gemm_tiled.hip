@@ -311,7 +311,9 @@ template <typename T, int B_NK, int BM, int BN, int NT, bool SPLIT, bool RAGGED 
 __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p_in, int tiles_m, int tiles_n, int remap, int nsplit, int kt_per, float* __restrict__ ws) {
   extern __shared__ u32x4 lds[];
   constexpr int BK = Elt<T>::BK;
-  constexpr int WM = BM / (NT / 128), WN = BN / 2, MI = WM / 32, NJ = WN / 32;
+  // waves over the tile: two columns of waves, except for a 32-row tile, whose waves sit side by side
+  constexpr int WAVES_M = BM >= 64 ? NT / 128 : 1, WAVES_N = NT / 64 / WAVES_M;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, MI = WM / 32, NJ = WN / 32;
   constexpr int STAGE = (BM + BN) * CHUNKS;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int bid = blockIdx.x;
@@ -340,7 +342,7 @@ __global__ void __launch_bounds__(NT) gemm_tiled(MMArgs p_in, int tiles_m, int t
   const BT* __restrict__ B =
       static_cast<const BT*>(p.b) + (size_t)batch * p.b_bs + (B_NK ? (size_t)n0 * p.b_cs + k_off_b : (size_t)n0 + k_off_b * (size_t)p.b_rs);
   const int KT = SPLIT ? min(kt_per, p.K / BK - kt0) : p.K / BK;
-  const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+  const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
 
   floatx16 acc[MI][NJ];
 #pragma unroll
@@ -497,20 +499,24 @@ hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int s
     case 2:
       return p.M % 128 || p.N % 64 ? launch<T, B_NK, 128, 64, 256, SPLIT, true>(stream, p, batch, nsplit, ws, epi)
                                    : launch<T, B_NK, 128, 64, 256, SPLIT>(stream, p, batch, nsplit, ws, epi);
-    default:
+    case 3:
       return p.M % 64 || p.N % 128 ? launch<T, B_NK, 64, 128, 256, SPLIT, true>(stream, p, batch, nsplit, ws, epi)
                                    : launch<T, B_NK, 64, 128, 256, SPLIT>(stream, p, batch, nsplit, ws, epi);
+    default:
+      return p.M % 32 || p.N % 128 ? launch<T, B_NK, 32, 128, 256, SPLIT, true>(stream, p, batch, nsplit, ws, epi)
+                                   : launch<T, B_NK, 32, 128, 256, SPLIT>(stream, p, batch, nsplit, ws, epi);
   }
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-constexpr int kNumShapes = 4;
-constexpr int kShapes[kNumShapes][2] = {{256, 128}, {128, 128}, {128, 64}, {64, 128}};
+constexpr int kNumShapes = 5;
+constexpr int kShapes[kNumShapes][2] = {{256, 128}, {128, 128}, {128, 64}, {64, 128}, {32, 128}};
 
 // Which of the tiles a problem can take: the 128- and 64-row tiles also take an lhs whose last tile is partly empty (any
 // M >= 9: fewer rows are the GEMV kernels' job) and, with an [n, k]-major rhs, an N they do not divide.  The 64-row tile
-// is for prompts of up to 64 positions: half the rows of a 128-row tile would be multiplied for nothing.
+// and the 32-row tile are for prompts of up to 64 and 32 positions: most rows of a 128-row tile would be multiplied for
+// nothing.
 bool shape_fits(const MMArgs& p, int s) {
   const bool rhs_nk = p.b_rs == 1 && p.b_cs != 1, ragged_ok = kShapes[s][0] <= 128;
   return !((p.M % kShapes[s][0] && !ragged_ok) || (p.N % kShapes[s][1] && !(ragged_ok && rhs_nk)));
@@ -560,8 +566,8 @@ Split pick_split(int dtype, const MMArgs& p, size_t batch, int shape, bool alway
 int pick_shape(const MMArgs& p, size_t batch, int dtype, bool always_fold = false) {
   // UGHIP_GEMM_SHAPE=0..2 forces a tile shape (tuning aid); ignored when it does not fit the problem.
   if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
-    const int s = atoi(e) == 6 ? 3 : atoi(e);  // 3..5 name the other kernel's tiles: 6 is the 64-row tile here
-    if (s >= 0 && s < kNumShapes && (s < 3 || atoi(e) == 6) && shape_fits(p, s)) return s;
+    const int v = atoi(e), s = v == 6 ? 3 : v == 7 ? 4 : v;  // 3..5 name the other kernel's tiles: 6 and 7 are the 64- and 32-row tiles here
+    if (s >= 0 && s < kNumShapes && (s < 3 || v >= 6) && shape_fits(p, s)) return s;
   }
   int best = -1;
   double best_cost = 0;
@@ -574,7 +580,7 @@ int pick_shape(const MMArgs& p, size_t batch, int dtype, bool always_fold = fals
     }
     // 64 x 128 against 128 x 64 (the same area): only when it is really cheaper, i.e. when the rows fit 64 -- two tile
     // rows of 64 read every weight twice
-    const bool few = s != 3 && tile_count(p, batch, best) < 256 && tile_count(p, batch, s) < 256;
+    const bool few = s < 3 && tile_count(p, batch, best) < 256 && tile_count(p, batch, s) < 256;
     if (few ? cost <= best_cost * 1.03 : cost < best_cost * 0.97) best = s, best_cost = cost;
   }
   return best;
