@@ -395,6 +395,29 @@ def test_matmul_16bit_one_wave_per_simd_tiles(hip, bmnk, bn, rhs_nk, dtype):
     np.testing.assert_array_equal(_raw_matmul(hip, dt, ai, wi, rhs_nk), want)
 
 
+def test_matmul_16bit_one_wave_per_simd_random_shapes(hip, monkeypatch):
+    """Seeded random shapes (rows from 9 up to a few tiles, columns any multiple of 8, 4 to 9 K tiles, one to three
+    batches, both rhs layouts and both 16-bit types) through each of the kernel's three tiles: float64 bound and the guard
+    region behind the result."""
+    gen = np.random.default_rng(20240713)
+    for case in range(18):
+        b = int(gen.integers(1, 4))
+        m, n, k = int(gen.integers(9, 600)), int(gen.integers(1, 80)) * 8, int(gen.integers(4, 10)) * 64
+        rhs_nk, f16 = bool(gen.integers(0, 2)), bool(gen.integers(0, 2))
+        shape = ("3", "4", "5")[case % 3]
+        print("one-wave-per-SIMD random", case, (b, m, n, k), "NT" if rhs_nk else "NN", "f16" if f16 else "bf16", "tile", shape, flush=True)
+        rnd = (lambda v: v.astype(np.float16).astype(np.float32)) if f16 else rng.bf16_round
+        a = rnd(rng.uniform_pm1(700 + case, b * m * k)).reshape(b, m, k)
+        w = rnd(rng.uniform_pm1(800 + case, b * k * n)).reshape(b, k, n)
+        monkeypatch.setenv("UGHIP_GEMM_SHAPE", shape)
+        got = _raw_matmul(hip, ug_amd.F16 if f16 else ug_amd.BF16, a, w, rhs_nk)
+        assert ug_amd.last_kernel().startswith("gemm_dma4<"), ug_amd.last_kernel()
+        exact = np.matmul(a.astype(np.float64), w.astype(np.float64))
+        half_ulp = 2.0 ** -11 if f16 else 2.0 ** -8
+        bound = half_ulp * np.abs(exact) + k * np.finfo(np.float32).eps * np.matmul(np.abs(a).astype(np.float64), np.abs(w).astype(np.float64))
+        assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-7), case
+
+
 @pytest.mark.parametrize("bmnk,want", [
     ((1, 4096, 4096, 1024), "gemm_dma4<bf16,NT,256x256,256t>"),      # 256 tiles of 256 x 256
     ((8, 1024, 1024, 1024), "gemm_dma4<bf16,NT,256x128,256t>"),      # 128 such tiles: the narrower one fills the chip
