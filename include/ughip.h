@@ -282,7 +282,7 @@ int ughip_causal_softmax_rows(ughip_device* dev, const ughip_slice* src, ughip_s
                               size_t bh, size_t s1, size_t s2);
 /* Attention of one query position, f32: q [b, n_heads, d], k and v [b, n_kv_heads, s, d]
  * (query head h reads kv head h / (n_heads / n_kv_heads), i.e. model.rs:80-92's repeat),
- * dst [b, n_heads, d] = softmax(q k^T * scale) v.  d a power of two in 16..256.  From 1024 keys up
+ * dst [b, n_heads, d] = softmax(q k^T * scale) v.  d a power of two in 16..256.  From 800 keys up
  * the keys of a head are split over several workgroups and merged by a second launch; the partial
  * rows live in a scratch block the device keeps (grown on demand). */
 int ughip_attention_decode(ughip_device* dev, const ughip_slice* q, const ughip_slice* k,

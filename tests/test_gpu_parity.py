@@ -907,7 +907,7 @@ def test_llama_bf16_matrices_are_the_rounded_f32_model(hip, cpu, hip_ops, cpu_op
 
 @pytest.mark.parametrize("b,nh,nkv,s,d", [(1, 8, 2, 1, 64), (1, 8, 2, 5, 64), (2, 4, 4, 700, 64), (1, 4, 1, 3000, 128), (1, 2, 2, 300, 32)])
 def test_attention_decode_key_ranges(hip, hip_ops, b, nh, nkv, s, d):
-    """The keys of a head split over 2, 8 or 64 workgroups and merged (what caches of 1024 rows and more get by
+    """The keys of a head split over 2, 8 or 64 workgroups and merged (what caches of 800 rows and more get by
     themselves), ranges without a key included: the single-workgroup result to rounding, and float64."""
     import os
     print("attention decode ranges", (b, nh, nkv, s, d), flush=True)

@@ -291,20 +291,36 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
 
 // The ranges of one head put together: out = sum_i exp(m_i - M) o_i / sum_i exp(m_i - M) l_i, in range order.
 __global__ void __launch_bounds__(64) attention_merge_kernel(const float* __restrict__ part, float* __restrict__ dst, int nsplit, int d) {
+  // One trip to memory: lane i fetches the (maximum, sum) pair of range i while every lane already has the rows of the
+  // first eight ranges for its four columns on their way; the factors reach the columns' lanes by lane reads.
+  // nsplit <= 64 (the launcher's limit); ranges are folded in index order, the sum of the weights in the fixed
+  // butterfly order of wave_sum.
+  typedef float att_f32x2 __attribute__((ext_vector_type(2)));
   const int bh = blockIdx.x, t = threadIdx.x;
-  if (t >= (d >> 2)) return;
+  const bool col = t < (d >> 2);
   const float* pp = part + (size_t)bh * nsplit * (size_t)(d + 4);
-  float mx = -INFINITY;
-  for (int i = 0; i < nsplit; ++i) mx = fmaxf(mx, pp[(size_t)i * (d + 4)]);
-  att_f32x4 o = {0.f, 0.f, 0.f, 0.f};
-  float sum = 0.f;
-  for (int i = 0; i < nsplit; ++i) {
-    const float* pi = pp + (size_t)i * (d + 4);
-    const float f = pi[0] == -INFINITY ? 0.f : expf(pi[0] - mx);  // 0 for a range without keys
-    o += f * reinterpret_cast<const att_f32x4*>(pi + 4)[t];
-    sum += f * pi[1];
+  att_f32x4 r[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = col && j < nsplit ? reinterpret_cast<const att_f32x4*>(pp + (size_t)j * (d + 4) + 4)[t] : att_f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  if (t < nsplit) {
+    const att_f32x2 ml = *reinterpret_cast<const att_f32x2*>(pp + (size_t)t * (d + 4));
+    m = ml.x, l = ml.y;
   }
-  reinterpret_cast<att_f32x4*>(dst + (size_t)bh * d)[t] = o / sum;
+  const float mx = ughip::wave_max(m);
+  const float f = m == -INFINITY ? 0.f : expf(m - mx);  // 0 for a range without keys (and for lanes past the last range)
+  const float sum = ughip::wave_sum(f * l);
+  att_f32x4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < 8; ++j) o += __shfl(f, j, 64) * r[j];
+  for (int i0 = 8; i0 < nsplit; i0 += 8) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      r[j] = col && i0 + j < nsplit ? reinterpret_cast<const att_f32x4*>(pp + (size_t)(i0 + j) * (d + 4) + 4)[t] : att_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o += __shfl(f, (i0 + j) & 63, 64) * r[j];
+  }
+  if (col) reinterpret_cast<att_f32x4*>(dst + (size_t)bh * d)[t] = o / sum;
 }
 
 // ---- cache append for one new position ------------------------------------------------------------
@@ -725,10 +741,13 @@ int ughip_attention_decode(ughip_device* dev, const ughip_slice* q, const ughip_
 
 namespace {
 // One query position per head against s keys of caches whose heads are cap rows apart.
-// Key ranges per head for `s` keys: one below 1024 (a merge launch costs what ~800 keys cost), then enough
-// ranges to give every CU a workgroup.  UGHIP_ATT_SPLIT forces a count (tests, tuning).
+// Key ranges per head for `s` keys: one below 800 (the merge launch costs 3 us, what ~700 keys cost one workgroup),
+// four up to 1280, then eight -- never more workgroups than CUs (32 heads, measured: 768 keys 8.8 us in one range, 8.9 in
+// four; 1024 keys 10.1 / 8.9 / 9.1 in one / four / eight; 2048 keys 15.9 / 10.2 / 9.1).  UGHIP_ATT_SPLIT forces a count
+// (tests, tuning).
 int decode_ranges(size_t s, size_t heads) {
-  int n = s >= 1024 ? (int)std::max<size_t>(1, std::min<size_t>(8, 256 / std::max<size_t>(heads, 1))) : 1;
+  const size_t want = s >= 1280 ? 8 : s >= 800 ? 4 : 1;
+  int n = (int)std::max<size_t>(1, std::min<size_t>(want, 256 / std::max<size_t>(heads, 1)));
   if (const char* e = getenv("UGHIP_ATT_SPLIT")) n = atoi(e);
   return std::max(1, std::min(n, 64));
 }
