@@ -161,6 +161,14 @@ ELEMENTWISE_AND_REDUCE = [
     ("softmax_1x8193", softmax((1, 8193)), 1e-5),
     ("softmax_2x3x5x130", softmax((2, 3, 5, 130)), 1e-5),
     ("softmax_decode_1x32x1x129", softmax((1, 32, 1, 129)), 1e-5),
+    # rows shared by 3, 6 and 12 waves, and rows whose last wave is partly idle (1000, 1284) or whose length is odd or 2 mod 4
+    ("softmax_5x768", softmax((5, 768)), 1e-5),
+    ("softmax_3x1536", softmax((3, 1536)), 1e-5),
+    ("softmax_2x3072", softmax((2, 3072)), 1e-5),
+    ("softmax_3x1000", softmax((3, 1000)), 1e-5),
+    ("softmax_3x1284", softmax((3, 1284)), 1e-5),
+    ("softmax_3x770", softmax((3, 770)), 1e-5),
+    ("softmax_2x1541", softmax((2, 1541)), 1e-5),
     ("sum_dim0_300x70", reduce_dim((300, 70), "sum", 0), 2e-5),
     ("sum_dim1_70x300", reduce_dim((70, 300), "sum", 1), 2e-5),
     ("max_dim0_narrow_513x9", reduce_narrow((513, 9), "max", 0), "exact"),

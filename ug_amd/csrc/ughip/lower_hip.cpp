@@ -1038,7 +1038,8 @@ class Lowering {
   }
 
   static int pick_vec(i64 extent, i64 threads) {
-    if (extent % 4 == 0 && extent >= threads * 4) return 4;
+    // the last wave of several may be partly idle: full-width loads still win over keeping it busy
+    if (extent % 4 == 0 && (extent >= threads * 4 || (threads > 64 && extent > (threads - 64) * 4))) return 4;
     if (extent % 2 == 0 && extent >= threads * 2) return 2;
     return 1;
   }
@@ -1190,8 +1191,9 @@ class Lowering {
     } else if (width <= 256) {
       tpr = 64;
     } else {
-      tpr = 64;
-      while (tpr < 1024 && (i64)tpr * 4 < width) tpr *= 2;
+      // one 128-bit slab per thread where the row allows it: whole waves, not a power of two of them (768 columns
+      // take 3 waves; rounding up to 4 left a quarter of the threads idle and halved the width of every load)
+      tpr = (int)std::min<i64>(1024, ((width + 3) / 4 + 63) / 64 * 64);
     }
     int rows_per_block = tpr == 64 ? 4 : 1;
     if (nr < rows_per_block) rows_per_block = 1;
@@ -1279,7 +1281,7 @@ class Lowering {
     for (const Item& it : items_) any_col |= (it.deps & col_mask) != 0;
     if (any_col) {
       i64 inner = cols.empty() ? 1 : loops_[cols.back()].trip;
-      int vec = (inner % 4 == 0 && nc >= (i64)tpr * 4) ? 4 : 1;
+      int vec = (inner % 4 == 0 && pick_vec(nc, tpr) == 4) ? 4 : 1;
       o << "    for (int ug_c = ug_t; ug_c < " << nc / vec << "; ug_c += " << tpr << ") {\n";
       o << "#pragma unroll\n";
       o << "      for (int ug_u = 0; ug_u < " << vec << "; ++ug_u) {\n";
