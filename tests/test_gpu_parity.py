@@ -1078,6 +1078,15 @@ def _attention_truth(q, k, v, s, t, scale, rep):
     (1, 4, 1, 5, 300, 300, 128, True),
     (1, 32, 4, 1, 77, 128, 64, True),        # one position: the single-query kernel on a cache with spare rows
     (1, 4, 1, 1, 9, 64, 16, True),
+    # one position over long caches: the keys split into 4 ranges from 800 keys and into 8 from 1280, fewer where many heads already fill the chip
+    (1, 32, 4, 1, 799, 1024, 64, True),
+    (1, 32, 4, 1, 800, 1024, 64, True),
+    (1, 32, 4, 1, 1279, 1300, 64, True),
+    (1, 32, 4, 1, 1281, 2048, 64, True),
+    (1, 48, 8, 1, 1500, 1500, 64, True),
+    (2, 32, 8, 1, 2100, 2200, 128, True),
+    (1, 64, 8, 1, 900, 1024, 64, False),
+    (1, 128, 8, 1, 1300, 1300, 32, False),
 ])
 def test_attention_cached(hip, cpu, hip_ops, cpu_ops, interleaved, b, nh, nkv, t, s, cap, d, with_rope):
     print("attention cached", (b, nh, nkv, t, s, cap, d, with_rope, interleaved), flush=True)
