@@ -2,23 +2,26 @@
 //
 //   block tile BM x BN (256 x 256, 256 x 128 or 128 x 128), K tile 64, 4 waves laid out 2 x 2, each owning BM/2 x BN/2 of the result
 //   (any M, N a multiple of 8: a last tile hangs over the end, reads the last row again and stores what exists):
-//   16 (8, 4) accumulators of 32 x 32 live in the accumulation registers -- all 256 of them for the largest tile, which
-//   a lone wave per SIMD can have -- and leave the architectural registers to two sets of operand fragments: 8 (6, 4)
-//   fragment reads feed 16 (8, 4) MFMAs, so the 128 x 128 tile is bound by its LDS reads like the register-staged
-//   kernel and is there for products whose larger tiles would leave CUs idle
-//   global -> LDS with global_load_lds_dwordx4 (no staging registers), two 64 KiB stages; the loads of tile t+2 are
-//   spread, one in front of every other MFMA, over the quarter of tile t that follows the barrier which frees their
-//   stage and over the first quarter of tile t+1: a wave alone on its SIMD has nobody to hide a burst of 16 loads
-//   behind, and with them spread the matrix pipe never waits for the issue of a memory instruction
+//   (BM / 32) x (BN / 32) accumulators of 16 x 16 (v_mfma_f32_16x16x32: 4 registers each) live in the accumulation
+//   registers -- all 256 of them for the largest tile, which a lone wave per SIMD can have -- and leave the
+//   architectural registers to two sets of operand fragments; a K tile is two steps of 32: 16 (12, 8) fragment reads
+//   feed 64 (32, 16) MFMAs, so the 128 x 128 tile is bound by its LDS reads like the register-staged kernel and is
+//   there for products whose larger tiles would leave CUs idle.  The 16 x 16 x 32 shape moves a fifth less through the
+//   register file per flop than 32 x 32 x 16 (half the accumulator traffic, twice the operand traffic); under this
+//   kernel the chip is held back by power, and the same schedule on the larger shape ran 5-6 % slower.
+//   global -> LDS with global_load_lds_dwordx4 (no staging registers), two 64 KiB stages.  The address unit of a CU
+//   needs 16 cycles per such instruction and a K tile takes 64 of them, half the tile's time: they are dealt one by one
+//   in front of MFMAs over as much of the tile as the stage they fill allows (see the two schedules in the kernel)
 //   rhs [n, k]-major: operand fragments are 128-bit LDS reads of k-contiguous rows (XOR-swizzled chunks, conflict free);
 //   rhs [k, n]-major: the tile stays [k][n] in LDS and ds_read_b64_tr_b16 hands every lane 4 consecutive k of its own
 //   column, so no transposing pass through registers is needed
 //   the MFMA operands are swapped (B fragment first): a lane then holds 4 consecutive columns of one result row, the
 //   epilogue packs them and goes through LDS so that the result leaves in 16-byte pieces of whole rows
 //
-// What bounds it: power.  With U(-1, 1) operands the chip runs this kernel at about 1.4 GHz of its 2.4 GHz (shader
-// clock against the 100 MHz reference, read in the kernel), and the matrix pipes are busy 80-90 % of those cycles
-// (SQ_VALU_MFMA_BUSY_CYCLES against SQ_WAVE_CYCLES: 83 % of a wave's whole residency at 4096^3).
+// What bounds it: power first, then the address unit.  With U(-1, 1) operands the chip runs this kernel at 1.4-1.8 GHz
+// of its 2.4 GHz by box (CU busy cycles against the kernel's duration), and the matrix pipes are busy 80 % of those
+// cycles at 8192^3 (89 % with the DMAs taken out, 92 % with the fragment reads taken out as well: the loads cost MFMA
+// issue slots, not waiting time -- warming L2 ahead of them or four stages of 32 k instead of two of 64 made it slower).
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -33,18 +36,18 @@
 namespace ughip {
 namespace {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ floatx16 mma(__bf16, const u32x4& a, const u32x4& b, const floatx16& c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ floatx4 mma16(__bf16, const u32x4& a, const u32x4& b, const floatx4& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
-__device__ __forceinline__ floatx16 mma(_Float16, const u32x4& a, const u32x4& b, const floatx16& c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+__device__ __forceinline__ floatx4 mma16(_Float16, const u32x4& a, const u32x4& b, const floatx4& c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
 }
 
 // s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8)
@@ -71,16 +74,15 @@ __device__ __forceinline__ int kn_byte(int k, int n) {
   return k * (BN * 2) + (((n >> 5) ^ (k & (BN / 32 - 1))) << 6) + (n & 31) * 2;
 }
 
-template <typename T, int BM, int BN, bool B_KN>
+// Lane l feeds row / column l % 16, k = 8 (l / 16) .. + 7 of a step of 32.  TWO: the schedule with two barriers per K tile.
+template <typename T, int BM, int BN, bool B_KN, bool TWO>
 __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tiles_n) {
   extern __shared__ u32x4 lds[];
-  constexpr int NI = BM / 64, NJ = BN / 64;            // 32-row and 32-column fragments per wave
-  constexpr int NM = NI * NJ;                          // MFMAs per k16 step
+  constexpr int NI = BM / 32, NJ = BN / 32;            // 16-row and 16-column fragments per wave
+  constexpr int NM = NI * NJ;                          // MFMAs per k32 step
   constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2, STAGE_BYTES = A_BYTES + B_BYTES;
   constexpr int NDA = BM / 32, NDB = BN / 32, ND = NDA + NDB;  // DMA instructions per wave and K tile
-  constexpr int H = ND / 2;                            // ... per step that carries them
   constexpr int R = NI + NJ;                           // fragment reads per step
-  static_assert(R == H, "reads and DMAs of a step alternate one for one");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
@@ -108,7 +110,6 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
   const int KT = p.K / BK;
   const int wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
   const unsigned lds_addr = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
-
   // per-lane byte offsets of this wave's DMA instructions (the same for every K tile; the scalar base moves)
   unsigned voff[ND];
   // a last tile may hang over the end of M or N: rows past the end fetch the last row again (their results are not
@@ -141,37 +142,32 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
     else dma16(Bb + tile * b_step, voff[idx], st + A_BYTES + ((idx - NDA) * 4 + wave) * 1024);
   };
 
-  floatx16 acc[NI][NJ];
+  floatx4 acc[NI][NJ];
 #pragma unroll
   for (int i = 0; i < NI; ++i)
 #pragma unroll
-    for (int j = 0; j < NJ; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    for (int j = 0; j < NJ; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  // operand fragments of one k16 step, two sets: lane l feeds row / column l % 32, k = 8 (l / 32) .. + 7
   u32x4 fa[2][NI], fb[2][NJ];
-  auto read_frag = [&](int stage, int s, int idx, int set) {  // idx < NI: A fragment idx, else B fragment idx - NI
+  auto read_frag = [&](int stage, int s, int idx, int set) {
     if (idx < NI) {
-      fa[set][idx] = lds[stage * (STAGE_BYTES / 16) + kc_idx(wm + idx * 32 + (lane & 31), 2 * s + (lane >> 5))];
+      fa[set][idx] = lds[stage * (STAGE_BYTES / 16) + kc_idx(wm + idx * 16 + (lane & 15), 4 * s + (lane >> 4))];
     } else if (!B_KN) {
-      fb[set][idx - NI] = lds[stage * (STAGE_BYTES / 16) + A_BYTES / 16 + kc_idx(wn + (idx - NI) * 32 + (lane & 31), 2 * s + (lane >> 5))];
+      fb[set][idx - NI] = lds[stage * (STAGE_BYTES / 16) + A_BYTES / 16 + kc_idx(wn + (idx - NI) * 16 + (lane & 15), 4 * s + (lane >> 4))];
     } else {
-      // A transposing read returns to lane i of a 16-lane group the 4 values at column i % 4 of the rows that lanes
-      // i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12 name.  Lane q + 4 e names row kbase + e, columns 4 q .. 4 q + 3 of its
-      // group's 16, so lane i receives k = kbase .. kbase + 3 of column i; two reads give the 8 consecutive k of the
-      // MFMA operand.  Groups 0, 1 hold k 0..7 of columns 0..15 and 16..31, groups 2, 3 hold k 8..15.
+      // lane q + 4 e of a 16-lane group names row k0 + e, columns 4 q .. 4 q + 3 of the fragment's 16: lane i receives
+      // k0 .. k0 + 3 of column i; group g takes k = 8 g .. 8 g + 7 of the step in two such reads
       typedef __attribute__((address_space(3))) s16x4 lds_v4;
       const int g = lane >> 4, li = lane & 15, q = li & 3, e = li >> 2;
       const char __attribute__((address_space(3)))* Bs = (const char __attribute__((address_space(3)))*)lds + stage * STAGE_BYTES + A_BYTES;
-      const int n = wn + (idx - NI) * 32 + 16 * (g & 1) + 4 * q, k0 = s * 16 + 8 * (g >> 1) + e;
+      const int n = wn + (idx - NI) * 16 + 4 * q, k0 = s * 32 + 8 * g + e;
       const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4*)(Bs + kn_byte<BN>(k0, n))));
       const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4*)(Bs + kn_byte<BN>(k0 + 4, n))));
       fb[set][idx - NI] = u32x4{lo.x, lo.y, hi.x, hi.y};
     }
   };
 
-  // prologue: tiles 0 and 1 requested, tile 0 landed (tile 1 is waited for at the barrier of tile 0's last step)
+  // prologue: tiles 0 and 1 requested, tile 0 landed (tile 1 is waited for at the first barrier that publishes it)
 #pragma unroll
   for (int i = 0; i < ND; ++i) dma(0, i);
 #pragma unroll
@@ -181,70 +177,123 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
 #pragma unroll
   for (int i = 0; i < R; ++i) read_frag(0, 0, i, 0);
 
-  // One K tile = 4 steps of NM MFMAs.  The memory instructions of a step -- the R fragment reads of the next step,
-  // then (D3: in step 3, D0: in step 0) one half of the DMAs that refill the stage everybody left at the barrier of
-  // step 3 -- are dealt evenly in front of the MFMAs.  RN: there is a next tile to read fragments from.
-  auto tile = [&](int kt, auto d0, auto d3, auto rn) {
-    constexpr bool D0 = decltype(d0)::value, D3 = decltype(d3)::value, RN = decltype(rn)::value;
+  // One barrier per K tile.  Step 0 carries the fragment reads of step 1; step 1 starts behind the barrier that frees
+  // this tile's stage and carries the reads of the next tile's step 0 (RN) and all the DMAs of tile kt + 2 (D), which
+  // then have a whole step's time to land.  (The memory instructions are pinned one by one in front of MFMAs: a wave
+  // alone on its SIMD has nobody to hide a burst of loads behind.)
+  auto tile_one = [&](int kt, auto d, auto rn) {
+    constexpr bool D = decltype(d)::value, RN = decltype(rn)::value;
     const int cur = kt & 1, nxt = cur ^ 1;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const int fc = s & 1, fn = fc ^ 1;
-      if (s == 3) {
-        // this wave's share of tile kt+1 has landed and its reads of stage cur are done; then everyone's
+    for (int s = 0; s < 2; ++s) {
+      const int fc = s, fn = s ^ 1;
+      if (s == 1) {
         wait_vmcnt<0>();
         wait_lgkmcnt0();
         __builtin_amdgcn_s_barrier();
       }
-      const bool reads = s < 3 || RN, dmas = (s == 3 && D3) || (s == 0 && D0);
-      const int n_ops = (reads ? R : 0) + (dmas ? H : 0);
+      const int n_reads = (s == 0 || RN) ? R : 0, n_dmas = (s == 1 && D) ? ND : 0;
+      const int n_ops = n_reads + n_dmas;
 #pragma unroll
       for (int g = 0; g < NM; ++g) {
+        // the memory instructions in front of MFMA g: those t with t * NM / n_ops == g
+        constexpr int PER = (R + ND + NM - 1) / NM;
+        const int t_lo = (g * n_ops + NM - 1) / NM, t_hi = ((g + 1) * n_ops + NM - 1) / NM;
 #pragma unroll
-        for (int t = 0; t < R + H; ++t) {
-          if (t < n_ops && t * NM / n_ops == g) {
-            // in a step with both kinds they alternate: read, DMA, read, DMA, ...
-            const bool both = reads && dmas;
-            const bool is_read = both ? (t & 1) == 0 && t / 2 < R : reads;
-            const int ri = both ? t / 2 : t, di = both ? ((t & 1) ? t / 2 : 0) : t;
-            if (is_read) read_frag(s < 3 ? cur : nxt, s < 3 ? s + 1 : 0, ri, fn);
-            else if (s == 3) dma(kt + 2, di);
-            else dma(kt + 1, H + di);
+        for (int u = 0; u < PER; ++u) {
+          const int t = t_lo + u;
+          if (t < t_hi) {
+            // reads and DMAs of a step are dealt in proportion: op t is DMA number t * n_dmas / n_ops when that number moves
+            const int di = t * n_dmas / n_ops, di_next = (t + 1) * n_dmas / n_ops;
+            const bool is_dma = di_next > di;
+            const int ri = t - di;
+            if (is_dma) dma(kt + 2, di);
+            else read_frag(s == 0 ? cur : nxt, s == 0 ? 1 : 0, ri, fn);
           }
         }
         const int i = g / NJ, j = g % NJ;
-        acc[i][j] = mma(T(), fb[fc][j], fa[fc][i], acc[i][j]);  // operands swapped: rows of the block are columns of C
+        acc[i][j] = mma16(T(), fb[fc][j], fa[fc][i], acc[i][j]);  // operands swapped: rows of the block are columns of C
         __builtin_amdgcn_sched_barrier(0);
       }
     }
   };
+  // Two barriers per K tile, so that the DMAs need not all come in one step (64 x 16 cycles of the address unit
+  // against the 1024 cycles of a step's MFMAs): 2-3 % faster with an [n, k]-major rhs.  Step 0 reads the fragments of
+  // step 1 in front of its first R MFMAs; barrier A, in front of MFMA BAR, then says that nobody reads this tile's
+  // stage any more, and the DMAs of tile kt + 2 go out from there to the end of step 1, evenly (EARLY of them in
+  // step 0).  Barrier B, at the head of step 1, says that tile kt + 1 has landed (its last DMA went out a whole step
+  // ago; the EARLY ones behind it may still be on their way).
+  auto tile_two = [&](int kt, auto d, auto rn) {
+    constexpr bool D = decltype(d)::value, RN = decltype(rn)::value;
+    constexpr int BAR = (R + 4 > NM * 3 / 8 ? R + 4 : NM * 3 / 8) < NM - 1 ? (R + 4 > NM * 3 / 8 ? R + 4 : NM * 3 / 8) : NM - 1;
+    constexpr int EARLY = ND * (NM - BAR) / (2 * NM - BAR);
+    const int cur = kt & 1, nxt = cur ^ 1;
+#pragma unroll
+    for (int g = 0; g < NM; ++g) {
+      if (g < R) read_frag(cur, 1, g, 1);
+      if (g == BAR) {
+        wait_lgkmcnt0();
+        __builtin_amdgcn_s_barrier();
+      }
+      if (D && g > BAR && EARLY > 0) {
+        const int e = (g - BAR - 1) * EARLY / (NM - BAR - 1), e_next = (g - BAR) * EARLY / (NM - BAR - 1);
+        if (e_next > e && e < EARLY) dma(kt + 2, e);
+      }
+      const int i = g / NJ, j = g % NJ;
+      acc[i][j] = mma16(T(), fb[0][j], fa[0][i], acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (RN) {
+      if (D) wait_vmcnt<EARLY>();
+      else wait_vmcnt<0>();
+      __builtin_amdgcn_s_barrier();
+    }
+    const int n_reads = RN ? R : 0, n_dmas = D ? ND - EARLY : 0;
+    const int n_ops = n_reads + n_dmas;
+#pragma unroll
+    for (int g = 0; g < NM; ++g) {
+      constexpr int PER = (R + ND + NM - 1) / NM;
+      const int t_lo = (g * n_ops + NM - 1) / NM, t_hi = ((g + 1) * n_ops + NM - 1) / NM;
+#pragma unroll
+      for (int u = 0; u < PER; ++u) {
+        const int t = t_lo + u;
+        if (t < t_hi) {
+          const int di = t * n_dmas / n_ops, di_next = (t + 1) * n_dmas / n_ops;
+          if (di_next > di) dma(kt + 2, EARLY + di);
+          else read_frag(nxt, 0, t - di, 0);
+        }
+      }
+      const int i = g / NJ, j = g % NJ;
+      acc[i][j] = mma16(T(), fb[1][j], fa[1][i], acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto tile = [&](int kt, auto d, auto rn) {
+    if constexpr (TWO) tile_two(kt, d, rn);
+    else tile_one(kt, d, rn);
+  };
   using Y = std::true_type;
   using N_ = std::false_type;
-  tile(0, N_(), Y(), Y());  // tile 1 went out whole in the prologue
-  for (int kt = 1; kt < KT - 2; ++kt) tile(kt, Y(), Y(), Y());
-  tile(KT - 2, Y(), N_(), Y());
-  tile(KT - 1, N_(), N_(), N_());
+  for (int kt = 0; kt < KT - 2; ++kt) tile(kt, Y(), Y());
+  tile(KT - 2, N_(), Y());
+  tile(KT - 1, N_(), N_());
 
-  // Epilogue through LDS (nobody reads a stage after the last barrier, no load is in flight).  Accumulator register r of
-  // lane l of block (i, j): column of C  wn + 32 j + 8 (r / 4) + 4 (l / 32) + r % 4,  row  wm + 32 i + l % 32: four
-  // consecutive columns per register quad.  Row pitch BN * 2 + 8 bytes: 32 lanes of consecutive rows hit 64 banks once.
+  // Epilogue through LDS.  Register e of lane l of block (i, j): row wm + 16 i + l % 16, column wn + 16 j + 4 (l / 16) + e.
   constexpr int PITCH = BN * 2 + 8;
   char __attribute__((address_space(3)))* Cs = (char __attribute__((address_space(3)))*)lds;
 #pragma unroll
   for (int i = 0; i < NI; ++i)
 #pragma unroll
-    for (int j = 0; j < NJ; ++j)
+    for (int j = 0; j < NJ; ++j) {
+      typedef T tx4 __attribute__((ext_vector_type(4)));
+      tx4 v;
 #pragma unroll
-      for (int rq = 0; rq < 4; ++rq) {
-        typedef T tx4 __attribute__((ext_vector_type(4)));
-        tx4 v;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = (T)acc[i][j][rq * 4 + e];
-        const int row = wm + i * 32 + (lane & 31), col = wn + j * 32 + rq * 8 + (lane >> 5) * 4;
-        *(u32x2 __attribute__((address_space(3)))*)(Cs + row * PITCH + col * 2) = __builtin_bit_cast(u32x2, v);
-      }
+      for (int e = 0; e < 4; ++e) v[e] = (T)acc[i][j][e];
+      const int row = wm + i * 16 + (lane & 15), col = wn + j * 16 + (lane >> 4) * 4;
+      *(u32x2 __attribute__((address_space(3)))*)(Cs + row * PITCH + col * 2) = __builtin_bit_cast(u32x2, v);
+    }
   __syncthreads();
-  constexpr int CPR = BN / 8, RPP = 256 / CPR;  // 16-byte chunks per row, rows per pass of the workgroup
+  constexpr int CPR = BN / 8, RPP = 256 / CPR;
   T* __restrict__ C = static_cast<T*>(p.c) + (size_t)batch * p.c_bs + (size_t)m0 * p.N + n0;
   const int c = tid % CPR, r0 = tid / CPR;
 #pragma unroll 4
@@ -261,7 +310,10 @@ hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch) {
   constexpr int STAGES = 2 * (BM + BN) * BK * 2, EPI = BM * (BN * 2 + 8);
   constexpr int LDS_BYTES = STAGES > EPI ? STAGES : EPI;
   static std::atomic<unsigned long long> configured{0};  // one bit per device: the attribute is per device
-  auto kernel = gemm_dma4<T, BM, BN, B_KN>;
+  // the schedule with two barriers, except where it does not fit the registers (the transposing reads of the
+  // largest tile need pairs of temporaries: 256 registers and spills)
+  constexpr bool TWO = !(B_KN && BM == 256 && BN == 256);
+  auto kernel = gemm_dma4<T, BM, BN, B_KN, TWO>;
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev)) return e;
   const unsigned long long bit = dev < 64 ? 1ull << dev : 0;
