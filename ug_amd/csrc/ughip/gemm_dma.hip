@@ -62,6 +62,11 @@ __device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc
 __device__ __forceinline__ void dma16(const void* base, unsigned voff, unsigned lds_byte_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
 }
+// The same in two halves with an MFMA between them as the wait state that the write of M0 needs.
+__device__ __forceinline__ void dma16_m0(unsigned lds_byte_addr, unsigned stage_offset) {
+  asm volatile("s_add_u32 m0, %0, %1" : : "s"(lds_byte_addr), "s"(stage_offset) : "memory", "scc");
+}
+__device__ __forceinline__ void dma16_go(const void* base, unsigned voff) { asm volatile("global_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base) : "memory"); }
 
 constexpr int BK = 64;
 
@@ -141,6 +146,14 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
     if (idx < NDA) dma16(Ab + tile * a_step, voff[idx], st + (idx * 4 + wave) * 1024);
     else dma16(Bb + tile * b_step, voff[idx], st + A_BYTES + ((idx - NDA) * 4 + wave) * 1024);
   };
+  auto dma_m0 = [&](int tile, int idx) {
+    const unsigned in_stage = lds_addr + (idx < NDA ? (idx * 4 + wave) * 1024 : A_BYTES + ((idx - NDA) * 4 + wave) * 1024);  // loop invariant
+    dma16_m0(in_stage, (tile & 1) * STAGE_BYTES);
+  };
+  auto dma_go = [&](int tile, int idx) {
+    if (idx < NDA) dma16_go(Ab + tile * a_step, voff[idx]);
+    else dma16_go(Bb + tile * b_step, voff[idx]);
+  };
 
   floatx4 acc[NI][NJ];
 #pragma unroll
@@ -198,6 +211,7 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
       for (int g = 0; g < NM; ++g) {
         // the memory instructions in front of MFMA g: those t with t * NM / n_ops == g
         constexpr int PER = (R + ND + NM - 1) / NM;
+        static_assert(PER == 1, "at most one memory instruction per MFMA: M0 is written one MFMA ahead of its DMA");
         const int t_lo = (g * n_ops + NM - 1) / NM, t_hi = ((g + 1) * n_ops + NM - 1) / NM;
 #pragma unroll
         for (int u = 0; u < PER; ++u) {
@@ -207,13 +221,21 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
             const int di = t * n_dmas / n_ops, di_next = (t + 1) * n_dmas / n_ops;
             const bool is_dma = di_next > di;
             const int ri = t - di;
-            if (is_dma) dma(kt + 2, di);
+            if (is_dma) dma_m0(kt + 2, di);  // M0 in front of this MFMA, the load behind it: the MFMA is the wait state M0 needs
             else read_frag(s == 0 ? cur : nxt, s == 0 ? 1 : 0, ri, fn);
           }
         }
         const int i = g / NJ, j = g % NJ;
         acc[i][j] = mma16(T(), fb[fc][j], fa[fc][i], acc[i][j]);  // operands swapped: rows of the block are columns of C
         __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+          const int t = t_lo + u;
+          if (t < t_hi) {
+            const int di = t * n_dmas / n_ops, di_next = (t + 1) * n_dmas / n_ops;
+            if (di_next > di) dma_go(kt + 2, di);
+          }
+        }
       }
     }
   };
@@ -227,6 +249,7 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
     constexpr bool D = decltype(d)::value, RN = decltype(rn)::value;
     constexpr int BAR = (R + 4 > NM * 3 / 8 ? R + 4 : NM * 3 / 8) < NM - 1 ? (R + 4 > NM * 3 / 8 ? R + 4 : NM * 3 / 8) : NM - 1;
     constexpr int EARLY = ND * (NM - BAR) / (2 * NM - BAR);
+    static_assert(R + ND - EARLY <= NM, "at most one memory instruction per MFMA: M0 is written one MFMA ahead of its DMA");
     const int cur = kt & 1, nxt = cur ^ 1;
 #pragma unroll
     for (int g = 0; g < NM; ++g) {
@@ -236,12 +259,17 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
         __builtin_amdgcn_s_barrier();
       }
       if (D && g > BAR && EARLY > 0) {
+        // DMA e goes out in front of the MFMA after this one; M0 is written in front of this one
         const int e = (g - BAR - 1) * EARLY / (NM - BAR - 1), e_next = (g - BAR) * EARLY / (NM - BAR - 1);
-        if (e_next > e && e < EARLY) dma(kt + 2, e);
+        if (e_next > e && e < EARLY) dma_m0(kt + 2, e);
       }
       const int i = g / NJ, j = g % NJ;
       acc[i][j] = mma16(T(), fb[0][j], fa[0][i], acc[i][j]);
       __builtin_amdgcn_sched_barrier(0);
+      if (D && g > BAR && EARLY > 0) {
+        const int e = (g - BAR - 1) * EARLY / (NM - BAR - 1), e_next = (g - BAR) * EARLY / (NM - BAR - 1);
+        if (e_next > e && e < EARLY) dma_go(kt + 2, e);
+      }
     }
     if (RN) {
       if (D) wait_vmcnt<EARLY>();
@@ -259,13 +287,21 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
         const int t = t_lo + u;
         if (t < t_hi) {
           const int di = t * n_dmas / n_ops, di_next = (t + 1) * n_dmas / n_ops;
-          if (di_next > di) dma(kt + 2, EARLY + di);
+          if (di_next > di) dma_m0(kt + 2, EARLY + di);
           else read_frag(nxt, 0, t - di, 0);
         }
       }
       const int i = g / NJ, j = g % NJ;
       acc[i][j] = mma16(T(), fb[1][j], fa[1][i], acc[i][j]);
       __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < PER; ++u) {
+        const int t = t_lo + u;
+        if (t < t_hi) {
+          const int di = t * n_dmas / n_ops, di_next = (t + 1) * n_dmas / n_ops;
+          if (di_next > di) dma_go(kt + 2, EARLY + di);
+        }
+      }
     }
   };
   auto tile = [&](int kt, auto d, auto rn) {
