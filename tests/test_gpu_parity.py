@@ -423,7 +423,8 @@ def test_matmul_16bit_one_wave_per_simd_random_shapes(hip, monkeypatch):
     ((8, 1024, 1024, 1024), "gemm_dma4<bf16,NT,256x128,256t>"),      # 128 such tiles: the narrower one fills the chip
     ((1, 3072, 4096, 1024), "gemm_dma4<bf16,NT,256x256,256t>"),      # 192 tiles: three quarters of the chip at a higher clock
     ((1, 2048, 2560, 2048), "gemm_dma4<bf16,NT,128x128,256t>"),      # 160 tiles of 256 x 128 leave a third of the chip idle, 320 of 128 x 128 share the CUs two by two
-    ((1, 2048, 2048, 5632), "gemm_tiled<bf16,NT,128x128,256t>"),     # 128 narrow tiles and a long K: the register-staged kernel
+    ((1, 2048, 2048, 5632), "gemm_dma4<bf16,NT,128x128,256t>"),      # 128 narrow tiles and a long K: 256 tiles of 128 x 128, one per CU
+    ((1, 2048, 2048, 2048), "gemm_tiled<bf16,NT,128x128,256t>"),     # the same tiles and a short K: the register-staged kernel is as fast and keeps the product
     ((1, 1024, 1024, 1024), "gemm_tiled<"),                          # a handful of tiles: K split
 ])
 def test_matmul_16bit_kernel_choice(hip, bmnk, want):

@@ -413,7 +413,9 @@ double gemm_dma_cost_us(const MMArgs& p, size_t batch, int tile) {
   const int kt = p.K / BK;
   const bool nn = p.b_cs == 1 && p.b_rs != 1;
   double us = 4.0 + (double)batch * p.M * p.N * 2 / 6.4e6;
-  const double layout = nn ? 1.08 : 1.0;
+  // (the figures below were fitted to the kernel on 32 x 32 x 16 MFMAs; on 16 x 16 x 32 and with the loads spread behind two
+  // barriers every K tile takes 8 % less: 4096^3 97 us, 8 x 1024^3 18.8, 1024 x 4096^2 41 on 128 x 128 tiles)
+  const double layout = (nn ? 1.08 : 1.0) * 0.92;
   if (tile == 64) {
     // two workgroups share a CU: a round is 512 tiles at 0.88 us per K tile; up to 256 tiles run one per CU at
     // 0.47 + 0.16 x busy, the next 256 fill the second slots (2048^3 24.7 us, 2304^3 31.3, 2816^3 45.5, 5120^2 x 1024 61)
