@@ -510,7 +510,7 @@ def bmm(dev, steps, warmup):
             cs.run()
             kernel = ug_amd.last_kernel()
             chk = check_product_rows(key, lb.data_vec().reshape(1, t, n), xh.reshape(1, t, k), np.swapaxes(wh.reshape(1, n, k), 1, 2), k, False, rows=(0, 1, 63, 64, 127))
-            _, ms = timed(dev, cs.run, steps, warmup)
+            _, ms = timed_hot(dev, cs.run, steps, warmup, 0.1)
             tf = 2.0 * t * n * k * steps / (ms * 1e-3) / 1e12
             out[key] = {"TFLOP/s": round(tf, 2), "frac_mfma_f32": round(tf / MFMA_F32_PEAK_TF, 4), "us": round(ms * 1e3 / steps, 1), "kernel": kernel, "verified": chk}
     return out
@@ -595,7 +595,7 @@ def llama_pieces(dev, steps, warmup):
         cs.run()
         chk = check_product_rows(name, mm.data_vec().reshape(b, m, n), a_h.reshape(b, m, k), w_kn.reshape(b, k, n), k, False, rows=(0, 1, 255, 256, 511))
         kernel = ug_amd.last_kernel()
-        _, ms = timed(dev, cs.run, steps, warmup)
+        _, ms = timed_hot(dev, cs.run, steps, warmup, 0.1)
         flop, nbytes = 2.0 * b * m * n * k, 4.0 * b * (m * k + k * n + m * n)
         sec = ms * 1e-3 / steps
         out[name] = {"TFLOP/s": round(flop / sec / 1e12, 2), "frac_mfma_f32": round(flop / sec / 1e12 / MFMA_F32_PEAK_TF, 4), "GB/s": round(nbytes / sec / 1e9, 1),
@@ -626,7 +626,7 @@ def llama_pieces(dev, steps, warmup):
         kv = h // (heads // nkv)
         p = softmax64(np.where(keep, qr @ kch[0, kv, :t].astype(np.float64).T * scale, -np.inf))
         verify(f"c4_attention_cached head {h}", got[:, h], p @ vch[0, kv, :t].astype(np.float64), rtol=0, atol=2e-5 * float(np.abs(got).max()))
-    _, ms = timed(dev, cs.run, steps, warmup)
+    _, ms = timed_hot(dev, cs.run, steps, warmup, 0.1)
     sec = ms * 1e-3 / steps
     flop = 2 * 2.0 * heads * hd * t * (t + 1) / 2
     nbytes = 4.0 * (2 * t * heads * hd + 2 * nkv * t * hd)
