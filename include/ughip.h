@@ -394,7 +394,9 @@ int ughip_gemv_add(ughip_device* dev, const ughip_slice* x, const ughip_slice* w
  *                         three planes by the matrix as it is stored: every product term is exact in f32, the sums are f32
  *                         sums in another order than the f32 pipe's, and three bf16 MFMAs replace eight times their work in
  *                         f32 ones.  Same accuracy class as the F32 product (k eps bound), not bit-identical to it.
- *                         Needs k % 64 == 0 and a BF16 matrix.
+ *                         Needs k % 64 == 0 and a BF16 matrix.  Products of many rows (a prompt of several hundred
+ *                         positions and more) run the planes on the one-wave-per-SIMD 16-bit kernel, whichever of the two
+ *                         is priced cheaper; the terms are the same, the order of the sums is that kernel's.
  * ughip_linear_rows: dst[m, n] = x w^T.
  * ughip_linear_add_rows: dst[m, n] = x w^T + residual[m, n]; dst may be residual itself (every element is read,
  * then written, by one thread).

@@ -1558,6 +1558,72 @@ def test_projections_of_several_rows_as_three_bf16_terms(hip, t, k, n):
         np.testing.assert_array_equal(back[:, :k], full)
 
 
+@pytest.mark.parametrize("t,k,n,force", [(300, 512, 640, "3"), (300, 512, 640, "4"), (300, 512, 640, "5"), (517, 256, 264, "5"), (260, 1024, 1032, "4"),
+                                         (1900, 2048, 2560, None), (1100, 2048, 2048, None)])
+def test_three_bf16_terms_on_the_one_wave_per_simd_kernel(hip, monkeypatch, t, k, n, force):
+    """Many rows of three bf16 planes take gemm_dma4 (f32 result straight from the accumulators, the residual added on the
+    way, SwiGLU through the scratch block and the fold).  Forced tiles on small ragged shapes, the library's own choice on
+    prompts of a thousand positions and more; against float64 with the k eps bound of the f32 product, against the
+    register-staged kernel (UGHIP_X3_DMA=0: the same exact terms, sums in another order), small integers exactly, and a
+    sentinel behind every result."""
+    import ctypes as C
+    print("three bf16 terms, one wave per SIMD", t, k, n, force, flush=True)
+    x = rng.normal(171, t * k)
+    w = rng.bf16_round(rng.normal(172, n * k, 0.05))
+    wgu = rng.bf16_round(rng.normal(173, 2 * n * k, 0.05))
+    r = rng.normal(174, t * n)
+    bits = rng.to_bf16_bits
+    lib, dev, z = ug_amd.ughip_lib(), C.c_void_p(hip.raw_hip()), C.c_size_t
+    raw = lambda s_: C.c_void_p(s_.raw())
+
+    def run(xv, wv, guv):
+        sx, sw, sgu, sr = hip.slice_from(xv), hip.slice_from(bits(wv)), hip.slice_from(bits(guv)), hip.slice_from(r)
+        guard = 64
+        d = hip.slice_from(np.full(t * n + guard, 7.0, np.float32))
+        out, kerns = [], []
+        for call in (lambda: lib.ughip_linear_rows(dev, raw(sx), raw(sw), raw(d), z(t), z(n), z(k), C.c_int(1)),
+                     lambda: lib.ughip_linear_add_rows(dev, raw(sx), raw(sw), raw(sr), raw(d), z(t), z(n), z(k), C.c_int(1)),
+                     lambda: lib.ughip_linear_swiglu_rows(dev, raw(sx), raw(sgu), raw(d), z(t), z(n), z(k), C.c_int(1))):
+            assert call() == 0, lib.ughip_last_error()
+            kerns.append(ug_amd.last_kernel())
+            v = d.to_vec()
+            assert np.all(v[t * n:] == 7.0), "wrote past the end of the result"
+            out.append(v[:t * n].reshape(t, n).copy())
+        return out, kerns
+
+    if force:
+        monkeypatch.setenv("UGHIP_X3_DMA", force)
+    (lin, add, glu), kerns = run(x, w, wgu)
+    tile = {"3": "256x256", "4": "256x128", "5": "128x128"}.get(force, "")
+    for kn, tail in zip(kerns, ("f32 out>", "+residual>", "swiglu fold>")):
+        assert kn.startswith("gemm_dma4<bf16,NT," + tile) and "3 planes" in kn and kn.endswith(tail), kn
+    monkeypatch.setenv("UGHIP_X3_DMA", "0")
+    (lin0, add0, glu0), kerns0 = run(x, w, wgu)
+    assert all(kn.startswith("gemm_tiled<bf16,NT,") for kn in kerns0), kerns0
+    x64, w64, gu64 = x.reshape(t, k).astype(np.float64), w.reshape(n, k).astype(np.float64), wgu.reshape(2 * n, k).astype(np.float64)
+    eps = float(np.finfo(np.float32).eps)
+    lin64 = x64 @ w64.T
+    bound = k * eps * (np.abs(x64) @ np.abs(w64).T) + 1e-7
+    assert np.all(np.abs(lin - lin64) <= bound)
+    assert np.all(np.abs(add - (lin64 + r.reshape(t, n))) <= bound + 2 * eps * np.abs(lin64 + r.reshape(t, n)))
+    gg, uu = x64 @ gu64[:n].T, x64 @ gu64[n:].T
+    g64 = gg / (1.0 + np.exp(-gg)) * uu
+    g_bound = k * eps * ((np.abs(x64) @ np.abs(gu64[:n]).T) * (np.abs(uu) * 1.3) + (np.abs(x64) @ np.abs(gu64[n:]).T) * np.abs(gg / (1.0 + np.exp(-gg)))) + 8 * eps * np.abs(g64) + 1e-7
+    assert np.all(np.abs(glu - g64) <= g_bound)
+    assert np.max(np.abs(lin - lin0)) <= 0.25 * np.max(bound) and np.max(np.abs(add - add0)) <= 0.25 * np.max(bound) + 2 * eps * np.abs(add0).max()
+    assert np.all(np.abs(glu - glu0) <= 2 * g_bound)
+    # small integers: every partial sum is exact
+    if force:
+        monkeypatch.setenv("UGHIP_X3_DMA", force)
+    else:
+        monkeypatch.delenv("UGHIP_X3_DMA")
+    xi, wi, gui = np.floor(x * 4).astype(np.float32), np.floor(w * 40).astype(np.float32), np.floor(wgu * 40).astype(np.float32)
+    (lin_i, add_i, _), kerns_i = run(xi, wi, gui)
+    assert kerns_i[0].startswith("gemm_dma4<"), kerns_i
+    want = (xi.reshape(t, k).astype(np.float64) @ wi.reshape(n, k).astype(np.float64).T).astype(np.float32)
+    np.testing.assert_array_equal(lin_i, want)
+
+
 def test_projections_of_several_rows_random_shapes(hip):
     """Straight through the C ABI over 30 seeded shapes (rows the tiles do not divide, column counts that leave a last
     tile partly empty, one to sixteen K tiles), both products, the three forms: against float64 with the k eps bound, and

@@ -50,5 +50,10 @@ bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int tile);
 hipError_t gemm_dma_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, int tile);
 // The tile code this kernel should take the problem with, 0 when another kernel should.
 int gemm_dma_pick(int dtype, const MMArgs& p, size_t batch);
+// The same kernel on three bf16 planes of f32 rows (p.K = 3 k, p.b_k_div = 3, [n, k]-major bf16 matrix): f32 result, residual added when given.
+hipError_t gemm_dma_launch_planes3(hipStream_t stream, const MMArgs& p, int tile, const float* residual, bool swiglu_fold_follows);
+// c[m, n / 2] = silu(product[:, :n / 2]) * product[:, n / 2:] for an f32 product [m, n] (n % 8 == 0): the fold of the tiled kernel on one slab.
+hipError_t gemm_swiglu_fold(hipStream_t stream, const float* product, float* c, size_t m, size_t n);
+double gemm_dma_cost_us(const MMArgs& p, size_t batch, int tile);
 
 }  // namespace ughip

@@ -80,8 +80,12 @@ __device__ __forceinline__ int kn_byte(int k, int n) {
 }
 
 // Lane l feeds row / column l % 16, k = 8 (l / 16) .. + 7 of a step of 32.  TWO: the schedule with two barriers per K tile.
-template <typename T, int BM, int BN, bool B_KN, bool TWO>
-__global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tiles_n) {
+// F32OUT: the result leaves as f32 straight from the accumulators (+ residual when given) instead of as T through LDS.
+// BDIV > 1 ([n, k]-major rhs): K tile t of the lhs meets K tile t / BDIV of the rhs -- an lhs that holds BDIV planes of every
+// 64 columns side by side (a row split into bf16 terms) against one matrix, whose tile then comes from cache for the other planes.
+template <typename T, int BM, int BN, bool B_KN, bool TWO, bool F32OUT = false, int BDIV = 1>
+__global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tiles_n, const float* __restrict__ residual) {
+  static_assert(BDIV == 1 || !B_KN, "planes of the lhs against an [n, k]-major rhs only");
   extern __shared__ u32x4 lds[];
   constexpr int NI = BM / 32, NJ = BN / 32;            // 16-row and 16-column fragments per wave
   constexpr int NM = NI * NJ;                          // MFMAs per k32 step
@@ -144,7 +148,7 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
   auto dma = [&](int tile, int idx) {  // idx: compile-time after unrolling
     const unsigned st = lds_addr + (tile & 1) * STAGE_BYTES;
     if (idx < NDA) dma16(Ab + tile * a_step, voff[idx], st + (idx * 4 + wave) * 1024);
-    else dma16(Bb + tile * b_step, voff[idx], st + A_BYTES + ((idx - NDA) * 4 + wave) * 1024);
+    else dma16(Bb + (tile / BDIV) * b_step, voff[idx], st + A_BYTES + ((idx - NDA) * 4 + wave) * 1024);
   };
   auto dma_m0 = [&](int tile, int idx) {
     const unsigned in_stage = lds_addr + (idx < NDA ? (idx * 4 + wave) * 1024 : A_BYTES + ((idx - NDA) * 4 + wave) * 1024);  // loop invariant
@@ -152,7 +156,7 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
   };
   auto dma_go = [&](int tile, int idx) {
     if (idx < NDA) dma16_go(Ab + tile * a_step, voff[idx]);
-    else dma16_go(Bb + tile * b_step, voff[idx]);
+    else dma16_go(Bb + (tile / BDIV) * b_step, voff[idx]);
   };
 
   floatx4 acc[NI][NJ];
@@ -314,7 +318,25 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
   tile(KT - 2, N_(), Y());
   tile(KT - 1, N_(), N_());
 
-  // Epilogue through LDS.  Register e of lane l of block (i, j): row wm + 16 i + l % 16, column wn + 16 j + 4 (l / 16) + e.
+  // Register e of lane l of block (i, j): row wm + 16 i + l % 16, column wn + 16 j + 4 (l / 16) + e.
+  if constexpr (F32OUT) {
+    // four consecutive f32 per lane: 16-byte stores, 64 contiguous bytes per row and instruction
+    float* __restrict__ C = static_cast<float*>(p.c) + (size_t)batch * p.c_bs + (size_t)m0 * p.N + n0;
+    const float* __restrict__ Rz = residual ? residual + (size_t)batch * p.c_bs + (size_t)m0 * p.N + n0 : nullptr;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const int row = wm + i * 16 + (lane & 15), col = wn + j * 16 + (lane >> 4) * 4;
+        if (row <= m_last && col < n_left) {  // N % 8 == 0: a group of 4 columns exists whole or not at all
+          floatx4 v = acc[i][j];
+          if (Rz) v += *reinterpret_cast<const floatx4*>(Rz + (size_t)row * p.N + col);
+          *reinterpret_cast<floatx4*>(C + (size_t)row * p.N + col) = v;
+        }
+      }
+    return;
+  }
+  // Epilogue through LDS.
   constexpr int PITCH = BN * 2 + 8;
   char __attribute__((address_space(3)))* Cs = (char __attribute__((address_space(3)))*)lds;
 #pragma unroll
@@ -341,15 +363,15 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
   }
 }
 
-template <typename T, int BM, int BN, bool B_KN>
-hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch) {
-  constexpr int STAGES = 2 * (BM + BN) * BK * 2, EPI = BM * (BN * 2 + 8);
+template <typename T, int BM, int BN, bool B_KN, bool F32OUT = false, int BDIV = 1>
+hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch, const float* residual = nullptr) {
+  constexpr int STAGES = 2 * (BM + BN) * BK * 2, EPI = F32OUT ? 0 : BM * (BN * 2 + 8);
   constexpr int LDS_BYTES = STAGES > EPI ? STAGES : EPI;
   static std::atomic<unsigned long long> configured{0};  // one bit per device: the attribute is per device
   // the schedule with two barriers, except where it does not fit the registers (the transposing reads of the
   // largest tile need pairs of temporaries: 256 registers and spills)
   constexpr bool TWO = !(B_KN && BM == 256 && BN == 256);
-  auto kernel = gemm_dma4<T, BM, BN, B_KN, TWO>;
+  auto kernel = gemm_dma4<T, BM, BN, B_KN, TWO, F32OUT, BDIV>;
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev)) return e;
   const unsigned long long bit = dev < 64 ? 1ull << dev : 0;
@@ -359,7 +381,7 @@ hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch) {
   }
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const size_t total = batch * (size_t)tiles_m * tiles_n;
-  kernel<<<dim3((unsigned)total), dim3(256), LDS_BYTES, stream>>>(p, tiles_m, tiles_n);
+  kernel<<<dim3((unsigned)total), dim3(256), LDS_BYTES, stream>>>(p, tiles_m, tiles_n, residual);
   return hipGetLastError();
 }
 
@@ -469,6 +491,19 @@ hipError_t gemm_dma_launch(hipStream_t stream, int dtype, const MMArgs& p, size_
   }
   UGHIP_DMA_CASE(__bf16)
 #undef UGHIP_DMA_CASE
+}
+
+// bf16 planes of f32 rows (three per 64 columns: p.K = 3 k, p.b_k_div = 3) against an [n, k]-major bf16 matrix, f32 result
+// [M, N] (+ residual [M, N] when given).  The same shapes as gemm_dma_supported with the result 16-byte aligned as f32.
+hipError_t gemm_dma_launch_planes3(hipStream_t stream, const MMArgs& p, int tile, const float* residual, bool swiglu_fold_follows) {
+  if (p.b_k_div != 3 || !(p.b_rs == 1 && p.b_cs != 1) || !gemm_dma_supported(UGHIP_BF16, p, 1, tile) || p.K % (3 * BK)) return hipErrorInvalidValue;
+  if (residual && !aligned16(residual)) return hipErrorInvalidValue;
+  int bm = 0, bn = 0;
+  tile_dims(tile, &bm, &bn);
+  note_kernel("gemm_dma4<bf16,NT,%dx%d,256t,3 planes,f32 out%s>", bm, bn, residual ? ",+residual" : swiglu_fold_follows ? ",swiglu fold" : "");
+  if (tile == 256) return launch<__bf16, 256, 256, false, true, 3>(stream, p, 1, residual);
+  if (tile == 128) return launch<__bf16, 256, 128, false, true, 3>(stream, p, 1, residual);
+  return launch<__bf16, 128, 128, false, true, 3>(stream, p, 1, residual);
 }
 
 }  // namespace ughip

@@ -607,6 +607,13 @@ bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf1
   return batch * (size_t)((p.M + kShapes[s][0] - 1) / kShapes[s][0]) * (size_t)((p.N + kShapes[s][1] - 1) / kShapes[s][1]) < (1u << 24);
 }
 
+hipError_t gemm_swiglu_fold(hipStream_t stream, const float* product, float* c, size_t m, size_t n) {
+  const size_t elems = m * n;  // of the product; c has half of them
+  if (elems == 0) return hipSuccess;
+  gemm_split_reduce<float, GemmEpilogue::SWIGLU><<<dim3((unsigned)((elems / 8 + 255) / 256)), dim3(256), 0, stream>>>(product, c, elems / 8, elems, 1, nullptr, (int)n);
+  return hipGetLastError();
+}
+
 double gemm_tiled_cost_us(int dtype, const MMArgs& p, size_t batch) {
   if (!gemm_tiled_supported(dtype, p, batch)) return -1.0;
   const int s = pick_shape(p, batch, dtype);

@@ -598,7 +598,27 @@ static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x
   if (int rc = device_activate(dev)) return rc;
   GemmEpilogue epi{kind, residual ? static_cast<const float*>(residual->ptr) : nullptr};
   epi.out_f32 = x3;
-  const size_t ws_bytes = (gemm_tiled_workspace_bytes(dtype, p, 1, &epi) + 255) & ~(size_t)255;
+  // Many rows of planes: the one-wave-per-SIMD kernel where it is priced cheaper (a prompt of a thousand positions and
+  // more).  Its result leaves as f32 with the residual added on the way; SwiGLU goes through the scratch block and the fold.
+  int dma_tile = 0;
+  if (x3 && !(getenv("UGHIP_X3_DMA") && atoi(getenv("UGHIP_X3_DMA")) == 0)) {
+    MMArgs q = p;
+    q.c = dst->ptr;  // alignment of the result as f32
+    double best = 0;
+    for (int tile : {256, 128, 64}) {
+      if (!gemm_dma_supported(UGHIP_BF16, q, 1, tile)) continue;
+      const double us = gemm_dma_cost_us(q, 1, tile) + (double)m * rows * (kind == GemmEpilogue::SWIGLU ? 10 : 2) / 6.4e6;  // f32 out; SwiGLU: product out, in again, result out
+      if (!dma_tile || us < best * 0.97) dma_tile = tile, best = us;
+    }
+    const double other = gemm_tiled_cost_us(dtype, p, 1);
+    if (dma_tile && other >= 0 && other < best) dma_tile = 0;
+    if (const char* e = getenv("UGHIP_X3_DMA")) {  // tuning aid: 3 / 4 / 5 force a tile where the kernel applies
+      const int f = atoi(e) == 3 ? 256 : atoi(e) == 4 ? 128 : atoi(e) == 5 ? 64 : 0;
+      if (f && gemm_dma_supported(UGHIP_BF16, q, 1, f)) dma_tile = f;
+    }
+  }
+  const size_t ws_bytes = dma_tile ? (kind == GemmEpilogue::SWIGLU ? (m * rows * sizeof(float) + 255) & ~(size_t)255 : 0)
+                                   : (gemm_tiled_workspace_bytes(dtype, p, 1, &epi) + 255) & ~(size_t)255;
   const size_t x3_bytes = x3 ? m * 3 * k * sizeof(uint16_t) : 0;
   if (int rc = grow_gemm_ws(dev, ws_bytes + x3_bytes)) return rc;
   if (x3) {
@@ -607,6 +627,16 @@ static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x
     split3_bf16_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, dev->stream>>>(static_cast<const float*>(x->ptr), planes, n4, (int)k);
     UGHIP_HIPCHK(hipGetLastError());
     p.a = planes;
+  }
+  if (dma_tile) {
+    if (kind == GemmEpilogue::SWIGLU) {
+      p.c = dev->gemm_ws;
+      UGHIP_HIPCHK(gemm_dma_launch_planes3(dev->stream, p, dma_tile, nullptr, true));
+      UGHIP_HIPCHK(gemm_swiglu_fold(dev->stream, static_cast<const float*>(dev->gemm_ws), static_cast<float*>(dst->ptr), m, rows));
+    } else {
+      UGHIP_HIPCHK(gemm_dma_launch_planes3(dev->stream, p, dma_tile, epi.residual, false));
+    }
+    return UGHIP_OK;
   }
   UGHIP_HIPCHK(gemm_tiled_launch(dev->stream, dtype, p, 1, static_cast<float*>(dev->gemm_ws), mixed, &epi));
   return UGHIP_OK;
