@@ -601,7 +601,7 @@ static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x
   // Many rows of planes: the one-wave-per-SIMD kernel where it is priced cheaper (a prompt of a thousand positions and
   // more).  Its result leaves as f32 with the residual added on the way; SwiGLU goes through the scratch block and the fold.
   int dma_tile = 0;
-  if (x3 && !(getenv("UGHIP_X3_DMA") && atoi(getenv("UGHIP_X3_DMA")) == 0)) {
+  if (x3 && m >= 256 && !(getenv("UGHIP_X3_DMA") && atoi(getenv("UGHIP_X3_DMA")) == 0)) {  // (one tile row: measured 74 us against 64-71 for the 128-row head)
     MMArgs q = p;
     q.c = dst->ptr;  // alignment of the result as f32
     double best = 0;
