@@ -62,7 +62,9 @@ __device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc
 __device__ __forceinline__ void dma16(const void* base, unsigned voff, unsigned lds_byte_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
 }
-// The same in two halves with an MFMA between them as the wait state that the write of M0 needs.
+// The same in two halves with an MFMA between them as the wait state that the write of M0 needs.  Nothing the compiler
+// emits between the two may write M0: this kernel has no instruction that would (no LDS instruction of gfx950 needs M0),
+// and the tests that hold its results bit for bit against the register-staged kernel's would show a load gone astray.
 __device__ __forceinline__ void dma16_m0(unsigned lds_byte_addr, unsigned stage_offset) {
   asm volatile("s_add_u32 m0, %0, %1" : : "s"(lds_byte_addr), "s"(stage_offset) : "memory", "scc");
 }
