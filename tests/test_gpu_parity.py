@@ -50,6 +50,35 @@ def test_graph_case(hip, cpu, name, build, tol):
         np.testing.assert_allclose(got, truth, rtol=1e-5, atol=1e-5 * float(np.max(np.abs(truth))))
 
 
+def test_row_kernels_random_widths(hip):
+    """Seeded random row widths (1 .. 6000, and whole multiples of 64) through the row-per-workgroup lowering -- the two
+    softmax kernels, RMSNorm, row sums and row maxima of the lazy graph -- against float64: every number of waves per
+    row, rows whose last wave is partly idle, widths that are odd or 2 mod 4."""
+    gen = np.random.default_rng(777)
+    L = ug_amd.llama
+    for case in range(48):
+        rows = int(gen.integers(1, 9)); kind = case % 4
+        w = int(gen.integers(1, 6000)) if case % 3 else int(gen.integers(1, 120)) * 64
+        print("row kernels random", case, kind, (rows, w), flush=True)
+        x = rng.normal(9000 + case, rows * w, 3.0 if kind == 0 else 1.0)
+        x64 = x.reshape(rows, w).astype(np.float64)
+        if kind == 0:
+            got = L.softmax(LB.copy(x, (rows, w), hip)).data_vec().reshape(rows, w)
+            e = np.exp(x64 - x64.max(1, keepdims=True))
+            np.testing.assert_allclose(got, e / e.sum(1, keepdims=True), rtol=2e-5, atol=1e-9)
+        elif kind == 1:
+            alpha = rng.normal(9500 + case, w, 0.5)
+            got = L.rms_norm(LB.copy(x, (rows, w), hip), LB.copy(alpha, (w,), hip), 1e-5).data_vec().reshape(rows, w)
+            want = x64 / np.sqrt((x64 * x64).mean(1, keepdims=True) + 1e-5) * alpha.astype(np.float64)
+            np.testing.assert_allclose(got, want, rtol=2e-5, atol=1e-6)
+        elif kind == 2:
+            got = LB.copy(x, (rows, w), hip).reduce("sum", 1).narrow(1, 0, 1).data_vec().reshape(rows)
+            np.testing.assert_allclose(got, x64.sum(1), rtol=1e-5, atol=2e-5 * np.abs(x64).sum(1).max())
+        else:
+            got = LB.copy(x, (rows, w), hip).reduce("max", 1).narrow(1, 0, 1).data_vec().reshape(rows)
+            np.testing.assert_array_equal(got, x.reshape(rows, w).max(1))
+
+
 def test_every_case_looser_than_1e_5_has_a_float64_leg():
     loose = [n for n, _, tol in cases.ELEMENTWISE_AND_REDUCE if tol != "exact" and tol > 1e-5]
     assert sorted(loose) == sorted(cases.TRUTH_F64)
@@ -1121,6 +1150,34 @@ def test_attention_cached(hip, cpu, hip_ops, cpu_ops, interleaved, b, nh, nkv, t
             cargs += [ccos, csin, LB.copy(np.array([pos0], np.int32), (1, 1), cpu), interleaved]
         want = cpu_ops.attention_cached(*cargs).data_vec().reshape(b, t, nh, d)
         assert np.all(np.abs(got - want) <= 2 * tol), float(np.abs(got - want).max())
+
+
+def test_attention_cached_random_shapes(hip, hip_ops):
+    """Seeded random shapes (one or a few query positions, caches of up to 3500 rows with spare rows behind them, 1-8 kv
+    heads with 1-8 query heads each, every built head size, with and without either rope, cache lengths at the thresholds
+    where the keys of a head are split over workgroups) against float64."""
+    gen = np.random.default_rng(31337)
+    for case in range(36):
+        d = int(gen.choice([32, 64, 128])); nkv = int(gen.choice([1, 2, 4, 8])); nh = nkv * int(gen.choice([1, 2, 4, 8]))
+        b = int(gen.choice([1, 1, 2])); t = 1 if case % 3 else int(gen.integers(2, 70))
+        s = int(gen.integers(t, 3500)) if case % 4 else int(gen.choice([799, 800, 801, 1279, 1280, 1281, 2047, 2048]))
+        s = max(s, t); cap = s + int(gen.integers(0, 100)); rope = bool(gen.integers(0, 2)); inter = bool(gen.integers(0, 2))
+        print("attention cached random", case, (b, nh, nkv, t, s, cap, d, rope, inter), flush=True)
+        q = rng.normal(100 + case, b * t * nh * d); k = rng.normal(300 + case, b * nkv * cap * d); v = rng.normal(500 + case, b * nkv * cap * d)
+        k4, v4 = k.reshape(b, nkv, cap, d).copy(), v.reshape(b, nkv, cap, d).copy()
+        k4[:, :, s:], v4[:, :, s:] = np.nan, np.inf
+        scale = float(np.float32(d) ** np.float32(-0.5)); pos0 = s - t
+        args = [LB.copy(q, (b, t, nh * d), hip), LB.copy(k4.ravel(), (b, nkv, cap, d), hip), LB.copy(v4.ravel(), (b, nkv, cap, d), hip), s, scale]
+        if rope:
+            cos, sin = _rope_tables(hip, d, max_pos=s + 8)
+            args += [cos, sin, LB.copy(np.array([pos0], np.int32), (1, 1), hip), inter]
+        got = hip_ops.attention_cached(*args).data_vec().reshape(b, t, nh, d)
+        q6 = q.reshape(b, t, nh, d).astype(np.float64)
+        if rope:
+            q6 = _rope_rows_f64(q6, cos.data_vec(), sin.data_vec(), pos0, inter)
+        truth = _attention_truth(q6.transpose(0, 2, 1, 3), k4[:, :, :s].astype(np.float64), v4[:, :, :s].astype(np.float64), s, t, scale, nh // nkv).transpose(0, 2, 1, 3)
+        tol = 2e-5 * np.abs(truth).max() + 2e-5 * np.abs(truth)
+        assert np.all(np.abs(got - truth) <= tol), (case, float(np.abs(got - truth).max()))
 
 
 @pytest.mark.parametrize("interleaved", [False, True])
