@@ -293,6 +293,41 @@ extern "C" __global__ void __launch_bounds__(256) bench_grid_barrier(unsigned* c
 """
 
 
+# Nothing but bf16 MFMAs, one wave per SIMD on every CU, eight independent accumulators of 32 x 32: what the matrix pipes sustain
+# for tens of milliseconds with operands in U(-1, 1) (random sign, mantissa and two exponent bits per element) and with zeros.
+FLOOR_MFMA_SRC = r"""
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ unsigned two_bf16(unsigned& s) {
+  s = s * 1664525u + 1013904223u;
+  const unsigned lo = ((s >> 3) & 0x807f) | (0x3f00 - ((s >> 20) & 3) * 0x80), hi = ((s >> 13) & 0x807f) | (0x3f00 - ((s >> 26) & 3) * 0x80);
+  return lo | (hi << 16);
+}
+extern "C" __global__ void __launch_bounds__(256) bench_mfma_only(float* out, const int* cfg) {
+  const int iters = cfg[0], zeros = cfg[1];
+  unsigned seed = blockIdx.x * 256 + threadIdx.x + 1;
+  u32x4 a[8], b[8];
+  for (int j = 0; j < 8; ++j) {
+    a[j] = zeros ? u32x4{0, 0, 0, 0} : u32x4{two_bf16(seed), two_bf16(seed), two_bf16(seed), two_bf16(seed)};
+    b[j] = zeros ? u32x4{0, 0, 0, 0} : u32x4{two_bf16(seed), two_bf16(seed), two_bf16(seed), two_bf16(seed)};
+  }
+  floatx16 acc[8];
+  for (int q = 0; q < 8; ++q) for (int r = 0; r < 16; ++r) acc[q][r] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+        acc[q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[(j + q) & 7]), __builtin_bit_cast(bf16x8, b[(j + 3 * q) & 7]), acc[q], 0, 0, 0);
+  }
+  float s = 0.f;
+  for (int q = 0; q < 8; ++q) for (int r = 0; r < 16; ++r) s += acc[q][r];
+  out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+"""
+
+
 def launch_and_barrier_floors(dev):
     """What one dependent step costs on this box, the two ways a decode step can be cut into steps: (a) a chain of
     launches on one stream, each reading what the one before wrote; (b) a grid-wide barrier with a value handed over
@@ -334,6 +369,20 @@ def launch_and_barrier_floors(dev):
         out[name] = {"us_per_dependent_launch": round(ms * 1e3 / (100 * reps), 2), "host_us_per_launch": round(wall * 1e6 / (100 * reps), 2),
                      "bytes_per_launch": 8 * n, "verified": True}
         lib.ughip_func_release(f)
+    # The matrix pipes alone: 64 MFMAs of 32 x 32 x 16 per iteration and wave, 4 waves on each of 256 CUs
+    mf_iters = 20000
+    f = compile_src(FLOOR_MFMA_SRC, "bench_mfma_only", [ug_amd.F32, ug_amd.I32], 256, 256)
+    sink = dev.slice_from(np.zeros(256 * 256, np.float32))
+    for label, zeros in (("random", 0), ("zero", 1)):
+        cfg = dev.slice_from(np.array([mf_iters, zeros], np.int32))
+        run(f, [sink, cfg])
+        _, ms = timed(dev, lambda: run(f, [sink, cfg]), 2, 0)
+        got = sink.to_vec()
+        if not np.all(np.isfinite(got)) or (zeros and np.any(got != 0.0)) or (not zeros and not np.any(got != 0.0)):
+            raise RuntimeError(f"mfma only, {label} operands: unexpected sums")
+        tf = 64.0 * 32768 * 4 * 256 * mf_iters * 2 / (ms * 1e-3) / 1e12
+        out[f"mfma_bf16_only_{label}_operands"] = {"TFLOP/s": round(tf, 1), "frac_mfma_bf16": round(tf / MFMA_BF16_PEAK_TF, 4), "ms_per_launch": round(ms / 2, 1), "verified": True}
+    lib.ughip_func_release(f)
     iters = 2000
     for wgs in (64, 256, 512):
         counters = dev.slice_from(np.zeros(16 * 64, np.int32))
