@@ -920,10 +920,10 @@ def main():
                 line.setdefault("extras", {})[key] = llama_decode(dev, n_prompt=n_prompt, n_steps=n_steps, fused_attention=fused, bf16_matrices=narrow, bf16x3=x3)
             except Exception as e:  # noqa: BLE001
                 line.setdefault("extras", {})[key] = {"error": f"{type(e).__name__}: {e}"}
-    # The same step behind half a second of the same launches: under streaming that goes on for tenths of a second the chip
-    # settles at a lower rate than the first few milliseconds show (measured: 21.6 us per step after 20 warm-up steps, 25-27 us
-    # after 20000).  `value` stays what the stated W and K measure; this is the figure for a job that never pauses
-    # (taken last, so that no other row of this run is measured in its wake).
+    # The same step behind half a second of the same launches.  In a process that has done nothing else the chip streams
+    # slower after tenths of a second than in its first milliseconds (measured: 21.6 us per step after 20 warm-up steps,
+    # 24-27 us after 20000); at the end of a full run it does not (21.4 us).  `value` stays what the stated W and K measure;
+    # this figure is taken last, so that no other row of this run is measured in its wake.
     r, cs, keep = fused_reduce(dev, a, b)
     cs.run()
     _, sus_ms = timed_hot(dev, cs.run, args.steps, 0, 0.5)
