@@ -1586,7 +1586,7 @@ def test_projections_of_several_rows_as_three_bf16_terms(hip, t, k, n):
         # up to 64 rows the hooks keep the f32 pipe (a 32- or 64-row tile there is as fast as the split, three planes and an f32 fold)
         assert kern3.startswith("gemm_tiled<f32xbf16,NT,"), kern3
         lin3, add3, glu3, kern3 = run_c_abi()
-    assert kern3.startswith("gemm_tiled<bf16,NT,") and "f32 out" in kern3, kern3
+    assert kern3.startswith(("gemm_tiled<bf16,NT,", "gemm_dma4<bf16,NT,") if t >= 256 else "gemm_tiled<bf16,NT,") and "f32 out" in kern3, kern3
     assert kern1.startswith("gemm_tiled<f32xbf16,NT,"), kern1
     x64, w64, gu64 = x.reshape(t, k).astype(np.float64), w.reshape(n, k).astype(np.float64), wgu.reshape(2 * n, k).astype(np.float64)
     eps = float(np.finfo(np.float32).eps)
@@ -1615,12 +1615,14 @@ def test_projections_of_several_rows_as_three_bf16_terms(hip, t, k, n):
         np.testing.assert_array_equal(back[:, :k], full)
 
 
-@pytest.mark.parametrize("t,k,n,force", [(300, 512, 640, "3"), (300, 512, 640, "4"), (300, 512, 640, "5"), (517, 256, 264, "5"), (260, 1024, 1032, "4"),
-                                         (1900, 2048, 2560, None), (1100, 2048, 2048, None)])
-def test_three_bf16_terms_on_the_one_wave_per_simd_kernel(hip, monkeypatch, t, k, n, force):
+@pytest.mark.parametrize("t,k,n,force,split", [(300, 512, 640, "3", None), (300, 512, 640, "4", None), (300, 512, 640, "5", None), (517, 256, 264, "5", None),
+                                               (260, 1024, 1032, "4", None), (1900, 2048, 2560, None, None), (1100, 2048, 2048, None, None),
+                                               (300, 512, 640, "3", "2"), (260, 1024, 1032, "4", "4"), (517, 768, 264, "5", "2"), (1100, 2048, 2048, "4", "8"),
+                                               (1900, 5632, 2048, None, None)])
+def test_three_bf16_terms_on_the_one_wave_per_simd_kernel(hip, monkeypatch, t, k, n, force, split):
     """Many rows of three bf16 planes take gemm_dma4 (f32 result straight from the accumulators, the residual added on the
-    way, SwiGLU through the scratch block and the fold).  Forced tiles on small ragged shapes, the library's own choice on
-    prompts of a thousand positions and more; against float64 with the k eps bound of the f32 product, against the
+    way, SwiGLU through the scratch block and the fold; with K split over workgroups, f32 slabs and the fold for all three).
+    Forced tiles and splits on small ragged shapes, the library's own choice on prompts of a thousand positions and more; against float64 with the k eps bound of the f32 product, against the
     register-staged kernel (UGHIP_X3_DMA=0: the same exact terms, sums in another order), small integers exactly, and a
     sentinel behind every result."""
     import ctypes as C
@@ -1650,10 +1652,16 @@ def test_three_bf16_terms_on_the_one_wave_per_simd_kernel(hip, monkeypatch, t, k
 
     if force:
         monkeypatch.setenv("UGHIP_X3_DMA", force)
+    if split:
+        monkeypatch.setenv("UGHIP_X3_SPLIT", split)
     (lin, add, glu), kerns = run(x, w, wgu)
     tile = {"3": "256x256", "4": "256x128", "5": "128x128"}.get(force, "")
-    for kn, tail in zip(kerns, ("f32 out>", "+residual>", "swiglu fold>")):
-        assert kn.startswith("gemm_dma4<bf16,NT," + tile) and "3 planes" in kn and kn.endswith(tail), kn
+    for kn, word in zip(kerns, ("f32 out", "residual", "swiglu fold")):
+        assert kn.startswith("gemm_dma4<bf16,NT," + tile) and "3 planes" in kn and word in kn, kn
+        assert ("splitK=" + split in kn) if split else True, kn
+    if (t, k, n) == (1900, 5632, 2048):
+        assert "splitK=" in kerns[0], kerns   # 64 tiles of 256 x 256 and 264 K tiles: the library splits K by itself
+    monkeypatch.delenv("UGHIP_X3_SPLIT", raising=False)
     monkeypatch.setenv("UGHIP_X3_DMA", "0")
     (lin0, add0, glu0), kerns0 = run(x, w, wgu)
     assert all(kn.startswith("gemm_tiled<bf16,NT,") for kn in kerns0), kerns0
@@ -1674,6 +1682,8 @@ def test_three_bf16_terms_on_the_one_wave_per_simd_kernel(hip, monkeypatch, t, k
         monkeypatch.setenv("UGHIP_X3_DMA", force)
     else:
         monkeypatch.delenv("UGHIP_X3_DMA")
+    if split:
+        monkeypatch.setenv("UGHIP_X3_SPLIT", split)
     xi, wi, gui = np.floor(x * 4).astype(np.float32), np.floor(w * 40).astype(np.float32), np.floor(wgu * 40).astype(np.float32)
     (lin_i, add_i, _), kerns_i = run(xi, wi, gui)
     assert kerns_i[0].startswith("gemm_dma4<"), kerns_i

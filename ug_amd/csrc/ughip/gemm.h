@@ -50,10 +50,15 @@ bool gemm_dma_supported(int dtype, const MMArgs& p, size_t batch, int tile);
 hipError_t gemm_dma_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, int tile);
 // The tile code this kernel should take the problem with, 0 when another kernel should.
 int gemm_dma_pick(int dtype, const MMArgs& p, size_t batch);
-// The same kernel on three bf16 planes of f32 rows (p.K = 3 k, p.b_k_div = 3, [n, k]-major bf16 matrix): f32 result, residual added when given.
-hipError_t gemm_dma_launch_planes3(hipStream_t stream, const MMArgs& p, int tile, const float* residual, bool swiglu_fold_follows);
-// c[m, n / 2] = silu(product[:, :n / 2]) * product[:, n / 2:] for an f32 product [m, n] (n % 8 == 0): the fold of the tiled kernel on one slab.
-hipError_t gemm_swiglu_fold(hipStream_t stream, const float* product, float* c, size_t m, size_t n);
+// The same kernel on three bf16 planes of f32 rows (p.K = 3 k, p.b_k_div = 3, [n, k]-major bf16 matrix), f32 result.
+// nsplit == 1: p.c [M, N] is written straight from the accumulators, residual [M, N] added when given.  nsplit > 1 (it
+// divides the K tiles, into a multiple of 3 and at least 4 each): workgroups share a tile's K range and leave nsplit
+// slabs [M, N] in p.c (scratch), for gemm_fold_f32 to add up.
+hipError_t gemm_dma_launch_planes3(hipStream_t stream, const MMArgs& p, int tile, int nsplit, const float* residual, const char* note_tail);
+bool gemm_dma_planes3_split_ok(const MMArgs& p, int nsplit);
+// c = fold of nsplit f32 slabs [m, n] in slab order, then the epilogue: NONE, ADD (+ residual[m, n]) or SWIGLU
+// (c[m, n / 2] = silu(sum[:, :n / 2]) * sum[:, n / 2:]); n % 8 == 0.
+hipError_t gemm_fold_f32(hipStream_t stream, const float* slabs, float* c, size_t m, size_t n, int nsplit, GemmEpilogue::Kind kind, const float* residual);
 double gemm_dma_cost_us(const MMArgs& p, size_t batch, int tile);
 
 }  // namespace ughip

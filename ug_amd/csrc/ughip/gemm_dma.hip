@@ -496,16 +496,31 @@ hipError_t gemm_dma_launch(hipStream_t stream, int dtype, const MMArgs& p, size_
 }
 
 // bf16 planes of f32 rows (three per 64 columns: p.K = 3 k, p.b_k_div = 3) against an [n, k]-major bf16 matrix, f32 result
-// [M, N] (+ residual [M, N] when given).  The same shapes as gemm_dma_supported with the result 16-byte aligned as f32.
-hipError_t gemm_dma_launch_planes3(hipStream_t stream, const MMArgs& p, int tile, const float* residual, bool swiglu_fold_follows) {
-  if (p.b_k_div != 3 || !(p.b_rs == 1 && p.b_cs != 1) || !gemm_dma_supported(UGHIP_BF16, p, 1, tile) || p.K % (3 * BK)) return hipErrorInvalidValue;
+// [M, N] (+ residual [M, N] when given), or nsplit slabs of it: the splits of K run as the kernel's batches, with the
+// batch strides of the operands standing for a split's offset in K (a whole number of groups of three planes).
+bool gemm_dma_planes3_split_ok(const MMArgs& p, int nsplit) {
+  if (nsplit < 1 || p.K % (BK * nsplit)) return false;
+  const int kts = p.K / BK / nsplit;
+  return kts % 3 == 0 && kts >= 4;
+}
+
+hipError_t gemm_dma_launch_planes3(hipStream_t stream, const MMArgs& p, int tile, int nsplit, const float* residual, const char* note_tail) {
+  if (p.b_k_div != 3 || !(p.b_rs == 1 && p.b_cs != 1) || !gemm_dma_planes3_split_ok(p, nsplit) || (nsplit > 1 && residual)) return hipErrorInvalidValue;
+  MMArgs q = p;
+  if (nsplit > 1) {
+    q.K = p.K / nsplit;
+    q.a_bs = q.K, q.b_bs = q.K / 3, q.c_bs = (long long)p.M * p.N;
+  }
+  if (!gemm_dma_supported(UGHIP_BF16, q, (size_t)nsplit, tile)) return hipErrorInvalidValue;
   if (residual && !aligned16(residual)) return hipErrorInvalidValue;
   int bm = 0, bn = 0;
   tile_dims(tile, &bm, &bn);
-  note_kernel("gemm_dma4<bf16,NT,%dx%d,256t,3 planes,f32 out%s>", bm, bn, residual ? ",+residual" : swiglu_fold_follows ? ",swiglu fold" : "");
-  if (tile == 256) return launch<__bf16, 256, 256, false, true, 3>(stream, p, 1, residual);
-  if (tile == 128) return launch<__bf16, 256, 128, false, true, 3>(stream, p, 1, residual);
-  return launch<__bf16, 128, 128, false, true, 3>(stream, p, 1, residual);
+  char split[24] = "";
+  if (nsplit > 1) snprintf(split, sizeof split, ",splitK=%d", nsplit);
+  note_kernel("gemm_dma4<bf16,NT,%dx%d,256t,3 planes%s,f32 out%s>", bm, bn, split, note_tail ? note_tail : "");
+  if (tile == 256) return launch<__bf16, 256, 256, false, true, 3>(stream, q, (size_t)nsplit, residual);
+  if (tile == 128) return launch<__bf16, 256, 128, false, true, 3>(stream, q, (size_t)nsplit, residual);
+  return launch<__bf16, 128, 128, false, true, 3>(stream, q, (size_t)nsplit, residual);
 }
 
 }  // namespace ughip

@@ -607,10 +607,13 @@ bool gemm_tiled_supported(int dtype, const MMArgs& p, size_t batch, bool rhs_bf1
   return batch * (size_t)((p.M + kShapes[s][0] - 1) / kShapes[s][0]) * (size_t)((p.N + kShapes[s][1] - 1) / kShapes[s][1]) < (1u << 24);
 }
 
-hipError_t gemm_swiglu_fold(hipStream_t stream, const float* product, float* c, size_t m, size_t n) {
-  const size_t elems = m * n;  // of the product; c has half of them
+hipError_t gemm_fold_f32(hipStream_t stream, const float* slabs, float* c, size_t m, size_t n, int nsplit, GemmEpilogue::Kind kind, const float* residual) {
+  const size_t elems = m * n;  // of one slab; with SwiGLU c has half of them
   if (elems == 0) return hipSuccess;
-  gemm_split_reduce<float, GemmEpilogue::SWIGLU><<<dim3((unsigned)((elems / 8 + 255) / 256)), dim3(256), 0, stream>>>(product, c, elems / 8, elems, 1, nullptr, (int)n);
+  const dim3 grid((unsigned)((elems / 4 + 255) / 256)), half_grid((unsigned)((elems / 8 + 255) / 256));
+  if (kind == GemmEpilogue::SWIGLU) gemm_split_reduce<float, GemmEpilogue::SWIGLU><<<half_grid, dim3(256), 0, stream>>>(slabs, c, elems / 8, elems, nsplit, nullptr, (int)n);
+  else if (kind == GemmEpilogue::ADD) gemm_split_reduce<float, GemmEpilogue::ADD><<<grid, dim3(256), 0, stream>>>(slabs, c, elems / 4, elems, nsplit, residual, (int)n);
+  else gemm_split_reduce<float, 0><<<grid, dim3(256), 0, stream>>>(slabs, c, elems / 4, elems, nsplit, nullptr, (int)n);
   return hipGetLastError();
 }
 

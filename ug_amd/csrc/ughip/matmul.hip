@@ -600,24 +600,33 @@ static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x
   epi.out_f32 = x3;
   // Many rows of planes: the one-wave-per-SIMD kernel where it is priced cheaper (a prompt of a thousand positions and
   // more).  Its result leaves as f32 with the residual added on the way; SwiGLU goes through the scratch block and the fold.
-  int dma_tile = 0;
+  int dma_tile = 0, dma_split = 1;
   if (x3 && m >= 256 && !(getenv("UGHIP_X3_DMA") && atoi(getenv("UGHIP_X3_DMA")) == 0)) {  // (one tile row: measured 74 us against 64-71 for the 128-row head)
     MMArgs q = p;
     q.c = dst->ptr;  // alignment of the result as f32
     double best = 0;
+    const int forced_tile = getenv("UGHIP_X3_DMA") ? (atoi(getenv("UGHIP_X3_DMA")) == 3 ? 256 : atoi(getenv("UGHIP_X3_DMA")) == 4 ? 128 : atoi(getenv("UGHIP_X3_DMA")) == 5 ? 64 : 0) : 0;
+    const int forced_split = getenv("UGHIP_X3_SPLIT") ? atoi(getenv("UGHIP_X3_SPLIT")) : 0;  // tuning aids: 3 / 4 / 5 force a tile, n a K split
     for (int tile : {256, 128, 64}) {
-      if (!gemm_dma_supported(UGHIP_BF16, q, 1, tile)) continue;
-      const double us = gemm_dma_cost_us(q, 1, tile) + (double)m * rows * (kind == GemmEpilogue::SWIGLU ? 10 : 2) / 6.4e6;  // f32 out; SwiGLU: product out, in again, result out
-      if (!dma_tile || us < best * 0.97) dma_tile = tile, best = us;
+      if (forced_tile && tile != forced_tile) continue;
+      for (int split : {1, 2, 4, 8}) {
+        if (forced_split && split != forced_split) continue;
+        if (!gemm_dma_planes3_split_ok(q, split)) continue;
+        MMArgs qs = q;
+        if (split > 1) qs.K = q.K / split, qs.a_bs = qs.K, qs.b_bs = qs.K / 3, qs.c_bs = (long long)(m * rows);
+        if (!gemm_dma_supported(UGHIP_BF16, qs, (size_t)split, tile)) continue;
+        // the kernel (its model counts 2 bytes per result element), the f32 result's other 2, and the fold where there is one:
+        // the slabs in, the result out, a launch
+        const bool fold = split > 1 || kind == GemmEpilogue::SWIGLU;
+        const double us = gemm_dma_cost_us(qs, (size_t)split, tile) + (double)split * m * rows * 2 / 6.4e6 + (fold ? 3.0 + (double)(split + 1) * m * rows * 4 / 6.4e6 : 0.0);
+        if (!dma_tile || us < best * 0.97) dma_tile = tile, dma_split = split, best = us;
+      }
     }
     const double other = gemm_tiled_cost_us(dtype, p, 1);
-    if (dma_tile && other >= 0 && other < best) dma_tile = 0;
-    if (const char* e = getenv("UGHIP_X3_DMA")) {  // tuning aid: 3 / 4 / 5 force a tile where the kernel applies
-      const int f = atoi(e) == 3 ? 256 : atoi(e) == 4 ? 128 : atoi(e) == 5 ? 64 : 0;
-      if (f && gemm_dma_supported(UGHIP_BF16, q, 1, f)) dma_tile = f;
-    }
+    if (dma_tile && !forced_tile && other >= 0 && other < best) dma_tile = 0;
   }
-  const size_t ws_bytes = dma_tile ? (kind == GemmEpilogue::SWIGLU ? (m * rows * sizeof(float) + 255) & ~(size_t)255 : 0)
+  const bool dma_fold = dma_tile && (dma_split > 1 || kind == GemmEpilogue::SWIGLU);
+  const size_t ws_bytes = dma_tile ? (dma_fold ? ((size_t)dma_split * m * rows * sizeof(float) + 255) & ~(size_t)255 : 0)
                                    : (gemm_tiled_workspace_bytes(dtype, p, 1, &epi) + 255) & ~(size_t)255;
   const size_t x3_bytes = x3 ? m * 3 * k * sizeof(uint16_t) : 0;
   if (int rc = grow_gemm_ws(dev, ws_bytes + x3_bytes)) return rc;
@@ -629,12 +638,12 @@ static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x
     p.a = planes;
   }
   if (dma_tile) {
-    if (kind == GemmEpilogue::SWIGLU) {
+    if (dma_fold) {
       p.c = dev->gemm_ws;
-      UGHIP_HIPCHK(gemm_dma_launch_planes3(dev->stream, p, dma_tile, nullptr, true));
-      UGHIP_HIPCHK(gemm_swiglu_fold(dev->stream, static_cast<const float*>(dev->gemm_ws), static_cast<float*>(dst->ptr), m, rows));
+      UGHIP_HIPCHK(gemm_dma_launch_planes3(dev->stream, p, dma_tile, dma_split, nullptr, kind == GemmEpilogue::SWIGLU ? ",swiglu fold" : kind == GemmEpilogue::ADD ? ",+residual in the fold" : ",fold"));
+      UGHIP_HIPCHK(gemm_fold_f32(dev->stream, static_cast<const float*>(dev->gemm_ws), static_cast<float*>(dst->ptr), m, rows, dma_split, kind, epi.residual));
     } else {
-      UGHIP_HIPCHK(gemm_dma_launch_planes3(dev->stream, p, dma_tile, epi.residual, false));
+      UGHIP_HIPCHK(gemm_dma_launch_planes3(dev->stream, p, dma_tile, 1, epi.residual, epi.residual ? ",+residual" : ""));
     }
     return UGHIP_OK;
   }
