@@ -601,7 +601,9 @@ static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x
   // Many rows of planes: the one-wave-per-SIMD kernel where it is priced cheaper (a prompt of a thousand positions and
   // more).  Its result leaves as f32 with the residual added on the way; SwiGLU goes through the scratch block and the fold.
   int dma_tile = 0, dma_split = 1;
-  if (x3 && m >= 256 && !(getenv("UGHIP_X3_DMA") && atoi(getenv("UGHIP_X3_DMA")) == 0)) {  // (one tile row: measured 74 us against 64-71 for the 128-row head)
+  // (from 384 rows: at 128 and 256 rows the register-staged kernel is as fast or faster for four of the five products of a
+  // llama step -- q|k|v 25.2 us against 28.6 at 256 rows -- and the model below does not see that; at 512 rows this kernel is)
+  if (x3 && m >= 384 && !(getenv("UGHIP_X3_DMA") && atoi(getenv("UGHIP_X3_DMA")) == 0)) {
     MMArgs q = p;
     q.c = dst->ptr;  // alignment of the result as f32
     double best = 0;
@@ -623,7 +625,7 @@ static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x
       }
     }
     const double other = gemm_tiled_cost_us(dtype, p, 1);
-    if (dma_tile && !forced_tile && other >= 0 && other < best) dma_tile = 0;
+    if (dma_tile && !forced_tile && other >= 0 && other < best * 1.05) dma_tile = 0;  // it has to be clearly cheaper: its model is the rougher one
   }
   const bool dma_fold = dma_tile && (dma_split > 1 || kind == GemmEpilogue::SWIGLU);
   const size_t ws_bytes = dma_tile ? (dma_fold ? ((size_t)dma_split * m * rows * sizeof(float) + 255) & ~(size_t)255 : 0)
