@@ -170,7 +170,7 @@ int ughip_compile(ughip_device* dev, const ughip_ssa* ssa, const char* name, ugh
 int ughip_func_release(ughip_func* f);
 /* args in ssa.args() order (schedule.rs:190-195); asynchronous; zero-sized launch is a
  * no-op (runtime.rs:269-277).  Fails with UGHIP_ERR_BOUNDS if a slice is shorter than the
- * largest offset the kernel can form. */
+ * largest offset the kernel can form (ughip_codegen_min_len says how that is counted under an If). */
 int ughip_run(ughip_device* dev, ughip_func* f, ughip_slice* const* args, size_t n_args);
 /* Timing aid with no counterpart in the reference: a func lowered to two kernels (a grid-wide reduction:
  * partial sums, then the fold) launches only its first (part 1) or second (part 2) kernel, with the checks of
@@ -198,6 +198,12 @@ int ughip_func_get_info(const ughip_func* f, ughip_func_info* out);
 /* Lowering only, no device needed: SSA -> HIP source (for CPU-side inspection/tests). */
 int ughip_codegen(const ughip_ssa* ssa, const char* name, char* buf, size_t buf_len,
                   size_t* out_len, ughip_func_info* info);
+/* Lowering only, no device needed: per kernel argument, the number of elements a slice must hold for
+ * ughip_run to accept it (1 + the largest offset the kernel can form; -1 where an offset is computed
+ * from loaded data and cannot be bounded).  An access under an If counts with what the guard lets
+ * through where the guard pins the offset (`If(max(n - i, 0))` around `dst[i]`: n elements); a guard
+ * that says nothing about the offset leaves the full requirement.  n_args must be the kernel's. */
+int ughip_codegen_min_len(const ughip_ssa* ssa, int64_t* min_len, size_t n_args);
 
 /* The same kernel translated statement by statement, for its own launch configuration: a serial
  * loop nest stays one thread's loop nest, as in the text ug-cuda/src/code_gen.rs:68-186 produces

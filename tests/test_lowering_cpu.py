@@ -203,3 +203,59 @@ def test_ref_suite_graph_shapes(cpu):
     r = ref_suite.fused_reduce_graph(a, b, cpu)
     assert r.dims() == [1]
     assert r.data_vec().tolist() == [12.0]
+
+
+def _guard_prog(store_offset_var, extra=()):
+    """A GPU-style kernel over 2 x 64 threads: i = bi * 64 + ti, then `extra` instructions, then a store of 3.0 at
+    variable `store_offset_var` under If(var 6) where var 6 = max(100 - i, 0)."""
+    from ug_amd.api import A, Instr
+    I32_, F32_ = int(ug_amd.I32), int(ug_amd.F32)
+
+    def var(i):
+        return A(0, I32_, 0, i, 0, 0.0, 0)
+
+    def ci(v):
+        return A(1, I32_, 0, 0, v, 0.0, 0)
+
+    def ins(op, dtype=0, sub=0, v=0, n=0, a=None, b=None):
+        return Instr(op, dtype, sub, v, n, a or A(), b or A())
+
+    extra = [ins(6, I32_, sub=sub, a=(var(a) if va else ci(a)), b=(var(b) if vb else ci(b))) for sub, va, a, vb, b in extra]
+    n_if = 7 + len(extra)
+    prog = [
+        ins(1, F32_, n=0),                              # 0 DefineGlobal{0, F32}
+        ins(3, I32_, sub=0),                            # 1 ThreadIdx
+        ins(3, I32_, sub=1),                            # 2 BlockIdx
+        ins(6, I32_, sub=2, a=var(2), b=ci(64)),        # 3 bi * 64
+        ins(6, I32_, sub=0, a=var(3), b=var(1)),        # 4 i = bi * 64 + ti
+        ins(6, I32_, sub=1, a=ci(100), b=var(4)),       # 5 100 - i
+        ins(6, I32_, sub=6, a=var(5), b=ci(0)),         # 6 max(100 - i, 0): non-zero iff i < 100
+    ] + extra + [
+        ins(11, v=n_if + 2, a=var(6)),                  # If
+        ins(13, F32_, v=0, a=var(store_offset_var), b=A(1, F32_, 0, 0, 0, 3.0, 0)),
+        ins(12),                                        # EndIf
+    ]
+    return SsaKernel.from_instrs(prog, grid=2, block=64)
+
+
+def test_a_guard_that_bounds_the_offset_narrows_the_length_a_slice_must_have():
+    """`If(max(100 - i, 0))` around `dst[i]` with i up to 127: the body runs for i <= 99 only, so 100 elements are asked
+    for; `dst[2 i + 1]` under the same guard: 200 (integers computed from the narrowed one narrow with it)."""
+    assert _guard_prog(4).min_lens() == [100]
+    two_i_plus_1 = [(2, True, 4, False, 2), (0, True, 7, False, 1)]   # 7 = i * 2, 8 = (i * 2) + 1
+    assert _guard_prog(8, two_i_plus_1).min_lens() == [200]
+
+
+def test_a_guard_that_says_nothing_about_the_offset_leaves_the_full_requirement():
+    """The store's offset is a second copy of bi * 64 + ti that the guard's expression does not go through (an unrelated
+    condition as far as the analysis can prove): all 128 offsets the grid can form count, and a 100-element slice
+    would be refused by ughip_run."""
+    other_i = [(2, True, 2, False, 64), (0, True, 7, True, 1)]        # 7 = bi * 64, 8 = 7 + ti
+    assert _guard_prog(8, other_i).min_lens() == [128]
+    # a guard on the thread index alone (ti < 50) bounds ti, not the block: 64 + 49 + 1
+    from ug_amd.api import A, Instr
+    k = _guard_prog(4)
+    prog = list(k.instrs())
+    I32_ = int(ug_amd.I32)
+    prog[5] = Instr(6, I32_, 1, 0, 0, A(1, I32_, 0, 0, 50, 0.0, 0), A(0, I32_, 0, 1, 0, 0.0, 0))   # 5 = 50 - ti
+    assert SsaKernel.from_instrs(prog, grid=2, block=64).min_lens() == [114]

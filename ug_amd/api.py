@@ -257,6 +257,15 @@ class SsaKernel(_Handle):
         w = self.wire()
         return [w.instrs[i] for i in range(w.n_instrs)]
 
+    def min_lens(self):
+        """Per kernel argument, the slice length ughip_run asks for (-1: not bounded statically); needs no device."""
+        w = self.wire()
+        out = (C.c_int64 * w.n_args)()
+        lib = ughip_lib()
+        if lib.ughip_codegen_min_len(C.byref(w), out, C.c_size_t(w.n_args)):
+            raise UgError(lib.ughip_last_error().decode())
+        return list(out)
+
     def hip_code(self, name=None):
         """Counterpart of `Kernel.cuda_code()` (ug-pyo3/src/lib.rs:396-401); needs no device."""
         w = self.wire()

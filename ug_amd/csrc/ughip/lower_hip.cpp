@@ -240,6 +240,7 @@ class Lowering {
   std::vector<int> encl_;      // per instr: innermost enclosing loop id (Range belongs to its parent)
   std::vector<int> arg_of_;    // per instr: kernel-arg index if DefineGlobal
   std::vector<bool> guarded_;  // per instr: inside an If
+  std::vector<int> if_of_;     // per instr: innermost enclosing If (instr index), -1 if none; for an If, the one around it
   std::vector<uint64_t> dep_;  // per var: loops it depends on
   std::vector<Itv> itv_;
   std::vector<Aff> aff_;
@@ -277,6 +278,7 @@ class Lowering {
     encl_.assign(n_, -1);
     arg_of_.assign(n_, -1);
     guarded_.assign(n_, false);
+    if_of_.assign(n_, -1);
     std::vector<int> stack;     // open loop ids / -2 for If
     std::vector<int> if_stack;  // instr index of open Ifs
     size_t n_globals = 0;
@@ -290,6 +292,7 @@ class Lowering {
         }
       encl_[i] = cur;
       guarded_[i] = !if_stack.empty();
+      if_of_[i] = if_stack.empty() ? -1 : if_stack.back();
       if (in.dtype < 0 || in.dtype > UGHIP_I64) fail("bad dtype at " + std::to_string(i));
       switch (in.op) {
         case UGHIP_I_DEFINE_ACC:
@@ -512,6 +515,93 @@ class Lowering {
       if (I_[i].op == UGHIP_I_ASSIGN) itv_[I_[i].v].known = false;
   }
 
+
+  // ---- what an enclosing If says about the integers of the kernel ------------------------------
+  // The SSA has no comparison: a guard is an integer that is non-zero when the body runs, built from Sub / Max / Min / Mul
+  // (`max(n - i, 0)`, `min(a, b)` or `a * b` of two such).  constrain(v, want) records that value v lies in `want`
+  // inside the body and pushes that through the defining instruction to its operands; every step is a necessary
+  // condition of the guard being taken, never a guess, so intervals only shrink.
+  static constexpr i64 kInf = 1ll << 41;
+  static Itv meet(const Itv& a, const Itv& b) {
+    if (!a.known) return b;
+    if (!b.known) return a;
+    return {true, std::max(a.lo, b.lo), std::min(a.hi, b.hi)};
+  }
+  void constrain(std::map<int, Itv>& over, const ughip_a& a, Itv want, int depth) const {
+    if (a.is_const || depth > 16) return;
+    const int v = (int)a.var;
+    if (!itv_[v].known) return;  // reassigned accumulators, floats: nothing static to narrow
+    Itv cur = over.count(v) ? over[v] : itv_[v];
+    Itv now = meet(cur, want);
+    if (now.lo == cur.lo && now.hi == cur.hi && over.count(v)) return;
+    over[v] = now;
+    const ughip_instr& d = I_[v];
+    auto of = [&](const ughip_a& x) { return x.is_const || !over.count((int)x.var) ? itv_of(x) : over.at((int)x.var); };
+    if (d.op == UGHIP_I_UNARY && d.sub == UGHIP_U_ID) constrain(over, d.a, now, depth + 1);
+    if (d.op == UGHIP_I_UNARY && d.sub == UGHIP_U_NEG) constrain(over, d.a, {true, -now.hi, -now.lo}, depth + 1);
+    if (d.op != UGHIP_I_BINARY) return;
+    const Itv x = of(d.a), y = of(d.b);
+    if (!x.known || !y.known) return;
+    switch (d.sub) {
+      case UGHIP_B_ADD:
+        constrain(over, d.a, {true, now.lo - y.hi, now.hi - y.lo}, depth + 1);
+        constrain(over, d.b, {true, now.lo - x.hi, now.hi - x.lo}, depth + 1);
+        break;
+      case UGHIP_B_SUB:  // v = a - b
+        constrain(over, d.a, {true, now.lo + y.lo, now.hi + y.hi}, depth + 1);
+        constrain(over, d.b, {true, x.lo - now.hi, x.hi - now.lo}, depth + 1);
+        break;
+      case UGHIP_B_MAX:  // v >= lo with one side below lo: the other side is at least lo; v <= hi holds for both
+        constrain(over, d.a, {true, y.hi < now.lo ? now.lo : -kInf, now.hi}, depth + 1);
+        constrain(over, d.b, {true, x.hi < now.lo ? now.lo : -kInf, now.hi}, depth + 1);
+        break;
+      case UGHIP_B_MIN:
+        constrain(over, d.a, {true, now.lo, y.lo > now.hi ? now.hi : kInf}, depth + 1);
+        constrain(over, d.b, {true, now.lo, x.lo > now.hi ? now.hi : kInf}, depth + 1);
+        break;
+      case UGHIP_B_MUL:  // a product of two non-negative integers is non-zero only if both are
+        if (x.lo >= 0 && y.lo >= 0 && now.lo >= 1) {
+          constrain(over, d.a, {true, 1, kInf}, depth + 1);
+          constrain(over, d.b, {true, 1, kInf}, depth + 1);
+        }
+        break;
+      default: break;
+    }
+  }
+
+  // Interval of the offset `off` of the access at instruction `at`, given that every If around it was taken.
+  Itv offset_under_guards(int at, const ughip_a& off) const {
+    if (off.is_const) return itv_of(off);
+    std::map<int, Itv> over;
+    for (int f = if_of_[at]; f >= 0; f = if_of_[f]) {
+      const Itv c = itv_of(I_[f].a);
+      if (!c.known) continue;
+      if (c.lo >= 0) constrain(over, I_[f].a, {true, 1, kInf}, 0);
+      else if (c.hi <= 0) constrain(over, I_[f].a, {true, -kInf, -1}, 0);
+    }
+    if (over.empty()) return itv_of(off);
+    // forward again from the first narrowed value: integers computed from narrowed ones narrow with them
+    std::vector<Itv> t(itv_.begin(), itv_.begin() + at);
+    for (auto& kv : over)
+      if (kv.first < at) t[kv.first] = kv.second;
+    auto of = [&](const ughip_a& x) -> Itv { return x.is_const ? itv_of(x) : ((int)x.var < at ? t[x.var] : Itv()); };
+    for (int i = over.begin()->first + 1; i < at; ++i) {
+      if (!itv_[i].known) continue;
+      const ughip_instr& in = I_[i];
+      Itv r;
+      if (in.op == UGHIP_I_BINARY) r = itv_binop(in.sub, of(in.a), of(in.b));
+      else if (in.op == UGHIP_I_UNARY && in.sub == UGHIP_U_ID) r = of(in.a);
+      else if (in.op == UGHIP_I_UNARY && in.sub == UGHIP_U_NEG) {
+        const Itv a = of(in.a);
+        if (a.known) r = {true, -a.hi, -a.lo};
+      } else continue;
+      if (r.known) t[i] = meet(t[i], r);
+    }
+    const Itv o = t[off.var];
+    if (o.known && o.lo > o.hi) return {true, 0, -1};  // the guard can never be taken: the access touches nothing
+    return o;
+  }
+
   // Is instruction i inside a loop that provably never runs?
   bool dead(int i) const {
     for (int l = encl_[i]; l >= 0; l = loops_[l].parent)
@@ -533,10 +623,9 @@ class Lowering {
       if (dead(i)) continue;
       if (in.op == UGHIP_I_STORE) live_store = true;
       // An access under an If may be exactly what the guard keeps in range (a grid rounded up to the block size with
-      // `if (i < n)` around the store): the interval of its offset says nothing about what is touched, so it adds
-      // no requirement (the unguarded accesses of the same argument still do).
-      if (guarded_[i]) continue;
-      Itv o = itv_of(in.a);
+      // `if (max(n - i, 0))` around the store).  Where the guard's value pins integers of the kernel (see narrow_by_guards)
+      // the offset is re-evaluated under those narrower intervals; any other condition leaves the full requirement.
+      Itv o = guarded_[i] ? offset_under_guards(i, in.a) : itv_of(in.a);
       if (!o.known || o.lo < 0)
         out_.min_len[a] = -1;
       else if (out_.min_len[a] >= 0)

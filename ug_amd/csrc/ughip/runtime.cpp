@@ -309,6 +309,14 @@ int ughip_codegen(const ughip_ssa* ssa, const char* name, char* buf, size_t buf_
   return UGHIP_OK;
 }
 
+int ughip_codegen_min_len(const ughip_ssa* ssa, int64_t* min_len, size_t n_args) {
+  Lowered low;
+  if (int rc = lower_checked(ssa, nullptr, &low)) return rc;
+  if (!min_len || n_args != low.min_len.size()) return set_error(UGHIP_ERR_INVALID, "codegen_min_len: the kernel has %zu arguments, room for %zu given", low.min_len.size(), n_args);
+  for (size_t a = 0; a < n_args; ++a) min_len[a] = low.min_len[a];
+  return UGHIP_OK;
+}
+
 int ughip_codegen_as_written(const ughip_ssa* ssa, const char* name, char* buf, size_t buf_len, size_t* out_len) {
   Lowered low;
   if (name) {
