@@ -13,8 +13,8 @@
 //   needs 16 cycles per such instruction and a K tile takes 64 of them, half the tile's time: they are dealt one by one
 //   in front of MFMAs over as much of the tile as the stage they fill allows (see the two schedules in the kernel)
 //   rhs [n, k]-major: operand fragments are 128-bit LDS reads of k-contiguous rows (XOR-swizzled chunks, conflict free);
-//   rhs [k, n]-major: the tile stays [k][n] in LDS and ds_read_b64_tr_b16 hands every lane 4 consecutive k of its own
-//   column, so no transposing pass through registers is needed
+//   rhs [k, n]-major: the tile stays [k][n] in LDS (32-byte pieces XOR-swizzled by k so that the reads meet no bank twice)
+//   and ds_read_b64_tr_b16 hands every lane 4 consecutive k of its own column: no transposing pass through registers
 //   the MFMA operands are swapped (B fragment first): a lane then holds 4 consecutive columns of one result row, the
 //   epilogue packs them and goes through LDS so that the result leaves in 16-byte pieces of whole rows
 //
@@ -60,13 +60,16 @@ __device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xc
 // Every lane's 16 bytes at base + voff go to LDS at lds_byte_addr + lane * 16.  The compiler does not see the load
 // (it would wait for all of them before any LDS read): the waits are explicit.
 __device__ __forceinline__ void dma16(const void* base, unsigned voff, unsigned lds_byte_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_byte_addr), "v"(voff), "s"(base) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_byte_addr), "v"(voff), "s"(base) : "memory", "m0");
 }
-// The same in two halves with an MFMA between them as the wait state that the write of M0 needs.  Nothing the compiler
-// emits between the two may write M0: this kernel has no instruction that would (no LDS instruction of gfx950 needs M0),
-// and the tests that hold its results bit for bit against the register-staged kernel's would show a load gone astray.
+// The same in two halves with an MFMA between them as the wait state that the write of M0 needs.  The first half names M0
+// as clobbered; nothing can tell the compiler that the second half reads it, so nothing it emits between the two may
+// write M0.  This kernel has no instruction that would (no LDS instruction of gfx950 needs M0); the build is held to that
+// by a test that reads the compiler's assembly of this file (every global_load_lds is preceded by our own write of M0
+// with exactly one MFMA and no other mention of M0 between), and the tests that hold the results bit for bit against the
+// register-staged kernel's would show a load gone astray.
 __device__ __forceinline__ void dma16_m0(unsigned lds_byte_addr, unsigned stage_offset) {
-  asm volatile("s_add_u32 m0, %0, %1" : : "s"(lds_byte_addr), "s"(stage_offset) : "memory", "scc");
+  asm volatile("s_add_u32 m0, %0, %1" : : "s"(lds_byte_addr), "s"(stage_offset) : "memory", "scc", "m0");
 }
 __device__ __forceinline__ void dma16_go(const void* base, unsigned voff) { asm volatile("global_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base) : "memory"); }
 
@@ -75,10 +78,14 @@ constexpr int BK = 64;
 // k-contiguous operand tile ([rows][64] 16-bit): 128-byte rows of 8 chunks, chunk' = chunk ^ ((row / 2) & 7)
 __device__ __forceinline__ int kc_idx(int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); }  // in 16-byte units
 
-// n-contiguous rhs tile ([64 k][BN n] 16-bit): rows of BN / 32 segments of 64 bytes, segment' = segment ^ (k & mask)
+// n-contiguous rhs tile ([64 k][BN n] 16-bit): rows of BN / 16 pieces of 32 bytes, piece' = piece ^ h(k) with
+// h(k) = (k & 3) | ((k >> 3) & 1) << 2.  A transposing read names, per half wave, 8 rows (k = 8 g + e: e = 0..3 and two values
+// of g) and 32 bytes of each; h sends those rows to 8 different pieces, i.e. to all 64 banks once.  (With 64-byte segments
+// swizzled by k & 7 the two g of a half wave met in the same banks: 4096^3 95.5 -> 94.2 us on one box.)
+__device__ __forceinline__ int kn_h(int k) { return (k & 3) | (((k >> 3) & 1) << 2); }
 template <int BN>
 __device__ __forceinline__ int kn_byte(int k, int n) {
-  return k * (BN * 2) + (((n >> 5) ^ (k & (BN / 32 - 1))) << 6) + (n & 31) * 2;
+  return k * (BN * 2) + (((n >> 4) ^ kn_h(k)) << 5) + (n & 15) * 2;
 }
 
 // Lane l feeds row / column l % 16, k = 8 (l / 16) .. + 7 of a step of 32.  TWO: the schedule with two barriers per K tile.
@@ -138,12 +145,12 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
       const int row = g * 8 + (lane >> 3), cp = lane & 7;
       voff[NDA + i] = (unsigned)(min(row, n_left - 1) * ldb * 2 + ((cp ^ ((row >> 1) & 7)) << 4));
     } else {
-      // one instruction fills 1 KB = 512 / BN rows of k; the lane at LDS position (k, 16-byte chunk c') fetches the
-      // chunk whose 64-byte segment the swizzle maps there
+      // one instruction fills 1 KB = 512 / BN rows of k; the lane at LDS position (k, 16-byte chunk cpos) fetches the
+      // chunk that the swizzle of the row's 32-byte pieces maps there
       constexpr int CPR = BN / 8;  // 16-byte chunks per row
       const int k = g * (64 / CPR) + lane / CPR, cpos = lane % CPR;
-      const int seg = (cpos >> 2) ^ (k & (BN / 32 - 1));
-      voff[NDA + i] = (unsigned)(k * ldb * 2 + (min((seg << 2) | (cpos & 3), n_left / 8 - 1) << 4));  // N % 8 == 0: whole 16-byte chunks
+      const int src = (((cpos >> 1) ^ kn_h(k)) << 1) | (cpos & 1);
+      voff[NDA + i] = (unsigned)(k * ldb * 2 + (min(src, n_left / 8 - 1) << 4));  // N % 8 == 0: whole 16-byte chunks
     }
   }
   const long long a_step = BK * 2, b_step = B_KN ? (long long)BK * ldb * 2 : BK * 2;
@@ -155,6 +162,9 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
   auto dma_m0 = [&](int tile, int idx) {
     const unsigned in_stage = lds_addr + (idx < NDA ? (idx * 4 + wave) * 1024 : A_BYTES + ((idx - NDA) * 4 + wave) * 1024);  // loop invariant
     dma16_m0(in_stage, (tile & 1) * STAGE_BYTES);
+    // the MFMA that follows in the source has to follow in the code: without this the compiler may hoist it above the
+    // write of M0, and the load would then come right behind that write, without the wait state it needs
+    __builtin_amdgcn_sched_barrier(0);
   };
   auto dma_go = [&](int tile, int idx) {
     if (idx < NDA) dma16_go(Ab + tile * a_step, voff[idx]);
@@ -361,7 +371,9 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
     const int row = pass * RPP + r0;
     const u32x2 lo = *(const u32x2 __attribute__((address_space(3)))*)(Cs + row * PITCH + c * 16);
     const u32x2 hi = *(const u32x2 __attribute__((address_space(3)))*)(Cs + row * PITCH + c * 16 + 8);
-    if (row <= m_last && c * 8 < n_left) *reinterpret_cast<u32x4*>(C + (size_t)row * p.N + c * 8) = u32x4{lo.x, lo.y, hi.x, hi.y};
+    // past the cache: nobody in this launch reads the result, and 256 CUs that store their tiles at the same moment are
+    // through sooner when L2 does not hold the lines for the write-back at the kernel's end (8 x 1024^3: 18.7 -> 17.5 us)
+    if (row <= m_last && c * 8 < n_left) __builtin_nontemporal_store(u32x4{lo.x, lo.y, hi.x, hi.y}, reinterpret_cast<u32x4*>(C + (size_t)row * p.N + c * 8));
   }
 }
 
