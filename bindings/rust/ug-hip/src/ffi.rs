@@ -133,6 +133,7 @@ extern "C" {
         out_len: *mut usize,
         info: *mut UghipFuncInfo,
     ) -> c_int;
+    pub fn ughip_set_tuning(name: *const c_char, set: c_int, value: i64) -> c_int;
     pub fn ughip_codegen_min_len(ssa: *const UghipSsa, min_len: *mut i64, n_args: usize) -> c_int;
     pub fn ughip_codegen_as_written(
         ssa: *const UghipSsa,

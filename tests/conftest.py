@@ -51,3 +51,38 @@ def hip():
 def hip_ops():
     import ug_amd
     return ug_amd.LlamaOps.hip()
+
+
+class _Tune:
+    """Tuning switches of the native libraries with monkeypatch's vocabulary: setenv / delenv on UGHIP_<NAME> go to
+    ughip_set_tuning, on UG_LLAMA_<NAME> to the host library's switches (both tables are read from the environment only
+    once per process, so changing os.environ would do nothing); everything set is cleared at teardown."""
+
+    def __init__(self):
+        self.touched = set()
+
+    def setenv(self, name, value):
+        import ug_amd
+        self.touched.add(name)
+        if name.startswith("UG_LLAMA_"):
+            ug_amd.set_llama_switch(name, True)
+        else:
+            ug_amd.set_tuning(name, int(value))
+
+    def delenv(self, name, raising=False):
+        import ug_amd
+        if name.startswith("UG_LLAMA_"):
+            ug_amd.set_llama_switch(name, False)
+        else:
+            ug_amd.set_tuning(name, None)
+
+    def undo(self):
+        for name in self.touched:
+            self.delenv(name)
+
+
+@pytest.fixture
+def tune():
+    t = _Tune()
+    yield t
+    t.undo()

@@ -6,6 +6,14 @@ ids from seed 10, then 128 greedy steps -- once with f32 weights and once with t
 
     python tests/golden/make_llama_config5_fixture.py [--layers 22] [--prompt 128] [--steps 128]
 
+Two more fixtures come from the same script.  BASELINE's weights make every norm vector N(0, 0.02): activations shrink
+fifty-fold at each norm, the logits end up within 1e-4 of each other and the greedy ids fall into a two-cycle, so
+equal ids say little there.  With the norm vectors at 1 + N(0, 0.02) -- what checkpoints hold -- logits spread
+over several units and the ids carry information:
+
+    python tests/golden/make_llama_config5_fixture.py --norm-mean 1 --out tests/golden/llama_config5_unit_norms_greedy.json
+    python tests/golden/make_llama_config5_fixture.py --norm-mean 1 --prompt 1900 --steps 64 --out tests/golden/llama_config5_unit_norms_prompt1900_greedy.json
+
 Per step it keeps the id picked, the largest logit and its gap to the second largest: the GPU tests hold the
 HIP device to these position by position.  About ten minutes on 8 host cores; nothing here needs a GPU.
 The values come from gcc-compiled kernels (-O3 -march=native -ffast-math): another host may differ in the
@@ -28,6 +36,9 @@ def main():
     ap.add_argument("--layers", type=int, default=22)
     ap.add_argument("--prompt", type=int, default=128)
     ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--norm-mean", type=float, default=0.0, help="norm vectors are this + N(0, 0.02)")
+    ap.add_argument("--embed-std", type=float, default=0.0, help="embedding table (tied head) N(0, this) instead of N(0, 0.02)")
+    ap.add_argument("--runs", default="f32,bf16_rounded")
     ap.add_argument("--out", default=os.path.join(ROOT, "tests", "golden", "llama_config5_greedy.json"))
     args = ap.parse_args()
 
@@ -45,11 +56,13 @@ def main():
     prompt = rng.token_ids(10, args.prompt, cfg.vocab_size)
     out = {"config": {"num_hidden_layers": args.layers, "hidden_size": 2048, "intermediate_size": 5632, "num_attention_heads": 32,
                       "num_key_value_heads": 4, "vocab_size": 32000, "max_position_embeddings": 2048, "rope_theta": 10000.0, "rms_norm_eps": 1e-5},
-           "weights": {"seed": 9, "std": 0.02}, "prompt": {"seed": 10, "n": args.prompt}, "steps": args.steps,
+           "weights": {"seed": 9, "std": 0.02, "norm_mean": args.norm_mean, "embed_std": args.embed_std}, "prompt": {"seed": 10, "n": args.prompt}, "steps": args.steps,
            "made_by": "tests/golden/make_llama_config5_fixture.py (CPU oracle, custom softmax, op-by-op graph)", "runs": {}}
     for key, round_bf16 in (("f32", False), ("bf16_rounded", True)):
+        if key not in args.runs.split(","):
+            continue
         t0 = time.perf_counter()
-        model = ug_amd.LlamaModel(cpu, cpu_ops, cfg, custom_softmax=True, seed=9, std=0.02, round_bf16=round_bf16)
+        model = ug_amd.LlamaModel(cpu, cpu_ops, cfg, custom_softmax=True, seed=9, std=0.02, round_bf16=round_bf16, norm_mean=args.norm_mean, embed_std=args.embed_std)
         toks, st = model.generate(prompt, args.steps)
         print(key, "done in", round(time.perf_counter() - t0, 1), "s; ids", toks[:8].tolist(), "min margin", float(st["margins"].min()), flush=True)
         out["runs"][key] = {"ids": toks.tolist(), "top1": [float(v) for v in st["top1"]], "margin": [float(v) for v in st["margins"]]}

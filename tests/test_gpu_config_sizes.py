@@ -95,13 +95,13 @@ def test_config3_bmm_bf16(hip, rhs_nk):
 @pytest.mark.parametrize("dtype_name", ["f32", "bf16"])
 @pytest.mark.parametrize("rhs_nk", [False, True], ids=["NN", "NT"])
 @pytest.mark.parametrize("bmnk,split", [((2, 256, 128, 96 * 2), 0), ((1, 512, 256, 64), 0), ((1, 256, 128, 1024), 4), ((3, 256, 384, 128), 0)])
-def test_matmul_256x128_tile_forced(hip, monkeypatch, bmnk, split, rhs_nk, dtype_name):
+def test_matmul_256x128_tile_forced(hip, tune, bmnk, split, rhs_nk, dtype_name):
     """The 256 x 128, 8-wave tile on problems small enough for an exact check: forced through UGHIP_GEMM_SHAPE=0
     (the dispatcher only picks it from 256 tiles up), with and without a K split."""
     b, m, n, k = bmnk
-    monkeypatch.setenv("UGHIP_GEMM_SHAPE", "0")
+    tune.setenv("UGHIP_GEMM_SHAPE", "0")
     if split:
-        monkeypatch.setenv("UGHIP_GEMM_SPLIT", str(split))
+        tune.setenv("UGHIP_GEMM_SPLIT", str(split))
     dtype = F32 if dtype_name == "f32" else ug_amd.BF16
     a = rng.uniform_pm1(71, b * m * k).reshape(b, m, k)
     w = rng.uniform_pm1(72, b * k * n).reshape(b, k, n)
@@ -314,18 +314,17 @@ LOGIT_TOL = 2e-5
 TIE_MARGIN = 2 * LOGIT_TOL
 
 
-def _config5_fixture():
-    with open(os.path.join(HERE, "golden", "llama_config5_greedy.json")) as f:
+def _config5_fixture(name="llama_config5_greedy.json"):
+    with open(os.path.join(HERE, "golden", name)) as f:
         return json.load(f)
 
 
-@pytest.mark.parametrize("variant", ["f32_level0", "f32_level3", "bf16_rounded_level0", "bf16_matrices_level3", "bf16_matrices_level3_x3"])
-def test_config5_full_depth_greedy_ids(hip, hip_ops, variant):
-    """BASELINE config 5 as stated against the oracle's run of the reference's op-by-op graph (the fixture):
-    free-running ids equal up to the first position where the oracle itself holds a near-tie, and -- fed the
-    oracle's ids, so that every position sees the same inputs -- the same id at every position outside the tie band,
-    top logits within LOGIT_TOL and margins within 2 LOGIT_TOL."""
-    fx = _config5_fixture()
+def _check_config5(hip, hip_ops, fx, variant, logit_tol, min_clear_frac, free_must_match=False):
+    """One fixture (the oracle's run of the reference's op-by-op graph) against one way of running the model on the HIP
+    device: free-running ids equal up to the first position where the oracle itself holds a near-tie (everywhere when
+    free_must_match), and -- fed the oracle's ids, so that every position sees the same inputs -- the same id at every
+    position outside the tie band (2 logit_tol), top logits within logit_tol and margins within 2 logit_tol."""
+    tie = 2 * logit_tol
     run = fx["runs"]["f32" if variant.startswith("f32") else "bf16_rounded"]
     ids_o, top_o, mar_o = np.array(run["ids"], np.int32), np.array(run["top1"]), np.array(run["margin"])
     n_steps = fx["steps"]
@@ -337,26 +336,56 @@ def test_config5_full_depth_greedy_ids(hip, hip_ops, variant):
     hip.set_zero_fill(False)
     try:
         model = ug_amd.LlamaModel(hip, hip_ops, cfg, custom_softmax=True, seed=fx["weights"]["seed"], std=fx["weights"]["std"], round_bf16=not variant.startswith("f32"),
-                                  fused_attention=level, bf16_matrices=variant.startswith("bf16_matrices"))
+                                  fused_attention=level, bf16_matrices=variant.startswith("bf16_matrices"),
+                                  norm_mean=fx["weights"].get("norm_mean", 0.0), embed_std=fx["weights"].get("embed_std", 0.0))
         free, st_free = model.generate(prompt, n_steps)
         forced, st = model.generate(prompt, n_steps, forced=ids_o[:-1])
     finally:
         hip.set_zero_fill(True)
-    clear = mar_o > TIE_MARGIN
+    clear = mar_o > tie
     differs = np.flatnonzero(free != ids_o)
     first = int(differs[0]) if differs.size else None
-    print(f"config 5 {variant}: free-running ids equal at {int((free == ids_o).sum())}/{ids_o.size} positions, first difference {first}; "
-          f"fed the oracle's ids: equal at {int((forced == ids_o).sum())}/{ids_o.size}, {int(clear.sum())} positions outside the tie band, "
-          f"max |top1 - oracle| {float(np.abs(st['top1'] - top_o).max()):.3g}, max |margin - oracle| {float(np.abs(st['margins'] - mar_o).max()):.3g}, "
+    print(f"config 5 {variant} (prompt {fx['prompt']['n']}, norm mean {fx['weights'].get('norm_mean', 0.0)}): free-running ids equal at {int((free == ids_o).sum())}/{ids_o.size} positions, "
+          f"first difference {first}; fed the oracle's ids: equal at {int((forced == ids_o).sum())}/{ids_o.size}, {int(clear.sum())} positions outside the tie band, "
+          f"distinct ids {len(set(ids_o.tolist()))}, max |top1 - oracle| {float(np.abs(st['top1'] - top_o).max()):.3g}, max |margin - oracle| {float(np.abs(st['margins'] - mar_o).max()):.3g}, "
           f"oracle margins min {mar_o.min():.3g} median {np.median(mar_o):.3g}", flush=True)
     for i in range(ids_o.size):
         print(f"  pos {i:3d} oracle id {ids_o[i]:5d} margin {mar_o[i]:.3e} | hip (same inputs) id {forced[i]:5d} margin {st['margins'][i]:.3e} | hip free id {free[i]:5d}", flush=True)
     assert np.all(forced[clear] == ids_o[clear])
-    np.testing.assert_allclose(st["top1"], top_o, rtol=0, atol=LOGIT_TOL)
-    np.testing.assert_allclose(st["margins"], mar_o, rtol=0, atol=2 * LOGIT_TOL)
+    np.testing.assert_allclose(st["top1"], top_o, rtol=0, atol=logit_tol)
+    np.testing.assert_allclose(st["margins"], mar_o, rtol=0, atol=2 * logit_tol)
     if first is not None:
-        assert mar_o[first] <= TIE_MARGIN, f"free-running ids part at position {first} where the oracle's margin is {mar_o[first]}"
-    assert clear.sum() >= ids_o.size // 2, "most positions should lie outside the tie band for the id comparison to mean something"
+        assert not free_must_match, f"free-running ids part at position {first}"
+        assert mar_o[first] <= tie, f"free-running ids part at position {first} where the oracle's margin is {mar_o[first]}"
+    assert clear.sum() >= min_clear_frac * ids_o.size, "too few positions outside the tie band for the id comparison to mean something"
+
+
+@pytest.mark.parametrize("variant", ["f32_level0", "f32_level3", "bf16_rounded_level0", "bf16_matrices_level3", "bf16_matrices_level3_x3"])
+def test_config5_full_depth_greedy_ids(hip, hip_ops, variant):
+    """BASELINE config 5 as stated (every weight N(0, 0.02), norm vectors included) against the oracle's fixture.  The norms
+    shrink the activations fifty-fold each, the logits lie within 1e-4 of each other and the ids fall into a two-cycle: the
+    logit comparison carries this test, half the positions are asked to lie outside the tie band."""
+    _check_config5(hip, hip_ops, _config5_fixture(), variant, LOGIT_TOL, 0.5)
+
+
+# The same model with norm vectors 1 + N(0, 0.02), what checkpoints hold: logits of 3 to 5, a median gap of 0.15 between
+# the two best and 113 distinct ids in 129 positions, so equal ids mean something.  On logits of that size the f32 rounding
+# of 22 layers in two summation orders shows as 1.5e-5 to 2.3e-5 (measured, all five variants); UNIT_LOGIT_TOL bounds it
+# nine-fold, and the oracle's smallest margin (2.5e-3) is still six tie bands wide: the free-running ids must be identical.
+UNIT_LOGIT_TOL = 2e-4
+
+
+@pytest.mark.parametrize("variant", ["f32_level0", "f32_level3", "bf16_rounded_level0", "bf16_matrices_level3", "bf16_matrices_level3_x3"])
+def test_config5_unit_norms_greedy_ids(hip, hip_ops, variant):
+    _check_config5(hip, hip_ops, _config5_fixture("llama_config5_unit_norms_greedy.json"), variant, UNIT_LOGIT_TOL, 0.9, free_must_match=True)
+
+
+@pytest.mark.parametrize("variant", ["f32_level3", "bf16_matrices_level3", "bf16_matrices_level3_x3"])
+def test_config5_unit_norms_prompt_of_1900_tokens(hip, hip_ops, variant):
+    """A prompt that fills the caches to 1900 of their 2048 rows, then 64 steps: the long-prompt kernels (key ranges split
+    over workgroups and merged, the three-term bf16 products on the one-wave-per-SIMD kernel with a K split) at the model
+    level, against the oracle's fixture."""
+    _check_config5(hip, hip_ops, _config5_fixture("llama_config5_unit_norms_prompt1900_greedy.json"), variant, UNIT_LOGIT_TOL, 0.9, free_must_match=True)
 
 
 def test_generate_refuses_ids_outside_the_vocabulary(hip, hip_ops):

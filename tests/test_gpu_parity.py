@@ -396,12 +396,8 @@ def test_matmul_16bit_one_wave_per_simd_tiles(hip, bmnk, bn, rhs_nk, dtype):
     dt = ug_amd.BF16 if dtype == "bf16" else ug_amd.F16
     a = rnd(rng.uniform_pm1(25, b * m * k)).reshape(b, m, k)
     w = rnd(rng.uniform_pm1(26, b * k * n)).reshape(b, k, n)
-    import os
-    os.environ["UGHIP_GEMM_SHAPE"] = {256: "3", 128: "4", 64: "5"}[bn]   # K this short is a toss-up between the kernels: the choice is tested below
-    try:
+    with ug_amd.tuning(GEMM_SHAPE={256: 3, 128: 4, 64: 5}[bn]):   # K this short is a toss-up between the kernels: the choice is tested below
         got = _raw_matmul(hip, dt, a, w, rhs_nk)
-    finally:
-        del os.environ["UGHIP_GEMM_SHAPE"]
     tile = {256: "256x256", 128: "256x128", 64: "128x128"}[bn]
     assert ug_amd.last_kernel() == f"gemm_dma4<{dtype},{'NT' if rhs_nk else 'NN'},{tile},256t>"
     exact = np.matmul(a.astype(np.float64), w.astype(np.float64))
@@ -409,13 +405,9 @@ def test_matmul_16bit_one_wave_per_simd_tiles(hip, bmnk, bn, rhs_nk, dtype):
     bound = half_ulp * np.abs(exact) + k * np.finfo(np.float32).eps * np.matmul(np.abs(a).astype(np.float64), np.abs(w).astype(np.float64))
     assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-7)
     # the same product through the register-staged 256 x 128 kernel: same k order, bit for bit
-    import os
-    os.environ["UGHIP_GEMM_SHAPE"] = "0"
-    try:
+    with ug_amd.tuning(GEMM_SHAPE=0):
         other = _raw_matmul(hip, dt, a, w, rhs_nk)
         assert ug_amd.last_kernel().startswith("gemm_tiled<")
-    finally:
-        del os.environ["UGHIP_GEMM_SHAPE"]
     np.testing.assert_array_equal(got, other)
     # small integers: every partial sum is exact, so the result is the integer product bit for bit
     ai, wi = np.floor(a * 4), np.floor(w * 4)
@@ -424,7 +416,7 @@ def test_matmul_16bit_one_wave_per_simd_tiles(hip, bmnk, bn, rhs_nk, dtype):
     np.testing.assert_array_equal(_raw_matmul(hip, dt, ai, wi, rhs_nk), want)
 
 
-def test_matmul_16bit_one_wave_per_simd_random_shapes(hip, monkeypatch):
+def test_matmul_16bit_one_wave_per_simd_random_shapes(hip, tune):
     """Seeded random shapes (rows from 9 up to a few tiles, columns any multiple of 8, 4 to 9 K tiles, one to three
     batches, both rhs layouts and both 16-bit types) through each of the kernel's three tiles: float64 bound and the guard
     region behind the result."""
@@ -438,7 +430,7 @@ def test_matmul_16bit_one_wave_per_simd_random_shapes(hip, monkeypatch):
         rnd = (lambda v: v.astype(np.float16).astype(np.float32)) if f16 else rng.bf16_round
         a = rnd(rng.uniform_pm1(700 + case, b * m * k)).reshape(b, m, k)
         w = rnd(rng.uniform_pm1(800 + case, b * k * n)).reshape(b, k, n)
-        monkeypatch.setenv("UGHIP_GEMM_SHAPE", shape)
+        tune.setenv("UGHIP_GEMM_SHAPE", shape)
         got = _raw_matmul(hip, ug_amd.F16 if f16 else ug_amd.BF16, a, w, rhs_nk)
         assert ug_amd.last_kernel().startswith("gemm_dma4<"), ug_amd.last_kernel()
         exact = np.matmul(a.astype(np.float64), w.astype(np.float64))
@@ -469,17 +461,17 @@ def test_matmul_16bit_kernel_choice(hip, bmnk, want):
     assert np.all(np.abs(got[:, rows] - exact) <= bound * 1.001 + 1e-7)
 
 
-def test_matmul_16bit_one_wave_per_simd_forced_and_limits(hip, monkeypatch):
+def test_matmul_16bit_one_wave_per_simd_forced_and_limits(hip, tune):
     """UGHIP_GEMM_SHAPE=3 / 4 / 5 force the kernel's three tiles onto a small problem (bit for bit the register-staged
     kernel's result); shapes it cannot take (K below 4 tiles, a column count that is not a multiple of 8) fall through to
     that kernel."""
     a = rng.bf16_round(rng.uniform_pm1(27, 2 * 512 * 256)).reshape(2, 512, 256)
     w = rng.bf16_round(rng.uniform_pm1(28, 2 * 256 * 256)).reshape(2, 256, 256)
-    monkeypatch.setenv("UGHIP_GEMM_SHAPE", "1")
+    tune.setenv("UGHIP_GEMM_SHAPE", "1")
     plain = _raw_matmul(hip, ug_amd.BF16, a, w, False)
     assert ug_amd.last_kernel().startswith("gemm_tiled<")
     for shape, tile in (("3", "256x256"), ("4", "256x128"), ("5", "128x128")):
-        monkeypatch.setenv("UGHIP_GEMM_SHAPE", shape)
+        tune.setenv("UGHIP_GEMM_SHAPE", shape)
         for rhs_nk in (True, False):
             got = _raw_matmul(hip, ug_amd.BF16, a, w, rhs_nk)
             assert ug_amd.last_kernel() == f"gemm_dma4<bf16,{'NT' if rhs_nk else 'NN'},{tile},256t>"
@@ -493,7 +485,7 @@ def test_matmul_16bit_one_wave_per_simd_forced_and_limits(hip, monkeypatch):
 @pytest.mark.parametrize("dtype", ["bf16", "f16"])
 @pytest.mark.parametrize("rhs_nk", [True, False], ids=["NT", "NN"])
 @pytest.mark.parametrize("bmnk", [(1, 300, 264, 256), (2, 257, 136, 320), (1, 1900, 520, 256), (3, 9, 8, 256), (1, 511, 248, 448), (1, 700, 392, 576)])
-def test_matmul_16bit_one_wave_per_simd_ragged(hip, monkeypatch, bmnk, rhs_nk, dtype):
+def test_matmul_16bit_one_wave_per_simd_ragged(hip, tune, bmnk, rhs_nk, dtype):
     """Rows and columns the 256-wide tiles do not divide (any M, N a multiple of 8): the last tiles hang over the end,
     read the last row again and store only what exists.  Both tile widths, forced; float64 bound, no write past the end
     (the guard region of _raw_matmul), and bit for bit the register-staged kernel where that takes the shape."""
@@ -506,10 +498,10 @@ def test_matmul_16bit_one_wave_per_simd_ragged(hip, monkeypatch, bmnk, rhs_nk, d
     exact = np.matmul(a.astype(np.float64), w.astype(np.float64))
     half_ulp = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
     bound = half_ulp * np.abs(exact) + k * np.finfo(np.float32).eps * np.matmul(np.abs(a).astype(np.float64), np.abs(w).astype(np.float64))
-    monkeypatch.setenv("UGHIP_GEMM_SHAPE", "1")
+    tune.setenv("UGHIP_GEMM_SHAPE", "1")
     other = _raw_matmul(hip, dt, a, w, rhs_nk) if rhs_nk or n % 128 == 0 else None   # the 128-row tiles take any N only with an [n, k]-major rhs
     for shape, tile in (("3", "256x256"), ("4", "256x128"), ("5", "128x128")):
-        monkeypatch.setenv("UGHIP_GEMM_SHAPE", shape)
+        tune.setenv("UGHIP_GEMM_SHAPE", shape)
         got = _raw_matmul(hip, dt, a, w, rhs_nk)
         assert ug_amd.last_kernel() == f"gemm_dma4<{dtype},{'NT' if rhs_nk else 'NN'},{tile},256t>"
         assert np.all(np.abs(got - exact) <= bound * 1.001 + 1e-7)
@@ -945,11 +937,8 @@ def test_attention_decode_key_ranges(hip, hip_ops, b, nh, nkv, s, d):
     scale = float(np.float32(d) ** np.float32(-0.5))
 
     def run(n):
-        os.environ["UGHIP_ATT_SPLIT"] = str(n)
-        try:
+        with ug_amd.tuning(ATT_SPLIT=n):
             return hip_ops.attention_decode(LB.copy(q, (b, nh, 1, d), hip), LB.copy(k, (b, nkv, s, d), hip), LB.copy(v, (b, nkv, s, d), hip), scale).data_vec()
-        finally:
-            del os.environ["UGHIP_ATT_SPLIT"]
 
     one = run(1)
     q6, k6, v6 = q.reshape(b, nh, d).astype(np.float64), k.reshape(b, nkv, s, d).astype(np.float64), v.reshape(b, nkv, s, d).astype(np.float64)
@@ -1502,7 +1491,7 @@ def test_bf16_matrices_meet_a_few_rows(hip, hip_ops, t):
 
 @pytest.mark.parametrize("t,k,n", [(128, 2048, 2048), (128, 5632, 2048), (100, 256, 192), (37, 64, 48), (9, 32, 16), (300, 512, 1000), (64, 2048, 2048), (16, 512, 264)])
 @pytest.mark.parametrize("bf16", [False, True])
-def test_projections_of_several_rows_with_the_neighbour_in_the_fold(hip, cpu, hip_ops, cpu_ops, monkeypatch, t, k, n, bf16):
+def test_projections_of_several_rows_with_the_neighbour_in_the_fold(hip, cpu, hip_ops, cpu_ops, tune, t, k, n, bf16):
     """Prefill shapes: linear_add and gate_up_stacked over 9 or more rows fold the residual add / SwiGLU into the fold of
     the split-K partial tiles.  Against the oracle's op-by-op composition (matmul_t, add / silu, mul), against float64, and
     against the same hooks with the folding switched off: where both split K alike, the residual form is bit for bit the
@@ -1532,7 +1521,7 @@ def test_projections_of_several_rows_with_the_neighbour_in_the_fold(hip, cpu, hi
     assert np.all(np.abs(o_hip - o64) <= o_bound) and np.all(np.abs(o_cpu - o64) <= o_bound)
     g_bound = k * eps * ((np.abs(x64) @ np.abs(gu64[:n]).T) * (np.abs(uu) * 1.3) + (np.abs(x64) @ np.abs(gu64[n:]).T) * np.abs(gg / (1.0 + np.exp(-gg)))) + 8 * eps * np.abs(g64) + 1e-7
     assert np.all(np.abs(g_hip - g64) <= g_bound) and np.all(np.abs(g_cpu - g64) <= g_bound)
-    monkeypatch.setenv("UG_LLAMA_NO_FOLD_EPILOGUES", "1")
+    tune.setenv("UG_LLAMA_NO_FOLD_EPILOGUES", "1")
     o_two, g_two = run(hip, hip_ops, True)
     if t == 128:       # the prefill shapes split K the same way with and without the neighbour: the same sums in the same order
         np.testing.assert_array_equal(o_hip, o_two)
@@ -1615,11 +1604,35 @@ def test_projections_of_several_rows_as_three_bf16_terms(hip, t, k, n):
         np.testing.assert_array_equal(back[:, :k], full)
 
 
+def test_three_bf16_terms_keep_infinities_and_nans_where_the_f32_pipe_has_them(hip):
+    """An infinite or NaN row element is all in the first of the three terms (its remainders would be inf - inf): the
+    product then has infinities and NaNs exactly where the f32 pipe has them, and finite rows are untouched."""
+    import ctypes as C
+    t, k, n = 128, 256, 192
+    x = rng.normal(171, t * k).reshape(t, k)
+    x[3, 17], x[5, 200], x[9, 0] = np.inf, -np.inf, np.nan
+    w = rng.bf16_round(rng.normal(172, n * k, 0.05)).reshape(n, k)
+    w[7, 17] = 0.0            # inf x 0: NaN on either pipe
+    lib, dev, z = ug_amd.ughip_lib(), C.c_void_p(hip.raw_hip()), C.c_size_t
+    sx, sw = hip.slice_from(x.ravel()), hip.slice_from(rng.to_bf16_bits(w.ravel()))
+    out = []
+    for product in (0, 1):    # UGHIP_PRODUCT_F32, UGHIP_PRODUCT_BF16X3
+        d = hip.allocate_uninit(ug_amd.F32, t * n)
+        assert lib.ughip_linear_rows(dev, C.c_void_p(sx.raw()), C.c_void_p(sw.raw()), C.c_void_p(d.raw()), z(t), z(n), z(k), C.c_int(product)) == 0, lib.ughip_last_error()
+        out.append(d.to_vec().reshape(t, n))
+    f32, x3 = out
+    assert np.array_equal(np.isnan(f32), np.isnan(x3)) and np.array_equal(np.isposinf(f32), np.isposinf(x3)) and np.array_equal(np.isneginf(f32), np.isneginf(x3))
+    assert np.isposinf(x3[3]).sum() + np.isneginf(x3[3]).sum() == n - 1 and np.isnan(x3[3, 7]) and np.all(np.isnan(x3[9]))
+    fin = np.isfinite(f32)
+    assert fin[[0, 1, 2, 4, 127]].all()
+    np.testing.assert_allclose(x3[fin], f32[fin], rtol=0, atol=k * float(np.finfo(np.float32).eps) * 4.0)
+
+
 @pytest.mark.parametrize("t,k,n,force,split", [(400, 512, 640, "3", None), (400, 512, 640, "4", None), (400, 512, 640, "5", None), (517, 256, 264, "5", None),
                                                (390, 1024, 1032, "4", None), (1900, 2048, 2560, None, None), (1100, 2048, 2048, None, None),
                                                (400, 512, 640, "3", "2"), (390, 1024, 1032, "4", "4"), (517, 768, 264, "5", "2"), (1100, 2048, 2048, "4", "8"),
                                                (1900, 5632, 2048, None, None)])
-def test_three_bf16_terms_on_the_one_wave_per_simd_kernel(hip, monkeypatch, t, k, n, force, split):
+def test_three_bf16_terms_on_the_one_wave_per_simd_kernel(hip, tune, t, k, n, force, split):
     """Many rows of three bf16 planes take gemm_dma4 (f32 result straight from the accumulators, the residual added on the
     way, SwiGLU through the scratch block and the fold; with K split over workgroups, f32 slabs and the fold for all three).
     Forced tiles and splits on small ragged shapes, the library's own choice on prompts of a thousand positions and more; against float64 with the k eps bound of the f32 product, against the
@@ -1651,9 +1664,9 @@ def test_three_bf16_terms_on_the_one_wave_per_simd_kernel(hip, monkeypatch, t, k
         return out, kerns
 
     if force:
-        monkeypatch.setenv("UGHIP_X3_DMA", force)
+        tune.setenv("UGHIP_X3_DMA", force)
     if split:
-        monkeypatch.setenv("UGHIP_X3_SPLIT", split)
+        tune.setenv("UGHIP_X3_SPLIT", split)
     (lin, add, glu), kerns = run(x, w, wgu)
     tile = {"3": "256x256", "4": "256x128", "5": "128x128"}.get(force, "")
     for kn, word in zip(kerns, ("f32 out", "residual", "swiglu fold")):
@@ -1661,8 +1674,8 @@ def test_three_bf16_terms_on_the_one_wave_per_simd_kernel(hip, monkeypatch, t, k
         assert ("splitK=" + split in kn) if split else True, kn
     if (t, k, n) == (1900, 5632, 2048):
         assert "splitK=" in kerns[0], kerns   # 64 tiles of 256 x 256 and 264 K tiles: the library splits K by itself
-    monkeypatch.delenv("UGHIP_X3_SPLIT", raising=False)
-    monkeypatch.setenv("UGHIP_X3_DMA", "0")
+    tune.delenv("UGHIP_X3_SPLIT", raising=False)
+    tune.setenv("UGHIP_X3_DMA", "0")
     (lin0, add0, glu0), kerns0 = run(x, w, wgu)
     assert all(kn.startswith("gemm_tiled<bf16,NT,") for kn in kerns0), kerns0
     x64, w64, gu64 = x.reshape(t, k).astype(np.float64), w.reshape(n, k).astype(np.float64), wgu.reshape(2 * n, k).astype(np.float64)
@@ -1679,11 +1692,11 @@ def test_three_bf16_terms_on_the_one_wave_per_simd_kernel(hip, monkeypatch, t, k
     assert np.all(np.abs(glu - glu0) <= 2 * g_bound)
     # small integers: every partial sum is exact
     if force:
-        monkeypatch.setenv("UGHIP_X3_DMA", force)
+        tune.setenv("UGHIP_X3_DMA", force)
     else:
-        monkeypatch.delenv("UGHIP_X3_DMA")
+        tune.delenv("UGHIP_X3_DMA")
     if split:
-        monkeypatch.setenv("UGHIP_X3_SPLIT", split)
+        tune.setenv("UGHIP_X3_SPLIT", split)
     xi, wi, gui = np.floor(x * 4).astype(np.float32), np.floor(w * 40).astype(np.float32), np.floor(wgu * 40).astype(np.float32)
     (lin_i, add_i, _), kerns_i = run(xi, wi, gui)
     assert kerns_i[0].startswith("gemm_dma4<"), kerns_i
@@ -2006,7 +2019,7 @@ def test_argmax_into(hip, hip_ops, rows, n, row):
 
 
 @pytest.mark.parametrize("level,n_steps", [(0, 12), (3, 12), (3, 400)])
-def test_queued_greedy_decode_matches_the_read_back_loop(hip, hip_ops, level, n_steps, monkeypatch):
+def test_queued_greedy_decode_matches_the_read_back_loop(hip, hip_ops, level, n_steps, tune):
     """Tokens picked on the device and fed to the next step without a read-back: same ids and
     margins as the loop that copies the logits to the host for every token.  400 steps let the
     launches run far ahead of the device and recycle every buffer of the pool many times."""
@@ -2014,7 +2027,7 @@ def test_queued_greedy_decode_matches_the_read_back_loop(hip, hip_ops, level, n_
     prompt = rng.token_ids(10, 16, cfg.vocab_size)
     model = ug_amd.LlamaModel(hip, hip_ops, cfg, True, seed=9, std=0.02, fused_attention=level)
     ids_q, st_q = model.generate(prompt, n_steps)
-    monkeypatch.setenv("UG_LLAMA_HOST_ARGMAX", "1")
+    tune.setenv("UG_LLAMA_HOST_ARGMAX", "1")
     ids_h, st_h = model.generate(prompt, n_steps)
     assert ids_q.tolist() == ids_h.tolist()
     np.testing.assert_array_equal(st_q["margins"], st_h["margins"])

@@ -24,18 +24,20 @@ def weight(name, *shape):
 
 
 class NumpyLlama:
-    def __init__(self, cfg):
+    def __init__(self, cfg, norm_mean=0.0):
         self.cfg = cfg
         h, isz = cfg.hidden_size, cfg.intermediate_size
         self.nh, self.nkv, self.hd = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
         kv = self.nkv * self.hd
         self.embed = weight("model.embed_tokens.weight", cfg.vocab_size, h)
-        self.norm = weight("model.norm.weight", h)
+        def norm_w(name):   # norm vectors are norm_mean + N(0, std), summed in f32 like the generator does
+            return (np.float32(norm_mean) + weight(name, h).astype(np.float32)).astype(np.float64)
+        self.norm = norm_w("model.norm.weight")
         self.layers = []
         for i in range(cfg.num_hidden_layers):
             p = f"model.layers.{i}"
             self.layers.append(dict(
-                rms1=weight(p + ".input_layernorm.weight", h), rms2=weight(p + ".post_attention_layernorm.weight", h),
+                rms1=norm_w(p + ".input_layernorm.weight"), rms2=norm_w(p + ".post_attention_layernorm.weight"),
                 gate=weight(p + ".mlp.gate_proj.weight", isz, h), up=weight(p + ".mlp.up_proj.weight", isz, h), down=weight(p + ".mlp.down_proj.weight", h, isz),
                 q=weight(p + ".self_attn.q_proj.weight", h, h), k=weight(p + ".self_attn.k_proj.weight", kv, h),
                 v=weight(p + ".self_attn.v_proj.weight", kv, h), o=weight(p + ".self_attn.o_proj.weight", h, h)))
@@ -116,3 +118,18 @@ def test_llama_restatement_matches_numpy_f64(cpu, cpu_ops, interleaved, custom_s
     assert ids.tolist() == want_ids.tolist()
     np.testing.assert_allclose(st["margins"], want_margins, rtol=1e-3, atol=1e-4)
     assert want_margins.min() > 1e-3   # the comparison of ids is not decided by rounding
+
+
+@pytest.mark.parametrize("fused", [0, 3])
+def test_llama_with_norm_vectors_around_one_matches_numpy_f64(cpu, cpu_ops, fused):
+    """norm_mean = 1 (the weights of the second config-5 fixture: norm vectors 1 + N(0, std) as checkpoints hold them)."""
+    cfg = ug_amd.LlamaConfig(hidden_size=128, intermediate_size=320, max_position_embeddings=64, num_attention_heads=4, num_key_value_heads=2,
+                             num_hidden_layers=2, vocab_size=512)
+    prompt = rng.token_ids(10, 12, cfg.vocab_size)
+    want_ids, want_margins = NumpyLlama(cfg, norm_mean=1.0).generate(prompt.tolist(), 6)
+    model = ug_amd.LlamaModel(cpu, cpu_ops, cfg, True, seed=SEED, std=STD, fused_attention=fused, norm_mean=1.0)
+    ids, st = model.generate(prompt, 6)
+    assert ids.tolist() == want_ids.tolist()
+    np.testing.assert_allclose(st["margins"], want_margins, rtol=1e-3, atol=1e-4)
+    plain, _ = ug_amd.LlamaModel(cpu, cpu_ops, cfg, True, seed=SEED, std=STD).generate(prompt, 6)
+    assert plain.tolist() != ids.tolist()      # the option changes the model

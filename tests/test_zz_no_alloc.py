@@ -83,12 +83,12 @@ def test_noalloc_other_shapes_match(hip, bmnk, rhs_nk):
     np.testing.assert_array_equal(got, ref)
 
 
-def test_noalloc_refuses_what_does_not_fit(hip, monkeypatch):
+def test_noalloc_refuses_what_does_not_fit(hip, tune):
     """A forced 32-way split of a 1024 x 1024 result needs 128 MiB of partial tiles: refused with both sizes in the
     message and nothing launched; ughip_matmul takes the same call."""
     b, m, n, k = 1, 1024, 1024, 4096
-    monkeypatch.setenv("UGHIP_GEMM_SHAPE", "1")
-    monkeypatch.setenv("UGHIP_GEMM_SPLIT", "32")
+    tune.setenv("UGHIP_GEMM_SHAPE", "1")
+    tune.setenv("UGHIP_GEMM_SPLIT", "32")
     sa, sw = hip.slice_from(np.ones(m * k, np.float32)), hip.slice_from(np.ones(k * n, np.float32))
     dst = hip.slice_from(np.full(m * n, 7.0, np.float32))
     rc, err, _ = _call("ughip_matmul_noalloc", hip, dst, sa, sw, b, m, n, k, True)

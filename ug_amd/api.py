@@ -1,6 +1,7 @@
 """ctypes bindings: the same names and argument meaning as ug's Rust API for this path
 (`LazyBuffer` builders of ug-core/src/lazy_buffer.rs, `Schedule`, `Device`/`Slice`), so tests
 read like the reference's own (ug-core/tests/lb_tests.rs, ug-core/src/common_tests.rs)."""
+import contextlib
 import ctypes as C
 import os
 
@@ -341,6 +342,43 @@ class Device(_Handle):
 def last_kernel():
     """The hand-written kernel this thread's last Device.matmul launched (ughip_last_kernel)."""
     return ughip_lib().ughip_last_kernel().decode()
+
+
+def set_tuning(name, value=None):
+    """One tuning switch of the backend (ughip_set_tuning): value None clears it.  The table is read from the environment
+    (UGHIP_<NAME>) once per process; later changes of the environment are not seen, this call is."""
+    lib = ughip_lib()
+    if lib.ughip_set_tuning(name.encode(), 0 if value is None else 1, C.c_int64(0 if value is None else int(value))):
+        raise UgError(lib.ughip_last_error().decode())
+
+
+@contextlib.contextmanager
+def tuning(**switches):
+    """with tuning(GEMM_SHAPE=0, GEMM_SPLIT=4): ...  -- sets the switches, clears them again on the way out."""
+    for k, v in switches.items():
+        set_tuning(k, v)
+    try:
+        yield
+    finally:
+        for k in switches:
+            set_tuning(k, None)
+
+
+def set_llama_switch(name, on=True):
+    """A switch of the host-side llama loops and hooks (NO_FOLD_EPILOGUES, NO_APPEND_PAIR, VERBOSE, NO_LAYER_STEPS,
+    HOST_ARGMAX, NO_OVERLAP); like the backend's table, read from the environment (UG_LLAMA_<NAME>) once per process."""
+    _chk(host_lib().ugh_llama_set_switch(name.encode(), int(bool(on))))
+
+
+@contextlib.contextmanager
+def llama_switches(*names):
+    for n in names:
+        set_llama_switch(n, True)
+    try:
+        yield
+    finally:
+        for n in names:
+            set_llama_switch(n, False)
 
 
 def hip_device(ordinal=0):
@@ -853,10 +891,12 @@ class LlamaModel(_Handle):
     """ug_llama::Model with random-init weights N(0, std) from the seeded generator."""
     _free = "ugh_llama_model_free"
 
-    def __init__(self, device, ops, cfg, custom_softmax=False, seed=9, std=0.02, round_bf16=False, fused_attention=False, bf16_matrices=False):
+    def __init__(self, device, ops, cfg, custom_softmax=False, seed=9, std=0.02, round_bf16=False, fused_attention=False, bf16_matrices=False,
+                 norm_mean=0.0, embed_std=0.0):
+        """norm_mean: the norm vectors are norm_mean + N(0, std); embed_std > 0: the embedding table (= the tied head) is N(0, embed_std)."""
         out = C.c_void_p()
-        _chk(host_lib().ugh_llama_model_new(_p(device.h), _p(ops.h), C.byref(cfg), int(custom_softmax), C.c_uint64(seed), C.c_float(std),
-                                            int(round_bf16), C.byref(out)))
+        _chk(host_lib().ugh_llama_model_new_ex(_p(device.h), _p(ops.h), C.byref(cfg), int(custom_softmax), C.c_uint64(seed), C.c_float(std),
+                                               int(round_bf16), C.c_float(norm_mean), C.c_float(embed_std), C.byref(out)))
         super().__init__(out.value)
         if fused_attention:
             _chk(host_lib().ugh_llama_model_set_fused_attention(_p(self.h), int(fused_attention)))
@@ -901,4 +941,6 @@ class LlamaModel(_Handle):
         _chk(host_lib().ugh_llama_generate_ex(_p(self.h), prompt.ctypes.data_as(C.c_void_p), C.c_size_t(prompt.size), C.c_size_t(n_steps), fp,
                                               toks.ctypes.data_as(C.c_void_p), C.byref(pre), C.byref(dec), margins.ctypes.data_as(C.c_void_p),
                                               top1.ctypes.data_as(C.c_void_p)))
-        return toks, {"prefill_ms": pre.value, "decode_ms": dec.value, "margins": margins, "top1": top1}
+        items = host_lib().ugh_llama_last_decode_items
+        items.restype = C.c_size_t
+        return toks, {"prefill_ms": pre.value, "decode_ms": dec.value, "margins": margins, "top1": top1, "decode_items": int(items())}

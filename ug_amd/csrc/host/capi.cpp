@@ -785,6 +785,13 @@ int ugh_llama_model_new(void* d, void* ops, const ugh_llama_config* c, int custo
     *out = new ug_llama::Model(cfg_of(c), custom_softmax != 0, *w, dev_of(d), *static_cast<OpsPtr*>(ops));
   });
 }
+int ugh_llama_model_new_ex(void* d, void* ops, const ugh_llama_config* c, int custom_softmax, uint64_t seed, float std, int round_bf16, float norm_mean, float embed_std,
+                           void** out) {
+  return guard([&] {
+    auto w = ug_llama::synthetic_weights(seed, std, round_bf16 != 0, norm_mean, embed_std);
+    *out = new ug_llama::Model(cfg_of(c), custom_softmax != 0, *w, dev_of(d), *static_cast<OpsPtr*>(ops));
+  });
+}
 int ugh_llama_model_from_safetensors(void* d, void* ops, const ugh_llama_config* c, int custom_softmax, const char* const* paths, size_t n_paths, void** out) {
   return guard([&] {
     std::vector<std::string> ps(paths, paths + n_paths);
@@ -811,6 +818,12 @@ int ugh_llama_generate(void* m, const int32_t* prompt, size_t n_prompt, size_t n
     if (margins) std::memcpy(margins, st.top1_margin.data(), st.top1_margin.size() * sizeof(float));
   });
 }
+int ugh_llama_set_switch(const char* name, int on) {
+  return guard([&] {
+    if (!name || !ug_llama::set_switch(name, on != 0)) throw std::runtime_error(std::string("no llama switch named '") + (name ? name : "(null)") + "'");
+  });
+}
+static thread_local size_t g_last_decode_items = 0;
 int ugh_llama_generate_ex(void* m, const int32_t* prompt, size_t n_prompt, size_t n_steps, const int32_t* forced, int32_t* out_tokens, double* prefill_ms,
                           double* decode_ms, float* margins, float* top1_values) {
   return guard([&] {
@@ -823,8 +836,11 @@ int ugh_llama_generate_ex(void* m, const int32_t* prompt, size_t n_prompt, size_
     if (decode_ms) *decode_ms = st.decode_ms;
     if (margins) std::memcpy(margins, st.top1_margin.data(), st.top1_margin.size() * sizeof(float));
     if (top1_values) std::memcpy(top1_values, st.top1_value.data(), st.top1_value.size() * sizeof(float));
+    g_last_decode_items = st.decode_items;
   });
 }
+// Schedule items (device launches) of the last single-token step of this thread's last ugh_llama_generate_ex.
+size_t ugh_llama_last_decode_items() { return g_last_decode_items; }
 int ugh_synthetic_weights(uint64_t seed, float std, int round_bf16, const char* name, size_t n, float* out) {
   return guard([&] {
     auto w = ug_llama::synthetic_weights(seed, std, round_bf16 != 0);

@@ -2,6 +2,8 @@
 // a device sees (names, shapes, argument order) are those of the reference.
 #include "llama.h"
 
+#include <atomic>
+#include <mutex>
 #include <chrono>
 #include <cmath>
 #include <thread>
@@ -12,6 +14,32 @@
 #include "ug/safetensors.h"
 
 namespace ug_llama {
+
+namespace {
+const char* const kSwitchNames[SW_COUNT] = {"NO_FOLD_EPILOGUES", "NO_APPEND_PAIR", "VERBOSE", "NO_LAYER_STEPS", "HOST_ARGMAX", "NO_OVERLAP"};
+std::atomic<int> g_switch[SW_COUNT];
+std::once_flag g_switch_once;
+void switches_init() {
+  std::call_once(g_switch_once, [] {
+    for (int i = 0; i < SW_COUNT; ++i) g_switch[i].store(getenv((std::string("UG_LLAMA_") + kSwitchNames[i]).c_str()) != nullptr, std::memory_order_relaxed);
+  });
+}
+}  // namespace
+bool switch_on(Switch s) {
+  switches_init();
+  return g_switch[s].load(std::memory_order_relaxed) != 0;
+}
+bool set_switch(const std::string& name, bool on) {
+  switches_init();
+  const std::string n = name.rfind("UG_LLAMA_", 0) == 0 ? name.substr(9) : name;
+  for (int i = 0; i < SW_COUNT; ++i)
+    if (n == kSwitchNames[i]) {
+      g_switch[i].store(on, std::memory_order_relaxed);
+      return true;
+    }
+  return false;
+}
+
 
 using namespace ug;
 
@@ -341,7 +369,7 @@ struct HipOps : Ops {
   }
 
   LB gate_up_stacked(const LB& x, const LB& w) const override {
-    if (!many_f32_rows(x, w, 16) || getenv("UG_LLAMA_NO_FOLD_EPILOGUES")) return Ops::gate_up_stacked(x, w);
+    if (!many_f32_rows(x, w, 16) || switch_on(SW_NO_FOLD_EPILOGUES)) return Ops::gate_up_stacked(x, w);
     const size_t k = x.dims().back(), rows = x.elem_count() / k, n = w.dims()[0] / 2;
     ughip_device* dev = hip_dev(x);
     const int product = product_for(w, k, rows);
@@ -356,7 +384,7 @@ struct HipOps : Ops {
 
   LB linear_add(const LB& x, const LB& w, const LB& residual) const override {
     if (many_f32_rows(x, w, 8) && residual.dtype() == DType::F32 && residual.elem_count() == x.elem_count() / x.dims().back() * w.dims()[0] &&
-        !getenv("UG_LLAMA_NO_FOLD_EPILOGUES")) {
+        !switch_on(SW_NO_FOLD_EPILOGUES)) {
       const size_t k = x.dims().back(), rows = x.elem_count() / k, n = w.dims()[0];
       ughip_device* dev = hip_dev(x);
       const int product = product_for(w, k, rows);
@@ -411,7 +439,7 @@ struct HipOps : Ops {
       bail("attention_steps: mismatched shapes " + qkv.shape().str() + " " + kcache.shape().str());
     if (len + t > cap) bail("attention_steps: " + std::to_string(len + t) + " rows exceed the cache capacity " + std::to_string(cap));
     // one position has a launch of its own kind, and head sizes without a multi-query kernel take the composition
-    if (t < 2 || !(d == 32 || d == 64 || d == 128) || qkv.dtype() != DType::F32 || getenv("UG_LLAMA_NO_APPEND_PAIR"))
+    if (t < 2 || !(d == 32 || d == 64 || d == 128) || qkv.dtype() != DType::F32 || switch_on(SW_NO_APPEND_PAIR))
       return Ops::attention_steps(qkv, kcache, vcache, len, n_heads, scale, cos, sin, pos, interleaved);
     ughip_device* dev = hip_dev(qkv);
     const bool with_rope = cos != nullptr;
@@ -462,12 +490,16 @@ struct SyntheticWeights : WeightSource {
   uint64_t seed;
   float std;
   bool round_bf16;
-  SyntheticWeights(uint64_t s, float sd, bool r) : seed(s), std(sd), round_bf16(r) {}
+  float norm_mean, embed_std;  // norm vectors are norm_mean + N(0, std); the embedding table N(0, embed_std) when embed_std > 0
+  SyntheticWeights(uint64_t s, float sd, bool r, float nm = 0.f, float es = 0.f) : seed(s), std(sd), round_bf16(r), norm_mean(nm), embed_std(es) {}
   std::vector<float> get(const std::string& name, const std::vector<size_t>& shape) override {
     size_t n = 1;
     for (size_t d : shape) n *= d;
     std::vector<float> out(n);
     uint64_t ts = ugrng::tensor_seed(seed, name);
+    const bool is_norm = name.find("norm") != std::string::npos;
+    const float mean = is_norm ? norm_mean : 0.f;
+    const float std = (embed_std > 0.f && name == "model.embed_tokens.weight") ? embed_std : this->std;
     unsigned nt = std::max(1u, std::min(16u, std::thread::hardware_concurrency()));
     if (n < (1u << 16)) nt = 1;
     size_t pairs = (n + 1) / 2, per = (pairs + nt - 1) / nt;
@@ -479,7 +511,7 @@ struct SyntheticWeights : WeightSource {
         for (size_t p = p0; p < p1; ++p) {
           double z0, z1;
           ugrng::normal_pair(ts, p, &z0, &z1);
-          float a = (float)(z0 * std), b = (float)(z1 * std);
+          float a = mean + (float)(z0 * std), b = mean + (float)(z1 * std);
           if (round_bf16) {
             a = bf16_bits_to_f32(f32_to_bf16_bits(a));
             b = bf16_bits_to_f32(f32_to_bf16_bits(b));
@@ -598,8 +630,8 @@ LB Ops::gate_up_stacked(const LB& x, const LB& w_gate_up) const {
 // model.rs:366-372: a projection, then the residual.
 LB Ops::linear_add(const LB& x, const LB& w, const LB& residual) const { return linear(x, w).binary(BinaryOp::Add, residual); }
 
-std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16) {
-  return std::make_shared<SyntheticWeights>(seed, std, round_bf16);
+std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16, float norm_mean, float embed_std) {
+  return std::make_shared<SyntheticWeights>(seed, std, round_bf16, norm_mean, embed_std);
 }
 
 LB WeightSource::load(const std::string& name, const std::vector<size_t>& shape, const DevicePtr& dev) {
@@ -990,7 +1022,7 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
   const Ops& ops = model.ops();
   std::vector<Cache> cache = model.new_cache();
   CompilationCache ccache;
-  const bool verbose = getenv("UG_LLAMA_VERBOSE") != nullptr;
+  const bool verbose = switch_on(SW_VERBOSE);
   model.rope().cos.realize();
   model.rope().sin.realize();
 
@@ -1018,7 +1050,7 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
 
   // run_now: every item is launched as soon as it is compiled (the prompt's step: its first kernels execute while the
   // rest of its 300 items are still being looked up)
-  const bool by_layer = getenv("UG_LLAMA_NO_LAYER_STEPS") == nullptr;
+  const bool by_layer = !switch_on(SW_NO_LAYER_STEPS);
   auto build = [&](size_t i, PreparedStep& st, bool run_now) {
     auto t0 = clock::now();
     st.t = i == 0 ? prompt.size() : 1;
@@ -1093,6 +1125,7 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
     if (verbose)
       fprintf(stderr, "step %zu: own build %.2fms gen %.2fms comp %.2fms; launches %.2fms, next build %.2fms gen %.2fms comp %.2fms, both %.2fms, items %zu (queued, no read-back)\n", step,
               cur.build_ms, cur.gen_ms, cur.comp_ms, ms_between(t0, t1), next.build_ms, next.gen_ms, next.comp_ms, ms_between(t0, clock::now()), cur.n_items);
+    if (stats && step != 0) stats->decode_items = cur.n_items;
     if (step == 0) {
       dev->synchronize();  // separates the prompt's time from the decode steps'
       t_decode = clock::now();
@@ -1143,14 +1176,14 @@ std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32
   };
   check_ids(prompt, "prompt");
   if (forced) check_ids(*forced, "forced");
-  if (dev->runs_async() && model.ops().device_argmax() && getenv("UG_LLAMA_HOST_ARGMAX") == nullptr && getenv("UG_LLAMA_NO_OVERLAP") == nullptr)
+  if (dev->runs_async() && model.ops().device_argmax() && !switch_on(SW_HOST_ARGMAX) && !switch_on(SW_NO_OVERLAP))
     return generate_greedy_queued(model, prompt, n_steps, stats, forced);
   std::vector<Cache> cache = model.new_cache();
   CompilationCache ccache;
   std::vector<int32_t> out;
   std::vector<float> logits;
-  const bool verbose = getenv("UG_LLAMA_VERBOSE") != nullptr;
-  const bool overlap = dev->runs_async() && getenv("UG_LLAMA_NO_OVERLAP") == nullptr;
+  const bool verbose = switch_on(SW_VERBOSE);
+  const bool overlap = dev->runs_async() && !switch_on(SW_NO_OVERLAP);
   // The rotary tables are shared by every step: realise them once, before two steps can be in
   // preparation and in flight at the same time.
   model.rope().cos.realize();
@@ -1263,6 +1296,7 @@ std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32
       else {
         stats->decode_ms += ms;
         stats->step_ms.push_back(ms);
+        stats->decode_items = cur.n_items;
       }
       stats->top1_margin.push_back(last[best] - second);
       stats->top1_value.push_back(last[best]);

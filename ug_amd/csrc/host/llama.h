@@ -135,7 +135,9 @@ struct WeightSource {
 
 // Random-init weights: N(0, std) from a counter-based generator keyed by (seed, tensor name),
 // optionally rounded to bf16 (round-to-nearest-even) and widened back.
-std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16);
+// norm_mean: the norm vectors are norm_mean + N(0, std) (checkpoints hold values near 1; BASELINE's config says N(0, 0.02), i.e. 0);
+// embed_std > 0: the embedding table (and with it the tied head) is N(0, embed_std) instead of N(0, std).
+std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16, float norm_mean = 0.f, float embed_std = 0.f);
 
 // Weights from safetensors files, any stored dtype, delivered as f32 (model.rs:118,140,313:
 // `load_with_cast(name, DType::F32, device)`); conversion happens on the device when it can.
@@ -223,11 +225,19 @@ class Model {
 
 // The greedy-decode harness (the loop of ug-llama/src/main.rs:118-170): one prefill call over `prompt`, then `n_steps` greedy
 // (argmax) single-token steps with the KV cache.  Returns the generated ids; timings in ms.
+// Switches of the host-side loops and hooks (measurements, tests): read once per process from the environment
+// (UG_LLAMA_<NAME>) and changed afterwards only through set_switch, so that the hooks running on the preparing
+// thread never call getenv next to a caller that changes the environment.
+enum Switch { SW_NO_FOLD_EPILOGUES, SW_NO_APPEND_PAIR, SW_VERBOSE, SW_NO_LAYER_STEPS, SW_HOST_ARGMAX, SW_NO_OVERLAP, SW_COUNT };
+bool switch_on(Switch s);
+bool set_switch(const std::string& name, bool on);  // false: no switch of that name ("NO_OVERLAP", "UG_LLAMA_NO_OVERLAP")
+
 struct GenerateStats {
   double prefill_ms = 0, decode_ms = 0;
   std::vector<double> step_ms;
   std::vector<float> top1_margin;  // logit gap between the best and second-best token per step
   std::vector<float> top1_value;   // the best token's logit per step
+  size_t decode_items = 0;         // schedule items (device launches) of the last single-token step
 };
 // forced != nullptr (n_steps ids): decode step i is fed (*forced)[i - 1] instead of the id picked at step i - 1, so that two
 // devices can be compared position by position on identical inputs; the ids returned are still each step's argmax.

@@ -748,7 +748,7 @@ namespace {
 int decode_ranges(size_t s, size_t heads) {
   const size_t want = s >= 1280 ? 8 : s >= 800 ? 4 : 1;
   int n = (int)std::max<size_t>(1, std::min<size_t>(want, 256 / std::max<size_t>(heads, 1)));
-  if (const char* e = getenv("UGHIP_ATT_SPLIT")) n = atoi(e);
+  if (long long v; tune_get(TUNE_ATT_SPLIT, &v)) n = (int)v;
   return std::max(1, std::min(n, 64));
 }
 

@@ -404,7 +404,7 @@ void launch_bf16_rows_kt(hipStream_t st, const FusedArgs& a) {
   int r = 2;
   if (NM == 1 && KT >= 2) r = 4;
   if (a.n_cols >= 16384) r = NM == 1 && KT == 1 ? 8 : 4;
-  if (const char* e = getenv("UGHIP_GEMV_ROWS")) r = atoi(e);  // tuning aid: 1, 2, 4 or 8
+  if (long long v; tune_get(TUNE_GEMV_ROWS, &v)) r = (int)v;  // tuning aid: 1, 2, 4 or 8
   if (r >= 8) launch_bf16_rows_r<8, KT, MODE, RMS>(st, a);
   else if (r >= 4) launch_bf16_rows_r<4, KT, MODE, RMS>(st, a);
   else if (r >= 2) launch_bf16_rows_r<2, KT, MODE, RMS>(st, a);
@@ -421,14 +421,14 @@ void launch_bf16_rows(hipStream_t st, const FusedArgs& a) {
 }
 
 bool bf16_rows_fit(const FusedArgs& a) {
-  if (const char* e = getenv("UGHIP_GEMV_BF16_ROWS")) if (atoi(e) == 0) return false;  // tuning aid: the older kernels
+  if (long long v; tune_get(TUNE_GEMV_BF16_ROWS, &v) && v == 0) return false;  // tuning aid: the older kernels
   return a.k % 8 == 0 && a.k >= 512 && a.k <= 2048 * ROWS_KT_MAX;
 }
 
 int pick_ks(size_t cols, size_t k) {
   // enough waves to hide HBM latency: about 8192 over the chip
   int ks = cols <= 2048 ? 4 : cols <= 6144 ? 2 : 1;
-  if (const char* e = getenv("UGHIP_GEMV_KS")) ks = atoi(e);  // tuning aid: 1, 2 or 4
+  if (long long v; tune_get(TUNE_GEMV_KS, &v)) ks = (int)v;  // tuning aid: 1, 2 or 4
   if (ks != 1 && ks != 2 && ks != 4) ks = 1;
   while (ks > 1 && k < (size_t)64 * 4 * ks) ks >>= 1;
   return ks;
@@ -462,18 +462,22 @@ void launch_t(hipStream_t st, const FusedArgs& a) {
 }
 
 template <int MODE>
-void launch(hipStream_t st, const FusedArgs& a, int w_dtype) {
+hipError_t launch(hipStream_t st, const FusedArgs& a, int w_dtype) {
+  // a norm in front of the residual form: no entry point asks for it and no kernel is built for it -- an error, not a launch
+  // that silently does nothing
+  if (MODE == MODE_ADD && a.alpha) return hipErrorInvalidValue;
   if (w_dtype == UGHIP_BF16 && bf16_rows_fit(a)) {
     if (a.alpha) {
-      constexpr int M = MODE == MODE_ADD ? MODE_MULTI : MODE;  // no entry point asks for a norm in front of the residual form
-      if (MODE != MODE_ADD) launch_bf16_rows<M, true>(st, a);
+      constexpr int M = MODE == MODE_ADD ? MODE_MULTI : MODE;
+      launch_bf16_rows<M, true>(st, a);
     } else {
       launch_bf16_rows<MODE, false>(st, a);
     }
-    return;
+    return hipGetLastError();
   }
   if (w_dtype == UGHIP_BF16) launch_t<uint16_t, MODE>(st, a);
   else launch_t<float, MODE>(st, a);
+  return hipGetLastError();
 }
 
 int check(const ughip_device* dev, const ughip_slice* s, size_t need, const char* what) {
@@ -551,8 +555,7 @@ int ughip_rms_gemv_multi(ughip_device* dev, const ughip_slice* x, const ughip_sl
   a.n_cols = (int)total;
   if (total == 0) return UGHIP_OK;
   if (int rc = device_activate(dev)) return rc;
-  launch<MODE_MULTI>(dev->stream, a, wdt);
-  UGHIP_HIPCHK(hipGetLastError());
+  UGHIP_HIPCHK(launch<MODE_MULTI>(dev->stream, a, wdt));
   return UGHIP_OK;
 }
 
@@ -583,8 +586,7 @@ int ughip_rms_gemv_gate_up(ughip_device* dev, const ughip_slice* x, const ughip_
   a.col_end[0] = a.col_end[1] = a.col_end[2] = a.n_cols = (int)n;
   a.k = (int)k;
   if (int rc = device_activate(dev)) return rc;
-  launch<MODE_GATE_UP>(dev->stream, a, wdt);
-  UGHIP_HIPCHK(hipGetLastError());
+  UGHIP_HIPCHK(launch<MODE_GATE_UP>(dev->stream, a, wdt));
   return UGHIP_OK;
 }
 
@@ -607,8 +609,7 @@ int ughip_gemv_add(ughip_device* dev, const ughip_slice* x, const ughip_slice* w
   a.k = (int)k;
   a.residual = static_cast<const float*>(residual->ptr);
   if (int rc = device_activate(dev)) return rc;
-  launch<MODE_ADD>(dev->stream, a, wdt);
-  UGHIP_HIPCHK(hipGetLastError());
+  UGHIP_HIPCHK(launch<MODE_ADD>(dev->stream, a, wdt));
   return UGHIP_OK;
 }
 

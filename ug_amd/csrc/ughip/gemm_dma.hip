@@ -470,8 +470,7 @@ double gemm_dma_cost_us(const MMArgs& p, size_t batch, int tile) {
 }
 
 int gemm_dma_pick(int dtype, const MMArgs& p, size_t batch) {
-  if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
-    const int s = atoi(e);
+  if (long long s; tune_get(TUNE_GEMM_SHAPE, &s)) {
     const int forced = s == 3 ? 256 : s == 4 ? 128 : s == 5 ? 64 : 0;
     return forced && gemm_dma_supported(dtype, p, batch, forced) ? forced : 0;
   }

@@ -491,7 +491,7 @@ template <typename T, int B_NK, bool SPLIT>
 hipError_t launch_shape(hipStream_t stream, const MMArgs& p, size_t batch, int shape, int nsplit, float* ws, const GemmEpilogue* epi = nullptr) {
   switch (shape) {
     case 0:
-      return getenv("UGHIP_GEMM_4WAVES") ? launch<T, B_NK, 256, 128, 256, SPLIT>(stream, p, batch, nsplit, ws, epi)
+      return tune_on(TUNE_GEMM_4WAVES) ? launch<T, B_NK, 256, 128, 256, SPLIT>(stream, p, batch, nsplit, ws, epi)
                                          : launch<T, B_NK, 256, 128, 512, SPLIT>(stream, p, batch, nsplit, ws, epi);
     case 1:
       return p.M % 128 || p.N % 128 ? launch<T, B_NK, 128, 128, 256, SPLIT, true>(stream, p, batch, nsplit, ws, epi)
@@ -547,7 +547,7 @@ Split pick_split(int dtype, const MMArgs& p, size_t batch, int shape, bool alway
   const double tile_us = (dtype == UGHIP_F32 ? 1.03 * area : area <= 1.0 ? 0.4 : 0.325 * area) * (p.b_cs == 1 ? 1.35 : 1.0);
   const double slab_us = 2.0 * (double)batch * p.M * p.N * 4 / 5e6, fold_us = 5.0;
   Split best{1, (double)((tiles + 255) / 256) * kt * tile_us + (always_fold ? slab_us + fold_us : 0.0)};  // an epilogue folds even one slab
-  if (const char* e = getenv("UGHIP_GEMM_SPLIT")) return Split{std::max(1, atoi(e)), best.cost_us};  // tuning aid
+  if (long long v; tune_get(TUNE_GEMM_SPLIT, &v)) return Split{std::max(1, (int)v), best.cost_us};  // tuning aid
   // only when the tiles alone leave CUs idle and K is long enough that every slab still has a few tiles to pipeline; the
   // fold of the partial tiles works on groups of 4 elements
   if (tiles >= 256 || kt < 8 || (batch * (size_t)p.M * (size_t)p.N) % 4 != 0) return best;
@@ -568,8 +568,8 @@ Split pick_split(int dtype, const MMArgs& p, size_t batch, int shape, bool alway
 // a half: 1000 us) and 2304^3 away from 324 tiles of 128 x 128 (303 -> 255 us).  -1: no tile fits M x N.
 int pick_shape(const MMArgs& p, size_t batch, int dtype, bool always_fold = false) {
   // UGHIP_GEMM_SHAPE=0..2 forces a tile shape (tuning aid); ignored when it does not fit the problem.
-  if (const char* e = getenv("UGHIP_GEMM_SHAPE")) {
-    const int v = atoi(e), s = v == 6 ? 3 : v == 7 ? 4 : v;  // 3..5 name the other kernel's tiles: 6 and 7 are the 64- and 32-row tiles here
+  if (long long tv; tune_get(TUNE_GEMM_SHAPE, &tv)) {
+    const int v = (int)tv, s = v == 6 ? 3 : v == 7 ? 4 : v;  // 3..5 name the other kernel's tiles: 6 and 7 are the 64- and 32-row tiles here
     if (s >= 0 && s < kNumShapes && (s < 3 || v >= 6) && shape_fits(p, s)) return s;
   }
   int best = -1;
@@ -653,7 +653,7 @@ hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, siz
     if (nsplit > 1 || epi)
       snprintf(split, sizeof split, ",splitK=%d%s%s", nsplit, !epi ? "" : epi->kind == GemmEpilogue::ADD ? ",+residual" : epi->kind == GemmEpilogue::SWIGLU ? ",swiglu" : "",
                epi && epi->out_f32 ? ",f32 out" : "");
-    note_kernel("gemm_tiled<%s,%s,%dx%d,%dt%s%s>", tn, nt ? "NT" : "NN", kShapes[s][0], kShapes[s][1], s == 0 && !getenv("UGHIP_GEMM_4WAVES") ? 512 : 256,
+    note_kernel("gemm_tiled<%s,%s,%dx%d,%dt%s%s>", tn, nt ? "NT" : "NN", kShapes[s][0], kShapes[s][1], s == 0 && !tune_on(TUNE_GEMM_4WAVES) ? 512 : 256,
                   ragged ? ",ragged" : "", split);
   }
   if (nsplit > 1 || epi) {

@@ -56,6 +56,32 @@ int device_activate(ughip_device* d);
 int matmul_scratch_setup(ughip_device* dev);  // matmul.hip
 const char* dtype_name(int dt);
 
+// Tuning switches (tile / split / kernel-family overrides for measurements and tests).  The table is filled once per
+// process from the environment (UGHIP_<NAME>), the first time any switch is asked for, and changes afterwards only
+// through ughip_set_tuning: dispatch reads an atomic, never the environment, so a launch thread and a test that
+// flips a switch do not meet in getenv / setenv.
+enum TuneKey {
+  TUNE_GEMM_SHAPE,          // 0..2: a gemm_tiled tile (keeps gemm_dma4 out); 3 / 4 / 5: gemm_dma4 with 256x256 / 256x128 / 128x128
+  TUNE_GEMM_SPLIT,          // K split of gemm_tiled
+  TUNE_GEMM_4WAVES,         // (set at all) the 256-thread form of the 256x128 tile
+  TUNE_GEMV_KS,             // waves per output column of the GEMV family: 1, 2 or 4
+  TUNE_GEMV_ROWS,           // rows per workgroup of fused_gemv_bf16_rows: 1, 2, 4 or 8
+  TUNE_GEMV_BF16_ROWS,      // 0: bf16 matrices take the f32 kernels' lane layout
+  TUNE_X3_DMA,              // three-term bf16 products: 0 keeps gemm_tiled, 3 / 4 / 5 force a gemm_dma4 tile
+  TUNE_X3_SPLIT,            // K split of the three-term product on gemm_dma4
+  TUNE_ATT_SPLIT,           // key ranges per head of single-query attention
+  TUNE_NO_PARAMETRIC,       // (set at all) shapes stay literals in generated kernels
+  TUNE_NO_NT_LOADS,         // (set at all) the grid-wide reduction reads with ordinary loads
+  TUNE_GRID_REDUCE_BLOCKS,  // workgroups of the grid-wide reduction's first stage
+  TUNE_GRID_REDUCE_THREADS, // threads per workgroup there: 64, 128, 256, 512 or 1024
+  TUNE_COUNT
+};
+bool tune_get(TuneKey k, long long* value);  // false: the switch is not set
+inline bool tune_on(TuneKey k) {
+  long long v;
+  return tune_get(k, &v);
+}
+
 }  // namespace ughip
 
 #define UGHIP_HIPCHK(expr)                                                                                 \

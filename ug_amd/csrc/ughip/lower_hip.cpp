@@ -21,6 +21,8 @@
 //    with the exact serial semantics of the CPU backend (cpu_code_gen.rs:68-186).
 #include "lower_hip.h"
 
+#include "internal.h"
+
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
@@ -1212,7 +1214,7 @@ class Lowering {
     // Small kernels (the per-token elementwise work of a decode step, whose shapes follow the KV
     // length) are emitted parametric so that a new shape does not mean a new hiprtc compile; large
     // ones keep their constants, which lets the compiler strength-reduce the index arithmetic.
-    parametric_ = total <= (1 << 20) && !getenv("UGHIP_NO_PARAMETRIC");
+    parametric_ = total <= (1 << 20) && !ughip::tune_on(ughip::TUNE_NO_PARAMETRIC);
     kparams_.clear();
     std::ostringstream b;
     b << "  const int ug_g = (int)blockIdx.x * " << block << " + (int)threadIdx.x;\n";
@@ -1262,11 +1264,9 @@ class Lowering {
     out_.grid = (unsigned)((nr + block - 1) / block);
   }
 
-  static unsigned env_u(const char* name, unsigned dflt) {
-    const char* e = getenv(name);
-    if (!e || !*e) return dflt;
-    long v = strtol(e, nullptr, 10);
-    return v > 0 ? (unsigned)v : dflt;
+  static unsigned tune_u(ughip::TuneKey k, unsigned dflt) {
+    long long v;
+    return ughip::tune_get(k, &v) && v > 0 ? (unsigned)v : dflt;
   }
 
   void emit_row_block(const std::vector<int>& rows, const std::vector<int>& cols, i64 nr, i64 nc, bool grid_reduce) {
@@ -1276,7 +1276,7 @@ class Lowering {
     for (const Region& r : regions_) width = std::max(width, r.trip);
     int tpr;  // threads that share a row
     if (grid_reduce) {
-      tpr = 256;
+      tpr = (int)tune_u(ughip::TUNE_GRID_REDUCE_THREADS, 256);
     } else if (width <= 256) {
       tpr = 64;
     } else {
@@ -1295,13 +1295,14 @@ class Lowering {
       const Region& r = regions_[0];
       int vec = pick_vec(r.trip, tpr);
       i64 per_block_iter = (i64)tpr * vec;
-      // Measured on MI355X (2 x 64 MiB streamed): 256-512 workgroups of 256 threads, each thread
-      // walking >= 4 slabs with four 128-bit loads in flight, is where the curve is flat (~6.2 TB/s);
-      // more workgroups only add scheduling cost.
+      // Measured on MI355X: one workgroup of 256 threads per CU (256 of them), each thread walking >= 4 slabs with
+      // four 128-bit loads per operand in flight.  Two per CU (512) is as fast on some boxes and 6-9 % slower on
+      // others, in bursts and behind seconds of the same launches alike (2 x 64 MiB: 21.4 against 23.4 us per step
+      // sustained; 2 x 512 MiB: 152 against 162 us); 128 or 384 leave CUs idle for half a round.
       i64 want = (r.trip + per_block_iter * 4 - 1) / (per_block_iter * 4);
-      unsigned cap = std::max<i64>(1, 512 / nr);
+      unsigned cap = std::max<i64>(1, 256 / nr);
       nb = (unsigned)std::max<i64>(1, std::min<i64>(want, cap));
-      nb = env_u("UGHIP_GRID_REDUCE_BLOCKS", nb);
+      nb = tune_u(ughip::TUNE_GRID_REDUCE_BLOCKS, nb);
       o << "  const int ug_row = (int)blockIdx.x / " << nb << ";\n";
       o << "  const int ug_blk = (int)blockIdx.x % " << nb << ";\n";
     } else {
@@ -1338,7 +1339,7 @@ class Lowering {
       // The first stage streams its operands once: loads that do not claim cache lines (measured on
       // 2 x 64 MiB: 22.0 -> 20.6 us).  Kernels that come back to a row (softmax, norms) and plain
       // copies lose with them (6.8 -> 5.9 TB/s for a 64 MiB copy), so nothing else uses them.
-      nt_loads_ = getenv("UGHIP_NO_NT_LOADS") == nullptr;
+      nt_loads_ = !ughip::tune_on(ughip::TUNE_NO_NT_LOADS);
       emit_region_partial(o, r, 2, tpr, nb);
       nt_loads_ = false;
       o << "    if (ug_t == 0) ug_part[ug_row * " << nb << " + ug_blk] = " << part << ";\n";

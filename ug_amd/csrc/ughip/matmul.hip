@@ -353,7 +353,7 @@ void launch_gemv_nt_any(hipStream_t st, const MMArgs& p, size_t b) {
   // enough waves to hide HBM latency: about 8192 over the chip
   const size_t cols = (size_t)p.N * b;
   int ks = cols <= 2048 ? 4 : cols <= 6144 ? 2 : 1;
-  if (const char* e = getenv("UGHIP_GEMV_KS")) ks = atoi(e);  // tuning aid: 1, 2 or 4
+  if (long long v; tune_get(TUNE_GEMV_KS, &v)) ks = (int)v;  // tuning aid: 1, 2 or 4
   if (ks != 1 && ks != 2 && ks != 4) ks = 1;
   while (ks > 1 && p.K < 64 * VE * ks) ks >>= 1;
   if (ks == 4) launch_gemv_nt<T, 4>(st, p, b);
@@ -551,7 +551,11 @@ __global__ void __launch_bounds__(256) split3_bf16_kernel(const float* __restric
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     hi[i] = bf16_rne(in[i]);
-    const float r1 = in[i] - __uint_as_float((uint32_t)hi[i] << 16);  // exact: hi shares the leading bits of x
+    const float h = __uint_as_float((uint32_t)hi[i] << 16);
+    // an infinity (given, or reached when |x| rounds up past the largest bf16) or a NaN is all in the first term: the
+    // remainders would be inf - inf, and the product has to give what the f32 pipe gives for such an x
+    const bool fin = (hi[i] & 0x7f80) != 0x7f80;
+    const float r1 = fin ? in[i] - h : 0.f;  // exact: hi shares the leading bits of x
     mid[i] = bf16_rne(r1);
     const float r2 = r1 - __uint_as_float((uint32_t)mid[i] << 16);
     lo[i] = bf16_rne(r2);
@@ -603,12 +607,15 @@ static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x
   int dma_tile = 0, dma_split = 1;
   // (from 384 rows: at 128 and 256 rows the register-staged kernel is as fast or faster for four of the five products of a
   // llama step -- q|k|v 25.2 us against 28.6 at 256 rows -- and the model below does not see that; at 512 rows this kernel is)
-  if (x3 && m >= 384 && !(getenv("UGHIP_X3_DMA") && atoi(getenv("UGHIP_X3_DMA")) == 0)) {
+  long long x3_dma = -1, x3_split = 0;  // tuning aids: X3_DMA 0 keeps the register-staged kernel, 3 / 4 / 5 force a tile; X3_SPLIT n a K split
+  tune_get(TUNE_X3_DMA, &x3_dma);
+  tune_get(TUNE_X3_SPLIT, &x3_split);
+  if (x3 && m >= 384 && x3_dma != 0) {
     MMArgs q = p;
     q.c = dst->ptr;  // alignment of the result as f32
     double best = 0;
-    const int forced_tile = getenv("UGHIP_X3_DMA") ? (atoi(getenv("UGHIP_X3_DMA")) == 3 ? 256 : atoi(getenv("UGHIP_X3_DMA")) == 4 ? 128 : atoi(getenv("UGHIP_X3_DMA")) == 5 ? 64 : 0) : 0;
-    const int forced_split = getenv("UGHIP_X3_SPLIT") ? atoi(getenv("UGHIP_X3_SPLIT")) : 0;  // tuning aids: 3 / 4 / 5 force a tile, n a K split
+    const int forced_tile = x3_dma == 3 ? 256 : x3_dma == 4 ? 128 : x3_dma == 5 ? 64 : 0;
+    const int forced_split = (int)x3_split;
     for (int tile : {256, 128, 64}) {
       if (forced_tile && tile != forced_tile) continue;
       for (int split : {1, 2, 4, 8}) {

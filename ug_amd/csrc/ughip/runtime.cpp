@@ -4,7 +4,9 @@
 
 #include <atomic>
 #include <cstdarg>
+#include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -88,6 +90,32 @@ static size_t size_class(size_t bytes) {
   return p * 2;
 }
 
+namespace ughip {
+namespace {
+const char* const kTuneNames[TUNE_COUNT] = {"GEMM_SHAPE", "GEMM_SPLIT", "GEMM_4WAVES", "GEMV_KS",        "GEMV_ROWS",   "GEMV_BF16_ROWS",
+                                            "X3_DMA",     "X3_SPLIT",   "ATT_SPLIT",   "NO_PARAMETRIC",  "NO_NT_LOADS", "GRID_REDUCE_BLOCKS", "GRID_REDUCE_THREADS"};
+constexpr long long kTuneUnset = INT64_MIN;
+std::atomic<long long> g_tune[TUNE_COUNT];
+std::once_flag g_tune_once;
+void tune_init() {
+  std::call_once(g_tune_once, [] {
+    for (int k = 0; k < TUNE_COUNT; ++k) {
+      const std::string name = std::string("UGHIP_") + kTuneNames[k];
+      const char* e = getenv(name.c_str());
+      g_tune[k].store(e ? strtoll(e, nullptr, 10) : kTuneUnset, std::memory_order_relaxed);
+    }
+  });
+}
+}  // namespace
+bool tune_get(TuneKey k, long long* value) {
+  tune_init();
+  const long long v = g_tune[k].load(std::memory_order_relaxed);
+  if (v == kTuneUnset) return false;
+  *value = v;
+  return true;
+}
+}  // namespace ughip
+
 extern "C" {
 
 const char* ughip_last_error(void) { return g_last_error.c_str(); }
@@ -95,7 +123,21 @@ const char* ughip_last_kernel(void) { return g_last_kernel.c_str(); }
 
 int ughip_use_grid(void) { return 0; }
 
+int ughip_set_tuning(const char* name, int set, int64_t value) {
+  if (!name) return ughip::set_error(UGHIP_ERR_INVALID, "set_tuning: null name");
+  ughip::tune_init();
+  if (!strncmp(name, "UGHIP_", 6)) name += 6;
+  for (int k = 0; k < ughip::TUNE_COUNT; ++k)
+    if (!strcmp(name, ughip::kTuneNames[k])) {
+      if (set && value == ughip::kTuneUnset) return ughip::set_error(UGHIP_ERR_INVALID, "set_tuning: value out of range");
+      ughip::g_tune[k].store(set ? value : ughip::kTuneUnset, std::memory_order_relaxed);
+      return UGHIP_OK;
+    }
+  return ughip::set_error(UGHIP_ERR_INVALID, "set_tuning: no switch named '%s'", name);
+}
+
 int ughip_device_create(int ordinal, ughip_device** out) {
+  ughip::tune_init();
   if (!out) return set_error(UGHIP_ERR_INVALID, "null out pointer");
   int count = 0;
   hipError_t e = hipGetDeviceCount(&count);
