@@ -684,6 +684,11 @@ def llama_pieces(dev, steps, warmup):
         _, ms = timed(dev, cs.run, steps, warmup)
         gbs = nbytes * steps / (ms * 1e-3) / 1e9
         out[name] = {"GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "us": round(ms * 1e3 / steps, 2), "algorithmic_bytes": nbytes, "verified": ok}
+        if gbs > HBM_PEAK_GBS:
+            # a working set of a few tens of MB lives in the caches (32 MB of L2, 256 MB memory-side): the rate is theirs, and a
+            # fraction of the HBM peak says nothing; the same kernel on a 1 GiB working set is under `hbm_large`
+            out[name]["frac_hbm"] = None
+            out[name]["note"] = "cache-resident working set: faster than HBM's peak, no HBM fraction quoted"
 
     xh, ah = rng.normal(6, t * hidden).reshape(1, t, hidden), rng.normal(6 + 100, hidden, 0.02)
     x = LB.copy(xh, (1, t, hidden), dev)

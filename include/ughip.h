@@ -165,7 +165,7 @@ int ughip_d2h(const ughip_slice* src, void* dst, int dtype, size_t len);
 
 /* Tuning switches, with no counterpart in the reference: tile, split and kernel-family overrides used by the
  * tests and for measurements (GEMM_SHAPE, GEMM_SPLIT, GEMM_4WAVES, GEMV_KS, GEMV_ROWS, GEMV_BF16_ROWS, X3_DMA,
- * X3_SPLIT, ATT_SPLIT, NO_PARAMETRIC, NO_NT_LOADS, GRID_REDUCE_BLOCKS, GRID_REDUCE_THREADS; a leading "UGHIP_" is accepted).  The
+ * X3_SPLIT, ATT_SPLIT, NO_PARAMETRIC, NO_NT_LOADS, GRID_REDUCE_BLOCKS, GRID_REDUCE_THREADS, NO_NT_STORES, SOFTMAX_STREAM; a leading "UGHIP_" is accepted).  The
  * table is read once per process from the environment (UGHIP_<NAME>) and changes afterwards only through this
  * call: set != 0 stores `value`, set == 0 clears the switch.  Dispatch reads the table, never the environment,
  * so the call is safe next to a thread that is launching. */

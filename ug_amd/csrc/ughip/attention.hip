@@ -69,7 +69,10 @@ __global__ void __launch_bounds__(256) causal_softmax_wave_v4(const float* __res
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     const int c = lane + i * 64;
-    if (c < n4) d4[c] = make_float4(x[i].x / sum, x[i].y / sum, x[i].z / sum, x[i].w / sum);
+    if (c < n4) {
+      typedef float f32x4 __attribute__((ext_vector_type(4)));
+      __builtin_nontemporal_store(f32x4{x[i].x / sum, x[i].y / sum, x[i].z / sum, x[i].w / sum}, reinterpret_cast<f32x4*>(d4 + c));  // past the cache
+    }
   }
 }
 

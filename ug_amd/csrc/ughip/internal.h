@@ -74,6 +74,8 @@ enum TuneKey {
   TUNE_NO_NT_LOADS,         // (set at all) the grid-wide reduction reads with ordinary loads
   TUNE_GRID_REDUCE_BLOCKS,  // workgroups of the grid-wide reduction's first stage
   TUNE_GRID_REDUCE_THREADS, // threads per workgroup there: 64, 128, 256, 512 or 1024
+  TUNE_NO_NT_STORES,        // (set at all) generated elementwise kernels store through the cache
+  TUNE_SOFTMAX_STREAM,      // ughip_softmax_rows: 0 never takes the resident wave-per-row kernel, n > 0 forces it onto n workgroups
   TUNE_COUNT
 };
 bool tune_get(TuneKey k, long long* value);  // false: the switch is not set

@@ -2,6 +2,8 @@
 // Semantics follow the CPU implementations in ug-llama/src/cpu_ops.rs:6-167; all f32.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include <cstdint>
 
 #include "internal.h"
@@ -26,6 +28,8 @@ __device__ __forceinline__ float block_reduce(float v, float* lds) {
   for (int i = 1; i < NW; ++i) r = IS_MAX ? fmaxf(r, lds[i]) : r + lds[i];
   return r;
 }
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // ---- custom_softmax (cpu_ops.rs:6-31) --------------------------------------------------------
 // One workgroup of NW waves per row; the row lives in registers (V float4 per thread), so HBM
@@ -70,7 +74,7 @@ __global__ void __launch_bounds__(NW * 64) softmax_rows_reg(const float* __restr
       x[i].y /= s;
       x[i].z /= s;
       x[i].w /= s;
-      d4[c] = x[i];
+      __builtin_nontemporal_store(f32x4{x[i].x, x[i].y, x[i].z, x[i].w}, reinterpret_cast<f32x4*>(d4 + c));  // nobody in this launch reads it
     }
   }
 }
@@ -143,6 +147,64 @@ __global__ void __launch_bounds__(256) softmax_rows_wave_v4(const float* __restr
   }
 }
 
+// Wave per row, resident: `gridDim.x` workgroups of four waves stay on the chip and every wave walks rows wave, wave +
+// n_waves, ...  The row lives in registers (V float4 per lane, n_cols % 4 == 0, n_cols <= 256 * V), both reductions stay
+// inside the wave (no LDS, no barrier), and the loads of the wave's next row are issued before the arithmetic of the
+// current one, so every lane keeps V 128-bit loads in flight through the reductions, the exponentials and the stores.
+// Loads are ordinary, stores go past the cache (nontemporal loads cost 10-20 % here: 4096 x 1024 6.6 against 5.5 us).
+template <int V>
+__global__ void __launch_bounds__(256) softmax_rows_wave_stream(const float* __restrict__ src, float* __restrict__ dst, int n_rows, int n_cols) {
+  const int n_waves = gridDim.x * 4, lane = threadIdx.x & 63, n4 = n_cols >> 2;
+  int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= n_rows) return;
+  auto load = [&](f32x4(&x)[V], int r) {
+    const f32x4* s4 = reinterpret_cast<const f32x4*>(src + (size_t)r * n_cols);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const int c = lane + i * 64;
+      x[i] = c < n4 ? s4[c] : f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    }
+  };
+  auto finish = [&](f32x4(&x)[V], int r) {
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < V; ++i) m = fmaxf(fmaxf(m, fmaxf(x[i].x, x[i].y)), fmaxf(x[i].z, x[i].w));
+    m = wave_max(m);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      // columns past the row end hold -inf and contribute exp(-inf) = 0
+      x[i].x = expf(x[i].x - m);
+      x[i].y = expf(x[i].y - m);
+      x[i].z = expf(x[i].z - m);
+      x[i].w = expf(x[i].w - m);
+      sum += (x[i].x + x[i].y) + (x[i].z + x[i].w);
+    }
+    sum = wave_sum(sum);
+    f32x4* d4 = reinterpret_cast<f32x4*>(dst + (size_t)r * n_cols);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const int c = lane + i * 64;
+      const f32x4 y{x[i].x / sum, x[i].y / sum, x[i].z / sum, x[i].w / sum};
+      if (c < n4) __builtin_nontemporal_store(y, d4 + c);
+    }
+  };
+  f32x4 a[V], b[V];
+  load(a, row);
+  while (true) {
+    int next = row + n_waves;
+    if (next < n_rows) load(b, next);
+    finish(a, row);
+    if (next >= n_rows) break;
+    row = next;
+    next = row + n_waves;
+    if (next < n_rows) load(a, next);
+    finish(b, row);
+    if (next >= n_rows) break;
+    row = next;
+  }
+}
+
 // Any row length: three passes over the row (the re-reads hit L2 for rows of this size).
 __global__ void __launch_bounds__(1024) softmax_rows_generic(const float* __restrict__ src, float* __restrict__ dst, int n_cols) {
   __shared__ float lds[16];
@@ -179,7 +241,7 @@ __global__ void __launch_bounds__(256) causal_mask_v4(const float* __restrict__ 
     if (i2 + 2 > i1) v.z = -INFINITY;
     if (i2 + 3 > i1) v.w = -INFINITY;
   }
-  reinterpret_cast<float4*>(dst)[g] = v;
+  __builtin_nontemporal_store(f32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<f32x4*>(dst) + g);  // past the cache: nobody in this launch reads it
 }
 
 __global__ void __launch_bounds__(256) causal_mask_scalar(const float* __restrict__ src, float* __restrict__ dst, size_t n, int s1, int s2) {
@@ -379,7 +441,26 @@ int ughip_softmax_rows(ughip_device* dev, const ughip_slice* src, ughip_slice* d
   float* d = static_cast<float*>(dst->ptr);
   hipStream_t st = dev->stream;
   const int nc = (int)n_cols, nr = (int)n_rows;
-  if (n_cols % 4 == 0 && n_cols <= 256) {
+  // Rows of up to 2048 columns, at least 2048 of them and up to ~100 MB of traffic: one wave per row on at most 2048
+  // workgroups (every wave slot of the chip), the loads of a wave's next row issued before the arithmetic of the current one.
+  // Measured against the kernels below, us: 4096 x 512 3.97 / 4.47, x 768 5.04 / 6.25, x 1024 5.55 / 7.15, x 1536 7.5 / 7.98,
+  // x 2048 9.0 / 10.6; 16384 x 512 9.6 / 11.3.  Larger problems walk too many rows per wave for that to win (16384 x 2048:
+  // 42.1 against 38.4; 131072 x 1024: 191 against 179) and keep a fresh workgroup per row (or four rows).  Every kernel stores
+  // past the cache: nobody in the launch reads the result (block per row, 2048 x 2048: 7.2 -> 5.4 us; 32768 x 4096: 178 -> 173).
+  // SOFTMAX_STREAM (tuning aid): 0 never takes the resident kernel, n > 0 forces it onto n workgroups where it applies.
+  long long stream = -1;
+  tune_get(TUNE_SOFTMAX_STREAM, &stream);
+  const bool stream_fits = n_cols % 4 == 0 && n_cols <= 8192;
+  const bool stream_pays = n_cols % 4 == 0 && n_cols > 256 && n_cols <= 2048 && n_rows >= 2048 && n_rows * n_cols <= (3u << 22);
+  if (stream_fits && (stream > 0 || (stream < 0 && stream_pays))) {
+    const unsigned g = (unsigned)std::min<size_t>(stream > 0 ? (size_t)stream : 2048, blocks_for(n_rows, 4));
+    if (n_cols <= 256) softmax_rows_wave_stream<1><<<g, 256, 0, st>>>(s, d, nr, nc);
+    else if (n_cols <= 512) softmax_rows_wave_stream<2><<<g, 256, 0, st>>>(s, d, nr, nc);
+    else if (n_cols <= 1024) softmax_rows_wave_stream<4><<<g, 256, 0, st>>>(s, d, nr, nc);
+    else if (n_cols <= 2048) softmax_rows_wave_stream<8><<<g, 256, 0, st>>>(s, d, nr, nc);
+    else if (n_cols <= 4096) softmax_rows_wave_stream<16><<<g, 256, 0, st>>>(s, d, nr, nc);
+    else softmax_rows_wave_stream<32><<<g, 256, 0, st>>>(s, d, nr, nc);
+  } else if (n_cols % 4 == 0 && n_cols <= 256) {
     softmax_rows_wave_v4<1><<<blocks_for(n_rows, 4), 256, 0, st>>>(s, d, nr, nc);
   } else if (n_cols % 4 == 0 && n_cols <= 512) {
     softmax_rows_wave_v4<2><<<blocks_for(n_rows, 4), 256, 0, st>>>(s, d, nr, nc);
