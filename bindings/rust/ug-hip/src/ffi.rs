@@ -133,6 +133,17 @@ extern "C" {
         out_len: *mut usize,
         info: *mut UghipFuncInfo,
     ) -> c_int;
+    pub fn ughip_matmul_plan(
+        dtype: c_int,
+        rhs_dtype: c_int,
+        b: usize,
+        m: usize,
+        n: usize,
+        k: usize,
+        rhs_nk: c_int,
+        buf: *mut c_char,
+        buf_len: usize,
+    ) -> c_int;
     pub fn ughip_set_tuning(name: *const c_char, set: c_int, value: i64) -> c_int;
     pub fn ughip_codegen_min_len(ssa: *const UghipSsa, min_len: *mut i64, n_args: usize) -> c_int;
     pub fn ughip_codegen_as_written(

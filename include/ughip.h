@@ -248,6 +248,12 @@ int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs,
                  const ughip_slice* rhs, size_t b, size_t m, size_t n, size_t k, size_t rank,
                  const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset,
                  const size_t* rhs_dims, const size_t* rhs_strides, size_t rhs_offset);
+/* No counterpart in the reference, no device needed: the kernel ughip_matmul would launch for contiguous operands of
+ * these shapes (rhs_nk != 0: the rhs stored [n, k]), by the name ughip_last_kernel() reports after the launch -- tile,
+ * K split and all.  The choice follows from shapes and from the library's cost models; tests pin it for the shapes
+ * that matter, so that a change of a model constant shows as a changed plan. */
+int ughip_matmul_plan(int dtype, int rhs_dtype, size_t b, size_t m, size_t n, size_t k, int rhs_nk, char* buf,
+                      size_t buf_len);
 
 /* ughip_matmul for callers that cannot allocate (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and

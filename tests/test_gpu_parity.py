@@ -461,6 +461,24 @@ def test_matmul_16bit_kernel_choice(hip, bmnk, want):
     assert np.all(np.abs(got[:, rows] - exact) <= bound * 1.001 + 1e-7)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype_name,bmnk,rhs_nk", [("f32", (2, 256, 128, 192), False), ("bf16", (8, 1024, 1024, 1024), False), ("bf16", (1, 2304, 2304, 2304), True),
+                                                    ("f32", (32, 512, 64, 512), False), ("f32", (1, 1, 2048, 2048), True), ("f32", (1, 100, 100, 100), False)])
+def test_plan_names_what_is_launched(hip, dtype_name, bmnk, rhs_nk):
+    """ughip_matmul_plan (no device) and the launch agree on the kernel, tile and split."""
+    import ctypes as C
+    b, m, n, k = bmnk
+    dt = F32 if dtype_name == "f32" else ug_amd.BF16
+    rnd = (lambda v: v) if dtype_name == "f32" else rng.bf16_round
+    a = rnd(rng.uniform_pm1(41, b * m * k)).reshape(b, m, k)
+    w = rnd(rng.uniform_pm1(42, b * k * n)).reshape(b, k, n)
+    _raw_matmul(hip, dt, a, w, rhs_nk)
+    buf = C.create_string_buffer(200)
+    lib = ug_amd.ughip_lib()
+    assert lib.ughip_matmul_plan(int(dt), int(dt), C.c_size_t(b), C.c_size_t(m), C.c_size_t(n), C.c_size_t(k), int(rhs_nk), buf, C.c_size_t(200)) == 0
+    assert buf.value.decode() == ug_amd.last_kernel()
+
+
 def test_matmul_16bit_one_wave_per_simd_forced_and_limits(hip, tune):
     """UGHIP_GEMM_SHAPE=3 / 4 / 5 force the kernel's three tiles onto a small problem (bit for bit the register-staged
     kernel's result); shapes it cannot take (K below 4 tiles, a column count that is not a multiple of 8) fall through to

@@ -259,3 +259,53 @@ def test_a_guard_that_says_nothing_about_the_offset_leaves_the_full_requirement(
     I32_ = int(ug_amd.I32)
     prog[5] = Instr(6, I32_, 1, 0, 0, A(1, I32_, 0, 0, 50, 0.0, 0), A(0, I32_, 0, 1, 0, 0.0, 0))   # 5 = 50 - ti
     assert SsaKernel.from_instrs(prog, grid=2, block=64).min_lens() == [114]
+
+
+def _plan(dtype, rhs_dtype, b, m, n, k, rhs_nk):
+    lib = ug_amd.ughip_lib()
+    buf = C.create_string_buffer(200)
+    rc = lib.ughip_matmul_plan(int(dtype), int(rhs_dtype), C.c_size_t(b), C.c_size_t(m), C.c_size_t(n), C.c_size_t(k), int(rhs_nk), buf, C.c_size_t(200))
+    if rc:
+        raise ug_amd.UgError(lib.ughip_last_error().decode())
+    return buf.value.decode()
+
+
+def test_kernel_choice_for_the_baseline_shapes_is_pinned():
+    """Which kernel, tile and K split a product gets follows from shapes and from cost models whose constants were fitted to
+    measurements (gemm_dma_cost_us, gemm_tiled's pick_shape / pick_split).  The plans for BASELINE's products are written
+    down here, so that a changed constant shows as a changed plan in a test that needs no GPU (the GPU suite then checks that
+    ughip_matmul launches what the plan names: test_plan_names_what_is_launched)."""
+    F, B = ug_amd.F32, ug_amd.BF16
+    want = {
+        # config 3: 8 x 1024^3, both rhs layouts
+        (F, F, 8, 1024, 1024, 1024, 0): "gemm_tiled<f32,NN,256x128,512t>",
+        (F, F, 8, 1024, 1024, 1024, 1): "gemm_tiled<f32,NT,256x128,512t>",
+        (B, B, 8, 1024, 1024, 1024, 0): "gemm_dma4<bf16,NN,256x128,256t>",
+        (B, B, 8, 1024, 1024, 1024, 1): "gemm_dma4<bf16,NT,256x128,256t>",
+        # the large products the bench line carries
+        (B, B, 1, 4096, 4096, 4096, 1): "gemm_dma4<bf16,NT,256x256,256t>",
+        (B, B, 1, 4096, 4096, 4096, 0): "gemm_dma4<bf16,NN,256x256,256t>",
+        (B, B, 1, 8192, 8192, 8192, 1): "gemm_dma4<bf16,NT,256x256,256t>",
+        (B, B, 1, 3000, 4096, 4096, 1): "gemm_dma4<bf16,NT,256x256,256t>",
+        # config 4: q k^T and att v at T = 512
+        (F, F, 32, 512, 512, 64, 1): "gemm_tiled<f32,NT,256x128,512t>",
+        (F, F, 32, 512, 64, 512, 0): "gemm_tiled<f32,NN,128x64,256t,splitK=2>",
+        # config 5: decode projections (one row), single-query attention output, a 128-token prompt against bf16 matrices
+        (F, F, 1, 1, 2048, 2048, 1): "gemv_nt<f32>",
+        (F, F, 1, 1, 32000, 2048, 1): "gemv_nt<f32>",
+        (F, F, 32, 1, 64, 1900, 0): "gemv_nn<f32>",
+        (F, B, 1, 128, 2560, 2048, 1): "gemm_tiled<f32xbf16,NT,128x64,256t,splitK=6>",
+        (F, B, 1, 128, 2048, 5632, 1): "gemm_tiled<f32xbf16,NT,128x64,256t,splitK=8>",
+        (F, B, 1, 128, 32000, 2048, 1): "gemm_tiled<f32xbf16,NT,128x128,256t>",
+        # mid-size 16-bit products where the two kernels are close
+        (B, B, 1, 2048, 2048, 2048, 1): "gemm_tiled<bf16,NT,128x128,256t>",
+        (B, B, 1, 2304, 2304, 2304, 1): "gemm_dma4<bf16,NT,128x128,256t>",
+        (B, B, 1, 3072, 4096, 4096, 1): "gemm_dma4<bf16,NT,256x256,256t>",
+        (F, F, 1, 100, 100, 100, 0): "gemm_any<f32>",
+    }
+    got = {key: _plan(*key) for key in want}
+    assert got == want
+    with pytest.raises(ug_amd.UgError, match=r"\[n, k\]-major"):
+        _plan(F, B, 1, 128, 2560, 2048, 0)
+    with pytest.raises(ug_amd.UgError):
+        _plan(ug_amd.I32, ug_amd.I32, 1, 8, 8, 8, 0)

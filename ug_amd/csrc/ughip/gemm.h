@@ -60,5 +60,9 @@ bool gemm_dma_planes3_split_ok(const MMArgs& p, int nsplit);
 // (c[m, n / 2] = silu(sum[:, :n / 2]) * sum[:, n / 2:]); n % 8 == 0.
 hipError_t gemm_fold_f32(hipStream_t stream, const float* slabs, float* c, size_t m, size_t n, int nsplit, GemmEpilogue::Kind kind, const float* residual);
 double gemm_dma_cost_us(const MMArgs& p, size_t batch, int tile);
+// The names ughip_last_kernel() reports for the two kernels' launches (tile, split and neighbour folded in): the launches use them, and so
+// does ughip_matmul_plan, which answers without launching.
+void gemm_dma_name(int dtype, const MMArgs& p, int tile, char* out, size_t out_len);
+void gemm_tiled_name(int dtype, const MMArgs& p, size_t batch, bool rhs_bf16, const GemmEpilogue* epi, char* out, size_t out_len);
 
 }  // namespace ughip

@@ -488,13 +488,23 @@ int gemm_dma_pick(int dtype, const MMArgs& p, size_t batch) {
   return other < 0 || best_us < other * (best == 64 ? 0.95 : 1.0) ? best : 0;
 }
 
+void gemm_dma_name(int dtype, const MMArgs& p, int tile, char* out, size_t out_len) {
+  int bm = 0, bn = 0;
+  tile_dims(tile, &bm, &bn);
+  const bool nn = p.b_cs == 1 && p.b_rs != 1;
+  snprintf(out, out_len, "gemm_dma4<%s,%s,%dx%d,256t>", dtype == UGHIP_F16 ? "f16" : "bf16", nn ? "NN" : "NT", bm, bn);
+}
+
 hipError_t gemm_dma_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, int tile) {
   if (!gemm_dma_supported(dtype, p, batch, tile)) return hipErrorInvalidValue;
   int bm = 0, bn = 0;
   tile_dims(tile, &bm, &bn);
   const bool nn = p.b_cs == 1 && p.b_rs != 1;
-  const char* tn = dtype == UGHIP_F16 ? "f16" : "bf16";
-  note_kernel("gemm_dma4<%s,%s,%dx%d,256t>", tn, nn ? "NN" : "NT", bm, bn);
+  {
+    char name[96];
+    gemm_dma_name(dtype, p, tile, name, sizeof name);
+    note_kernel("%s", name);
+  }
 #define UGHIP_DMA_CASE(T)                                                                                                  \
   if (tile == 256) return nn ? launch<T, 256, 256, true>(stream, p, batch) : launch<T, 256, 256, false>(stream, p, batch); \
   if (tile == 128) return nn ? launch<T, 256, 128, true>(stream, p, batch) : launch<T, 256, 128, false>(stream, p, batch); \

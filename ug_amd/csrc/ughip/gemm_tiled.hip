@@ -637,6 +637,24 @@ size_t gemm_tiled_workspace_bytes(int dtype, const MMArgs& p, size_t batch, cons
   return nsplit > 1 || epi ? (size_t)nsplit * batch * (size_t)p.M * p.N * sizeof(float) : 0;
 }
 
+void gemm_tiled_name(int dtype, const MMArgs& p, size_t batch, bool rhs_bf16, const GemmEpilogue* epi, char* out, size_t out_len) {
+  const bool nt = p.b_rs == 1 && p.b_cs != 1;
+  const int s = pick_shape(p, batch, dtype, epi != nullptr);
+  if (s < 0) {
+    snprintf(out, out_len, "gemm_tiled<does not take this product>");
+    return;
+  }
+  const int nsplit = pick_split(dtype, p, batch, s, epi != nullptr).nsplit;
+  const char* tn = rhs_bf16 ? "f32xbf16" : dtype == UGHIP_F32 ? "f32" : dtype == UGHIP_F16 ? "f16" : "bf16";
+  const bool ragged = s != 0 && (p.M % kShapes[s][0] || p.N % kShapes[s][1]);
+  char split[48] = "";
+  if (nsplit > 1 || epi)
+    snprintf(split, sizeof split, ",splitK=%d%s%s", nsplit, !epi ? "" : epi->kind == GemmEpilogue::ADD ? ",+residual" : epi->kind == GemmEpilogue::SWIGLU ? ",swiglu" : "",
+             epi && epi->out_f32 ? ",f32 out" : "");
+  snprintf(out, out_len, "gemm_tiled<%s,%s,%dx%d,%dt%s%s>", tn, nt ? "NT" : "NN", kShapes[s][0], kShapes[s][1], s == 0 && !tune_on(TUNE_GEMM_4WAVES) ? 512 : 256,
+           ragged ? ",ragged" : "", split);
+}
+
 hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, size_t batch, float* workspace, bool rhs_bf16, const GemmEpilogue* epi) {
   const bool nt = p.b_rs == 1 && p.b_cs != 1;
   if (rhs_bf16 && (dtype != UGHIP_F32 || !nt)) return hipErrorInvalidValue;
@@ -647,14 +665,9 @@ hipError_t gemm_tiled_launch(hipStream_t stream, int dtype, const MMArgs& p, siz
   if (s < 0) return hipErrorInvalidValue;
   const int nsplit = pick_split(dtype, p, batch, s, epi != nullptr).nsplit;
   {
-    const char* tn = rhs_bf16 ? "f32xbf16" : dtype == UGHIP_F32 ? "f32" : dtype == UGHIP_F16 ? "f16" : "bf16";
-    const bool ragged = s != 0 && (p.M % kShapes[s][0] || p.N % kShapes[s][1]);
-    char split[48] = "";
-    if (nsplit > 1 || epi)
-      snprintf(split, sizeof split, ",splitK=%d%s%s", nsplit, !epi ? "" : epi->kind == GemmEpilogue::ADD ? ",+residual" : epi->kind == GemmEpilogue::SWIGLU ? ",swiglu" : "",
-               epi && epi->out_f32 ? ",f32 out" : "");
-    note_kernel("gemm_tiled<%s,%s,%dx%d,%dt%s%s>", tn, nt ? "NT" : "NN", kShapes[s][0], kShapes[s][1], s == 0 && !tune_on(TUNE_GEMM_4WAVES) ? 512 : 256,
-                  ragged ? ",ragged" : "", split);
+    char name[160];
+    gemm_tiled_name(dtype, p, batch, rhs_bf16, epi, name, sizeof name);
+    note_kernel("%s", name);
   }
   if (nsplit > 1 || epi) {
     if (!workspace) return hipErrorInvalidValue;

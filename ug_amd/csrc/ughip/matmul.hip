@@ -420,6 +420,30 @@ static int grow_gemm_ws(ughip_device* dev, size_t bytes) {
   return UGHIP_OK;
 }
 
+// Which kernel family a product goes to: decided from shapes, strides, offsets and alignment alone, so that the choice can be
+// asked for without a device (ughip_matmul_plan) and is the same one the launch makes.
+enum Route { ROUTE_GEMV_NT, ROUTE_GEMV_NN, ROUTE_DMA, ROUTE_TILED, ROUTE_ANY, ROUTE_UNSUPPORTED };
+static Route matmul_route(int dtype, bool mixed, const MMArgs& p, size_t b, size_t lhs_offset, size_t rhs_offset, int* dma_tile) {
+  const size_t m = (size_t)p.M, n = (size_t)p.N, k = (size_t)p.K;
+  const bool f32 = dtype == UGHIP_F32;
+  const size_t vec = f32 ? 4 : 8;
+  // m <= 8: GEMV kernels.  Vector loads need 16-byte aligned rows; strides of size-1 dims are never used.
+  const long long lv = (long long)vec;
+  const bool small_m = m <= 8 && p.a_cs == 1 && b <= 65535;
+  const bool lhs_vec_ok = (m == 1 || p.a_rs % lv == 0) && (b == 1 || p.a_bs % lv == 0) && lhs_offset % vec == 0;
+  const bool rhs_vec_ok = (b == 1 || p.b_bs % lv == 0) && rhs_offset % vec == 0;
+  const bool gemv_nt_ok = small_m && lhs_vec_ok && rhs_vec_ok && k % vec == 0 && p.b_rs == 1 && (n == 1 || p.b_cs % lv == 0);
+  const bool gemv_nn_ok = small_m && f32 && rhs_vec_ok && n % 4 == 0 && p.b_cs == 1 && (k == 1 || p.b_rs % 4 == 0);
+  if (mixed && (!gemm_tiled_supported(UGHIP_F32, p, b, true) || rhs_offset % 8 != 0)) return ROUTE_UNSUPPORTED;
+  if (!mixed && gemv_nt_ok) return ROUTE_GEMV_NT;
+  if (!mixed && gemv_nn_ok) return ROUTE_GEMV_NN;
+  if (const int bn = mixed ? 0 : gemm_dma_pick(dtype, p, b)) {
+    *dma_tile = bn;
+    return ROUTE_DMA;
+  }
+  return gemm_tiled_supported(dtype, p, b, mixed) ? ROUTE_TILED : ROUTE_ANY;
+}
+
 static int matmul_impl(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs, const ughip_slice* rhs, size_t b, size_t m, size_t n, size_t k,
                        size_t rank, const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset, const size_t* rhs_dims, const size_t* rhs_strides,
                        size_t rhs_offset, bool no_alloc) {
@@ -461,21 +485,14 @@ static int matmul_impl(ughip_device* dev, ughip_slice* dst, const ughip_slice* l
   p.c = dst->ptr;
   const bool f32 = dst->dtype == UGHIP_F32;
   hipStream_t st = dev->stream;
-  const size_t vec = f32 ? 4 : 8;
-  // m <= 8: GEMV kernels.  Vector loads need 16-byte aligned rows; strides of size-1 dims are never used.
-  const long long lv = (long long)vec;
-  const bool small_m = m <= 8 && p.a_cs == 1 && b <= 65535;
-  const bool lhs_vec_ok = (m == 1 || p.a_rs % lv == 0) && (b == 1 || p.a_bs % lv == 0) && lhs_offset % vec == 0;
-  const bool rhs_vec_ok = (b == 1 || p.b_bs % lv == 0) && rhs_offset % vec == 0;
-  const bool gemv_nt_ok = small_m && lhs_vec_ok && rhs_vec_ok && k % vec == 0 && p.b_rs == 1 && (n == 1 || p.b_cs % lv == 0);
-  const bool gemv_nn_ok = small_m && f32 && rhs_vec_ok && n % 4 == 0 && p.b_cs == 1 && (k == 1 || p.b_rs % 4 == 0);
-  if (mixed) {
-    if (!gemm_tiled_supported(UGHIP_F32, p, b, true) || rhs_offset % 8 != 0)
-      return set_error(UGHIP_ERR_UNSUPPORTED,
-                       "matmul: an F32 product with a BF16 rhs is built for an [n, k]-major rhs with k a multiple of 32 and rows that "
-                       "start on 8-byte boundaries (got m %zu, n %zu, k %zu, rhs strides %lld, %lld)",
-                       m, n, k, p.b_rs, p.b_cs);
-  }
+  int dma_tile = 0;
+  const Route route = matmul_route(dst->dtype, mixed, p, b, lhs_offset, rhs_offset, &dma_tile);
+  const bool gemv_nt_ok = route == ROUTE_GEMV_NT, gemv_nn_ok = route == ROUTE_GEMV_NN;
+  if (route == ROUTE_UNSUPPORTED)
+    return set_error(UGHIP_ERR_UNSUPPORTED,
+                     "matmul: an F32 product with a BF16 rhs is built for an [n, k]-major rhs with k a multiple of 32 and rows that "
+                     "start on 8-byte boundaries (got m %zu, n %zu, k %zu, rhs strides %lld, %lld)",
+                     m, n, k, p.b_rs, p.b_cs);
   const char* tn = f32 ? "f32" : dst->dtype == UGHIP_F16 ? "f16" : "bf16";
   if (!mixed && gemv_nt_ok) {
     note_kernel("gemv_nt<%s>", tn);
@@ -488,10 +505,10 @@ static int matmul_impl(ughip_device* dev, ughip_slice* dst, const ughip_slice* l
     if (m == 1) gemv_nn_f32<1><<<grid, 1024, 0, st>>>(p);
     else if (m <= 4) gemv_nn_f32<4><<<grid, 1024, 0, st>>>(p);
     else gemv_nn_f32<8><<<grid, 1024, 0, st>>>(p);
-  } else if (const int bn = mixed ? 0 : gemm_dma_pick(dst->dtype, p, b)) {
-    UGHIP_HIPCHK(gemm_dma_launch(st, dst->dtype, p, b, bn));
+  } else if (route == ROUTE_DMA) {
+    UGHIP_HIPCHK(gemm_dma_launch(st, dst->dtype, p, b, dma_tile));
     return UGHIP_OK;
-  } else if (gemm_tiled_supported(dst->dtype, p, b, mixed)) {
+  } else if (route == ROUTE_TILED) {
     const size_t ws_bytes = gemm_tiled_workspace_bytes(dst->dtype, p, b);
     if (no_alloc) {
       // the partial tiles go to the device's copy of the static array; every slab writes its whole tile before
@@ -657,6 +674,34 @@ static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x
     return UGHIP_OK;
   }
   UGHIP_HIPCHK(gemm_tiled_launch(dev->stream, dtype, p, 1, static_cast<float*>(dev->gemm_ws), mixed, &epi));
+  return UGHIP_OK;
+}
+
+// The kernel ughip_matmul would launch for contiguous operands of these shapes (rhs_nk: the rhs stored [n, k], i.e. strides (1, k)),
+// by the name ughip_last_kernel() reports after the launch.  Needs no device: the choice depends on shapes and on the cost models.
+extern "C" int ughip_matmul_plan(int dtype, int rhs_dtype, size_t b, size_t m, size_t n, size_t k, int rhs_nk, char* buf, size_t buf_len) {
+  if (!buf || !buf_len) return set_error(UGHIP_ERR_INVALID, "matmul_plan: no buffer");
+  const bool mixed = dtype == UGHIP_F32 && rhs_dtype == UGHIP_BF16;
+  if ((!mixed && dtype != rhs_dtype) || (dtype != UGHIP_F32 && dtype != UGHIP_BF16 && dtype != UGHIP_F16))
+    return set_error(UGHIP_ERR_UNSUPPORTED, "matmul_plan: dtypes %s x %s", dtype_name(dtype), dtype_name(rhs_dtype));
+  if (!b || !m || !n || !k || b > 65535 || m > 0x7fffffffull || n > 0x7fffffffull || k > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "matmul_plan: bad shape");
+  MMArgs p;
+  p.M = (int)m, p.N = (int)n, p.K = (int)k;
+  p.a_rs = (long long)k, p.a_cs = 1;
+  p.b_rs = rhs_nk ? 1 : (long long)n, p.b_cs = rhs_nk ? (long long)k : 1;
+  p.a_bs = (long long)(m * k), p.b_bs = (long long)(n * k), p.c_bs = (long long)(m * n);
+  p.a = p.b = reinterpret_cast<const void*>(uintptr_t(1) << 20);  // stand-ins with the alignment every allocation has; never dereferenced
+  p.c = reinterpret_cast<void*>(uintptr_t(1) << 20);
+  int tile = 0;
+  const char* tn = dtype == UGHIP_F32 ? "f32" : dtype == UGHIP_F16 ? "f16" : "bf16";
+  switch (matmul_route(dtype, mixed, p, b, 0, 0, &tile)) {
+    case ROUTE_UNSUPPORTED: return set_error(UGHIP_ERR_UNSUPPORTED, "matmul_plan: an F32 product with a BF16 rhs needs an [n, k]-major rhs and k %% 32 == 0");
+    case ROUTE_GEMV_NT: snprintf(buf, buf_len, "gemv_nt<%s>", tn); break;
+    case ROUTE_GEMV_NN: snprintf(buf, buf_len, "gemv_nn<f32>"); break;
+    case ROUTE_DMA: gemm_dma_name(dtype, p, tile, buf, buf_len); break;
+    case ROUTE_TILED: gemm_tiled_name(dtype, p, b, mixed, nullptr, buf, buf_len); break;
+    default: snprintf(buf, buf_len, "gemm_any<%s>", tn); break;
+  }
   return UGHIP_OK;
 }
 
