@@ -32,7 +32,7 @@ ALGO_BYTES = 2 * N * 4 + 4      # read a, read b, write one f32
 # HBM bytes per step from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`, scaled by the counters' reading for the
 # --copy-probe kernel.  A run of bench.py cannot read those counters itself: the figure is the one recorded in the
 # profile named here, taken with the command that file gives, and the line says so.
-TRAFFIC_BYTES = 134222184
+TRAFFIC_BYTES = 134212407
 TRAFFIC_SOURCE = "profiles/fused_reduce_2pow24_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE; not measured by this run)"
 
 
