@@ -1589,11 +1589,14 @@ def test_projections_of_several_rows_as_three_bf16_terms(hip, t, k, n):
 
     lin3, add3, glu3, kern3 = run(x3_ops)
     lin1, add1, glu1, kern1 = run(f32_ops)
-    if t <= 64:
-        # up to 64 rows the hooks keep the f32 pipe (a 32- or 64-row tile there is as fast as the split, three planes and an f32 fold)
+    if t <= 32:
+        # up to 32 rows the hooks keep the f32 pipe (a 32-row tile there is faster than three terms on a 128-row tile)
         assert kern3.startswith("gemm_tiled<f32xbf16,NT,"), kern3
         lin3, add3, glu3, kern3 = run_c_abi()
-    assert kern3.startswith("gemm_tiled<bf16,NT,") and "f32 out" in kern3, kern3   # (fewer than 384 rows in every case here)
+    if 32 < t <= 128:
+        assert kern3.startswith("rows_x3<128x128,3 terms split in the kernel,"), kern3   # the split happens inside the product
+    else:
+        assert kern3.startswith("gemm_tiled<bf16,NT,") and "f32 out" in kern3, kern3   # (fewer than 384 rows in every case here)
     assert kern1.startswith("gemm_tiled<f32xbf16,NT,"), kern1
     x64, w64, gu64 = x.reshape(t, k).astype(np.float64), w.reshape(n, k).astype(np.float64), wgu.reshape(2 * n, k).astype(np.float64)
     eps = float(np.finfo(np.float32).eps)
@@ -1644,6 +1647,89 @@ def test_three_bf16_terms_keep_infinities_and_nans_where_the_f32_pipe_has_them(h
     fin = np.isfinite(f32)
     assert fin[[0, 1, 2, 4, 127]].all()
     np.testing.assert_allclose(x3[fin], f32[fin], rtol=0, atol=k * float(np.finfo(np.float32).eps) * 4.0)
+
+
+@pytest.mark.parametrize("t,k,n,units", [(128, 2048, 11264, None), (128, 5632, 2048, None), (128, 2048, 2560, None), (100, 256, 192, "1"), (65, 512, 1000, "3"),
+                                         (97, 192, 136, "2"), (128, 320, 392, "7"), (77, 64, 8, None), (128, 1024, 640, "16"), (113, 448, 264, "5"), (33, 2048, 2048, None), (48, 128, 520, "1")])
+def test_three_bf16_terms_split_inside_the_product(hip, tune, t, k, n, units):
+    """33 .. 128 rows: rows_x3 reads the f32 rows as they are and splits them on their way into LDS; workgroups take runs of
+    (column tile, k tile) units that may cross from one column tile into the next, and the fold adds every tile's slabs in a
+    fixed order.  The library's own choice of units at the projection shapes of a llama layer (gate|up: 11 units for each of
+    256 workgroups, a third of which cross a tile boundary), forced unit counts on small ragged shapes (last tiles that hang
+    over the end of the columns and of the rows, fewer units than a tile has k tiles and more); against float64 with the k eps
+    bound of the f32 product, against the kernels that take planes (UGHIP_X3_ROWS=0: the same exact terms, sums in another
+    order), small integers exactly, twice the same bits, and a sentinel behind every result."""
+    import ctypes as C
+    print("three bf16 terms, split in the kernel", t, k, n, units, flush=True)
+    x = rng.normal(181, t * k)
+    w = rng.bf16_round(rng.normal(182, n * k, 0.05))
+    wgu = rng.bf16_round(rng.normal(183, 2 * n * k, 0.05))
+    r = rng.normal(184, t * n)
+    bits = rng.to_bf16_bits
+    lib, dev, z = ug_amd.ughip_lib(), C.c_void_p(hip.raw_hip()), C.c_size_t
+    raw = lambda s_: C.c_void_p(s_.raw())
+
+    def run(xv, wv, guv):
+        sx, sw, sgu, sr = hip.slice_from(xv), hip.slice_from(bits(wv)), hip.slice_from(bits(guv)), hip.slice_from(r)
+        guard = 64
+        d = hip.slice_from(np.full(t * n + guard, 7.0, np.float32))
+        out, kerns = [], []
+        for call in (lambda: lib.ughip_linear_rows(dev, raw(sx), raw(sw), raw(d), z(t), z(n), z(k), C.c_int(1)),
+                     lambda: lib.ughip_linear_add_rows(dev, raw(sx), raw(sw), raw(sr), raw(d), z(t), z(n), z(k), C.c_int(1)),
+                     lambda: lib.ughip_linear_swiglu_rows(dev, raw(sx), raw(sgu), raw(d), z(t), z(n), z(k), C.c_int(1))):
+            assert call() == 0, lib.ughip_last_error()
+            kerns.append(ug_amd.last_kernel())
+            v = d.to_vec()
+            assert np.all(v[t * n:] == 7.0), "wrote past the end of the result"
+            out.append(v[:t * n].reshape(t, n).copy())
+        return out, kerns
+
+    if units:
+        tune.setenv("UGHIP_X3_ROWS", units)
+    (lin, add, glu), kerns = run(x, w, wgu)
+    for kn, word in zip(kerns, (",fold>", "+residual in the fold", "swiglu fold")):
+        assert kn.startswith("rows_x3<128x128,3 terms split in the kernel,") and word in kn, kn
+    if units and -(-n // 128) * (k // 64) <= 256 * int(units):
+        assert f",{units} units x " in kerns[0], kerns[0]
+    if (t, k, n) == (128, 2048, 11264):
+        # 2816 units: 11 or 12 for each of at most 256 workgroups, a third of which cross from one column tile into the next
+        import re
+        u_, g_, s_ = map(int, re.search(r",(\d+) units x (\d+) workgroups,(\d+) slabs", kerns[0]).groups())
+        assert u_ in (11, 12) and g_ == -(-2816 // u_) and s_ == 4, kerns[0]
+    (lin_b, add_b, glu_b), _ = run(x, w, wgu)
+    assert np.array_equal(lin, lin_b) and np.array_equal(add, add_b) and np.array_equal(glu, glu_b)
+    tune.setenv("UGHIP_X3_ROWS", "0")
+    (lin0, add0, glu0), kerns0 = run(x, w, wgu)
+    assert all(kn.startswith("gemm_tiled<bf16,NT,") for kn in kerns0), kerns0
+    x64, w64, gu64 = x.reshape(t, k).astype(np.float64), w.reshape(n, k).astype(np.float64), wgu.reshape(2 * n, k).astype(np.float64)
+    eps = float(np.finfo(np.float32).eps)
+    lin64 = x64 @ w64.T
+    bound = k * eps * (np.abs(x64) @ np.abs(w64).T) + 1e-7
+    assert np.all(np.abs(lin - lin64) <= bound)
+    assert np.all(np.abs(add - (lin64 + r.reshape(t, n))) <= bound + 2 * eps * np.abs(lin64 + r.reshape(t, n)))
+    gg, uu = x64 @ gu64[:n].T, x64 @ gu64[n:].T
+    g64 = gg / (1.0 + np.exp(-gg)) * uu
+    g_bound = k * eps * ((np.abs(x64) @ np.abs(gu64[:n]).T) * (np.abs(uu) * 1.3) + (np.abs(x64) @ np.abs(gu64[n:]).T) * np.abs(gg / (1.0 + np.exp(-gg)))) + 8 * eps * np.abs(g64) + 1e-7
+    assert np.all(np.abs(glu - g64) <= g_bound)
+    assert np.max(np.abs(lin - lin0)) <= 0.25 * np.max(bound) and np.max(np.abs(add - add0)) <= 0.25 * np.max(bound) + 2 * eps * np.abs(add0).max()
+    assert np.all(np.abs(glu - glu0) <= 2 * g_bound)
+    # small integers: every partial sum is exact
+    if units:
+        tune.setenv("UGHIP_X3_ROWS", units)
+    else:
+        tune.delenv("UGHIP_X3_ROWS")
+    xi, wi, gui = np.floor(x * 4).astype(np.float32), np.floor(w * 40).astype(np.float32), np.floor(wgu * 40).astype(np.float32)
+    (lin_i, add_i, _), kerns_i = run(xi, wi, gui)
+    assert kerns_i[0].startswith("rows_x3<"), kerns_i
+    want = (xi.reshape(t, k).astype(np.float64) @ wi.reshape(n, k).astype(np.float64).T).astype(np.float32)
+    np.testing.assert_array_equal(lin_i, want)
+    # all 24 mantissa bits survive the split: x against rows of the identity comes back bit for bit
+    if n >= k:
+        full = (np.float32(1.0) + np.arange(t * k, dtype=np.float32).reshape(t, k) % 8388607 * np.float32(2.0 ** -23)) * rng.normal(185, t * k).reshape(t, k).astype(np.float32)
+        eye = np.zeros((n, k), np.float32)
+        eye[np.arange(k), np.arange(k)] = 1.0
+        (back, _, _), _ = run(full.ravel(), eye.ravel(), wgu)
+        np.testing.assert_array_equal(back[:, :k], full)
 
 
 @pytest.mark.parametrize("t,k,n,force,split", [(400, 512, 640, "3", None), (400, 512, 640, "4", None), (400, 512, 640, "5", None), (517, 256, 264, "5", None),

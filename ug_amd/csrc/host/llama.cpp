@@ -352,10 +352,10 @@ struct HipOps : Ops {
 
   // How nine or more f32 rows meet this matrix: three bf16 terms per row element on the bf16 matrix pipe when that was
   // asked for and the matrix is bf16 with k a multiple of 64, else the f32 pipe.
-  // Up to 64 rows the f32 pipe on a 32- or 64-row tile is as fast as three bf16 terms (which cost a split and an f32
-  // fold per product): 1.95-2.1 ms against 2.2 for a prompt of 2 .. 32 tokens, the same at 64.
+  // Up to 32 rows the f32 pipe on a 32-row tile is faster (2.0-2.1 ms for a prompt of 9 .. 32 tokens against 2.3); from 33
+  // rows the product that splits the rows itself is (2.30-2.39 ms for 40 .. 64 tokens against 2.50-2.57).
   int product_for(const LB& w, size_t k, size_t rows) const {
-    return bf16x3_ && rows > 64 && w.dtype() == DType::BF16 && k % 64 == 0 ? UGHIP_PRODUCT_BF16X3 : UGHIP_PRODUCT_F32;
+    return bf16x3_ && rows > 32 && w.dtype() == DType::BF16 && k % 64 == 0 ? UGHIP_PRODUCT_BF16X3 : UGHIP_PRODUCT_F32;
   }
 
   // Several positions of f32 rows against a row-major [n, k] matrix (f32 or bf16) in shapes the tiled kernel takes:

@@ -65,4 +65,18 @@ double gemm_dma_cost_us(const MMArgs& p, size_t batch, int tile);
 void gemm_dma_name(int dtype, const MMArgs& p, int tile, char* out, size_t out_len);
 void gemm_tiled_name(int dtype, const MMArgs& p, size_t batch, bool rhs_bf16, const GemmEpilogue* epi, char* out, size_t out_len);
 
+
+// 1 .. 128 f32 rows x [m, k] against a bf16 matrix [n, k] as three bf16 terms per row element, the split done inside the product
+// (rows_x3.hip): partial sums of `units` consecutive (column tile, k tile) units per workgroup go to f32 slabs in `ws`, a fold adds
+// them in a fixed order and applies the epilogue.  n % 8 == 0, k % 64 == 0, 16-byte aligned buffers.
+struct RowsX3Plan {
+  int units = 0, groups = 0, max_slabs = 0;
+  size_t ws_bytes = 0;
+};
+bool rows_x3_supported(const void* x, const void* w, const void* c, const void* residual, size_t m, size_t n, size_t k);
+RowsX3Plan rows_x3_plan(size_t m, size_t n, size_t k, int forced_units, int num_cus);
+void rows_x3_name(const RowsX3Plan& pl, GemmEpilogue::Kind kind, char* out, size_t out_len);
+hipError_t rows_x3_launch(hipStream_t stream, const float* x, const void* w, float* ws, float* c, size_t m, size_t n, size_t k, const RowsX3Plan& pl, GemmEpilogue::Kind kind,
+                          const float* residual);
+
 }  // namespace ughip

@@ -69,6 +69,7 @@ enum TuneKey {
   TUNE_GEMV_BF16_ROWS,      // 0: bf16 matrices take the f32 kernels' lane layout
   TUNE_X3_DMA,              // three-term bf16 products: 0 keeps gemm_tiled, 3 / 4 / 5 force a gemm_dma4 tile
   TUNE_X3_SPLIT,            // K split of the three-term product on gemm_dma4
+  TUNE_X3_ROWS,             // three-term bf16 products of 65 .. 128 rows: 0 keeps the kernels that take planes, n > 0 forces n units per workgroup of rows_x3
   TUNE_ATT_SPLIT,           // key ranges per head of single-query attention
   TUNE_NO_PARAMETRIC,       // (set at all) shapes stay literals in generated kernels
   TUNE_NO_NT_LOADS,         // (set at all) the grid-wide reduction reads with ordinary loads

@@ -619,6 +619,19 @@ static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x
   if (int rc = device_activate(dev)) return rc;
   GemmEpilogue epi{kind, residual ? static_cast<const float*>(residual->ptr) : nullptr};
   epi.out_f32 = x3;
+  // 33 .. 128 rows: the kernel that splits the rows itself (no planes through memory, no launch for the split).  In a 22-layer
+  // prefill of 128 positions, with the matrices coming from memory: q|k|v 13.4 us against 17.9 (split + product), o 12.6 against
+  // 19.5, gate|up 30.6 against 37.2, down 19.7 against 26.5.  Two row tiles (129 .. 256 rows) were slower than the kernels below,
+  // and up to 32 rows its 128-row tile is mostly padding.
+  long long x3_rows = -1;
+  tune_get(TUNE_X3_ROWS, &x3_rows);
+  if (x3 && m > 32 && m <= 128 && x3_rows != 0 && rows_x3_supported(x->ptr, w->ptr, dst->ptr, residual ? residual->ptr : nullptr, m, rows, k)) {
+    const RowsX3Plan pl = rows_x3_plan(m, rows, k, x3_rows > 0 ? (int)x3_rows : 0, dev->num_cus);
+    if (int rc = grow_gemm_ws(dev, pl.ws_bytes)) return rc;
+    UGHIP_HIPCHK(rows_x3_launch(dev->stream, static_cast<const float*>(x->ptr), w->ptr, static_cast<float*>(dev->gemm_ws), static_cast<float*>(dst->ptr), m, rows, k, pl, kind,
+                                epi.residual));
+    return UGHIP_OK;
+  }
   // Many rows of planes: the one-wave-per-SIMD kernel where it is priced cheaper (a prompt of a thousand positions and
   // more).  Its result leaves as f32 with the residual added on the way; SwiGLU goes through the scratch block and the fold.
   int dma_tile = 0, dma_split = 1;
