@@ -961,7 +961,7 @@ std::vector<Cache> Model::new_cache() const {
 }
 
 // model.rs:259-269, 365-373
-LB Model::fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache, const std::function<void(const LB&)>* after_layer) const {
+LB Model::fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache, const std::function<void(const LB&)>* after_layer, bool last_position_only) const {
   if (cache.size() != layers_.size()) bail("cache/layer count mismatch");
   LB xs = index_select(embedding_, tokens);
   float eps = (float)cfg_.rms_norm_eps;
@@ -983,7 +983,12 @@ LB Model::fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache, const 
     }
     if (after_layer) (*after_layer)(xs);
   }
-  if (fused_attention_ >= 3) return ops_->linear_packed(xs, {head_}, &ln_f_, eps);
+  if (fused_attention_ >= 3) {
+    // a prompt whose logits are read at the last position only: one row through the norm and the head (the row-vector kernel
+    // streams the head once, as in a decode step) instead of all of them
+    if (last_position_only && xs.rank() == 3 && xs.dims()[1] > 1) xs = xs.narrow(1, xs.dims()[1] - 1, 1);
+    return ops_->linear_packed(xs, {head_}, &ln_f_, eps);
+  }
   xs = rms_norm(xs, ln_f_, eps);
   return ops_->linear(xs, head_);
 }
@@ -1063,8 +1068,8 @@ std::vector<int32_t> generate_greedy_queued(const Model& model, const std::vecto
       st.layers.push_back(std::make_unique<CompiledSchedule>(part.compile_and_run(ccache)));
       st.n_items += part.items().size();
     };
-    LB logits = model.fwd(st.tokens, pos[i], cache, run_now && by_layer ? &realise_layer : nullptr);
-    st.logits = ops.argmax_into(forced ? picked : tokens[i + 1], logits, st.t - 1, ids, vals, i);
+    LB logits = model.fwd(st.tokens, pos[i], cache, run_now && by_layer ? &realise_layer : nullptr, true);
+    st.logits = ops.argmax_into(forced ? picked : tokens[i + 1], logits, logits.dims()[logits.rank() - 2] - 1, ids, vals, i);
     auto t1 = clock::now();
     Schedule schedule = Schedule::create_one(st.logits);
     auto t2 = clock::now();

@@ -194,7 +194,10 @@ class Model {
   std::vector<Cache> new_cache() const;
   // after_layer, when given, is called with the hidden state behind every layer: a caller that realises it there
   // (schedule, compile, launch) has the device working on layer i while the graph of layer i + 1 is still being built.
-  LB fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache, const std::function<void(const LB&)>* after_layer = nullptr) const;
+  // last_position_only (fusion level 3): the head runs on the last position alone and the result is [b, 1, vocab] -- what a
+  // generation loop reads of a prompt's logits; the layers and the caches are the same.
+  LB fwd(const LB& tokens, const LB& pos, std::vector<Cache>& cache, const std::function<void(const LB&)>* after_layer = nullptr,
+         bool last_position_only = false) const;
   const Config& config() const { return cfg_; }
   const ug::DevicePtr& device() const { return dev_; }
   const Rope& rope() const { return rope_; }

@@ -266,9 +266,18 @@ __global__ void __launch_bounds__(512) rows_x3_kernel(const float* __restrict__ 
 // (c[m, n / 2] = silu(sum[:, :n / 2]) * sum[:, n / 2:], x / (1 + exp(-x)) as the lazy graph of ug-llama/src/model.rs:44-52 computes it).
 // Tile T has the slabs of the workgroups (T KT) / U .. (T KT + KT - 1) / U.
 __device__ __forceinline__ f32x4 tile_sum(const float* __restrict__ slabs, size_t slab_elems, size_t at, int col, int KT, int U) {
-  const int T = col / BN, first = (T * KT) / U, last = (T * KT + KT - 1) / U;
+  const int T = col / BN, first = (T * KT) / U, last = (T * KT + KT - 1) / U, cnt = last - first;
   f32x4 s = *reinterpret_cast<const f32x4*>(slabs + at);
-  for (int g = 1; g <= last - first; ++g) s += *reinterpret_cast<const f32x4*>(slabs + (size_t)g * slab_elems + at);
+  // eight slabs at a time, all eight loads on their way before the first is added (a slab past the last is the last one again,
+  // loaded and not added): the order of the sum stays slab by slab
+  for (int g = 1; g <= cnt; g += 8) {
+    f32x4 v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = *reinterpret_cast<const f32x4*>(slabs + (size_t)min(g + e, cnt) * slab_elems + at);
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (g + e <= cnt) s += v[e];
+  }
   return s;
 }
 template <int EPI>
