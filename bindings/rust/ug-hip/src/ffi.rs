@@ -445,6 +445,16 @@ extern "C" {
         k: usize,
         product: c_int,
     ) -> c_int;
+    pub fn ughip_linear_rows_plan(
+        w_dtype: c_int,
+        product: c_int,
+        form: c_int,
+        m: usize,
+        n: usize,
+        k: usize,
+        buf: *mut c_char,
+        buf_len: usize,
+    ) -> c_int;
     pub fn ughip_argmax_row(
         dev: *mut UghipDevice,
         logits: *const UghipSlice,

@@ -414,7 +414,10 @@ int ughip_gemv_add(ughip_device* dev, const ughip_slice* x, const ughip_slice* w
  *                         three planes by the matrix as it is stored: every product term is exact in f32, the sums are f32
  *                         sums in another order than the f32 pipe's, and three bf16 MFMAs replace eight times their work in
  *                         f32 ones.  Same accuracy class as the F32 product (k eps bound), not bit-identical to it.
- *                         Needs k % 64 == 0 and a BF16 matrix.  Products of many rows (a prompt of several hundred
+ *                         Needs k % 64 == 0 and a BF16 matrix.  33 .. 128 rows take a kernel that reads the f32 rows as
+ *                         they are and splits them on their way into LDS (no planes in memory, no launch for the
+ *                         split); workgroups take runs of (column tile, k tile) units and a fold adds every tile's
+ *                         partial sums in a fixed order.  Products of many rows (a prompt of several hundred
  *                         positions and more) run the planes on the one-wave-per-SIMD 16-bit kernel, whichever of the two
  *                         is priced cheaper; the terms are the same, the order of the sums is that kernel's.
  * ughip_linear_rows: dst[m, n] = x w^T.
@@ -430,6 +433,12 @@ int ughip_linear_add_rows(ughip_device* dev, const ughip_slice* x, const ughip_s
                           int product);
 int ughip_linear_swiglu_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w,
                              ughip_slice* dst, size_t m, size_t n, size_t k, int product);
+/* No counterpart in the reference, no device needed: the kernel the three entry points above would launch (form 0:
+ * ughip_linear_rows, 1: ughip_linear_add_rows, 2: ughip_linear_swiglu_rows) for m rows against an [n, k] matrix of
+ * w_dtype, by the name ughip_last_kernel() reports after the launch -- kernel family, tile, units or K split, fold.
+ * Like ughip_matmul_plan: tests pin the plans of the shapes that matter. */
+int ughip_linear_rows_plan(int w_dtype, int product, int form, size_t m, size_t n, size_t k, char* buf,
+                           size_t buf_len);
 
 /* ---- greedy step on the device ----------------------------------------------------------------
  * Row `row` of logits [rows, n] (F32): the index of its largest value (the lowest index among

@@ -479,6 +479,32 @@ def test_plan_names_what_is_launched(hip, dtype_name, bmnk, rhs_nk):
     assert buf.value.decode() == ug_amd.last_kernel()
 
 
+@pytest.mark.parametrize("w_bf16,product,form,m,n,k", [(True, 1, 0, 128, 2560, 2048), (True, 1, 2, 128, 5632, 2048), (True, 1, 1, 100, 2048, 5632), (True, 1, 0, 32, 520, 128),
+                                                       (True, 1, 1, 200, 264, 256), (True, 1, 2, 517, 264, 768), (True, 1, 0, 1100, 2048, 2048), (True, 0, 0, 128, 2560, 2048),
+                                                       (False, 0, 1, 128, 2048, 2048), (True, 0, 2, 16, 64, 64)])
+def test_rows_plan_names_what_is_launched(hip, w_bf16, product, form, m, n, k):
+    """ughip_linear_rows_plan (no device) and the launches of ughip_linear_rows / _add_rows / _swiglu_rows agree on the kernel:
+    family, tile, units or K split, and what the fold does."""
+    import ctypes as C
+    lib, dev, z = ug_amd.ughip_lib(), C.c_void_p(hip.raw_hip()), C.c_size_t
+    raw = lambda s_: C.c_void_p(s_.raw())
+    rows = 2 * n if form == 2 else n
+    wv = rng.bf16_round(rng.normal(52, rows * k, 0.05))
+    sx, sw = hip.slice_from(rng.normal(51, m * k)), hip.slice_from(rng.to_bf16_bits(wv) if w_bf16 else wv)
+    sr, d = hip.slice_from(rng.normal(53, m * n)), hip.allocate_uninit(ug_amd.F32, m * n)
+    if form == 0:
+        rc = lib.ughip_linear_rows(dev, raw(sx), raw(sw), raw(d), z(m), z(n), z(k), C.c_int(product))
+    elif form == 1:
+        rc = lib.ughip_linear_add_rows(dev, raw(sx), raw(sw), raw(sr), raw(d), z(m), z(n), z(k), C.c_int(product))
+    else:
+        rc = lib.ughip_linear_swiglu_rows(dev, raw(sx), raw(sw), raw(d), z(m), z(n), z(k), C.c_int(product))
+    assert rc == 0, lib.ughip_last_error()
+    launched = ug_amd.last_kernel()
+    buf = C.create_string_buffer(200)
+    assert lib.ughip_linear_rows_plan(int(ug_amd.BF16 if w_bf16 else ug_amd.F32), product, form, z(m), z(n), z(k), buf, z(200)) == 0, lib.ughip_last_error()
+    assert buf.value.decode() == launched
+
+
 def test_matmul_16bit_one_wave_per_simd_forced_and_limits(hip, tune):
     """UGHIP_GEMM_SHAPE=3 / 4 / 5 force the kernel's three tiles onto a small problem (bit for bit the register-staged
     kernel's result); shapes it cannot take (K below 4 tiles, a column count that is not a multiple of 8) fall through to

@@ -270,6 +270,47 @@ def _plan(dtype, rhs_dtype, b, m, n, k, rhs_nk):
     return buf.value.decode()
 
 
+def _rows_plan(w_dtype, product, form, m, n, k):
+    lib = ug_amd.ughip_lib()
+    buf = C.create_string_buffer(200)
+    rc = lib.ughip_linear_rows_plan(int(w_dtype), int(product), int(form), C.c_size_t(m), C.c_size_t(n), C.c_size_t(k), buf, C.c_size_t(200))
+    if rc:
+        raise ug_amd.UgError(lib.ughip_last_error().decode())
+    return buf.value.decode()
+
+
+def test_kernel_choice_for_the_rows_of_a_prompt_is_pinned():
+    """The projections of a llama layer (TinyLlama-1.1B shapes) for prompts of several lengths, f32 rows against bf16 matrices
+    as three bf16 terms: 33 .. 128 rows take rows_x3 with the units per workgroup its cost rule picks (every CU busy in one
+    round, then as few slabs as the units' time allows); fewer rows and more take the kernels that read planes.  Written down
+    so that a changed rule shows here (the GPU suite checks that the launch reports the planned name:
+    test_rows_plan_names_what_is_launched)."""
+    B, F = ug_amd.BF16, ug_amd.F32
+    X3, F32P = 1, 0
+    want = {
+        # (w dtype, product, form, m, n, k)
+        (B, X3, 0, 128, 2560, 2048): "rows_x3<128x128,3 terms split in the kernel,4 units x 160 workgroups,8 slabs,fold>",
+        (B, X3, 1, 128, 2048, 2048): "rows_x3<128x128,3 terms split in the kernel,4 units x 128 workgroups,8 slabs,+residual in the fold>",
+        (B, X3, 2, 128, 5632, 2048): "rows_x3<128x128,3 terms split in the kernel,12 units x 235 workgroups,4 slabs,swiglu fold>",
+        (B, X3, 1, 128, 2048, 5632): "rows_x3<128x128,3 terms split in the kernel,8 units x 176 workgroups,11 slabs,+residual in the fold>",
+        (B, X3, 0, 128, 32000, 2048): "rows_x3<128x128,3 terms split in the kernel,32 units x 250 workgroups,1 slabs,fold>",
+        (B, X3, 0, 33, 2560, 2048): "rows_x3<128x128,3 terms split in the kernel,4 units x 160 workgroups,8 slabs,fold>",
+        (B, X3, 0, 77, 8, 64): "rows_x3<128x128,3 terms split in the kernel,1 units x 1 workgroups,1 slabs,fold>",
+    }
+    got = {key: _rows_plan(*key) for key in want}
+    assert got == want
+    # outside 33 .. 128 rows: planes through the register-staged kernel, and from a few hundred rows the one-wave-per-SIMD kernel
+    assert _rows_plan(B, X3, 0, 32, 2560, 2048).startswith("gemm_tiled<bf16,NT,")
+    assert _rows_plan(B, X3, 0, 200, 2560, 2048).startswith("gemm_tiled<bf16,NT,")
+    assert _rows_plan(B, X3, 0, 1900, 2560, 2048).startswith("gemm_dma4<bf16,NT,") and "3 planes" in _rows_plan(B, X3, 0, 1900, 2560, 2048)
+    assert _rows_plan(B, F32P, 0, 128, 2560, 2048) == "gemm_tiled<f32xbf16,NT,128x64,256t,splitK=6>"
+    assert _rows_plan(F, F32P, 1, 128, 2048, 2048).startswith("gemm_tiled<f32,NT,")
+    with pytest.raises(ug_amd.UgError):
+        _rows_plan(F, X3, 0, 128, 2560, 2048)      # three terms need a bf16 matrix
+    with pytest.raises(ug_amd.UgError):
+        _rows_plan(B, X3, 0, 128, 2560, 2000)      # k % 64
+
+
 def test_kernel_choice_for_the_baseline_shapes_is_pinned():
     """Which kernel, tile and K split a product gets follows from shapes and from cost models whose constants were fitted to
     measurements (gemm_dma_cost_us, gemm_tiled's pick_shape / pick_split).  The plans for BASELINE's products are written

@@ -583,6 +583,66 @@ __global__ void __launch_bounds__(256) split3_bf16_kernel(const float* __restric
   *reinterpret_cast<ushort4*>(o + 128) = make_ushort4(lo[0], lo[1], lo[2], lo[3]);
 }
 
+// Which kernel a product of rows takes: decided from shapes, alignment and the cost models alone, so that ughip_linear_rows_plan
+// can answer without a device.
+struct RowsRoute {
+  enum Kind { X3_ROWS, DMA_PLANES, TILED } kind = TILED;
+  RowsX3Plan x3;                    // X3_ROWS
+  int dma_tile = 0, dma_split = 1;  // DMA_PLANES
+};
+static RowsRoute rows_route(const MMArgs& p, int dtype, bool x3, GemmEpilogue::Kind kind, const void* x, const void* w, const void* dst, const void* residual, size_t m,
+                            size_t rows, size_t k, int num_cus) {
+  RowsRoute r;
+  // 33 .. 128 rows: the kernel that splits the rows itself (no planes through memory, no launch for the split).  In a 22-layer
+  // prefill of 128 positions, with the matrices coming from memory: q|k|v 13.4 us against 17.9 (split + product), o 12.6 against
+  // 19.5, gate|up 30.6 against 37.2, down 19.7 against 26.5.  Two row tiles (129 .. 256 rows) were slower than the kernels below,
+  // and up to 32 rows its 128-row tile is mostly padding.
+  long long x3_rows = -1;
+  tune_get(TUNE_X3_ROWS, &x3_rows);
+  if (x3 && m > 32 && m <= 128 && x3_rows != 0 && rows_x3_supported(x, w, dst, residual, m, rows, k)) {
+    r.kind = RowsRoute::X3_ROWS;
+    r.x3 = rows_x3_plan(m, rows, k, x3_rows > 0 ? (int)x3_rows : 0, num_cus);
+    return r;
+  }
+  // Many rows of planes: the one-wave-per-SIMD kernel where it is priced cheaper (a prompt of a thousand positions and
+  // more).  Its result leaves as f32 with the residual added on the way; SwiGLU goes through the scratch block and the fold.
+  // (from 384 rows: at 128 and 256 rows the register-staged kernel is as fast or faster for four of the five products of a
+  // llama step -- q|k|v 25.2 us against 28.6 at 256 rows -- and the model below does not see that; at 512 rows this kernel is)
+  long long x3_dma = -1, x3_split = 0;  // tuning aids: X3_DMA 0 keeps the register-staged kernel, 3 / 4 / 5 force a tile; X3_SPLIT n a K split
+  tune_get(TUNE_X3_DMA, &x3_dma);
+  tune_get(TUNE_X3_SPLIT, &x3_split);
+  if (x3 && m >= 384 && x3_dma != 0) {
+    MMArgs q = p;
+    q.c = const_cast<void*>(dst);  // alignment of the result as f32
+    double best = 0;
+    const int forced_tile = x3_dma == 3 ? 256 : x3_dma == 4 ? 128 : x3_dma == 5 ? 64 : 0;
+    const int forced_split = (int)x3_split;
+    for (int tile : {256, 128, 64}) {
+      if (forced_tile && tile != forced_tile) continue;
+      for (int split : {1, 2, 4, 8}) {
+        if (forced_split && split != forced_split) continue;
+        if (!gemm_dma_planes3_split_ok(q, split)) continue;
+        MMArgs qs = q;
+        if (split > 1) qs.K = q.K / split, qs.a_bs = qs.K, qs.b_bs = qs.K / 3, qs.c_bs = (long long)(m * rows);
+        if (!gemm_dma_supported(UGHIP_BF16, qs, (size_t)split, tile)) continue;
+        // the kernel (its model counts 2 bytes per result element), the f32 result's other 2, and the fold where there is one:
+        // the slabs in, the result out, a launch
+        const bool fold = split > 1 || kind == GemmEpilogue::SWIGLU;
+        const double us = gemm_dma_cost_us(qs, (size_t)split, tile) + (double)split * m * rows * 2 / 6.4e6 + (fold ? 3.0 + (double)(split + 1) * m * rows * 4 / 6.4e6 : 0.0);
+        if (!r.dma_tile || us < best * 0.97) r.dma_tile = tile, r.dma_split = split, best = us;
+      }
+    }
+    const double other = gemm_tiled_cost_us(dtype, p, 1);
+    if (r.dma_tile && !forced_tile && other >= 0 && other < best * 1.05) r.dma_tile = 0;  // it has to be clearly cheaper: its model is the rougher one
+  }
+  if (r.dma_tile) r.kind = RowsRoute::DMA_PLANES;
+  return r;
+}
+static const char* dma_planes_tail(GemmEpilogue::Kind kind, bool fold, bool residual) {
+  if (!fold) return residual ? ",+residual" : "";
+  return kind == GemmEpilogue::SWIGLU ? ",swiglu fold" : kind == GemmEpilogue::ADD ? ",+residual in the fold" : ",fold";
+}
+
 // x [m, k] f32 against a row-major [rows, k] matrix (f32 or bf16) through the tiled kernel, the fold applying `kind`.
 // product == UGHIP_PRODUCT_BF16X3 (bf16 matrix): the rows are split into three bf16 planes first and the product runs on
 // the bf16 matrix pipe over a K of 3 k, every K tile of the matrix meeting the three planes of its columns in turn.
@@ -619,51 +679,14 @@ static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x
   if (int rc = device_activate(dev)) return rc;
   GemmEpilogue epi{kind, residual ? static_cast<const float*>(residual->ptr) : nullptr};
   epi.out_f32 = x3;
-  // 33 .. 128 rows: the kernel that splits the rows itself (no planes through memory, no launch for the split).  In a 22-layer
-  // prefill of 128 positions, with the matrices coming from memory: q|k|v 13.4 us against 17.9 (split + product), o 12.6 against
-  // 19.5, gate|up 30.6 against 37.2, down 19.7 against 26.5.  Two row tiles (129 .. 256 rows) were slower than the kernels below,
-  // and up to 32 rows its 128-row tile is mostly padding.
-  long long x3_rows = -1;
-  tune_get(TUNE_X3_ROWS, &x3_rows);
-  if (x3 && m > 32 && m <= 128 && x3_rows != 0 && rows_x3_supported(x->ptr, w->ptr, dst->ptr, residual ? residual->ptr : nullptr, m, rows, k)) {
-    const RowsX3Plan pl = rows_x3_plan(m, rows, k, x3_rows > 0 ? (int)x3_rows : 0, dev->num_cus);
-    if (int rc = grow_gemm_ws(dev, pl.ws_bytes)) return rc;
-    UGHIP_HIPCHK(rows_x3_launch(dev->stream, static_cast<const float*>(x->ptr), w->ptr, static_cast<float*>(dev->gemm_ws), static_cast<float*>(dst->ptr), m, rows, k, pl, kind,
-                                epi.residual));
+  const RowsRoute route = rows_route(p, dtype, x3, kind, x->ptr, w->ptr, dst->ptr, residual ? residual->ptr : nullptr, m, rows, k, dev->num_cus);
+  if (route.kind == RowsRoute::X3_ROWS) {
+    if (int rc = grow_gemm_ws(dev, route.x3.ws_bytes)) return rc;
+    UGHIP_HIPCHK(rows_x3_launch(dev->stream, static_cast<const float*>(x->ptr), w->ptr, static_cast<float*>(dev->gemm_ws), static_cast<float*>(dst->ptr), m, rows, k, route.x3,
+                                kind, epi.residual));
     return UGHIP_OK;
   }
-  // Many rows of planes: the one-wave-per-SIMD kernel where it is priced cheaper (a prompt of a thousand positions and
-  // more).  Its result leaves as f32 with the residual added on the way; SwiGLU goes through the scratch block and the fold.
-  int dma_tile = 0, dma_split = 1;
-  // (from 384 rows: at 128 and 256 rows the register-staged kernel is as fast or faster for four of the five products of a
-  // llama step -- q|k|v 25.2 us against 28.6 at 256 rows -- and the model below does not see that; at 512 rows this kernel is)
-  long long x3_dma = -1, x3_split = 0;  // tuning aids: X3_DMA 0 keeps the register-staged kernel, 3 / 4 / 5 force a tile; X3_SPLIT n a K split
-  tune_get(TUNE_X3_DMA, &x3_dma);
-  tune_get(TUNE_X3_SPLIT, &x3_split);
-  if (x3 && m >= 384 && x3_dma != 0) {
-    MMArgs q = p;
-    q.c = dst->ptr;  // alignment of the result as f32
-    double best = 0;
-    const int forced_tile = x3_dma == 3 ? 256 : x3_dma == 4 ? 128 : x3_dma == 5 ? 64 : 0;
-    const int forced_split = (int)x3_split;
-    for (int tile : {256, 128, 64}) {
-      if (forced_tile && tile != forced_tile) continue;
-      for (int split : {1, 2, 4, 8}) {
-        if (forced_split && split != forced_split) continue;
-        if (!gemm_dma_planes3_split_ok(q, split)) continue;
-        MMArgs qs = q;
-        if (split > 1) qs.K = q.K / split, qs.a_bs = qs.K, qs.b_bs = qs.K / 3, qs.c_bs = (long long)(m * rows);
-        if (!gemm_dma_supported(UGHIP_BF16, qs, (size_t)split, tile)) continue;
-        // the kernel (its model counts 2 bytes per result element), the f32 result's other 2, and the fold where there is one:
-        // the slabs in, the result out, a launch
-        const bool fold = split > 1 || kind == GemmEpilogue::SWIGLU;
-        const double us = gemm_dma_cost_us(qs, (size_t)split, tile) + (double)split * m * rows * 2 / 6.4e6 + (fold ? 3.0 + (double)(split + 1) * m * rows * 4 / 6.4e6 : 0.0);
-        if (!dma_tile || us < best * 0.97) dma_tile = tile, dma_split = split, best = us;
-      }
-    }
-    const double other = gemm_tiled_cost_us(dtype, p, 1);
-    if (dma_tile && !forced_tile && other >= 0 && other < best * 1.05) dma_tile = 0;  // it has to be clearly cheaper: its model is the rougher one
-  }
+  const int dma_tile = route.dma_tile, dma_split = route.dma_split;
   const bool dma_fold = dma_tile && (dma_split > 1 || kind == GemmEpilogue::SWIGLU);
   const size_t ws_bytes = dma_tile ? (dma_fold ? ((size_t)dma_split * m * rows * sizeof(float) + 255) & ~(size_t)255 : 0)
                                    : (gemm_tiled_workspace_bytes(dtype, p, 1, &epi) + 255) & ~(size_t)255;
@@ -679,10 +702,10 @@ static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x
   if (dma_tile) {
     if (dma_fold) {
       p.c = dev->gemm_ws;
-      UGHIP_HIPCHK(gemm_dma_launch_planes3(dev->stream, p, dma_tile, dma_split, nullptr, kind == GemmEpilogue::SWIGLU ? ",swiglu fold" : kind == GemmEpilogue::ADD ? ",+residual in the fold" : ",fold"));
+      UGHIP_HIPCHK(gemm_dma_launch_planes3(dev->stream, p, dma_tile, dma_split, nullptr, dma_planes_tail(kind, true, false)));
       UGHIP_HIPCHK(gemm_fold_f32(dev->stream, static_cast<const float*>(dev->gemm_ws), static_cast<float*>(dst->ptr), m, rows, dma_split, kind, epi.residual));
     } else {
-      UGHIP_HIPCHK(gemm_dma_launch_planes3(dev->stream, p, dma_tile, 1, epi.residual, epi.residual ? ",+residual" : ""));
+      UGHIP_HIPCHK(gemm_dma_launch_planes3(dev->stream, p, dma_tile, 1, epi.residual, dma_planes_tail(kind, false, epi.residual != nullptr)));
     }
     return UGHIP_OK;
   }
@@ -714,6 +737,46 @@ extern "C" int ughip_matmul_plan(int dtype, int rhs_dtype, size_t b, size_t m, s
     case ROUTE_DMA: gemm_dma_name(dtype, p, tile, buf, buf_len); break;
     case ROUTE_TILED: gemm_tiled_name(dtype, p, b, mixed, nullptr, buf, buf_len); break;
     default: snprintf(buf, buf_len, "gemm_any<%s>", tn); break;
+  }
+  return UGHIP_OK;
+}
+
+// The kernel ughip_linear_rows (form 0), ughip_linear_add_rows (1) or ughip_linear_swiglu_rows (2; n output columns from 2 n matrix
+// rows) would launch for m rows, by the name ughip_last_kernel() reports after the launch.  Needs no device (256 CUs assumed).
+extern "C" int ughip_linear_rows_plan(int w_dtype, int product, int form, size_t m, size_t n, size_t k, char* buf, size_t buf_len) {
+  if (!buf || !buf_len) return set_error(UGHIP_ERR_INVALID, "linear_rows_plan: no buffer");
+  if ((w_dtype != UGHIP_F32 && w_dtype != UGHIP_BF16) || (product != UGHIP_PRODUCT_F32 && product != UGHIP_PRODUCT_BF16X3) || form < 0 || form > 2 ||
+      (product == UGHIP_PRODUCT_BF16X3 && w_dtype != UGHIP_BF16))
+    return set_error(UGHIP_ERR_INVALID, "linear_rows_plan: bad dtype, product or form");
+  const size_t rows = form == 2 ? 2 * n : n;
+  if (!m || !n || !k || m > 0x7fffffffull || rows > 0x7fffffffull || k > 0x7fffffffull / 3) return set_error(UGHIP_ERR_INVALID, "linear_rows_plan: bad shape");
+  const GemmEpilogue::Kind kind = form == 2 ? GemmEpilogue::SWIGLU : form == 1 ? GemmEpilogue::ADD : GemmEpilogue::NONE;
+  const bool x3 = product == UGHIP_PRODUCT_BF16X3, mixed = !x3 && w_dtype == UGHIP_BF16;
+  const int dtype = x3 ? UGHIP_BF16 : UGHIP_F32;
+  void* stand_in = reinterpret_cast<void*>(uintptr_t(1) << 20);  // the alignment every allocation has; never dereferenced
+  MMArgs p;
+  p.M = (int)m, p.N = (int)rows, p.K = (int)(x3 ? 3 * k : k);
+  p.a_rs = (long long)(x3 ? 3 * k : k), p.a_cs = 1, p.b_rs = 1, p.b_cs = (long long)k;
+  p.a_bs = (long long)(m * (x3 ? 3 * k : k)), p.b_bs = (long long)(rows * k), p.c_bs = (long long)(m * rows);
+  p.a = p.b = stand_in, p.c = stand_in;
+  if (x3) p.b_k_div = 3;
+  const size_t min_rows = w_dtype == UGHIP_BF16 ? 2 : 9;
+  if (m < min_rows || rows % 8 != 0 || (kind == GemmEpilogue::SWIGLU && rows % 16 != 0) || (x3 && k % 64 != 0) || !gemm_tiled_supported(dtype, p, 1, mixed))
+    return set_error(UGHIP_ERR_UNSUPPORTED, "linear_rows_plan: a shape the entry points refuse (m %zu, n %zu, k %zu)", m, n, k);
+  GemmEpilogue epi{kind, form == 1 ? static_cast<const float*>(stand_in) : nullptr};
+  epi.out_f32 = x3;
+  const RowsRoute route = rows_route(p, dtype, x3, kind, stand_in, stand_in, stand_in, form == 1 ? stand_in : nullptr, m, rows, k, 256);
+  if (route.kind == RowsRoute::X3_ROWS) {
+    rows_x3_name(route.x3, kind, buf, buf_len);
+  } else if (route.kind == RowsRoute::DMA_PLANES) {
+    const bool fold = route.dma_split > 1 || kind == GemmEpilogue::SWIGLU;
+    int bm = 256, bn = route.dma_tile == 256 ? 256 : 128;
+    if (route.dma_tile == 64) bm = 128;
+    char split[24] = "";
+    if (route.dma_split > 1) snprintf(split, sizeof split, ",splitK=%d", route.dma_split);
+    snprintf(buf, buf_len, "gemm_dma4<bf16,NT,%dx%d,256t,3 planes%s,f32 out%s>", bm, bn, split, dma_planes_tail(kind, fold, form == 1));
+  } else {
+    gemm_tiled_name(dtype, p, 1, mixed, &epi, buf, buf_len);
   }
   return UGHIP_OK;
 }
