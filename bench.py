@@ -631,7 +631,9 @@ def bmm(dev, steps, warmup):
     out["mm_bf16_nt_8192^3"] = {"TFLOP/s": round(tf, 2), "frac_mfma_bf16": round(tf / MFMA_BF16_PEAK_TF, 4), "us": round(ms * 1e3 / 20, 1), "kernel": kernel, "verified": chk}
     del sa, sw, dst
     # The products of a 128-token prompt (f32 rows against bf16 matrices stored [n, k]): the f32 matrix pipe on the widened
-    # matrix against three bf16 terms per row element on the bf16 pipe.  TFLOP/s counts 2 m n k either way.
+    # matrix against three bf16 terms per row element on the bf16 pipe.  TFLOP/s counts 2 m n k either way.  The same matrix
+    # every step: up to 131 MB that stay in the 256 MB memory-side cache; inside a model every layer's matrices come from HBM
+    # and the same kernels take 1-2 us longer (the llama rows' prefill_ms_warm has that).
     t = 128
     for label, n, k in (("qkv", 2560, 2048), ("gate_up", 11264, 2048), ("down", 2048, 5632), ("head", 32000, 2048)):
         xh = rng.normal(21, t * k)

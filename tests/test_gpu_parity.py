@@ -1713,7 +1713,7 @@ def test_three_bf16_terms_split_inside_the_product(hip, tune, t, k, n, units):
     if units:
         tune.setenv("UGHIP_X3_ROWS", units)
     (lin, add, glu), kerns = run(x, w, wgu)
-    for kn, word in zip(kerns, (",fold>", "+residual in the fold", "swiglu fold")):
+    for kn, word in zip(kerns, ("fold>", "+residual in the fold", "swiglu fold")):   # ("no fold" where every tile has one slab: it is the result)
         assert kn.startswith("rows_x3<128x128,3 terms split in the kernel,") and word in kn, kn
     if units and -(-n // 128) * (k // 64) <= 256 * int(units):
         assert f",{units} units x " in kerns[0], kerns[0]

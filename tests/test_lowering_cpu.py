@@ -293,9 +293,9 @@ def test_kernel_choice_for_the_rows_of_a_prompt_is_pinned():
         (B, X3, 1, 128, 2048, 2048): "rows_x3<128x128,3 terms split in the kernel,4 units x 128 workgroups,8 slabs,+residual in the fold>",
         (B, X3, 2, 128, 5632, 2048): "rows_x3<128x128,3 terms split in the kernel,12 units x 235 workgroups,4 slabs,swiglu fold>",
         (B, X3, 1, 128, 2048, 5632): "rows_x3<128x128,3 terms split in the kernel,8 units x 176 workgroups,11 slabs,+residual in the fold>",
-        (B, X3, 0, 128, 32000, 2048): "rows_x3<128x128,3 terms split in the kernel,32 units x 250 workgroups,1 slabs,fold>",
+        (B, X3, 0, 128, 32000, 2048): "rows_x3<128x128,3 terms split in the kernel,32 units x 250 workgroups,1 slabs,no fold>",
         (B, X3, 0, 33, 2560, 2048): "rows_x3<128x128,3 terms split in the kernel,4 units x 160 workgroups,8 slabs,fold>",
-        (B, X3, 0, 77, 8, 64): "rows_x3<128x128,3 terms split in the kernel,1 units x 1 workgroups,1 slabs,fold>",
+        (B, X3, 0, 77, 8, 64): "rows_x3<128x128,3 terms split in the kernel,1 units x 1 workgroups,1 slabs,no fold>",
     }
     got = {key: _rows_plan(*key) for key in want}
     assert got == want

@@ -1202,7 +1202,7 @@ std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32
   };
   auto build = [&](PreparedStep& st, const LB& pos) {
     auto t0 = clock::now();
-    st.logits = model.fwd(st.tokens, pos, cache);
+    st.logits = model.fwd(st.tokens, pos, cache, nullptr, true);  // read at the last position only, like the queued loop
     auto t1 = clock::now();
     Schedule schedule = Schedule::create_one(st.logits);
     auto t2 = clock::now();
@@ -1272,7 +1272,7 @@ std::vector<int32_t> generate_greedy(const Model& model, const std::vector<int32
     logits.resize(cur.logits.elem_count());
     cur.logits.data_vec(logits.data(), DType::F32);
     auto t3 = clock::now();
-    const float* last = logits.data() + (cur.t - 1) * cfg.vocab_size;
+    const float* last = logits.data() + (cur.logits.elem_count() / cfg.vocab_size - 1) * cfg.vocab_size;
     size_t best = 0;
     float second = -INFINITY;
     for (size_t i = 1; i < cfg.vocab_size; ++i) {

@@ -344,7 +344,7 @@ RowsX3Plan rows_x3_plan(size_t m, size_t n, size_t k, int forced_units, int num_
 
 void rows_x3_name(const RowsX3Plan& pl, GemmEpilogue::Kind kind, char* out, size_t out_len) {
   snprintf(out, out_len, "rows_x3<128x128,3 terms split in the kernel,%d units x %d workgroups,%d slabs%s>", pl.units, pl.groups, pl.max_slabs,
-           kind == GemmEpilogue::SWIGLU ? ",swiglu fold" : kind == GemmEpilogue::ADD ? ",+residual in the fold" : ",fold");
+           kind == GemmEpilogue::SWIGLU ? ",swiglu fold" : kind == GemmEpilogue::ADD ? ",+residual in the fold" : pl.max_slabs == 1 ? ",no fold" : ",fold");
 }
 
 hipError_t rows_x3_launch(hipStream_t stream, const float* x, const void* w, float* ws, float* c, size_t m, size_t n, size_t k, const RowsX3Plan& pl, GemmEpilogue::Kind kind,
@@ -358,8 +358,16 @@ hipError_t rows_x3_launch(hipStream_t stream, const float* x, const void* w, flo
     configured.fetch_or(bit, std::memory_order_relaxed);
   }
   const int KT = (int)(k / 64), tiles = (int)((n + BN - 1) / BN), total = tiles * KT;
-  rows_x3_kernel<<<dim3((unsigned)pl.groups), dim3(512), LDS_TOTAL, stream>>>(x, static_cast<const uint16_t*>(w), ws, (int)m, (int)n, (int)k, KT, pl.units, total);
+  // one slab per tile and nothing for the fold to do: the slab is the result
+  const bool direct = pl.max_slabs == 1 && kind == GemmEpilogue::NONE;
+  rows_x3_kernel<<<dim3((unsigned)pl.groups), dim3(512), LDS_TOTAL, stream>>>(x, static_cast<const uint16_t*>(w), direct ? c : ws, (int)m, (int)n, (int)k, KT, pl.units, total);
   if (hipError_t e = hipGetLastError()) return e;
+  if (direct) {
+    char name[160];
+    rows_x3_name(pl, kind, name, sizeof name);
+    note_kernel("%s", name);
+    return hipSuccess;
+  }
   const size_t groups4 = kind == GemmEpilogue::SWIGLU ? m * n / 8 : m * n / 4;
   const dim3 grid((unsigned)((groups4 + 255) / 256));
   if (kind == GemmEpilogue::ADD)
