@@ -308,8 +308,9 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 }  // namespace
 
 bool rows_x3_supported(const void* x, const void* w, const void* c, const void* residual, size_t m, size_t n, size_t k) {
-  return m >= 1 && m <= (size_t)BM && n >= 8 && n % 8 == 0 && k >= 64 && k % 64 == 0 && k <= (1u << 20) && n <= (1u << 24) && aligned16(x) && aligned16(w) && aligned16(c) &&
-         aligned16(residual);
+  // (the unit count and the byte offsets inside one column tile's rows are held in 32 bits)
+  return m >= 1 && m <= (size_t)BM && n >= 8 && n % 8 == 0 && k >= 64 && k % 64 == 0 && k <= (1u << 20) && n <= (1u << 24) && n * k <= (1ull << 31) && aligned16(x) &&
+         aligned16(w) && aligned16(c) && aligned16(residual);
 }
 
 // Units per workgroup: every CU busy in one round, and past that as few slabs as the units' time allows -- a unit costs a
