@@ -1185,6 +1185,47 @@ def test_attention_cached(hip, cpu, hip_ops, cpu_ops, interleaved, b, nh, nkv, t
         assert np.all(np.abs(got - want) <= 2 * tol), float(np.abs(got - want).max())
 
 
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("b,nh,nkv,t,s,cap,with_rope", [
+    (1, 8, 2, 33, 33, 33, True),           # ragged last block, cache exactly full
+    (1, 4, 4, 200, 200, 512, False),
+    (1, 8, 2, 2, 2, 16, True),             # two positions
+    (1, 8, 2, 40, 100, 128, True),         # 40 new positions after 60 cached ones
+    (2, 8, 4, 70, 131, 200, True),         # two sequences, keys end inside a block
+    (1, 32, 4, 512, 512, 600, True),       # paired query blocks (two per workgroup)
+    (1, 16, 4, 300, 1000, 1000, True),     # an odd count of paired query blocks behind 700 cached keys
+])
+def test_attention_cached_six_bf16_terms(hip, hip_ops, tune, interleaved, b, nh, nkv, t, s, cap, with_rope):
+    """Head size 64 with both products as six bf16 terms on planes of K and V (the path prompts of 256 positions and up
+    take; UGHIP_ATT_X6=1 forces it for any count): held to float64 with the same bound as the f32 products, and to the f32
+    kernel's result, from which it may differ by roundings only."""
+    d = 64
+    q = rng.normal(83, b * t * nh * d)
+    k4, v4 = rng.normal(84, b * nkv * cap * d).reshape(b, nkv, cap, d).copy(), rng.normal(85, b * nkv * cap * d).reshape(b, nkv, cap, d).copy()
+    k4[:, :, s:], v4[:, :, s:] = np.nan, np.inf    # rows past s must not matter
+    scale = float(np.float32(d) ** np.float32(-0.5))
+    pos0 = s - t
+    args = [LB.copy(q, (b, t, nh * d), hip), LB.copy(k4.ravel(), (b, nkv, cap, d), hip), LB.copy(v4.ravel(), (b, nkv, cap, d), hip), s, scale]
+    if with_rope:
+        cos, sin = _rope_tables(hip, d, max_pos=s + 8)
+        args += [cos, sin, LB.copy(np.array([pos0], np.int32), (1, 1), hip), interleaved]
+    got = {}
+    for x6 in (0, 1):
+        tune.setenv("UGHIP_ATT_X6", str(x6))
+        print("attention cached, six bf16 terms", x6, (b, nh, nkv, t, s, cap, with_rope, interleaved), flush=True)
+        got[x6] = hip_ops.attention_cached(*args).data_vec().reshape(b, t, nh, d)
+    q6 = q.reshape(b, t, nh, d).astype(np.float64)
+    if with_rope:
+        q6 = _rope_rows_f64(q6, cos.data_vec(), sin.data_vec(), pos0, interleaved)
+    truth = _attention_truth(q6.transpose(0, 2, 1, 3), k4[:, :, :s].astype(np.float64), v4[:, :, :s].astype(np.float64), s, t, scale, nh // nkv).transpose(0, 2, 1, 3)
+    tol = 2e-5 * np.abs(truth).max() + 2e-5 * np.abs(truth)
+    assert np.all(np.abs(got[1] - truth) <= tol), float(np.abs(got[1] - truth).max())
+    assert np.all(np.abs(got[1] - got[0]) <= 0.2 * tol), float(np.abs(got[1] - got[0]).max())
+    # what the split drops is the size of an f32 rounding: the error against float64 stays in the f32 kernel's class
+    e0, e1 = float(np.abs(got[0] - truth).max()), float(np.abs(got[1] - truth).max())
+    assert e1 <= 4 * e0 + 1e-7 * float(np.abs(truth).max()), (e0, e1)
+
+
 def test_attention_cached_random_shapes(hip, hip_ops):
     """Seeded random shapes (one or a few query positions, caches of up to 3500 rows with spare rows behind them, 1-8 kv
     heads with 1-8 query heads each, every built head size, with and without either rope, cache lengths at the thresholds

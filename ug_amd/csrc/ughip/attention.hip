@@ -694,6 +694,311 @@ __global__ void __launch_bounds__(256 * GROUPS) attention_prefill_kernel(const f
   }
 }
 
+// ---- the same with both products as six bf16 terms ------------------------------------------------
+// On this chip an f32 MFMA runs on the vector ALU's own datapath: while one executes, no wave of that SIMD issues a
+// vector instruction (measured: one wave, v_mfma_f32_32x32x2_f32 + 8 independent v_fma: 113 cycles against 64 + 42 apart;
+// with the v_fma in a second wave of the SIMD the same; v_mfma_f32_32x32x16_bf16 + 8 v_fma: 45 against 32 + 42).  The
+// kernel above therefore pays for its softmax, masks and staging on top of its 4096 MFMA cycles per block of 32 x 32
+// scores, whatever the schedule.  Here the operands are split into three bf16 terms each (x = hi + mid + lo to 2^-25 |x|)
+// and a product is the six term pairs whose weight is 2^-16 and up -- (hi, lo), (lo, hi), (mid, mid), (hi, mid),
+// (mid, hi), (hi, hi), smallest first, every one accumulated in f32 by v_mfma_f32_32x32x16_bf16: 1536 MFMA cycles per
+// block on the matrix cores proper, beside the vector instructions instead of in front of them.  What is dropped is
+// 3 x 2^-24 |x| |y| per element, the size of the f32 product's own rounding.
+//
+// K and V come as planes written by a pass in front (att_planes_kernel), in operand order: per kv head and block of 32
+// keys 24 KiB = [K: plane p][k step ks][lane] 16 bytes, then [V: plane p][d block e][key step st][lane] 16 bytes, so
+// that an operand is one coalesced 128-bit load straight into the registers the MFMA reads: no LDS in the loop.
+//   K operand (p, ks), lane l: K[key = l % 32][16 ks + 8 (l / 32) + 0..7]
+//   V operand (p, e, st), lane l: V[key = 16 st + 8 (i / 4) + 4 (l / 32) + i % 4][d = 32 e + l % 32], i = 0..7 -- the keys that
+//       registers 8 st .. 8 st + 7 of a lane's score accumulator hold, so the exponentials feed back as the other operand
+//       from where they are (as in the kernel above).
+// Keys past s are planes of zeros.
+typedef __bf16 att_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 att_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float att_f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned att_u32x4 __attribute__((ext_vector_type(4)));
+constexpr int ATT_PLANE_BLOCK = 1536;  // 16-byte units per block of 32 keys: 2 x 3 planes x 4 operands x 64 lanes
+
+// (x0, x1) -> three words of two bf16 each (x0 in the low half); remainders are exact f32 subtractions.  An infinity or a
+// NaN stays whole in the first term.
+__device__ __forceinline__ void att_split_pair(float x0, float x1, unsigned& hi, unsigned& mid, unsigned& lo) {
+  const unsigned h = __builtin_bit_cast(unsigned, __builtin_convertvector(att_f32x2{x0, x1}, att_bf16x2));
+  float r0 = x0 - __uint_as_float(h << 16), r1 = x1 - __uint_as_float(h & 0xffff0000u);
+  if ((h & 0x7f80u) == 0x7f80u) r0 = 0.f;
+  if ((h & 0x7f800000u) == 0x7f800000u) r1 = 0.f;
+  const unsigned m = __builtin_bit_cast(unsigned, __builtin_convertvector(att_f32x2{r0, r1}, att_bf16x2));
+  const float q0 = r0 - __uint_as_float(m << 16), q1 = r1 - __uint_as_float(m & 0xffff0000u);
+  hi = h, mid = m, lo = __builtin_bit_cast(unsigned, __builtin_convertvector(att_f32x2{q0, q1}, att_bf16x2));
+}
+// eight values -> one operand per plane
+__device__ __forceinline__ void att_split8(const float (&x)[8], att_u32x4& hi, att_u32x4& mid, att_u32x4& lo) {
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    unsigned h, md, l;
+    att_split_pair(x[2 * m], x[2 * m + 1], h, md, l);
+    hi[m] = h, mid[m] = md, lo[m] = l;
+  }
+}
+
+// k, v: [bh, cap, 64] with rows 0 .. s-1 valid; planes: [bh][ceil(s / 32)][ATT_PLANE_BLOCK] 16-byte units.
+// Grid (blocks of 32 keys, bh), 256 threads: thread u writes K operand (ks = u / 64, lane u % 64) and V operand
+// (e = u / 128, st = u / 64 % 2, lane u % 64) of all three planes.
+__global__ void __launch_bounds__(256) att_planes_kernel(const float* __restrict__ k, const float* __restrict__ v, att_u32x4* __restrict__ planes, int s, size_t cap) {
+  const int u = threadIdx.x, l = u & 63, col = l & 31, hh = l >> 5, kb = blockIdx.x;
+  const size_t bh = blockIdx.y;
+  const float* kbase = k + bh * cap * 64;
+  const float* vbase = v + bh * cap * 64;
+  att_u32x4* out = planes + (bh * gridDim.x + kb) * ATT_PLANE_BLOCK;
+  float x[8];
+  att_u32x4 hi, mid, lo;
+  {
+    const int ks = u >> 6, key = kb * 32 + col;
+    if (key < s) {
+      const float4 a = *reinterpret_cast<const float4*>(kbase + (size_t)key * 64 + ks * 16 + hh * 8);
+      const float4 b = *reinterpret_cast<const float4*>(kbase + (size_t)key * 64 + ks * 16 + hh * 8 + 4);
+      x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w, x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = 0.f;
+    }
+    att_split8(x, hi, mid, lo);
+    out[(0 * 4 + ks) * 64 + l] = hi;
+    out[(1 * 4 + ks) * 64 + l] = mid;
+    out[(2 * 4 + ks) * 64 + l] = lo;
+  }
+  {
+    const int e = u >> 7, st = (u >> 6) & 1, d = e * 32 + col;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int key = kb * 32 + st * 16 + (i >> 2) * 8 + hh * 4 + (i & 3);
+      x[i] = key < s ? vbase[(size_t)key * 64 + d] : 0.f;
+    }
+    att_split8(x, hi, mid, lo);
+    att_u32x4* vo = out + 768;
+    vo[((0 * 2 + e) * 2 + st) * 64 + l] = hi;
+    vo[((1 * 2 + e) * 2 + st) * 64 + l] = mid;
+    vo[((2 * 2 + e) * 2 + st) * 64 + l] = lo;
+  }
+}
+
+__device__ __forceinline__ att_f32x16 att_mma_bf16(const att_u32x4& a, const att_u32x4& b, const att_f32x16& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(att_bf16x8, a), __builtin_bit_cast(att_bf16x8, b), c, 0, 0, 0);
+}
+
+// Same work split, statistics, merge and output as attention_prefill_kernel<64, GROUPS>; q is scaled before it is split
+// (scores come out of the MFMAs scaled).  planes: what att_planes_kernel wrote for these caches, n_kb blocks per kv head.
+template <int GROUPS>
+__global__ void __launch_bounds__(256 * GROUPS, 2) attention_prefill_x6_kernel(const float* __restrict__ q, const att_u32x4* __restrict__ planes, float* __restrict__ dst,
+                                                                               int nh, int nkv, int t, int s, int n_kb, size_t q_row_stride, float scale,
+                                                                               const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                                               const int* __restrict__ pos, size_t table_len, int interleaved) {
+  constexpr int D = 64, H = D / 2, DB = D / 32;
+  __shared__ float merge_ml_all[GROUPS][3][2][64];
+  __shared__ float merge_o_all[GROUPS][3][DB * 16][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = (tid >> 6) & 3, group = tid >> 8;
+  const int col = lane & 31, hh = lane >> 5;
+  const int bh = blockIdx.y, b = bh / nh, head = bh % nh, kvh = head / (nh / nkv);
+  const int n_qb = (t + 31) / 32;
+  const int qb = GROUPS == 1 ? n_qb - 1 - (int)blockIdx.x : (group == 0 ? n_qb - 1 - (int)blockIdx.x : (int)blockIdx.x);
+  const bool idle = GROUPS == 2 && group == 1 && qb == n_qb - 1 - qb;
+  float (*merge_ml)[2][64] = merge_ml_all[group];
+  float (*merge_o)[64] = merge_o_all[group][0];
+  const int q0 = qb * 32;
+  const int qi = min(q0 + col, t - 1);
+  const int q_pos = s - t + qi;
+  const int last_pos = s - t + min(q0 + 31, t - 1);
+  const int q_pos_min = s - t + min(q0, t - 1);
+  const att_u32x4* pl = planes + ((size_t)b * nkv + kvh) * (size_t)n_kb * ATT_PLANE_BLOCK + lane;
+  const int n_blocks = idle ? 0 : last_pos / 32 + 1;
+
+  // K operands of this wave's first block set out before the query row is touched
+  att_u32x4 kop[3][4], vop[3][DB][2];
+  auto load_k = [&](int kb) {
+    const att_u32x4* base = pl + (size_t)min(kb, n_kb - 1) * ATT_PLANE_BLOCK;
+#pragma unroll
+    for (int p = 0; p < 3; ++p)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) kop[p][ks] = base[(p * 4 + ks) * 64];
+  };
+  auto load_v = [&](int kb) {
+    const att_u32x4* base = pl + (size_t)min(kb, n_kb - 1) * ATT_PLANE_BLOCK + 768;
+#pragma unroll
+    for (int p = 0; p < 3; ++p)
+#pragma unroll
+      for (int e = 0; e < DB; ++e)
+#pragma unroll
+        for (int st = 0; st < 2; ++st) vop[p][e][st] = base[((p * 2 + e) * 2 + st) * 64];
+  };
+  load_k(wave);
+
+  // this lane's 32 elements of its (rotated, scaled) query row: chunk ks holds columns 16 ks + 8 hh .. + 7
+  att_u32x4 qop[3][4];
+  {
+    float qr[4][8];
+    const float* qrow = q + ((size_t)b * t + qi) * q_row_stride + (size_t)head * D;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const float4 a = *reinterpret_cast<const float4*>(qrow + ks * 16 + hh * 8);
+      const float4 c = *reinterpret_cast<const float4*>(qrow + ks * 16 + hh * 8 + 4);
+      qr[ks][0] = a.x, qr[ks][1] = a.y, qr[ks][2] = a.z, qr[ks][3] = a.w, qr[ks][4] = c.x, qr[ks][5] = c.y, qr[ks][6] = c.z, qr[ks][7] = c.w;
+    }
+    if (cos_t) {
+      const long long p = (long long)pos[0] + qi;
+      const bool ok = p >= 0 && (size_t)(p + 1) * H <= table_len;
+      const size_t row = ok ? (size_t)p * H : 0;
+      if (interleaved) {
+        // pairs (2 i, 2 i + 1) with table entry i: chunk ks holds pairs 8 ks + 4 hh .. + 3
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          const float4 c = *reinterpret_cast<const float4*>(cos_t + row + ks * 8 + hh * 4);
+          const float4 sn = *reinterpret_cast<const float4*>(sin_t + row + ks * 8 + hh * 4);
+          const float cs[4] = {c.x, c.y, c.z, c.w}, ss[4] = {sn.x, sn.y, sn.z, sn.w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float x1 = qr[ks][2 * i], x2 = qr[ks][2 * i + 1];
+            qr[ks][2 * i] = x1 * cs[i] - x2 * ss[i];
+            qr[ks][2 * i + 1] = x1 * ss[i] + x2 * cs[i];
+          }
+        }
+      } else {
+        // pairs (i, i + 32) with table entry i: chunks ks and ks + 2 hold the two halves of pairs 16 ks + 8 hh .. + 7
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+          const float4 c0 = *reinterpret_cast<const float4*>(cos_t + row + ks * 16 + hh * 8);
+          const float4 c1 = *reinterpret_cast<const float4*>(cos_t + row + ks * 16 + hh * 8 + 4);
+          const float4 s0 = *reinterpret_cast<const float4*>(sin_t + row + ks * 16 + hh * 8);
+          const float4 s1 = *reinterpret_cast<const float4*>(sin_t + row + ks * 16 + hh * 8 + 4);
+          const float cs[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w}, ss[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float x1 = qr[ks][i], x2 = qr[ks + 2][i];
+            qr[ks][i] = x1 * cs[i] - x2 * ss[i];
+            qr[ks + 2][i] = x1 * ss[i] + x2 * cs[i];
+          }
+        }
+      }
+      if (!ok) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) qr[ks][i] = NAN;
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) qr[ks][i] *= scale;
+      att_split8(qr[ks], qop[0][ks], qop[1][ks], qop[2][ks]);
+    }
+  }
+
+  float m_run = ATT_MASKED, l_half = 0.f;
+  att_f32x16 o[DB];
+#pragma unroll
+  for (int e = 0; e < DB; ++e)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[e][r] = 0.f;
+
+  // term pairs (plane of the first operand, plane of the second), smallest first
+  constexpr int TA[6] = {0, 2, 1, 0, 1, 0}, TB[6] = {2, 0, 1, 1, 0, 0};
+  for (int kb = wave; kb < n_blocks; kb += 4) {
+    const int key0 = kb * 32;
+    load_v(kb);
+    att_f32x16 sc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+#pragma unroll
+    for (int term = 0; term < 6; ++term)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) sc = att_mma_bf16(kop[TA[term]][ks], qop[TB[term]][ks], sc);
+    __builtin_amdgcn_sched_barrier(0);
+    load_k(kb + 4);  // into the registers the MFMAs above have read
+    float mx = ATT_MASKED;
+    if (key0 + 31 > q_pos_min) {  // wave-uniform: only blocks that touch the diagonal have anything to mask
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = key0 + (r >> 2) * 8 + hh * 4 + (r & 3);
+        sc[r] = key <= q_pos ? sc[r] : ATT_MASKED;
+        mx = fmaxf(mx, sc[r]);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sc[r]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = m_new <= ATT_MASKED ? 0.f : m_new;
+    const float alpha = att_exp(m_run - m_use);
+    m_run = m_new;
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      sc[r] = att_exp(sc[r] - m_use);
+      psum += sc[r];
+    }
+    l_half = l_half * alpha + psum;
+    // the exponentials as operands: registers 8 st .. 8 st + 7 are key step st
+    att_u32x4 pop[3][2];
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const float x[8] = {sc[st * 8], sc[st * 8 + 1], sc[st * 8 + 2], sc[st * 8 + 3], sc[st * 8 + 4], sc[st * 8 + 5], sc[st * 8 + 6], sc[st * 8 + 7]};
+      att_split8(x, pop[0][st], pop[1][st], pop[2][st]);
+    }
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int e = 0; e < DB; ++e)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[e][r] *= alpha;
+    }
+#pragma unroll
+    for (int term = 0; term < 6; ++term)
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int e = 0; e < DB; ++e) o[e] = att_mma_bf16(vop[TA[term]][e][st], pop[TB[term]][st], o[e]);
+  }
+
+  // merge the four waves' partial results in wave order
+  if (wave != 0) {
+    merge_ml[wave - 1][0][lane] = m_run;
+    merge_ml[wave - 1][1][lane] = l_half;
+#pragma unroll
+    for (int e = 0; e < DB; ++e)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) merge_o[(wave - 1) * DB * 16 + e * 16 + r][lane] = o[e][r];
+  }
+  __syncthreads();
+  if (wave != 0 || idle) return;
+  float m_tot = m_run;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) m_tot = fmaxf(m_tot, merge_ml[w][0][lane]);
+  float f = att_exp(m_run - m_tot);
+  float l_tot = l_half * f;
+#pragma unroll
+  for (int e = 0; e < DB; ++e)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[e][r] *= f;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+    f = att_exp(merge_ml[w][0][lane] - m_tot);
+    l_tot += merge_ml[w][1][lane] * f;
+#pragma unroll
+    for (int e = 0; e < DB; ++e)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[e][r] += merge_o[w * DB * 16 + e * 16 + r][lane] * f;
+  }
+  l_tot += __shfl_xor(l_tot, 32, 64);
+  if (q0 + col < t) {
+    float* orow = dst + ((size_t)b * t + qi) * ((size_t)nh * D) + (size_t)head * D;
+#pragma unroll
+    for (int e = 0; e < DB; ++e)
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+        *reinterpret_cast<float4*>(orow + e * 32 + a * 8 + hh * 4) =
+            make_float4(o[e][a * 4] / l_tot, o[e][a * 4 + 1] / l_tot, o[e][a * 4 + 2] / l_tot, o[e][a * 4 + 3] / l_tot);
+  }
+}
+
 int check_f32(const ughip_slice* s, size_t need, const char* what) {
   if (!s) return set_error(UGHIP_ERR_INVALID, "%s: null slice", what);
   if (s->dtype != UGHIP_F32) return set_error(UGHIP_ERR_INVALID, "%s: unexpected dtype %s, expected F32", what, dtype_name(s->dtype));
@@ -992,6 +1297,24 @@ int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_off
     if (err != hipSuccess) return;
     kernel<<<grid, 256 * groups, lds, dev->stream>>>(qp, kp, vp, op, inh, inkv, it, is, cap, q_row_stride, scale, cp, sp, pp, tl, interleaved);
   };
+  // Head size 64 and enough positions to pay for the pass that writes the planes: both products as six bf16 terms
+  // (UGHIP_ATT_X6: 0 never, 1 for any t > 1).
+  bool x6 = d == 64 && t >= 256;
+  if (long long v; tune_get(TUNE_ATT_X6, &v)) x6 = d == 64 && v != 0;
+  if (x6) {
+    const size_t n_kb = (s + 31) / 32, bkv = b * n_kv_heads;
+    float* ws = nullptr;
+    if (int rc = decode_scratch(dev, bkv * n_kb * ATT_PLANE_BLOCK * sizeof(att_u32x4), &ws)) return rc;
+    att_u32x4* planes = reinterpret_cast<att_u32x4*>(ws);
+    att_planes_kernel<<<dim3((unsigned)n_kb, (unsigned)bkv), 256, 0, dev->stream>>>(kp, vp, planes, is, cap);
+    UGHIP_HIPCHK(hipGetLastError());
+    if (pair)
+      attention_prefill_x6_kernel<2><<<paired, 512, 0, dev->stream>>>(qp, planes, op, inh, inkv, it, is, (int)n_kb, q_row_stride, scale, cp, sp, pp, tl, interleaved);
+    else
+      attention_prefill_x6_kernel<1><<<single, 256, 0, dev->stream>>>(qp, planes, op, inh, inkv, it, is, (int)n_kb, q_row_stride, scale, cp, sp, pp, tl, interleaved);
+    UGHIP_HIPCHK(hipGetLastError());
+    return UGHIP_OK;
+  }
   if (d == 32 && pair) go(attention_prefill_kernel<32, 2>, 32, 2, paired);
   else if (d == 32) go(attention_prefill_kernel<32, 1>, 32, 1, single);
   else if (d == 64 && pair) go(attention_prefill_kernel<64, 2>, 64, 2, paired);

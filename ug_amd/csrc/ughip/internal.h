@@ -77,6 +77,7 @@ enum TuneKey {
   TUNE_GRID_REDUCE_THREADS, // threads per workgroup there: 64, 128, 256, 512 or 1024
   TUNE_NO_NT_STORES,        // (set at all) generated elementwise kernels store through the cache
   TUNE_SOFTMAX_STREAM,      // ughip_softmax_rows: 0 never takes the resident wave-per-row kernel, n > 0 forces it onto n workgroups
+  TUNE_ATT_X6,              // attention over several query positions, head size 64: 0 keeps the f32 products, 1 takes six bf16 terms for any count
   TUNE_COUNT
 };
 bool tune_get(TuneKey k, long long* value);  // false: the switch is not set
