@@ -720,22 +720,27 @@ typedef unsigned att_u32x4 __attribute__((ext_vector_type(4)));
 constexpr int ATT_PLANE_BLOCK = 1536;  // 16-byte units per block of 32 keys: 2 x 3 planes x 4 operands x 64 lanes
 
 // (x0, x1) -> three words of two bf16 each (x0 in the low half); remainders are exact f32 subtractions.  An infinity or a
-// NaN stays whole in the first term.
+// NaN stays whole in the first term (FINITE: the caller knows there is no infinity, e.g. among the exponentials of a softmax;
+// a NaN then gives three NaNs).
+template <bool FINITE = false>
 __device__ __forceinline__ void att_split_pair(float x0, float x1, unsigned& hi, unsigned& mid, unsigned& lo) {
   const unsigned h = __builtin_bit_cast(unsigned, __builtin_convertvector(att_f32x2{x0, x1}, att_bf16x2));
   float r0 = x0 - __uint_as_float(h << 16), r1 = x1 - __uint_as_float(h & 0xffff0000u);
-  if ((h & 0x7f80u) == 0x7f80u) r0 = 0.f;
-  if ((h & 0x7f800000u) == 0x7f800000u) r1 = 0.f;
+  if (!FINITE) {
+    if ((h & 0x7f80u) == 0x7f80u) r0 = 0.f;
+    if ((h & 0x7f800000u) == 0x7f800000u) r1 = 0.f;
+  }
   const unsigned m = __builtin_bit_cast(unsigned, __builtin_convertvector(att_f32x2{r0, r1}, att_bf16x2));
   const float q0 = r0 - __uint_as_float(m << 16), q1 = r1 - __uint_as_float(m & 0xffff0000u);
   hi = h, mid = m, lo = __builtin_bit_cast(unsigned, __builtin_convertvector(att_f32x2{q0, q1}, att_bf16x2));
 }
 // eight values -> one operand per plane
+template <bool FINITE = false>
 __device__ __forceinline__ void att_split8(const float (&x)[8], att_u32x4& hi, att_u32x4& mid, att_u32x4& lo) {
 #pragma unroll
   for (int m = 0; m < 4; ++m) {
     unsigned h, md, l;
-    att_split_pair(x[2 * m], x[2 * m + 1], h, md, l);
+    att_split_pair<FINITE>(x[2 * m], x[2 * m + 1], h, md, l);
     hi[m] = h, mid[m] = md, lo[m] = l;
   }
 }
@@ -786,7 +791,7 @@ __device__ __forceinline__ att_f32x16 att_mma_bf16(const att_u32x4& a, const att
 }
 
 // Same work split, statistics, merge and output as attention_prefill_kernel<64, GROUPS>; q is scaled before it is split
-// (scores come out of the MFMAs scaled).  planes: what att_planes_kernel wrote for these caches, n_kb blocks per kv head.
+// (scores come out of the MFMAs scaled, and in units of log 2).  planes: what att_planes_kernel wrote for these caches, n_kb blocks per kv head.
 template <int GROUPS>
 __global__ void __launch_bounds__(256 * GROUPS, 2) attention_prefill_x6_kernel(const float* __restrict__ q, const att_u32x4* __restrict__ planes, float* __restrict__ dst,
                                                                                int nh, int nkv, int t, int s, int n_kb, size_t q_row_stride, float scale,
@@ -831,7 +836,11 @@ __global__ void __launch_bounds__(256 * GROUPS, 2) attention_prefill_x6_kernel(c
   };
   load_k(wave);
 
-  // this lane's 32 elements of its (rotated, scaled) query row: chunk ks holds columns 16 ks + 8 hh .. + 7
+  // this lane's 32 elements of its (rotated, scaled) query row: chunk ks holds columns 16 ks + 8 hh .. + 7.  The scale
+  // carries log2(e) as well: scores, running maxima and their differences are in units of log 2, an exponential is one
+  // v_exp_f32 (2^x, within an ulp) instead of the seven instructions of att_exp -- this loop is bound by its vector
+  // instructions, not by its MFMAs.
+  const float scale_log2e = scale * 1.44269504088896340736f;
   att_u32x4 qop[3][4];
   {
     float qr[4][8];
@@ -887,7 +896,7 @@ __global__ void __launch_bounds__(256 * GROUPS, 2) attention_prefill_x6_kernel(c
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) qr[ks][i] *= scale;
+      for (int i = 0; i < 8; ++i) qr[ks][i] *= scale_log2e;
       att_split8(qr[ks], qop[0][ks], qop[1][ks], qop[2][ks]);
     }
   }
@@ -928,12 +937,12 @@ __global__ void __launch_bounds__(256 * GROUPS, 2) attention_prefill_x6_kernel(c
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m_run, mx);
     const float m_use = m_new <= ATT_MASKED ? 0.f : m_new;
-    const float alpha = att_exp(m_run - m_use);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
     m_run = m_new;
     float psum = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      sc[r] = att_exp(sc[r] - m_use);
+      sc[r] = __builtin_amdgcn_exp2f(sc[r] - m_use);
       psum += sc[r];
     }
     l_half = l_half * alpha + psum;
@@ -942,7 +951,7 @@ __global__ void __launch_bounds__(256 * GROUPS, 2) attention_prefill_x6_kernel(c
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
       const float x[8] = {sc[st * 8], sc[st * 8 + 1], sc[st * 8 + 2], sc[st * 8 + 3], sc[st * 8 + 4], sc[st * 8 + 5], sc[st * 8 + 6], sc[st * 8 + 7]};
-      att_split8(x, pop[0][st], pop[1][st], pop[2][st]);
+      att_split8<true>(x, pop[0][st], pop[1][st], pop[2][st]);
     }
     if (__any(alpha != 1.f)) {
 #pragma unroll
@@ -972,7 +981,7 @@ __global__ void __launch_bounds__(256 * GROUPS, 2) attention_prefill_x6_kernel(c
   float m_tot = m_run;
 #pragma unroll
   for (int w = 0; w < 3; ++w) m_tot = fmaxf(m_tot, merge_ml[w][0][lane]);
-  float f = att_exp(m_run - m_tot);
+  float f = __builtin_amdgcn_exp2f(m_run - m_tot);
   float l_tot = l_half * f;
 #pragma unroll
   for (int e = 0; e < DB; ++e)
@@ -980,7 +989,7 @@ __global__ void __launch_bounds__(256 * GROUPS, 2) attention_prefill_x6_kernel(c
     for (int r = 0; r < 16; ++r) o[e][r] *= f;
 #pragma unroll
   for (int w = 0; w < 3; ++w) {
-    f = att_exp(merge_ml[w][0][lane] - m_tot);
+    f = __builtin_amdgcn_exp2f(merge_ml[w][0][lane] - m_tot);
     l_tot += merge_ml[w][1][lane] * f;
 #pragma unroll
     for (int e = 0; e < DB; ++e)
