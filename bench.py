@@ -12,6 +12,7 @@ reported under "extras" of the same line; --headline-only (or --no-extras / --no
 them out, which is what the profiler runs use.  Only one GPU is ever used.
 """
 import argparse
+import contextlib
 import ctypes as C
 import json
 import os
@@ -779,9 +780,35 @@ def llama_pieces(dev, steps, warmup):
     sec = ms * 1e-3 / steps
     flop = 2 * 2.0 * heads * hd * t * (t + 1) / 2
     nbytes = 4.0 * (2 * t * heads * hd + 2 * nkv * t * hd)
+    # 256 positions and up take both products as six bf16 terms on the bf16 matrix pipe (the f32 MFMAs of the other kernel
+    # occupy the vector ALU): TFLOP/s and frac_mfma_f32 are the f32 products the op stands for against the f32 peak,
+    # frac_mfma_bf16 prices the six-fold flops it actually issues against the bf16 peak.
     out["c4_attention_cached_t512"] = {"us": round(sec * 1e6, 2), "TFLOP/s": round(flop / sec / 1e12, 2), "frac_mfma_f32": round(flop / sec / 1e12 / MFMA_F32_PEAK_TF, 4),
+                                       "frac_mfma_bf16": round(6 * flop / sec / 1e12 / MFMA_BF16_PEAK_TF, 4), "kernel": "att_planes_kernel + attention_prefill_x6_kernel<2>",
                                        "algorithmic_bytes": int(nbytes), "verified": True,
                                        "replaces": "c4_rope_q + c4_qk_t + c4_causal_softmax_fused + c4_att_v + 2 repeats + 2 transposes"}
+    # the same op over a prompt of 2048 positions (a full cache), and with the f32 products it had before
+    t2 = cap
+    q2h = rng.normal(17, t2 * heads * hd).reshape(1, t2, heads * hd)
+    q2 = LB.copy(q2h, (1, t2, heads * hd), dev)
+    flop2 = 2 * 2.0 * heads * hd * t2 * (t2 + 1) / 2
+    for name, x6 in (("attention_cached_t2048", None), ("attention_cached_t2048_f32_products", 0)):
+        with (ug_amd.tuning(ATT_X6=x6) if x6 is not None else contextlib.nullcontext()):
+            att2 = ops.attention_cached(q2, kc, vc, t2, scale)
+            cs2 = Schedule.create_one(att2).compile()
+            cs2.run()
+            got2 = att2.data_vec().reshape(t2, heads, hd)
+            for h in (5, 30):     # two heads, the last 64 positions against float64
+                kv = h // (heads // nkv)
+                qq = q2h.reshape(t2, heads, hd)[-64:, h].astype(np.float64)
+                sc = qq @ kch[0, kv, :t2].astype(np.float64).T * scale
+                sc = np.where(np.arange(t2)[None, :] <= (t2 - 64 + np.arange(64))[:, None], sc, -np.inf)
+                verify(f"{name} head {h}", got2[-64:, h], softmax64(sc) @ vch[0, kv, :t2].astype(np.float64), rtol=0, atol=2e-5 * float(np.abs(got2).max()))
+            _, ms = timed_hot(dev, cs2.run, max(10, steps // 4), warmup, 0.1)
+        sec = ms * 1e-3 / max(10, steps // 4)
+        out[name] = {"us": round(sec * 1e6, 2), "TFLOP/s": round(flop2 / sec / 1e12, 2), "frac_mfma_f32": round(flop2 / sec / 1e12 / MFMA_F32_PEAK_TF, 4), "verified": True}
+        if x6 is None:
+            out[name]["frac_mfma_bf16"] = round(6 * flop2 / sec / 1e12 / MFMA_BF16_PEAK_TF, 4)
     return out
 
 
@@ -963,8 +990,8 @@ def config_summary(line):
     for key in ("c4_rms_norm_512x2048", "c4_rope_q_1x32x512x64", "c4_causal_mask_1x32x512x512", "c4_softmax_custom_1x32x512x512", "c4_softmax_lazy_1x32x512x512",
                 "c4_causal_softmax_fused"):
         take(key, key, ("us", "GB/s", "frac_hbm"))
-    for key in ("c4_qk_t_b32_512x512x64", "c4_att_v_b32_512x64x512", "c4_attention_cached_t512"):
-        take(key, key, ("us", "TFLOP/s", "frac_mfma_f32", "GB/s", "frac_hbm"))
+    for key in ("c4_qk_t_b32_512x512x64", "c4_att_v_b32_512x64x512", "c4_attention_cached_t512", "attention_cached_t2048"):
+        take(key, key, ("us", "TFLOP/s", "frac_mfma_f32", "frac_mfma_bf16", "GB/s", "frac_hbm"))
     for dst, src in (("c5_decode_f32_reference_graph", "llama_decode_f32"), ("c5_decode_f32_fused_level3", "llama_decode_f32_fused_projections"),
                      ("c5_decode_bf16_matrices_level3", "llama_decode_bf16_matrices"), ("c5_decode_bf16_matrices_prefill_bf16x3", "llama_decode_bf16_matrices_prefill_bf16x3"),
                      ("c5_unit_norms_decode_f32_reference_graph", "llama_decode_f32_reference_graph_unit_norms"),

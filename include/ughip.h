@@ -355,7 +355,10 @@ int ughip_kv_append_pair(ughip_device* dev, ughip_slice* kcache, ughip_slice* vc
  * cos/sin/pos are given.  t == 1 is ughip_attention_decode_rope on a cache of capacity cap;
  * t > 1 needs d = 32, 64 or 128 (UGHIP_ERR_UNSUPPORTED otherwise).  s - t == 0 and cap == s give
  * the reference's prefill.  q_offset / q_row_stride: as x_offset / x_row_stride of
- * ughip_kv_append (dst is always dense). */
+ * ughip_kv_append (dst is always dense).  With d = 64 and t >= 256 both products run as six bf16
+ * terms per f32 product (operands split into three bf16 terms each, f32 accumulation: the accuracy
+ * of the f32 products, not their bits) over planes of K and V that a first launch writes into a
+ * scratch block of the device (24 KiB per kv head and 32 keys, grown on demand). */
 int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_offset,
                            size_t q_row_stride, const ughip_slice* k, const ughip_slice* v,
                            ughip_slice* dst, size_t b, size_t n_heads, size_t n_kv_heads,
