@@ -61,7 +61,8 @@ def test_config3_bmm_f32(hip, cpu, rhs_nk):
     a, w = _config3_operands(False)
     got, kernel = _matmul(hip, F32, a, w, rhs_nk)
     print("config 3 f32", "NT" if rhs_nk else "NN", kernel, flush=True)
-    assert kernel == f"gemm_tiled<f32,{'NT' if rhs_nk else 'NN'},256x128,512t>"
+    # row-major rhs: the one-wave-per-SIMD f32 kernel; [n, k]-major rhs: the register-staged one (the faster of the two there)
+    assert kernel == ("gemm_tiled<f32,NT,256x128,512t>" if rhs_nk else "gemm_dma_f32<f32,NN,256x128,256t>")
     exact, mag = _f64_product(a, w)
     bound = 1024 * EPS32 * mag
     assert np.all(np.abs(got - exact) <= bound + 1e-12)
@@ -74,6 +75,36 @@ def test_config3_bmm_f32(hip, cpu, rhs_nk):
         lazy = LB.copy(a, a.shape, hip).matmul(LB.copy(w, w.shape, hip)).data_vec().reshape(got.shape)
         assert ug_amd.last_kernel() == kernel
         np.testing.assert_array_equal(lazy, got)
+
+
+@pytest.mark.parametrize("rhs_nk", [False, True], ids=["NN", "NT"])
+@pytest.mark.parametrize("bmnk", [
+    (2, 256, 128, 64),       # one tile per batch element, two K tiles (the shortest loop)
+    (1, 512, 256, 96),       # three K tiles: both stages come round again
+    (3, 300, 132, 128),      # a last tile that hangs over M and N (132 = 128 + 4)
+    (1, 1000, 2052, 512),    # many tiles, ragged both ways
+    (1, 37, 4, 64),          # a sliver of a tile
+    (2, 1024, 1024, 256),    # the XCD remap of the tile order (64 workgroups)
+])
+def test_matmul_f32_one_wave_per_simd(hip, tune, bmnk, rhs_nk):
+    """gemm_dma_f32 (f32, 256 x 128 tiles, loads that write LDS directly) forced through UGHIP_GEMM_SHAPE=8 on problems the
+    dispatcher would leave to the other kernels: against float64 within k eps sum|a||b|, and -- same k order -- bit for bit
+    against the register-staged kernel where that one takes the product."""
+    b, m, n, k = bmnk
+    a = rng.uniform_pm1(21, b * m * k).reshape(b, m, k)
+    w = rng.uniform_pm1(22, b * k * n).reshape(b, k, n)
+    tune.setenv("UGHIP_GEMM_SHAPE", "8")
+    got, kernel = _matmul(hip, F32, a, w, rhs_nk)
+    print("f32 one wave per SIMD", bmnk, "NT" if rhs_nk else "NN", kernel, flush=True)
+    assert kernel == f"gemm_dma_f32<f32,{'NT' if rhs_nk else 'NN'},256x128,256t>"
+    exact, mag = _f64_product(a, w)
+    assert np.all(np.abs(got - exact) <= k * EPS32 * mag + 1e-12), float(np.abs(got - exact).max())
+    tune.delenv("UGHIP_GEMM_SHAPE")
+    other, kernel2 = _matmul(hip, F32, a, w, rhs_nk)
+    if kernel2.startswith("gemm_tiled<f32") and "splitK" not in kernel2:
+        np.testing.assert_array_equal(got, other)
+    else:
+        assert np.all(np.abs(got - other) <= 2 * k * EPS32 * mag + 1e-12)
 
 
 @pytest.mark.parametrize("rhs_nk", [False, True], ids=["NN", "NT"])

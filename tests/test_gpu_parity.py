@@ -463,7 +463,8 @@ def test_matmul_16bit_kernel_choice(hip, bmnk, want):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype_name,bmnk,rhs_nk", [("f32", (2, 256, 128, 192), False), ("bf16", (8, 1024, 1024, 1024), False), ("bf16", (1, 2304, 2304, 2304), True),
-                                                    ("f32", (32, 512, 64, 512), False), ("f32", (1, 1, 2048, 2048), True), ("f32", (1, 100, 100, 100), False)])
+                                                    ("f32", (32, 512, 64, 512), False), ("f32", (1, 1, 2048, 2048), True), ("f32", (1, 100, 100, 100), False),
+                                                    ("f32", (8, 1024, 1024, 1024), False), ("f32", (1, 2048, 4096, 512), True)])
 def test_plan_names_what_is_launched(hip, dtype_name, bmnk, rhs_nk):
     """ughip_matmul_plan (no device) and the launch agree on the kernel, tile and split."""
     import ctypes as C

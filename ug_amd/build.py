@@ -32,7 +32,7 @@ def _run(cmd):
         raise RuntimeError("build step failed: " + " ".join(cmd))
 
 
-UGHIP_SOURCES = ("runtime.cpp", "lower_hip.cpp", "llama_ops.hip", "matmul.hip", "gemm_tiled.hip", "gemm_dma.hip", "rows_x3.hip", "attention.hip", "fused_linear.hip", "convert.hip")
+UGHIP_SOURCES = ("runtime.cpp", "lower_hip.cpp", "llama_ops.hip", "matmul.hip", "gemm_tiled.hip", "gemm_dma.hip", "gemm_dma_f32.hip", "rows_x3.hip", "attention.hip", "fused_linear.hip", "convert.hip")
 
 
 def build_ughip(only_changed=False):

@@ -65,6 +65,14 @@ double gemm_dma_cost_us(const MMArgs& p, size_t batch, int tile);
 void gemm_dma_name(int dtype, const MMArgs& p, int tile, char* out, size_t out_len);
 void gemm_tiled_name(int dtype, const MMArgs& p, size_t batch, bool rhs_bf16, const GemmEpilogue* epi, char* out, size_t out_len);
 
+// f32, one wave per SIMD: 256 x 128 tiles of v_mfma_f32_32x32x2_f32, loads that write LDS directly, rhs [n, k]- or [k, n]-major
+// (gemm_dma_f32.hip).  Any M, N % 4 == 0, K % 32 == 0 and K >= 64, 16-byte aligned rows, contiguous [batch, M, N] result.
+// _pick: whether this kernel should take the problem ([k, n]-major rhs, whole rounds of 256 tiles or nearly, K >= 512;
+// UGHIP_GEMM_SHAPE=8 forces it wherever it applies, any other value keeps it out).
+bool gemm_dma_f32_supported(const MMArgs& p, size_t batch);
+bool gemm_dma_f32_pick(const MMArgs& p, size_t batch);
+hipError_t gemm_dma_f32_launch(hipStream_t stream, const MMArgs& p, size_t batch);
+void gemm_dma_f32_name(const MMArgs& p, char* out, size_t out_len);
 
 // 1 .. 128 f32 rows x [m, k] against a bf16 matrix [n, k] as three bf16 terms per row element, the split done inside the product
 // (rows_x3.hip): partial sums of `units` consecutive (column tile, k tile) units per workgroup go to f32 slabs in `ws`, a fold adds

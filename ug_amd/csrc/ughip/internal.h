@@ -61,7 +61,7 @@ const char* dtype_name(int dt);
 // through ughip_set_tuning: dispatch reads an atomic, never the environment, so a launch thread and a test that
 // flips a switch do not meet in getenv / setenv.
 enum TuneKey {
-  TUNE_GEMM_SHAPE,          // 0..2: a gemm_tiled tile (keeps gemm_dma4 out); 3 / 4 / 5: gemm_dma4 with 256x256 / 256x128 / 128x128
+  TUNE_GEMM_SHAPE,          // 0..2: a gemm_tiled tile (keeps gemm_dma4 out); 3 / 4 / 5: gemm_dma4 with 256x256 / 256x128 / 128x128; 8: gemm_dma_f32 for f32 products
   TUNE_GEMM_SPLIT,          // K split of gemm_tiled
   TUNE_GEMM_4WAVES,         // (set at all) the 256-thread form of the 256x128 tile
   TUNE_GEMV_KS,             // waves per output column of the GEMV family: 1, 2 or 4

@@ -422,7 +422,7 @@ static int grow_gemm_ws(ughip_device* dev, size_t bytes) {
 
 // Which kernel family a product goes to: decided from shapes, strides, offsets and alignment alone, so that the choice can be
 // asked for without a device (ughip_matmul_plan) and is the same one the launch makes.
-enum Route { ROUTE_GEMV_NT, ROUTE_GEMV_NN, ROUTE_DMA, ROUTE_TILED, ROUTE_ANY, ROUTE_UNSUPPORTED };
+enum Route { ROUTE_GEMV_NT, ROUTE_GEMV_NN, ROUTE_DMA, ROUTE_DMA_F32, ROUTE_TILED, ROUTE_ANY, ROUTE_UNSUPPORTED };
 static Route matmul_route(int dtype, bool mixed, const MMArgs& p, size_t b, size_t lhs_offset, size_t rhs_offset, int* dma_tile) {
   const size_t m = (size_t)p.M, n = (size_t)p.N, k = (size_t)p.K;
   const bool f32 = dtype == UGHIP_F32;
@@ -441,6 +441,7 @@ static Route matmul_route(int dtype, bool mixed, const MMArgs& p, size_t b, size
     *dma_tile = bn;
     return ROUTE_DMA;
   }
+  if (f32 && !mixed && gemm_dma_f32_pick(p, b)) return ROUTE_DMA_F32;
   return gemm_tiled_supported(dtype, p, b, mixed) ? ROUTE_TILED : ROUTE_ANY;
 }
 
@@ -507,6 +508,9 @@ static int matmul_impl(ughip_device* dev, ughip_slice* dst, const ughip_slice* l
     else gemv_nn_f32<8><<<grid, 1024, 0, st>>>(p);
   } else if (route == ROUTE_DMA) {
     UGHIP_HIPCHK(gemm_dma_launch(st, dst->dtype, p, b, dma_tile));
+    return UGHIP_OK;
+  } else if (route == ROUTE_DMA_F32) {
+    UGHIP_HIPCHK(gemm_dma_f32_launch(st, p, b));
     return UGHIP_OK;
   } else if (route == ROUTE_TILED) {
     const size_t ws_bytes = gemm_tiled_workspace_bytes(dst->dtype, p, b);
@@ -735,6 +739,7 @@ extern "C" int ughip_matmul_plan(int dtype, int rhs_dtype, size_t b, size_t m, s
     case ROUTE_GEMV_NT: snprintf(buf, buf_len, "gemv_nt<%s>", tn); break;
     case ROUTE_GEMV_NN: snprintf(buf, buf_len, "gemv_nn<f32>"); break;
     case ROUTE_DMA: gemm_dma_name(dtype, p, tile, buf, buf_len); break;
+    case ROUTE_DMA_F32: gemm_dma_f32_name(p, buf, buf_len); break;
     case ROUTE_TILED: gemm_tiled_name(dtype, p, b, mixed, nullptr, buf, buf_len); break;
     default: snprintf(buf, buf_len, "gemm_any<%s>", tn); break;
   }
