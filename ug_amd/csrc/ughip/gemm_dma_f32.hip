@@ -21,9 +21,10 @@
 //   The operands are swapped (rhs first), so that a lane's accumulator holds four consecutive columns of one result row:
 //   16-byte stores, straight from the registers.
 //
-//   Schedule: the DMAs of tile t + 2 go out right behind the barrier of tile t (between its steps 2 and 3), which says
-//   both that tile t + 1 has landed everywhere and that nobody reads tile t's stage any more (step 3's operands were read
-//   during step 2); they have a whole tile's time to land.  Step 3 reads the first operands of tile t + 1.
+//   Schedule: one barrier per K tile, between its steps 2 and 3, which says both that tile t + 1 has landed everywhere and
+//   that nobody reads tile t's stage any more (step 3's operands were read during step 2): from there on the DMAs of tile
+//   t + 2 may go out, a wave at a time over the next four steps, and they have until the next barrier to land.  Step 3
+//   reads the first operands of tile t + 1.
 //
 // Any M (rows past the end fetch the last row again and are not stored), N % 4 == 0, K % 32 == 0 and K >= 64, lhs rows
 // contiguous and 16-byte aligned, rhs [n, k]- or [k, n]-major with 16-byte aligned rows, contiguous [batch, M, N] result.
@@ -161,11 +162,21 @@ __global__ void __launch_bounds__(256) gemm_dma_f32_kernel(MMArgs p, int tiles_m
   }
   __builtin_amdgcn_s_barrier();
   read_frags(0, 0, 0);
+  // The four waves of a workgroup send their DMA instructions at different steps: the CU's one address unit takes 16
+  // cycles per instruction, and 48 of them at once behind the barrier kept every wave from its MFMAs for 770 cycles per K
+  // tile (8 x 1024^3: 134 us, 131.5 this way).  (Dealing a wave's twelve one by one behind MFMAs was slower however it was
+  // written: as a second copy of the step the compiler kept a second set of accumulation registers, 142 us; as skips inside
+  // one copy the branches between the MFMAs cost more than the burst, 157 us.)  Tile t's loads may go out once barrier t - 2 has freed its stage and must have landed at
+  // barrier t - 1: wave 0 sends its part right behind barrier t - 2 (step 3), wave 1 in the next tile's step 0, waves 2
+  // and 3 in its step 1.
   for (int kt = 0; kt < KT; ++kt) {
     const int cur = kt & 1;
+    const bool mid = kt >= 1 && kt + 1 < KT;  // tile kt + 1 is not one of the two the prologue requested
     read_frags(cur, 1, 1);
+    if (mid && wave == 1) dma_tile(kt + 1);
     step(0);
     read_frags(cur, 2, 0);
+    if (mid && wave >= 2) dma_tile(kt + 1);
     step(1);
     read_frags(cur, 3, 1);
     step(0);
@@ -173,11 +184,12 @@ __global__ void __launch_bounds__(256) gemm_dma_f32_kernel(MMArgs p, int tiles_m
       wait_vmcnt<0>();   // this wave's part of tile kt + 1 has landed
       wait_lgkmcnt0();   // and its last reads of this tile's stage are done
       __builtin_amdgcn_s_barrier();
-      if (kt + 2 < KT) dma_tile(kt + 2);
+      if (kt + 2 < KT && wave == 0) dma_tile(kt + 2);
       read_frags(cur ^ 1, 0, 0);
     }
     step(1);
   }
+
   // Register r of lane l of accumulator (i, j): result row m0 + wm + 32 i + l % 32, columns n0 + wn + 32 j + 8 (r / 4) + 4 (l / 32) + r % 4.
   // Through the cache: an instruction writes 32 bytes of each of 32 rows, and the four instructions that complete a row's
   // 128-byte line merge there (stored past the cache they reach memory as they are: 8 x 1024^3 157 us against 133).
