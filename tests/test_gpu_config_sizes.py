@@ -107,6 +107,23 @@ def test_matmul_f32_one_wave_per_simd(hip, tune, bmnk, rhs_nk):
         assert np.all(np.abs(got - other) <= 2 * k * EPS32 * mag + 1e-12)
 
 
+def test_matmul_f32_one_wave_per_simd_random_shapes(hip, tune):
+    """Seeded random shapes for gemm_dma_f32 (forced): any M, N a multiple of 4, K a multiple of 32 from 64 up, both rhs
+    layouts, 1-3 batch elements, against float64 within k eps sum|a||b|."""
+    tune.setenv("UGHIP_GEMM_SHAPE", "8")
+    gen = np.random.default_rng(777)
+    for case in range(12):
+        b = int(gen.integers(1, 4)); m = int(gen.integers(1, 700)); n = 4 * int(gen.integers(1, 120)); k = 32 * int(gen.integers(2, 12))
+        rhs_nk = bool(gen.integers(0, 2))
+        a = rng.uniform_pm1(1000 + case, b * m * k).reshape(b, m, k)
+        w = rng.uniform_pm1(2000 + case, b * k * n).reshape(b, k, n)
+        print("f32 one wave per SIMD, random", case, (b, m, n, k), "NT" if rhs_nk else "NN", flush=True)
+        got, kernel = _matmul(hip, F32, a, w, rhs_nk)
+        assert kernel.startswith("gemm_dma_f32<f32,"), kernel
+        exact, mag = _f64_product(a, w)
+        assert np.all(np.abs(got - exact) <= k * EPS32 * mag + 1e-12), (case, float(np.abs(got - exact).max()))
+
+
 @pytest.mark.parametrize("rhs_nk", [False, True], ids=["NN", "NT"])
 def test_config3_bmm_bf16(hip, rhs_nk):
     """bf16 8 x 1024^3 (RNE-rounded copies of the f32 operands): no reference result exists (cpu_runtime.rs:345-356

@@ -1227,6 +1227,35 @@ def test_attention_cached_six_bf16_terms(hip, hip_ops, tune, interleaved, b, nh,
     assert e1 <= 4 * e0 + 1e-7 * float(np.abs(truth).max()), (e0, e1)
 
 
+def test_attention_cached_six_bf16_terms_random_shapes(hip, hip_ops, tune):
+    """Seeded random shapes for the six-term kernel (forced for any count of positions): 2-600 query positions behind 0-1500
+    cached ones, spare rows behind the cache, 1-8 kv heads with 1-8 query heads each, with and without either rope."""
+    tune.setenv("UGHIP_ATT_X6", "1")
+    gen = np.random.default_rng(4242)
+    d = 64
+    for case in range(14):
+        nkv = int(gen.choice([1, 2, 4, 8])); nh = nkv * int(gen.choice([1, 2, 4, 8])); b = int(gen.choice([1, 1, 2]))
+        t = int(gen.integers(2, 600)) if case % 2 else int(gen.integers(2, 70))
+        s = t + (int(gen.integers(0, 1500)) if case % 3 else 0); cap = s + int(gen.integers(0, 100))
+        rope = bool(gen.integers(0, 2)); inter = bool(gen.integers(0, 2))
+        print("attention cached, six bf16 terms, random", case, (b, nh, nkv, t, s, cap, rope, inter), flush=True)
+        q = rng.normal(700 + case, b * t * nh * d); k = rng.normal(800 + case, b * nkv * cap * d); v = rng.normal(900 + case, b * nkv * cap * d)
+        k4, v4 = k.reshape(b, nkv, cap, d).copy(), v.reshape(b, nkv, cap, d).copy()
+        k4[:, :, s:], v4[:, :, s:] = np.nan, np.inf
+        scale = float(np.float32(d) ** np.float32(-0.5)); pos0 = s - t
+        args = [LB.copy(q, (b, t, nh * d), hip), LB.copy(k4.ravel(), (b, nkv, cap, d), hip), LB.copy(v4.ravel(), (b, nkv, cap, d), hip), s, scale]
+        if rope:
+            cos, sin = _rope_tables(hip, d, max_pos=s + 8)
+            args += [cos, sin, LB.copy(np.array([pos0], np.int32), (1, 1), hip), inter]
+        got = hip_ops.attention_cached(*args).data_vec().reshape(b, t, nh, d)
+        q6 = q.reshape(b, t, nh, d).astype(np.float64)
+        if rope:
+            q6 = _rope_rows_f64(q6, cos.data_vec(), sin.data_vec(), pos0, inter)
+        truth = _attention_truth(q6.transpose(0, 2, 1, 3), k4[:, :, :s].astype(np.float64), v4[:, :, :s].astype(np.float64), s, t, scale, nh // nkv).transpose(0, 2, 1, 3)
+        tol = 2e-5 * np.abs(truth).max() + 2e-5 * np.abs(truth)
+        assert np.all(np.abs(got - truth) <= tol), (case, float(np.abs(got - truth).max()))
+
+
 def test_attention_cached_random_shapes(hip, hip_ops):
     """Seeded random shapes (one or a few query positions, caches of up to 3500 rows with spare rows behind them, 1-8 kv
     heads with 1-8 query heads each, every built head size, with and without either rope, cache lengths at the thresholds
