@@ -268,16 +268,41 @@ __global__ void __launch_bounds__(ATT_THREADS) attention_decode_kernel(const flo
     wave_l[wave] = l_run;
   }
   __syncthreads();
-  if (tid < lpk) {
-    float mx = wave_m[0];  // the first key of the range belongs to wave 0: finite unless the range is empty or the data is not
+  // Thread w * lpk + c weighs column group c of wave w; the 64 / lpk waves that share a wave of these threads are added
+  // by a butterfly over the lanes lpk apart, the ATT_WAVES * lpk / 64 such sums by the first lpk threads in wave order: a
+  // fixed order, and 16 times fewer instructions than one lane group walking all the waves.
+  const int n_merge = ATT_WAVES * lpk;  // <= ATT_THREADS: lpk <= 64
+  att_f32x4 o = {0.f, 0.f, 0.f, 0.f};
+  float sum = 0.f, mx = -INFINITY;
+  if (tid < n_merge) {
+    mx = wave_m[0];  // the first key of the range belongs to wave 0: finite unless the range is empty or the data is not
 #pragma unroll
     for (int w = 1; w < ATT_WAVES; ++w) mx = fmaxf(mx, wave_m[w]);
-    att_f32x4 o = {0.f, 0.f, 0.f, 0.f};
-    float sum = 0.f;
-    for (int w = 0; w < ATT_WAVES; ++w) {
-      const float f = wave_m[w] == -INFINITY ? 0.f : expf(wave_m[w] - mx);  // 0 for a wave without keys
-      o += f * red[w * 64 + tid];
-      sum += f * wave_l[w];
+    const int w = tid / lpk, c = tid % lpk;
+    const float f = wave_m[w] == -INFINITY ? 0.f : expf(wave_m[w] - mx);  // 0 for a wave without keys
+    o = f * red[w * 64 + c];
+    sum = f * wave_l[w];
+    for (int off = lpk; off < 64; off <<= 1) {
+      sum += __shfl_xor(sum, off, 64);
+      o.x += __shfl_xor(o.x, off, 64);
+      o.y += __shfl_xor(o.y, off, 64);
+      o.z += __shfl_xor(o.z, off, 64);
+      o.w += __shfl_xor(o.w, off, 64);
+    }
+  }
+  __syncthreads();  // every partial has been read: the merge buffers are free for the second stage
+  const int n_stage2 = (n_merge + 63) / 64;
+  if (tid < n_merge && lane < lpk) {
+    red[wave * 64 + lane] = o;
+    if (lane == 0) wave_l[wave] = sum;
+  }
+  __syncthreads();
+  if (tid < lpk) {
+    o = red[tid];
+    sum = wave_l[0];
+    for (int w = 1; w < n_stage2; ++w) {
+      o += red[w * 64 + tid];
+      sum += wave_l[w];
     }
     if (nsplit == 1) {
       reinterpret_cast<att_f32x4*>(dst + (size_t)bh * d)[tid] = o / sum;
