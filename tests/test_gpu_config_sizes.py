@@ -62,7 +62,7 @@ def test_config3_bmm_f32(hip, cpu, rhs_nk):
     got, kernel = _matmul(hip, F32, a, w, rhs_nk)
     print("config 3 f32", "NT" if rhs_nk else "NN", kernel, flush=True)
     # row-major rhs: the one-wave-per-SIMD f32 kernel; [n, k]-major rhs: the register-staged one (the faster of the two there)
-    assert kernel == ("gemm_tiled<f32,NT,256x128,512t>" if rhs_nk else "gemm_dma_f32<f32,NN,256x128,256t>")
+    assert kernel == ("gemm_tiled<f32,NT,256x128,512t>" if rhs_nk else "gemm_dma_f32<f32,NN,256x128,320t>")
     exact, mag = _f64_product(a, w)
     bound = 1024 * EPS32 * mag
     assert np.all(np.abs(got - exact) <= bound + 1e-12)
@@ -96,7 +96,7 @@ def test_matmul_f32_one_wave_per_simd(hip, tune, bmnk, rhs_nk):
     tune.setenv("UGHIP_GEMM_SHAPE", "8")
     got, kernel = _matmul(hip, F32, a, w, rhs_nk)
     print("f32 one wave per SIMD", bmnk, "NT" if rhs_nk else "NN", kernel, flush=True)
-    assert kernel == f"gemm_dma_f32<f32,{'NT' if rhs_nk else 'NN'},256x128,256t>"
+    assert kernel == f"gemm_dma_f32<f32,{'NT' if rhs_nk else 'NN'},256x128,320t>"
     exact, mag = _f64_product(a, w)
     assert np.all(np.abs(got - exact) <= k * EPS32 * mag + 1e-12), float(np.abs(got - exact).max())
     tune.delenv("UGHIP_GEMM_SHAPE")

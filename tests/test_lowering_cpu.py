@@ -319,7 +319,7 @@ def test_kernel_choice_for_the_baseline_shapes_is_pinned():
     F, B = ug_amd.F32, ug_amd.BF16
     want = {
         # config 3: 8 x 1024^3, both rhs layouts
-        (F, F, 8, 1024, 1024, 1024, 0): "gemm_dma_f32<f32,NN,256x128,256t>",
+        (F, F, 8, 1024, 1024, 1024, 0): "gemm_dma_f32<f32,NN,256x128,320t>",
         (F, F, 8, 1024, 1024, 1024, 1): "gemm_tiled<f32,NT,256x128,512t>",
         (B, B, 8, 1024, 1024, 1024, 0): "gemm_dma4<bf16,NN,256x128,256t>",
         (B, B, 8, 1024, 1024, 1024, 1): "gemm_dma4<bf16,NT,256x128,256t>",
@@ -344,9 +344,9 @@ def test_kernel_choice_for_the_baseline_shapes_is_pinned():
         (B, B, 1, 3072, 4096, 4096, 1): "gemm_dma4<bf16,NT,256x256,256t>",
         (F, F, 1, 100, 100, 100, 0): "gemm_any<f32>",
         # large f32 products: row-major rhs in whole rounds of tiles on the one-wave-per-SIMD kernel, the rest register-staged
-        (F, F, 1, 4096, 4096, 4096, 0): "gemm_dma_f32<f32,NN,256x128,256t>",
+        (F, F, 1, 4096, 4096, 4096, 0): "gemm_dma_f32<f32,NN,256x128,320t>",
         (F, F, 1, 4096, 4096, 4096, 1): "gemm_tiled<f32,NT,256x128,512t>",
-        (F, F, 4, 2048, 2048, 2048, 0): "gemm_dma_f32<f32,NN,256x128,256t>",
+        (F, F, 4, 2048, 2048, 2048, 0): "gemm_dma_f32<f32,NN,256x128,320t>",
     }
     got = {key: _plan(*key) for key in want}
     assert got == want

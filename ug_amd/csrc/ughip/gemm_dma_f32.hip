@@ -1,14 +1,14 @@
-// f32 GEMM for gfx950 with one wave per SIMD: 256 x 128 block tile, 4 waves laid out 2 x 2, a wave owns 128 x 64 of it
-// as eight 32 x 32 accumulators of v_mfma_f32_32x32x2_f32.  The counterpart for f32 of the 16-bit kernel in gemm_dma.hip,
-// replacing the cuBLAS call of ug-cuda/src/gemm.rs:130-332 for large f32 products with a [k, n]-major rhs (BASELINE's
-// batched matmul of row-major operands).
+// f32 GEMM for gfx950 with one multiplying wave per SIMD: 256 x 128 block tile, 4 waves laid out 2 x 2, a wave owns
+// 128 x 64 of it as eight 32 x 32 accumulators of v_mfma_f32_32x32x2_f32; a fifth wave sends the loads.  The counterpart
+// for f32 of the 16-bit kernel in gemm_dma.hip, replacing the cuBLAS call of ug-cuda/src/gemm.rs:130-332 for large f32
+// products with a [k, n]-major rhs (the batched matmul of row-major operands).
 //
 // Why a second f32 kernel beside the register-staged one (gemm_tiled.hip): on this chip an f32 MFMA executes on the vector
 // ALU's datapath -- while one runs, no vector instruction of any wave issues on that SIMD -- and takes 64 cycles, so the
 // matrix rate is reached only by a stream of MFMAs with next to nothing vector between them.  Here operand tiles go from
 // memory into LDS without passing registers (global_load_lds_dwordx4: no staging loads, stores or address arithmetic in
-// the loop), a K tile of 32 is 128 MFMAs per wave (8192 cycles) behind ONE barrier, and the 24-48 LDS reads and 12 DMA
-// instructions a wave issues per K tile sit between MFMAs that each leave 60 idle issue cycles.
+// the loop), a K tile of 32 is 128 MFMAs per wave (8192 cycles) behind ONE barrier, and the 24-48 LDS reads a multiplying
+// wave issues per K tile sit between MFMAs that each leave 60 idle issue cycles.
 //
 //   LDS, two stages of 48 KiB: A tile [256 rows][32 k] and, rhs [n, k]-major, B tile [128 rows][32 k]: 128-byte rows of 8
 //   chunks of 16 bytes, chunk' = chunk ^ ((row / 2) & 7) (the 16 rows a 128-bit operand read names in one pass land on all
@@ -21,10 +21,10 @@
 //   The operands are swapped (rhs first), so that a lane's accumulator holds four consecutive columns of one result row:
 //   16-byte stores, straight from the registers.
 //
-//   Schedule: one barrier per K tile, between its steps 2 and 3, which says both that tile t + 1 has landed everywhere and
-//   that nobody reads tile t's stage any more (step 3's operands were read during step 2): from there on the DMAs of tile
-//   t + 2 may go out, a wave at a time over the next four steps, and they have until the next barrier to land.  Step 3
-//   reads the first operands of tile t + 1.
+//   Schedule: one barrier per K tile, between its steps 2 and 3, which says both that tile t + 1 has landed (the loader
+//   waits for its loads in front of it) and that nobody reads tile t's stage any more (step 3's operands were read during
+//   step 2): behind it the loader sends the DMAs of tile t + 2, which have until the next barrier to land.  Step 3 reads
+//   the first operands of tile t + 1.
 //
 // Any M (rows past the end fetch the last row again and are not stored), N % 4 == 0, K % 32 == 0 and K >= 64, lhs rows
 // contiguous and 16-byte aligned, rhs [n, k]- or [k, n]-major with 16-byte aligned rows, contiguous [batch, M, N] result.
@@ -46,7 +46,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 256, BN = 128, BK = 32;
 constexpr int A_BYTES = BM * BK * 4, B_BYTES = BN * BK * 4, STAGE_BYTES = A_BYTES + B_BYTES;
-constexpr int NDA = A_BYTES / 1024 / 4, NDB = B_BYTES / 1024 / 4, ND = NDA + NDB;  // DMA instructions per wave and K tile
+constexpr int NDA = A_BYTES / 1024 / 4, NDB = B_BYTES / 1024 / 4, ND = NDA + NDB;  // a quarter of the DMA instructions of a K tile (lhs, rhs, both)
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -66,7 +66,7 @@ __device__ __forceinline__ int kc_idx(int row, int chunk) { return row * 8 + (ch
 __device__ __forceinline__ int kn_byte(int k, int n) { return k * (BN * 4) + ((((n >> 2) ^ (((k >> 2) & 1) << 3))) << 4) + (n & 3) * 4; }
 
 template <bool B_KN>
-__global__ void __launch_bounds__(256) gemm_dma_f32_kernel(MMArgs p, int tiles_m, int tiles_n) {
+__global__ void __launch_bounds__(320) gemm_dma_f32_kernel(MMArgs p, int tiles_m, int tiles_n) {
   extern __shared__ f32x4 lds[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -87,34 +87,54 @@ __global__ void __launch_bounds__(256) gemm_dma_f32_kernel(MMArgs p, int tiles_m
   const unsigned lds_addr = (unsigned)(size_t)(__attribute__((address_space(3))) char*)lds;
   const int m_last = p.M - 1 - m0, n_left = p.N - n0;
 
-  // per-lane byte offsets of this wave's DMA instructions (the same for every K tile; the scalar base moves).  Rows and
-  // chunks past the end of the operand fetch the last one again (their results are not stored).
-  unsigned voff[ND];
-#pragma unroll
-  for (int i = 0; i < NDA; ++i) {
-    const int row = (i * 4 + wave) * 8 + (lane >> 3), cp = lane & 7;
-    voff[i] = (unsigned)(min(row, m_last) * lda * 4 + ((cp ^ ((row >> 1) & 7)) << 4));
-  }
-#pragma unroll
-  for (int i = 0; i < NDB; ++i) {
-    const int g = i * 4 + wave;
-    if (!B_KN) {
-      const int row = g * 8 + (lane >> 3), cp = lane & 7;
-      voff[NDA + i] = (unsigned)(min(row, n_left - 1) * ldb * 4 + ((cp ^ ((row >> 1) & 7)) << 4));
-    } else {
-      const int k = g * 2 + (lane >> 5), cpos = lane & 31;
-      const int src = cpos ^ (((k >> 2) & 1) << 3);
-      voff[NDA + i] = (unsigned)(k * ldb * 4 + (min(src, n_left / 4 - 1) << 4));  // N % 4 == 0: whole 16-byte chunks
-    }
-  }
   const long long a_step = BK * 4, b_step = B_KN ? (long long)BK * ldb * 4 : BK * 4;
-  auto dma_tile = [&](int tile) {
-    const unsigned st = lds_addr + (tile & 1) * STAGE_BYTES;
+  if (wave == 4) {
+    // The loader: all 48 DMA instructions of a K tile (lhs rows 8 i + lane / 8, then the rhs), none of the MFMAs.  Its
+    // instructions are scalar and memory ones: they issue beside the MFMAs of the wave it shares a SIMD with, and the four
+    // multiplying waves never wait for the CU's one address unit, which takes 16 cycles per instruction (with every wave
+    // sending its twelve behind the barrier each was kept from its MFMAs for 770 cycles per K tile, 8 x 1024^3 134 us;
+    // a wave at a time over the tile's steps 131.5; this way 127.9 on the box that gave 129.3 for the latter).
+    // Per-lane byte offsets are the same for every K tile (the scalar base moves); rows and chunks past the end of the
+    // operand fetch the last one again (their results are not stored).
+    unsigned vo[4 * ND];
 #pragma unroll
-    for (int i = 0; i < NDA; ++i) dma16(Ab + tile * a_step, voff[i], st + (i * 4 + wave) * 1024);
+    for (int i = 0; i < 4 * NDA; ++i) {
+      const int row = i * 8 + (lane >> 3), cp = lane & 7;
+      vo[i] = (unsigned)(min(row, m_last) * lda * 4 + ((cp ^ ((row >> 1) & 7)) << 4));
+    }
 #pragma unroll
-    for (int i = 0; i < NDB; ++i) dma16(Bb + tile * b_step, voff[NDA + i], st + A_BYTES + (i * 4 + wave) * 1024);
-  };
+    for (int g = 0; g < 4 * NDB; ++g) {
+      if (!B_KN) {
+        const int row = g * 8 + (lane >> 3), cp = lane & 7;
+        vo[4 * NDA + g] = (unsigned)(min(row, n_left - 1) * ldb * 4 + ((cp ^ ((row >> 1) & 7)) << 4));
+      } else {
+        const int k = g * 2 + (lane >> 5), cpos = lane & 31;
+        const int src = cpos ^ (((k >> 2) & 1) << 3);
+        vo[4 * NDA + g] = (unsigned)(k * ldb * 4 + (min(src, n_left / 4 - 1) << 4));
+      }
+    }
+    auto dma_all = [&](int tile) {
+      const unsigned st = lds_addr + (tile & 1) * STAGE_BYTES;
+#pragma unroll
+      for (int i = 0; i < 4 * NDA; ++i) dma16(Ab + tile * a_step, vo[i], st + i * 1024);
+#pragma unroll
+      for (int g = 0; g < 4 * NDB; ++g) dma16(Bb + tile * b_step, vo[4 * NDA + g], st + A_BYTES + g * 1024);
+    };
+    dma_all(0);
+    if (KT > 1) {
+      dma_all(1);
+      wait_vmcnt<4 * ND>();
+    } else {
+      wait_vmcnt<0>();
+    }
+    __builtin_amdgcn_s_barrier();
+    for (int kt = 0; kt + 1 < KT; ++kt) {
+      wait_vmcnt<0>();  // tile kt + 1 has landed
+      __builtin_amdgcn_s_barrier();
+      if (kt + 2 < KT) dma_all(kt + 2);  // into the stage of tile kt, which nobody reads any more
+    }
+    return;
+  }
 
   f32x16 acc[4][2];
 #pragma unroll
@@ -152,39 +172,20 @@ __global__ void __launch_bounds__(256) gemm_dma_f32_kernel(MMArgs p, int tiles_m
         for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[set][j][e], fa[set][i][e], acc[i][j], 0, 0, 0);  // rhs first: see above
   };
 
-  // tiles 0 and 1 requested; tile 0 landed everywhere; its first operands read
-  dma_tile(0);
-  if (KT > 1) {
-    dma_tile(1);
-    wait_vmcnt<ND>();
-  } else {
-    wait_vmcnt<0>();
-  }
+  // tile 0 has landed (the loader says so); its first operands read
   __builtin_amdgcn_s_barrier();
   read_frags(0, 0, 0);
-  // The four waves of a workgroup send their DMA instructions at different steps: the CU's one address unit takes 16
-  // cycles per instruction, and 48 of them at once behind the barrier kept every wave from its MFMAs for 770 cycles per K
-  // tile (8 x 1024^3: 134 us, 131.5 this way).  (Dealing a wave's twelve one by one behind MFMAs was slower however it was
-  // written: as a second copy of the step the compiler kept a second set of accumulation registers, 142 us; as skips inside
-  // one copy the branches between the MFMAs cost more than the burst, 157 us.)  Tile t's loads may go out once barrier t - 2 has freed its stage and must have landed at
-  // barrier t - 1: wave 0 sends its part right behind barrier t - 2 (step 3), wave 1 in the next tile's step 0, waves 2
-  // and 3 in its step 1.
   for (int kt = 0; kt < KT; ++kt) {
     const int cur = kt & 1;
-    const bool mid = kt >= 1 && kt + 1 < KT;  // tile kt + 1 is not one of the two the prologue requested
     read_frags(cur, 1, 1);
-    if (mid && wave == 1) dma_tile(kt + 1);
     step(0);
     read_frags(cur, 2, 0);
-    if (mid && wave >= 2) dma_tile(kt + 1);
     step(1);
     read_frags(cur, 3, 1);
     step(0);
     if (kt + 1 < KT) {
-      wait_vmcnt<0>();   // this wave's part of tile kt + 1 has landed
-      wait_lgkmcnt0();   // and its last reads of this tile's stage are done
+      wait_lgkmcnt0();  // this wave's last reads of the tile's stage are done
       __builtin_amdgcn_s_barrier();
-      if (kt + 2 < KT && wave == 0) dma_tile(kt + 2);
       read_frags(cur ^ 1, 0, 0);
     }
     step(1);
@@ -224,7 +225,7 @@ hipError_t launch(hipStream_t stream, const MMArgs& p, size_t batch) {
   }
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const size_t total = batch * (size_t)tiles_m * tiles_n;
-  kernel<<<dim3((unsigned)total), dim3(256), LDS_BYTES, stream>>>(p, tiles_m, tiles_n);
+  kernel<<<dim3((unsigned)total), dim3(320), LDS_BYTES, stream>>>(p, tiles_m, tiles_n);  // four multiplying waves and the loader
   return hipGetLastError();
 }
 
@@ -262,7 +263,7 @@ bool gemm_dma_f32_pick(const MMArgs& p, size_t batch) {
 
 void gemm_dma_f32_name(const MMArgs& p, char* out, size_t out_len) {
   const bool nn = p.b_cs == 1 && p.b_rs != 1;
-  snprintf(out, out_len, "gemm_dma_f32<f32,%s,%dx%d,256t>", nn ? "NN" : "NT", BM, BN);
+  snprintf(out, out_len, "gemm_dma_f32<f32,%s,%dx%d,320t>", nn ? "NN" : "NT", BM, BN);
 }
 
 hipError_t gemm_dma_f32_launch(hipStream_t stream, const MMArgs& p, size_t batch) {
