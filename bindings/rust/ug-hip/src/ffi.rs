@@ -445,6 +445,33 @@ extern "C" {
         k: usize,
         product: c_int,
     ) -> c_int;
+    pub fn ughip_rms_linear_rows(
+        dev: *mut UghipDevice,
+        x: *const UghipSlice,
+        alpha: *const UghipSlice,
+        eps: f32,
+        w: *const UghipSlice,
+        dst: *mut UghipSlice,
+        m: usize,
+        n: usize,
+        k: usize,
+        product: c_int,
+    ) -> c_int;
+    pub fn ughip_rms_mlp_rows(
+        dev: *mut UghipDevice,
+        x: *const UghipSlice,
+        alpha: *const UghipSlice,
+        eps: f32,
+        w_gate_up: *const UghipSlice,
+        w_down: *const UghipSlice,
+        residual: *const UghipSlice,
+        dst: *mut UghipSlice,
+        m: usize,
+        n: usize,
+        inter: usize,
+        k: usize,
+        product: c_int,
+    ) -> c_int;
     pub fn ughip_linear_rows_plan(
         w_dtype: c_int,
         product: c_int,

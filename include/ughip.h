@@ -436,6 +436,26 @@ int ughip_linear_add_rows(ughip_device* dev, const ughip_slice* x, const ughip_s
                           int product);
 int ughip_linear_swiglu_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* w,
                              ughip_slice* dst, size_t m, size_t n, size_t k, int product);
+/* The same with more of the layer folded in (model.rs:65-78 in front of 206-208 and 366-372; 160-168 whole).
+ * ughip_rms_linear_rows: dst[m, n] = y w^T with y = x / sqrt(mean(x^2) + eps) * alpha (alpha: k F32 values; the
+ *   division as a multiplication by the reciprocal, like ughip_rms_gemv_multi).  Where the three-term product reads
+ *   planes from memory, the pass that writes them normalises the rows on its way (one launch and one round trip
+ *   less); everywhere else the normalised rows go through the device's own scratch.
+ * ughip_rms_mlp_rows: dst[m, n] = (silu(y gate^T) * (y up^T)) w_down^T + residual[m, n], with y as above, or y = x when
+ *   alpha is NULL; w_gate_up is [2 inter, k] (gate rows, then up rows), w_down [n, inter], both of one dtype; dst may be
+ *   residual.  The [m, inter] rows between the two products stay in the device's scratch: where both products read
+ *   planes, the fold of the first writes them as the second one's planes (no f32 rows, no pass that splits them).
+ *   ughip_last_kernel() names both products ("... -> ...").
+ * Same shapes, dtypes and `product` as the entry points above (inter % 8 == 0), same results as the pieces run one
+ * after the other (the norm's sum of squares is added in this library's order, not a generated kernel's).  The scratch
+ * grows to m (k + 1.5 inter) floats and is kept until the device is released. */
+int ughip_rms_linear_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* alpha, float eps,
+                          const ughip_slice* w, ughip_slice* dst, size_t m, size_t n, size_t k,
+                          int product);
+int ughip_rms_mlp_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* alpha, float eps,
+                       const ughip_slice* w_gate_up, const ughip_slice* w_down,
+                       const ughip_slice* residual, ughip_slice* dst, size_t m, size_t n, size_t inter,
+                       size_t k, int product);
 /* No counterpart in the reference, no device needed: the kernel the three entry points above would launch (form 0:
  * ughip_linear_rows, 1: ughip_linear_add_rows, 2: ughip_linear_swiglu_rows) for m rows against an [n, k] matrix of
  * w_dtype, by the name ughip_last_kernel() reports after the launch -- kernel family, tile, units or K split, fold.

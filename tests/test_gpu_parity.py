@@ -2329,3 +2329,94 @@ def test_half_precision_elementwise_and_reduce(hip, dtype):
     s = dec(ly.reduce("sum", 1).data_vec()).reshape(rows, -1)[:, 0]
     eps16 = 2.0 ** -8 if dtype == ug_amd.BF16 else 2.0 ** -11
     assert np.all(np.abs(s - y.astype(np.float64).sum(1)) <= cols * eps16 * np.abs(y).sum(1))
+
+
+@pytest.mark.parametrize("t,k,inter,n,product,w_bf16", [(1900, 2048, 5632, 2048, 1, True), (700, 1024, 2816, 1024, 1, True), (300, 512, 1024, 512, 1, True),
+                                                        (128, 2048, 5632, 2048, 1, True), (40, 256, 512, 256, 1, True), (50, 256, 512, 264, 0, True),
+                                                        (37, 128, 96, 72, 0, False), (9, 64, 64, 64, 1, True)])
+def test_norm_and_mlp_folded_into_the_products_of_rows(hip, t, k, inter, n, product, w_bf16):
+    """ughip_rms_linear_rows and ughip_rms_mlp_rows: the RMSNorm in front of a product of rows and the MLP block whole
+    (model.rs:65-78, 160-168, 366-372).  Against float64 with the bounds of the pieces; without a norm, bit for bit what
+    ughip_linear_swiglu_rows followed by ughip_linear_add_rows give (where the second product reads planes the fold of
+    the first writes them: same terms); with the norm, within a few ulps of the pieces run on rows normalised on the host
+    (the sum of squares is added in another order); a sentinel behind every result."""
+    import ctypes as C
+    print("norm and mlp folded in", t, k, inter, n, product, w_bf16, flush=True)
+    x = rng.normal(181, t * k)
+    alpha = (1.0 + rng.normal(182, k, 0.1)).astype(np.float32)
+    wgu = rng.normal(183, 2 * inter * k, 0.05)
+    wd = rng.normal(184, n * inter, 0.05)
+    r = rng.normal(185, t * n)
+    eps_n = 1e-5
+    if w_bf16:
+        wgu, wd = rng.bf16_round(wgu), rng.bf16_round(wd)
+    store = (lambda v: rng.to_bf16_bits(v)) if w_bf16 else (lambda v: v)
+    lib, dev, z = ug_amd.ughip_lib(), C.c_void_p(hip.raw_hip()), C.c_size_t
+    for fn in (lib.ughip_rms_linear_rows, lib.ughip_rms_mlp_rows):
+        fn.restype = C.c_int
+    raw = lambda s_: C.c_void_p(s_.raw())
+    sx, sa, sgu, sd, sr = hip.slice_from(x), hip.slice_from(alpha), hip.slice_from(store(wgu)), hip.slice_from(store(wd)), hip.slice_from(r)
+    guard = 64
+
+    def result(call, cols):
+        d = hip.slice_from(np.full(t * cols + guard, 7.0, np.float32))
+        assert call(d) == 0, lib.ughip_last_error()
+        kern = ug_amd.last_kernel()
+        v = d.to_vec()
+        assert np.all(v[t * cols:] == 7.0), "wrote past the end of the result"
+        return v[:t * cols].reshape(t, cols).copy(), kern
+
+    P, f = C.c_int(product), C.c_float
+    x64, a64 = x.reshape(t, k).astype(np.float64), alpha.astype(np.float64)
+    gu64, d64 = wgu.reshape(2 * inter, k).astype(np.float64), wd.reshape(n, inter).astype(np.float64)
+    eps = float(np.finfo(np.float32).eps)
+
+    def mlp64(y64):
+        gg, uu = y64 @ gu64[:inter].T, y64 @ gu64[inter:].T
+        sg = gg / (1.0 + np.exp(-gg))
+        h = sg * uu
+        h_bound = k * eps * ((np.abs(y64) @ np.abs(gu64[:inter]).T) * (np.abs(uu) * 1.3) + (np.abs(y64) @ np.abs(gu64[inter:]).T) * np.abs(sg)) + 8 * eps * np.abs(h) + 1e-7
+        out = h @ d64.T + r.reshape(t, n)
+        bound = h_bound @ np.abs(d64).T + inter * eps * (np.abs(h) @ np.abs(d64).T) + 2 * eps * np.abs(out) + 1e-6
+        return out, bound
+
+    # the MLP block without a norm: against float64, and bit for bit the two pieces
+    got, kern = result(lambda d: lib.ughip_rms_mlp_rows(dev, raw(sx), None, f(0.0), raw(sgu), raw(sd), raw(sr), raw(d), z(t), z(n), z(inter), z(k), P), n)
+    assert " -> " in kern, kern
+    if product == 1 and t > 128 and inter % 64 == 0 and kern.startswith("gemm_dma4"):
+        assert "swiglu fold onto planes" in kern, kern
+    want, bound = mlp64(x64)
+    assert np.all(np.abs(got - want) <= bound)
+    h_piece, _ = result(lambda d: lib.ughip_linear_swiglu_rows(dev, raw(sx), raw(sgu), raw(d), z(t), z(inter), z(k), P), inter)
+    sh = hip.slice_from(h_piece.reshape(-1))
+    piece, _ = result(lambda d: lib.ughip_linear_add_rows(dev, raw(sh), raw(sd), raw(sr), raw(d), z(t), z(n), z(inter), P), n)
+    np.testing.assert_array_equal(got, piece)
+
+    # with the norm in front
+    ms = np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + eps_n)
+    y64 = x64 / ms * a64
+    got_n, kern_n = result(lambda d: lib.ughip_rms_mlp_rows(dev, raw(sx), raw(sa), f(eps_n), raw(sgu), raw(sd), raw(sr), raw(d), z(t), z(n), z(inter), z(k), P), n)
+    want_n, bound_n = mlp64(y64)
+    # the normalised rows themselves carry 3 roundings
+    slack = 4 * eps * (np.abs(want_n) + np.abs(r.reshape(t, n))) + 4 * eps * inter * np.max(np.abs(d64)) * np.max(np.abs(want_n))
+    assert np.all(np.abs(got_n - want_n) <= bound_n + slack)
+    y32 = (x.reshape(t, k) * (np.float32(1.0) / ms.astype(np.float32)) * alpha).astype(np.float32)
+    sy = hip.slice_from(y32.reshape(-1))
+    piece_n, _ = result(lambda d: lib.ughip_rms_mlp_rows(dev, raw(sy), None, f(0.0), raw(sgu), raw(sd), raw(sr), raw(d), z(t), z(n), z(inter), z(k), P), n)
+    assert np.max(np.abs(got_n - piece_n)) <= 1e-5 * max(1.0, float(np.max(np.abs(piece_n))))
+
+    # the norm in front of a single product: the stacked gate | up matrix stands in for q | k | v
+    rows = 2 * inter
+    got_l, kern_l = result(lambda d: lib.ughip_rms_linear_rows(dev, raw(sx), raw(sa), f(eps_n), raw(sgu), raw(d), z(t), z(rows), z(k), P), rows)
+    lin64 = y64 @ gu64.T
+    lin_bound = (k + 4) * eps * (np.abs(y64) @ np.abs(gu64).T) + 1e-7
+    assert np.all(np.abs(got_l - lin64) <= lin_bound)
+    piece_l, kern_p = result(lambda d: lib.ughip_linear_rows(dev, raw(sy), raw(sgu), raw(d), z(t), z(rows), z(k), P), rows)
+    assert kern_l == kern_p, (kern_l, kern_p)
+    assert np.max(np.abs(got_l - piece_l)) <= 1e-5 * max(1.0, float(np.max(np.abs(piece_l))))
+    # refused: no alpha, a short alpha
+    d = hip.allocate_uninit(ug_amd.F32, t * rows)
+    assert lib.ughip_rms_linear_rows(dev, raw(sx), None, f(eps_n), raw(sgu), raw(d), z(t), z(rows), z(k), P) != 0
+    short = hip.slice_from(alpha[:k - 4].copy())
+    assert lib.ughip_rms_linear_rows(dev, raw(sx), raw(short), f(eps_n), raw(sgu), raw(d), z(t), z(rows), z(k), P) != 0
+    assert lib.ughip_rms_mlp_rows(dev, raw(sx), raw(short), f(eps_n), raw(sgu), raw(sd), raw(sr), raw(d), z(t), z(n), z(inter), z(k), P) != 0

@@ -52,6 +52,8 @@ def test_entry_points_refuse_a_null_device_without_touching_the_gpu():
         "ughip_linear_rows": (None, None, None, None, C.c_size_t(16), z, C.c_size_t(32), C.c_int(0)),
         "ughip_linear_add_rows": (None, None, None, None, None, C.c_size_t(16), z, C.c_size_t(32), C.c_int(0)),
         "ughip_linear_swiglu_rows": (None, None, None, None, C.c_size_t(16), z, C.c_size_t(32), C.c_int(0)),
+        "ughip_rms_linear_rows": (None, None, None, f, None, None, C.c_size_t(16), z, C.c_size_t(32), C.c_int(0)),
+        "ughip_rms_mlp_rows": (None, None, None, f, None, None, None, None, C.c_size_t(16), z, C.c_size_t(32), C.c_size_t(32), C.c_int(0)),
         "ughip_argmax_row": (None, None, C.c_size_t(4), z, None, None, None, z),
         "ughip_convert": (None, None, None),
         "ughip_matmul": (None, None, None, None, z, z, z, z, z, None, None, z, None, None, z),

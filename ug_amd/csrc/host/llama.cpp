@@ -404,6 +404,50 @@ struct HipOps : Ops {
     return LB::custom(f, {x, w, residual}, residual.shape(), x.dtype(), x.device());
   }
 
+  // The norm in front of a product of many rows, and the MLP block whole: one schedule item each, and where the
+  // three-term product reads planes the passes that write them do the norm / come out of the SwiGLU fold.
+  LB linear_norm(const LB& x, const LB& alpha, float eps, const LB& w) const override {
+    if (!many_f32_rows(x, w, 8) || alpha.dtype() != DType::F32 || alpha.elem_count() != x.dims().back() || switch_on(SW_NO_FOLD_EPILOGUES))
+      return Ops::linear_norm(x, alpha, eps, w);
+    const size_t k = x.dims().back(), rows = x.elem_count() / k, n = w.dims()[0];
+    ughip_device* dev = hip_dev(x);
+    const int product = product_for(w, k, rows);
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != 4) bail("linear_norm: expected 4 slices");
+      hip_check(ughip_rms_linear_rows(dev, hip_raw_slice(*vs[0]), hip_raw_slice(*vs[1]), eps, hip_raw_slice(*vs[2]), hip_raw_slice(*vs[3]), rows, n, k, product), "linear_norm");
+    };
+    std::vector<size_t> dims = x.dims();
+    dims.back() = n;
+    return LB::custom(f, {x, alpha, w}, Shape(dims), DType::F32, x.device());
+  }
+
+  LB mlp_stacked(const LB& x, const LB* alpha, float eps, const LB& w_gate_up, const LB& w_down, const LB& residual) const override {
+    const size_t k = x.rank() ? x.dims().back() : 0, inter = w_gate_up.rank() == 2 ? w_gate_up.dims()[0] / 2 : 0;
+    if (!many_f32_rows(x, w_gate_up, 16) || w_down.rank() != 2 || w_down.dtype() != w_gate_up.dtype() || w_down.dims()[1] != inter || inter % 32 != 0 ||
+        w_down.dims()[0] % 8 != 0 || residual.dtype() != DType::F32 || residual.elem_count() != x.elem_count() / k * w_down.dims()[0] ||
+        (alpha && (alpha->dtype() != DType::F32 || alpha->elem_count() != k)) || switch_on(SW_NO_FOLD_EPILOGUES))
+      return Ops::mlp_stacked(x, alpha, eps, w_gate_up, w_down, residual);
+    const size_t rows = x.elem_count() / k, n = w_down.dims()[0];
+    ughip_device* dev = hip_dev(x);
+    // one choice for both products, the one the pieces would make for the first (the second has the longer k)
+    const int product = product_for(w_gate_up, k, rows) == UGHIP_PRODUCT_BF16X3 && product_for(w_down, inter, rows) == UGHIP_PRODUCT_BF16X3 ? UGHIP_PRODUCT_BF16X3
+                                                                                                                                        : UGHIP_PRODUCT_F32;
+    const bool norm = alpha != nullptr;
+    // with the norm folded in, the rows and the residual are usually one buffer: a schedule item names a buffer once
+    const bool same = x.data().get() == residual.data().get();
+    const size_t n_args = 4 + (same ? 0 : 1) + (norm ? 1 : 0);
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != n_args) bail("mlp_stacked: unexpected number of slices");
+      hip_check(ughip_rms_mlp_rows(dev, hip_raw_slice(*vs[0]), norm ? hip_raw_slice(*vs[n_args - 2]) : nullptr, eps, hip_raw_slice(*vs[1]), hip_raw_slice(*vs[2]),
+                                   hip_raw_slice(*vs[same ? 0 : 3]), hip_raw_slice(*vs.back()), rows, n, inter, k, product),
+                "mlp_stacked");
+    };
+    std::vector<LB> args = {x, w_gate_up, w_down};
+    if (!same) args.push_back(residual);
+    if (norm) args.push_back(*alpha);
+    return LB::custom(f, args, residual.shape(), DType::F32, x.device());
+  }
+
   LB attention_step(const LB& qkv, const LB& kcache, const LB& vcache, size_t len, size_t n_heads, float scale, const LB* cos, const LB* sin, const LB* pos,
                     bool interleaved) const override {
     if (qkv.rank() != 3 || qkv.dims()[1] != 1 || kcache.rank() != 4 || kcache.dims() != vcache.dims()) bail("attention_step: expected qkv [b, 1, row] and caches [b, nkv, cap, d]");
@@ -630,6 +674,12 @@ LB Ops::gate_up_stacked(const LB& x, const LB& w_gate_up) const {
 // model.rs:366-372: a projection, then the residual.
 LB Ops::linear_add(const LB& x, const LB& w, const LB& residual) const { return linear(x, w).binary(BinaryOp::Add, residual); }
 
+LB Ops::linear_norm(const LB& x, const LB& alpha, float eps, const LB& w) const { return linear(rms_norm(x, alpha, eps), w); }
+
+LB Ops::mlp_stacked(const LB& x, const LB* alpha, float eps, const LB& w_gate_up, const LB& w_down, const LB& residual) const {
+  return linear_add(gate_up_stacked(alpha ? rms_norm(x, *alpha, eps) : x, w_gate_up), w_down, residual);
+}
+
 std::shared_ptr<WeightSource> synthetic_weights(uint64_t seed, float std, bool round_bf16, float norm_mean, float embed_std) {
   return std::make_shared<SyntheticWeights>(seed, std, round_bf16, norm_mean, embed_std);
 }
@@ -833,15 +883,15 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
     LB vc = ops_->kv_append(cache.prev_v, len, qkv, nullptr, nullptr, nullptr, false, nq + nk, row);
     return finish(ops_->attention_cached(qkv, kc, vc, cache.len, scale, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, 0, row, nh));
   }
-  LB xs = norm_first ? rms_norm(xs_in, l.rms1, eps) : xs_in;
   if (fused_attention_ >= 3 && cache.capacity && l.qkv_stacked.valid()) {
-    // several positions: one product gives q | k | v side by side and everything behind it reads its
-    // column range of the wide rows in place (a preallocated cache implies a head size the kernels take)
+    // several positions: one product (with the norm in front) gives q | k | v side by side and everything behind it reads
+    // its column range of the wide rows in place (a preallocated cache implies a head size the kernels take)
     const size_t len = cache.len;
-    LB qkv = ops_->linear(xs, l.qkv_stacked);
+    LB qkv = norm_first ? ops_->linear_norm(xs_in, l.rms1, eps, l.qkv_stacked) : ops_->linear(xs_in, l.qkv_stacked);
     cache.len = len + seq_len;
     return finish(ops_->attention_steps(qkv, cache.prev_k, cache.prev_v, len, nh, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved));
   }
+  LB xs = norm_first ? rms_norm(xs_in, l.rms1, eps) : xs_in;
   LB q = ops_->linear(xs, l.q_proj);
   LB k = ops_->linear(xs, l.k_proj);
   LB v = ops_->linear(xs, l.v_proj);
@@ -902,9 +952,8 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
 // model.rs:160-168
 LB Model::mlp(const Layer& l, const LB& xs, const LB* residual, bool norm_first) const {
   if (residual && l.gate_up_stacked.valid() && xs.rank() == 3 && xs.dims()[0] * xs.dims()[1] > 1) {
-    // several positions: gate and up in one product, SwiGLU on the two halves of its rows
-    LB x = norm_first ? rms_norm(xs, l.rms2, (float)cfg_.rms_norm_eps) : xs;
-    return ops_->linear_add(ops_->gate_up_stacked(x, l.gate_up_stacked), l.down_proj, *residual);
+    // several positions: gate and up in one product, SwiGLU on the two halves of its rows, the down projection and the residual
+    return ops_->mlp_stacked(xs, norm_first ? &l.rms2 : nullptr, (float)cfg_.rms_norm_eps, l.gate_up_stacked, l.down_proj, *residual);
   }
   if (residual)
     return ops_->linear_add(ops_->gate_up(xs, l.gate_proj, l.up_proj, norm_first ? &l.rms2 : nullptr, (float)cfg_.rms_norm_eps), l.down_proj, *residual);

@@ -80,6 +80,12 @@ struct Ops {
   virtual LB gate_up_stacked(const LB& x, const LB& w_gate_up) const;
   // x w^T + residual
   virtual LB linear_add(const LB& x, const LB& w, const LB& residual) const;
+  // Several positions with more of the layer in one schedule item (the defaults compose the ops above):
+  // rms_norm(x, alpha, eps) w^T -- model.rs:65-78 in front of 206-208 --
+  virtual LB linear_norm(const LB& x, const LB& alpha, float eps, const LB& w) const;
+  // and the whole MLP block of model.rs:160-168 with its residual: gate_up_stacked on x (normalised first when
+  // alpha != nullptr), the down projection, + residual.
+  virtual LB mlp_stacked(const LB& x, const LB* alpha, float eps, const LB& w_gate_up, const LB& w_down, const LB& residual) const;
 
   // One decode position in one launch (devices with packed_projections()): the k and v parts of
   // the packed row qkv [b, 1, (nh + 2 nkv) d] go into row `len` of both caches (k rotated), the q

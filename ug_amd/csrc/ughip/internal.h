@@ -37,6 +37,9 @@ struct ughip_device {
   // Partial rows of single-query attention over a long cache (one per head and key range); same life cycle.
   void* att_ws = nullptr;
   size_t att_ws_bytes = 0;
+  // What lies between the launches of one call on rows (ughip_rms_linear_rows, ughip_rms_mlp_rows); same life cycle.
+  void* rows_ws = nullptr;
+  size_t rows_ws_bytes = 0;
 };
 
 struct ughip_slice {

@@ -420,6 +420,21 @@ static int grow_gemm_ws(ughip_device* dev, size_t bytes) {
   return UGHIP_OK;
 }
 
+// The per-device block for what lies between the launches of one call on rows (normalised rows, the rows between the two
+// products of an MLP block); same life cycle.
+static int grow_rows_ws(ughip_device* dev, size_t bytes) {
+  if (bytes <= dev->rows_ws_bytes) return UGHIP_OK;
+  std::lock_guard<std::mutex> g(dev->mu);
+  UGHIP_HIPCHK(hipStreamSynchronize(dev->stream));
+  if (dev->rows_ws) (void)hipFree(dev->rows_ws);
+  dev->rows_ws = nullptr;
+  dev->rows_ws_bytes = 0;
+  const size_t want = std::max<size_t>(bytes, (size_t)16 << 20);
+  UGHIP_HIPCHK(hipMalloc(&dev->rows_ws, want));
+  dev->rows_ws_bytes = want;
+  return UGHIP_OK;
+}
+
 // Which kernel family a product goes to: decided from shapes, strides, offsets and alignment alone, so that the choice can be
 // asked for without a device (ughip_matmul_plan) and is the same one the launch makes.
 enum Route { ROUTE_GEMV_NT, ROUTE_GEMV_NN, ROUTE_DMA, ROUTE_DMA_F32, ROUTE_TILED, ROUTE_ANY, ROUTE_UNSUPPORTED };
@@ -562,12 +577,8 @@ __device__ __forceinline__ uint16_t bf16_rne(float f) {
   if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);  // NaN stays NaN
   return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
 }
-__global__ void __launch_bounds__(256) split3_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ x3, size_t n4, int k) {
-  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (g >= n4) return;
-  const size_t e = g * 4, row = e / (size_t)k, col = e % (size_t)k;
-  const float4 v = reinterpret_cast<const float4*>(x)[g];
-  const float in[4] = {v.x, v.y, v.z, v.w};
+// Four consecutive elements of a row of k, split, to their places in the row's planes (x3_row: the row's first element).
+__device__ __forceinline__ void split3_store4(const float in[4], uint16_t* __restrict__ x3_row, size_t col) {
   uint16_t hi[4], mid[4], lo[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -581,10 +592,67 @@ __global__ void __launch_bounds__(256) split3_bf16_kernel(const float* __restric
     const float r2 = r1 - __uint_as_float((uint32_t)mid[i] << 16);
     lo[i] = bf16_rne(r2);
   }
-  uint16_t* o = x3 + row * 3 * (size_t)k + (col / 64) * 192 + col % 64;
+  uint16_t* o = x3_row + (col / 64) * 192 + col % 64;
   *reinterpret_cast<ushort4*>(o) = make_ushort4(hi[0], hi[1], hi[2], hi[3]);
   *reinterpret_cast<ushort4*>(o + 64) = make_ushort4(mid[0], mid[1], mid[2], mid[3]);
   *reinterpret_cast<ushort4*>(o + 128) = make_ushort4(lo[0], lo[1], lo[2], lo[3]);
+}
+__global__ void __launch_bounds__(256) split3_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ x3, size_t n4, int k) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n4) return;
+  const size_t e = g * 4, row = e / (size_t)k, col = e % (size_t)k;
+  const float4 v = reinterpret_cast<const float4*>(x)[g];
+  const float in[4] = {v.x, v.y, v.z, v.w};
+  split3_store4(in, x3 + row * 3 * (size_t)k, col);
+}
+
+// RMSNorm of the rows of x [m, k] (model.rs:65-78: x / sqrt(mean(x^2) + eps) * alpha, the division as a multiplication by
+// the reciprocal, like the single-row projections do), one workgroup per row; the row's second pass comes from cache.
+// PLANES: the normalised row goes out as its three bf16 planes (what split3_bf16_kernel would make of it), else as f32.
+template <bool PLANES>
+__global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float* __restrict__ x, const float* __restrict__ alpha, float eps, void* __restrict__ out, int k) {
+  __shared__ float part[4];
+  const size_t row = blockIdx.x;
+  const float4* __restrict__ xr = reinterpret_cast<const float4*>(x + row * (size_t)k);
+  const int k4 = k / 4, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < k4; i += 256) {
+    const float4 v = xr[i];
+    ss += v.x * v.x;
+    ss += v.y * v.y;
+    ss += v.z * v.z;
+    ss += v.w * v.w;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+  if (lane == 0) part[wave] = ss;
+  __syncthreads();
+  ss = (part[0] + part[1]) + (part[2] + part[3]);
+  const float inv = 1.f / sqrtf(ss * (1.f / (float)k) + eps);
+  for (int i = threadIdx.x; i < k4; i += 256) {
+    const float4 v = xr[i], a = reinterpret_cast<const float4*>(alpha)[i];
+    const float y[4] = {v.x * inv * a.x, v.y * inv * a.y, v.z * inv * a.z, v.w * inv * a.w};
+    if (PLANES) split3_store4(y, static_cast<uint16_t*>(out) + row * 3 * (size_t)k, (size_t)i * 4);
+    else reinterpret_cast<float4*>(static_cast<float*>(out) + row * (size_t)k)[i] = make_float4(y[0], y[1], y[2], y[3]);
+  }
+}
+
+// The fold of a stacked gate | up product (gemm_split_reduce with SwiGLU: the slabs added in index order, then
+// silu(gate) * up) whose result goes out as the three bf16 planes of rows of n / 2 elements instead of f32: what the
+// product behind it (down) reads, without the f32 rows in between and the pass that splits them.
+__global__ void __launch_bounds__(256) swiglu_fold_planes_kernel(const float* __restrict__ ws, uint16_t* __restrict__ x3, size_t n4, size_t slab_elems, int nsplit, int n) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n4) return;
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  const size_t half4 = (size_t)n / 8, r = g / half4, j4 = g % half4;
+  const size_t gate = r * ((size_t)n / 4) + j4, up = gate + half4;
+  f32x4 a = reinterpret_cast<const f32x4*>(ws)[gate], b = reinterpret_cast<const f32x4*>(ws)[up];
+  for (int k = 1; k < nsplit; ++k) {
+    a += reinterpret_cast<const f32x4*>(ws + (size_t)k * slab_elems)[gate];
+    b += reinterpret_cast<const f32x4*>(ws + (size_t)k * slab_elems)[up];
+  }
+  const float y[4] = {a.x / (1.f + expf(-a.x)) * b.x, a.y / (1.f + expf(-a.y)) * b.y, a.z / (1.f + expf(-a.z)) * b.z, a.w / (1.f + expf(-a.w)) * b.w};
+  split3_store4(y, x3 + r * 3 * ((size_t)n / 2), j4 * 4);
 }
 
 // Which kernel a product of rows takes: decided from shapes, alignment and the cost models alone, so that ughip_linear_rows_plan
@@ -647,73 +715,172 @@ static const char* dma_planes_tail(GemmEpilogue::Kind kind, bool fold, bool resi
   return kind == GemmEpilogue::SWIGLU ? ",swiglu fold" : kind == GemmEpilogue::ADD ? ",+residual in the fold" : ",fold";
 }
 
-// x [m, k] f32 against a row-major [rows, k] matrix (f32 or bf16) through the tiled kernel, the fold applying `kind`.
-// product == UGHIP_PRODUCT_BF16X3 (bf16 matrix): the rows are split into three bf16 planes first and the product runs on
-// the bf16 matrix pipe over a K of 3 k, every K tile of the matrix meeting the three planes of its columns in turn.
-static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x, const ughip_slice* w, const ughip_slice* residual, ughip_slice* dst, size_t m,
-                       size_t rows, size_t k, GemmEpilogue::Kind kind, int product) {
-  if (!dev || !x || !w || !dst || (kind == GemmEpilogue::ADD && !residual)) return set_error(UGHIP_ERR_INVALID, "%s: null argument", what);
-  if (x->dtype != UGHIP_F32 || dst->dtype != UGHIP_F32 || (residual && residual->dtype != UGHIP_F32) || (w->dtype != UGHIP_F32 && w->dtype != UGHIP_BF16))
-    return set_error(UGHIP_ERR_INVALID, "%s: x, residual and dst are F32, the matrix F32 or BF16 (got x %s, w %s, dst %s)", what, dtype_name(x->dtype),
-                     dtype_name(w->dtype), dtype_name(dst->dtype));
-  if (product != UGHIP_PRODUCT_F32 && product != UGHIP_PRODUCT_BF16X3) return set_error(UGHIP_ERR_INVALID, "%s: unknown product %d", what, product);
-  if (product == UGHIP_PRODUCT_BF16X3 && w->dtype != UGHIP_BF16)
-    return set_error(UGHIP_ERR_INVALID, "%s: the three-term bf16 product needs a BF16 matrix (an F32 one would have to be split as well), got %s", what, dtype_name(w->dtype));
-  if (dst == x || dst == w) return set_error(UGHIP_ERR_INVALID, "%s: dst aliases an operand", what);
-  if (m > 0x7fffffffull || rows > 0x7fffffffull || k > 0x7fffffffull / 3) return set_error(UGHIP_ERR_INVALID, "%s: shape too large", what);
-  const size_t out_cols = kind == GemmEpilogue::SWIGLU ? rows / 2 : rows;
-  if (x->len < m * k || w->len < rows * k || dst->len < m * out_cols || (residual && residual->len < m * rows))
-    return set_error(UGHIP_ERR_BOUNDS, "%s: a buffer is too short for m %zu, n %zu, k %zu", what, m, out_cols, k);
-  if (m == 0 || rows == 0) return UGHIP_OK;
-  const bool x3 = product == UGHIP_PRODUCT_BF16X3;
+// What a product of rows does around itself besides `kind`.
+struct RowsAround {
+  const float* alpha = nullptr;  // the rows are RMS-normalised first (x / sqrt(mean(x^2) + eps) * alpha) ...
+  float eps = 0.f;
+  float* xn = nullptr;                  // ... into these m * k floats, unless the pass that writes the planes does it on its way
+  const uint16_t* planes_in = nullptr;  // three-term product: the planes of x, already made (x is not read)
+  uint16_t* planes_out = nullptr;       // SwiGLU on a route that folds slabs: the result may go here as planes instead of to dst ...
+  bool wrote_planes = false;            // ... and this says whether it did
+};
+
+static MMArgs rows_args(const void* x, const void* w, void* dst, size_t m, size_t rows, size_t k, bool x3) {
   MMArgs p;
   p.M = (int)m, p.N = (int)rows, p.K = (int)(x3 ? 3 * k : k);
   p.a_rs = (long long)(x3 ? 3 * k : k), p.a_cs = 1, p.b_rs = 1, p.b_cs = (long long)k;
   p.a_bs = (long long)(m * (x3 ? 3 * k : k)), p.b_bs = (long long)(rows * k), p.c_bs = (long long)(m * rows);
-  p.a = x->ptr, p.b = w->ptr, p.c = dst->ptr;
+  p.a = x, p.b = w, p.c = dst;
   if (x3) p.b_k_div = 3;
+  return p;
+}
+
+// x [m, k] f32 against a row-major [rows, k] matrix (f32 or bf16) through the tiled kernel, the fold applying `kind`.
+// product == UGHIP_PRODUCT_BF16X3 (bf16 matrix): the rows are split into three bf16 planes first and the product runs on
+// the bf16 matrix pipe over a K of 3 k, every K tile of the matrix meeting the three planes of its columns in turn.
+// Buffers are checked by the callers; x, residual and dst are device pointers to f32.
+static int linear_rows_core(ughip_device* dev, const char* what, const float* x, const ughip_slice* w, const float* residual, float* dst, size_t m, size_t rows,
+                            size_t k, GemmEpilogue::Kind kind, int product, RowsAround* ar) {
+  if (product != UGHIP_PRODUCT_F32 && product != UGHIP_PRODUCT_BF16X3) return set_error(UGHIP_ERR_INVALID, "%s: unknown product %d", what, product);
+  if (product == UGHIP_PRODUCT_BF16X3 && w->dtype != UGHIP_BF16)
+    return set_error(UGHIP_ERR_INVALID, "%s: the three-term bf16 product needs a BF16 matrix (an F32 one would have to be split as well), got %s", what, dtype_name(w->dtype));
+  if (m > 0x7fffffffull || rows > 0x7fffffffull || k > 0x7fffffffull / 3) return set_error(UGHIP_ERR_INVALID, "%s: shape too large", what);
+  const size_t out_cols = kind == GemmEpilogue::SWIGLU ? rows / 2 : rows;
+  if (m == 0 || rows == 0) return UGHIP_OK;
+  const bool x3 = product == UGHIP_PRODUCT_BF16X3;
+  const bool norm = ar && ar->alpha, planes_in = ar && ar->planes_in;
+  if (planes_in && (!x3 || norm)) return set_error(UGHIP_ERR_INVALID, "%s: planes stand for the rows of a three-term product as they are", what);
+  if (norm && (k % 4 != 0 || (reinterpret_cast<uintptr_t>(ar->alpha) & 15))) return set_error(UGHIP_ERR_UNSUPPORTED, "%s: the norm reads 16 bytes at a time (k %zu)", what, k);
+  // (x3: p.a is checked for alignment below with the f32 rows standing in; the planes live in 256-byte aligned scratch blocks)
+  const void* x_stand_in = planes_in ? static_cast<const void*>(ar->planes_in) : static_cast<const void*>(x);
+  MMArgs p = rows_args(x_stand_in, w->ptr, dst, m, rows, k, x3);
   const bool mixed = !x3 && w->dtype == UGHIP_BF16;
   const int dtype = x3 ? UGHIP_BF16 : UGHIP_F32;
-  // (x3: p.a is checked for alignment below with the f32 rows standing in; the planes live in the 256-byte aligned scratch block)
   // an F32 matrix under 2 .. 8 rows is the row-vector kernels' job (ughip_matmul); those do not read a BF16 matrix
   const size_t min_rows = w->dtype == UGHIP_BF16 ? 2 : 9;
   if (m < min_rows || rows % 8 != 0 || (kind == GemmEpilogue::SWIGLU && rows % 16 != 0) || (x3 && k % 64 != 0) || !gemm_tiled_supported(dtype, p, 1, mixed))
     return set_error(UGHIP_ERR_UNSUPPORTED, "%s: built for m >= 9 rows (m >= 2 with a BF16 matrix), k %% 32 == 0 (k %% 64 == 0 for the three-term bf16 product), n %% 8 == 0 and 16-byte aligned buffers (got m %zu, n %zu, k %zu)",
                      what, m, out_cols, k);
   if (int rc = device_activate(dev)) return rc;
-  GemmEpilogue epi{kind, residual ? static_cast<const float*>(residual->ptr) : nullptr};
+  GemmEpilogue epi{kind, residual};
   epi.out_f32 = x3;
-  const RowsRoute route = rows_route(p, dtype, x3, kind, x->ptr, w->ptr, dst->ptr, residual ? residual->ptr : nullptr, m, rows, k, dev->num_cus);
+  const RowsRoute route = rows_route(p, dtype, x3, kind, x_stand_in, w->ptr, dst, residual, m, rows, k, dev->num_cus);
+  const unsigned m_grid = (unsigned)m;
   if (route.kind == RowsRoute::X3_ROWS) {
+    if (planes_in) return set_error(UGHIP_ERR_INVALID, "%s: this product splits its rows itself", what);
+    if (norm) {
+      rms_norm_rows_kernel<false><<<m_grid, 256, 0, dev->stream>>>(x, ar->alpha, ar->eps, ar->xn, (int)k);
+      UGHIP_HIPCHK(hipGetLastError());
+      x = ar->xn;
+    }
     if (int rc = grow_gemm_ws(dev, route.x3.ws_bytes)) return rc;
-    UGHIP_HIPCHK(rows_x3_launch(dev->stream, static_cast<const float*>(x->ptr), w->ptr, static_cast<float*>(dev->gemm_ws), static_cast<float*>(dst->ptr), m, rows, k, route.x3,
-                                kind, epi.residual));
+    UGHIP_HIPCHK(rows_x3_launch(dev->stream, x, w->ptr, static_cast<float*>(dev->gemm_ws), dst, m, rows, k, route.x3, kind, epi.residual));
     return UGHIP_OK;
   }
   const int dma_tile = route.dma_tile, dma_split = route.dma_split;
   const bool dma_fold = dma_tile && (dma_split > 1 || kind == GemmEpilogue::SWIGLU);
   const size_t ws_bytes = dma_tile ? (dma_fold ? ((size_t)dma_split * m * rows * sizeof(float) + 255) & ~(size_t)255 : 0)
                                    : (gemm_tiled_workspace_bytes(dtype, p, 1, &epi) + 255) & ~(size_t)255;
-  const size_t x3_bytes = x3 ? m * 3 * k * sizeof(uint16_t) : 0;
+  const size_t x3_bytes = x3 && !planes_in ? m * 3 * k * sizeof(uint16_t) : 0;
   if (int rc = grow_gemm_ws(dev, ws_bytes + x3_bytes)) return rc;
-  if (x3) {
+  if (planes_in) {
+    p.a = ar->planes_in;
+  } else if (x3) {
     uint16_t* planes = reinterpret_cast<uint16_t*>(static_cast<char*>(dev->gemm_ws) + ws_bytes);
     const size_t n4 = m * k / 4;
-    split3_bf16_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, dev->stream>>>(static_cast<const float*>(x->ptr), planes, n4, (int)k);
+    if (norm) rms_norm_rows_kernel<true><<<m_grid, 256, 0, dev->stream>>>(x, ar->alpha, ar->eps, planes, (int)k);
+    else split3_bf16_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, dev->stream>>>(x, planes, n4, (int)k);
     UGHIP_HIPCHK(hipGetLastError());
     p.a = planes;
+  } else if (norm) {
+    rms_norm_rows_kernel<false><<<m_grid, 256, 0, dev->stream>>>(x, ar->alpha, ar->eps, ar->xn, (int)k);
+    UGHIP_HIPCHK(hipGetLastError());
+    p.a = ar->xn;
   }
   if (dma_tile) {
     if (dma_fold) {
       p.c = dev->gemm_ws;
-      UGHIP_HIPCHK(gemm_dma_launch_planes3(dev->stream, p, dma_tile, dma_split, nullptr, dma_planes_tail(kind, true, false)));
-      UGHIP_HIPCHK(gemm_fold_f32(dev->stream, static_cast<const float*>(dev->gemm_ws), static_cast<float*>(dst->ptr), m, rows, dma_split, kind, epi.residual));
+      const bool to_planes = kind == GemmEpilogue::SWIGLU && ar && ar->planes_out && out_cols % 64 == 0;
+      UGHIP_HIPCHK(gemm_dma_launch_planes3(dev->stream, p, dma_tile, dma_split, nullptr, to_planes ? ",swiglu fold onto planes" : dma_planes_tail(kind, true, false)));
+      if (to_planes) {
+        const size_t elems = m * rows, n4 = elems / 8;
+        swiglu_fold_planes_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, dev->stream>>>(static_cast<const float*>(dev->gemm_ws), ar->planes_out, n4, elems, dma_split, (int)rows);
+        UGHIP_HIPCHK(hipGetLastError());
+        ar->wrote_planes = true;
+      } else {
+        UGHIP_HIPCHK(gemm_fold_f32(dev->stream, static_cast<const float*>(dev->gemm_ws), dst, m, rows, dma_split, kind, epi.residual));
+      }
     } else {
       UGHIP_HIPCHK(gemm_dma_launch_planes3(dev->stream, p, dma_tile, 1, epi.residual, dma_planes_tail(kind, false, epi.residual != nullptr)));
     }
     return UGHIP_OK;
   }
   UGHIP_HIPCHK(gemm_tiled_launch(dev->stream, dtype, p, 1, static_cast<float*>(dev->gemm_ws), mixed, &epi));
+  return UGHIP_OK;
+}
+
+static int linear_rows(ughip_device* dev, const char* what, const ughip_slice* x, const ughip_slice* w, const ughip_slice* residual, ughip_slice* dst, size_t m,
+                       size_t rows, size_t k, GemmEpilogue::Kind kind, int product, const ughip_slice* alpha = nullptr, float eps = 0.f) {
+  if (!dev || !x || !w || !dst || (kind == GemmEpilogue::ADD && !residual)) return set_error(UGHIP_ERR_INVALID, "%s: null argument", what);
+  if (x->dtype != UGHIP_F32 || dst->dtype != UGHIP_F32 || (residual && residual->dtype != UGHIP_F32) || (w->dtype != UGHIP_F32 && w->dtype != UGHIP_BF16) ||
+      (alpha && alpha->dtype != UGHIP_F32))
+    return set_error(UGHIP_ERR_INVALID, "%s: x, residual, alpha and dst are F32, the matrix F32 or BF16 (got x %s, w %s, dst %s)", what, dtype_name(x->dtype),
+                     dtype_name(w->dtype), dtype_name(dst->dtype));
+  if (dst == x || dst == w || dst == alpha) return set_error(UGHIP_ERR_INVALID, "%s: dst aliases an operand", what);
+  if (m > 0x7fffffffull || rows > 0x7fffffffull || k > 0x7fffffffull / 3) return set_error(UGHIP_ERR_INVALID, "%s: shape too large", what);
+  const size_t out_cols = kind == GemmEpilogue::SWIGLU ? rows / 2 : rows;
+  if (x->len < m * k || w->len < rows * k || dst->len < m * out_cols || (residual && residual->len < m * rows) || (alpha && alpha->len < k))
+    return set_error(UGHIP_ERR_BOUNDS, "%s: a buffer is too short for m %zu, n %zu, k %zu", what, m, out_cols, k);
+  RowsAround ar;
+  if (alpha) {
+    if (int rc = device_activate(dev)) return rc;
+    if (int rc = grow_rows_ws(dev, m * k * sizeof(float))) return rc;
+    ar.alpha = static_cast<const float*>(alpha->ptr), ar.eps = eps, ar.xn = static_cast<float*>(dev->rows_ws);
+  }
+  return linear_rows_core(dev, what, static_cast<const float*>(x->ptr), w, residual ? static_cast<const float*>(residual->ptr) : nullptr, static_cast<float*>(dst->ptr), m,
+                          rows, k, kind, product, &ar);
+}
+
+// dst[m, n] = silu(y gate^T) * (y up^T) w_down^T + residual with y = x, or RMSNorm(x) when alpha is given: the two products of
+// an MLP block (model.rs:160-168 between the residual adds of 366-372) with what lies between them kept in the device's own
+// scratch -- as the three bf16 planes the second product reads where both run on planes, else as f32 rows.
+static int mlp_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* alpha, float eps, const ughip_slice* w_gate_up, const ughip_slice* w_down,
+                    const ughip_slice* residual, ughip_slice* dst, size_t m, size_t n, size_t inter, size_t k, int product) {
+  const char* what = "rms_mlp_rows";
+  if (!dev || !x || !w_gate_up || !w_down || !residual || !dst) return set_error(UGHIP_ERR_INVALID, "%s: null argument", what);
+  if (x->dtype != UGHIP_F32 || dst->dtype != UGHIP_F32 || residual->dtype != UGHIP_F32 || (alpha && alpha->dtype != UGHIP_F32) ||
+      (w_gate_up->dtype != UGHIP_F32 && w_gate_up->dtype != UGHIP_BF16) || w_down->dtype != w_gate_up->dtype)
+    return set_error(UGHIP_ERR_INVALID, "%s: x, alpha, residual and dst are F32, the two matrices both F32 or both BF16", what);
+  if (dst == x || dst == alpha || dst == w_gate_up || dst == w_down) return set_error(UGHIP_ERR_INVALID, "%s: dst aliases an operand", what);
+  if (m > 0x7fffffffull || n > 0x7fffffffull || inter > 0x7fffffffull / 3 || k > 0x7fffffffull / 3) return set_error(UGHIP_ERR_INVALID, "%s: shape too large", what);
+  if (x->len < m * k || w_gate_up->len < 2 * inter * k || w_down->len < n * inter || dst->len < m * n || residual->len < m * n || (alpha && alpha->len < k))
+    return set_error(UGHIP_ERR_BOUNDS, "%s: a buffer is too short for m %zu, n %zu, inter %zu, k %zu", what, m, n, inter, k);
+  if (m == 0 || n == 0) return UGHIP_OK;
+  if (inter == 0 || inter % 8 != 0) return set_error(UGHIP_ERR_UNSUPPORTED, "%s: inter %% 8 == 0 (got %zu)", what, inter);
+  // scratch: [normalised rows, f32, if any | what the first product leaves: m * inter elements as f32 (4 bytes) or as planes (6)]
+  const size_t xn_bytes = alpha ? (m * k * sizeof(float) + 255) & ~(size_t)255 : 0;
+  if (int rc = device_activate(dev)) return rc;
+  if (int rc = grow_rows_ws(dev, xn_bytes + m * inter * 6)) return rc;
+  float* h = reinterpret_cast<float*>(static_cast<char*>(dev->rows_ws) + xn_bytes);
+  RowsAround first, second;
+  if (alpha) first.alpha = static_cast<const float*>(alpha->ptr), first.eps = eps, first.xn = static_cast<float*>(dev->rows_ws);
+  const bool x3 = product == UGHIP_PRODUCT_BF16X3;
+  if (x3 && w_down->dtype == UGHIP_BF16 && inter % 64 == 0 && n % 8 == 0 && m >= 2) {
+    // the second product reads planes unless it is one that splits its rows itself
+    const MMArgs pd = rows_args(h, w_down->ptr, dst->ptr, m, n, inter, true);
+    if (gemm_tiled_supported(UGHIP_BF16, pd, 1, false) &&
+        rows_route(pd, UGHIP_BF16, true, GemmEpilogue::ADD, h, w_down->ptr, dst->ptr, residual->ptr, m, n, inter, dev->num_cus).kind != RowsRoute::X3_ROWS)
+      first.planes_out = reinterpret_cast<uint16_t*>(h);
+  }
+  if (int rc = linear_rows_core(dev, what, static_cast<const float*>(x->ptr), w_gate_up, nullptr, h, m, 2 * inter, k, GemmEpilogue::SWIGLU, product, &first)) return rc;
+  char first_kernel[160];
+  snprintf(first_kernel, sizeof first_kernel, "%s", ughip_last_kernel());
+  if (first.wrote_planes) second.planes_in = reinterpret_cast<const uint16_t*>(h);
+  if (int rc = linear_rows_core(dev, what, h, w_down, static_cast<const float*>(residual->ptr), static_cast<float*>(dst->ptr), m, n, inter, GemmEpilogue::ADD, product, &second))
+    return rc;
+  char second_kernel[160];
+  snprintf(second_kernel, sizeof second_kernel, "%s", ughip_last_kernel());
+  note_kernel("%s -> %s", first_kernel, second_kernel);
   return UGHIP_OK;
 }
 
@@ -799,4 +966,15 @@ extern "C" int ughip_linear_swiglu_rows(ughip_device* dev, const ughip_slice* x,
                                         int product) {
   if (n > 0x3fffffffull) return set_error(UGHIP_ERR_INVALID, "linear_swiglu_rows: shape too large");
   return linear_rows(dev, "linear_swiglu_rows", x, w, nullptr, dst, m, 2 * n, k, GemmEpilogue::SWIGLU, product);
+}
+
+extern "C" int ughip_rms_linear_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* alpha, float eps, const ughip_slice* w, ughip_slice* dst, size_t m,
+                                     size_t n, size_t k, int product) {
+  if (!alpha) return set_error(UGHIP_ERR_INVALID, "rms_linear_rows: null argument");
+  return linear_rows(dev, "rms_linear_rows", x, w, nullptr, dst, m, n, k, GemmEpilogue::NONE, product, alpha, eps);
+}
+
+extern "C" int ughip_rms_mlp_rows(ughip_device* dev, const ughip_slice* x, const ughip_slice* alpha, float eps, const ughip_slice* w_gate_up, const ughip_slice* w_down,
+                                  const ughip_slice* residual, ughip_slice* dst, size_t m, size_t n, size_t inter, size_t k, int product) {
+  return mlp_rows(dev, x, alpha, eps, w_gate_up, w_down, residual, dst, m, n, inter, k, product);
 }

@@ -175,6 +175,7 @@ int ughip_device_release(ughip_device* dev) {
   hipStreamSynchronize(dev->stream);
   if (dev->gemm_ws) hipFree(dev->gemm_ws);
   if (dev->att_ws) hipFree(dev->att_ws);
+  if (dev->rows_ws) hipFree(dev->rows_ws);
   for (auto& kv : dev->pool)
     for (void* p : kv.second) hipFree(p);
   for (auto& kv : dev->modules) hipModuleUnload(kv.second.module);
