@@ -2333,7 +2333,8 @@ def test_half_precision_elementwise_and_reduce(hip, dtype):
 
 @pytest.mark.parametrize("t,k,inter,n,product,w_bf16", [(1900, 2048, 5632, 2048, 1, True), (700, 1024, 2816, 1024, 1, True), (300, 512, 1024, 512, 1, True),
                                                         (128, 2048, 5632, 2048, 1, True), (40, 256, 512, 256, 1, True), (50, 256, 512, 264, 0, True),
-                                                        (37, 128, 96, 72, 0, False), (9, 64, 64, 64, 1, True)])
+                                                        (37, 128, 96, 72, 0, False), (9, 64, 64, 64, 1, True), (40, 4096, 64, 64, 1, True), (300, 4160, 128, 64, 1, True),
+                                                        (12, 4160, 64, 64, 0, False)])
 def test_norm_and_mlp_folded_into_the_products_of_rows(hip, t, k, inter, n, product, w_bf16):
     """ughip_rms_linear_rows and ughip_rms_mlp_rows: the RMSNorm in front of a product of rows and the MLP block whole
     (model.rs:65-78, 160-168, 366-372).  Against float64 with the bounds of the pieces; without a norm, bit for bit what

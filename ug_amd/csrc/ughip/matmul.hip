@@ -609,19 +609,39 @@ __global__ void __launch_bounds__(256) split3_bf16_kernel(const float* __restric
 // RMSNorm of the rows of x [m, k] (model.rs:65-78: x / sqrt(mean(x^2) + eps) * alpha, the division as a multiplication by
 // the reciprocal, like the single-row projections do), one workgroup per row; the row's second pass comes from cache.
 // PLANES: the normalised row goes out as its three bf16 planes (what split3_bf16_kernel would make of it), else as f32.
-template <bool PLANES>
+// NV: 16-byte groups a thread keeps of its row between the two passes (k <= 1024 NV; the row and alpha are requested at
+// once, and only the reduction lies between the loads and the stores); 0: any k, the second pass reads the row again.
+template <bool PLANES, int NV>
 __global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float* __restrict__ x, const float* __restrict__ alpha, float eps, void* __restrict__ out, int k) {
   __shared__ float part[4];
   const size_t row = blockIdx.x;
   const float4* __restrict__ xr = reinterpret_cast<const float4*>(x + row * (size_t)k);
+  const float4* __restrict__ ar = reinterpret_cast<const float4*>(alpha);
   const int k4 = k / 4, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float4 v[NV ? NV : 1], a[NV ? NV : 1];
   float ss = 0.f;
-  for (int i = threadIdx.x; i < k4; i += 256) {
-    const float4 v = xr[i];
-    ss += v.x * v.x;
-    ss += v.y * v.y;
-    ss += v.z * v.z;
-    ss += v.w * v.w;
+  if (NV) {
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int i = j * 256 + (int)threadIdx.x;
+      v[j] = i < k4 ? xr[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+      a[j] = i < k4 ? ar[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      ss += v[j].x * v[j].x;
+      ss += v[j].y * v[j].y;
+      ss += v[j].z * v[j].z;
+      ss += v[j].w * v[j].w;
+    }
+  } else {
+    for (int i = threadIdx.x; i < k4; i += 256) {
+      const float4 t = xr[i];
+      ss += t.x * t.x;
+      ss += t.y * t.y;
+      ss += t.z * t.z;
+      ss += t.w * t.w;
+    }
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
@@ -629,12 +649,28 @@ __global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float* __restr
   __syncthreads();
   ss = (part[0] + part[1]) + (part[2] + part[3]);
   const float inv = 1.f / sqrtf(ss * (1.f / (float)k) + eps);
-  for (int i = threadIdx.x; i < k4; i += 256) {
-    const float4 v = xr[i], a = reinterpret_cast<const float4*>(alpha)[i];
-    const float y[4] = {v.x * inv * a.x, v.y * inv * a.y, v.z * inv * a.z, v.w * inv * a.w};
+  auto put = [&](int i, const float4& t, const float4& al) {
+    const float y[4] = {t.x * inv * al.x, t.y * inv * al.y, t.z * inv * al.z, t.w * inv * al.w};
     if (PLANES) split3_store4(y, static_cast<uint16_t*>(out) + row * 3 * (size_t)k, (size_t)i * 4);
     else reinterpret_cast<float4*>(static_cast<float*>(out) + row * (size_t)k)[i] = make_float4(y[0], y[1], y[2], y[3]);
+  };
+  if (NV) {
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int i = j * 256 + (int)threadIdx.x;
+      if (i < k4) put(i, v[j], a[j]);
+    }
+  } else {
+    for (int i = threadIdx.x; i < k4; i += 256) put(i, xr[i], ar[i]);
   }
+}
+template <bool PLANES>
+static hipError_t rms_norm_rows_launch(hipStream_t stream, const float* x, const float* alpha, float eps, void* out, size_t m, size_t k) {
+  const dim3 grid((unsigned)m), block(256);
+  if (k <= 2048) rms_norm_rows_kernel<PLANES, 2><<<grid, block, 0, stream>>>(x, alpha, eps, out, (int)k);
+  else if (k <= 4096) rms_norm_rows_kernel<PLANES, 4><<<grid, block, 0, stream>>>(x, alpha, eps, out, (int)k);
+  else rms_norm_rows_kernel<PLANES, 0><<<grid, block, 0, stream>>>(x, alpha, eps, out, (int)k);
+  return hipGetLastError();
 }
 
 // The fold of a stacked gate | up product (gemm_split_reduce with SwiGLU: the slabs added in index order, then
@@ -765,12 +801,10 @@ static int linear_rows_core(ughip_device* dev, const char* what, const float* x,
   GemmEpilogue epi{kind, residual};
   epi.out_f32 = x3;
   const RowsRoute route = rows_route(p, dtype, x3, kind, x_stand_in, w->ptr, dst, residual, m, rows, k, dev->num_cus);
-  const unsigned m_grid = (unsigned)m;
   if (route.kind == RowsRoute::X3_ROWS) {
     if (planes_in) return set_error(UGHIP_ERR_INVALID, "%s: this product splits its rows itself", what);
     if (norm) {
-      rms_norm_rows_kernel<false><<<m_grid, 256, 0, dev->stream>>>(x, ar->alpha, ar->eps, ar->xn, (int)k);
-      UGHIP_HIPCHK(hipGetLastError());
+      UGHIP_HIPCHK(rms_norm_rows_launch<false>(dev->stream, x, ar->alpha, ar->eps, ar->xn, m, k));
       x = ar->xn;
     }
     if (int rc = grow_gemm_ws(dev, route.x3.ws_bytes)) return rc;
@@ -788,13 +822,12 @@ static int linear_rows_core(ughip_device* dev, const char* what, const float* x,
   } else if (x3) {
     uint16_t* planes = reinterpret_cast<uint16_t*>(static_cast<char*>(dev->gemm_ws) + ws_bytes);
     const size_t n4 = m * k / 4;
-    if (norm) rms_norm_rows_kernel<true><<<m_grid, 256, 0, dev->stream>>>(x, ar->alpha, ar->eps, planes, (int)k);
+    if (norm) UGHIP_HIPCHK(rms_norm_rows_launch<true>(dev->stream, x, ar->alpha, ar->eps, planes, m, k));
     else split3_bf16_kernel<<<(unsigned)((n4 + 255) / 256), 256, 0, dev->stream>>>(x, planes, n4, (int)k);
     UGHIP_HIPCHK(hipGetLastError());
     p.a = planes;
   } else if (norm) {
-    rms_norm_rows_kernel<false><<<m_grid, 256, 0, dev->stream>>>(x, ar->alpha, ar->eps, ar->xn, (int)k);
-    UGHIP_HIPCHK(hipGetLastError());
+    UGHIP_HIPCHK(rms_norm_rows_launch<false>(dev->stream, x, ar->alpha, ar->eps, ar->xn, m, k));
     p.a = ar->xn;
   }
   if (dma_tile) {
