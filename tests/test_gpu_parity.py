@@ -2392,6 +2392,12 @@ def test_norm_and_mlp_folded_into_the_products_of_rows(hip, t, k, inter, n, prod
     sh = hip.slice_from(h_piece.reshape(-1))
     piece, _ = result(lambda d: lib.ughip_linear_add_rows(dev, raw(sh), raw(sd), raw(sr), raw(d), z(t), z(n), z(inter), P), n)
     np.testing.assert_array_equal(got, piece)
+    # the result may take the residual's place
+    d_r = hip.slice_from(np.concatenate([r, np.full(guard, 7.0, np.float32)]))
+    assert lib.ughip_rms_mlp_rows(dev, raw(sx), None, f(0.0), raw(sgu), raw(sd), raw(d_r), raw(d_r), z(t), z(n), z(inter), z(k), P) == 0, lib.ughip_last_error()
+    v = d_r.to_vec()
+    np.testing.assert_array_equal(v[:t * n].reshape(t, n), got)
+    assert np.all(v[t * n:] == 7.0)
 
     # with the norm in front
     ms = np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + eps_n)
