@@ -343,6 +343,31 @@ extern "C" {
         pos: *const UghipSlice,
         interleaved: c_int,
     ) -> c_int;
+    pub fn ughip_attention_cached_linear_add_rows(
+        dev: *mut UghipDevice,
+        q: *const UghipSlice,
+        q_offset: usize,
+        q_row_stride: usize,
+        k: *const UghipSlice,
+        v: *const UghipSlice,
+        b: usize,
+        n_heads: usize,
+        n_kv_heads: usize,
+        t: usize,
+        s: usize,
+        cap: usize,
+        d: usize,
+        scale: f32,
+        cos: *const UghipSlice,
+        sin: *const UghipSlice,
+        pos: *const UghipSlice,
+        interleaved: c_int,
+        w: *const UghipSlice,
+        residual: *const UghipSlice,
+        dst: *mut UghipSlice,
+        n: usize,
+        product: c_int,
+    ) -> c_int;
     pub fn ughip_attention_step(
         dev: *mut UghipDevice,
         qkv: *const UghipSlice,

@@ -364,6 +364,20 @@ int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_off
                            ughip_slice* dst, size_t b, size_t n_heads, size_t n_kv_heads,
                            size_t t, size_t s, size_t cap, size_t d, float scale, const ughip_slice* cos, const ughip_slice* sin,
                            const ughip_slice* pos, int interleaved);
+/* ughip_attention_cached for t >= 2 query positions followed by the output projection and its residual
+ * (model.rs:231-247 and 366-372): dst[b t, n] = attention(...) w^T + residual[b t, n], w a row-major [n, n_heads * d]
+ * matrix stored as F32 or BF16, `product` as for ughip_linear_add_rows, dst may be residual.  The [b t, n_heads * d]
+ * rows between the two stay in the device's scratch; where the kernel that takes the attention is the one on six bf16
+ * terms and the projection reads planes, the attention writes its result as those planes (no f32 rows, no pass that
+ * splits them).  Same results as the two entry points run one after the other. */
+int ughip_attention_cached_linear_add_rows(ughip_device* dev, const ughip_slice* q, size_t q_offset,
+                                           size_t q_row_stride, const ughip_slice* k,
+                                           const ughip_slice* v, size_t b, size_t n_heads,
+                                           size_t n_kv_heads, size_t t, size_t s, size_t cap, size_t d,
+                                           float scale, const ughip_slice* cos, const ughip_slice* sin,
+                                           const ughip_slice* pos, int interleaved, const ughip_slice* w,
+                                           const ughip_slice* residual, ughip_slice* dst, size_t n,
+                                           int product);
 
 /* One decode position in one launch: ughip_kv_append of the k and v parts of a packed q|k|v row
  * (qkv [b, row_stride], parts at q_offset / k_offset / v_offset) into row s_old of both caches,

@@ -2427,3 +2427,65 @@ def test_norm_and_mlp_folded_into_the_products_of_rows(hip, t, k, inter, n, prod
     short = hip.slice_from(alpha[:k - 4].copy())
     assert lib.ughip_rms_linear_rows(dev, raw(sx), raw(short), f(eps_n), raw(sgu), raw(d), z(t), z(rows), z(k), P) != 0
     assert lib.ughip_rms_mlp_rows(dev, raw(sx), raw(short), f(eps_n), raw(sgu), raw(sd), raw(sr), raw(d), z(t), z(n), z(inter), z(k), P) != 0
+
+
+@pytest.mark.parametrize("b,nh,nkv,t,s,cap,d,n,product,w_bf16,with_rope", [
+    (1, 32, 4, 1900, 1900, 2048, 64, 2048, 1, True, True),     # six-term attention writes the projection's planes
+    (1, 8, 2, 300, 420, 512, 64, 512, 1, True, False),         # the same in front of the register-staged kernel on planes
+    (1, 8, 2, 300, 300, 300, 64, 512, 0, True, True),          # six-term attention, f32 rows for the f32 pipe
+    (1, 4, 2, 40, 40, 64, 64, 256, 1, True, True),             # f32 attention kernel, a product that splits its rows itself
+    (2, 4, 4, 33, 50, 64, 32, 128, 0, False, False),
+    (1, 2, 1, 20, 57, 60, 128, 264, 0, True, True),
+    (1, 16, 4, 512, 512, 512, 64, 1024, 1, True, True)])
+def test_attention_followed_by_the_output_projection(hip, tune, b, nh, nkv, t, s, cap, d, n, product, w_bf16, with_rope):
+    """ughip_attention_cached_linear_add_rows against ughip_attention_cached followed by ughip_linear_add_rows: bit for
+    bit (the rows between the two are the same values, kept as f32 or written as the projection's planes by the attention
+    kernel), the residual's place taken, a sentinel behind the result, t = 1 refused."""
+    import ctypes as C
+    print("attention + o", (b, nh, nkv, t, s, cap, d, n, product, w_bf16, with_rope), flush=True)
+    width, m = nh * d, b * t
+    q = rng.normal(191, m * width)
+    k4, v4 = rng.normal(192, b * nkv * cap * d).reshape(b, nkv, cap, d).copy(), rng.normal(193, b * nkv * cap * d).reshape(b, nkv, cap, d).copy()
+    k4[:, :, s:], v4[:, :, s:] = np.nan, np.inf
+    w = rng.normal(194, n * width, 0.05)
+    r = rng.normal(195, m * n)
+    if w_bf16:
+        w = rng.to_bf16_bits(rng.bf16_round(w))
+    scale = float(np.float32(d) ** np.float32(-0.5))
+    lib, dev, z = ug_amd.ughip_lib(), C.c_void_p(hip.raw_hip()), C.c_size_t
+    lib.ughip_attention_cached_linear_add_rows.restype = C.c_int
+    raw = lambda s_: C.c_void_p(s_.raw())
+    sq, sk, sv, sw, sr = hip.slice_from(q), hip.slice_from(k4.ravel()), hip.slice_from(v4.ravel()), hip.slice_from(w), hip.slice_from(r)
+    rope = (None, None, None)
+    keep = []
+    if with_rope:
+        cos, sin = _rope_tables(hip, d, max_pos=s + 8)
+        keep = [hip.slice_from(cos.data_vec()), hip.slice_from(sin.data_vec()), hip.slice_from(np.array([s - t], np.int32))]
+        rope = tuple(raw(x) for x in keep)
+    f, P, guard = C.c_float, C.c_int(product), 64
+
+    def fused(res, dst, tt=t):
+        return lib.ughip_attention_cached_linear_add_rows(dev, raw(sq), z(0), z(0), raw(sk), raw(sv), z(b), z(nh), z(nkv), z(tt), z(s), z(cap), z(d), f(scale), *rope, C.c_int(0),
+                                                          raw(sw), raw(res), raw(dst), z(n), P)
+
+    d_att = hip.allocate_uninit(ug_amd.F32, m * width)
+    assert lib.ughip_attention_cached(dev, raw(sq), z(0), z(0), raw(sk), raw(sv), raw(d_att), z(b), z(nh), z(nkv), z(t), z(s), z(cap), z(d), f(scale), *rope, C.c_int(0)) == 0, lib.ughip_last_error()
+    att_kernel = ug_amd.last_kernel()
+    d_want = hip.allocate_uninit(ug_amd.F32, m * n)
+    assert lib.ughip_linear_add_rows(dev, raw(d_att), raw(sw), raw(sr), raw(d_want), z(m), z(n), z(width), P) == 0, lib.ughip_last_error()
+    want, o_kernel = d_want.to_vec().reshape(m, n), ug_amd.last_kernel()
+    assert np.all(np.isfinite(want))
+    d_got = hip.slice_from(np.full(m * n + guard, 7.0, np.float32))
+    assert fused(sr, d_got) == 0, lib.ughip_last_error()
+    assert ug_amd.last_kernel() == o_kernel, (ug_amd.last_kernel(), o_kernel, att_kernel)
+    v = d_got.to_vec()
+    assert np.all(v[m * n:] == 7.0), "wrote past the end of the result"
+    np.testing.assert_array_equal(v[:m * n].reshape(m, n), want)
+    # the result in the residual's place
+    d_r = hip.slice_from(np.concatenate([r, np.full(guard, 7.0, np.float32)]))
+    assert fused(d_r, d_r) == 0, lib.ughip_last_error()
+    v = d_r.to_vec()
+    np.testing.assert_array_equal(v[:m * n].reshape(m, n), want)
+    assert np.all(v[m * n:] == 7.0)
+    # one position is not this entry point's
+    assert fused(sr, d_got, 1) != 0

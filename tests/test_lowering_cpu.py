@@ -43,6 +43,7 @@ def test_entry_points_refuse_a_null_device_without_touching_the_gpu():
         "ughip_kv_append": (None, None, None, z, z, z, z, z, z, z, z, None, None, None, 0),
         "ughip_kv_append_pair": (None, None, None, None, z, z, z, z, z, z, z, z, z, None, None, None, 0),
         "ughip_attention_cached": (None, None, z, z, None, None, None, z, z, z, C.c_size_t(2), z, z, C.c_size_t(64), f, None, None, None, 0),
+        "ughip_attention_cached_linear_add_rows": (None, None, z, z, None, None, z, z, C.c_size_t(2), C.c_size_t(2), z, z, C.c_size_t(64), f, None, None, None, 0, None, None, None, z, C.c_int(0)),
         "ughip_attention_step": (None, None, z, z, z, z, None, None, None, z, z, z, z, z, z, f, None, None, None, 0),
         "ughip_gemv_multi": (None, None, C.c_size_t(1), None, n3, C.c_size_t(4), None),
         "ughip_rms_gemv_multi": (None, None, None, f, C.c_size_t(1), None, n3, C.c_size_t(4), None),

@@ -506,6 +506,39 @@ struct HipOps : Ops {
     return LB::custom(f, args, Shape({b, t, nq}), qkv.dtype(), qkv.device());
   }
 
+  LB attention_steps_add(const LB& qkv, const LB& kcache, const LB& vcache, size_t len, size_t n_heads, float scale, const LB* cos, const LB* sin, const LB* pos,
+                         bool interleaved, const LB& w_o, const LB& residual) const override {
+    const bool shapes = qkv.rank() == 3 && kcache.rank() == 4 && kcache.dims() == vcache.dims() && w_o.rank() == 2;
+    const size_t b = shapes ? qkv.dims()[0] : 0, t = shapes ? qkv.dims()[1] : 0, row = shapes ? qkv.dims()[2] : 0, nkv = shapes ? kcache.dims()[1] : 0;
+    const size_t cap = shapes ? kcache.dims()[2] : 0, d = shapes ? kcache.dims()[3] : 0, nq = n_heads * d, nk = nkv * d, n = shapes ? w_o.dims()[0] : 0, rows = b * t;
+    // the shapes the two pieces take on this device, else their composition
+    if (!shapes || kcache.dims()[0] != b || row != nq + 2 * nk || len + t > cap || t < 2 || !(d == 32 || d == 64 || d == 128) || qkv.dtype() != DType::F32 ||
+        switch_on(SW_NO_APPEND_PAIR) || switch_on(SW_NO_FOLD_EPILOGUES) || (w_o.dtype() != DType::F32 && w_o.dtype() != DType::BF16) || w_o.dims()[1] != nq ||
+        rows < (w_o.dtype() == DType::BF16 ? 2u : 9u) || nq % 32 != 0 || n % 8 != 0 || residual.dtype() != DType::F32 || residual.elem_count() != rows * n)
+      return Ops::attention_steps_add(qkv, kcache, vcache, len, n_heads, scale, cos, sin, pos, interleaved, w_o, residual);
+    ughip_device* dev = hip_dev(qkv);
+    const bool with_rope = cos != nullptr;
+    const int il = interleaved ? 1 : 0, product = product_for(w_o, nq, rows);
+    auto f = [=](const std::vector<Slice*>& vs) {
+      if (vs.size() != (with_rope ? 9u : 6u)) bail("attention_steps_add: unexpected number of slices");
+      ughip_slice *x = hip_raw_slice(*vs[0]), *kc = hip_raw_slice(*vs[1]), *vc = hip_raw_slice(*vs[2]);
+      const ughip_slice* c = with_rope ? hip_raw_slice(*vs[5]) : nullptr;
+      const ughip_slice* sn = with_rope ? hip_raw_slice(*vs[6]) : nullptr;
+      const ughip_slice* p = with_rope ? hip_raw_slice(*vs[7]) : nullptr;
+      hip_check(ughip_kv_append_pair(dev, kc, vc, x, nq, nq + nk, row, b, nkv, cap, len, t, d, c, sn, p, il), "attention_steps_add");
+      hip_check(ughip_attention_cached_linear_add_rows(dev, x, 0, row, kc, vc, b, n_heads, nkv, t, len + t, cap, d, scale, c, sn, p, il, hip_raw_slice(*vs[3]),
+                                                       hip_raw_slice(*vs[4]), hip_raw_slice(*vs.back()), n, product),
+                "attention_steps_add");
+    };
+    std::vector<LB> args = {qkv, kcache, vcache, w_o, residual};
+    if (with_rope) {
+      args.push_back(*cos);
+      args.push_back(*sin);
+      args.push_back(*pos);
+    }
+    return LB::custom(f, args, residual.shape(), DType::F32, qkv.device());
+  }
+
   bool device_argmax() const override { return true; }
 
   LB argmax_into(const LB& token, const LB& logits, size_t row, const LB& ids, const LB& vals, size_t slot) const override {
@@ -675,6 +708,11 @@ LB Ops::gate_up_stacked(const LB& x, const LB& w_gate_up) const {
 LB Ops::linear_add(const LB& x, const LB& w, const LB& residual) const { return linear(x, w).binary(BinaryOp::Add, residual); }
 
 LB Ops::linear_norm(const LB& x, const LB& alpha, float eps, const LB& w) const { return linear(rms_norm(x, alpha, eps), w); }
+
+LB Ops::attention_steps_add(const LB& qkv, const LB& kcache, const LB& vcache, size_t len, size_t n_heads, float scale, const LB* cos, const LB* sin, const LB* pos,
+                            bool interleaved, const LB& w_o, const LB& residual) const {
+  return linear_add(attention_steps(qkv, kcache, vcache, len, n_heads, scale, cos, sin, pos, interleaved), w_o, residual);
+}
 
 LB Ops::mlp_stacked(const LB& x, const LB* alpha, float eps, const LB& w_gate_up, const LB& w_down, const LB& residual) const {
   return linear_add(gate_up_stacked(alpha ? rms_norm(x, *alpha, eps) : x, w_gate_up), w_down, residual);
@@ -889,7 +927,9 @@ LB Model::attention(const Layer& l, const LB& xs_in, const LB& pos, Cache& cache
     const size_t len = cache.len;
     LB qkv = norm_first ? ops_->linear_norm(xs_in, l.rms1, eps, l.qkv_stacked) : ops_->linear(xs_in, l.qkv_stacked);
     cache.len = len + seq_len;
-    return finish(ops_->attention_steps(qkv, cache.prev_k, cache.prev_v, len, nh, std::pow((float)hd, -0.5f), &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved));
+    const float scale = std::pow((float)hd, -0.5f);
+    if (residual) return ops_->attention_steps_add(qkv, cache.prev_k, cache.prev_v, len, nh, scale, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved, l.o_proj, *residual);
+    return finish(ops_->attention_steps(qkv, cache.prev_k, cache.prev_v, len, nh, scale, &rope_.cos, &rope_.sin, &pos, cfg_.rope_interleaved));
   }
   LB xs = norm_first ? rms_norm(xs_in, l.rms1, eps) : xs_in;
   LB q = ops_->linear(xs, l.q_proj);

@@ -101,6 +101,11 @@ struct Ops {
   virtual LB attention_steps(const LB& qkv, const LB& kcache, const LB& vcache, size_t len, size_t n_heads, float scale, const LB* cos, const LB* sin,
                              const LB* pos, bool interleaved) const;
 
+  // attention_steps followed by the output projection and its residual (model.rs:247 and 366-372): one schedule item on
+  // devices that keep the rows between the two to themselves.  The default composes attention_steps and linear_add.
+  virtual LB attention_steps_add(const LB& qkv, const LB& kcache, const LB& vcache, size_t len, size_t n_heads, float scale, const LB* cos, const LB* sin,
+                                 const LB* pos, bool interleaved, const LB& w_o, const LB& residual) const;
+
   // Greedy step on the device (device_argmax() == true): the index of the largest value of row
   // `row` of logits [b, rows, n] is written into `token` (I32, one element, in place: the result
   // names the same storage) and recorded with the two largest values at ids[slot], vals[2 slot],

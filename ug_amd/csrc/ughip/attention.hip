@@ -13,6 +13,7 @@
 // All reduce in a fixed order (no atomics): results do not change from run to run.
 #include <hip/hip_runtime.h>
 
+#include "bf16_split.h"
 #include "internal.h"
 #include "ughip.h"
 #include "wave_ops.h"
@@ -817,9 +818,11 @@ __device__ __forceinline__ att_f32x16 att_mma_bf16(const att_u32x4& a, const att
 
 // Same work split, statistics, merge and output as attention_prefill_kernel<64, GROUPS>; q is scaled before it is split
 // (scores come out of the MFMAs scaled, and in units of log 2).  planes: what att_planes_kernel wrote for these caches, n_kb blocks per kv head.
+// dst_planes != nullptr: the result goes there as the three bf16 planes of rows of nh * 64 elements (what a product of
+// these rows on the bf16 matrix pipe reads) and dst is not written.
 template <int GROUPS>
 __global__ void __launch_bounds__(256 * GROUPS, 2) attention_prefill_x6_kernel(const float* __restrict__ q, const att_u32x4* __restrict__ planes, float* __restrict__ dst,
-                                                                               int nh, int nkv, int t, int s, int n_kb, size_t q_row_stride, float scale,
+                                                                               uint16_t* __restrict__ dst_planes, int nh, int nkv, int t, int s, int n_kb, size_t q_row_stride, float scale,
                                                                                const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                                                                const int* __restrict__ pos, size_t table_len, int interleaved) {
   constexpr int D = 64, H = D / 2, DB = D / 32;
@@ -1023,13 +1026,16 @@ __global__ void __launch_bounds__(256 * GROUPS, 2) attention_prefill_x6_kernel(c
   }
   l_tot += __shfl_xor(l_tot, 32, 64);
   if (q0 + col < t) {
-    float* orow = dst + ((size_t)b * t + qi) * ((size_t)nh * D) + (size_t)head * D;
+    const size_t row = (size_t)b * t + qi, width = (size_t)nh * D;
+    float* orow = dst + row * width + (size_t)head * D;
 #pragma unroll
     for (int e = 0; e < DB; ++e)
 #pragma unroll
-      for (int a = 0; a < 4; ++a)
-        *reinterpret_cast<float4*>(orow + e * 32 + a * 8 + hh * 4) =
-            make_float4(o[e][a * 4] / l_tot, o[e][a * 4 + 1] / l_tot, o[e][a * 4 + 2] / l_tot, o[e][a * 4 + 3] / l_tot);
+      for (int a = 0; a < 4; ++a) {
+        const float y[4] = {o[e][a * 4] / l_tot, o[e][a * 4 + 1] / l_tot, o[e][a * 4 + 2] / l_tot, o[e][a * 4 + 3] / l_tot};
+        if (dst_planes) split3_store4(y, dst_planes + row * 3 * width, (size_t)head * D + e * 32 + a * 8 + hh * 4);
+        else *reinterpret_cast<float4*>(orow + e * 32 + a * 8 + hh * 4) = make_float4(y[0], y[1], y[2], y[3]);
+      }
   }
 }
 
@@ -1285,10 +1291,13 @@ int ughip_kv_append_pair(ughip_device* dev, ughip_slice* kcache, ughip_slice* vc
   return UGHIP_OK;
 }
 
-int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_offset, size_t q_row_stride, const ughip_slice* k, const ughip_slice* v,
-                           ughip_slice* dst, size_t b, size_t n_heads, size_t n_kv_heads, size_t t, size_t s, size_t cap, size_t d, float scale,
-                           const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos, int interleaved) {
-  if (t == 1) return attention_decode_launch(dev, q, q_offset, q_row_stride, k, v, dst, b, n_heads, n_kv_heads, s, cap, d, scale, cos, sin, pos, interleaved);
+// Several query positions over the caches.  The result goes to `out` [b * t, n_heads * d] as f32, or -- when out_planes is
+// given and the kernel that takes these shapes can write them (*wrote_planes says so) -- to out_planes as the three bf16
+// planes of those rows.  `out` is checked by the caller (b * t * n_heads * d floats, no alias of an input).
+static int attention_prefill_launch(ughip_device* dev, const ughip_slice* q, size_t q_offset, size_t q_row_stride, const ughip_slice* k, const ughip_slice* v, float* out,
+                                    uint16_t* out_planes, bool* wrote_planes, size_t b, size_t n_heads, size_t n_kv_heads, size_t t, size_t s, size_t cap, size_t d,
+                                    float scale, const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos, int interleaved) {
+  if (wrote_planes) *wrote_planes = false;
   if (!dev) return set_error(UGHIP_ERR_INVALID, "null device");
   const bool rope = cos || sin || pos;
   if (rope)
@@ -1305,8 +1314,6 @@ int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_off
   if (int rc = check_f32(q, b ? q_offset + (b * t - 1) * q_row_stride + n_heads * d : 0, "attention_cached q")) return rc;
   if (int rc = check_f32(k, b * n_kv_heads * cap * d, "attention_cached k")) return rc;
   if (int rc = check_f32(v, b * n_kv_heads * cap * d, "attention_cached v")) return rc;
-  if (int rc = check_f32(dst, b * t * n_heads * d, "attention_cached dst")) return rc;
-  if (dst == q || dst == k || dst == v) return set_error(UGHIP_ERR_INVALID, "attention_cached: dst aliases an input");
   if (b * n_heads == 0) return UGHIP_OK;
   if (b * n_heads > 65535 || s > 0x7fffffffull || cap > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "attention_cached: shape too large");
   if (int rc = device_activate(dev)) return rc;
@@ -1318,7 +1325,7 @@ int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_off
   const float* qp = static_cast<const float*>(q->ptr) + q_offset;
   const float* kp = static_cast<const float*>(k->ptr);
   const float* vp = static_cast<const float*>(v->ptr);
-  float* op = static_cast<float*>(dst->ptr);
+  float* op = out;
   const int inh = (int)n_heads, inkv = (int)n_kv_heads, it = (int)t, is = (int)s;
   // Two query blocks per workgroup of 8 waves (equal work under the causal mask) once one block per
   // workgroup would give every CU two workgroups anyway; d = 128 needs the whole register file for 4 waves.
@@ -1343,10 +1350,11 @@ int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_off
     att_planes_kernel<<<dim3((unsigned)n_kb, (unsigned)bkv), 256, 0, dev->stream>>>(kp, vp, planes, is, cap);
     UGHIP_HIPCHK(hipGetLastError());
     if (pair)
-      attention_prefill_x6_kernel<2><<<paired, 512, 0, dev->stream>>>(qp, planes, op, inh, inkv, it, is, (int)n_kb, q_row_stride, scale, cp, sp, pp, tl, interleaved);
+      attention_prefill_x6_kernel<2><<<paired, 512, 0, dev->stream>>>(qp, planes, op, out_planes, inh, inkv, it, is, (int)n_kb, q_row_stride, scale, cp, sp, pp, tl, interleaved);
     else
-      attention_prefill_x6_kernel<1><<<single, 256, 0, dev->stream>>>(qp, planes, op, inh, inkv, it, is, (int)n_kb, q_row_stride, scale, cp, sp, pp, tl, interleaved);
+      attention_prefill_x6_kernel<1><<<single, 256, 0, dev->stream>>>(qp, planes, op, out_planes, inh, inkv, it, is, (int)n_kb, q_row_stride, scale, cp, sp, pp, tl, interleaved);
     UGHIP_HIPCHK(hipGetLastError());
+    if (wrote_planes) *wrote_planes = out_planes != nullptr;
     return UGHIP_OK;
   }
   if (d == 32 && pair) go(attention_prefill_kernel<32, 2>, 32, 2, paired);
@@ -1357,6 +1365,44 @@ int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_off
   UGHIP_HIPCHK(err);
   UGHIP_HIPCHK(hipGetLastError());
   return UGHIP_OK;
+}
+
+int ughip_attention_cached(ughip_device* dev, const ughip_slice* q, size_t q_offset, size_t q_row_stride, const ughip_slice* k, const ughip_slice* v,
+                           ughip_slice* dst, size_t b, size_t n_heads, size_t n_kv_heads, size_t t, size_t s, size_t cap, size_t d, float scale,
+                           const ughip_slice* cos, const ughip_slice* sin, const ughip_slice* pos, int interleaved) {
+  if (t == 1) return attention_decode_launch(dev, q, q_offset, q_row_stride, k, v, dst, b, n_heads, n_kv_heads, s, cap, d, scale, cos, sin, pos, interleaved);
+  if (int rc = check_f32(dst, b * t * n_heads * d, "attention_cached dst")) return rc;
+  if (dst == q || dst == k || dst == v) return set_error(UGHIP_ERR_INVALID, "attention_cached: dst aliases an input");
+  return attention_prefill_launch(dev, q, q_offset, q_row_stride, k, v, static_cast<float*>(dst->ptr), nullptr, nullptr, b, n_heads, n_kv_heads, t, s, cap, d, scale, cos, sin,
+                                  pos, interleaved);
+}
+
+int ughip_attention_cached_linear_add_rows(ughip_device* dev, const ughip_slice* q, size_t q_offset, size_t q_row_stride, const ughip_slice* k, const ughip_slice* v,
+                                           size_t b, size_t n_heads, size_t n_kv_heads, size_t t, size_t s, size_t cap, size_t d, float scale, const ughip_slice* cos,
+                                           const ughip_slice* sin, const ughip_slice* pos, int interleaved, const ughip_slice* w, const ughip_slice* residual,
+                                           ughip_slice* dst, size_t n, int product) {
+  const char* what = "attention_cached_linear_add_rows";
+  if (!dev || !w || !residual || !dst) return set_error(UGHIP_ERR_INVALID, "%s: null argument", what);
+  if (t < 2) return set_error(UGHIP_ERR_UNSUPPORTED, "%s: built for several query positions (one position: ughip_attention_step and ughip_gemv_add)", what);
+  const size_t m = b * t, width = n_heads * d;
+  if (w->dtype != UGHIP_F32 && w->dtype != UGHIP_BF16) return set_error(UGHIP_ERR_INVALID, "%s: the matrix is F32 or BF16, got %s", what, dtype_name(w->dtype));
+  if (int rc = check_f32(residual, m * n, "attention_cached_linear_add_rows residual")) return rc;
+  if (int rc = check_f32(dst, m * n, "attention_cached_linear_add_rows dst")) return rc;
+  if (w->len < n * width) return set_error(UGHIP_ERR_BOUNDS, "%s: the matrix has %zu elements, [%zu, %zu] needs %zu", what, w->len, n, width, n * width);
+  if (dst == q || dst == k || dst == v || dst == w) return set_error(UGHIP_ERR_INVALID, "%s: dst aliases an input", what);
+  if (m == 0 || width == 0 || n == 0) return UGHIP_OK;
+  if (m > 0x7fffffffull || width > 0x7fffffffull / 3) return set_error(UGHIP_ERR_INVALID, "%s: shape too large", what);
+  if (int rc = device_activate(dev)) return rc;
+  // the rows between the two: f32 (4 bytes an element) or planes (6)
+  void* rows = nullptr;
+  if (int rc = rows_scratch(dev, m * width * 6, &rows)) return rc;
+  const bool want_planes = rows_add_product_reads_planes(dev, w, rows, residual->ptr, dst->ptr, m, n, width, product);
+  bool wrote_planes = false;
+  if (int rc = attention_prefill_launch(dev, q, q_offset, q_row_stride, k, v, static_cast<float*>(rows), want_planes ? static_cast<uint16_t*>(rows) : nullptr, &wrote_planes, b,
+                                        n_heads, n_kv_heads, t, s, cap, d, scale, cos, sin, pos, interleaved))
+    return rc;
+  return rows_add_product_from(dev, what, static_cast<const float*>(rows), wrote_planes ? static_cast<const uint16_t*>(rows) : nullptr, w,
+                               static_cast<const float*>(residual->ptr), static_cast<float*>(dst->ptr), m, n, width, product);
 }
 
 }  // extern "C"

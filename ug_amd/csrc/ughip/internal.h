@@ -57,6 +57,13 @@ int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3
 void note_kernel(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 int device_activate(ughip_device* d);
 int matmul_scratch_setup(ughip_device* dev);  // matmul.hip
+// For entry points of other files that end in a projection with its residual (matmul.hip): the device's block for what lies
+// between their launches, grown to `bytes`; whether dst[m, n] = x w^T + residual would read x as three bf16 planes from
+// memory; and that product on f32 rows x, or on `planes` when they were written already (x is then only a stand-in).
+int rows_scratch(ughip_device* dev, size_t bytes, void** out);
+bool rows_add_product_reads_planes(ughip_device* dev, const ughip_slice* w, const void* x, const void* residual, const void* dst, size_t m, size_t n, size_t k, int product);
+int rows_add_product_from(ughip_device* dev, const char* what, const float* x, const uint16_t* planes, const ughip_slice* w, const float* residual, float* dst, size_t m,
+                          size_t n, size_t k, int product);
 const char* dtype_name(int dt);
 
 // Tuning switches (tile / split / kernel-family overrides for measurements and tests).  The table is filled once per

@@ -8,6 +8,7 @@
 #include <cstdlib>
 #include <mutex>
 
+#include "bf16_split.h"
 #include "gemm.h"
 #include "internal.h"
 #include "ughip.h"
@@ -568,35 +569,6 @@ extern "C" int ughip_matmul_noalloc(ughip_device* dev, ughip_slice* dst, const u
   return matmul_impl(dev, dst, lhs, rhs, b, m, n, k, rank, lhs_dims, lhs_strides, lhs_offset, rhs_dims, rhs_strides, rhs_offset, true);
 }
 
-// x = hi + mid + lo with every term a bf16 (round to nearest even of what the terms before left): 24 mantissa bits in
-// three pieces, so |x - (hi + mid + lo)| <= 2^-25 |x|.  x3 row r holds, for every 64 columns c0 .. c0 + 63 of x, the
-// three planes side by side: [hi(c0..) | mid(c0..) | lo(c0..)], i.e. K tile t of x3 is plane t % 3 of K tile t / 3 of x,
-// and the three of them meet the same K tile of the matrix one after the other.
-__device__ __forceinline__ uint16_t bf16_rne(float f) {
-  const uint32_t x = __float_as_uint(f);
-  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);  // NaN stays NaN
-  return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
-}
-// Four consecutive elements of a row of k, split, to their places in the row's planes (x3_row: the row's first element).
-__device__ __forceinline__ void split3_store4(const float in[4], uint16_t* __restrict__ x3_row, size_t col) {
-  uint16_t hi[4], mid[4], lo[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    hi[i] = bf16_rne(in[i]);
-    const float h = __uint_as_float((uint32_t)hi[i] << 16);
-    // an infinity (given, or reached when |x| rounds up past the largest bf16) or a NaN is all in the first term: the
-    // remainders would be inf - inf, and the product has to give what the f32 pipe gives for such an x
-    const bool fin = (hi[i] & 0x7f80) != 0x7f80;
-    const float r1 = fin ? in[i] - h : 0.f;  // exact: hi shares the leading bits of x
-    mid[i] = bf16_rne(r1);
-    const float r2 = r1 - __uint_as_float((uint32_t)mid[i] << 16);
-    lo[i] = bf16_rne(r2);
-  }
-  uint16_t* o = x3_row + (col / 64) * 192 + col % 64;
-  *reinterpret_cast<ushort4*>(o) = make_ushort4(hi[0], hi[1], hi[2], hi[3]);
-  *reinterpret_cast<ushort4*>(o + 64) = make_ushort4(mid[0], mid[1], mid[2], mid[3]);
-  *reinterpret_cast<ushort4*>(o + 128) = make_ushort4(lo[0], lo[1], lo[2], lo[3]);
-}
 __global__ void __launch_bounds__(256) split3_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ x3, size_t n4, int k) {
   const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (g >= n4) return;
@@ -1011,3 +983,28 @@ extern "C" int ughip_rms_mlp_rows(ughip_device* dev, const ughip_slice* x, const
                                   const ughip_slice* residual, ughip_slice* dst, size_t m, size_t n, size_t inter, size_t k, int product) {
   return mlp_rows(dev, x, alpha, eps, w_gate_up, w_down, residual, dst, m, n, inter, k, product);
 }
+
+namespace ughip {
+
+int rows_scratch(ughip_device* dev, size_t bytes, void** out) {
+  if (int rc = grow_rows_ws(dev, bytes)) return rc;
+  *out = dev->rows_ws;
+  return UGHIP_OK;
+}
+
+bool rows_add_product_reads_planes(ughip_device* dev, const ughip_slice* w, const void* x, const void* residual, const void* dst, size_t m, size_t n, size_t k, int product) {
+  if (product != UGHIP_PRODUCT_BF16X3 || !w || w->dtype != UGHIP_BF16 || k % 64 != 0 || n % 8 != 0 || m < 2 || m > 0x7fffffffull || n > 0x7fffffffull || k > 0x7fffffffull / 3)
+    return false;
+  const MMArgs p = rows_args(x, w->ptr, const_cast<void*>(dst), m, n, k, true);
+  return gemm_tiled_supported(UGHIP_BF16, p, 1, false) &&
+         rows_route(p, UGHIP_BF16, true, GemmEpilogue::ADD, x, w->ptr, dst, residual, m, n, k, dev->num_cus).kind != RowsRoute::X3_ROWS;
+}
+
+int rows_add_product_from(ughip_device* dev, const char* what, const float* x, const uint16_t* planes, const ughip_slice* w, const float* residual, float* dst, size_t m,
+                          size_t n, size_t k, int product) {
+  RowsAround ar;
+  ar.planes_in = planes;
+  return linear_rows_core(dev, what, x, w, residual, dst, m, n, k, GemmEpilogue::ADD, product, &ar);
+}
+
+}  // namespace ughip
