@@ -2489,3 +2489,86 @@ def test_attention_followed_by_the_output_projection(hip, tune, b, nh, nkv, t, s
     assert np.all(v[m * n:] == 7.0)
     # one position is not this entry point's
     assert fused(sr, d_got, 1) != 0
+
+
+@pytest.mark.parametrize("x3", [False, True])
+@pytest.mark.parametrize("t,length,hidden,inter,nh,nkv,bf16", [(300, 0, 512, 1024, 8, 2, True), (40, 7, 256, 512, 4, 2, True), (12, 0, 128, 256, 2, 1, False), (2, 3, 256, 512, 4, 4, True)])
+def test_layer_hooks_with_neighbours_folded_in(hip, x3, t, length, hidden, inter, nh, nkv, bf16):
+    """Ops::linear_norm, Ops::attention_steps_add and Ops::mlp_stacked on the HIP device (one schedule item each) against
+    the hooks they fold together on the same device -- bit for bit where no norm is folded in, a few ulps with it (the
+    norm's sum of squares is added in another order) -- and against the same layer in float64."""
+    if x3 and not bf16:
+        pytest.skip("three bf16 terms need bf16 matrices")
+    print("layer hooks", (x3, t, length, hidden, inter, nh, nkv, bf16), flush=True)
+    ops = ug_amd.LlamaOps.hip(bf16x3=x3)
+    d = hidden // nh
+    nq, nk = nh * d, nkv * d
+    row, cap = nq + 2 * nk, length + t + 5
+    x = rng.normal(201, t * hidden)
+    alpha = (1.0 + rng.normal(202, hidden, 0.1)).astype(np.float32)
+    wqkv, wo = rng.normal(203, row * hidden, 0.05), rng.normal(204, hidden * nq, 0.05)
+    wgu, wd = rng.normal(205, 2 * inter * hidden, 0.05), rng.normal(206, hidden * inter, 0.05)
+    k0, v0 = rng.normal(207, nkv * cap * d), rng.normal(208, nkv * cap * d)
+    if bf16:
+        wqkv, wo, wgu, wd = (rng.bf16_round(w) for w in (wqkv, wo, wgu, wd))
+    scale, eps_n = float(np.float32(d) ** np.float32(-0.5)), 1e-5
+
+    def mat(w, shape, dev):
+        return LB.copy(rng.to_bf16_bits(w), shape, dev) if bf16 and dev is hip else LB.copy(w, shape, dev)
+
+    def chain(o, dev, folded):
+        xs = LB.copy(x, (1, t, hidden), dev)
+        al = LB.copy(alpha, (hidden,), dev)
+        kc, vc = LB.copy(k0, (1, nkv, cap, d), dev), LB.copy(v0, (1, nkv, cap, d), dev)
+        kc.realize()
+        vc.realize()
+        cos, sin = _rope_tables(dev, d, max_pos=cap + 8)
+        pos = LB.copy(np.array([length], np.int32), (1, 1), dev)
+        Wqkv, Wo, Wgu, Wd = mat(wqkv, (row, hidden), dev), mat(wo, (hidden, nq), dev), mat(wgu, (2 * inter, hidden), dev), mat(wd, (hidden, inter), dev)
+        if folded:
+            qkv = o.linear_norm(xs, al, eps_n, Wqkv)
+            h = o.attention_steps_add(qkv, kc, vc, length, nh, scale, Wo, xs, cos, sin, pos, False)
+            out = o.mlp_stacked(h, Wgu, Wd, h, al, eps_n)
+            plain = o.mlp_stacked(xs, Wgu, Wd, xs)
+        else:
+            qkv = o.linear(ug_amd.llama.rms_norm(xs, al, eps_n), Wqkv)
+            h = o.linear_add(o.attention_steps(qkv, kc, vc, length, nh, scale, cos, sin, pos, False), Wo, xs)
+            out = o.linear_add(o.gate_up_stacked(ug_amd.llama.rms_norm(h, al, eps_n), Wgu), Wd, h)
+            plain = o.linear_add(o.gate_up_stacked(xs, Wgu), Wd, xs)
+        return [v.data_vec().reshape(t, -1) for v in (qkv, h, out, plain)] + [kc.data_vec(), vc.data_vec()]
+
+    def truth():
+        """the same layer in float64 (model.rs:65-78, 160-168, 203-248, 366-372)"""
+        x64, a64 = x.reshape(t, hidden).astype(np.float64), alpha.astype(np.float64)
+        norm = lambda v: v / np.sqrt((v * v).mean(axis=1, keepdims=True) + eps_n) * a64
+        W = lambda w, shape: w.reshape(shape).astype(np.float64)
+        qkv = norm(x64) @ W(wqkv, (row, hidden)).T
+        cos, sin = _rope_tables(hip, d, max_pos=cap + 8)
+        cv, sv = cos.data_vec(), sin.data_vec()
+        q = np.asarray(_rope_rows_f64(qkv[:, :nq].reshape(1, t, nh, d), cv, sv, length, False))
+        kn = np.asarray(_rope_rows_f64(qkv[:, nq:nq + nk].reshape(1, t, nkv, d), cv, sv, length, False))
+        vn = qkv[:, nq + nk:].reshape(1, t, nkv, d)
+        K, V = k0.reshape(1, nkv, cap, d).astype(np.float64), v0.reshape(1, nkv, cap, d).astype(np.float64)
+        K[:, :, length:length + t], V[:, :, length:length + t] = kn.transpose(0, 2, 1, 3), vn.transpose(0, 2, 1, 3)
+        s_ = length + t
+        att = _attention_truth(q.transpose(0, 2, 1, 3), K[:, :, :s_], V[:, :, :s_], s_, t, scale, nh // nkv).transpose(0, 2, 1, 3).reshape(t, nq)
+        h = att @ W(wo, (hidden, nq)).T + x64
+
+        def mlp(v, y):
+            gu = y @ W(wgu, (2 * inter, hidden)).T
+            g, u = gu[:, :inter], gu[:, inter:]
+            return (g / (1.0 + np.exp(-g)) * u) @ W(wd, (hidden, inter)).T + v
+
+        return [qkv, h, mlp(h, norm(h)), mlp(x64, x64)]
+
+    got = chain(ops, hip, True)
+    pieces = chain(ops, hip, False)
+    want = truth()
+    np.testing.assert_array_equal(got[3], pieces[3])          # no norm: the same terms in the same order
+    for g, p_ in zip(got[4:], pieces[4:]):                    # the caches hold rows of the normalised product
+        assert np.max(np.abs(g - p_)) <= 2e-5 * max(1.0, float(np.abs(p_).max()))
+    for g, p_, w_, name in zip(got[:3], pieces[:3], want[:3], ("qkv", "attention + o", "mlp")):
+        scale_ = max(1.0, float(np.abs(w_).max()))
+        assert np.max(np.abs(g - p_)) <= 2e-5 * scale_, (name, float(np.max(np.abs(g - p_))))
+        assert np.max(np.abs(g - w_)) <= 2e-4 * scale_, (name, float(np.max(np.abs(g - w_))))
+    assert np.max(np.abs(got[3] - want[3])) <= 2e-4 * max(1.0, float(np.abs(want[3]).max()))

@@ -772,6 +772,27 @@ class LlamaOps(_Handle):
                       _p(cos.h) if rope else None, _p(sin.h) if rope else None, _p(pos.h) if rope else None, int(interleaved))
         lb._keep += [kcache, vcache] + ([cos, sin, pos] if rope else [])
         return lb
+
+    def attention_steps_add(self, qkv, kcache, vcache, length, n_heads, scale, w_o, residual, cos=None, sin=None, pos=None, interleaved=False):
+        """attention_steps followed by the output projection and its residual -> [b, t, n]."""
+        rope = cos is not None
+        lb = self._op("ugh_llama_attention_steps_add", qkv, _p(kcache.h), _p(vcache.h), C.c_size_t(length), C.c_size_t(n_heads), C.c_float(scale),
+                      _p(cos.h) if rope else None, _p(sin.h) if rope else None, _p(pos.h) if rope else None, int(interleaved), _p(w_o.h), _p(residual.h))
+        lb._keep += [kcache, vcache, w_o, residual] + ([cos, sin, pos] if rope else [])
+        return lb
+
+    def linear_norm(self, x, alpha, eps, w):
+        """rms_norm(x, alpha, eps) w^T."""
+        lb = self._op("ugh_llama_linear_norm", x, _p(alpha.h), C.c_float(eps), _p(w.h))
+        lb._keep += [alpha, w]
+        return lb
+
+    def mlp_stacked(self, x, w_gate_up, w_down, residual, alpha=None, eps=0.0):
+        """(silu(y gate^T) * (y up^T)) w_down^T + residual with y = x, or rms_norm(x, alpha, eps) when alpha is given."""
+        lb = self._op("ugh_llama_mlp_stacked", x, _p(alpha.h) if alpha is not None else None, C.c_float(eps), _p(w_gate_up.h), _p(w_down.h), _p(residual.h))
+        lb._keep += [w_gate_up, w_down, residual] + ([alpha] if alpha is not None else [])
+        return lb
+
     def device_argmax(self):
         return bool(host_lib().ugh_llama_device_argmax(_p(self.h)))
 

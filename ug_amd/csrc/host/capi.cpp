@@ -719,6 +719,19 @@ int ugh_llama_attention_steps(void* ops, void* qkv, void* kcache, void* vcache, 
     else *out = box(ops_of(ops).attention_steps(lb_of(qkv), lb_of(kcache), lb_of(vcache), len, n_heads, scale, nullptr, nullptr, nullptr, false));
   });
 }
+int ugh_llama_attention_steps_add(void* ops, void* qkv, void* kcache, void* vcache, size_t len, size_t n_heads, float scale, void* cos, void* sin, void* pos,
+                                  int interleaved, void* w_o, void* residual, void** out) {
+  return guard([&] {
+    *out = box(ops_of(ops).attention_steps_add(lb_of(qkv), lb_of(kcache), lb_of(vcache), len, n_heads, scale, cos ? &lb_of(cos) : nullptr, cos ? &lb_of(sin) : nullptr,
+                                               cos ? &lb_of(pos) : nullptr, cos && interleaved != 0, lb_of(w_o), lb_of(residual)));
+  });
+}
+int ugh_llama_linear_norm(void* ops, void* x, void* alpha, float eps, void* w, void** out) {
+  return guard([&] { *out = box(ops_of(ops).linear_norm(lb_of(x), lb_of(alpha), eps, lb_of(w))); });
+}
+int ugh_llama_mlp_stacked(void* ops, void* x, void* alpha, float eps, void* w_gate_up, void* w_down, void* residual, void** out) {
+  return guard([&] { *out = box(ops_of(ops).mlp_stacked(lb_of(x), alpha ? &lb_of(alpha) : nullptr, eps, lb_of(w_gate_up), lb_of(w_down), lb_of(residual))); });
+}
 int ugh_llama_device_argmax(void* ops) { return ops_of(ops).device_argmax() ? 1 : 0; }
 int ugh_llama_argmax_into(void* ops, void* token, void* logits, size_t row, void* ids, void* vals, size_t slot, void** out) {
   return guard([&] { *out = box(ops_of(ops).argmax_into(lb_of(token), lb_of(logits), row, lb_of(ids), lb_of(vals), slot)); });
