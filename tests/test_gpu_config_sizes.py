@@ -125,6 +125,48 @@ def test_matmul_f32_one_wave_per_simd_random_shapes(hip, tune):
 
 
 @pytest.mark.parametrize("rhs_nk", [False, True], ids=["NN", "NT"])
+@pytest.mark.parametrize("bmnk", [
+    (8, 1024, 1024, 1024),   # config 3
+    (1, 300, 264, 192),      # ragged M and N, three k tiles of 64: 18 K tiles in the loop
+    (2, 517, 768, 256),
+    (1, 1000, 2048, 512),
+    (3, 129, 136, 64),       # one k tile: the loop is the six terms
+    (1, 2048, 2048, 2048),
+])
+def test_matmul_f32_as_six_bf16_terms(hip, tune, bmnk, rhs_nk):
+    """UGHIP_MATMUL_X6=1: an f32 product of contiguous operands runs on the bf16 matrix pipe -- both operands split into three
+    bf16 terms (24 mantissa bits), six of the nine term products accumulated in f32 (the three left out stay below 2^-24 of
+    the product).  Against float64 within the k eps bound of the f32 product and within a tenth of it of the f32 pipe's
+    own result; small integers exactly; an operand against the identity bit for bit (all 24 bits survive both splits);
+    without the switch the f32 pipe takes the product."""
+    b, m, n, k = bmnk
+    a = rng.uniform_pm1(31, b * m * k).reshape(b, m, k)
+    w = rng.uniform_pm1(32, b * k * n).reshape(b, k, n)
+    plain, kernel0 = _matmul(hip, F32, a, w, rhs_nk)
+    assert "6 terms" not in kernel0, kernel0
+    tune.setenv("UGHIP_MATMUL_X6", "1")
+    got, kernel = _matmul(hip, F32, a, w, rhs_nk)
+    print("f32 as six bf16 terms", bmnk, "NT" if rhs_nk else "NN", kernel, flush=True)
+    assert kernel.startswith(f"gemm_dma4<bf16,{'NT' if rhs_nk else 'NN'},") and "6 terms of 3 x 3 planes,f32 out" in kernel, kernel
+    exact, mag = _f64_product(a, w)
+    err = np.abs(got - exact)
+    assert np.all(err <= k * EPS32 * mag + 1e-12), float(err.max())
+    # the terms left out and the f32 sums: a few roundings of the sum of magnitudes, whatever k
+    assert np.all(err <= (8 + 2 * np.sqrt(k)) * EPS32 * mag + 1e-12), float((err / (EPS32 * mag + 1e-30)).max())
+    assert np.all(np.abs(got - plain) <= 0.1 * k * EPS32 * mag + (8 + 2 * np.sqrt(k)) * EPS32 * mag + 1e-12)
+    # small integers: every term product and every partial sum is exact
+    ai, wi = np.floor(a * 8).astype(np.float32), np.floor(w * 8).astype(np.float32)
+    goti, _ = _matmul(hip, F32, ai, wi, rhs_nk)
+    np.testing.assert_array_equal(goti, _f64_product(ai, wi)[0].astype(np.float32))
+    # all 24 bits of an operand survive: against the identity (k == n) the lhs comes back bit for bit
+    if k == n and b == 1:
+        full = ((np.float32(1.0) + (np.arange(m * k, dtype=np.float32) % 8388607) * np.float32(2.0 ** -23)) * rng.normal(33, m * k)).astype(np.float32).reshape(1, m, k)
+        eye = np.eye(k, dtype=np.float32).reshape(1, k, k)
+        back, _ = _matmul(hip, F32, full, eye, rhs_nk)
+        np.testing.assert_array_equal(back, full)
+
+
+@pytest.mark.parametrize("rhs_nk", [False, True], ids=["NN", "NT"])
 def test_config3_bmm_bf16(hip, rhs_nk):
     """bf16 8 x 1024^3 (RNE-rounded copies of the f32 operands): no reference result exists (cpu_runtime.rs:345-356
     refuses BF16), so the expectation is the exact product of the rounded operands, f32 accumulation (k eps sum|a||b|)

@@ -15,21 +15,24 @@ __device__ __forceinline__ uint16_t bf16_rne(float f) {
   if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);  // NaN stays NaN
   return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
 }
+// hi + mid + lo of one value
+__device__ __forceinline__ void split3(float x, uint16_t& hi, uint16_t& mid, uint16_t& lo) {
+  hi = bf16_rne(x);
+  const float h = __uint_as_float((uint32_t)hi << 16);
+  // an infinity (given, or reached when |x| rounds up past the largest bf16) or a NaN is all in the first term: the
+  // remainders would be inf - inf, and the product has to give what the f32 pipe gives for such an x
+  const bool fin = (hi & 0x7f80) != 0x7f80;
+  const float r1 = fin ? x - h : 0.f;  // exact: hi shares the leading bits of x
+  mid = bf16_rne(r1);
+  const float r2 = r1 - __uint_as_float((uint32_t)mid << 16);
+  lo = bf16_rne(r2);
+}
+
 // Four consecutive elements of a row of k, split, to their places in the row's planes (x3_row: the row's first element).
 __device__ __forceinline__ void split3_store4(const float in[4], uint16_t* __restrict__ x3_row, size_t col) {
   uint16_t hi[4], mid[4], lo[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    hi[i] = bf16_rne(in[i]);
-    const float h = __uint_as_float((uint32_t)hi[i] << 16);
-    // an infinity (given, or reached when |x| rounds up past the largest bf16) or a NaN is all in the first term: the
-    // remainders would be inf - inf, and the product has to give what the f32 pipe gives for such an x
-    const bool fin = (hi[i] & 0x7f80) != 0x7f80;
-    const float r1 = fin ? in[i] - h : 0.f;  // exact: hi shares the leading bits of x
-    mid[i] = bf16_rne(r1);
-    const float r2 = r1 - __uint_as_float((uint32_t)mid[i] << 16);
-    lo[i] = bf16_rne(r2);
-  }
+  for (int i = 0; i < 4; ++i) split3(in[i], hi[i], mid[i], lo[i]);
   uint16_t* o = x3_row + (col / 64) * 192 + col % 64;
   *reinterpret_cast<ushort4*>(o) = make_ushort4(hi[0], hi[1], hi[2], hi[3]);
   *reinterpret_cast<ushort4*>(o + 64) = make_ushort4(mid[0], mid[1], mid[2], mid[3]);

@@ -55,6 +55,11 @@ int gemm_dma_pick(int dtype, const MMArgs& p, size_t batch);
 // divides the K tiles, into a multiple of 3 and at least 4 each): workgroups share a tile's K range and leave nsplit
 // slabs [M, N] in p.c (scratch), for gemm_fold_f32 to add up.
 hipError_t gemm_dma_launch_planes3(hipStream_t stream, const MMArgs& p, int tile, int nsplit, const float* residual, const char* note_tail);
+// f32 operands as three bf16 planes each (rows of 3 k elements, the planes of every 64 elements of k side by side; p.K = 6 k):
+// the product as six bf16 terms with an f32 result, on either rhs layout.
+bool gemm_dma_planes6_supported(const MMArgs& p, size_t batch, int tile);
+void gemm_dma_planes6_name(const MMArgs& p, int tile, char* out, size_t out_len);
+hipError_t gemm_dma_launch_planes6(hipStream_t stream, const MMArgs& p, size_t batch, int tile);
 bool gemm_dma_planes3_split_ok(const MMArgs& p, int nsplit);
 // c = fold of nsplit f32 slabs [m, n] in slab order, then the epilogue: NONE, ADD (+ residual[m, n]) or SWIGLU
 // (c[m, n / 2] = silu(sum[:, :n / 2]) * sum[:, n / 2:]); n % 8 == 0.

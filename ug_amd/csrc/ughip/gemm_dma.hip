@@ -92,9 +92,13 @@ __device__ __forceinline__ int kn_byte(int k, int n) {
 // F32OUT: the result leaves as f32 straight from the accumulators (+ residual when given) instead of as T through LDS.
 // BDIV > 1 ([n, k]-major rhs): K tile t of the lhs meets K tile t / BDIV of the rhs -- an lhs that holds BDIV planes of every
 // 64 columns side by side (a row split into bf16 terms) against one matrix, whose tile then comes from cache for the other planes.
+// BDIV == 6 (either rhs layout): both operands hold three planes (hi, mid, lo: planes 0, 1, 2) of every 64 elements of k side
+// by side, and K tile t of the loop is term t % 6 of k tile t / 6 of an f32 product taken as six bf16 ones -- (hi, lo),
+// (lo, hi), (mid, mid), (hi, mid), (mid, hi), (hi, hi), the small ones first; (mid, lo), (lo, mid) and (lo, lo) stay below
+// 2^-24 of the product and are left out.
 template <typename T, int BM, int BN, bool B_KN, bool TWO, bool F32OUT = false, int BDIV = 1>
 __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tiles_n, const float* __restrict__ residual) {
-  static_assert(BDIV == 1 || !B_KN, "planes of the lhs against an [n, k]-major rhs only");
+  static_assert(BDIV == 1 || BDIV == 6 || !B_KN, "planes of the lhs alone: against an [n, k]-major rhs only");
   extern __shared__ u32x4 lds[];
   constexpr int NI = BM / 32, NJ = BN / 32;            // 16-row and 16-column fragments per wave
   constexpr int NM = NI * NJ;                          // MFMAs per k32 step
@@ -154,10 +158,27 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
     }
   }
   const long long a_step = BK * 2, b_step = B_KN ? (long long)BK * ldb * 2 : BK * 2;
+  // which K tile of the lhs and of the rhs in memory the loop's K tile `tile` reads (scalar arithmetic)
+  auto a_tile = [&](int tile) -> int {
+    if constexpr (BDIV == 6) {
+      const int g = tile / 6, r = tile - 6 * g;
+      return 3 * g + ((0x010120 >> (4 * r)) & 3);  // planes 0, 2, 1, 0, 1, 0
+    } else {
+      return tile;
+    }
+  };
+  auto b_tile = [&](int tile) -> int {
+    if constexpr (BDIV == 6) {
+      const int g = tile / 6, r = tile - 6 * g;
+      return 3 * g + ((0x001102 >> (4 * r)) & 3);  // planes 2, 0, 1, 1, 0, 0
+    } else {
+      return tile / BDIV;
+    }
+  };
   auto dma = [&](int tile, int idx) {  // idx: compile-time after unrolling
     const unsigned st = lds_addr + (tile & 1) * STAGE_BYTES;
-    if (idx < NDA) dma16(Ab + tile * a_step, voff[idx], st + (idx * 4 + wave) * 1024);
-    else dma16(Bb + (tile / BDIV) * b_step, voff[idx], st + A_BYTES + ((idx - NDA) * 4 + wave) * 1024);
+    if (idx < NDA) dma16(Ab + a_tile(tile) * a_step, voff[idx], st + (idx * 4 + wave) * 1024);
+    else dma16(Bb + b_tile(tile) * b_step, voff[idx], st + A_BYTES + ((idx - NDA) * 4 + wave) * 1024);
   };
   auto dma_m0 = [&](int tile, int idx) {
     const unsigned in_stage = lds_addr + (idx < NDA ? (idx * 4 + wave) * 1024 : A_BYTES + ((idx - NDA) * 4 + wave) * 1024);  // loop invariant
@@ -167,8 +188,8 @@ __global__ void __launch_bounds__(256) gemm_dma4(MMArgs p, int tiles_m, int tile
     __builtin_amdgcn_sched_barrier(0);
   };
   auto dma_go = [&](int tile, int idx) {
-    if (idx < NDA) dma16_go(Ab + tile * a_step, voff[idx]);
-    else dma16_go(Bb + (tile / BDIV) * b_step, voff[idx]);
+    if (idx < NDA) dma16_go(Ab + a_tile(tile) * a_step, voff[idx]);
+    else dma16_go(Bb + b_tile(tile) * b_step, voff[idx]);
   };
 
   floatx4 acc[NI][NJ];
@@ -542,6 +563,28 @@ hipError_t gemm_dma_launch_planes3(hipStream_t stream, const MMArgs& p, int tile
   if (tile == 256) return launch<__bf16, 256, 256, false, true, 3>(stream, q, (size_t)nsplit, residual);
   if (tile == 128) return launch<__bf16, 256, 128, false, true, 3>(stream, q, (size_t)nsplit, residual);
   return launch<__bf16, 128, 128, false, true, 3>(stream, q, (size_t)nsplit, residual);
+}
+
+
+// Both operands as three bf16 planes per 64 elements of k (p.K = 6 k, rows of 3 k elements), f32 result: see BDIV == 6.
+bool gemm_dma_planes6_supported(const MMArgs& p, size_t batch, int tile) { return p.K % (6 * BK) == 0 && gemm_dma_supported(UGHIP_BF16, p, batch, tile); }
+
+void gemm_dma_planes6_name(const MMArgs& p, int tile, char* out, size_t out_len) {
+  int bm = 0, bn = 0;
+  tile_dims(tile, &bm, &bn);
+  const bool nn = p.b_cs == 1 && p.b_rs != 1;
+  snprintf(out, out_len, "gemm_dma4<bf16,%s,%dx%d,256t,6 terms of 3 x 3 planes,f32 out>", nn ? "NN" : "NT", bm, bn);
+}
+
+hipError_t gemm_dma_launch_planes6(hipStream_t stream, const MMArgs& p, size_t batch, int tile) {
+  if (!gemm_dma_planes6_supported(p, batch, tile)) return hipErrorInvalidValue;
+  char name[112];
+  gemm_dma_planes6_name(p, tile, name, sizeof name);
+  note_kernel("%s", name);
+  const bool nn = p.b_cs == 1 && p.b_rs != 1;
+  if (tile == 256) return nn ? launch<__bf16, 256, 256, true, true, 6>(stream, p, batch) : launch<__bf16, 256, 256, false, true, 6>(stream, p, batch);
+  if (tile == 128) return nn ? launch<__bf16, 256, 128, true, true, 6>(stream, p, batch) : launch<__bf16, 256, 128, false, true, 6>(stream, p, batch);
+  return nn ? launch<__bf16, 128, 128, true, true, 6>(stream, p, batch) : launch<__bf16, 128, 128, false, true, 6>(stream, p, batch);
 }
 
 }  // namespace ughip

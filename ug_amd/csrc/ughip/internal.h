@@ -88,6 +88,7 @@ enum TuneKey {
   TUNE_NO_NT_STORES,        // (set at all) generated elementwise kernels store through the cache
   TUNE_SOFTMAX_STREAM,      // ughip_softmax_rows: 0 never takes the resident wave-per-row kernel, n > 0 forces it onto n workgroups
   TUNE_ATT_X6,              // attention over several query positions, head size 64: 0 keeps the f32 products, 1 takes six bf16 terms for any count
+  TUNE_MATMUL_X6,           // f32 products of ughip_matmul: 1 takes those of contiguous operands with k % 64 == 0, n % 8 == 0 as six bf16 terms on the bf16 matrix pipe
   TUNE_COUNT
 };
 bool tune_get(TuneKey k, long long* value);  // false: the switch is not set

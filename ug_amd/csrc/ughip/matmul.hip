@@ -438,8 +438,42 @@ static int grow_rows_ws(ughip_device* dev, size_t bytes) {
 
 // Which kernel family a product goes to: decided from shapes, strides, offsets and alignment alone, so that the choice can be
 // asked for without a device (ughip_matmul_plan) and is the same one the launch makes.
-enum Route { ROUTE_GEMV_NT, ROUTE_GEMV_NN, ROUTE_DMA, ROUTE_DMA_F32, ROUTE_TILED, ROUTE_ANY, ROUTE_UNSUPPORTED };
-static Route matmul_route(int dtype, bool mixed, const MMArgs& p, size_t b, size_t lhs_offset, size_t rhs_offset, int* dma_tile) {
+enum Route { ROUTE_GEMV_NT, ROUTE_GEMV_NN, ROUTE_DMA, ROUTE_DMA_F32, ROUTE_X6, ROUTE_TILED, ROUTE_ANY, ROUTE_UNSUPPORTED };
+
+__global__ void split3_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ x3, size_t n4, int k);     // defined with the products of rows below
+__global__ void split3_kn_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ x3, size_t n4, int n);
+
+// An f32 product as six bf16 terms (UGHIP_MATMUL_X6=1; never the default: the f32 product's accuracy, not its bits): the
+// problem as the 16-bit kernel sees it once both operands are split into three bf16 planes per 64 elements of k -- rows of
+// 3 k elements, a loop over 6 k -- and the tile it takes it with (0: not this product's route).  Contiguous operands, either
+// rhs layout, k % 64 == 0, n % 8 == 0.  The pointers of the result are stand-ins until the planes exist.
+static int matmul_x6_plan(const MMArgs& p, size_t b, size_t lhs_offset, size_t rhs_offset, MMArgs* out) {
+  long long on = 0;
+  if (!tune_get(TUNE_MATMUL_X6, &on) || !on) return 0;
+  const long long m = p.M, n = p.N, k = p.K;
+  if (m < 9 || k % 64 != 0 || n % 8 != 0 || k > 0x7fffffffll / 6) return 0;
+  if (p.a_cs != 1 || p.a_rs != k || (b > 1 && p.a_bs != m * k) || lhs_offset % 4 != 0 || rhs_offset % 4 != 0) return 0;
+  const bool nn = p.b_cs == 1 && p.b_rs == n && n != 1, nt = p.b_rs == 1 && p.b_cs == k;
+  if (nn == nt || (b > 1 && p.b_bs != n * k)) return 0;
+  if ((reinterpret_cast<uintptr_t>(p.a) | reinterpret_cast<uintptr_t>(p.b) | reinterpret_cast<uintptr_t>(p.c)) & 15) return 0;
+  MMArgs q = p;
+  q.K = (int)(6 * k);
+  q.a_rs = 3 * k, q.a_cs = 1, q.a_bs = m * 3 * k;
+  if (nn) q.b_rs = n, q.b_cs = 1;
+  else q.b_rs = 1, q.b_cs = 3 * k;
+  q.b_bs = n * 3 * k;
+  q.a = q.b = reinterpret_cast<const void*>(uintptr_t(1) << 20);
+  int best = 0;
+  double best_us = 0;
+  for (int tile : {256, 128, 64}) {
+    if (!gemm_dma_planes6_supported(q, b, tile)) continue;
+    const double us = gemm_dma_cost_us(q, b, tile);
+    if (!best || us < best_us * 0.97) best = tile, best_us = us;
+  }
+  if (best && out) *out = q;
+  return best;
+}
+static Route matmul_route(int dtype, bool mixed, const MMArgs& p, size_t b, size_t lhs_offset, size_t rhs_offset, int* dma_tile, bool allow_x6 = true) {
   const size_t m = (size_t)p.M, n = (size_t)p.N, k = (size_t)p.K;
   const bool f32 = dtype == UGHIP_F32;
   const size_t vec = f32 ? 4 : 8;
@@ -457,6 +491,11 @@ static Route matmul_route(int dtype, bool mixed, const MMArgs& p, size_t b, size
     *dma_tile = bn;
     return ROUTE_DMA;
   }
+  if (f32 && !mixed && allow_x6)
+    if (const int tile = matmul_x6_plan(p, b, lhs_offset, rhs_offset, nullptr)) {
+      *dma_tile = tile;
+      return ROUTE_X6;
+    }
   if (f32 && !mixed && gemm_dma_f32_pick(p, b)) return ROUTE_DMA_F32;
   return gemm_tiled_supported(dtype, p, b, mixed) ? ROUTE_TILED : ROUTE_ANY;
 }
@@ -503,7 +542,7 @@ static int matmul_impl(ughip_device* dev, ughip_slice* dst, const ughip_slice* l
   const bool f32 = dst->dtype == UGHIP_F32;
   hipStream_t st = dev->stream;
   int dma_tile = 0;
-  const Route route = matmul_route(dst->dtype, mixed, p, b, lhs_offset, rhs_offset, &dma_tile);
+  const Route route = matmul_route(dst->dtype, mixed, p, b, lhs_offset, rhs_offset, &dma_tile, !no_alloc);
   const bool gemv_nt_ok = route == ROUTE_GEMV_NT, gemv_nn_ok = route == ROUTE_GEMV_NN;
   if (route == ROUTE_UNSUPPORTED)
     return set_error(UGHIP_ERR_UNSUPPORTED,
@@ -527,6 +566,22 @@ static int matmul_impl(ughip_device* dev, ughip_slice* dst, const ughip_slice* l
     return UGHIP_OK;
   } else if (route == ROUTE_DMA_F32) {
     UGHIP_HIPCHK(gemm_dma_f32_launch(st, p, b));
+    return UGHIP_OK;
+  } else if (route == ROUTE_X6) {
+    MMArgs q;
+    if (matmul_x6_plan(p, b, lhs_offset, rhs_offset, &q) != dma_tile) return set_error(UGHIP_ERR_HIP, "matmul: the six-term plan changed between its two readings");
+    // [planes of the lhs | planes of the rhs] in the scratch block, 6 bytes an element
+    const size_t a_elems = b * m * k, b_elems = b * n * k, a_bytes = (a_elems * 6 + 255) & ~(size_t)255;
+    if (int rc = grow_gemm_ws(dev, a_bytes + b_elems * 6)) return rc;
+    uint16_t* ap = static_cast<uint16_t*>(dev->gemm_ws);
+    uint16_t* bp = reinterpret_cast<uint16_t*>(static_cast<char*>(dev->gemm_ws) + a_bytes);
+    split3_bf16_kernel<<<(unsigned)((a_elems / 4 + 255) / 256), 256, 0, st>>>(static_cast<const float*>(p.a), ap, a_elems / 4, (int)k);
+    UGHIP_HIPCHK(hipGetLastError());
+    if (q.b_cs == 1) split3_kn_bf16_kernel<<<(unsigned)((b_elems / 4 + 255) / 256), 256, 0, st>>>(static_cast<const float*>(p.b), bp, b_elems / 4, (int)n);
+    else split3_bf16_kernel<<<(unsigned)((b_elems / 4 + 255) / 256), 256, 0, st>>>(static_cast<const float*>(p.b), bp, b_elems / 4, (int)k);
+    UGHIP_HIPCHK(hipGetLastError());
+    q.a = ap, q.b = bp, q.c = dst->ptr;
+    UGHIP_HIPCHK(gemm_dma_launch_planes6(st, q, b, dma_tile));
     return UGHIP_OK;
   } else if (route == ROUTE_TILED) {
     const size_t ws_bytes = gemm_tiled_workspace_bytes(dst->dtype, p, b);
@@ -581,6 +636,24 @@ __global__ void __launch_bounds__(256) split3_bf16_kernel(const float* __restric
 // RMSNorm of the rows of x [m, k] (model.rs:65-78: x / sqrt(mean(x^2) + eps) * alpha, the division as a multiplication by
 // the reciprocal, like the single-row projections do), one workgroup per row; the row's second pass comes from cache.
 // PLANES: the normalised row goes out as its three bf16 planes (what split3_bf16_kernel would make of it), else as f32.
+// The same split for an operand stored [k, n] (k % 64 == 0): the planes of rows kk .. kk + 63 are rows 3 kk .. of the result,
+// 64 rows of first terms, then 64 of second, then 64 of third ones; rows counts all rows of all batch elements (each a
+// multiple of 64), n4 groups of 4 elements.
+__global__ void __launch_bounds__(256) split3_kn_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ x3, size_t n4, int n) {
+  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (g >= n4) return;
+  const size_t e = g * 4, row = e / (size_t)n, col = e % (size_t)n;
+  const float4 v = reinterpret_cast<const float4*>(x)[g];
+  const float in[4] = {v.x, v.y, v.z, v.w};
+  uint16_t hi[4], mid[4], lo[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) split3(in[i], hi[i], mid[i], lo[i]);
+  uint16_t* o = x3 + ((row / 64) * 192 + row % 64) * (size_t)n + col;
+  *reinterpret_cast<ushort4*>(o) = make_ushort4(hi[0], hi[1], hi[2], hi[3]);
+  *reinterpret_cast<ushort4*>(o + 64 * (size_t)n) = make_ushort4(mid[0], mid[1], mid[2], mid[3]);
+  *reinterpret_cast<ushort4*>(o + 128 * (size_t)n) = make_ushort4(lo[0], lo[1], lo[2], lo[3]);
+}
+
 // NV: 16-byte groups a thread keeps of its row between the two passes (k <= 1024 NV; the row and alpha are requested at
 // once, and only the reduction lies between the loads and the stores); 0: any k, the second pass reads the row again.
 template <bool PLANES, int NV>
@@ -912,6 +985,12 @@ extern "C" int ughip_matmul_plan(int dtype, int rhs_dtype, size_t b, size_t m, s
     case ROUTE_GEMV_NN: snprintf(buf, buf_len, "gemv_nn<f32>"); break;
     case ROUTE_DMA: gemm_dma_name(dtype, p, tile, buf, buf_len); break;
     case ROUTE_DMA_F32: gemm_dma_f32_name(p, buf, buf_len); break;
+    case ROUTE_X6: {
+      MMArgs q;
+      matmul_x6_plan(p, b, 0, 0, &q);
+      gemm_dma_planes6_name(q, tile, buf, buf_len);
+      break;
+    }
     case ROUTE_TILED: gemm_tiled_name(dtype, p, b, mixed, nullptr, buf, buf_len); break;
     default: snprintf(buf, buf_len, "gemm_any<%s>", tn); break;
   }

@@ -93,7 +93,7 @@ static size_t size_class(size_t bytes) {
 namespace ughip {
 namespace {
 const char* const kTuneNames[TUNE_COUNT] = {"GEMM_SHAPE", "GEMM_SPLIT", "GEMM_4WAVES", "GEMV_KS",        "GEMV_ROWS",   "GEMV_BF16_ROWS",
-                                            "X3_DMA",     "X3_SPLIT", "X3_ROWS",   "ATT_SPLIT",   "NO_PARAMETRIC",  "NO_NT_LOADS", "GRID_REDUCE_BLOCKS", "GRID_REDUCE_THREADS", "NO_NT_STORES", "SOFTMAX_STREAM", "ATT_X6"};
+                                            "X3_DMA",     "X3_SPLIT", "X3_ROWS",   "ATT_SPLIT",   "NO_PARAMETRIC",  "NO_NT_LOADS", "GRID_REDUCE_BLOCKS", "GRID_REDUCE_THREADS", "NO_NT_STORES", "SOFTMAX_STREAM", "ATT_X6", "MATMUL_X6"};
 constexpr long long kTuneUnset = INT64_MIN;
 std::atomic<long long> g_tune[TUNE_COUNT];
 std::once_flag g_tune_once;
