@@ -577,6 +577,35 @@ def bmm(dev, steps, warmup):
     _, ms = timed_hot(dev, cs.run, steps, warmup)
     tf = flop * steps / (ms * 1e-3) / 1e12
     out["bmm_f32_8x1024^3"] = {"TFLOP/s": round(tf, 2), "frac_mfma_f32": round(tf / MFMA_F32_PEAK_TF, 4), "us": round(ms * 1e3 / steps, 1), "kernel": kernel, "verified": chk}
+    # the same product, and a large one, as six bf16 terms on the bf16 matrix pipe (UGHIP_MATMUL_X6=1, opt-in: the f32
+    # product's accuracy, not its bits): the rate is that of the f32 product it stands for, frac_mfma_bf16 counts 6 x the flops
+    with ug_amd.tuning(MATMUL_X6=1):
+        cs.run()
+        chk = check_product_rows("bmm_f32_x6", mm.data_vec().reshape(b, m, m), a.reshape(b, m, m), w.reshape(b, m, m), m, False)
+        kernel = ug_amd.last_kernel()
+        _, ms = timed_hot(dev, cs.run, steps, warmup)
+    tf = flop * steps / (ms * 1e-3) / 1e12
+    out["bmm_f32_8x1024^3_six_bf16_terms"] = {"TFLOP/s_f32_equivalent": round(tf, 2), "times_the_f32_matrix_peak": round(tf / MFMA_F32_PEAK_TF, 3), "frac_mfma_bf16": round(6 * tf / MFMA_BF16_PEAK_TF, 4),
+                                              "us": round(ms * 1e3 / steps, 1), "kernel": kernel, "verified": chk}
+    m4 = 4096
+    a4, w4 = rng.uniform_pm1(4, m4 * m4), rng.uniform_pm1(5, m4 * m4)
+    mm4 = LB.copy(a4, (1, m4, m4), dev).matmul(LB.copy(w4, (1, m4, m4), dev))
+    cs4 = Schedule.create_one(mm4).compile()
+    for key, sw_ in (("mm_f32_nn_4096^3", {}), ("mm_f32_nn_4096^3_six_bf16_terms", {"MATMUL_X6": 1})):
+        with ug_amd.tuning(**sw_):
+            cs4.run()
+            chk = check_product_rows(key, mm4.data_vec().reshape(1, m4, m4), a4.reshape(1, m4, m4), w4.reshape(1, m4, m4), m4, False)
+            kernel = ug_amd.last_kernel()
+            _, ms = timed_hot(dev, cs4.run, max(5, steps // 4), 2)
+        tf = 2.0 * m4 ** 3 * max(5, steps // 4) / (ms * 1e-3) / 1e12
+        row = {"us": round(ms * 1e3 / max(5, steps // 4), 1), "kernel": kernel, "verified": chk}
+        row["TFLOP/s_f32_equivalent" if sw_ else "TFLOP/s"] = round(tf, 2)
+        if sw_:
+            row["times_the_f32_matrix_peak"], row["frac_mfma_bf16"] = round(tf / MFMA_F32_PEAK_TF, 3), round(6 * tf / MFMA_BF16_PEAK_TF, 4)
+        else:
+            row["frac_mfma_f32"] = round(tf / MFMA_F32_PEAK_TF, 4)
+        out[key] = row
+    del mm4, cs4
     ab, wb = rng.bf16_round(a), rng.bf16_round(w)
     sa, sw = dev.slice_from(rng.to_bf16_bits(a)), dev.slice_from(rng.to_bf16_bits(w))
     dst = dev.allocate_uninit(ug_amd.BF16, b * m * m)
@@ -982,6 +1011,9 @@ def config_summary(line):
     take("softmax_custom_4096x4096", "softmax_custom_4096x4096", ("us_per_softmax", "GB/s", "frac_hbm"))
     take("softmax_custom_32768x4096_1GiB", "softmax_custom_32768x4096", ("us", "GB/s", "frac_hbm"))
     take("c3_bmm_f32_8x1024^3", "bmm_f32_8x1024^3", ("TFLOP/s", "frac_mfma_f32", "us", "kernel"))
+    take("c3_bmm_f32_8x1024^3_six_bf16_terms", "bmm_f32_8x1024^3_six_bf16_terms", ("TFLOP/s_f32_equivalent", "times_the_f32_matrix_peak", "frac_mfma_bf16", "us", "kernel"))
+    for key in ("mm_f32_nn_4096^3", "mm_f32_nn_4096^3_six_bf16_terms"):
+        take(key, key, ("TFLOP/s", "TFLOP/s_f32_equivalent", "frac_mfma_f32", "times_the_f32_matrix_peak", "frac_mfma_bf16", "us"))
     take("c3_bmm_bf16_8x1024^3", "bmm_bf16_8x1024^3", ("TFLOP/s", "frac_mfma_bf16", "us", "kernel"))
     if "c3_bmm_bf16_8x1024^3" in out and "bound_us" in ex.get("bmm_bf16_8x1024^3", {}):
         out["c3_bmm_bf16_8x1024^3"]["bound_us"] = ex["bmm_bf16_8x1024^3"]["bound_us"]["sum"]

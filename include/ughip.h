@@ -243,7 +243,12 @@ int ughip_rtc_check(const char* source, const char* arch, size_t* code_size);
  * ug-core/src/safetensors.rs:120-271).  The rhs is widened on its way into LDS, so the result is
  * bit for bit that of the F32 product on the widened values.  Built for an [n, k]-major rhs
  * (strides (1, k)) with k % 32 == 0; other layouts are UGHIP_ERR_UNSUPPORTED (convert the rhs
- * with ughip_convert first). */
+ * with ughip_convert first).
+ * With the tuning switch MATMUL_X6 set to 1 (ughip_set_tuning, or UGHIP_MATMUL_X6=1 in the environment), an F32 product of
+ * contiguous operands with k % 64 == 0, n % 8 == 0 and m >= 9 runs on the bf16 matrix pipe: both operands are split into
+ * three bf16 terms each (x = hi + mid + lo exactly) in a scratch block of the device (6 bytes per operand element), and six
+ * of the nine term products -- everything above 2^-24 of a product -- are accumulated in f32.  The f32 product's accuracy
+ * (same k eps bound against float64), not its bits; off by default. */
 int ughip_matmul(ughip_device* dev, ughip_slice* dst, const ughip_slice* lhs,
                  const ughip_slice* rhs, size_t b, size_t m, size_t n, size_t k, size_t rank,
                  const size_t* lhs_dims, const size_t* lhs_strides, size_t lhs_offset,

@@ -357,3 +357,11 @@ def test_kernel_choice_for_the_baseline_shapes_is_pinned():
         _plan(F, B, 1, 128, 2560, 2048, 0)
     with pytest.raises(ug_amd.UgError):
         _plan(ug_amd.I32, ug_amd.I32, 1, 8, 8, 8, 0)
+    # f32 products as six bf16 terms: only with the switch, only where k % 64 == 0 and n % 8 == 0
+    with ug_amd.tuning(MATMUL_X6=1):
+        assert _plan(F, F, 8, 1024, 1024, 1024, 0) == "gemm_dma4<bf16,NN,256x128,256t,6 terms of 3 x 3 planes,f32 out>"
+        assert _plan(F, F, 1, 4096, 4096, 4096, 1) == "gemm_dma4<bf16,NT,256x256,256t,6 terms of 3 x 3 planes,f32 out>"
+        assert _plan(F, F, 1, 1024, 1020, 1024, 0) == "gemm_tiled<f32,NN,128x128,256t,ragged>" or "6 terms" not in _plan(F, F, 1, 1024, 1020, 1024, 0)
+        assert "6 terms" not in _plan(F, F, 1, 1024, 1024, 1000, 1)
+        assert "6 terms" not in _plan(B, B, 1, 4096, 4096, 4096, 1)
+    assert "6 terms" not in _plan(F, F, 8, 1024, 1024, 1024, 0)
