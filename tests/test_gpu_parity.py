@@ -2491,14 +2491,12 @@ def test_attention_followed_by_the_output_projection(hip, tune, b, nh, nkv, t, s
     assert fused(sr, d_got, 1) != 0
 
 
-@pytest.mark.parametrize("x3", [False, True])
-@pytest.mark.parametrize("t,length,hidden,inter,nh,nkv,bf16", [(300, 0, 512, 1024, 8, 2, True), (40, 7, 256, 512, 4, 2, True), (12, 0, 128, 256, 2, 1, False), (2, 3, 256, 512, 4, 4, True)])
+@pytest.mark.parametrize("x3,t,length,hidden,inter,nh,nkv,bf16", [(x3, *shape) for shape in ((300, 0, 512, 1024, 8, 2, True), (40, 7, 256, 512, 4, 2, True), (12, 0, 128, 256, 2, 1, False),
+                                                                                                (2, 3, 256, 512, 4, 4, True)) for x3 in (False, True) if shape[-1] or not x3])
 def test_layer_hooks_with_neighbours_folded_in(hip, x3, t, length, hidden, inter, nh, nkv, bf16):
     """Ops::linear_norm, Ops::attention_steps_add and Ops::mlp_stacked on the HIP device (one schedule item each) against
     the hooks they fold together on the same device -- bit for bit where no norm is folded in, a few ulps with it (the
     norm's sum of squares is added in another order) -- and against the same layer in float64."""
-    if x3 and not bf16:
-        pytest.skip("three bf16 terms need bf16 matrices")
     print("layer hooks", (x3, t, length, hidden, inter, nh, nkv, bf16), flush=True)
     ops = ug_amd.LlamaOps.hip(bf16x3=x3)
     d = hidden // nh
