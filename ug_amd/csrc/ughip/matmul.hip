@@ -440,8 +440,8 @@ static int grow_rows_ws(ughip_device* dev, size_t bytes) {
 // asked for without a device (ughip_matmul_plan) and is the same one the launch makes.
 enum Route { ROUTE_GEMV_NT, ROUTE_GEMV_NN, ROUTE_DMA, ROUTE_DMA_F32, ROUTE_X6, ROUTE_TILED, ROUTE_ANY, ROUTE_UNSUPPORTED };
 
-__global__ void split3_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ x3, size_t n4, int k);     // defined with the products of rows below
-__global__ void split3_kn_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ x3, size_t n4, int n);
+__global__ void split3_operands_kernel(const float* __restrict__ xa, uint16_t* __restrict__ pa, size_t na4, int ka, unsigned a_blocks, const float* __restrict__ xb,
+                                       uint16_t* __restrict__ pb, size_t nb4, int bk, int b_kn);  // defined with the products of rows below
 
 // An f32 product as six bf16 terms (UGHIP_MATMUL_X6=1; never the default: the f32 product's accuracy, not its bits): the
 // problem as the 16-bit kernel sees it once both operands are split into three bf16 planes per 64 elements of k -- rows of
@@ -575,10 +575,11 @@ static int matmul_impl(ughip_device* dev, ughip_slice* dst, const ughip_slice* l
     if (int rc = grow_gemm_ws(dev, a_bytes + b_elems * 6)) return rc;
     uint16_t* ap = static_cast<uint16_t*>(dev->gemm_ws);
     uint16_t* bp = reinterpret_cast<uint16_t*>(static_cast<char*>(dev->gemm_ws) + a_bytes);
-    split3_bf16_kernel<<<(unsigned)((a_elems / 4 + 255) / 256), 256, 0, st>>>(static_cast<const float*>(p.a), ap, a_elems / 4, (int)k);
-    UGHIP_HIPCHK(hipGetLastError());
-    if (q.b_cs == 1) split3_kn_bf16_kernel<<<(unsigned)((b_elems / 4 + 255) / 256), 256, 0, st>>>(static_cast<const float*>(p.b), bp, b_elems / 4, (int)n);
-    else split3_bf16_kernel<<<(unsigned)((b_elems / 4 + 255) / 256), 256, 0, st>>>(static_cast<const float*>(p.b), bp, b_elems / 4, (int)k);
+    const size_t a_blocks = (a_elems / 4 + 255) / 256, b_blocks = (b_elems / 4 + 255) / 256;
+    if (a_blocks + b_blocks > 0x7fffffffull) return set_error(UGHIP_ERR_INVALID, "matmul: operands too large for the pass that splits them");
+    const bool b_kn = q.b_cs == 1;
+    split3_operands_kernel<<<(unsigned)(a_blocks + b_blocks), 256, 0, st>>>(static_cast<const float*>(p.a), ap, a_elems / 4, (int)k, (unsigned)a_blocks,
+                                                                           static_cast<const float*>(p.b), bp, b_elems / 4, (int)(b_kn ? n : k), b_kn ? 1 : 0);
     UGHIP_HIPCHK(hipGetLastError());
     q.a = ap, q.b = bp, q.c = dst->ptr;
     UGHIP_HIPCHK(gemm_dma_launch_planes6(st, q, b, dma_tile));
@@ -636,22 +637,31 @@ __global__ void __launch_bounds__(256) split3_bf16_kernel(const float* __restric
 // RMSNorm of the rows of x [m, k] (model.rs:65-78: x / sqrt(mean(x^2) + eps) * alpha, the division as a multiplication by
 // the reciprocal, like the single-row projections do), one workgroup per row; the row's second pass comes from cache.
 // PLANES: the normalised row goes out as its three bf16 planes (what split3_bf16_kernel would make of it), else as f32.
-// The same split for an operand stored [k, n] (k % 64 == 0): the planes of rows kk .. kk + 63 are rows 3 kk .. of the result,
-// 64 rows of first terms, then 64 of second, then 64 of third ones; rows counts all rows of all batch elements (each a
-// multiple of 64), n4 groups of 4 elements.
-__global__ void __launch_bounds__(256) split3_kn_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ x3, size_t n4, int n) {
-  const size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (g >= n4) return;
-  const size_t e = g * 4, row = e / (size_t)n, col = e % (size_t)n;
+// An operand stored [k, n] (k % 64 == 0) is split the same way with the planes of rows kk .. kk + 63 as rows 3 kk .. of the
+// result: 64 rows of first terms, then 64 of second, then 64 of third ones (every batch element a multiple of 64 rows).
+// Both operands of a product in one launch: blocks 0 .. a_blocks - 1 split the lhs like split3_bf16_kernel, the rest the rhs,
+// like split3_bf16_kernel ([n, k]-major: b_kn == 0, bk = k) or by rows as described above ([k, n]-major: bk = n).
+__global__ void __launch_bounds__(256) split3_operands_kernel(const float* __restrict__ xa, uint16_t* __restrict__ pa, size_t na4, int ka, unsigned a_blocks,
+                                                              const float* __restrict__ xb, uint16_t* __restrict__ pb, size_t nb4, int bk, int b_kn) {
+  const bool lhs = blockIdx.x < a_blocks;
+  const size_t g = (size_t)(lhs ? blockIdx.x : blockIdx.x - a_blocks) * 256 + threadIdx.x;
+  if (g >= (lhs ? na4 : nb4)) return;
+  const float* __restrict__ x = lhs ? xa : xb;
+  uint16_t* __restrict__ x3 = lhs ? pa : pb;
+  const size_t w = (size_t)(lhs ? ka : bk), e = g * 4, row = e / w, col = e % w;
   const float4 v = reinterpret_cast<const float4*>(x)[g];
   const float in[4] = {v.x, v.y, v.z, v.w};
-  uint16_t hi[4], mid[4], lo[4];
+  if (lhs || !b_kn) {
+    split3_store4(in, x3 + row * 3 * w, col);
+  } else {
+    uint16_t hi[4], mid[4], lo[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) split3(in[i], hi[i], mid[i], lo[i]);
-  uint16_t* o = x3 + ((row / 64) * 192 + row % 64) * (size_t)n + col;
-  *reinterpret_cast<ushort4*>(o) = make_ushort4(hi[0], hi[1], hi[2], hi[3]);
-  *reinterpret_cast<ushort4*>(o + 64 * (size_t)n) = make_ushort4(mid[0], mid[1], mid[2], mid[3]);
-  *reinterpret_cast<ushort4*>(o + 128 * (size_t)n) = make_ushort4(lo[0], lo[1], lo[2], lo[3]);
+    for (int i = 0; i < 4; ++i) split3(in[i], hi[i], mid[i], lo[i]);
+    uint16_t* o = x3 + ((row / 64) * 192 + row % 64) * w + col;
+    *reinterpret_cast<ushort4*>(o) = make_ushort4(hi[0], hi[1], hi[2], hi[3]);
+    *reinterpret_cast<ushort4*>(o + 64 * w) = make_ushort4(mid[0], mid[1], mid[2], mid[3]);
+    *reinterpret_cast<ushort4*>(o + 128 * w) = make_ushort4(lo[0], lo[1], lo[2], lo[3]);
+  }
 }
 
 // NV: 16-byte groups a thread keeps of its row between the two passes (k <= 1024 NV; the row and alpha are requested at
