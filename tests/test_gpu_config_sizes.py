@@ -166,6 +166,31 @@ def test_matmul_f32_as_six_bf16_terms(hip, tune, bmnk, rhs_nk):
         np.testing.assert_array_equal(back, full)
 
 
+def test_matmul_f32_as_six_bf16_terms_random_shapes(hip, tune):
+    """Seeded random shapes for the six-term f32 product: 9-700 rows, N a multiple of 8, K a multiple of 64, both rhs layouts,
+    1-3 batch elements, against float64 within a few roundings of sum|a||b|; shapes the route does not take (K or N off
+    its multiples, fewer than 9 rows) fall back to the f32 kernels with the switch on."""
+    tune.setenv("UGHIP_MATMUL_X6", "1")
+    gen = np.random.default_rng(909)
+    for case in range(14):
+        b = int(gen.integers(1, 4)); m = int(gen.integers(9, 700)); n = 8 * int(gen.integers(1, 90)); k = 64 * int(gen.integers(1, 11))
+        rhs_nk = bool(gen.integers(0, 2))
+        a = rng.uniform_pm1(3000 + case, b * m * k).reshape(b, m, k)
+        w = rng.uniform_pm1(4000 + case, b * k * n).reshape(b, k, n)
+        got, kernel = _matmul(hip, F32, a, w, rhs_nk)
+        print("f32 as six bf16 terms, random", case, (b, m, n, k), "NT" if rhs_nk else "NN", kernel, flush=True)
+        assert "6 terms" in kernel, kernel
+        exact, mag = _f64_product(a, w)
+        assert np.all(np.abs(got - exact) <= (8 + 2 * np.sqrt(k)) * EPS32 * mag + 1e-12), (case, float(np.abs(got - exact).max()))
+    for (b, m, n, k) in ((1, 64, 64, 96), (1, 64, 60, 128), (2, 8, 64, 128)):
+        a = rng.uniform_pm1(51, b * m * k).reshape(b, m, k)
+        w = rng.uniform_pm1(52, b * k * n).reshape(b, k, n)
+        got, kernel = _matmul(hip, F32, a, w, False)
+        assert "6 terms" not in kernel, kernel
+        exact, mag = _f64_product(a, w)
+        assert np.all(np.abs(got - exact) <= k * EPS32 * mag + 1e-12)
+
+
 @pytest.mark.parametrize("rhs_nk", [False, True], ids=["NN", "NT"])
 def test_config3_bmm_bf16(hip, rhs_nk):
     """bf16 8 x 1024^3 (RNE-rounded copies of the f32 operands): no reference result exists (cpu_runtime.rs:345-356
